@@ -1,0 +1,444 @@
+// CPU oracle: a literal restatement of Composable Kernel's host reference
+// operators for the MFMA GEMM hot path. THIS IS TEST INFRASTRUCTURE: only the
+// test-suite, the smoke check and the benchmark's cpu_baseline leg may load it.
+// The shipped library never links or calls anything in this file.
+//
+// What is restated (reference file:line):
+//   cko_gemm_i8 / cko_gemm_f16       ReferenceGemm::Invoker::Run
+//       library/include/ck/library/reference_tensor_operation/cpu/reference_gemm.hpp:57-88
+//   cko_conv2d_fwd_{f32,f16,i8}      ReferenceConvFwd (NumDimSpatial == 2 branch)
+//       library/include/ck/library/reference_tensor_operation/cpu/reference_conv_fwd.hpp:132-185
+//   cko_batched_gemm_f16             ReferenceBatchedGemm::Invoker::Run
+//       library/include/ck/library/reference_tensor_operation/cpu/reference_batched_gemm.hpp:56-88
+//   cko_batched_gemm_gemm_f16        two chained ReferenceBatchedGemm with an
+//       fp16 intermediate (the fused operator does not exist in the reference
+//       snapshot: parity UNPINNED by reference vectors, pinned by brute force
+//       and closed forms in tests/test_oracle.py)
+//   epilogue functors                RequantReluRequant
+//       example/14_gemm_xdl_requant_relu_requant/gemm_xdl_requant_relu_requant_int8.cpp:21-39
+//       PassThrough include/ck/tensor_operation/gpu/element/unary_element_wise_operation.hpp:13-25
+//   type_convert                     include/ck/utility/data_type.hpp:934-938
+//   work split over threads          ParallelTensorFunctor
+//       library/include/ck/library/host_tensor/host_tensor.hpp:143-194
+//   conv output size                 ConvParams::GetOutputSpatialLengths
+//       library/src/utility/conv_util.cpp:89-116
+//   magic division                   include/ck/utility/magic_division.hpp:28-54,132-137
+//   check_err                        library/include/ck/library/utility/check_err.hpp:24-193
+//
+// Pinning status of each function is listed in oracle/README.md and checked by
+// tests/test_oracle.py (golden vectors of the reference's own tests, closed
+// forms, brute force, and the compiled reference in oracle/_ref when present).
+//
+// Build: g++ -O3 -ffp-contract=off -std=c++17 -shared -fPIC (no fast-math: the
+// epilogue's two fp32 multiplies must stay two roundings).
+
+#include <algorithm>
+#include <cmath>
+#include <cstdint>
+#include <cstring>
+#include <functional>
+#include <thread>
+#include <vector>
+
+namespace {
+
+// ---- fp16 <-> fp32, software, round-to-nearest-even (== _Float16 casts) ----
+inline float half_to_float(uint16_t h)
+{
+    const uint32_t sign = (uint32_t)(h & 0x8000u) << 16;
+    uint32_t exp        = (h >> 10) & 0x1Fu;
+    uint32_t man        = h & 0x3FFu;
+    uint32_t bits;
+    if(exp == 0)
+    {
+        if(man == 0)
+        {
+            bits = sign;
+        }
+        else
+        {
+            // subnormal: normalise
+            int e = -1;
+            do
+            {
+                man <<= 1;
+                ++e;
+            } while((man & 0x400u) == 0);
+            man &= 0x3FFu;
+            bits = sign | ((uint32_t)(127 - 15 - e) << 23) | (man << 13);
+        }
+    }
+    else if(exp == 31)
+    {
+        bits = sign | 0x7F800000u | (man << 13);
+    }
+    else
+    {
+        bits = sign | ((exp + 127 - 15) << 23) | (man << 13);
+    }
+    float f;
+    std::memcpy(&f, &bits, 4);
+    return f;
+}
+
+inline uint16_t float_to_half(float f)
+{
+    uint32_t x;
+    std::memcpy(&x, &f, 4);
+    const uint16_t sign = (uint16_t)((x >> 16) & 0x8000u);
+    const uint32_t absx = x & 0x7FFFFFFFu;
+    if(absx >= 0x7F800000u)
+    { // inf / nan
+        return (uint16_t)(sign | 0x7C00u | ((absx > 0x7F800000u) ? (0x200u | ((absx >> 13) & 0x3FFu)) : 0u));
+    }
+    if(absx >= 0x477FF000u)
+    { // >= 65520 rounds to inf
+        return (uint16_t)(sign | 0x7C00u);
+    }
+    if(absx < 0x33000001u)
+    { // < 2^-25 (or == 2^-25 tie -> even = 0)
+        return sign;
+    }
+    int32_t e    = (int32_t)(absx >> 23) - 127;
+    uint32_t man = (absx & 0x7FFFFFu) | 0x800000u; // 24-bit significand
+    uint32_t shift;
+    uint32_t base;
+    if(e < -14)
+    { // subnormal half
+        shift = (uint32_t)(13 + (-14 - e));
+        base  = 0;
+    }
+    else
+    {
+        shift = 13;
+        base  = (uint32_t)(e + 15) << 10;
+        man &= 0x7FFFFFu;
+    }
+    uint32_t q   = man >> shift;
+    uint32_t rem = man & ((1u << shift) - 1u);
+    uint32_t hlf = 1u << (shift - 1);
+    if(rem > hlf || (rem == hlf && (q & 1u)))
+        ++q;
+    return (uint16_t)(sign | (base + q)); // carry into exponent is the correct result
+}
+
+// ---- element-wise functors ----
+enum
+{
+    EPI_PASSTHROUGH = 0,
+    EPI_REQUANT_CK  = 1, // example 14, literal: no rounding, clamp, caller truncates
+    EPI_REQUANT_RND = 2  // clamp(rint(sR * relu(clamp(rint(sG * x)))))
+};
+
+struct Epilogue
+{
+    int kind;
+    float scale_gemm;
+    float scale_relu;
+    // y = op(x), both fp32 (CElementwiseOperation(float& y, const float& x))
+    inline float operator()(float x) const
+    {
+        if(kind == EPI_PASSTHROUGH)
+            return x;
+        if(kind == EPI_REQUANT_CK)
+        {
+            float g = scale_gemm * x;
+            float r = g > 0 ? g : 0;
+            float q = scale_relu * r;
+            return q > 127 ? 127 : (q < -128 ? -128 : q);
+        }
+        float t = std::nearbyint(scale_gemm * x);
+        t       = t > 127 ? 127 : (t < -128 ? -128 : t);
+        float r = t > 0 ? t : 0;
+        float u = std::nearbyint(scale_relu * r);
+        return u > 127 ? 127 : (u < -128 ? -128 : u);
+    }
+};
+
+// type_convert<int8_t>(float): static_cast truncates toward zero. Out-of-range
+// floats are undefined in C++; x86 gives cvttss2si + low byte, which is what the
+// reference's int8 conv tests rely on. Done here in a defined way.
+inline int8_t float_to_i8_trunc_wrap(float v)
+{
+    int32_t a;
+    if(!(v > -2147483648.0f && v < 2147483648.0f))
+        a = INT32_MIN; // cvttss2si "integer indefinite"
+    else
+        a = (int32_t)v;
+    return (int8_t)(uint8_t)(a & 0xFF);
+}
+
+// Contiguous split of the flattened index range over threads.
+void parallel_for(std::size_t n, int nthreads, const std::function<void(std::size_t, std::size_t)>& body)
+{
+    if(nthreads <= 0)
+        nthreads = (int)std::thread::hardware_concurrency();
+    if(nthreads <= 1 || n < 2)
+    {
+        body(0, n);
+        return;
+    }
+    std::size_t per = (n + (std::size_t)nthreads - 1) / (std::size_t)nthreads;
+    std::vector<std::thread> ts;
+    for(int t = 0; t < nthreads; ++t)
+    {
+        std::size_t b = (std::size_t)t * per;
+        std::size_t e = std::min(b + per, n);
+        if(b >= e)
+            break;
+        ts.emplace_back([=, &body] { body(b, e); });
+    }
+    for(auto& t : ts)
+        t.join();
+}
+
+} // namespace
+
+extern "C" {
+
+int cko_hardware_threads() { return (int)std::thread::hardware_concurrency(); }
+
+uint16_t cko_float_to_half(float f) { return float_to_half(f); }
+float cko_half_to_float(uint16_t h) { return half_to_float(h); }
+
+// Scalar epilogue exposed so the tests can pin it exhaustively.
+int8_t cko_epilogue_i8(int32_t acc, int kind, float scale_gemm, float scale_relu)
+{
+    Epilogue ep{kind, scale_gemm, scale_relu};
+    if(kind == EPI_PASSTHROUGH)
+        return (int8_t)(uint8_t)(acc & 0xFF);
+    return float_to_i8_trunc_wrap(ep((float)acc));
+}
+
+// int8 GEMM. A is logical [M,K] with strides (sa_m, sa_k), B logical [K,N] with
+// (sb_k, sb_n), C logical [M,N] with (sc_m, sc_n); all in elements.
+// acc_float != 0: AccDataType = float (example 14); else int32 (tests/profiler).
+// With int32 accumulation only PassThrough is valid (the low byte is kept).
+void cko_gemm_i8(const int8_t* a, const int8_t* b, int8_t* c, int M, int N, int K,
+                 int64_t sa_m, int64_t sa_k, int64_t sb_k, int64_t sb_n, int64_t sc_m, int64_t sc_n,
+                 int acc_float, int epi_kind, float scale_gemm, float scale_relu, int nthreads)
+{
+    Epilogue ep{epi_kind, scale_gemm, scale_relu};
+    parallel_for((std::size_t)M * (std::size_t)N, nthreads, [&](std::size_t i0, std::size_t i1) {
+        for(std::size_t i = i0; i < i1; ++i)
+        {
+            const std::size_t m = i / (std::size_t)N, n = i % (std::size_t)N;
+            if(acc_float)
+            {
+                float acc = 0;
+                for(int k = 0; k < K; ++k)
+                    acc += (float)a[m * sa_m + k * sa_k] * (float)b[k * sb_k + n * sb_n];
+                c[m * sc_m + n * sc_n] = float_to_i8_trunc_wrap(ep(acc));
+            }
+            else
+            {
+                int32_t acc = 0;
+                for(int k = 0; k < K; ++k)
+                    acc += (int32_t)a[m * sa_m + k * sa_k] * (int32_t)b[k * sb_k + n * sb_n];
+                c[m * sc_m + n * sc_n] = (int8_t)(uint8_t)(acc & 0xFF);
+            }
+        }
+    });
+}
+
+// int8 GEMM returning the raw int32 accumulators (row-major [M,N]); used to
+// drive epilogue checks and to pin the GEMM part by closed forms.
+void cko_gemm_i8_acc(const int8_t* a, const int8_t* b, int32_t* acc_out, int M, int N, int K,
+                     int64_t sa_m, int64_t sa_k, int64_t sb_k, int64_t sb_n, int nthreads)
+{
+    parallel_for((std::size_t)M * (std::size_t)N, nthreads, [&](std::size_t i0, std::size_t i1) {
+        for(std::size_t i = i0; i < i1; ++i)
+        {
+            const std::size_t m = i / (std::size_t)N, n = i % (std::size_t)N;
+            int32_t acc         = 0;
+            for(int k = 0; k < K; ++k)
+                acc += (int32_t)a[m * sa_m + k * sa_k] * (int32_t)b[k * sb_k + n * sb_n];
+            acc_out[i] = acc;
+        }
+    });
+}
+
+// fp16 GEMM, AccDataType = float, sequential k, PassThrough everywhere.
+void cko_gemm_f16(const uint16_t* a, const uint16_t* b, uint16_t* c, int M, int N, int K,
+                  int64_t sa_m, int64_t sa_k, int64_t sb_k, int64_t sb_n, int64_t sc_m, int64_t sc_n,
+                  int nthreads)
+{
+    parallel_for((std::size_t)M * (std::size_t)N, nthreads, [&](std::size_t i0, std::size_t i1) {
+        for(std::size_t i = i0; i < i1; ++i)
+        {
+            const std::size_t m = i / (std::size_t)N, n = i % (std::size_t)N;
+            float acc           = 0;
+            for(int k = 0; k < K; ++k)
+                acc += half_to_float(a[m * sa_m + k * sa_k]) * half_to_float(b[k * sb_k + n * sb_n]);
+            c[m * sc_m + n * sc_n] = float_to_half(acc);
+        }
+    });
+}
+
+// Strided batched fp16 GEMM: A [G,M,K], B [G,K,N], C [G,M,N], element strides.
+void cko_batched_gemm_f16(const uint16_t* a, const uint16_t* b, uint16_t* c, int G, int M, int N, int K,
+                          int64_t sa_g, int64_t sa_m, int64_t sa_k, int64_t sb_g, int64_t sb_k,
+                          int64_t sb_n, int64_t sc_g, int64_t sc_m, int64_t sc_n, int nthreads)
+{
+    parallel_for((std::size_t)G * M * N, nthreads, [&](std::size_t i0, std::size_t i1) {
+        for(std::size_t i = i0; i < i1; ++i)
+        {
+            const std::size_t g = i / ((std::size_t)M * N);
+            const std::size_t m = (i / (std::size_t)N) % (std::size_t)M, n = i % (std::size_t)N;
+            float acc           = 0;
+            for(int k = 0; k < K; ++k)
+                acc += half_to_float(a[g * sa_g + m * sa_m + k * sa_k]) *
+                       half_to_float(b[g * sb_g + k * sb_k + n * sb_n]);
+            c[g * sc_g + m * sc_m + n * sc_n] = float_to_half(acc);
+        }
+    });
+}
+
+// C[g] = fp16( fp16(A[g] * B0[g]) * B1[g] ): A [G,M,K], B0 logical [G,K,N],
+// B1 logical [G,N,O], C [G,M,O].
+void cko_batched_gemm_gemm_f16(const uint16_t* a, const uint16_t* b0, const uint16_t* b1, uint16_t* c,
+                               int G, int M, int N, int K, int O, int64_t sa_g, int64_t sa_m,
+                               int64_t sa_k, int64_t sb0_g, int64_t sb0_k, int64_t sb0_n, int64_t sb1_g,
+                               int64_t sb1_n, int64_t sb1_o, int64_t sc_g, int64_t sc_m, int64_t sc_o,
+                               int nthreads)
+{
+    std::vector<uint16_t> s((std::size_t)G * M * N);
+    cko_batched_gemm_f16(a, b0, s.data(), G, M, N, K, sa_g, sa_m, sa_k, sb0_g, sb0_k, sb0_n,
+                         (int64_t)M * N, N, 1, nthreads);
+    cko_batched_gemm_f16(s.data(), b1, c, G, M, O, N, (int64_t)M * N, N, 1, sb1_g, sb1_n, sb1_o, sc_g,
+                         sc_m, sc_o, nthreads);
+}
+
+// conv output length along one spatial dimension
+int cko_conv_out_len(int in_len, int filter_len, int stride, int dilation, int pad_left, int pad_right)
+{
+    const int eff = (filter_len - 1) * dilation + 1;
+    return (in_len + pad_left + pad_right - eff) / stride + 1;
+}
+
+} // extern "C"
+
+namespace {
+
+// 2-D forward convolution, NHWC / KYXC / NHWK memory, fp32 accumulation in the
+// loop order c -> y -> x, out = convert(out_op(acc)).
+template <typename LoadIn, typename LoadWei, typename StoreOut>
+void conv2d_fwd(int N, int K, int C, int Hi, int Wi, int Y, int X, int Ho, int Wo, int sH, int sW,
+                int dH, int dW, int pH, int pW, int nthreads, LoadIn in_at, LoadWei wei_at,
+                StoreOut store)
+{
+    // parallel index space is the logical (n, k, ho, wo), k before ho before wo
+    parallel_for((std::size_t)N * K * Ho * Wo, nthreads, [&](std::size_t i0, std::size_t i1) {
+        for(std::size_t i = i0; i < i1; ++i)
+        {
+            std::size_t r  = i;
+            const int wo   = (int)(r % (std::size_t)Wo);
+            r /= (std::size_t)Wo;
+            const int ho = (int)(r % (std::size_t)Ho);
+            r /= (std::size_t)Ho;
+            const int k = (int)(r % (std::size_t)K);
+            const int n = (int)(r / (std::size_t)K);
+            float acc   = 0;
+            for(int c = 0; c < C; ++c)
+                for(int y = 0; y < Y; ++y)
+                {
+                    const long hi = (long)ho * sH + (long)y * dH - pH;
+                    for(int x = 0; x < X; ++x)
+                    {
+                        const long wi = (long)wo * sW + (long)x * dW - pW;
+                        if(hi >= 0 && hi < Hi && wi >= 0 && wi < Wi)
+                        {
+                            const float v_in  = in_at((((std::size_t)n * Hi + hi) * Wi + wi) * C + c);
+                            const float v_wei = wei_at((((std::size_t)k * Y + y) * X + x) * C + c);
+                            acc += v_in * v_wei;
+                        }
+                    }
+                }
+            store((((std::size_t)n * Ho + ho) * Wo + wo) * K + k, acc);
+        }
+    });
+}
+
+} // namespace
+
+extern "C" {
+
+void cko_conv2d_fwd_f32(const float* in, const float* wei, float* out, int N, int K, int C, int Hi,
+                        int Wi, int Y, int X, int Ho, int Wo, int sH, int sW, int dH, int dW, int pH,
+                        int pW, int nthreads)
+{
+    conv2d_fwd(
+        N, K, C, Hi, Wi, Y, X, Ho, Wo, sH, sW, dH, dW, pH, pW, nthreads,
+        [=](std::size_t o) { return in[o]; }, [=](std::size_t o) { return wei[o]; },
+        [=](std::size_t o, float acc) { out[o] = acc; });
+}
+
+void cko_conv2d_fwd_f16(const uint16_t* in, const uint16_t* wei, uint16_t* out, int N, int K, int C,
+                        int Hi, int Wi, int Y, int X, int Ho, int Wo, int sH, int sW, int dH, int dW,
+                        int pH, int pW, int nthreads)
+{
+    conv2d_fwd(
+        N, K, C, Hi, Wi, Y, X, Ho, Wo, sH, sW, dH, dW, pH, pW, nthreads,
+        [=](std::size_t o) { return half_to_float(in[o]); },
+        [=](std::size_t o) { return half_to_float(wei[o]); },
+        [=](std::size_t o, float acc) { out[o] = float_to_half(acc); });
+}
+
+void cko_conv2d_fwd_i8(const int8_t* in, const int8_t* wei, int8_t* out, int N, int K, int C, int Hi,
+                       int Wi, int Y, int X, int Ho, int Wo, int sH, int sW, int dH, int dW, int pH,
+                       int pW, int epi_kind, float scale_gemm, float scale_relu, int nthreads)
+{
+    Epilogue ep{epi_kind, scale_gemm, scale_relu};
+    conv2d_fwd(
+        N, K, C, Hi, Wi, Y, X, Ho, Wo, sH, sW, dH, dW, pH, pW, nthreads,
+        [=](std::size_t o) { return (float)in[o]; }, [=](std::size_t o) { return (float)wei[o]; },
+        [=](std::size_t o, float acc) { out[o] = float_to_i8_trunc_wrap(ep(acc)); });
+}
+
+// ---- magic-number division (dividend < 2^31, divisor >= 1) ----
+void cko_magic_division_params(uint32_t divisor, uint32_t* multiplier, uint32_t* shift)
+{
+    uint32_t s = 0;
+    while(s < 32 && ((uint64_t)1 << s) < divisor)
+        ++s;
+    const uint64_t one = 1;
+    *multiplier        = (uint32_t)(((one << 32) * ((one << s) - divisor)) / divisor + 1);
+    *shift             = s;
+}
+
+uint32_t cko_magic_division_divide(uint32_t dividend, uint32_t multiplier, uint32_t shift)
+{
+    const uint32_t hi = (uint32_t)(((uint64_t)dividend * multiplier) >> 32);
+    return (hi + dividend) >> shift;
+}
+
+// ---- check_err: count of elements violating |o-r| <= atol + rtol*|r| or non-finite ----
+int64_t cko_check_err_f16(const uint16_t* out, const uint16_t* ref, int64_t n, double rtol, double atol,
+                          double* max_err)
+{
+    int64_t bad = 0;
+    double me   = 0;
+    for(int64_t i = 0; i < n; ++i)
+    {
+        const double o = half_to_float(out[i]), r = half_to_float(ref[i]);
+        const double err = std::fabs(o - r);
+        if(err > atol + rtol * std::fabs(r) || !std::isfinite(o) || !std::isfinite(r))
+        {
+            ++bad;
+            me = std::max(me, err);
+        }
+    }
+    if(max_err)
+        *max_err = me;
+    return bad;
+}
+
+int64_t cko_check_err_i8(const int8_t* out, const int8_t* ref, int64_t n)
+{
+    int64_t bad = 0;
+    for(int64_t i = 0; i < n; ++i)
+        bad += out[i] != ref[i];
+    return bad;
+}
+
+} // extern "C"

@@ -1,0 +1,95 @@
+"""numpy forms of the oracle for full-size checks. Test infrastructure.
+
+int8 products summed in fp32 stay exact while sum(|a*b|) < 2**24, so an fp32
+BLAS GEMM on int8-valued floats returns the exact integer accumulators in any
+summation order (asserted below). The epilogue is the reference functor written
+with numpy float32 ufuncs: each ufunc rounds once, nothing is fused.
+Equality of these forms with the literal restatement (oracle.lit) on small
+shapes is asserted in tests/test_oracle.py.
+"""
+import numpy as np
+
+from .lit import EPI_PASSTHROUGH, EPI_REQUANT_CK, EPI_REQUANT_RND
+
+
+def epilogue_i8(acc_i32, epi, scale_gemm=1.0, scale_relu=1.0):
+    acc_i32 = np.asarray(acc_i32)
+    if epi == EPI_PASSTHROUGH:
+        return (acc_i32.astype(np.int64) & 0xFF).astype(np.uint8).view(np.int8)
+    x = acc_i32.astype(np.float32)
+    sg, sr = np.float32(scale_gemm), np.float32(scale_relu)
+    lo, hi = np.float32(-128), np.float32(127)
+    if epi == EPI_REQUANT_CK:
+        g = sg * x
+        r = np.where(g > 0, g, np.float32(0))
+        q = sr * r
+        y = np.where(q > hi, hi, np.where(q < lo, lo, q))
+    elif epi == EPI_REQUANT_RND:
+        t = np.rint(sg * x)
+        t = np.where(t > hi, hi, np.where(t < lo, lo, t))
+        r = np.where(t > 0, t, np.float32(0))
+        u = np.rint(sr * r)
+        y = np.where(u > hi, hi, np.where(u < lo, lo, u))
+    else:
+        raise ValueError(epi)
+    assert y.dtype == np.float32
+    return y.astype(np.int32).astype(np.int8)  # truncation toward zero; in range after the clamp
+
+
+def gemm_i8_acc(a_mk, b_kn):
+    a = np.asarray(a_mk)
+    b = np.asarray(b_kn)
+    bound = int(np.abs(a).max(initial=0)) * int(np.abs(b).max(initial=0)) * a.shape[1]
+    assert bound < 2 ** 24, "fp32 BLAS would not be exact for these magnitudes"
+    acc = a.astype(np.float32) @ b.astype(np.float32)
+    return acc.astype(np.int32)
+
+
+def gemm_i8(a_mk, b_kn, epi=EPI_PASSTHROUGH, scale_gemm=1.0, scale_relu=1.0):
+    return epilogue_i8(gemm_i8_acc(a_mk, b_kn), epi, scale_gemm, scale_relu)
+
+
+def gemm_f16(a_mk, b_kn):
+    """fp32-accumulated product rounded once to fp16 (BLAS summation order)."""
+    return (np.asarray(a_mk, np.float32) @ np.asarray(b_kn, np.float32)).astype(np.float16)
+
+
+def im2col(inp_nhwc, Y, X, strides, dilations, pads, right_pads=None):
+    """[N,Hi,Wi,C] -> [N*Ho*Wo, Y*X*C] with (y,x,c) ordering, c fastest; zero padding."""
+    if right_pads is None:
+        right_pads = pads
+    N, Hi, Wi, C = inp_nhwc.shape
+    sH, sW = strides
+    dH, dW = dilations
+    Ho = (Hi + pads[0] + right_pads[0] - ((Y - 1) * dH + 1)) // sH + 1
+    Wo = (Wi + pads[1] + right_pads[1] - ((X - 1) * dW + 1)) // sW + 1
+    p = np.zeros((N, Hi + pads[0] + right_pads[0], Wi + pads[1] + right_pads[1], C), inp_nhwc.dtype)
+    p[:, pads[0]:pads[0] + Hi, pads[1]:pads[1] + Wi, :] = inp_nhwc
+    cols = np.empty((N, Ho, Wo, Y, X, C), inp_nhwc.dtype)
+    for y in range(Y):
+        for x in range(X):
+            cols[:, :, :, y, x, :] = p[:, y * dH:y * dH + (Ho - 1) * sH + 1:sH,
+                                       x * dW:x * dW + (Wo - 1) * sW + 1:sW, :]
+    return cols.reshape(N * Ho * Wo, Y * X * C), Ho, Wo
+
+
+def conv2d_fwd_i8(inp_nhwc, wei_kyxc, strides=(1, 1), dilations=(1, 1), pads=(0, 0), right_pads=None,
+                  epi=EPI_PASSTHROUGH, scale_gemm=1.0, scale_relu=1.0):
+    N = inp_nhwc.shape[0]
+    K, Y, X, C = wei_kyxc.shape
+    cols, Ho, Wo = im2col(inp_nhwc, Y, X, strides, dilations, pads, right_pads)
+    acc = gemm_i8_acc(cols, wei_kyxc.reshape(K, Y * X * C).T)
+    return epilogue_i8(acc, epi, scale_gemm, scale_relu).reshape(N, Ho, Wo, K)
+
+
+def conv2d_fwd_f16(inp_nhwc, wei_kyxc, strides=(1, 1), dilations=(1, 1), pads=(0, 0), right_pads=None):
+    N = inp_nhwc.shape[0]
+    K, Y, X, C = wei_kyxc.shape
+    cols, Ho, Wo = im2col(inp_nhwc, Y, X, strides, dilations, pads, right_pads)
+    out = cols.astype(np.float32) @ wei_kyxc.reshape(K, Y * X * C).T.astype(np.float32)
+    return out.astype(np.float16).reshape(N, Ho, Wo, K)
+
+
+def batched_gemm_gemm_f16(a_gmk, b0_gkn, b1_gno):
+    s = np.matmul(np.asarray(a_gmk, np.float32), np.asarray(b0_gkn, np.float32)).astype(np.float16)
+    return np.matmul(s.astype(np.float32), np.asarray(b1_gno, np.float32)).astype(np.float16)

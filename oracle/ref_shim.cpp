@@ -1,0 +1,215 @@
+// C-ABI shim around the reference's OWN host operators, compiled from the
+// sources where they lie under /root/reference (never copied). TEST
+// INFRASTRUCTURE ONLY: validates oracle/ck_oracle.cpp and can serve as the
+// benchmark's cpu_baseline. Built by oracle/Makefile into oracle/_ref/.
+//
+// Instantiates, exactly as the reference's examples/tests/profiler do:
+//   ReferenceGemm<int8,int8,int8,float,Pass,Pass,RequantReluRequant>  (example 14, :103-109)
+//   ReferenceGemm<int8,int8,int8,int32,Pass,Pass,Pass>                 (profile_gemm.cpp int8)
+//   ReferenceGemm<half,half,half,float,Pass,Pass,Pass>                 (example 01 fp16)
+//   ReferenceConvFwd<T,T,T,Pass,Pass,Pass,2> for float / half / int8
+//   ReferenceBatchedGemm<half,half,half,Pass,Pass,Pass>
+//
+// RequantReluRequant lives inside the example's translation unit
+// (example/14_.../gemm_xdl_requant_relu_requant_int8.cpp:21-39), which also pulls
+// in the device-side headers; those do not compile with this ROCm release
+// (get_id.hpp's constexpr warpSize), so the five-line functor is restated here
+// and handed to the reference's own ReferenceGemm template. The rounded variant
+// has no counterpart in the reference at all.
+
+#include <cmath>
+#include <cstdint>
+#include <cstring>
+#include <vector>
+
+#include "ck/utility/magic_division.hpp"
+#include "ck/tensor_operation/gpu/element/element_wise_operation.hpp"
+#include "ck/library/host_tensor/host_tensor.hpp"
+#include "ck/library/utility/conv_util.hpp"
+#include "ck/library/reference_tensor_operation/cpu/reference_gemm.hpp"
+#include "ck/library/reference_tensor_operation/cpu/reference_conv_fwd.hpp"
+#include "ck/library/reference_tensor_operation/cpu/reference_batched_gemm.hpp"
+
+namespace {
+
+using PassThrough = ck::tensor_operation::element_wise::PassThrough;
+
+struct RequantReluRequant
+{
+    RequantReluRequant(float sg, float sr) : sg_(sg), sr_(sr) {}
+    void operator()(float& y, const float& x) const
+    {
+        float g = sg_ * x;
+        float r = g > 0 ? g : 0;
+        float q = sr_ * r;
+        y       = q > 127 ? 127 : q < -128 ? -128 : q;
+    }
+    float sg_, sr_;
+};
+
+using ReferenceGemmInstance = ck::tensor_operation::host::
+    ReferenceGemm<int8_t, int8_t, int8_t, float, PassThrough, PassThrough, RequantReluRequant>;
+
+struct RequantRoundReluRequantRound
+{
+    RequantRoundReluRequantRound(float sg, float sr) : sg_(sg), sr_(sr) {}
+    void operator()(float& y, const float& x) const
+    {
+        float t = std::nearbyint(sg_ * x);
+        t       = t > 127 ? 127 : (t < -128 ? -128 : t);
+        float r = t > 0 ? t : 0;
+        float u = std::nearbyint(sr_ * r);
+        y       = u > 127 ? 127 : (u < -128 ? -128 : u);
+    }
+    float sg_, sr_;
+};
+
+template <typename T>
+Tensor<T> make_tensor(std::vector<std::size_t> lens, std::vector<std::size_t> strides, const T* src)
+{
+    Tensor<T> t(HostTensorDescriptor(lens, strides));
+    if(src)
+        std::memcpy(t.mData.data(), src, t.mData.size() * sizeof(T));
+    return t;
+}
+
+template <typename Ref, typename TA, typename TC, typename COp>
+void run_gemm(const TA* a, const TA* b, TC* c, int M, int N, int K, long sa_m, long sa_k, long sb_k,
+              long sb_n, long sc_m, long sc_n, COp cop)
+{
+    using sz = std::size_t;
+    auto ta  = make_tensor<TA>({(sz)M, (sz)K}, {(sz)sa_m, (sz)sa_k}, a);
+    auto tb  = make_tensor<TA>({(sz)K, (sz)N}, {(sz)sb_k, (sz)sb_n}, b);
+    auto tc  = make_tensor<TC>({(sz)M, (sz)N}, {(sz)sc_m, (sz)sc_n}, c);
+    Ref ref;
+    auto inv = ref.MakeInvoker();
+    auto arg = ref.MakeArgument(ta, tb, tc, PassThrough{}, PassThrough{}, cop);
+    inv.Run(arg);
+    std::memcpy(c, tc.mData.data(), tc.mData.size() * sizeof(TC));
+}
+
+template <typename T>
+void run_conv(const T* in, const T* wei, T* out, int N, int K, int C, int Hi, int Wi, int Y, int X,
+              int Ho, int Wo, int sH, int sW, int dH, int dW, int pH, int pW)
+{
+    using sz = std::size_t;
+    // logical N,C,H,W with NHWC strides (conv_util.hpp:209-215)
+    auto ti = make_tensor<T>({(sz)N, (sz)C, (sz)Hi, (sz)Wi},
+                             {(sz)C * Hi * Wi, 1, (sz)Wi * C, (sz)C}, in);
+    auto tw = make_tensor<T>({(sz)K, (sz)C, (sz)Y, (sz)X}, {(sz)C * Y * X, 1, (sz)X * C, (sz)C}, wei);
+    auto to = make_tensor<T>({(sz)N, (sz)K, (sz)Ho, (sz)Wo},
+                             {(sz)K * Ho * Wo, 1, (sz)Wo * K, (sz)K}, (const T*)nullptr);
+    using Ref =
+        ck::tensor_operation::host::ReferenceConvFwd<T, T, T, PassThrough, PassThrough, PassThrough, 2>;
+    Ref ref;
+    auto inv = ref.MakeInvoker();
+    auto arg = ref.MakeArgument(ti, tw, to, {sH, sW}, {dH, dW}, {pH, pW}, {pH, pW}, PassThrough{},
+                                PassThrough{}, PassThrough{});
+    inv.Run(arg);
+    std::memcpy(out, to.mData.data(), to.mData.size() * sizeof(T));
+}
+
+} // namespace
+
+extern "C" {
+
+// epi: 1 = example-14 functor, 2 = rounded variant
+void ckref_gemm_i8_requant(const int8_t* a, const int8_t* b, int8_t* c, int M, int N, int K, long sa_m,
+                           long sa_k, long sb_k, long sb_n, long sc_m, long sc_n, int epi,
+                           float scale_gemm, float scale_relu)
+{
+    if(epi == 1)
+        run_gemm<ReferenceGemmInstance, int8_t, int8_t>(a, b, c, M, N, K, sa_m, sa_k, sb_k, sb_n, sc_m,
+                                                        sc_n, RequantReluRequant{scale_gemm, scale_relu});
+    else
+        run_gemm<ck::tensor_operation::host::ReferenceGemm<int8_t, int8_t, int8_t, float, PassThrough,
+                                                           PassThrough, RequantRoundReluRequantRound>,
+                 int8_t, int8_t>(a, b, c, M, N, K, sa_m, sa_k, sb_k, sb_n, sc_m, sc_n,
+                                 RequantRoundReluRequantRound{scale_gemm, scale_relu});
+}
+
+void ckref_gemm_i8(const int8_t* a, const int8_t* b, int8_t* c, int M, int N, int K, long sa_m,
+                   long sa_k, long sb_k, long sb_n, long sc_m, long sc_n)
+{
+    run_gemm<ck::tensor_operation::host::ReferenceGemm<int8_t, int8_t, int8_t, int32_t, PassThrough,
+                                                       PassThrough, PassThrough>,
+             int8_t, int8_t>(a, b, c, M, N, K, sa_m, sa_k, sb_k, sb_n, sc_m, sc_n, PassThrough{});
+}
+
+void ckref_gemm_f16(const uint16_t* a, const uint16_t* b, uint16_t* c, int M, int N, int K, long sa_m,
+                    long sa_k, long sb_k, long sb_n, long sc_m, long sc_n)
+{
+    using H = ck::half_t;
+    run_gemm<ck::tensor_operation::host::ReferenceGemm<H, H, H, float, PassThrough, PassThrough,
+                                                       PassThrough>,
+             H, H>((const H*)a, (const H*)b, (H*)c, M, N, K, sa_m, sa_k, sb_k, sb_n, sc_m, sc_n,
+                   PassThrough{});
+}
+
+void ckref_conv2d_fwd_f32(const float* in, const float* wei, float* out, int N, int K, int C, int Hi,
+                          int Wi, int Y, int X, int Ho, int Wo, int sH, int sW, int dH, int dW, int pH,
+                          int pW)
+{
+    run_conv<float>(in, wei, out, N, K, C, Hi, Wi, Y, X, Ho, Wo, sH, sW, dH, dW, pH, pW);
+}
+
+void ckref_conv2d_fwd_f16(const uint16_t* in, const uint16_t* wei, uint16_t* out, int N, int K, int C,
+                          int Hi, int Wi, int Y, int X, int Ho, int Wo, int sH, int sW, int dH, int dW,
+                          int pH, int pW)
+{
+    using H = ck::half_t;
+    run_conv<H>((const H*)in, (const H*)wei, (H*)out, N, K, C, Hi, Wi, Y, X, Ho, Wo, sH, sW, dH, dW, pH,
+                pW);
+}
+
+void ckref_conv2d_fwd_i8(const int8_t* in, const int8_t* wei, int8_t* out, int N, int K, int C, int Hi,
+                         int Wi, int Y, int X, int Ho, int Wo, int sH, int sW, int dH, int dW, int pH,
+                         int pW)
+{
+    run_conv<int8_t>(in, wei, out, N, K, C, Hi, Wi, Y, X, Ho, Wo, sH, sW, dH, dW, pH, pW);
+}
+
+void ckref_batched_gemm_f16(const uint16_t* a, const uint16_t* b, uint16_t* c, int G, int M, int N,
+                            int K, long sa_g, long sa_m, long sa_k, long sb_g, long sb_k, long sb_n,
+                            long sc_g, long sc_m, long sc_n)
+{
+    using H  = ck::half_t;
+    using sz = std::size_t;
+    auto ta  = make_tensor<H>({(sz)G, (sz)M, (sz)K}, {(sz)sa_g, (sz)sa_m, (sz)sa_k}, (const H*)a);
+    auto tb  = make_tensor<H>({(sz)G, (sz)K, (sz)N}, {(sz)sb_g, (sz)sb_k, (sz)sb_n}, (const H*)b);
+    auto tc  = make_tensor<H>({(sz)G, (sz)M, (sz)N}, {(sz)sc_g, (sz)sc_m, (sz)sc_n}, (const H*)nullptr);
+    using Ref =
+        ck::tensor_operation::host::ReferenceBatchedGemm<H, H, H, PassThrough, PassThrough, PassThrough>;
+    Ref ref;
+    auto inv = ref.MakeInvoker();
+    auto arg = ref.MakeArgument(ta, tb, tc, PassThrough{}, PassThrough{}, PassThrough{});
+    inv.Run(arg);
+    std::memcpy(c, tc.mData.data(), tc.mData.size() * sizeof(H));
+}
+
+int ckref_conv_out_len(int in_len, int filter_len, int stride, int dilation, int pad_left, int pad_right)
+{
+    ck::utils::conv::ConvParams p;
+    p.num_dim_spatial_        = 1;
+    p.filter_spatial_lengths_ = {filter_len};
+    p.input_spatial_lengths_  = {in_len};
+    p.conv_filter_strides_    = {stride};
+    p.conv_filter_dilations_  = {dilation};
+    p.input_left_pads_        = {pad_left};
+    p.input_right_pads_       = {pad_right};
+    return p.GetOutputSpatialLengths()[0];
+}
+
+void ckref_magic_division_params(uint32_t divisor, uint32_t* multiplier, uint32_t* shift)
+{
+    auto t      = ck::MagicDivision::CalculateMagicNumbers(divisor);
+    *multiplier = t[ck::Number<0>{}];
+    *shift      = t[ck::Number<1>{}];
+}
+
+uint32_t ckref_magic_division_divide(uint32_t dividend, uint32_t multiplier, uint32_t shift)
+{
+    return ck::MagicDivision::DoMagicDivision(dividend, multiplier, shift);
+}
+
+} // extern "C"

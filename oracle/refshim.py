@@ -1,0 +1,109 @@
+"""ctypes binding of oracle/_ref/libck_ref.so: the reference's own host operators
+(ReferenceGemm / ReferenceConvFwd / ReferenceBatchedGemm) compiled in place by
+`make -C oracle ref`. Test infrastructure. The file only exists where it was
+built (or travelled with the tree); `load_ref()` returns None otherwise.
+"""
+import ctypes as C
+import os
+import subprocess
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_SO = os.path.join(_HERE, "_ref", "libck_ref.so")
+_REF_TREE = "/root/reference"
+
+
+def build_ref():
+    """Compile the reference host operators where the reference tree is mounted."""
+    if os.path.isdir(os.path.join(_REF_TREE, "library", "include")):
+        subprocess.check_call(["make", "-C", _HERE, "ref"], stdout=subprocess.DEVNULL)
+    return _SO if os.path.exists(_SO) else None
+
+
+def _p(a):
+    return a.ctypes.data_as(C.c_void_p)
+
+
+def _es(a):
+    return [C.c_long(s // a.itemsize) for s in a.strides]
+
+
+class _Ref:
+    def __init__(self, path):
+        self.lib = C.CDLL(path)
+        self.lib.ckref_conv_out_len.restype = C.c_int
+        self.lib.ckref_magic_division_divide.restype = C.c_uint32
+        self.lib.ckref_magic_division_divide.argtypes = [C.c_uint32] * 3
+
+    def gemm_i8_requant(self, a_mk, b_kn, epi, scale_gemm, scale_relu):
+        M, K = a_mk.shape
+        _, N = b_kn.shape
+        c = np.zeros((M, N), np.int8)
+        self.lib.ckref_gemm_i8_requant(_p(a_mk), _p(b_kn), _p(c), M, N, K, *_es(a_mk), *_es(b_kn),
+                                       C.c_long(N), C.c_long(1), int(epi), C.c_float(scale_gemm),
+                                       C.c_float(scale_relu))
+        return c
+
+    def gemm_i8(self, a_mk, b_kn):
+        M, K = a_mk.shape
+        _, N = b_kn.shape
+        c = np.zeros((M, N), np.int8)
+        self.lib.ckref_gemm_i8(_p(a_mk), _p(b_kn), _p(c), M, N, K, *_es(a_mk), *_es(b_kn), C.c_long(N),
+                               C.c_long(1))
+        return c
+
+    def gemm_f16(self, a_mk, b_kn):
+        M, K = a_mk.shape
+        _, N = b_kn.shape
+        c = np.zeros((M, N), np.float16)
+        self.lib.ckref_gemm_f16(_p(a_mk), _p(b_kn), _p(c), M, N, K, *_es(a_mk), *_es(b_kn), C.c_long(N),
+                                C.c_long(1))
+        return c
+
+    def batched_gemm_f16(self, a_gmk, b_gkn):
+        G, M, K = a_gmk.shape
+        _, _, N = b_gkn.shape
+        c = np.zeros((G, M, N), np.float16)
+        self.lib.ckref_batched_gemm_f16(_p(a_gmk), _p(b_gkn), _p(c), G, M, N, K, *_es(a_gmk),
+                                        *_es(b_gkn), C.c_long(M * N), C.c_long(N), C.c_long(1))
+        return c
+
+    def conv2d_fwd(self, inp_nhwc, wei_kyxc, strides=(1, 1), dilations=(1, 1), pads=(0, 0)):
+        inp = np.ascontiguousarray(inp_nhwc)
+        wei = np.ascontiguousarray(wei_kyxc)
+        N, Hi, Wi, Cc = inp.shape
+        K, Y, X, _ = wei.shape
+        Ho = self.conv_out_len(Hi, Y, strides[0], dilations[0], pads[0], pads[0])
+        Wo = self.conv_out_len(Wi, X, strides[1], dilations[1], pads[1], pads[1])
+        out = np.zeros((N, Ho, Wo, K), inp.dtype)
+        fn = {np.dtype(np.float32): self.lib.ckref_conv2d_fwd_f32,
+              np.dtype(np.float16): self.lib.ckref_conv2d_fwd_f16,
+              np.dtype(np.int8): self.lib.ckref_conv2d_fwd_i8}[inp.dtype]
+        fn(_p(inp), _p(wei), _p(out), N, K, Cc, Hi, Wi, Y, X, Ho, Wo, strides[0], strides[1],
+           dilations[0], dilations[1], pads[0], pads[1])
+        return out
+
+    def conv_out_len(self, in_len, filt, stride, dil, pl, pr):
+        return int(self.lib.ckref_conv_out_len(in_len, filt, stride, dil, pl, pr))
+
+    def magic_params(self, d):
+        m, s = C.c_uint32(), C.c_uint32()
+        self.lib.ckref_magic_division_params(C.c_uint32(d), C.byref(m), C.byref(s))
+        return m.value, s.value
+
+    def magic_divide(self, n, mult, shift):
+        return int(self.lib.ckref_magic_division_divide(n, mult, shift))
+
+
+_ref = None
+
+
+def load_ref():
+    global _ref
+    if _ref is None and os.path.exists(_SO):
+        try:
+            _ref = _Ref(_SO)
+        except OSError:
+            _ref = None
+    return _ref

@@ -1,0 +1,328 @@
+"""Pins the CPU oracle (oracle/) before anything is compared against it.
+
+Sources of truth, none of which is the oracle's own formula retyped:
+  * golden vectors the reference's own tests hold (tests/golden/*.json),
+  * the reference's host operators compiled in place (oracle/_ref) when built,
+  * closed forms, exact rational arithmetic, and brute force on tiny inputs.
+"""
+import json
+import os
+
+import numpy as np
+import pytest
+
+import oracle
+from oracle import lit, fast
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+GOLD = json.load(open(os.path.join(HERE, "golden", "reference_conv_fwd_vectors.json")))
+REF = oracle.load_ref()
+needs_ref = pytest.mark.skipif(REF is None, reason="oracle/_ref not built")
+
+
+# ----------------------------------------------------------------- conv golden
+@pytest.mark.parametrize("case", GOLD["cases"])
+def test_conv2d_reference_golden_vectors(case):
+    N, K, C = case["N"], case["K"], case["C"]
+    Hi, Wi = case["input"]
+    Y, X = case["filter"]
+    inp = np.arange(N * Hi * Wi * C, dtype=np.float32).reshape(N, Hi, Wi, C)
+    wei = np.full((K, Y, X, C), 0.5, np.float32)
+    out = lit.conv2d_fwd(inp, wei, case["strides"], case["dilations"], case["left_pads"],
+                         case["right_pads"])
+    n, k, ho, wo = case["out_dims_nkhw"]
+    assert out.shape == (n, ho, wo, k)
+    np.testing.assert_array_equal(out.ravel(), np.array(case["expected"], np.float32))
+    # the numpy im2col form must agree as well (fp32 exact here: small integers and halves)
+    cols, Ho, Wo = fast.im2col(inp, Y, X, case["strides"], case["dilations"], case["left_pads"],
+                               case["right_pads"])
+    np.testing.assert_array_equal((cols @ wei.reshape(K, -1).T).ravel(),
+                                  np.array(case["expected"], np.float32))
+    if REF is not None:
+        np.testing.assert_array_equal(
+            REF.conv2d_fwd(inp, wei, case["strides"], case["dilations"], case["left_pads"]), out)
+
+
+def test_conv_out_len_known_answers():
+    for c in GOLD["conv_out_len_known_answers"]["cases"]:
+        assert lit.conv_out_len(c["in"], c["filter"], c["stride"], c["dilation"], c["pad_l"],
+                                c["pad_r"]) == c["out"]
+        if REF is not None:
+            assert REF.conv_out_len(c["in"], c["filter"], c["stride"], c["dilation"], c["pad_l"],
+                                    c["pad_r"]) == c["out"]
+
+
+# -------------------------------------------------------------- magic division
+def test_magic_division_matches_integer_division():
+    # same sweep as test/magic_number_division/magic_number_division.cpp:59-138
+    rng = np.random.default_rng(1)
+    dividends = np.concatenate([np.arange(0, 5000), rng.integers(0, 2 ** 31 - 1, 3000),
+                                [2 ** 31 - 1, 2 ** 31 - 2, 2 ** 30]]).astype(np.uint64)
+    for d in list(range(1, 4097)) + [65535, 65536, 802816, 2 ** 31 - 1]:
+        m, s = lit.magic_params(d)
+        q = ((dividends * np.uint64(m)) >> np.uint64(32)) + dividends
+        q = (q & np.uint64(0xFFFFFFFF)) >> np.uint64(s)
+        np.testing.assert_array_equal(q, dividends // np.uint64(d), err_msg=f"divisor {d}")
+    for d in (1, 3, 7, 56, 576, 4096):
+        m, s = lit.magic_params(d)
+        for n in (0, 1, d - 1, d, d + 1, 123456789, 2 ** 31 - 1):
+            assert lit.magic_divide(n, m, s) == n // d
+        if REF is not None:
+            assert REF.magic_params(d) == (m, s)
+
+
+# ------------------------------------------------------------ fp16 conversions
+def test_half_conversions_match_ieee():
+    L = lit.lib()
+    allh = np.arange(65536, dtype=np.uint16)
+    want = allh.view(np.float16).astype(np.float32)
+    got = np.array([L.cko_half_to_float(int(h)) for h in allh], np.float32)
+    fin = np.isfinite(want)
+    np.testing.assert_array_equal(got[fin], want[fin])
+    assert np.all(np.isnan(got[np.isnan(want)]))
+    np.testing.assert_array_equal(got[np.isinf(want)], want[np.isinf(want)])
+    rng = np.random.default_rng(2)
+    f = np.concatenate([
+        rng.uniform(-70000, 70000, 4000), rng.uniform(-1, 1, 4000), rng.uniform(-1e-4, 1e-4, 4000),
+        rng.uniform(-1e-7, 1e-7, 2000),
+        # exact ties between neighbouring halves
+        (allh[1:30000:7].view(np.float16).astype(np.float64)
+         + allh[2:30001:7].view(np.float16).astype(np.float64)) / 2,
+        [65504, 65519.99, 65520, 65536, 5.9604645e-08, 2.9802322e-08, 2.98023224e-08 * 1.0000001, 0.0]
+    ]).astype(np.float32)
+    want16 = f.astype(np.float16).view(np.uint16)
+    got16 = np.array([L.cko_float_to_half(float(x)) for x in f], np.uint16)
+    np.testing.assert_array_equal(got16, want16)
+
+
+# ------------------------------------------------------------------- epilogue
+def _epilogue_exact(acc, epi, sg, sr):
+    """Independent derivation: a float32 x float32 product is exact in float64, so one
+    float64 multiply followed by one rounding to float32 equals the IEEE fp32 multiply."""
+    if epi == lit.EPI_PASSTHROUGH:
+        return ((acc + 128) % 256) - 128
+    sg, sr = np.float32(sg), np.float32(sr)
+    x = np.float32(acc)
+    assert float(x) == acc
+    g = np.float32(np.float64(sg) * np.float64(x))
+    if epi == lit.EPI_REQUANT_CK:
+        r = g if g > 0 else np.float32(0)
+        q = np.float32(np.float64(sr) * np.float64(r))
+        y = min(max(float(q), -128.0), 127.0)
+        return int(y)  # toward zero
+    t = float(round(float(g)))  # Python round() is half-to-even on an exact binary value
+    t = min(max(t, -128.0), 127.0)
+    r = max(t, 0.0)
+    u = float(round(float(np.float32(np.float64(sr) * np.float64(np.float32(r))))))
+    return int(min(max(u, -128.0), 127.0))
+
+
+@pytest.mark.parametrize("epi,sg,sr", [
+    (lit.EPI_REQUANT_CK, 0.03, 1.0), (lit.EPI_REQUANT_RND, 0.5, 0.03), (lit.EPI_REQUANT_RND, 0.02, 0.4),
+    (lit.EPI_REQUANT_CK, 0.5, 0.03), (lit.EPI_REQUANT_RND, 0.03, 1.0), (lit.EPI_PASSTHROUGH, 1.0, 1.0),
+])
+def test_epilogue_scalar_against_exact_arithmetic(epi, sg, sr):
+    rng = np.random.default_rng(3)
+    accs = list(range(-700, 9000)) + [int(v) for v in rng.integers(-2 ** 20, 2 ** 20, 4000)] + \
+        [2 ** 24 - 1, -(2 ** 24 - 1), 704512, -704512]
+    for acc in accs:
+        assert lit.epilogue_i8(acc, epi, sg, sr) == _epilogue_exact(acc, epi, sg, sr), (acc, epi)
+    arr = np.array(accs, np.int32)
+    np.testing.assert_array_equal(fast.epilogue_i8(arr, epi, sg, sr),
+                                  np.array([lit.epilogue_i8(a, epi, sg, sr) for a in accs], np.int8))
+
+
+def test_epilogue_special_cases():
+    R, Cc = lit.EPI_REQUANT_RND, lit.EPI_REQUANT_CK
+    # ties go to even with scale 0.5
+    assert [lit.epilogue_i8(a, R, 0.5, 1.0) for a in (1, 3, 5, 7, 2, 254, 255, 256, 1000)] == \
+        [0, 2, 2, 4, 1, 127, 127, 127, 127]
+    # negative accumulators die in the ReLU
+    assert all(lit.epilogue_i8(a, m, 0.5, 0.03) == 0 for a in (-1, -77, -10 ** 6) for m in (R, Cc))
+    # literal functor truncates toward zero instead of rounding: 0.03*66 = 1.98 -> 1
+    assert lit.epilogue_i8(66, Cc, 0.03, 1.0) == 1
+    assert lit.epilogue_i8(66, R, 0.03, 1.0) == 2
+    assert lit.epilogue_i8(10 ** 6, Cc, 0.03, 1.0) == 127
+    # inner saturation is visible in the rounded mode: 0.5*400=200 -> 127 -> *0.5 = 63.5 -> 64
+    assert lit.epilogue_i8(400, R, 0.5, 0.5) == 64
+    # passthrough keeps the low byte
+    assert [lit.epilogue_i8(a, lit.EPI_PASSTHROUGH, 1, 1) for a in (14400, -300, 255, 128)] == \
+        [64, -44, -1, -128]
+
+
+# ----------------------------------------------------------------------- GEMM
+def _rand_i8(rng, shape, lo=-5, hi=5):
+    return rng.integers(lo, hi + 1, shape).astype(np.int8)
+
+
+def test_gemm_i8_closed_forms():
+    M, N, K = 7, 9, 40
+    ones_a, ones_b = np.ones((M, K), np.int8), np.ones((K, N), np.int8)
+    np.testing.assert_array_equal(lit.gemm_i8_acc(ones_a, ones_b), np.full((M, N), K, np.int32))
+    a = np.repeat(np.arange(M, dtype=np.int8)[:, None], K, 1)   # A(m,k) = m
+    b = np.repeat(np.arange(N, dtype=np.int8)[None, :], K, 0)   # B(k,n) = n
+    want = K * np.arange(M)[:, None] * np.arange(N)[None, :]
+    np.testing.assert_array_equal(lit.gemm_i8_acc(a, b), want)
+    # int32 accumulate + PassThrough keeps the low byte; float accumulate agrees
+    np.testing.assert_array_equal(lit.gemm_i8(a, b), (want & 0xFF).astype(np.uint8).view(np.int8))
+    np.testing.assert_array_equal(lit.gemm_i8(a, b, acc_float=True),
+                                  (want & 0xFF).astype(np.uint8).view(np.int8))
+    # identity B
+    rng = np.random.default_rng(4)
+    a = _rand_i8(rng, (5, 6), -128, 127)
+    np.testing.assert_array_equal(lit.gemm_i8(a, np.eye(6, dtype=np.int8)), a)
+
+
+def test_gemm_i8_brute_force_and_layouts():
+    rng = np.random.default_rng(5)
+    M, N, K = 6, 5, 33
+    a = _rand_i8(rng, (M, K), -128, 127)
+    b_nk = _rand_i8(rng, (N, K), -128, 127)          # column-major B: K contiguous
+    want = np.zeros((M, N), np.int64)
+    for m in range(M):
+        for n in range(N):
+            for k in range(K):
+                want[m, n] += int(a[m, k]) * int(b_nk[n, k])
+    np.testing.assert_array_equal(lit.gemm_i8_acc(a, b_nk.T), want)
+    # row-major B gives the same through different strides
+    np.testing.assert_array_equal(lit.gemm_i8_acc(a, np.ascontiguousarray(b_nk.T)), want)
+    # column-major A
+    np.testing.assert_array_equal(lit.gemm_i8_acc(np.asfortranarray(a), b_nk.T), want)
+    # transposition symmetry C(A,B)^T = C(B^T, A^T)
+    np.testing.assert_array_equal(lit.gemm_i8_acc(b_nk, a.T), want.T)
+
+
+@pytest.mark.parametrize("epi,sg,sr", [(lit.EPI_REQUANT_CK, 0.03, 1.0), (lit.EPI_REQUANT_RND, 0.5, 0.03),
+                                       (lit.EPI_REQUANT_RND, 0.02, 0.4), (lit.EPI_PASSTHROUGH, 1, 1)])
+def test_gemm_i8_lit_fast_ref_agree(epi, sg, sr):
+    rng = np.random.default_rng(6)
+    for (M, N, K, lo, hi) in [(64, 48, 80, -5, 5), (33, 17, 1024, -8, 8), (1, 130, 256, -5, 5)]:
+        a = _rand_i8(rng, (M, K), lo, hi)
+        b_nk = _rand_i8(rng, (N, K), lo, hi)
+        c_lit = lit.gemm_i8(a, b_nk.T, epi, sg, sr)
+        np.testing.assert_array_equal(fast.gemm_i8(a, b_nk.T, epi, sg, sr), c_lit)
+        # epilogue of the exact accumulators, element by element, through the exact-arithmetic form
+        acc = lit.gemm_i8_acc(a, b_nk.T)
+        idx = rng.integers(0, acc.size, 200)
+        for i in idx:
+            assert c_lit.ravel()[i] == _epilogue_exact(int(acc.ravel()[i]), epi, sg, sr)
+        if REF is not None:
+            if epi == lit.EPI_PASSTHROUGH:
+                np.testing.assert_array_equal(REF.gemm_i8(a, b_nk.T), c_lit)
+            else:
+                np.testing.assert_array_equal(REF.gemm_i8_requant(a, b_nk.T, epi, sg, sr), c_lit)
+
+
+def test_gemm_i8_thread_count_is_unobservable():
+    rng = np.random.default_rng(7)
+    a, b = _rand_i8(rng, (37, 64)), _rand_i8(rng, (64, 29))
+    c1 = lit.gemm_i8(a, b, lit.EPI_REQUANT_RND, 0.5, 0.03, nthreads=1)
+    for t in (2, 3, 8, 64):
+        np.testing.assert_array_equal(lit.gemm_i8(a, b, lit.EPI_REQUANT_RND, 0.5, 0.03, nthreads=t), c1)
+
+
+def test_gemm_f16_against_float64_and_ref():
+    rng = np.random.default_rng(8)
+    M, N, K = 24, 40, 96
+    a = rng.uniform(-1, 1, (M, K)).astype(np.float16)
+    b_nk = rng.uniform(-1, 1, (N, K)).astype(np.float16)
+    c = lit.gemm_f16(a, b_nk.T)
+    # sequential fp32 summation restated independently with numpy scalars
+    want = np.zeros((M, N), np.float16)
+    for m in range(M):
+        for n in range(N):
+            acc = np.float32(0)
+            for k in range(K):
+                acc = np.float32(acc + np.float32(a[m, k]) * np.float32(b_nk[n, k]))
+            want[m, n] = np.float16(acc)
+    np.testing.assert_array_equal(c.view(np.uint16), want.view(np.uint16))
+    exact = a.astype(np.float64) @ b_nk.T.astype(np.float64)
+    assert np.max(np.abs(c.astype(np.float64) - exact)) < 2e-2
+    bad, _ = lit.check_err_f16(fast.gemm_f16(a, b_nk.T), c, 1e-3, 1e-3)
+    assert bad == 0
+    if REF is not None:
+        np.testing.assert_array_equal(REF.gemm_f16(a, b_nk.T).view(np.uint16), c.view(np.uint16))
+    # closed form: all ones -> K (exact in fp16 for K <= 2048)
+    np.testing.assert_array_equal(lit.gemm_f16(np.ones((3, 512), np.float16), np.ones((512, 4), np.float16)),
+                                  np.full((3, 4), 512, np.float16))
+
+
+def test_batched_gemm_and_gemm_gemm():
+    rng = np.random.default_rng(9)
+    G, M, K, N, O = 3, 10, 16, 12, 8
+    a = rng.uniform(-0.5, 0.5, (G, M, K)).astype(np.float16)
+    b0_gnk = rng.uniform(-0.5, 0.5, (G, N, K)).astype(np.float16)   # column-major K x N per batch
+    b1 = rng.uniform(-0.5, 0.5, (G, N, O)).astype(np.float16)
+    b0 = b0_gnk.transpose(0, 2, 1)
+    s = lit.batched_gemm_f16(a, b0)
+    for g in range(G):   # batch independence + equality with the plain GEMM oracle
+        np.testing.assert_array_equal(s[g].view(np.uint16), lit.gemm_f16(a[g], b0[g]).view(np.uint16))
+    if REF is not None:
+        np.testing.assert_array_equal(REF.batched_gemm_f16(a, b0).view(np.uint16), s.view(np.uint16))
+    c = lit.batched_gemm_gemm_f16(a, b0, b1)
+    # brute force with an fp16 intermediate
+    want = np.zeros((G, M, O), np.float16)
+    for g in range(G):
+        for m in range(M):
+            for o in range(O):
+                acc = np.float32(0)
+                for n in range(N):
+                    acc = np.float32(acc + np.float32(s[g, m, n]) * np.float32(b1[g, n, o]))
+                want[g, m, o] = np.float16(acc)
+    np.testing.assert_array_equal(c.view(np.uint16), want.view(np.uint16))
+    if REF is not None:
+        np.testing.assert_array_equal(REF.batched_gemm_f16(s, b1).view(np.uint16), c.view(np.uint16))
+    bad, _ = lit.check_err_f16(fast.batched_gemm_gemm_f16(a, b0, b1), c, 1e-2, 1e-2)
+    assert bad == 0
+    # closed form: ones -> K then N*K
+    one = np.ones
+    np.testing.assert_array_equal(
+        lit.batched_gemm_gemm_f16(one((1, 2, 4), np.float16), one((1, 4, 8), np.float16),
+                                  one((1, 8, 3), np.float16)), np.full((1, 2, 3), 32, np.float16))
+
+
+# ----------------------------------------------------------------------- conv
+@pytest.mark.parametrize("dtype", [np.float16, np.int8])
+def test_conv2d_lit_fast_ref_agree(dtype):
+    rng = np.random.default_rng(10)
+    for (N, C, K, Hi, Wi, Y, X, s, d, p) in [(2, 8, 16, 5, 6, 3, 3, (2, 1), (1, 2), (1, 2)),
+                                             (1, 16, 4, 7, 7, 1, 1, (2, 2), (1, 1), (0, 0)),
+                                             (2, 3, 5, 9, 8, 3, 2, (1, 1), (1, 1), (1, 0))]:
+        if dtype == np.int8:
+            inp = _rand_i8(rng, (N, Hi, Wi, C))
+            wei = _rand_i8(rng, (K, Y, X, C))
+        else:
+            inp = rng.uniform(-1, 1, (N, Hi, Wi, C)).astype(np.float16)
+            wei = rng.uniform(-1, 1, (K, Y, X, C)).astype(np.float16)
+        out = lit.conv2d_fwd(inp, wei, s, d, p)
+        if dtype == np.int8:
+            np.testing.assert_array_equal(fast.conv2d_fwd_i8(inp, wei, s, d, p), out)
+            # the requant functor as OutElementOp
+            o2 = lit.conv2d_fwd(inp, wei, s, d, p, epi=lit.EPI_REQUANT_RND, scale_gemm=0.5, scale_relu=0.3)
+            np.testing.assert_array_equal(
+                fast.conv2d_fwd_i8(inp, wei, s, d, p, epi=lit.EPI_REQUANT_RND, scale_gemm=0.5,
+                                   scale_relu=0.3), o2)
+        else:
+            bad, _ = lit.check_err_f16(fast.conv2d_fwd_f16(inp, wei, s, d, p), out, 1e-3, 1e-3)
+            assert bad == 0
+        if REF is not None:
+            np.testing.assert_array_equal(REF.conv2d_fwd(inp, wei, s, d, p).view(np.uint8),
+                                          out.view(np.uint8))
+
+
+def test_conv2d_int8_passthrough_wraps_modulo_256():
+    # the reference's int8 conv keeps the low byte of an out-of-range sum
+    inp = np.full((1, 4, 4, 16), 5, np.int8)
+    wei = np.full((2, 3, 3, 16), 5, np.int8)
+    out = lit.conv2d_fwd(inp, wei, pads=(0, 0))
+    assert out.shape == (1, 2, 2, 2)
+    total = 25 * 9 * 16   # 3600
+    assert int(out[0, 0, 0, 0]) == ((total + 128) % 256) - 128
+
+
+def test_conv2d_is_a_gemm_for_1x1():
+    rng = np.random.default_rng(11)
+    inp = _rand_i8(rng, (2, 4, 5, 32))
+    wei = _rand_i8(rng, (8, 1, 1, 32))
+    out = lit.conv2d_fwd(inp, wei)
+    np.testing.assert_array_equal(out.reshape(-1, 8), lit.gemm_i8(inp.reshape(-1, 32), wei.reshape(8, 32).T))
