@@ -1,0 +1,13 @@
+"""MI355X-native MFMA GEMM hot path behind Composable Kernel's device-operator surface.
+
+    csrc/        HIP kernels for gfx950 + the C ABI (include/ckx.h) -> lib/libckx.so
+    host/        C++ operator classes, instance factory, ckx_profiler driver
+    capi.py      ctypes binding of the C ABI
+    device_ops.py  Python mirror of DeviceGemm / DeviceConvFwd / DeviceBatchedGemmGemm
+    host_tensor.py seeded generators for synthetic inputs
+"""
+from . import capi, device_ops, host_tensor  # noqa: F401
+from .device_ops import (  # noqa: F401
+    PassThrough, RequantReluRequant, RowMajor, ColumnMajor, StreamConfig,
+    DeviceGemmInt8, DeviceGemmF16, DeviceConv2dFwdInt8, DeviceConv2dFwdF16, DeviceBatchedGemmGemmF16,
+)

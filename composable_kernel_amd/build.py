@@ -1,0 +1,55 @@
+"""Builds libckx.so (HIP kernels + C ABI) for gfx950 with hipcc, in-tree.
+
+    python -m composable_kernel_amd.build [--force]
+
+Flags: -ffp-contract=off keeps the requant epilogue's fp32 multiplies unfused;
+packed fp32 VALU forms are disabled for the device pass.
+"""
+import os
+import subprocess
+import sys
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+ROOT = os.path.dirname(HERE)
+CSRC = os.path.join(HERE, "csrc")
+LIBDIR = os.path.join(HERE, "lib")
+LIB = os.path.join(LIBDIR, "libckx.so")
+HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
+
+DEVICE_FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-ffp-contract=off",
+                "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+                "-Wno-unused-command-line-argument"]
+
+
+def sources():
+    return [os.path.join(CSRC, f) for f in sorted(os.listdir(CSRC))]
+
+
+def stale():
+    if not os.path.exists(LIB):
+        return True
+    t = os.path.getmtime(LIB)
+    deps = sources() + [os.path.join(ROOT, "include", "ckx.h")]
+    return any(os.path.getmtime(p) > t for p in deps)
+
+
+def build_lib(force=False, verbose=False, extra_flags=()):
+    """Compile csrc/*.hip into lib/libckx.so. Returns the library path."""
+    if not force and not stale():
+        return LIB
+    os.makedirs(LIBDIR, exist_ok=True)
+    cmd = [HIPCC] + DEVICE_FLAGS + list(extra_flags) + ["-fPIC", "-shared", "-I" + os.path.join(ROOT, "include"),
+                                                        "-I" + CSRC, os.path.join(CSRC, "ckx_api.hip"), "-o", LIB]
+    if verbose:
+        print(" ".join(cmd))
+    r = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    out = "\n".join(l for l in r.stdout.splitlines() if "packed-fp32-ops" not in l)
+    if r.returncode != 0:
+        raise RuntimeError("hipcc failed:\n" + out)
+    if verbose and out.strip():
+        print(out)
+    return LIB
+
+
+if __name__ == "__main__":
+    print(build_lib(force="--force" in sys.argv, verbose=True))

@@ -1,0 +1,91 @@
+"""ctypes binding of libckx.so -- the C ABI declared in include/ckx.h.
+
+The library is loaded from composable_kernel_amd/lib/ (built in-tree by
+composable_kernel_amd.build). There is no fallback: if it is missing, loading
+raises, and every operator raises with it.
+"""
+import ctypes as C
+import os
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(HERE, "lib", "libckx.so")
+
+OK, UNSUPPORTED, INVALID_VALUE, HIP_ERROR = 0, -1, -2, -3
+ROW_MAJOR, COL_MAJOR = 0, 1
+EPI_PASSTHROUGH, EPI_REQUANT_CK, EPI_REQUANT_RND = 0, 1, 2
+OP_GEMM_I8, OP_GEMM_F16, OP_CONV2D_FWD_I8, OP_CONV2D_FWD_F16, OP_BATCHED_GEMM_GEMM = range(5)
+INSTANCE_AUTO = -1
+
+# every symbol include/ckx.h declares
+SYMBOLS = [
+    "ckx_version", "ckx_last_error", "ckx_num_instances", "ckx_instance_name",
+    "ckx_gemm_i8_is_supported", "ckx_gemm_i8", "ckx_gemm_f16_is_supported", "ckx_gemm_f16",
+    "ckx_conv2d_fwd_is_supported", "ckx_conv2d_fwd_i8", "ckx_conv2d_fwd_f16",
+    "ckx_batched_gemm_gemm_f16_is_supported", "ckx_batched_gemm_gemm_f16", "ckx_time_launches",
+]
+
+
+class Conv2dDesc(C.Structure):
+    _fields_ = [(n, C.c_int32) for n in (
+        "N", "K", "C", "Hi", "Wi", "Y", "X", "Ho", "Wo", "stride_h", "stride_w", "dilation_h",
+        "dilation_w", "pad_top", "pad_left", "pad_bottom", "pad_right")]
+
+
+LAUNCH_FN = C.CFUNCTYPE(C.c_int, C.c_void_p)
+
+_lib = None
+
+
+class CkxError(RuntimeError):
+    def __init__(self, status, msg):
+        super().__init__(f"ckx status {status}: {msg}")
+        self.status = status
+
+
+def lib():
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise FileNotFoundError(
+            f"{LIB_PATH} is missing: build it with `python -m composable_kernel_amd.build` "
+            "(there is no CPU fallback)")
+    L = C.CDLL(LIB_PATH)
+    i32, f32, vp, i64 = C.c_int32, C.c_float, C.c_void_p, C.c_int64
+    L.ckx_version.restype = C.c_char_p
+    L.ckx_last_error.restype = C.c_char_p
+    L.ckx_num_instances.argtypes = [C.c_int]
+    L.ckx_instance_name.restype = C.c_char_p
+    L.ckx_instance_name.argtypes = [C.c_int, C.c_int]
+    shape = [i32] * 6 + [C.c_int] * 3
+    L.ckx_gemm_i8_is_supported.argtypes = shape + [C.c_int, C.c_int]
+    L.ckx_gemm_i8.argtypes = [vp, vp, vp] + shape + [C.c_int, f32, f32, C.c_int, vp]
+    L.ckx_gemm_f16_is_supported.argtypes = shape + [C.c_int]
+    L.ckx_gemm_f16.argtypes = [vp, vp, vp] + shape + [C.c_int, vp]
+    dp = C.POINTER(Conv2dDesc)
+    L.ckx_conv2d_fwd_is_supported.argtypes = [C.c_int, dp, C.c_int, C.c_int]
+    L.ckx_conv2d_fwd_i8.argtypes = [vp, vp, vp, dp, C.c_int, f32, f32, C.c_int, vp]
+    L.ckx_conv2d_fwd_f16.argtypes = [vp, vp, vp, dp, C.c_int, vp]
+    gg = [i32] * 9 + [i64] * 4 + [C.c_int]
+    L.ckx_batched_gemm_gemm_f16_is_supported.argtypes = gg
+    L.ckx_batched_gemm_gemm_f16.argtypes = [vp] * 4 + gg + [vp]
+    L.ckx_time_launches.argtypes = [LAUNCH_FN, vp, C.c_int, C.c_int, vp, C.POINTER(C.c_float)]
+    _lib = L
+    return L
+
+
+def last_error():
+    return lib().ckx_last_error().decode()
+
+
+def check(status):
+    if status != OK:
+        raise CkxError(status, last_error())
+
+
+def time_launches(fn, n_warmup, n_repeat, stream):
+    """Mean milliseconds of `fn()` (which must enqueue on `stream` and return a ckx status)."""
+    ms = C.c_float()
+    cb = LAUNCH_FN(lambda _u: int(fn()))
+    check(lib().ckx_time_launches(cb, None, int(n_warmup), int(n_repeat), C.c_void_p(stream or 0), C.byref(ms)))
+    return float(ms.value)

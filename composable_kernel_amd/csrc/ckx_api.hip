@@ -1,0 +1,399 @@
+// C ABI of the library (declared in include/ckx.h): argument validation, instance
+// selection and kernel launch. No allocation, no synchronisation, no CPU fallback: a
+// request no kernel instance covers is reported as CKX_UNSUPPORTED.
+#include <hip/hip_runtime.h>
+
+#include <cstdio>
+#include <cstring>
+#include <mutex>
+#include <string>
+
+#include "ckx.h"
+#include "gemm_tile.hpp"
+#include "gemm_gemm.hpp"
+
+namespace {
+
+thread_local std::string g_last_error;
+
+int fail(int code, const std::string& msg)
+{
+    g_last_error = msg;
+    return code;
+}
+
+int hip_fail(hipError_t e, const char* what)
+{
+    return fail(CKX_HIP_ERROR, std::string(what) + ": " + hipGetErrorString(e));
+}
+
+ckx::MagicDiv make_magic(uint32_t d)
+{
+    // include/ck/utility/magic_division.hpp:28-54
+    uint32_t shift = 0;
+    while(shift < 32 && (1ull << shift) < d)
+        ++shift;
+    const uint64_t one = 1;
+    ckx::MagicDiv m;
+    m.mul   = (uint32_t)(((one << 32) * ((one << shift) - d)) / d + 1);
+    m.shift = shift;
+    m.d     = d;
+    return m;
+}
+
+// ------------------------------------------------------------ tile instances
+typedef hipError_t (*tile_launch_fn)(const ckx::GemmArgs&, int grid, hipStream_t);
+
+template <int DT, int BM, int BN, int WM, int WN, bool IM2COL>
+hipError_t launch_tile(const ckx::GemmArgs& a, int grid, hipStream_t s)
+{
+    using T              = ckx::GemmTile<DT, BM, BN, WM, WN, IM2COL>;
+    auto* kern           = &ckx::gemm_tile_kernel<DT, BM, BN, WM, WN, IM2COL>;
+    static std::once_flag once;
+    static hipError_t attr_err = hipSuccess;
+    std::call_once(once, [&] {
+        attr_err = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, T::LDS);
+    });
+    if(attr_err != hipSuccess)
+        return attr_err;
+    hipLaunchKernelGGL(kern, dim3(grid), dim3(T::NT), T::LDS, s, a);
+    return hipGetLastError();
+}
+
+struct TileInstance
+{
+    const char* name;
+    int bm, bn, threads;
+    tile_launch_fn dense_i8, dense_f16, conv_i8, conv_f16;
+};
+
+#define CKX_TILE(BM, BN, WM, WN)                                                                      \
+    {                                                                                                 \
+        "MI355X_Mfma16_Tile<" #BM ", " #BN ", 128B, waves " #WM "x" #WN ">", BM, BN, WM* WN * 64,          \
+            &launch_tile<ckx::DT_I8, BM, BN, WM, WN, false>, &launch_tile<ckx::DT_F16, BM, BN, WM, WN, false>, \
+            &launch_tile<ckx::DT_I8, BM, BN, WM, WN, true>, &launch_tile<ckx::DT_F16, BM, BN, WM, WN, true>    \
+    }
+
+const TileInstance kTiles[] = {
+    CKX_TILE(256, 256, 2, 4),
+    CKX_TILE(256, 128, 4, 2),
+    CKX_TILE(128, 128, 2, 2),
+    CKX_TILE(128, 64, 4, 1),
+    CKX_TILE(64, 64, 4, 1),
+    CKX_TILE(32, 64, 2, 1),
+    CKX_TILE(16, 64, 1, 1),
+    CKX_TILE(256, 256, 2, 2),
+};
+constexpr int kNumTiles = sizeof(kTiles) / sizeof(kTiles[0]);
+
+// Pick the largest tile that still yields enough workgroups to occupy 256 CUs.
+int pick_tile(int M, int N)
+{
+    auto tiles = [&](int i) {
+        return (long)((M + kTiles[i].bm - 1) / kTiles[i].bm) * ((N + kTiles[i].bn - 1) / kTiles[i].bn);
+    };
+    const int order[] = {0, 1, 2, 3, 4, 5, 6};
+    for(int i : order)
+    {
+        if(kTiles[i].bm > 16 && M <= kTiles[i].bm / 2)
+            continue; // more than half of the tile rows would be padding
+        if(tiles(i) >= 224)
+            return i;
+    }
+    // nothing fills the machine: smallest tile that is not mostly padding
+    for(int i = 6; i >= 0; --i)
+        if(M >= kTiles[i].bm || i == 6)
+            return i;
+    return 6;
+}
+
+const char* family_prefix(int op)
+{
+    switch(op)
+    {
+    case CKX_OP_GEMM_I8: return "DeviceGemm_i8_i8_i8_mk_nk_mn";
+    case CKX_OP_GEMM_F16: return "DeviceGemm_f16_f16_f16_mk_nk_mn";
+    case CKX_OP_CONV2D_FWD_I8: return "DeviceConv2dFwd_i8_nhwc_kyxc_nhwk";
+    case CKX_OP_CONV2D_FWD_F16: return "DeviceConv2dFwd_f16_nhwc_kyxc_nhwk";
+    case CKX_OP_BATCHED_GEMM_GEMM: return "DeviceBatchedGemmGemm_f16_gmk_gnk_gno_gmo";
+    default: return nullptr;
+    }
+}
+
+int check_gemm_shape(int dt, int M, int N, int K, int sa, int sb, int sc, int al, int bl, int cl, int epi,
+                     int instance)
+{
+    const int es = dt == ckx::DT_I8 ? 1 : 2;
+    if(M < 0 || N < 0 || K < 0)
+        return fail(CKX_INVALID_VALUE, "negative GEMM dimension");
+    if(instance != CKX_INSTANCE_AUTO && (instance < 0 || instance >= kNumTiles))
+        return fail(CKX_INVALID_VALUE, "no such instance");
+    if(epi < CKX_EPI_PASSTHROUGH || epi > CKX_EPI_REQUANT_RND)
+        return fail(CKX_INVALID_VALUE, "unknown epilogue");
+    if(dt == ckx::DT_F16 && epi != CKX_EPI_PASSTHROUGH)
+        return fail(CKX_UNSUPPORTED, "fp16 GEMM only has the PassThrough epilogue");
+    if(al != CKX_ROW_MAJOR || bl != CKX_COL_MAJOR || cl != CKX_ROW_MAJOR)
+        return fail(CKX_UNSUPPORTED, "only A row-major, B column-major, C row-major (mk_nk_mn) is built");
+    if(sa < K || sb < K || sc < N)
+        return fail(CKX_UNSUPPORTED, "stride smaller than the contiguous extent");
+    if(((long)K * es) % 16 || ((long)sa * es) % 16 || ((long)sb * es) % 16)
+        return fail(CKX_UNSUPPORTED, "K and the A/B strides must be multiples of 16 bytes");
+    if((long)M * sa * es >= (1l << 31) || (long)N * sb * es >= (1l << 31) || (long)M * sc * es >= (1l << 31))
+        return fail(CKX_UNSUPPORTED, "operands of 2 GiB or more are not addressed");
+    return CKX_OK;
+}
+
+int run_gemm(int dt, const void* a, const void* b, void* c, int M, int N, int K, int sa, int sb, int sc,
+             int al, int bl, int cl, int epi, float sg, float sr, int instance, void* stream)
+{
+    int st = check_gemm_shape(dt, M, N, K, sa, sb, sc, al, bl, cl, epi, instance);
+    if(st != CKX_OK)
+        return st;
+    if(M == 0 || N == 0)
+        return CKX_OK;
+    if(!a || !b || !c)
+        return fail(CKX_INVALID_VALUE, "null operand pointer");
+    if((reinterpret_cast<uintptr_t>(a) | reinterpret_cast<uintptr_t>(b)) & 15)
+        return fail(CKX_UNSUPPORTED, "A and B must be 16-byte aligned");
+    const int es = dt == ckx::DT_I8 ? 1 : 2;
+    const int ti = instance == CKX_INSTANCE_AUTO ? pick_tile(M, N) : instance;
+    const TileInstance& t = kTiles[ti];
+    ckx::GemmArgs g;
+    std::memset(&g, 0, sizeof(g));
+    g.a = a, g.b = b, g.c = c;
+    g.M = M, g.N = N, g.K = K;
+    g.lda = sa, g.ldb = sb, g.ldc = sc;
+    g.a_bytes    = (uint32_t)(((long)(M - 1) * sa + K) * es);
+    g.b_bytes    = (uint32_t)(((long)(N - 1) * sb + K) * es);
+    g.tiles_m    = (M + t.bm - 1) / t.bm;
+    g.tiles_n    = (N + t.bn - 1) / t.bn;
+    g.epi        = epi;
+    g.scale_gemm = sg;
+    g.scale_relu = sr;
+    hipError_t e = (dt == ckx::DT_I8 ? t.dense_i8 : t.dense_f16)(g, g.tiles_m * g.tiles_n, (hipStream_t)stream);
+    if(e != hipSuccess)
+        return hip_fail(e, t.name);
+    return CKX_OK;
+}
+
+int check_conv(int op, const ckx_conv2d_desc* d, int epi, int instance)
+{
+    if(!d)
+        return fail(CKX_INVALID_VALUE, "null conv descriptor");
+    if(op != CKX_OP_CONV2D_FWD_I8 && op != CKX_OP_CONV2D_FWD_F16)
+        return fail(CKX_INVALID_VALUE, "not a conv operator family");
+    const int es = op == CKX_OP_CONV2D_FWD_I8 ? 1 : 2;
+    if(instance != CKX_INSTANCE_AUTO && (instance < 0 || instance >= kNumTiles))
+        return fail(CKX_INVALID_VALUE, "no such instance");
+    if(epi < CKX_EPI_PASSTHROUGH || epi > CKX_EPI_REQUANT_RND || (es == 2 && epi != CKX_EPI_PASSTHROUGH))
+        return fail(CKX_INVALID_VALUE, "epilogue not available for this dtype");
+    if(d->N < 0 || d->K < 0 || d->C < 0 || d->Hi <= 0 || d->Wi <= 0 || d->Y <= 0 || d->X <= 0 ||
+       d->Ho < 0 || d->Wo < 0 || d->stride_h <= 0 || d->stride_w <= 0 || d->dilation_h <= 0 ||
+       d->dilation_w <= 0 || d->pad_top < 0 || d->pad_left < 0 || d->pad_bottom < 0 || d->pad_right < 0)
+        return fail(CKX_INVALID_VALUE, "bad conv geometry");
+    // the output extent has to be what the geometry implies (conv_util.cpp:103-114)
+    const int ho = (d->Hi + d->pad_top + d->pad_bottom - ((d->Y - 1) * d->dilation_h + 1)) / d->stride_h + 1;
+    const int wo = (d->Wi + d->pad_left + d->pad_right - ((d->X - 1) * d->dilation_w + 1)) / d->stride_w + 1;
+    if(ho != d->Ho || wo != d->Wo)
+        return fail(CKX_UNSUPPORTED, "output spatial lengths do not match the conv geometry");
+    // a 16-byte vector along c must not cross a filter tap
+    // (device_conv2d_fwd_xdl_nhwc_kyxc_nhwk.hpp:595-601)
+    if(((long)d->C * es) % 16)
+        return fail(CKX_UNSUPPORTED, "C must be a multiple of 16 bytes");
+    const long in_b  = (long)d->N * d->Hi * d->Wi * d->C * es;
+    const long wei_b = (long)d->K * d->Y * d->X * d->C * es;
+    const long out_b = (long)d->N * d->Ho * d->Wo * d->K * es;
+    if(in_b >= (1l << 31) || wei_b >= (1l << 31) || out_b >= (1l << 31) ||
+       (long)d->N * d->Ho * d->Wo >= (1l << 31))
+        return fail(CKX_UNSUPPORTED, "tensors of 2 GiB or more are not addressed");
+    return CKX_OK;
+}
+
+int run_conv(int op, const void* in, const void* wei, void* out, const ckx_conv2d_desc* d, int epi, float sg,
+             float sr, int instance, void* stream)
+{
+    int st = check_conv(op, d, epi, instance);
+    if(st != CKX_OK)
+        return st;
+    const int es = op == CKX_OP_CONV2D_FWD_I8 ? 1 : 2;
+    const int M = d->N * d->Ho * d->Wo, N = d->K, K = d->Y * d->X * d->C;
+    if(M == 0 || N == 0)
+        return CKX_OK;
+    if(!in || !wei || !out)
+        return fail(CKX_INVALID_VALUE, "null operand pointer");
+    if((reinterpret_cast<uintptr_t>(in) | reinterpret_cast<uintptr_t>(wei)) & 15)
+        return fail(CKX_UNSUPPORTED, "input and weight must be 16-byte aligned");
+    const int ti = instance == CKX_INSTANCE_AUTO ? pick_tile(M, N) : instance;
+    const TileInstance& t = kTiles[ti];
+    ckx::GemmArgs g;
+    std::memset(&g, 0, sizeof(g));
+    g.a = in, g.b = wei, g.c = out;
+    g.M = M, g.N = N, g.K = K;
+    g.lda = 0, g.ldb = K, g.ldc = N;
+    g.a_bytes    = (uint32_t)((long)d->N * d->Hi * d->Wi * d->C * es);
+    g.b_bytes    = (uint32_t)((long)N * K * es);
+    g.tiles_m    = (M + t.bm - 1) / t.bm;
+    g.tiles_n    = (N + t.bn - 1) / t.bn;
+    g.epi        = epi;
+    g.scale_gemm = sg;
+    g.scale_relu = sr;
+    g.cv.Hi = d->Hi, g.cv.Wi = d->Wi, g.cv.C = d->C;
+    g.cv.sH = d->stride_h, g.cv.sW = d->stride_w, g.cv.dH = d->dilation_h, g.cv.dW = d->dilation_w;
+    g.cv.pT = d->pad_top, g.cv.pL = d->pad_left;
+    g.cv.div_howo = make_magic((uint32_t)(d->Ho * d->Wo));
+    g.cv.div_wo   = make_magic((uint32_t)d->Wo);
+    g.cv.div_xc   = make_magic((uint32_t)(d->X * d->C));
+    g.cv.div_c    = make_magic((uint32_t)d->C);
+    hipError_t e  = (es == 1 ? t.conv_i8 : t.conv_f16)(g, g.tiles_m * g.tiles_n, (hipStream_t)stream);
+    if(e != hipSuccess)
+        return hip_fail(e, t.name);
+    return CKX_OK;
+}
+
+} // namespace
+
+extern "C" {
+
+const char* ckx_version(void) { return "ckx-mi355 0.1 (gfx950)"; }
+const char* ckx_last_error(void) { return g_last_error.c_str(); }
+
+int ckx_num_instances(int op)
+{
+    if(op >= CKX_OP_GEMM_I8 && op <= CKX_OP_CONV2D_FWD_F16)
+        return kNumTiles;
+    if(op == CKX_OP_BATCHED_GEMM_GEMM)
+        return ckx::kNumGemmGemmInstances;
+    return 0;
+}
+
+const char* ckx_instance_name(int op, int instance)
+{
+    static thread_local std::string s;
+    const char* fam = family_prefix(op);
+    if(!fam || instance < 0 || instance >= ckx_num_instances(op))
+        return nullptr;
+    s = std::string(fam) + "<" +
+        (op == CKX_OP_BATCHED_GEMM_GEMM ? ckx::gemm_gemm_instance_name(instance) : kTiles[instance].name) + ">";
+    return s.c_str();
+}
+
+int ckx_gemm_i8_is_supported(int32_t M, int32_t N, int32_t K, int32_t sa, int32_t sb, int32_t sc, int al,
+                             int bl, int cl, int epilogue, int instance)
+{
+    return check_gemm_shape(ckx::DT_I8, M, N, K, sa, sb, sc, al, bl, cl, epilogue, instance);
+}
+
+int ckx_gemm_i8(const void* a, const void* b, void* c, int32_t M, int32_t N, int32_t K, int32_t sa,
+                int32_t sb, int32_t sc, int al, int bl, int cl, int epilogue, float scale_gemm,
+                float scale_relu, int instance, void* stream)
+{
+    return run_gemm(ckx::DT_I8, a, b, c, M, N, K, sa, sb, sc, al, bl, cl, epilogue, scale_gemm, scale_relu,
+                    instance, stream);
+}
+
+int ckx_gemm_f16_is_supported(int32_t M, int32_t N, int32_t K, int32_t sa, int32_t sb, int32_t sc, int al,
+                              int bl, int cl, int instance)
+{
+    return check_gemm_shape(ckx::DT_F16, M, N, K, sa, sb, sc, al, bl, cl, CKX_EPI_PASSTHROUGH, instance);
+}
+
+int ckx_gemm_f16(const void* a, const void* b, void* c, int32_t M, int32_t N, int32_t K, int32_t sa,
+                 int32_t sb, int32_t sc, int al, int bl, int cl, int instance, void* stream)
+{
+    return run_gemm(ckx::DT_F16, a, b, c, M, N, K, sa, sb, sc, al, bl, cl, CKX_EPI_PASSTHROUGH, 1.0f, 1.0f,
+                    instance, stream);
+}
+
+int ckx_conv2d_fwd_is_supported(int op, const ckx_conv2d_desc* desc, int epilogue, int instance)
+{
+    return check_conv(op, desc, epilogue, instance);
+}
+
+int ckx_conv2d_fwd_i8(const void* in, const void* wei, void* out, const ckx_conv2d_desc* desc, int epilogue,
+                      float scale_gemm, float scale_relu, int instance, void* stream)
+{
+    return run_conv(CKX_OP_CONV2D_FWD_I8, in, wei, out, desc, epilogue, scale_gemm, scale_relu, instance,
+                    stream);
+}
+
+int ckx_conv2d_fwd_f16(const void* in, const void* wei, void* out, const ckx_conv2d_desc* desc, int instance,
+                       void* stream)
+{
+    return run_conv(CKX_OP_CONV2D_FWD_F16, in, wei, out, desc, CKX_EPI_PASSTHROUGH, 1.0f, 1.0f, instance,
+                    stream);
+}
+
+int ckx_batched_gemm_gemm_f16_is_supported(int32_t M, int32_t N, int32_t K, int32_t O, int32_t batch,
+                                           int32_t sa, int32_t sb0, int32_t sb1, int32_t sc, int64_t bsa,
+                                           int64_t bsb0, int64_t bsb1, int64_t bsc, int instance)
+{
+    std::string why;
+    if(!ckx::gemm_gemm_supported(M, N, K, O, batch, sa, sb0, sb1, sc, bsa, bsb0, bsb1, bsc, instance, why))
+        return fail(why.rfind("invalid", 0) == 0 ? CKX_INVALID_VALUE : CKX_UNSUPPORTED, why);
+    return CKX_OK;
+}
+
+int ckx_batched_gemm_gemm_f16(const void* a, const void* b0, const void* b1, void* c, int32_t M, int32_t N,
+                              int32_t K, int32_t O, int32_t batch, int32_t sa, int32_t sb0, int32_t sb1,
+                              int32_t sc, int64_t bsa, int64_t bsb0, int64_t bsb1, int64_t bsc, int instance,
+                              void* stream)
+{
+    int st = ckx_batched_gemm_gemm_f16_is_supported(M, N, K, O, batch, sa, sb0, sb1, sc, bsa, bsb0, bsb1, bsc,
+                                                    instance);
+    if(st != CKX_OK)
+        return st;
+    if(M == 0 || O == 0 || batch == 0)
+        return CKX_OK;
+    if(!a || !b0 || !b1 || !c)
+        return fail(CKX_INVALID_VALUE, "null operand pointer");
+    if((reinterpret_cast<uintptr_t>(a) | reinterpret_cast<uintptr_t>(b0) | reinterpret_cast<uintptr_t>(b1) |
+        reinterpret_cast<uintptr_t>(c)) & 15)
+        return fail(CKX_UNSUPPORTED, "operands must be 16-byte aligned");
+    hipError_t e = ckx::gemm_gemm_launch(a, b0, b1, c, M, N, K, O, batch, sa, sb0, sb1, sc, bsa, bsb0, bsb1, bsc,
+                                         instance, (hipStream_t)stream);
+    if(e != hipSuccess)
+        return hip_fail(e, "batched_gemm_gemm");
+    return CKX_OK;
+}
+
+int ckx_time_launches(ckx_launch_fn fn, void* user, int n_warmup, int n_repeat, void* stream, float* ms)
+{
+    if(!fn || !ms || n_repeat <= 0 || n_warmup < 0)
+        return fail(CKX_INVALID_VALUE, "bad timing request");
+    hipStream_t s = (hipStream_t)stream;
+    for(int i = 0; i < n_warmup; ++i)
+        if(int r = fn(user))
+            return r;
+    hipEvent_t e0, e1;
+    hipError_t e = hipEventCreate(&e0);
+    if(e != hipSuccess)
+        return hip_fail(e, "hipEventCreate");
+    e = hipEventCreate(&e1);
+    if(e != hipSuccess)
+    {
+        (void)hipEventDestroy(e0);
+        return hip_fail(e, "hipEventCreate");
+    }
+    int rc = CKX_OK;
+    e      = hipStreamSynchronize(s);
+    if(e == hipSuccess)
+        e = hipEventRecord(e0, s);
+    for(int i = 0; i < n_repeat && e == hipSuccess && rc == CKX_OK; ++i)
+        rc = fn(user);
+    if(e == hipSuccess)
+        e = hipEventRecord(e1, s);
+    if(e == hipSuccess)
+        e = hipEventSynchronize(e1);
+    float total = 0;
+    if(e == hipSuccess)
+        e = hipEventElapsedTime(&total, e0, e1);
+    (void)hipEventDestroy(e0);
+    (void)hipEventDestroy(e1);
+    if(e != hipSuccess)
+        return hip_fail(e, "ckx_time_launches");
+    *ms = total / (float)n_repeat;
+    return rc;
+}
+
+} // extern "C"

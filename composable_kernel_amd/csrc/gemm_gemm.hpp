@@ -1,0 +1,263 @@
+// Batched fused GEMM-GEMM for gfx950, fp16:  C[g] = half( half(A[g] * B0[g]) * B1[g] ).
+// A [G,M,K] row-major, B0 stored [G,N,K] (column-major K x N), B1 [G,N,O] row-major,
+// C [G,M,O] row-major (layout gmk_gnk_gno_gmo of upstream's DeviceBatchedGemmGemm; batch
+// offsets as in kernel_batched_gemm_xdlops_v2r3, device_batched_gemm_xdl.hpp:79-88).
+//
+// One workgroup (4 waves) owns 128 rows of one batch and walks N in chunks of 128 columns.
+// The [128 x 128] slice of the intermediate never leaves registers:
+//   gemm0 is issued as S^T = B0_frag x A_frag, so lane (l%16 = m, l/16 = q) holds S[m][n]
+//   for 4 values of n per MFMA tile; the B0 rows fed to a PAIR of tiles are chosen so that
+//   the pair gives the lane n = 32*pair + 8q .. +7, i.e. exactly the eight K-slots that the
+//   same lane must supply as the second operand of gemm1 (C^T = B1T_frag x S_frag) after a
+//   round-to-nearest-even conversion to fp16. B1 is transposed while it is staged into LDS
+//   so that its fragment is one 16-byte read as well.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include <mutex>
+#include <string>
+
+#include "gemm_tile.hpp"
+
+namespace ckx {
+
+struct GemmGemmArgs
+{
+    const _Float16* a;
+    const _Float16* b0;
+    const _Float16* b1;
+    _Float16* c;
+    int M, N, K, O, batch;
+    int sa, sb0, sb1, sc;
+    int64_t bsa, bsb0, bsb1, bsc;
+    int slabs; // ceil(M / 128)
+};
+
+template <int KS, int OG>
+struct GemmGemmCfg
+{
+    static constexpr int BM   = 128; // rows per workgroup
+    static constexpr int BNC  = 128; // columns of the intermediate per step
+    static constexpr int KP   = KS * 32;
+    static constexpr int OP   = OG * 64;
+    static constexpr int AST  = KP * 2 + 16;  // padded LDS row strides (bytes)
+    static constexpr int B1ST = BNC * 2 + 16;
+    static constexpr int A_BYTES   = BM * AST;
+    static constexpr int B0_BYTES  = BNC * AST;
+    static constexpr int B1T_BYTES = OP * B1ST;
+    static constexpr int LDS       = A_BYTES + B0_BYTES + B1T_BYTES;
+};
+
+template <int KS, int OG>
+__global__ __launch_bounds__(256) void gemm_gemm_kernel(const GemmGemmArgs p)
+{
+    using Cfg = GemmGemmCfg<KS, OG>;
+    extern __shared__ __attribute__((aligned(16))) uint8_t gg_smem[];
+    uint8_t* sA   = gg_smem;
+    uint8_t* sB0  = sA + Cfg::A_BYTES;
+    uint8_t* sB1T = sB0 + Cfg::B0_BYTES;
+
+    const int tid  = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = tid >> 6;
+    const int fr   = lane & 15; // MFMA row/col index supplied by this lane
+    const int q    = lane >> 4; // K-slot group
+
+    const int g    = blockIdx.x / p.slabs;
+    const int m0   = (blockIdx.x - g * p.slabs) * Cfg::BM;
+    const _Float16* A  = p.a + (int64_t)g * p.bsa;
+    const _Float16* B0 = p.b0 + (int64_t)g * p.bsb0;
+    const _Float16* B1 = p.b1 + (int64_t)g * p.bsb1;
+    _Float16* C        = p.c + (int64_t)g * p.bsc;
+
+    constexpr int KCH = Cfg::KP / 8; // 16-byte chunks per staged row of A / B0
+    constexpr int OCH = Cfg::OP / 8;
+    const i32x4 zero4 = {0, 0, 0, 0};
+
+    // ---- A slab -> LDS -> registers (kept for the whole kernel) -----------------------
+    for(int idx = tid; idx < Cfg::BM * KCH; idx += 256)
+    {
+        const int row = idx / KCH, ch = idx - row * KCH;
+        const int m = m0 + row, k = ch * 8;
+        i32x4 v = zero4;
+        if(m < p.M && k < p.K)
+            v = *reinterpret_cast<const i32x4*>(A + (int64_t)m * p.sa + k);
+        *reinterpret_cast<i32x4*>(sA + row * Cfg::AST + ch * 16) = v;
+    }
+    __syncthreads();
+    f16x8 af[2][KS];
+#pragma unroll
+    for(int mt = 0; mt < 2; ++mt)
+#pragma unroll
+        for(int ks = 0; ks < KS; ++ks)
+            af[mt][ks] = *reinterpret_cast<const f16x8*>(sA + (wave * 32 + mt * 16 + fr) * Cfg::AST +
+                                                         (ks * 4 + q) * 16);
+
+    f32x4 acc1[2][OG * 4];
+#pragma unroll
+    for(int mt = 0; mt < 2; ++mt)
+#pragma unroll
+        for(int t = 0; t < OG * 4; ++t)
+            acc1[mt][t] = f32x4{0, 0, 0, 0};
+
+    for(int n0 = 0; n0 < p.N; n0 += Cfg::BNC)
+    {
+        __syncthreads(); // everyone is done reading the previous chunk
+        for(int idx = tid; idx < Cfg::BNC * KCH; idx += 256)
+        {
+            const int row = idx / KCH, ch = idx - row * KCH;
+            const int n = n0 + row, k = ch * 8;
+            i32x4 v = zero4;
+            if(n < p.N && k < p.K)
+                v = *reinterpret_cast<const i32x4*>(B0 + (int64_t)n * p.sb0 + k);
+            *reinterpret_cast<i32x4*>(sB0 + row * Cfg::AST + ch * 16) = v;
+        }
+        for(int idx = tid; idx < Cfg::BNC * OCH; idx += 256)
+        {
+            const int row = idx / OCH, ch = idx - row * OCH;
+            const int n = n0 + row, o = ch * 8;
+            f16x8 v = {0, 0, 0, 0, 0, 0, 0, 0};
+            if(n < p.N && o < p.O)
+                v = *reinterpret_cast<const f16x8*>(B1 + (int64_t)n * p.sb1 + o);
+#pragma unroll
+            for(int e = 0; e < 8; ++e)
+                *reinterpret_cast<_Float16*>(sB1T + (o + e) * Cfg::B1ST + row * 2) = v[e];
+        }
+        __syncthreads();
+
+        // ---- gemm0: S^T tiles, 8 tiles of 16 columns, pairs share a 32-column span -----
+        f32x4 s[2][8];
+#pragma unroll
+        for(int mt = 0; mt < 2; ++mt)
+#pragma unroll
+            for(int t = 0; t < 8; ++t)
+                s[mt][t] = f32x4{0, 0, 0, 0};
+#pragma unroll
+        for(int ks = 0; ks < KS; ++ks)
+#pragma unroll
+            for(int t = 0; t < 8; ++t)
+            {
+                const int row = 32 * (t >> 1) + 8 * (fr >> 2) + 4 * (t & 1) + (fr & 3);
+                const f16x8 b0f =
+                    *reinterpret_cast<const f16x8*>(sB0 + row * Cfg::AST + (ks * 4 + q) * 16);
+#pragma unroll
+                for(int mt = 0; mt < 2; ++mt)
+                    s[mt][t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(b0f, af[mt][ks], s[mt][t], 0, 0, 0);
+            }
+
+        // ---- fp32 -> fp16 (RNE): the pair (2*pr, 2*pr+1) is the gemm1 operand for 32 n ----
+        f16x8 sf[2][4];
+#pragma unroll
+        for(int mt = 0; mt < 2; ++mt)
+#pragma unroll
+            for(int pr = 0; pr < 4; ++pr)
+#pragma unroll
+                for(int j = 0; j < 4; ++j)
+                {
+                    sf[mt][pr][j]     = (_Float16)s[mt][2 * pr][j];
+                    sf[mt][pr][4 + j] = (_Float16)s[mt][2 * pr + 1][j];
+                }
+
+        // ---- gemm1: C^T tiles ------------------------------------------------------------
+#pragma unroll
+        for(int pr = 0; pr < 4; ++pr)
+#pragma unroll
+            for(int ot = 0; ot < OG * 4; ++ot)
+            {
+                const int o = 64 * (ot >> 2) + 16 * (fr >> 2) + 4 * (ot & 3) + (fr & 3);
+                const f16x8 b1f =
+                    *reinterpret_cast<const f16x8*>(sB1T + o * Cfg::B1ST + (32 * pr + 8 * q) * 2);
+#pragma unroll
+                for(int mt = 0; mt < 2; ++mt)
+                    acc1[mt][ot] =
+                        __builtin_amdgcn_mfma_f32_16x16x32_f16(b1f, sf[mt][pr], acc1[mt][ot], 0, 0, 0);
+            }
+    }
+
+    const bool vec_ok = ((reinterpret_cast<uintptr_t>(C) | ((uintptr_t)p.sc * 2)) & 15u) == 0;
+#pragma unroll
+    for(int mt = 0; mt < 2; ++mt)
+    {
+        const int m = m0 + wave * 32 + mt * 16 + fr;
+        if(m >= p.M)
+            continue;
+#pragma unroll
+        for(int og = 0; og < OG; ++og)
+        {
+            const int o0 = 64 * og + 16 * q;
+            if(o0 >= p.O)
+                continue;
+            const f32x4 v[4] = {acc1[mt][og * 4], acc1[mt][og * 4 + 1], acc1[mt][og * 4 + 2],
+                                acc1[mt][og * 4 + 3]};
+            store_row16_f16(C + (int64_t)m * p.sc, o0, p.O, vec_ok, v);
+        }
+    }
+}
+
+// ---------------------------------------------------------------- host side
+constexpr int kNumGemmGemmInstances = 1;
+
+inline const char* gemm_gemm_instance_name(int)
+{
+    return "MI355X_Mfma16_GemmGemm<128 rows, 128-col steps, K<=128, O<=128>";
+}
+
+inline bool gemm_gemm_supported(int M, int N, int K, int O, int batch, int sa, int sb0, int sb1, int sc,
+                                int64_t bsa, int64_t bsb0, int64_t bsb1, int64_t bsc, int instance,
+                                std::string& why)
+{
+    (void)bsc;
+    if(M < 0 || N < 0 || K < 0 || O < 0 || batch < 0)
+        return why = "invalid: negative dimension", false;
+    if(instance != -1 && instance != 0)
+        return why = "invalid: no such instance", false;
+    if(K > 128 || O > 128)
+        return why = "K and O above 128 are not built", false;
+    if(K % 8 || O % 8 || sa % 8 || sb0 % 8 || sb1 % 8 || bsa % 8 || bsb0 % 8 || bsb1 % 8)
+        return why = "K, O and the A/B0/B1 strides must be multiples of 8 elements (16 bytes)", false;
+    if(sa < K || sb0 < K || sb1 < O || sc < O)
+        return why = "stride smaller than the contiguous extent", false;
+    if((long)((M + 127) / 128) * batch >= (1l << 31))
+        return why = "grid too large", false;
+    return true;
+}
+
+template <int KS, int OG>
+inline hipError_t gemm_gemm_launch_t(const GemmGemmArgs& a, hipStream_t s)
+{
+    using Cfg  = GemmGemmCfg<KS, OG>;
+    auto* kern = &gemm_gemm_kernel<KS, OG>;
+    static std::once_flag once;
+    static hipError_t attr_err = hipSuccess;
+    std::call_once(once, [&] {
+        attr_err = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, Cfg::LDS);
+    });
+    if(attr_err != hipSuccess)
+        return attr_err;
+    hipLaunchKernelGGL(kern, dim3(a.slabs * a.batch), dim3(256), Cfg::LDS, s, a);
+    return hipGetLastError();
+}
+
+inline hipError_t gemm_gemm_launch(const void* a, const void* b0, const void* b1, void* c, int M, int N, int K,
+                                   int O, int batch, int sa, int sb0, int sb1, int sc, int64_t bsa,
+                                   int64_t bsb0, int64_t bsb1, int64_t bsc, int /*instance*/, hipStream_t s)
+{
+    GemmGemmArgs g;
+    g.a = (const _Float16*)a, g.b0 = (const _Float16*)b0, g.b1 = (const _Float16*)b1, g.c = (_Float16*)c;
+    g.M = M, g.N = N, g.K = K, g.O = O, g.batch = batch;
+    g.sa = sa, g.sb0 = sb0, g.sb1 = sb1, g.sc = sc;
+    g.bsa = bsa, g.bsb0 = bsb0, g.bsb1 = bsb1, g.bsc = bsc;
+    g.slabs      = (M + 127) / 128;
+    const int ks = K <= 32 ? 1 : (K <= 64 ? 2 : 4);
+    const int og = O <= 64 ? 1 : 2;
+    if(ks == 1)
+        return og == 1 ? gemm_gemm_launch_t<1, 1>(g, s) : gemm_gemm_launch_t<1, 2>(g, s);
+    if(ks == 2)
+        return og == 1 ? gemm_gemm_launch_t<2, 1>(g, s) : gemm_gemm_launch_t<2, 2>(g, s);
+    return og == 1 ? gemm_gemm_launch_t<4, 1>(g, s) : gemm_gemm_launch_t<4, 2>(g, s);
+}
+
+} // namespace ckx

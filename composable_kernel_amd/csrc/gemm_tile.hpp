@@ -1,0 +1,460 @@
+// Tile GEMM for gfx950 (MI355X): C[M,N] = epilogue(A[M,K] * B[N,K]^T), both operands
+// K-contiguous ("mk_nk_mn": A row-major, B column-major, C row-major), with an optional
+// implicit-im2col A operand for NHWC conv2d forward.
+//
+// Takes the place of kernel_gemm_xdl_cshuffle_v1 / kernel_gemm_xdlops_v2r3 of the
+// reference (include/ck/tensor_operation/gpu/grid/gridwise_gemm_xdl_cshuffle_v1.hpp:32-74,
+// gridwise_gemm_xdlops_v2r3.hpp:30-72). Nothing of their structure is kept:
+//
+//  * byte-generic K tiling: one K tile is 128 BYTES of every row (128 int8 / 64 fp16), so a
+//    row of a staged tile is eight 16-byte chunks for either dtype, and one MFMA k-step
+//    (16x16x64 i8 or 16x16x32 f16) consumes four of them: lane l reads chunk 4*ks + l/16 of
+//    row l%16 with a single ds_read_b128.
+//  * global -> LDS staging is direct (buffer_load_dwordx4 ... lds): a wave instruction
+//    deposits 64 x 16 B = 8 rows x 8 chunks contiguously, and each lane picks WHICH global
+//    chunk lands in its slot, which is how the XOR swizzle and the B row permutation are
+//    applied for free. Out-of-range rows / K tail / conv padding use an out-of-range buffer
+//    offset, which the hardware turns into zeros.
+//  * two LDS stages, one barrier per K tile; the loads of tile k+1 are in flight while
+//    tile k is multiplied.
+//  * MFMA is issued as D^T = B_frag x A_frag, so a lane ends up owning, for one row m, the
+//    accumulators of 4 consecutive columns per MFMA tile; the B rows of a 64-column group
+//    are permuted in LDS so that the 4 tiles of the group give the lane 16 CONSECUTIVE
+//    columns. The epilogue (requant, ReLU, saturation, conversion) runs on registers and
+//    each lane stores 16 contiguous outputs: no trip through LDS.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <type_traits>
+
+namespace ckx {
+
+typedef int i32x4 __attribute__((ext_vector_type(4)));
+typedef int i32x2 __attribute__((ext_vector_type(2)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+
+enum
+{
+    DT_I8  = 0,
+    DT_F16 = 1
+};
+
+enum
+{
+    EPI_PASSTHROUGH = 0,
+    EPI_REQUANT_CK  = 1,
+    EPI_REQUANT_RND = 2
+};
+
+#ifndef CKX_SWZ_SHIFT
+#define CKX_SWZ_SHIFT 0
+#endif
+
+// q = n / d for 0 <= n < 2^31 (include/ck/utility/magic_division.hpp:28-54,132-137)
+struct MagicDiv
+{
+    uint32_t mul;
+    uint32_t shift;
+    uint32_t d;
+};
+
+__device__ __forceinline__ uint32_t magic_div(uint32_t n, const MagicDiv& m)
+{
+    return (__umulhi(n, m.mul) + n) >> m.shift;
+}
+
+// Geometry of the implicit-GEMM view of a conv2d forward
+// (device_conv2d_fwd_xdl_nhwc_kyxc_nhwk.hpp:224-301 in closed form):
+//   row m -> (n, ho, wo), k -> (y, x, c) with c fastest.
+struct ConvGeom
+{
+    int Hi, Wi, C;
+    int sH, sW, dH, dW, pT, pL;
+    MagicDiv div_howo; // Ho*Wo
+    MagicDiv div_wo;   // Wo
+    MagicDiv div_xc;   // X*C
+    MagicDiv div_c;    // C
+};
+
+struct GemmArgs
+{
+    const void* a;
+    const void* b;
+    void* c;
+    int M, N, K;
+    int lda, ldb, ldc;      // elements
+    uint32_t a_bytes;       // extent of the A / B allocations seen by the buffer resource
+    uint32_t b_bytes;
+    int tiles_m, tiles_n;
+    int epi;
+    float scale_gemm, scale_relu;
+    ConvGeom cv;
+};
+
+constexpr uint32_t kOutOfRange = 0x80000000u;
+
+__device__ __forceinline__ uint32_t swz(uint32_t row) { return (row >> CKX_SWZ_SHIFT) & 7u; }
+
+__device__ __forceinline__ uint32_t lds_chunk_offset(uint32_t row, uint32_t chunk)
+{
+    return row * 128u + ((chunk ^ swz(row)) << 4);
+}
+
+// LDS row (position in the staged B tile) -> column of the tile. Within a 64-column group,
+// LDS row 16*t + j (MFMA tile t, MFMA row j) holds column 16*(j/4) + 4*t + j%4.
+__device__ __forceinline__ uint32_t b_row_to_col(uint32_t r)
+{
+    return (r & ~63u) | (((r & 15u) >> 2) << 4) | (((r >> 4) & 3u) << 2) | (r & 3u);
+}
+
+// Workgroup id -> tile. Workgroups are dealt round-robin to the 8 XCDs, each with a private
+// L2: first make the ids that land on one XCD contiguous, then sweep tiles in groups of 8
+// tile-rows, column by column, so that the tiles resident on an XCD share few A/B panels.
+// (BlockToCTileMap_M00_N0_M01Adapt, block_to_ctile_map.hpp:112-173, is the reference's
+// single-L2 analogue; the order is not observable in the results.)
+__device__ __forceinline__ void tile_of_block(int bid, int tiles_m, int tiles_n, int& tm, int& tn)
+{
+    const int nb    = tiles_m * tiles_n;
+    const int xcd   = bid & 7;
+    const int local = bid >> 3;
+    const int q = nb >> 3, r = nb & 7;
+    const int id = xcd * q + (xcd < r ? xcd : r) + local;
+    constexpr int GM    = 8;
+    const int per_group = GM * tiles_n;
+    const int grp       = id / per_group;
+    const int first_m   = grp * GM;
+    const int gsz       = (tiles_m - first_m) < GM ? (tiles_m - first_m) : GM;
+    const int in        = id - grp * per_group;
+    tm                  = first_m + in % gsz;
+    tn                  = in / gsz;
+}
+
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* p, uint32_t bytes)
+{
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(p), 0, (int)bytes, 0x00020000);
+}
+
+typedef __attribute__((address_space(3))) void* lds_ptr_t;
+
+// ---------------------------------------------------------------- epilogues
+__device__ __forceinline__ int requant_ck(int acc, float sg, float sr)
+{
+    float x = (float)acc;
+    float g = sg * x;
+    float r = g > 0.0f ? g : 0.0f;
+    float q = sr * r;
+    float y = q > 127.0f ? 127.0f : (q < -128.0f ? -128.0f : q);
+    return (int)y; // toward zero
+}
+
+__device__ __forceinline__ int requant_rnd(int acc, float sg, float sr)
+{
+    float x = (float)acc;
+    float t = __builtin_rintf(sg * x);
+    t       = t > 127.0f ? 127.0f : (t < -128.0f ? -128.0f : t);
+    float r = t > 0.0f ? t : 0.0f;
+    float u = __builtin_rintf(sr * r);
+    u       = u > 127.0f ? 127.0f : (u < -128.0f ? -128.0f : u);
+    return (int)u;
+}
+
+template <int EPI>
+__device__ __forceinline__ int epilogue_i8(int acc, float sg, float sr)
+{
+    if constexpr(EPI == EPI_REQUANT_CK)
+        return requant_ck(acc, sg, sr) & 0xFF;
+    else if constexpr(EPI == EPI_REQUANT_RND)
+        return requant_rnd(acc, sg, sr) & 0xFF;
+    else
+        return acc & 0xFF;
+}
+
+// 16 consecutive int8 outputs of one row
+template <int EPI>
+__device__ __forceinline__ void store_row16_i8(int8_t* crow, int n0, int N, bool vec_ok, const i32x4 (&v)[4],
+                                               float sg, float sr)
+{
+    int b[16];
+#pragma unroll
+    for(int t = 0; t < 4; ++t)
+#pragma unroll
+        for(int j = 0; j < 4; ++j)
+            b[t * 4 + j] = epilogue_i8<EPI>(v[t][j], sg, sr);
+    if(vec_ok && n0 + 16 <= N)
+    {
+        i32x4 pk;
+#pragma unroll
+        for(int w = 0; w < 4; ++w)
+            pk[w] = b[4 * w] | (b[4 * w + 1] << 8) | (b[4 * w + 2] << 16) | (b[4 * w + 3] << 24);
+        *reinterpret_cast<i32x4*>(crow + n0) = pk;
+    }
+    else
+    {
+#pragma unroll
+        for(int e = 0; e < 16; ++e)
+            if(n0 + e < N)
+                crow[n0 + e] = (int8_t)b[e];
+    }
+}
+
+__device__ __forceinline__ void store_row16_f16(_Float16* crow, int n0, int N, bool vec_ok,
+                                                const f32x4 (&v)[4])
+{
+    if(vec_ok && n0 + 16 <= N)
+    {
+        f16x8 lo, hi;
+#pragma unroll
+        for(int j = 0; j < 4; ++j)
+        {
+            lo[j]     = (_Float16)v[0][j];
+            lo[4 + j] = (_Float16)v[1][j];
+            hi[j]     = (_Float16)v[2][j];
+            hi[4 + j] = (_Float16)v[3][j];
+        }
+        *reinterpret_cast<f16x8*>(crow + n0)     = lo;
+        *reinterpret_cast<f16x8*>(crow + n0 + 8) = hi;
+    }
+    else
+    {
+#pragma unroll
+        for(int t = 0; t < 4; ++t)
+#pragma unroll
+            for(int j = 0; j < 4; ++j)
+                if(n0 + t * 4 + j < N)
+                    crow[n0 + t * 4 + j] = (_Float16)v[t][j];
+    }
+}
+
+// ------------------------------------------------------------------- kernel
+template <int DT, int BM, int BN, int WM, int WN, bool IM2COL>
+struct GemmTile
+{
+    static constexpr int NW      = WM * WN;
+    static constexpr int NT      = NW * 64;
+    static constexpr int ES      = DT == DT_I8 ? 1 : 2;
+    static constexpr int CE      = 16 / ES; // elements per 16-byte chunk
+    static constexpr int BKE     = 128 / ES;
+    static constexpr int WTM     = BM / WM;
+    static constexpr int WTN     = BN / WN;
+    static constexpr int MT      = WTM / 16;
+    static constexpr int NG      = WTN / 64;
+    static constexpr int A_TILE  = BM * 128;
+    static constexpr int B_TILE  = BN * 128;
+    static constexpr int STAGE   = A_TILE + B_TILE;
+    static constexpr int LDS     = 2 * STAGE;
+    static constexpr int NLA     = BM * 8 / NT; // 16-byte loads per thread and K tile, A
+    static constexpr int NLB     = BN * 8 / NT;
+    static_assert(WTM % 16 == 0 && WTN % 64 == 0, "wave tile must be 16k x 64k");
+    static_assert((BM * 8) % NT == 0 && (BN * 8) % NT == 0, "tile rows must split over the waves");
+
+    using acc_t = typename std::conditional<DT == DT_I8, i32x4, f32x4>::type;
+
+    __device__ static void run(const GemmArgs& p, uint8_t* smem)
+    {
+        const int tid  = threadIdx.x;
+        const int lane = tid & 63;
+        const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+        const int wm   = wave / WN;
+        const int wn   = wave % WN;
+
+        int tm, tn;
+        tile_of_block(blockIdx.x, p.tiles_m, p.tiles_n, tm, tn);
+
+        const uint32_t kbytes = (uint32_t)p.K * ES;
+        const int nk          = (int)((kbytes + 127u) >> 7);
+
+        const __amdgpu_buffer_rsrc_t rsrc_a = make_rsrc(p.a, p.a_bytes);
+        const __amdgpu_buffer_rsrc_t rsrc_b = make_rsrc(p.b, p.b_bytes);
+
+        // ---- per-thread load slots -------------------------------------------------
+        // slot j of this thread fills LDS row (j*NW + wave)*8 + lane/8, chunk position lane%8
+        uint32_t a_off[NLA];  // dense: byte offset of (row, chunk) at K tile 0, or kOutOfRange
+        uint32_t a_kb[NLA];   // byte offset of the chunk inside a K tile
+        int a_hi0[NLA], a_wi0[NLA]; // im2col: top-left input coordinate of the row's window
+        uint32_t b_off[NLB];
+        uint32_t b_kb[NLB];
+#pragma unroll
+        for(int j = 0; j < NLA; ++j)
+        {
+            const uint32_t r  = (uint32_t)((j * NW + wave) * 8 + (lane >> 3));
+            const uint32_t ch = (uint32_t)(lane & 7) ^ swz(r);
+            a_kb[j]           = ch << 4;
+            const uint32_t gm = (uint32_t)tm * BM + r;
+            if constexpr(!IM2COL)
+            {
+                a_off[j] = gm < (uint32_t)p.M ? gm * (uint32_t)p.lda * ES + a_kb[j] : kOutOfRange;
+                a_hi0[j] = a_wi0[j] = 0;
+            }
+            else
+            {
+                if(gm < (uint32_t)p.M)
+                {
+                    const uint32_t n   = magic_div(gm, p.cv.div_howo);
+                    const uint32_t rem = gm - n * p.cv.div_howo.d;
+                    const uint32_t ho  = magic_div(rem, p.cv.div_wo);
+                    const uint32_t wo  = rem - ho * p.cv.div_wo.d;
+                    a_hi0[j]           = (int)ho * p.cv.sH - p.cv.pT;
+                    a_wi0[j]           = (int)wo * p.cv.sW - p.cv.pL;
+                    a_off[j]           = n * (uint32_t)(p.cv.Hi * p.cv.Wi) * (uint32_t)p.cv.C; // elements
+                }
+                else
+                {
+                    a_hi0[j] = a_wi0[j] = -0x40000000; // every tap out of range
+                    a_off[j]            = 0;
+                }
+            }
+        }
+#pragma unroll
+        for(int j = 0; j < NLB; ++j)
+        {
+            const uint32_t r  = (uint32_t)((j * NW + wave) * 8 + (lane >> 3));
+            const uint32_t ch = (uint32_t)(lane & 7) ^ swz(r);
+            b_kb[j]           = ch << 4;
+            const uint32_t gn = (uint32_t)tn * BN + b_row_to_col(r);
+            b_off[j] = gn < (uint32_t)p.N ? gn * (uint32_t)p.ldb * ES + b_kb[j] : kOutOfRange;
+        }
+
+        auto issue_loads = [&](int kt, int stage) {
+            uint8_t* sa           = smem + stage * STAGE;
+            uint8_t* sb           = sa + A_TILE;
+            const uint32_t k0     = (uint32_t)kt << 7; // byte offset of the K tile
+            const bool tail       = (k0 + 128u > kbytes);
+#pragma unroll
+            for(int j = 0; j < NLA; ++j)
+            {
+                uint32_t voff;
+                if constexpr(!IM2COL)
+                {
+                    voff = a_off[j] + k0;
+                    if(tail && k0 + a_kb[j] >= kbytes)
+                        voff = kOutOfRange;
+                }
+                else
+                {
+                    const uint32_t ke  = (k0 + a_kb[j]) / ES; // element index along GEMM-K
+                    const uint32_t y   = magic_div(ke, p.cv.div_xc);
+                    const uint32_t rem = ke - y * p.cv.div_xc.d;
+                    const uint32_t x   = magic_div(rem, p.cv.div_c);
+                    const uint32_t cc  = rem - x * p.cv.div_c.d;
+                    const int hi       = a_hi0[j] + (int)y * p.cv.dH;
+                    const int wi       = a_wi0[j] + (int)x * p.cv.dW;
+                    const bool ok      = (uint32_t)hi < (uint32_t)p.cv.Hi && (uint32_t)wi < (uint32_t)p.cv.Wi &&
+                                    ke < (uint32_t)p.K;
+                    voff = ok ? (a_off[j] + (uint32_t)(hi * p.cv.Wi + wi) * (uint32_t)p.cv.C + cc) * ES
+                              : kOutOfRange;
+                }
+                __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_a, (lds_ptr_t)(sa + (j * NW + wave) * 1024), 16,
+                                                         voff, 0, 0, 0);
+            }
+#pragma unroll
+            for(int j = 0; j < NLB; ++j)
+            {
+                uint32_t voff = b_off[j] + k0;
+                if(tail && k0 + b_kb[j] >= kbytes)
+                    voff = kOutOfRange;
+                __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_b, (lds_ptr_t)(sb + (j * NW + wave) * 1024), 16,
+                                                         voff, 0, 0, 0);
+            }
+        };
+
+        // ---- accumulators ------------------------------------------------------------
+        acc_t acc[MT][NG * 4];
+#pragma unroll
+        for(int i = 0; i < MT; ++i)
+#pragma unroll
+            for(int t = 0; t < NG * 4; ++t)
+                acc[i][t] = acc_t{0, 0, 0, 0};
+
+        // fragment addresses: row = base + lane%16, chunk = 4*ks + lane/16
+        const uint32_t frow = (uint32_t)(lane & 15);
+        const uint32_t fq   = (uint32_t)(lane >> 4);
+
+        issue_loads(0, 0);
+
+        for(int kt = 0; kt < nk; ++kt)
+        {
+            __syncthreads(); // waits for this wave's direct loads, then for everybody's
+            if(kt + 1 < nk)
+                issue_loads(kt + 1, (kt + 1) & 1);
+
+            const uint8_t* sa = smem + (kt & 1) * STAGE;
+            const uint8_t* sb = sa + A_TILE;
+#pragma unroll
+            for(int ks = 0; ks < 2; ++ks)
+            {
+                i32x4 af[MT];
+                i32x4 bf[NG * 4];
+#pragma unroll
+                for(int i = 0; i < MT; ++i)
+                {
+                    const uint32_t row = (uint32_t)(wm * WTM + 16 * i) + frow;
+                    af[i] = *reinterpret_cast<const i32x4*>(sa + lds_chunk_offset(row, ks * 4 + fq));
+                }
+#pragma unroll
+                for(int t = 0; t < NG * 4; ++t)
+                {
+                    const uint32_t row = (uint32_t)(wn * WTN + 16 * t) + frow;
+                    bf[t] = *reinterpret_cast<const i32x4*>(sb + lds_chunk_offset(row, ks * 4 + fq));
+                }
+#pragma unroll
+                for(int i = 0; i < MT; ++i)
+#pragma unroll
+                    for(int t = 0; t < NG * 4; ++t)
+                    {
+                        if constexpr(DT == DT_I8)
+                            acc[i][t] = __builtin_amdgcn_mfma_i32_16x16x64_i8(bf[t], af[i], acc[i][t], 0, 0, 0);
+                        else
+                            acc[i][t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(
+                                __builtin_bit_cast(f16x8, bf[t]), __builtin_bit_cast(f16x8, af[i]), acc[i][t], 0,
+                                0, 0);
+                    }
+            }
+        }
+
+        // ---- epilogue: registers -> global, 16 consecutive columns per lane -------------
+        const bool vec_ok = ((reinterpret_cast<uintptr_t>(p.c) | ((uintptr_t)p.ldc * ES)) & 15u) == 0;
+#pragma unroll
+        for(int i = 0; i < MT; ++i)
+        {
+            const int m = tm * BM + wm * WTM + 16 * i + (lane & 15);
+            if(m >= p.M)
+                continue;
+#pragma unroll
+            for(int g = 0; g < NG; ++g)
+            {
+                const int n0 = tn * BN + wn * WTN + 64 * g + 16 * (lane >> 4);
+                if(n0 >= p.N)
+                    continue;
+                if constexpr(DT == DT_I8)
+                {
+                    int8_t* crow = reinterpret_cast<int8_t*>(p.c) + (size_t)m * p.ldc;
+                    const i32x4 v[4] = {acc[i][g * 4], acc[i][g * 4 + 1], acc[i][g * 4 + 2], acc[i][g * 4 + 3]};
+                    if(p.epi == EPI_REQUANT_RND)
+                        store_row16_i8<EPI_REQUANT_RND>(crow, n0, p.N, vec_ok, v, p.scale_gemm, p.scale_relu);
+                    else if(p.epi == EPI_REQUANT_CK)
+                        store_row16_i8<EPI_REQUANT_CK>(crow, n0, p.N, vec_ok, v, p.scale_gemm, p.scale_relu);
+                    else
+                        store_row16_i8<EPI_PASSTHROUGH>(crow, n0, p.N, vec_ok, v, p.scale_gemm, p.scale_relu);
+                }
+                else
+                {
+                    _Float16* crow     = reinterpret_cast<_Float16*>(p.c) + (size_t)m * p.ldc;
+                    const f32x4 v[4] = {acc[i][g * 4], acc[i][g * 4 + 1], acc[i][g * 4 + 2], acc[i][g * 4 + 3]};
+                    store_row16_f16(crow, n0, p.N, vec_ok, v);
+                }
+            }
+        }
+    }
+};
+
+template <int DT, int BM, int BN, int WM, int WN, bool IM2COL>
+__global__ __launch_bounds__(WM* WN * 64) void gemm_tile_kernel(const GemmArgs p)
+{
+    extern __shared__ __attribute__((aligned(1024))) uint8_t ckx_smem[];
+    GemmTile<DT, BM, BN, WM, WN, IM2COL>::run(p, ckx_smem);
+}
+
+} // namespace ckx

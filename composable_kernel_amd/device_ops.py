@@ -1,0 +1,250 @@
+"""Python mirror of Composable Kernel's device-operator surface over the C ABI.
+
+The product host layer is C++ (host/ckx/device_ops.hpp); this mirror exists so
+that tests and the benchmark can drive the same C entry points with the
+reference's vocabulary:
+
+    op  = DeviceGemmInt8(...)                      # one instance
+    arg = op.MakeArgumentPointer(p_a, p_b, p_c, M, N, K, StrideA, StrideB, StrideC,
+                                 PassThrough(), PassThrough(), RequantReluRequant(0.03, 1))
+    if op.IsSupportedArgument(arg):
+        ms = op.MakeInvokerPointer().Run(arg, StreamConfig(stream, time_kernel=True))
+
+Names, argument order and error behaviour follow
+include/ck/tensor_operation/gpu/device/device_base.hpp:14-57, device_gemm.hpp:24-41,
+device_conv_fwd.hpp:18-39 and (for GEMM-GEMM) upstream's
+device_batched_gemm_gemm.hpp:15-56. Pointers are device addresses (ints) or
+torch CUDA tensors. Nothing here computes: a missing libckx.so raises.
+"""
+from dataclasses import dataclass
+import ctypes as C
+
+from . import capi
+
+
+# ---------------------------------------------------------------- functors
+class PassThrough:
+    """element_wise::PassThrough (unary_element_wise_operation.hpp:13-25)"""
+    epilogue = capi.EPI_PASSTHROUGH
+    scale_gemm = 1.0
+    scale_relu = 1.0
+
+
+class RequantReluRequant:
+    """example/14_gemm_xdl_requant_relu_requant/gemm_xdl_requant_relu_requant_int8.cpp:21-39.
+    rounded=False is the literal functor (no rounding, truncating cast);
+    rounded=True is sat8(rint(sR*relu(sat8(rint(sG*x)))))."""
+
+    def __init__(self, scale_gemm, scale_relu, rounded=False):
+        self.scale_gemm = float(scale_gemm)
+        self.scale_relu = float(scale_relu)
+        self.epilogue = capi.EPI_REQUANT_RND if rounded else capi.EPI_REQUANT_CK
+
+
+class RowMajor:
+    code = capi.ROW_MAJOR
+
+
+class ColumnMajor:
+    code = capi.COL_MAJOR
+
+
+@dataclass
+class StreamConfig:
+    """include/ck/stream_config.hpp:9-13"""
+    stream_id_: int = 0
+    time_kernel_: bool = False
+    nrepeat_: int = 10   # kernel_launch.hpp:20-62: 1 warm-up + 10 timed launches
+    nwarmup_: int = 1
+
+
+def _ptr(x):
+    if x is None:
+        return 0
+    if isinstance(x, int):
+        return x
+    return int(x.data_ptr())
+
+
+class BaseArgument:
+    p_workspace_ = None
+
+
+class BaseInvoker:
+    def __init__(self, op):
+        self._op = op
+
+    def Run(self, arg, stream_config=None):
+        """Launches; returns mean kernel milliseconds if time_kernel_, else 0
+        (kernel_launch.hpp:61,67). Unsupported arguments raise, as the reference's
+        Invoker::Run throws (device_gemm_xdl_cshuffle.hpp:475-481)."""
+        sc = stream_config or StreamConfig()
+        if not self._op.IsSupportedArgument(arg):
+            raise RuntimeError("wrong! " + self._op.GetTypeString() + " has invalid setting: "
+                               + capi.last_error())
+        if not sc.time_kernel_:
+            capi.check(self._op._launch(arg, sc.stream_id_))
+            return 0.0
+        return capi.time_launches(lambda: self._op._launch(arg, sc.stream_id_), sc.nwarmup_,
+                                  sc.nrepeat_, sc.stream_id_)
+
+
+class BaseOperator:
+    op_family = None
+
+    def __init__(self, instance=capi.INSTANCE_AUTO):
+        self.instance = instance
+
+    def IsSupportedArgument(self, arg):
+        return self._supported(arg) == capi.OK
+
+    def GetTypeString(self):
+        if self.instance == capi.INSTANCE_AUTO:
+            return f"ckx<auto:{self.op_family}>"
+        return capi.lib().ckx_instance_name(self.op_family, self.instance).decode()
+
+    def GetWorkSpaceSize(self, arg):
+        return 0
+
+    def SetWorkSpacePointer(self, arg, p):
+        arg.p_workspace_ = p
+
+    def MakeInvokerPointer(self):
+        return BaseInvoker(self)
+
+    @classmethod
+    def GetInstances(cls):
+        """DeviceOperationInstanceFactory<DeviceOp>::GetInstances()
+        (library/include/ck/library/tensor_operation_instance/gpu/gemm.hpp:233-379)"""
+        n = capi.lib().ckx_num_instances(cls.op_family)
+        return [cls(i) for i in range(n)]
+
+
+# -------------------------------------------------------------------- GEMM
+class _GemmArgument(BaseArgument):
+    def __init__(self, p_a, p_b, p_c, M, N, K, sa, sb, sc, a_op, b_op, c_op, layouts):
+        self.p_a, self.p_b, self.p_c = _ptr(p_a), _ptr(p_b), _ptr(p_c)
+        self.M, self.N, self.K = int(M), int(N), int(K)
+        self.StrideA, self.StrideB, self.StrideC = int(sa), int(sb), int(sc)
+        self.a_op, self.b_op, self.c_op = a_op, b_op, c_op
+        self.layouts = layouts
+
+
+class _DeviceGemm(BaseOperator):
+    def __init__(self, instance=capi.INSTANCE_AUTO, ALayout=RowMajor, BLayout=ColumnMajor, CLayout=RowMajor):
+        super().__init__(instance)
+        self.layouts = (ALayout.code, BLayout.code, CLayout.code)
+
+    def MakeArgumentPointer(self, p_a, p_b, p_c, M, N, K, StrideA, StrideB, StrideC, a_element_op=None,
+                            b_element_op=None, c_element_op=None):
+        a_op = a_element_op or PassThrough()
+        b_op = b_element_op or PassThrough()
+        if not isinstance(a_op, PassThrough) or not isinstance(b_op, PassThrough):
+            raise TypeError("A/B element-wise operations other than PassThrough are not built")
+        return _GemmArgument(p_a, p_b, p_c, M, N, K, StrideA, StrideB, StrideC, a_op, b_op,
+                             c_element_op or PassThrough(), self.layouts)
+
+
+class DeviceGemmInt8(_DeviceGemm):
+    """DeviceGemm<..., int8_t, int8_t, int8_t, PassThrough, PassThrough, COp>"""
+    op_family = capi.OP_GEMM_I8
+
+    def _supported(self, a):
+        return capi.lib().ckx_gemm_i8_is_supported(a.M, a.N, a.K, a.StrideA, a.StrideB, a.StrideC,
+                                                   *a.layouts, a.c_op.epilogue, self.instance)
+
+    def _launch(self, a, stream):
+        return capi.lib().ckx_gemm_i8(a.p_a, a.p_b, a.p_c, a.M, a.N, a.K, a.StrideA, a.StrideB, a.StrideC,
+                                      *a.layouts, a.c_op.epilogue, a.c_op.scale_gemm, a.c_op.scale_relu,
+                                      self.instance, C.c_void_p(stream or 0))
+
+
+class DeviceGemmF16(_DeviceGemm):
+    """DeviceGemm<..., half_t, half_t, half_t, PassThrough, PassThrough, PassThrough>"""
+    op_family = capi.OP_GEMM_F16
+
+    def _supported(self, a):
+        if not isinstance(a.c_op, PassThrough):
+            capi.lib().ckx_gemm_f16_is_supported(-1, 0, 0, 0, 0, 0, 0, 0, 0, 0)  # sets an error string
+            return capi.UNSUPPORTED
+        return capi.lib().ckx_gemm_f16_is_supported(a.M, a.N, a.K, a.StrideA, a.StrideB, a.StrideC,
+                                                    *a.layouts, self.instance)
+
+    def _launch(self, a, stream):
+        return capi.lib().ckx_gemm_f16(a.p_a, a.p_b, a.p_c, a.M, a.N, a.K, a.StrideA, a.StrideB, a.StrideC,
+                                       *a.layouts, self.instance, C.c_void_p(stream or 0))
+
+
+# -------------------------------------------------------------------- conv
+class _ConvArgument(BaseArgument):
+    def __init__(self, p_in, p_wei, p_out, desc, out_op):
+        self.p_in, self.p_wei, self.p_out = _ptr(p_in), _ptr(p_wei), _ptr(p_out)
+        self.desc = desc
+        self.out_op = out_op
+
+
+class _DeviceConvFwd(BaseOperator):
+    """DeviceConvFwd<InOp, WeiOp, OutOp>, 2-D NHWC / KYXC / NHWK (device_conv_fwd.hpp:18-39)"""
+
+    def MakeArgumentPointer(self, p_in, p_wei, p_out, N, K, C_, input_spatial_lengths,
+                            filter_spatial_lengths, output_spatial_lengths, conv_filter_strides,
+                            conv_filter_dilations, input_left_pads, input_right_pads, in_element_op=None,
+                            wei_element_op=None, out_element_op=None):
+        for v in (input_spatial_lengths, filter_spatial_lengths, output_spatial_lengths,
+                  conv_filter_strides, conv_filter_dilations, input_left_pads, input_right_pads):
+            if len(v) != 2:
+                raise ValueError("only NumDimSpatial == 2 is built")
+        d = capi.Conv2dDesc(N, K, C_, *input_spatial_lengths, *filter_spatial_lengths,
+                            *output_spatial_lengths, *conv_filter_strides, *conv_filter_dilations,
+                            *input_left_pads, *input_right_pads)
+        return _ConvArgument(p_in, p_wei, p_out, d, out_element_op or PassThrough())
+
+    def _supported(self, a):
+        return capi.lib().ckx_conv2d_fwd_is_supported(self.op_family, C.byref(a.desc), a.out_op.epilogue,
+                                                      self.instance)
+
+
+class DeviceConv2dFwdInt8(_DeviceConvFwd):
+    op_family = capi.OP_CONV2D_FWD_I8
+
+    def _launch(self, a, stream):
+        return capi.lib().ckx_conv2d_fwd_i8(a.p_in, a.p_wei, a.p_out, C.byref(a.desc), a.out_op.epilogue,
+                                            a.out_op.scale_gemm, a.out_op.scale_relu, self.instance,
+                                            C.c_void_p(stream or 0))
+
+
+class DeviceConv2dFwdF16(_DeviceConvFwd):
+    op_family = capi.OP_CONV2D_FWD_F16
+
+    def _launch(self, a, stream):
+        return capi.lib().ckx_conv2d_fwd_f16(a.p_in, a.p_wei, a.p_out, C.byref(a.desc), self.instance,
+                                             C.c_void_p(stream or 0))
+
+
+# --------------------------------------------------------------- GEMM-GEMM
+class _GemmGemmArgument(BaseArgument):
+    pass
+
+
+class DeviceBatchedGemmGemmF16(BaseOperator):
+    """DeviceBatchedGemmGemm<Row, Col, Row, Row, half x4, PassThrough x5>"""
+    op_family = capi.OP_BATCHED_GEMM_GEMM
+
+    def MakeArgumentPointer(self, p_a, p_b0, p_b1, p_c, M, N, K, O, Batch, StrideA, StrideB0, StrideB1,
+                            StrideC, BatchStrideA, BatchStrideB0, BatchStrideB1, BatchStrideC,
+                            a_element_op=None, b0_element_op=None, acc0_element_op=None,
+                            b1_element_op=None, c_element_op=None):
+        for op in (a_element_op, b0_element_op, acc0_element_op, b1_element_op, c_element_op):
+            if op is not None and not isinstance(op, PassThrough):
+                raise TypeError("only PassThrough element-wise operations are built")
+        a = _GemmGemmArgument()
+        a.ptrs = (_ptr(p_a), _ptr(p_b0), _ptr(p_b1), _ptr(p_c))
+        a.dims = (int(M), int(N), int(K), int(O), int(Batch), int(StrideA), int(StrideB0), int(StrideB1),
+                  int(StrideC), int(BatchStrideA), int(BatchStrideB0), int(BatchStrideB1), int(BatchStrideC))
+        return a
+
+    def _supported(self, a):
+        return capi.lib().ckx_batched_gemm_gemm_f16_is_supported(*a.dims, self.instance)
+
+    def _launch(self, a, stream):
+        return capi.lib().ckx_batched_gemm_gemm_f16(*a.ptrs, *a.dims, self.instance, C.c_void_p(stream or 0))

@@ -1,0 +1,158 @@
+/*
+ * ckx.h -- C ABI of the MI355X (gfx950) MFMA GEMM hot path.
+ *
+ * Every entry point replaces the launch half of one Composable Kernel device
+ * operator (MakeArgumentPointer + IsSupportedArgument + Invoker::Run); the C++
+ * operator classes in composable_kernel_amd/host/ckx/device_ops.hpp sit on top of
+ * these calls and carry CK's own interface. All pointers are DEVICE pointers,
+ * strides are in ELEMENTS, dimensions are int32 (CK's index_t, include/ck/ck.hpp:176),
+ * `stream` is a hipStream_t passed as void* (NULL = default stream). Launches are
+ * asynchronous; nothing is allocated, nothing is synchronised.
+ *
+ * Return value: 0 on success, a negative ckx_status otherwise; the message for
+ * the calling thread's last failure is returned by ckx_last_error().
+ */
+#ifndef CKX_H_
+#define CKX_H_
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef enum ckx_status
+{
+    CKX_OK            = 0,
+    CKX_UNSUPPORTED   = -1, /* IsSupportedArgument would be false */
+    CKX_INVALID_VALUE = -2, /* null pointer, negative size, unknown enum */
+    CKX_HIP_ERROR     = -3  /* launch failed; ckx_last_error() has hipGetErrorString */
+} ckx_status;
+
+/* tensor_layout::gemm::{RowMajor,ColumnMajor}
+ * (include/ck/tensor_operation/gpu/device/tensor_layout.hpp) */
+enum
+{
+    CKX_ROW_MAJOR = 0,
+    CKX_COL_MAJOR = 1
+};
+
+/* C / Out element-wise operation applied to the accumulator before the store.
+ *  PASSTHROUGH  element_wise::PassThrough (unary_element_wise_operation.hpp:13-25);
+ *               int8 output keeps the low byte of the int32 accumulator.
+ *  REQUANT_CK   RequantReluRequant, literal
+ *               (example/14_gemm_xdl_requant_relu_requant/gemm_xdl_requant_relu_requant_int8.cpp:21-39):
+ *               y = clamp(sR * relu(sG * acc), -128, 127), then truncation toward zero.
+ *  REQUANT_RND  y = sat8(rint(sR * relu(sat8(rint(sG * acc))))), rint = half-to-even.
+ * All arithmetic is fp32 on the exactly converted int32 accumulator, two separate
+ * multiplies, no contraction. */
+enum
+{
+    CKX_EPI_PASSTHROUGH = 0,
+    CKX_EPI_REQUANT_CK  = 1,
+    CKX_EPI_REQUANT_RND = 2
+};
+
+/* Operator families, for the instance queries below. */
+enum
+{
+    CKX_OP_GEMM_I8           = 0,
+    CKX_OP_GEMM_F16          = 1,
+    CKX_OP_CONV2D_FWD_I8     = 2,
+    CKX_OP_CONV2D_FWD_F16    = 3,
+    CKX_OP_BATCHED_GEMM_GEMM = 4
+};
+
+#define CKX_INSTANCE_AUTO (-1)
+
+/* ---- library ------------------------------------------------------------ */
+const char* ckx_version(void);
+const char* ckx_last_error(void);
+
+/* Instance list of one operator family: what
+ * DeviceOperationInstanceFactory<DeviceOp>::GetInstances() enumerates
+ * (library/include/ck/library/tensor_operation_instance/gpu/gemm.hpp:233-379).
+ * ckx_instance_name() is the GetTypeString() of that instance
+ * (device_gemm_xdl_cshuffle.hpp:655-672). */
+int ckx_num_instances(int op);
+const char* ckx_instance_name(int op, int instance);
+
+/* ---- int8 GEMM:  C = c_op(A * B), int32 accumulation ----------------------
+ * Replaces DeviceGemm<..., int8_t, int8_t, int8_t, PassThrough, PassThrough, COp>
+ * ::MakeArgumentPointer + Invoker::Run (device_gemm.hpp:24-41,
+ * device_gemm_xdl_cshuffle.hpp:399-556) and kernel_gemm_xdl_cshuffle_v1
+ * (gridwise_gemm_xdl_cshuffle_v1.hpp:32-74).
+ * A is [M,K], B is [K,N], C is [M,N]; *_layout selects which stride is 1. */
+int ckx_gemm_i8_is_supported(int32_t M, int32_t N, int32_t K, int32_t stride_a, int32_t stride_b,
+                             int32_t stride_c, int a_layout, int b_layout, int c_layout, int epilogue,
+                             int instance);
+int ckx_gemm_i8(const void* p_a, const void* p_b, void* p_c, int32_t M, int32_t N, int32_t K,
+                int32_t stride_a, int32_t stride_b, int32_t stride_c, int a_layout, int b_layout,
+                int c_layout, int epilogue, float scale_gemm, float scale_relu, int instance,
+                void* stream);
+
+/* ---- fp16 GEMM:  C = half(A * B), fp32 accumulation -----------------------
+ * Replaces DeviceGemm<..., half_t, half_t, half_t, PassThrough x3>
+ * (device_gemm.hpp:24-41; device_gemm_xdl.hpp:60-545, kernel_gemm_xdlops_v2r3). */
+int ckx_gemm_f16_is_supported(int32_t M, int32_t N, int32_t K, int32_t stride_a, int32_t stride_b,
+                              int32_t stride_c, int a_layout, int b_layout, int c_layout, int instance);
+int ckx_gemm_f16(const void* p_a, const void* p_b, void* p_c, int32_t M, int32_t N, int32_t K,
+                 int32_t stride_a, int32_t stride_b, int32_t stride_c, int a_layout, int b_layout,
+                 int c_layout, int instance, void* stream);
+
+/* ---- conv2d forward, NHWC input / KYXC weight / NHWK output, implicit GEMM --
+ * Replaces DeviceConvFwd<PassThrough, PassThrough, OutOp>::MakeArgumentPointer + Run
+ * (device_conv_fwd.hpp:18-39) as implemented by
+ * DeviceConv2dFwdXdl_Input_N_Hi_Wi_C_Weight_K_Y_X_C_Output_N_Ho_Wo_K
+ * (device_conv2d_fwd_xdl_nhwc_kyxc_nhwk.hpp:57-720).
+ * The vectors of the reference interface are passed as scalars in (H, W) order:
+ * in_spatial = {Hi, Wi}, filter = {Y, X}, out_spatial = {Ho, Wo}, strides = {sH, sW},
+ * dilations = {dH, dW}, left pads = {pad_top, pad_left}, right pads = {pad_bottom, pad_right}. */
+typedef struct ckx_conv2d_desc
+{
+    int32_t N, K, C;
+    int32_t Hi, Wi;
+    int32_t Y, X;
+    int32_t Ho, Wo;
+    int32_t stride_h, stride_w;
+    int32_t dilation_h, dilation_w;
+    int32_t pad_top, pad_left;
+    int32_t pad_bottom, pad_right;
+} ckx_conv2d_desc;
+
+int ckx_conv2d_fwd_is_supported(int op, const ckx_conv2d_desc* desc, int epilogue, int instance);
+int ckx_conv2d_fwd_i8(const void* p_in, const void* p_wei, void* p_out, const ckx_conv2d_desc* desc,
+                      int epilogue, float scale_gemm, float scale_relu, int instance, void* stream);
+int ckx_conv2d_fwd_f16(const void* p_in, const void* p_wei, void* p_out, const ckx_conv2d_desc* desc,
+                       int instance, void* stream);
+
+/* ---- batched fused GEMM-GEMM, fp16:  C[g] = half( half(A[g]*B0[g]) * B1[g] ) --
+ * The reference snapshot has no such operator; the surface is upstream's
+ * DeviceBatchedGemmGemm::MakeArgumentPointer (device_batched_gemm_gemm.hpp:15-56 of
+ * later Composable Kernel releases), with the batch offsets of
+ * kernel_batched_gemm_xdlops_v2r3 (device_batched_gemm_xdl.hpp:49-117).
+ * Layout "gmk_gnk_gno_gmo": A [G,M,K] row-major, B0 column-major (memory [G,N,K]),
+ * B1 [G,N,O] row-major, C [G,M,O] row-major. The [M,N] intermediate stays on chip. */
+int ckx_batched_gemm_gemm_f16_is_supported(int32_t M, int32_t N, int32_t K, int32_t O, int32_t batch,
+                                           int32_t stride_a, int32_t stride_b0, int32_t stride_b1,
+                                           int32_t stride_c, int64_t batch_stride_a,
+                                           int64_t batch_stride_b0, int64_t batch_stride_b1,
+                                           int64_t batch_stride_c, int instance);
+int ckx_batched_gemm_gemm_f16(const void* p_a, const void* p_b0, const void* p_b1, void* p_c, int32_t M,
+                              int32_t N, int32_t K, int32_t O, int32_t batch, int32_t stride_a,
+                              int32_t stride_b0, int32_t stride_b1, int32_t stride_c,
+                              int64_t batch_stride_a, int64_t batch_stride_b0, int64_t batch_stride_b1,
+                              int64_t batch_stride_c, int instance, void* stream);
+
+/* ---- timing helper --------------------------------------------------------
+ * launch_and_time_kernel (include/ck/device_utility/kernel_launch.hpp:13-74):
+ * `fn(user)` is called n_warmup times untimed, then n_repeat times between two
+ * HIP events recorded on `stream`; the mean milliseconds per call is stored in
+ * *ms. fn must enqueue its work on `stream` and return 0. */
+typedef int (*ckx_launch_fn)(void* user);
+int ckx_time_launches(ckx_launch_fn fn, void* user, int n_warmup, int n_repeat, void* stream, float* ms);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* CKX_H_ */

@@ -1,0 +1,84 @@
+"""Helpers shared by the GPU parity tests: device buffers come from torch (plumbing only),
+every computation goes through the C ABI of libckx.so."""
+import numpy as np
+import torch
+
+import composable_kernel_amd as ck
+from composable_kernel_amd import capi
+
+
+def dev(a):
+    return torch.from_numpy(np.ascontiguousarray(a)).cuda()
+
+
+def stream():
+    return torch.cuda.current_stream().cuda_stream
+
+
+def gemm_i8(a_mk, b_nk, c_op, instance=capi.INSTANCE_AUTO, ldc=None, time_kernel=False):
+    """A [M,K] row-major, B given as [N,K] (column-major K x N). Returns int8 [M,N] (and ms)."""
+    M, K = a_mk.shape
+    N = b_nk.shape[0]
+    ldc = ldc or N
+    da, db = dev(a_mk), dev(b_nk)
+    dc = torch.full((M, ldc), 77, dtype=torch.int8, device="cuda")
+    op = ck.DeviceGemmInt8(instance)
+    arg = op.MakeArgumentPointer(da, db, dc, M, N, K, a_mk.shape[1], b_nk.shape[1], ldc,
+                                 ck.PassThrough(), ck.PassThrough(), c_op)
+    assert op.IsSupportedArgument(arg), capi.last_error()
+    ms = op.MakeInvokerPointer().Run(arg, ck.StreamConfig(stream(), time_kernel))
+    torch.cuda.synchronize()
+    out = dc.cpu().numpy()
+    if ldc != N:
+        assert np.all(out[:, N:] == 77), "wrote outside the C rows"
+    return (out[:, :N], ms) if time_kernel else out[:, :N]
+
+
+def gemm_f16(a_mk, b_nk, instance=capi.INSTANCE_AUTO, time_kernel=False):
+    M, K = a_mk.shape
+    N = b_nk.shape[0]
+    da, db = dev(a_mk), dev(b_nk)
+    dc = torch.full((M, N), float("nan"), dtype=torch.float16, device="cuda")
+    op = ck.DeviceGemmF16(instance)
+    arg = op.MakeArgumentPointer(da, db, dc, M, N, K, K, K, N)
+    assert op.IsSupportedArgument(arg), capi.last_error()
+    ms = op.MakeInvokerPointer().Run(arg, ck.StreamConfig(stream(), time_kernel))
+    torch.cuda.synchronize()
+    out = dc.cpu().numpy()
+    return (out, ms) if time_kernel else out
+
+
+def conv2d_fwd(inp_nhwc, wei_kyxc, strides, dilations, pads, out_op=None, instance=capi.INSTANCE_AUTO,
+               right_pads=None):
+    N, Hi, Wi, C = inp_nhwc.shape
+    K, Y, X, _ = wei_kyxc.shape
+    right_pads = right_pads or pads
+    Ho = (Hi + pads[0] + right_pads[0] - ((Y - 1) * dilations[0] + 1)) // strides[0] + 1
+    Wo = (Wi + pads[1] + right_pads[1] - ((X - 1) * dilations[1] + 1)) // strides[1] + 1
+    di, dw = dev(inp_nhwc), dev(wei_kyxc)
+    if inp_nhwc.dtype == np.int8:
+        do = torch.full((N, Ho, Wo, K), 77, dtype=torch.int8, device="cuda")
+        op = ck.DeviceConv2dFwdInt8(instance)
+    else:
+        do = torch.full((N, Ho, Wo, K), float("nan"), dtype=torch.float16, device="cuda")
+        op = ck.DeviceConv2dFwdF16(instance)
+    arg = op.MakeArgumentPointer(di, dw, do, N, K, C, [Hi, Wi], [Y, X], [Ho, Wo], list(strides),
+                                 list(dilations), list(pads), list(right_pads), None, None, out_op)
+    assert op.IsSupportedArgument(arg), capi.last_error()
+    op.MakeInvokerPointer().Run(arg, ck.StreamConfig(stream()))
+    torch.cuda.synchronize()
+    return do.cpu().numpy()
+
+
+def gemm_gemm_f16(a_gmk, b0_gnk, b1_gno):
+    G, M, K = a_gmk.shape
+    N = b0_gnk.shape[1]
+    O = b1_gno.shape[2]
+    da, db0, db1 = dev(a_gmk), dev(b0_gnk), dev(b1_gno)
+    dc = torch.full((G, M, O), float("nan"), dtype=torch.float16, device="cuda")
+    op = ck.DeviceBatchedGemmGemmF16()
+    arg = op.MakeArgumentPointer(da, db0, db1, dc, M, N, K, O, G, K, K, O, O, M * K, N * K, N * O, M * O)
+    assert op.IsSupportedArgument(arg), capi.last_error()
+    op.MakeInvokerPointer().Run(arg, ck.StreamConfig(stream()))
+    torch.cuda.synchronize()
+    return dc.cpu().numpy()
