@@ -1,0 +1,238 @@
+#!/usr/bin/env python3
+"""Benchmark of the MFMA GEMM hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--all] [--no-cpu]
+
+A "step" is one launch of the workload's kernel over synthetic inputs that are already resident
+in HBM. The default workload is BASELINE.json's configs[1], the fp16 GEMM at 4096^3 on which the
+metric (TFLOP/s and fraction of the dense fp16 MFMA peak) is quoted; the int8 half of the metric
+(4096^3 requant GEMM, TOP/s) and every other config are measured too and attached under "also".
+Prints ONE JSON line on stdout.
+
+Timing: W untimed launches, then K launches between two events recorded on the launch stream
+(torch's current stream, whose handle is what the C ABI receives), bracketed by device
+synchronisation; wall-clock over the same region gives ms_per_step.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+PEAK = {"f16": 2516.6, "i8": 5033.2}   # dense MFMA TFLOP/s / TOP/s, 256 CUs x 2.4 GHz
+HBM_PEAK_GBS = 8000.0
+
+
+def _conv_workload(name, dtype, C, K, f, HW, st, pd, N=256):
+    Ho = (HW + 2 * pd - f) // st + 1
+    ops = 2.0 * N * K * Ho * Ho * C * f * f
+    es = 1 if dtype == "i8" else 2
+    touched_in = N * HW * HW * C if st == 1 or f > 1 else N * Ho * Ho * C
+    byts = (touched_in + K * f * f * C + N * Ho * Ho * K) * es
+    return dict(name=name, kind="conv", dtype=dtype, N=N, C=C, K=K, f=f, HW=HW, st=st, pd=pd, ops=ops, bytes=byts)
+
+
+def _gemm_workload(name, dtype, M, N, K, values=5, scales=(0.5, 0.03)):
+    es = 1 if dtype == "i8" else 2
+    return dict(name=name, kind="gemm", dtype=dtype, M=M, N=N, K=K, values=values, scales=scales,
+                ops=2.0 * M * N * K, bytes=(M * K + N * K + M * N) * es)
+
+
+WORKLOADS = {}
+for w in (
+    [_gemm_workload("fp16_gemm_4096", "f16", 4096, 4096, 4096),
+     _gemm_workload("int8_requant_gemm_4096", "i8", 4096, 4096, 4096),
+     _gemm_workload("int8_requant_gemm_1024", "i8", 1024, 1024, 1024)]
+    + [_gemm_workload(f"int8_requant_llm_m{m}_n11008_k4096", "i8", m, 11008, 4096, 8, (0.02, 0.4)) for m in (1, 16, 128, 4096)]
+    + [_gemm_workload(f"int8_requant_llm_m{m}_n4096_k11008", "i8", m, 4096, 11008, 8, (0.02, 0.4)) for m in (1, 16, 128, 4096)]
+    + [_conv_workload(f"conv_{dt}_c64_k64_3x3_56", dt, 64, 64, 3, 56, 1, 1) for dt in ("f16", "i8")]
+    + [_conv_workload(f"conv_{dt}_c256_k512_1x1_56_s2", dt, 256, 512, 1, 56, 2, 0) for dt in ("f16", "i8")]
+    + [_conv_workload(f"conv_{dt}_c512_k512_3x3_7", dt, 512, 512, 3, 7, 1, 1) for dt in ("f16", "i8")]
+    + [dict(name="gemm_gemm_f16_b64_512x64x512x64", kind="gemm_gemm", dtype="f16", G=64, M=512, N=512, K=64, O=64,
+            ops=2.0 * 64 * 512 * 512 * 64 * 2, bytes=4 * 64 * 512 * 64 * 2)]
+):
+    WORKLOADS[w["name"]] = w
+
+
+def make_launcher(w, instance=-1):
+    """Allocates the workload's synthetic operands on the GPU, returns (launch_fn, description)."""
+    import torch
+    import composable_kernel_amd as ck
+    from composable_kernel_amd import capi
+    from composable_kernel_amd.host_tensor import uniform_f16, uniform_int8
+
+    stream = torch.cuda.current_stream().cuda_stream
+    keep = []
+
+    def dev(a):
+        t = torch.from_numpy(a).cuda()
+        keep.append(t)
+        return t
+
+    if w["kind"] == "gemm":
+        M, N, K = w["M"], w["N"], w["K"]
+        if w["dtype"] == "i8":
+            a, b = dev(uniform_int8((M, K), -w["values"], w["values"], 1)), dev(uniform_int8((N, K), -w["values"], w["values"], 2))
+            c = torch.empty((M, N), dtype=torch.int8, device="cuda")
+            op = ck.DeviceGemmInt8(instance)
+            cop = ck.RequantReluRequant(w["scales"][0], w["scales"][1], rounded=True)
+        else:
+            a, b = dev(uniform_f16((M, K), -1, 1, 1)), dev(uniform_f16((N, K), -1, 1, 2))
+            c = torch.empty((M, N), dtype=torch.float16, device="cuda")
+            op = ck.DeviceGemmF16(instance)
+            cop = ck.PassThrough()
+        arg = op.MakeArgumentPointer(a, b, c, M, N, K, K, K, N, None, None, cop)
+    elif w["kind"] == "conv":
+        N, C, K, f, HW, st, pd = (w[k] for k in ("N", "C", "K", "f", "HW", "st", "pd"))
+        Ho = (HW + 2 * pd - f) // st + 1
+        if w["dtype"] == "i8":
+            i, wt = dev(uniform_int8((N, HW, HW, C), -5, 5, 3)), dev(uniform_int8((K, f, f, C), -5, 5, 4))
+            c = torch.empty((N, Ho, Ho, K), dtype=torch.int8, device="cuda")
+            op = ck.DeviceConv2dFwdInt8(instance)
+            cop = ck.RequantReluRequant(0.01, 0.5, rounded=True)
+        else:
+            i, wt = dev(uniform_f16((N, HW, HW, C), -1, 1, 3)), dev(uniform_f16((K, f, f, C), -1, 1, 4))
+            c = torch.empty((N, Ho, Ho, K), dtype=torch.float16, device="cuda")
+            op = ck.DeviceConv2dFwdF16(instance)
+            cop = ck.PassThrough()
+        arg = op.MakeArgumentPointer(i, wt, c, N, K, C, [HW, HW], [f, f], [Ho, Ho], [st, st], [1, 1], [pd, pd],
+                                     [pd, pd], None, None, cop)
+    else:
+        G, M, N, K, O = (w[k] for k in ("G", "M", "N", "K", "O"))
+        a, b0, b1 = (dev(uniform_f16(s, -0.5, 0.5, 5 + j)) for j, s in enumerate([(G, M, K), (G, N, K), (G, N, O)]))
+        c = torch.empty((G, M, O), dtype=torch.float16, device="cuda")
+        op = ck.DeviceBatchedGemmGemmF16(instance)
+        arg = op.MakeArgumentPointer(a, b0, b1, c, M, N, K, O, G, K, K, O, O, M * K, N * K, N * O, M * O)
+    keep.append(c)
+    if not op.IsSupportedArgument(arg):
+        raise RuntimeError(f"{w['name']}: not supported: {capi.last_error()}")
+
+    def launch():
+        st_ = op._launch(arg, stream)
+        if st_ != 0:
+            raise RuntimeError(capi.last_error())
+
+    launch.keep = keep
+    return launch
+
+
+def time_workload(w, steps, warmup, instance=-1):
+    import torch
+    launch = make_launcher(w, instance)
+    for _ in range(warmup):
+        launch()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    e0.record()
+    for _ in range(steps):
+        launch()
+    e1.record()
+    torch.cuda.synchronize()
+    wall_ms = (time.perf_counter() - t0) * 1e3 / steps
+    ev_ms = e0.elapsed_time(e1) / steps
+    tput = w["ops"] / (ev_ms * 1e-3) / 1e12
+    gbs = w["bytes"] / (ev_ms * 1e-3) / 1e9
+    compute_frac = tput / PEAK[w["dtype"]]
+    hbm_frac = gbs / HBM_PEAK_GBS
+    bound = "mfma" if compute_frac >= hbm_frac else "hbm"
+    return dict(workload=w["name"], dtype=w["dtype"], ms=ev_ms, wall_ms=wall_ms, tput=tput, gbs=gbs,
+                mfma_frac=compute_frac, hbm_frac=hbm_frac, bound=bound)
+
+
+def cpu_baseline(w, target_seconds=12.0):
+    """The oracle's literal ReferenceGemm restatement on a bounded row sample of the same
+    workload, on the host cores of this box."""
+    from oracle import lit
+    from composable_kernel_amd.host_tensor import uniform_f16, uniform_int8
+    threads = max(1, min(16, os.cpu_count() or 1))
+    N, K = w["N"], w["K"]
+    if w["dtype"] == "f16":
+        b = uniform_f16((N, K), -1, 1, 2)
+        mk = lambda m: uniform_f16((m, K), -1, 1, 1)
+        run = lambda a: lit.gemm_f16(a, b.T, nthreads=threads)
+    else:
+        b = uniform_int8((N, K), -5, 5, 2)
+        mk = lambda m: uniform_int8((m, K), -5, 5, 1)
+        run = lambda a: lit.gemm_i8(a, b.T, lit.EPI_REQUANT_RND, 0.5, 0.03, nthreads=threads)
+    m0 = 2 * threads
+    t0 = time.perf_counter()
+    run(mk(m0))
+    dt = max(time.perf_counter() - t0, 1e-4)
+    rows = int(min(w["M"], max(m0, m0 * target_seconds / dt)))
+    a = mk(rows)
+    t0 = time.perf_counter()
+    run(a)
+    dt = time.perf_counter() - t0
+    unit = "TFLOP/s" if w["dtype"] == "f16" else "TOP/s"
+    return {"value": 2.0 * rows * N * K / dt / 1e12, "unit": unit, "cores": threads, "kind": "port",
+            "sample": f"{rows} of {w['M']} rows of the same {w['M']}x{N}x{K} problem, literal ReferenceGemm "
+                      f"restatement (oracle/ck_oracle.cpp), {dt:.1f} s"}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--workload", default="fp16_gemm_4096")
+    ap.add_argument("--instance", type=int, default=-1)
+    ap.add_argument("--all", action="store_true", help="also time every other config (reported under 'also')")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this hot path is a single-GPU kernel library; run with --gpus 1 "
+              "(sharding is over independent output tiles, see DESIGN.md)", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        sys.exit(1)
+    from composable_kernel_amd import capi
+    capi.lib()   # fail loudly if the HIP library is missing
+
+    w = WORKLOADS[args.workload]
+    r = time_workload(w, args.steps, args.warmup, args.instance)
+    also = []
+    extra = ["int8_requant_gemm_4096"] if args.workload == "fp16_gemm_4096" else []
+    if args.all:
+        extra = [n for n in WORKLOADS if n != args.workload]
+    for n in extra:
+        x = time_workload(WORKLOADS[n], max(10, args.steps // 2), max(3, args.warmup // 2))
+        also.append({"workload": n, "dtype": x["dtype"], "ms": round(x["ms"], 5),
+                     "value": round(x["tput"], 2), "unit": "TOP/s" if x["dtype"] == "i8" else "TFLOP/s",
+                     "GB/s": round(x["gbs"], 1), "bound": x["bound"],
+                     "frac_of_bound": round(max(x["mfma_frac"], x["hbm_frac"]), 4)})
+
+    unit = "TFLOP/s" if w["dtype"] == "f16" else "TOP/s"
+    if r["bound"] == "mfma":
+        roof = {"bound": "mfma", "achieved": round(r["tput"], 2), "peak": PEAK[w["dtype"]], "unit": unit,
+                "frac": round(r["mfma_frac"], 4), "traffic": None}
+    else:
+        roof = {"bound": "hbm", "achieved": round(r["gbs"], 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                "frac": round(r["hbm_frac"], 4), "traffic": None}
+    line = {
+        "metric": "int8 TOPS & fp16 TFLOPS at 4096^3 on 1 MI355X; % of dtype MFMA peak",
+        "value": round(r["tput"], 2), "unit": unit, "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(r["wall_ms"], 5), "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "f16" if w["dtype"] == "f16" else "i8", "data": "synthetic",
+        "config": {"workload": w["name"], "layout": "A row-major, B column-major, C row-major",
+                   "accumulate": "fp32" if w["dtype"] == "f16" else "int32",
+                   "ops_per_step": w["ops"], "algorithmic_bytes_per_step": w["bytes"]},
+        "roofline": roof,
+        "kernel_ms": round(r["ms"], 5),
+        "also": also,
+    }
+    if not args.no_cpu:
+        line["cpu_baseline"] = cpu_baseline(w)
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()
