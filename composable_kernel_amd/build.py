@@ -51,5 +51,37 @@ def build_lib(force=False, verbose=False, extra_flags=()):
     return LIB
 
 
+HOST = os.path.join(HERE, "host")
+BINDIR = os.path.join(HERE, "bin")
+HOST_PROGRAMS = {
+    "ckx_profiler": os.path.join(HOST, "profiler", "ckx_profiler.cpp"),
+    "example_gemm_requant_relu_requant_int8": os.path.join(HOST, "example", "gemm_requant_relu_requant_int8.cpp"),
+}
+
+
+def build_host(force=False, verbose=False):
+    """Compile the C++ host programs (operator classes are header-only) against libckx.so."""
+    build_lib()
+    os.makedirs(BINDIR, exist_ok=True)
+    hdrs = [os.path.join(HOST, "ckx", f) for f in os.listdir(os.path.join(HOST, "ckx"))] + [LIB]
+    out = []
+    for name, src in HOST_PROGRAMS.items():
+        exe = os.path.join(BINDIR, name)
+        out.append(exe)
+        if not force and os.path.exists(exe) and all(os.path.getmtime(exe) >= os.path.getmtime(p) for p in hdrs + [src]):
+            continue
+        cmd = [HIPCC, "-x", "c++", "-std=c++17", "-O2", "-D__HIP_PLATFORM_AMD__", "-I/opt/rocm/include",
+               "-I" + os.path.join(ROOT, "include"), "-I" + HOST, src, "-x", "none", "-o", exe,
+               "-L" + LIBDIR, "-lckx", "-L/opt/rocm/lib", "-lamdhip64", "-Wl,-rpath,$ORIGIN/../lib",
+               "-Wl,-rpath,/opt/rocm/lib", "-Wno-unused-command-line-argument"]
+        if verbose:
+            print(" ".join(cmd))
+        r = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+        if r.returncode != 0:
+            raise RuntimeError("host build failed:\n" + r.stdout)
+    return out
+
+
 if __name__ == "__main__":
+    print(build_host(force="--force" in sys.argv, verbose=True))
     print(build_lib(force="--force" in sys.argv, verbose=True))

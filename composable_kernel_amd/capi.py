@@ -8,7 +8,8 @@ import ctypes as C
 import os
 
 HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(HERE, "lib", "libckx.so")
+# CKX_LIB_PATH selects another build of the same library (A/B comparisons of tuning variants)
+LIB_PATH = os.environ.get("CKX_LIB_PATH") or os.path.join(HERE, "lib", "libckx.so")
 
 OK, UNSUPPORTED, INVALID_VALUE, HIP_ERROR = 0, -1, -2, -3
 ROW_MAJOR, COL_MAJOR = 0, 1

@@ -44,11 +44,11 @@ ckx::MagicDiv make_magic(uint32_t d)
 // ------------------------------------------------------------ tile instances
 typedef hipError_t (*tile_launch_fn)(const ckx::GemmArgs&, int grid, hipStream_t);
 
-template <int DT, int BM, int BN, int WM, int WN, bool IM2COL>
+template <int DT, int BM, int BN, int WM, int WN, int BKB, int NST, bool IM2COL, bool PP>
 hipError_t launch_tile(const ckx::GemmArgs& a, int grid, hipStream_t s)
 {
-    using T              = ckx::GemmTile<DT, BM, BN, WM, WN, IM2COL>;
-    auto* kern           = &ckx::gemm_tile_kernel<DT, BM, BN, WM, WN, IM2COL>;
+    using T              = ckx::GemmTile<DT, BM, BN, WM, WN, BKB, NST, IM2COL, PP>;
+    auto* kern           = &ckx::gemm_tile_kernel<DT, BM, BN, WM, WN, BKB, NST, IM2COL, PP>;
     static std::once_flag once;
     static hipError_t attr_err = hipSuccess;
     std::call_once(once, [&] {
@@ -68,22 +68,25 @@ struct TileInstance
     tile_launch_fn dense_i8, dense_f16, conv_i8, conv_f16;
 };
 
-#define CKX_TILE(BM, BN, WM, WN)                                                                      \
-    {                                                                                                 \
-        "MI355X_Mfma16_Tile<" #BM ", " #BN ", 128B, waves " #WM "x" #WN ">", BM, BN, WM* WN * 64,          \
-            &launch_tile<ckx::DT_I8, BM, BN, WM, WN, false>, &launch_tile<ckx::DT_F16, BM, BN, WM, WN, false>, \
-            &launch_tile<ckx::DT_I8, BM, BN, WM, WN, true>, &launch_tile<ckx::DT_F16, BM, BN, WM, WN, true>    \
+#define CKX_TILE(BM, BN, WM, WN, BKB, NST, PP)                                                          \
+    {                                                                                                   \
+        "MI355X_Mfma16_Tile<" #BM ", " #BN ", " #BKB "B x" #NST ", waves " #WM "x" #WN ", pp" #PP ">", BM, BN,     \
+            WM* WN * 64, &launch_tile<ckx::DT_I8, BM, BN, WM, WN, BKB, NST, false, PP>,                       \
+            &launch_tile<ckx::DT_F16, BM, BN, WM, WN, BKB, NST, false, PP>,                                 \
+            &launch_tile<ckx::DT_I8, BM, BN, WM, WN, BKB, NST, true, PP>,                                   \
+            &launch_tile<ckx::DT_F16, BM, BN, WM, WN, BKB, NST, true, PP>                                   \
     }
 
 const TileInstance kTiles[] = {
-    CKX_TILE(256, 256, 2, 4),
-    CKX_TILE(256, 128, 4, 2),
-    CKX_TILE(128, 128, 2, 2),
-    CKX_TILE(128, 64, 4, 1),
-    CKX_TILE(64, 64, 4, 1),
-    CKX_TILE(32, 64, 2, 1),
-    CKX_TILE(16, 64, 1, 1),
-    CKX_TILE(256, 256, 2, 2),
+    CKX_TILE(256, 256, 2, 4, 128, 2, 0),
+    CKX_TILE(256, 128, 4, 2, 128, 2, 0),
+    CKX_TILE(128, 128, 2, 2, 128, 2, 0),
+    CKX_TILE(128, 64, 4, 1, 128, 2, 0),
+    CKX_TILE(64, 64, 4, 1, 128, 2, 0),
+    CKX_TILE(32, 64, 2, 1, 128, 2, 0),
+    CKX_TILE(16, 64, 1, 1, 128, 2, 0),
+    CKX_TILE(256, 256, 2, 4, 128, 2, 1),
+    CKX_TILE(256, 128, 4, 2, 128, 2, 1),
 };
 constexpr int kNumTiles = sizeof(kTiles) / sizeof(kTiles[0]);
 

@@ -52,6 +52,16 @@ enum
 #ifndef CKX_SWZ_SHIFT
 #define CKX_SWZ_SHIFT 0
 #endif
+// C tile stores: plain, or streaming (CKX_NT_STORE) so the lines do not linger dirty in L2
+#ifdef CKX_NT_STORE
+#define CKX_STORE(ptr, val) __builtin_nontemporal_store((val), (ptr))
+#else
+#define CKX_STORE(ptr, val) (*(ptr) = (val))
+#endif
+// which of the two ping-pong groups a wave belongs to: waves w and w+4 share a SIMD
+#ifndef CKX_PP_GROUP
+#define CKX_PP_GROUP(wave) ((wave) >> 2)
+#endif
 
 // q = n / d for 0 <= n < 2^31 (include/ck/utility/magic_division.hpp:28-54,132-137)
 struct MagicDiv
@@ -96,13 +106,6 @@ struct GemmArgs
 
 constexpr uint32_t kOutOfRange = 0x80000000u;
 
-__device__ __forceinline__ uint32_t swz(uint32_t row) { return (row >> CKX_SWZ_SHIFT) & 7u; }
-
-__device__ __forceinline__ uint32_t lds_chunk_offset(uint32_t row, uint32_t chunk)
-{
-    return row * 128u + ((chunk ^ swz(row)) << 4);
-}
-
 // LDS row (position in the staged B tile) -> column of the tile. Within a 64-column group,
 // LDS row 16*t + j (MFMA tile t, MFMA row j) holds column 16*(j/4) + 4*t + j%4.
 __device__ __forceinline__ uint32_t b_row_to_col(uint32_t r)
@@ -140,13 +143,17 @@ __device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* p, uint3
 typedef __attribute__((address_space(3))) void* lds_ptr_t;
 
 // ---------------------------------------------------------------- epilogues
+// All in fp32 on the exactly converted int32 accumulator; the two multiplies are separate
+// roundings (the translation unit is built with -ffp-contract=off). v_med3_f32 does a
+// two-sided clamp in one instruction; "clamp to [-128,127] then ReLU" is the single clamp
+// to [0,127]. Scales are finite by contract, so no NaN reaches the min/max/med3 forms.
 __device__ __forceinline__ int requant_ck(int acc, float sg, float sr)
 {
     float x = (float)acc;
     float g = sg * x;
-    float r = g > 0.0f ? g : 0.0f;
+    float r = __builtin_fmaxf(g, 0.0f);
     float q = sr * r;
-    float y = q > 127.0f ? 127.0f : (q < -128.0f ? -128.0f : q);
+    float y = __builtin_amdgcn_fmed3f(q, -128.0f, 127.0f);
     return (int)y; // toward zero
 }
 
@@ -154,10 +161,9 @@ __device__ __forceinline__ int requant_rnd(int acc, float sg, float sr)
 {
     float x = (float)acc;
     float t = __builtin_rintf(sg * x);
-    t       = t > 127.0f ? 127.0f : (t < -128.0f ? -128.0f : t);
-    float r = t > 0.0f ? t : 0.0f;
+    float r = __builtin_amdgcn_fmed3f(t, 0.0f, 127.0f);
     float u = __builtin_rintf(sr * r);
-    u       = u > 127.0f ? 127.0f : (u < -128.0f ? -128.0f : u);
+    u       = __builtin_amdgcn_fmed3f(u, -128.0f, 127.0f);
     return (int)u;
 }
 
@@ -165,11 +171,19 @@ template <int EPI>
 __device__ __forceinline__ int epilogue_i8(int acc, float sg, float sr)
 {
     if constexpr(EPI == EPI_REQUANT_CK)
-        return requant_ck(acc, sg, sr) & 0xFF;
+        return requant_ck(acc, sg, sr);
     else if constexpr(EPI == EPI_REQUANT_RND)
-        return requant_rnd(acc, sg, sr) & 0xFF;
+        return requant_rnd(acc, sg, sr);
     else
-        return acc & 0xFF;
+        return acc;
+}
+
+// low bytes of four ints -> one dword (b0 in bits 0-7): three byte permutes
+__device__ __forceinline__ int pack4_low_bytes(int b0, int b1, int b2, int b3)
+{
+    const uint32_t lo = __builtin_amdgcn_perm((uint32_t)b1, (uint32_t)b0, 0x0c0c0400u);
+    const uint32_t hi = __builtin_amdgcn_perm((uint32_t)b3, (uint32_t)b2, 0x0c0c0400u);
+    return (int)__builtin_amdgcn_perm(hi, lo, 0x05040100u);
 }
 
 // 16 consecutive int8 outputs of one row
@@ -188,8 +202,8 @@ __device__ __forceinline__ void store_row16_i8(int8_t* crow, int n0, int N, bool
         i32x4 pk;
 #pragma unroll
         for(int w = 0; w < 4; ++w)
-            pk[w] = b[4 * w] | (b[4 * w + 1] << 8) | (b[4 * w + 2] << 16) | (b[4 * w + 3] << 24);
-        *reinterpret_cast<i32x4*>(crow + n0) = pk;
+            pk[w] = pack4_low_bytes(b[4 * w], b[4 * w + 1], b[4 * w + 2], b[4 * w + 3]);
+        CKX_STORE(reinterpret_cast<i32x4*>(crow + n0), pk);
     }
     else
     {
@@ -214,8 +228,8 @@ __device__ __forceinline__ void store_row16_f16(_Float16* crow, int n0, int N, b
             hi[j]     = (_Float16)v[2][j];
             hi[4 + j] = (_Float16)v[3][j];
         }
-        *reinterpret_cast<f16x8*>(crow + n0)     = lo;
-        *reinterpret_cast<f16x8*>(crow + n0 + 8) = hi;
+        CKX_STORE(reinterpret_cast<f16x8*>(crow + n0), lo);
+        CKX_STORE(reinterpret_cast<f16x8*>(crow + n0 + 8), hi);
     }
     else
     {
@@ -229,28 +243,48 @@ __device__ __forceinline__ void store_row16_f16(_Float16* crow, int n0, int N, b
 }
 
 // ------------------------------------------------------------------- kernel
-template <int DT, int BM, int BN, int WM, int WN, bool IM2COL>
+// BKB   bytes of every row staged per K tile (64 or 128)
+// NST   LDS stages; the loads of K tile k+NST-1 are issued while tile k is multiplied
+template <int DT, int BM, int BN, int WM, int WN, int BKB, int NST, bool IM2COL, bool PINGPONG = false>
 struct GemmTile
 {
     static constexpr int NW      = WM * WN;
     static constexpr int NT      = NW * 64;
     static constexpr int ES      = DT == DT_I8 ? 1 : 2;
-    static constexpr int CE      = 16 / ES; // elements per 16-byte chunk
-    static constexpr int BKE     = 128 / ES;
+    static constexpr int CPR     = BKB / 16;  // 16-byte chunks per staged row
+    static constexpr int RPI     = 64 / CPR;  // rows covered by one wave-wide direct load
+    static constexpr int KSTEPS  = BKB / 64;  // MFMA k-steps per K tile
     static constexpr int WTM     = BM / WM;
     static constexpr int WTN     = BN / WN;
     static constexpr int MT      = WTM / 16;
     static constexpr int NG      = WTN / 64;
-    static constexpr int A_TILE  = BM * 128;
-    static constexpr int B_TILE  = BN * 128;
+    static constexpr int A_TILE  = BM * BKB;
+    static constexpr int B_TILE  = BN * BKB;
     static constexpr int STAGE   = A_TILE + B_TILE;
-    static constexpr int LDS     = 2 * STAGE;
-    static constexpr int NLA     = BM * 8 / NT; // 16-byte loads per thread and K tile, A
-    static constexpr int NLB     = BN * 8 / NT;
+    static constexpr int LDS     = NST * STAGE;
+    static constexpr int NLA     = BM * CPR / NT; // 16-byte loads per thread and K tile, A
+    static constexpr int NLB     = BN * CPR / NT;
+    static constexpr int LPT     = NLA + NLB;
+    static_assert(BKB == 64 || BKB == 128, "K tile is 64 or 128 bytes per row");
+    static_assert(NST >= 2 && (NST - 2) * LPT < 64, "vmcnt is a 6-bit counter");
     static_assert(WTM % 16 == 0 && WTN % 64 == 0, "wave tile must be 16k x 64k");
-    static_assert((BM * 8) % NT == 0 && (BN * 8) % NT == 0, "tile rows must split over the waves");
+    static_assert((BM * CPR) % NT == 0 && (BN * CPR) % NT == 0, "tile rows must split over the waves");
 
     using acc_t = typename std::conditional<DT == DT_I8, i32x4, f32x4>::type;
+
+    // XOR swizzle of the chunk position: the 16 rows read by one MFMA fragment load spread
+    // over all LDS banks.
+    __device__ static __forceinline__ uint32_t swz(uint32_t row)
+    {
+        if constexpr(CPR == 8)
+            return (row >> CKX_SWZ_SHIFT) & 7u;
+        else
+            return (row >> 2) & 3u;
+    }
+    __device__ static __forceinline__ uint32_t chunk_offset(uint32_t row, uint32_t chunk)
+    {
+        return row * BKB + ((chunk ^ swz(row)) << 4);
+    }
 
     __device__ static void run(const GemmArgs& p, uint8_t* smem)
     {
@@ -264,13 +298,13 @@ struct GemmTile
         tile_of_block(blockIdx.x, p.tiles_m, p.tiles_n, tm, tn);
 
         const uint32_t kbytes = (uint32_t)p.K * ES;
-        const int nk          = (int)((kbytes + 127u) >> 7);
+        const int nk          = (int)((kbytes + BKB - 1) / BKB);
 
         const __amdgpu_buffer_rsrc_t rsrc_a = make_rsrc(p.a, p.a_bytes);
         const __amdgpu_buffer_rsrc_t rsrc_b = make_rsrc(p.b, p.b_bytes);
 
         // ---- per-thread load slots -------------------------------------------------
-        // slot j of this thread fills LDS row (j*NW + wave)*8 + lane/8, chunk position lane%8
+        // slot j of this thread fills LDS row (j*NW + wave)*RPI + lane/CPR, chunk position lane%CPR
         uint32_t a_off[NLA];  // dense: byte offset of (row, chunk) at K tile 0, or kOutOfRange
         uint32_t a_kb[NLA];   // byte offset of the chunk inside a K tile
         int a_hi0[NLA], a_wi0[NLA]; // im2col: top-left input coordinate of the row's window
@@ -279,8 +313,8 @@ struct GemmTile
 #pragma unroll
         for(int j = 0; j < NLA; ++j)
         {
-            const uint32_t r  = (uint32_t)((j * NW + wave) * 8 + (lane >> 3));
-            const uint32_t ch = (uint32_t)(lane & 7) ^ swz(r);
+            const uint32_t r  = (uint32_t)((j * NW + wave) * RPI + lane / CPR);
+            const uint32_t ch = (uint32_t)(lane % CPR) ^ swz(r);
             a_kb[j]           = ch << 4;
             const uint32_t gm = (uint32_t)tm * BM + r;
             if constexpr(!IM2COL)
@@ -310,18 +344,22 @@ struct GemmTile
 #pragma unroll
         for(int j = 0; j < NLB; ++j)
         {
-            const uint32_t r  = (uint32_t)((j * NW + wave) * 8 + (lane >> 3));
-            const uint32_t ch = (uint32_t)(lane & 7) ^ swz(r);
+            const uint32_t r  = (uint32_t)((j * NW + wave) * RPI + lane / CPR);
+            const uint32_t ch = (uint32_t)(lane % CPR) ^ swz(r);
             b_kb[j]           = ch << 4;
             const uint32_t gn = (uint32_t)tn * BN + b_row_to_col(r);
             b_off[j] = gn < (uint32_t)p.N ? gn * (uint32_t)p.ldb * ES + b_kb[j] : kOutOfRange;
         }
 
-        auto issue_loads = [&](int kt, int stage) {
+        // K tiles at or beyond nk are legal to request: every chunk of them is out of range,
+        // so the hardware writes zeros into a stage nobody reads. This keeps the number of
+        // loads in flight constant, which the vmcnt arithmetic below relies on.
+        auto issue_loads = [&](int kt) {
+            const int stage       = kt % NST;
             uint8_t* sa           = smem + stage * STAGE;
             uint8_t* sb           = sa + A_TILE;
-            const uint32_t k0     = (uint32_t)kt << 7; // byte offset of the K tile
-            const bool tail       = (k0 + 128u > kbytes);
+            const uint32_t k0     = (uint32_t)kt * BKB; // byte offset of the K tile
+            const bool tail       = (k0 + BKB > kbytes);
 #pragma unroll
             for(int j = 0; j < NLA; ++j)
             {
@@ -372,47 +410,143 @@ struct GemmTile
         const uint32_t frow = (uint32_t)(lane & 15);
         const uint32_t fq   = (uint32_t)(lane >> 4);
 
-        issue_loads(0, 0);
-
-        for(int kt = 0; kt < nk; ++kt)
-        {
-            __syncthreads(); // waits for this wave's direct loads, then for everybody's
-            if(kt + 1 < nk)
-                issue_loads(kt + 1, (kt + 1) & 1);
-
-            const uint8_t* sa = smem + (kt & 1) * STAGE;
-            const uint8_t* sb = sa + A_TILE;
+        auto read_frags = [&](const uint8_t* sa, const uint8_t* sb, int ks, i32x4(&af)[MT], i32x4(&bf)[NG * 4]) {
 #pragma unroll
-            for(int ks = 0; ks < 2; ++ks)
+            for(int i = 0; i < MT; ++i)
             {
-                i32x4 af[MT];
-                i32x4 bf[NG * 4];
+                const uint32_t row = (uint32_t)(wm * WTM + 16 * i) + frow;
+                af[i] = *reinterpret_cast<const i32x4*>(sa + chunk_offset(row, ks * 4 + fq));
+            }
 #pragma unroll
-                for(int i = 0; i < MT; ++i)
-                {
-                    const uint32_t row = (uint32_t)(wm * WTM + 16 * i) + frow;
-                    af[i] = *reinterpret_cast<const i32x4*>(sa + lds_chunk_offset(row, ks * 4 + fq));
-                }
+            for(int t = 0; t < NG * 4; ++t)
+            {
+                const uint32_t row = (uint32_t)(wn * WTN + 16 * t) + frow;
+                bf[t] = *reinterpret_cast<const i32x4*>(sb + chunk_offset(row, ks * 4 + fq));
+            }
+        };
+        auto mfma_block = [&](const i32x4(&af)[MT], const i32x4(&bf)[NG * 4]) {
+#pragma unroll
+            for(int i = 0; i < MT; ++i)
 #pragma unroll
                 for(int t = 0; t < NG * 4; ++t)
                 {
-                    const uint32_t row = (uint32_t)(wn * WTN + 16 * t) + frow;
-                    bf[t] = *reinterpret_cast<const i32x4*>(sb + lds_chunk_offset(row, ks * 4 + fq));
+                    if constexpr(DT == DT_I8)
+                        acc[i][t] = __builtin_amdgcn_mfma_i32_16x16x64_i8(bf[t], af[i], acc[i][t], 0, 0, 0);
+                    else
+                        acc[i][t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(
+                            __builtin_bit_cast(f16x8, bf[t]), __builtin_bit_cast(f16x8, af[i]), acc[i][t], 0, 0, 0);
                 }
+        };
+        // Tell the scheduler to keep the order written below: the LDS reads of the NEXT k-step
+        // are spread between the MFMAs of the CURRENT one (1 read : 2 MFMA, then the rest).
+        auto interleave = [&]() {
+            constexpr int NR = MT + NG * 4, NM = MT * NG * 4;
 #pragma unroll
-                for(int i = 0; i < MT; ++i)
-#pragma unroll
-                    for(int t = 0; t < NG * 4; ++t)
-                    {
-                        if constexpr(DT == DT_I8)
-                            acc[i][t] = __builtin_amdgcn_mfma_i32_16x16x64_i8(bf[t], af[i], acc[i][t], 0, 0, 0);
-                        else
-                            acc[i][t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(
-                                __builtin_bit_cast(f16x8, bf[t]), __builtin_bit_cast(f16x8, af[i]), acc[i][t], 0,
-                                0, 0);
-                    }
+            for(int r = 0; r < NR; ++r)
+            {
+                __builtin_amdgcn_sched_group_barrier(0x100, 1, 0); // DS read
+                __builtin_amdgcn_sched_group_barrier(0x008, (NM / NR) > 0 ? (NM / NR) : 1, 0); // MFMA
+            }
+            __builtin_amdgcn_sched_group_barrier(0x008, NM - NR * (NM / NR), 0);
+        };
+
+        static_assert(KSTEPS == 2 && NST == 2, "pipeline written for 128-byte K tiles, two stages");
+        i32x4 af0[MT], bf0[NG * 4], af1[MT], bf1[NG * 4];
+        auto barrier = [&]() {
+            __builtin_amdgcn_s_barrier();
+            asm volatile("" ::: "memory");
+        };
+
+        if constexpr(PINGPONG)
+        {
+            // Eight waves = two groups of four, one wave of each group per SIMD. The groups run
+            // the same two-segment loop (MEM: pull a whole K tile from LDS into registers;
+            // COMP: 2 x MT x NG*4 MFMAs straight from registers) half an iteration apart, so
+            // that on every SIMD one wave is always inside its MFMA burst while its partner
+            // does LDS reads, global->LDS load issue and waiting. Barrier B(2k) is the point at
+            // which tile k has landed for everybody and nobody reads tile k-1 any more; both
+            // groups issue the loads of tile k+1 right after it.
+            static_assert(NW == 8, "ping-pong needs two waves per SIMD");
+            const int group = CKX_PP_GROUP(wave);
+            issue_loads(0);
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+            barrier(); // B0
+            if(group == 0)
+            {
+                for(int kt = 0; kt < nk; ++kt)
+                {
+                    const uint8_t* sa = smem + (kt & 1) * STAGE;
+                    issue_loads(kt + 1);
+                    read_frags(sa, sa + A_TILE, 0, af0, bf0);
+                    read_frags(sa, sa + A_TILE, 1, af1, bf1);
+                    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+                    barrier(); // B(2kt+1)
+                    __builtin_amdgcn_s_setprio(1);
+                    mfma_block(af0, bf0);
+                    mfma_block(af1, bf1);
+                    __builtin_amdgcn_s_setprio(0);
+                    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+                    barrier(); // B(2kt+2)
+                }
+                barrier(); // pairs with the other group's last one
+            }
+            else
+            {
+                issue_loads(1);
+                barrier(); // B1
+                for(int kt = 0; kt < nk; ++kt)
+                {
+                    const uint8_t* sa = smem + (kt & 1) * STAGE;
+                    read_frags(sa, sa + A_TILE, 0, af0, bf0);
+                    read_frags(sa, sa + A_TILE, 1, af1, bf1);
+                    asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+                    barrier(); // B(2kt+2)
+                    issue_loads(kt + 2);
+                    __builtin_amdgcn_s_setprio(1);
+                    mfma_block(af0, bf0);
+                    mfma_block(af1, bf1);
+                    __builtin_amdgcn_s_setprio(0);
+                    barrier(); // B(2kt+3)
+                }
             }
         }
+        else
+        {
+            // Register double buffer over the two k-steps of a K tile. The barrier sits between
+            // them: by then every wave has pulled ALL of tile kt into registers, so the stage of
+            // tile kt can be refilled right away, and the first fragments of tile kt+1 are read
+            // while the second half of tile kt is still being multiplied.
+            issue_loads(0);
+            issue_loads(1);
+            asm volatile("s_waitcnt vmcnt(%0)" ::"n"(LPT) : "memory");
+            barrier();
+            read_frags(smem, smem + A_TILE, 0, af0, bf0);
+
+            for(int kt = 0; kt < nk; ++kt)
+            {
+                const uint8_t* sa  = smem + (kt & 1) * STAGE;
+                const uint8_t* sb  = sa + A_TILE;
+                const uint8_t* san = smem + ((kt + 1) & 1) * STAGE;
+                const uint8_t* sbn = san + A_TILE;
+
+                read_frags(sa, sb, 1, af1, bf1);
+                mfma_block(af0, bf0);
+                interleave();
+
+                // tile kt+1 has landed (its loads are the only ones in flight) and tile kt is
+                // entirely in registers
+                asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+                barrier();
+                issue_loads(kt + 2);
+
+                read_frags(san, sbn, 0, af0, bf0);
+                mfma_block(af1, bf1);
+                interleave();
+            }
+        }
+        // the trailing (all-zero) loads still target LDS: let them retire before the workgroup
+        // gives its LDS back
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 
         // ---- epilogue: registers -> global, 16 consecutive columns per lane -------------
         const bool vec_ok = ((reinterpret_cast<uintptr_t>(p.c) | ((uintptr_t)p.ldc * ES)) & 15u) == 0;
@@ -441,7 +575,7 @@ struct GemmTile
                 }
                 else
                 {
-                    _Float16* crow     = reinterpret_cast<_Float16*>(p.c) + (size_t)m * p.ldc;
+                    _Float16* crow   = reinterpret_cast<_Float16*>(p.c) + (size_t)m * p.ldc;
                     const f32x4 v[4] = {acc[i][g * 4], acc[i][g * 4 + 1], acc[i][g * 4 + 2], acc[i][g * 4 + 3]};
                     store_row16_f16(crow, n0, p.N, vec_ok, v);
                 }
@@ -450,11 +584,11 @@ struct GemmTile
     }
 };
 
-template <int DT, int BM, int BN, int WM, int WN, bool IM2COL>
+template <int DT, int BM, int BN, int WM, int WN, int BKB, int NST, bool IM2COL, bool PINGPONG>
 __global__ __launch_bounds__(WM* WN * 64) void gemm_tile_kernel(const GemmArgs p)
 {
     extern __shared__ __attribute__((aligned(1024))) uint8_t ckx_smem[];
-    GemmTile<DT, BM, BN, WM, WN, IM2COL>::run(p, ckx_smem);
+    GemmTile<DT, BM, BN, WM, WN, BKB, NST, IM2COL, PINGPONG>::run(p, ckx_smem);
 }
 
 } // namespace ckx

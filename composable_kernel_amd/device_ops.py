@@ -151,11 +151,11 @@ class DeviceGemmInt8(_DeviceGemm):
 
     def _supported(self, a):
         return capi.lib().ckx_gemm_i8_is_supported(a.M, a.N, a.K, a.StrideA, a.StrideB, a.StrideC,
-                                                   *a.layouts, a.c_op.epilogue, self.instance)
+                                                   *self.layouts, a.c_op.epilogue, self.instance)
 
     def _launch(self, a, stream):
         return capi.lib().ckx_gemm_i8(a.p_a, a.p_b, a.p_c, a.M, a.N, a.K, a.StrideA, a.StrideB, a.StrideC,
-                                      *a.layouts, a.c_op.epilogue, a.c_op.scale_gemm, a.c_op.scale_relu,
+                                      *self.layouts, a.c_op.epilogue, a.c_op.scale_gemm, a.c_op.scale_relu,
                                       self.instance, C.c_void_p(stream or 0))
 
 
@@ -168,11 +168,11 @@ class DeviceGemmF16(_DeviceGemm):
             capi.lib().ckx_gemm_f16_is_supported(-1, 0, 0, 0, 0, 0, 0, 0, 0, 0)  # sets an error string
             return capi.UNSUPPORTED
         return capi.lib().ckx_gemm_f16_is_supported(a.M, a.N, a.K, a.StrideA, a.StrideB, a.StrideC,
-                                                    *a.layouts, self.instance)
+                                                    *self.layouts, self.instance)
 
     def _launch(self, a, stream):
         return capi.lib().ckx_gemm_f16(a.p_a, a.p_b, a.p_c, a.M, a.N, a.K, a.StrideA, a.StrideB, a.StrideC,
-                                       *a.layouts, self.instance, C.c_void_p(stream or 0))
+                                       *self.layouts, self.instance, C.c_void_p(stream or 0))
 
 
 # -------------------------------------------------------------------- conv

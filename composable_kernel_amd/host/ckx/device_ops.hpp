@@ -1,0 +1,584 @@
+// Host-side operator surface over the C ABI (include/ckx.h), carrying Composable Kernel's
+// own names so that code written against the reference's device operators compiles against
+// this header instead:
+//
+//   ck::StreamConfig                                  include/ck/stream_config.hpp:9-13
+//   ck::tensor_operation::device::BaseArgument/BaseInvoker/BaseOperator
+//                                                     .../gpu/device/device_base.hpp:14-57
+//   ...::device::DeviceGemm<...>                      .../gpu/device/device_gemm.hpp:24-41
+//   ...::device::DeviceConvFwd<...>                   .../gpu/device/device_conv_fwd.hpp:18-39
+//   ...::device::DeviceBatchedGemmGemm<...>           upstream device_batched_gemm_gemm.hpp:15-56
+//   ...::device::instance::DeviceOperationInstanceFactory<DeviceOp>::GetInstances()
+//                                  library/.../tensor_operation_instance/gpu/gemm.hpp:233-379
+//   element_wise::PassThrough                         .../gpu/element/unary_element_wise_operation.hpp:13-25
+//
+// The kernels are precompiled in libckx.so; an element-wise functor is therefore not inlined
+// into a kernel but MAPPED to one of the library's fused epilogues through
+// ckx::EpilogueOf<Functor> (specialise it for your own functor type; a functor with public
+// members scaleGemm_ and scaleRelu_, like example 14's RequantReluRequant, is recognised
+// automatically). Unsupported problems make IsSupportedArgument() return false and Run()
+// throw std::runtime_error, as the reference does (device_gemm_xdl_cshuffle.hpp:475-481).
+#pragma once
+
+#include <hip/hip_runtime.h>
+
+#include <cstdint>
+#include <memory>
+#include <sstream>
+#include <stdexcept>
+#include <string>
+#include <type_traits>
+#include <vector>
+
+#include "ckx.h"
+
+namespace ck {
+
+using index_t      = int32_t;
+using long_index_t = int64_t;
+using half_t       = _Float16;
+
+struct StreamConfig
+{
+    hipStream_t stream_id_ = nullptr;
+    bool time_kernel_      = false;
+    int nrepeat_           = 10; // launch_and_time_kernel: 1 warm-up + 10 timed launches
+    int nwarmup_           = 1;
+};
+
+namespace tensor_layout {
+namespace gemm {
+struct RowMajor
+{
+    static constexpr int code = CKX_ROW_MAJOR;
+};
+struct ColumnMajor
+{
+    static constexpr int code = CKX_COL_MAJOR;
+};
+} // namespace gemm
+namespace convolution {
+struct NHWC
+{
+};
+struct KYXC
+{
+};
+struct NHWK
+{
+};
+} // namespace convolution
+} // namespace tensor_layout
+
+namespace tensor_operation {
+namespace element_wise {
+
+struct PassThrough
+{
+    template <typename Y, typename X>
+    void operator()(Y& y, const X& x) const
+    {
+        y = static_cast<Y>(x);
+    }
+};
+
+// y = clamp(scaleRelu * relu(scaleGemm * x), -128, 127); the int8 cast truncates
+// (example/14_gemm_xdl_requant_relu_requant/gemm_xdl_requant_relu_requant_int8.cpp:21-39)
+struct RequantReluRequant
+{
+    RequantReluRequant(float scaleGemm, float scaleRelu) : scaleGemm_(scaleGemm), scaleRelu_(scaleRelu) {}
+    void operator()(float& y, const float& x) const
+    {
+        float g = scaleGemm_ * x;
+        float r = g > 0 ? g : 0;
+        float q = scaleRelu_ * r;
+        y       = q > 127 ? 127 : q < -128 ? -128 : q;
+    }
+    float scaleGemm_, scaleRelu_;
+};
+
+// y = sat8(rint(scaleRelu * relu(sat8(rint(scaleGemm * x))))), rint = round-half-to-even
+struct RequantRoundReluRequantRound
+{
+    RequantRoundReluRequantRound(float scaleGemm, float scaleRelu) : scaleGemm_(scaleGemm), scaleRelu_(scaleRelu)
+    {
+    }
+    float scaleGemm_, scaleRelu_;
+};
+
+} // namespace element_wise
+} // namespace tensor_operation
+} // namespace ck
+
+namespace ckx {
+
+// Functor type -> fused epilogue of the library.
+template <typename Op, typename = void>
+struct EpilogueOf; // not defined: an unknown functor is a compile error, not a silent PassThrough
+
+template <>
+struct EpilogueOf<ck::tensor_operation::element_wise::PassThrough>
+{
+    static constexpr int kind = CKX_EPI_PASSTHROUGH;
+    static float scale_gemm(const ck::tensor_operation::element_wise::PassThrough&) { return 1.f; }
+    static float scale_relu(const ck::tensor_operation::element_wise::PassThrough&) { return 1.f; }
+};
+
+template <>
+struct EpilogueOf<ck::tensor_operation::element_wise::RequantRoundReluRequantRound>
+{
+    using Op                  = ck::tensor_operation::element_wise::RequantRoundReluRequantRound;
+    static constexpr int kind = CKX_EPI_REQUANT_RND;
+    static float scale_gemm(const Op& o) { return o.scaleGemm_; }
+    static float scale_relu(const Op& o) { return o.scaleRelu_; }
+};
+
+// any functor shaped like example 14's RequantReluRequant
+template <typename Op>
+struct EpilogueOf<Op,
+                  std::enable_if_t<!std::is_same_v<Op, ck::tensor_operation::element_wise::RequantRoundReluRequantRound> &&
+                                   std::is_same_v<decltype(std::declval<Op>().scaleGemm_), float> &&
+                                   std::is_same_v<decltype(std::declval<Op>().scaleRelu_), float>>>
+{
+    static constexpr int kind = CKX_EPI_REQUANT_CK;
+    static float scale_gemm(const Op& o) { return o.scaleGemm_; }
+    static float scale_relu(const Op& o) { return o.scaleRelu_; }
+};
+
+inline void throw_on(int status, const char* what)
+{
+    if(status != CKX_OK)
+        throw std::runtime_error(std::string(what) + ": " + ckx_last_error());
+}
+
+} // namespace ckx
+
+namespace ck {
+namespace tensor_operation {
+namespace device {
+
+struct BaseArgument
+{
+    virtual ~BaseArgument() {}
+    void* p_workspace_ = nullptr;
+};
+
+struct BaseInvoker
+{
+    virtual float Run(const BaseArgument*, const StreamConfig& = StreamConfig{}) { return 0.f; }
+    virtual ~BaseInvoker() {}
+};
+
+struct BaseOperator
+{
+    virtual bool IsSupportedArgument(const BaseArgument*) { return false; }
+    virtual std::string GetTypeString() const { return ""; }
+    virtual size_t GetWorkSpaceSize(const BaseArgument*) const { return 0; }
+    virtual void SetWorkSpacePointer(BaseArgument* p_arg, void* p_workspace) const
+    {
+        p_arg->p_workspace_ = p_workspace;
+    }
+    virtual ~BaseOperator() {}
+};
+
+// ------------------------------------------------------------------ interfaces
+template <typename ALayout, typename BLayout, typename CLayout, typename ADataType, typename BDataType,
+          typename CDataType, typename AElementwiseOperation, typename BElementwiseOperation,
+          typename CElementwiseOperation>
+struct DeviceGemm : public BaseOperator
+{
+    virtual std::unique_ptr<BaseArgument>
+    MakeArgumentPointer(const void* p_a, const void* p_b, void* p_c, index_t M, index_t N, index_t K,
+                        index_t StrideA, index_t StrideB, index_t StrideC, AElementwiseOperation a_element_op,
+                        BElementwiseOperation b_element_op, CElementwiseOperation c_element_op) = 0;
+    virtual std::unique_ptr<BaseInvoker> MakeInvokerPointer()                                   = 0;
+};
+
+template <typename InElementwiseOperation, typename WeiElementwiseOperation, typename OutElementwiseOperation>
+struct DeviceConvFwd : public BaseOperator
+{
+    virtual std::unique_ptr<BaseArgument>
+    MakeArgumentPointer(const void* p_in, const void* p_wei, void* p_out, index_t N, index_t K, index_t C,
+                        std::vector<index_t> input_spatial_lengths, std::vector<index_t> filter_spatial_lengths,
+                        std::vector<index_t> output_spatial_lengths, std::vector<index_t> conv_filter_strides,
+                        std::vector<index_t> conv_filter_dilations, std::vector<index_t> input_left_pads,
+                        std::vector<index_t> input_right_pads, InElementwiseOperation in_element_op,
+                        WeiElementwiseOperation wei_element_op, OutElementwiseOperation out_element_op) = 0;
+    virtual std::unique_ptr<BaseInvoker> MakeInvokerPointer()                                          = 0;
+};
+
+template <typename ALayout, typename B0Layout, typename B1Layout, typename CLayout, typename ADataType,
+          typename B0DataType, typename B1DataType, typename CDataType, typename AElementwiseOperation,
+          typename B0ElementwiseOperation, typename Acc0ElementwiseOperation, typename B1ElementwiseOperation,
+          typename CElementwiseOperation>
+struct DeviceBatchedGemmGemm : public BaseOperator
+{
+    virtual std::unique_ptr<BaseArgument>
+    MakeArgumentPointer(const void* p_a, const void* p_b0, const void* p_b1, void* p_c, index_t M, index_t N,
+                        index_t K, index_t O, index_t Batch, index_t StrideA, index_t StrideB0, index_t StrideB1,
+                        index_t StrideC, index_t BatchStrideA, index_t BatchStrideB0, index_t BatchStrideB1,
+                        index_t BatchStrideC, AElementwiseOperation a_element_op,
+                        B0ElementwiseOperation b0_element_op, Acc0ElementwiseOperation acc0_element_op,
+                        B1ElementwiseOperation b1_element_op, CElementwiseOperation c_element_op) = 0;
+    virtual std::unique_ptr<BaseInvoker> MakeInvokerPointer()                                     = 0;
+};
+
+// ------------------------------------------------------------------- common invoker
+namespace detail {
+
+// launch_and_time_kernel (include/ck/device_utility/kernel_launch.hpp:13-74): timed mode runs
+// the launch nwarmup_ + nrepeat_ times and returns the mean milliseconds; otherwise one
+// asynchronous launch and 0.
+template <typename Argument, int (*Supported)(const Argument&, int), int (*Launch)(const Argument&, int, void*)>
+struct InvokerT : public BaseInvoker
+{
+    explicit InvokerT(int instance) : instance_(instance) {}
+    float Run(const Argument& arg, const StreamConfig& sc = StreamConfig{})
+    {
+        if(Supported(arg, instance_) != CKX_OK)
+            throw std::runtime_error(std::string("wrong! the device operator has invalid setting: ") +
+                                     ckx_last_error());
+        if(!sc.time_kernel_)
+        {
+            ckx::throw_on(Launch(arg, instance_, sc.stream_id_), "HIP runtime error");
+            return 0.f;
+        }
+        struct Ctx
+        {
+            const Argument* a;
+            int inst;
+            void* s;
+        } ctx{&arg, instance_, sc.stream_id_};
+        float ms = 0.f;
+        ckx::throw_on(ckx_time_launches(
+                          [](void* u) {
+                              auto* c = static_cast<Ctx*>(u);
+                              return Launch(*c->a, c->inst, c->s);
+                          },
+                          &ctx, sc.nwarmup_, sc.nrepeat_, sc.stream_id_, &ms),
+                      "HIP runtime error");
+        return ms;
+    }
+    float Run(const BaseArgument* p_arg, const StreamConfig& sc = StreamConfig{}) override
+    {
+        const auto* a = dynamic_cast<const Argument*>(p_arg);
+        if(!a)
+            throw std::runtime_error("wrong! argument does not belong to this device operator");
+        return Run(*a, sc);
+    }
+    int instance_;
+};
+
+template <typename T>
+struct DTypeOf;
+template <>
+struct DTypeOf<int8_t>
+{
+    static constexpr bool is_i8 = true;
+};
+template <>
+struct DTypeOf<half_t>
+{
+    static constexpr bool is_i8 = false;
+};
+
+} // namespace detail
+
+// ------------------------------------------------------------------------ GEMM
+// One instance (tile configuration) of the MFMA GEMM. instance = CKX_INSTANCE_AUTO lets the
+// library choose by problem shape.
+template <typename ALayout, typename BLayout, typename CLayout, typename ADataType, typename BDataType,
+          typename CDataType, typename AElementwiseOperation, typename BElementwiseOperation,
+          typename CElementwiseOperation>
+struct DeviceGemmMfma : public DeviceGemm<ALayout, BLayout, CLayout, ADataType, BDataType, CDataType,
+                                          AElementwiseOperation, BElementwiseOperation, CElementwiseOperation>
+{
+    static_assert(std::is_same_v<ADataType, BDataType> && std::is_same_v<ADataType, CDataType>,
+                  "A, B and C share one data type (int8_t or half_t)");
+    static_assert(std::is_same_v<AElementwiseOperation, element_wise::PassThrough> &&
+                      std::is_same_v<BElementwiseOperation, element_wise::PassThrough>,
+                  "A/B element-wise operations other than PassThrough are not built");
+    static constexpr bool is_i8 = detail::DTypeOf<ADataType>::is_i8;
+    using Epi                   = ckx::EpilogueOf<CElementwiseOperation>;
+    static_assert(is_i8 || Epi::kind == CKX_EPI_PASSTHROUGH, "fp16 GEMM only has the PassThrough epilogue");
+
+    struct Argument : public BaseArgument
+    {
+        const void* p_a;
+        const void* p_b;
+        void* p_c;
+        index_t M, N, K, StrideA, StrideB, StrideC;
+        CElementwiseOperation c_element_op;
+        Argument(const void* a, const void* b, void* c, index_t m, index_t n, index_t k, index_t sa, index_t sb,
+                 index_t sc, CElementwiseOperation cop)
+            : p_a(a), p_b(b), p_c(c), M(m), N(n), K(k), StrideA(sa), StrideB(sb), StrideC(sc), c_element_op(cop)
+        {
+        }
+    };
+
+    static int Supported(const Argument& a, int inst)
+    {
+        if constexpr(is_i8)
+            return ckx_gemm_i8_is_supported(a.M, a.N, a.K, a.StrideA, a.StrideB, a.StrideC, ALayout::code,
+                                            BLayout::code, CLayout::code, Epi::kind, inst);
+        else
+            return ckx_gemm_f16_is_supported(a.M, a.N, a.K, a.StrideA, a.StrideB, a.StrideC, ALayout::code,
+                                             BLayout::code, CLayout::code, inst);
+    }
+    static int Launch(const Argument& a, int inst, void* stream)
+    {
+        if constexpr(is_i8)
+            return ckx_gemm_i8(a.p_a, a.p_b, a.p_c, a.M, a.N, a.K, a.StrideA, a.StrideB, a.StrideC, ALayout::code,
+                               BLayout::code, CLayout::code, Epi::kind, Epi::scale_gemm(a.c_element_op),
+                               Epi::scale_relu(a.c_element_op), inst, stream);
+        else
+            return ckx_gemm_f16(a.p_a, a.p_b, a.p_c, a.M, a.N, a.K, a.StrideA, a.StrideB, a.StrideC, ALayout::code,
+                                BLayout::code, CLayout::code, inst, stream);
+    }
+    using Invoker = detail::InvokerT<Argument, &Supported, &Launch>;
+
+    explicit DeviceGemmMfma(int instance = CKX_INSTANCE_AUTO) : instance_(instance) {}
+
+    static Argument MakeArgument(const ADataType* p_a, const BDataType* p_b, CDataType* p_c, index_t M, index_t N,
+                                 index_t K, index_t StrideA, index_t StrideB, index_t StrideC,
+                                 AElementwiseOperation, BElementwiseOperation, CElementwiseOperation c_element_op)
+    {
+        return Argument{p_a, p_b, p_c, M, N, K, StrideA, StrideB, StrideC, c_element_op};
+    }
+    Invoker MakeInvoker() const { return Invoker{instance_}; }
+    bool IsSupportedArgument(const Argument& a) const { return Supported(a, instance_) == CKX_OK; }
+
+    bool IsSupportedArgument(const BaseArgument* p) override
+    {
+        const auto* a = dynamic_cast<const Argument*>(p);
+        return a && IsSupportedArgument(*a);
+    }
+    std::unique_ptr<BaseArgument> MakeArgumentPointer(const void* p_a, const void* p_b, void* p_c, index_t M,
+                                                      index_t N, index_t K, index_t StrideA, index_t StrideB,
+                                                      index_t StrideC, AElementwiseOperation,
+                                                      BElementwiseOperation,
+                                                      CElementwiseOperation c_element_op) override
+    {
+        return std::make_unique<Argument>(p_a, p_b, p_c, M, N, K, StrideA, StrideB, StrideC, c_element_op);
+    }
+    std::unique_ptr<BaseInvoker> MakeInvokerPointer() override { return std::make_unique<Invoker>(instance_); }
+    std::string GetTypeString() const override
+    {
+        const int op = is_i8 ? CKX_OP_GEMM_I8 : CKX_OP_GEMM_F16;
+        if(instance_ == CKX_INSTANCE_AUTO)
+            return is_i8 ? "DeviceGemm_i8_i8_i8_mk_nk_mn<auto>" : "DeviceGemm_f16_f16_f16_mk_nk_mn<auto>";
+        return ckx_instance_name(op, instance_);
+    }
+    int instance_;
+};
+
+// ------------------------------------------------------------------------ conv2d fwd
+template <typename InDataType, typename WeiDataType, typename OutDataType, typename InElementwiseOperation,
+          typename WeiElementwiseOperation, typename OutElementwiseOperation>
+struct DeviceConv2dFwdMfma_Input_N_Hi_Wi_C_Weight_K_Y_X_C_Output_N_Ho_Wo_K
+    : public DeviceConvFwd<InElementwiseOperation, WeiElementwiseOperation, OutElementwiseOperation>
+{
+    static_assert(std::is_same_v<InDataType, WeiDataType> && std::is_same_v<InDataType, OutDataType>,
+                  "input, weight and output share one data type (int8_t or half_t)");
+    static constexpr bool is_i8 = detail::DTypeOf<InDataType>::is_i8;
+    using Epi                   = ckx::EpilogueOf<OutElementwiseOperation>;
+    static constexpr int op_code = is_i8 ? CKX_OP_CONV2D_FWD_I8 : CKX_OP_CONV2D_FWD_F16;
+
+    struct Argument : public BaseArgument
+    {
+        const void* p_in;
+        const void* p_wei;
+        void* p_out;
+        ckx_conv2d_desc desc;
+        bool two_d;
+        OutElementwiseOperation out_element_op;
+        Argument(const void* in, const void* wei, void* out, index_t N, index_t K, index_t C,
+                 const std::vector<index_t>& isp, const std::vector<index_t>& fsp, const std::vector<index_t>& osp,
+                 const std::vector<index_t>& st, const std::vector<index_t>& dl, const std::vector<index_t>& lp,
+                 const std::vector<index_t>& rp, OutElementwiseOperation oop)
+            : p_in(in), p_wei(wei), p_out(out), desc{}, out_element_op(oop)
+        {
+            two_d = isp.size() == 2 && fsp.size() == 2 && osp.size() == 2 && st.size() == 2 && dl.size() == 2 &&
+                    lp.size() == 2 && rp.size() == 2;
+            if(two_d)
+                desc = ckx_conv2d_desc{N,     K,     C,     isp[0], isp[1], fsp[0], fsp[1], osp[0], osp[1],
+                                       st[0], st[1], dl[0], dl[1],  lp[0],  lp[1],  rp[0],  rp[1]};
+        }
+    };
+    static int Supported(const Argument& a, int inst)
+    {
+        if(!a.two_d)
+            return CKX_UNSUPPORTED;
+        return ckx_conv2d_fwd_is_supported(op_code, &a.desc, Epi::kind, inst);
+    }
+    static int Launch(const Argument& a, int inst, void* stream)
+    {
+        if constexpr(is_i8)
+            return ckx_conv2d_fwd_i8(a.p_in, a.p_wei, a.p_out, &a.desc, Epi::kind,
+                                     Epi::scale_gemm(a.out_element_op), Epi::scale_relu(a.out_element_op), inst,
+                                     stream);
+        else
+            return ckx_conv2d_fwd_f16(a.p_in, a.p_wei, a.p_out, &a.desc, inst, stream);
+    }
+    using Invoker = detail::InvokerT<Argument, &Supported, &Launch>;
+
+    explicit DeviceConv2dFwdMfma_Input_N_Hi_Wi_C_Weight_K_Y_X_C_Output_N_Ho_Wo_K(int instance = CKX_INSTANCE_AUTO)
+        : instance_(instance)
+    {
+    }
+    static Argument MakeArgument(const InDataType* p_in, const WeiDataType* p_wei, OutDataType* p_out, index_t N,
+                                 index_t K, index_t C, std::vector<index_t> isp, std::vector<index_t> fsp,
+                                 std::vector<index_t> osp, std::vector<index_t> st, std::vector<index_t> dl,
+                                 std::vector<index_t> lp, std::vector<index_t> rp, InElementwiseOperation,
+                                 WeiElementwiseOperation, OutElementwiseOperation oop)
+    {
+        return Argument{p_in, p_wei, p_out, N, K, C, isp, fsp, osp, st, dl, lp, rp, oop};
+    }
+    Invoker MakeInvoker() const { return Invoker{instance_}; }
+    bool IsSupportedArgument(const Argument& a) const { return Supported(a, instance_) == CKX_OK; }
+    bool IsSupportedArgument(const BaseArgument* p) override
+    {
+        const auto* a = dynamic_cast<const Argument*>(p);
+        return a && IsSupportedArgument(*a);
+    }
+    std::unique_ptr<BaseArgument>
+    MakeArgumentPointer(const void* p_in, const void* p_wei, void* p_out, index_t N, index_t K, index_t C,
+                        std::vector<index_t> isp, std::vector<index_t> fsp, std::vector<index_t> osp,
+                        std::vector<index_t> st, std::vector<index_t> dl, std::vector<index_t> lp,
+                        std::vector<index_t> rp, InElementwiseOperation, WeiElementwiseOperation,
+                        OutElementwiseOperation oop) override
+    {
+        return std::make_unique<Argument>(p_in, p_wei, p_out, N, K, C, isp, fsp, osp, st, dl, lp, rp, oop);
+    }
+    std::unique_ptr<BaseInvoker> MakeInvokerPointer() override { return std::make_unique<Invoker>(instance_); }
+    std::string GetTypeString() const override
+    {
+        if(instance_ == CKX_INSTANCE_AUTO)
+            return is_i8 ? "DeviceConv2dFwd_i8_nhwc_kyxc_nhwk<auto>" : "DeviceConv2dFwd_f16_nhwc_kyxc_nhwk<auto>";
+        return ckx_instance_name(op_code, instance_);
+    }
+    int instance_;
+};
+
+// -------------------------------------------------------------------- GEMM-GEMM
+template <typename AElementwiseOperation = element_wise::PassThrough,
+          typename B0ElementwiseOperation = element_wise::PassThrough,
+          typename Acc0ElementwiseOperation = element_wise::PassThrough,
+          typename B1ElementwiseOperation = element_wise::PassThrough,
+          typename CElementwiseOperation = element_wise::PassThrough>
+struct DeviceBatchedGemmGemmMfma
+    : public DeviceBatchedGemmGemm<tensor_layout::gemm::RowMajor, tensor_layout::gemm::ColumnMajor,
+                                   tensor_layout::gemm::RowMajor, tensor_layout::gemm::RowMajor, half_t, half_t,
+                                   half_t, half_t, AElementwiseOperation, B0ElementwiseOperation,
+                                   Acc0ElementwiseOperation, B1ElementwiseOperation, CElementwiseOperation>
+{
+    static_assert(std::is_same_v<AElementwiseOperation, element_wise::PassThrough> &&
+                      std::is_same_v<B0ElementwiseOperation, element_wise::PassThrough> &&
+                      std::is_same_v<Acc0ElementwiseOperation, element_wise::PassThrough> &&
+                      std::is_same_v<B1ElementwiseOperation, element_wise::PassThrough> &&
+                      std::is_same_v<CElementwiseOperation, element_wise::PassThrough>,
+                  "only PassThrough element-wise operations are built");
+    struct Argument : public BaseArgument
+    {
+        const void *p_a, *p_b0, *p_b1;
+        void* p_c;
+        index_t M, N, K, O, Batch, StrideA, StrideB0, StrideB1, StrideC;
+        int64_t BatchStrideA, BatchStrideB0, BatchStrideB1, BatchStrideC;
+    };
+    static int Supported(const Argument& a, int inst)
+    {
+        return ckx_batched_gemm_gemm_f16_is_supported(a.M, a.N, a.K, a.O, a.Batch, a.StrideA, a.StrideB0, a.StrideB1,
+                                                      a.StrideC, a.BatchStrideA, a.BatchStrideB0, a.BatchStrideB1,
+                                                      a.BatchStrideC, inst);
+    }
+    static int Launch(const Argument& a, int inst, void* stream)
+    {
+        return ckx_batched_gemm_gemm_f16(a.p_a, a.p_b0, a.p_b1, a.p_c, a.M, a.N, a.K, a.O, a.Batch, a.StrideA,
+                                         a.StrideB0, a.StrideB1, a.StrideC, a.BatchStrideA, a.BatchStrideB0,
+                                         a.BatchStrideB1, a.BatchStrideC, inst, stream);
+    }
+    using Invoker = detail::InvokerT<Argument, &Supported, &Launch>;
+
+    explicit DeviceBatchedGemmGemmMfma(int instance = CKX_INSTANCE_AUTO) : instance_(instance) {}
+    static Argument MakeArgument(const half_t* p_a, const half_t* p_b0, const half_t* p_b1, half_t* p_c, index_t M,
+                                 index_t N, index_t K, index_t O, index_t Batch, index_t StrideA, index_t StrideB0,
+                                 index_t StrideB1, index_t StrideC, index_t BatchStrideA, index_t BatchStrideB0,
+                                 index_t BatchStrideB1, index_t BatchStrideC, AElementwiseOperation = {},
+                                 B0ElementwiseOperation = {}, Acc0ElementwiseOperation = {},
+                                 B1ElementwiseOperation = {}, CElementwiseOperation = {})
+    {
+        Argument a;
+        a.p_a = p_a, a.p_b0 = p_b0, a.p_b1 = p_b1, a.p_c = p_c;
+        a.M = M, a.N = N, a.K = K, a.O = O, a.Batch = Batch;
+        a.StrideA = StrideA, a.StrideB0 = StrideB0, a.StrideB1 = StrideB1, a.StrideC = StrideC;
+        a.BatchStrideA = BatchStrideA, a.BatchStrideB0 = BatchStrideB0, a.BatchStrideB1 = BatchStrideB1,
+        a.BatchStrideC = BatchStrideC;
+        return a;
+    }
+    Invoker MakeInvoker() const { return Invoker{instance_}; }
+    bool IsSupportedArgument(const Argument& a) const { return Supported(a, instance_) == CKX_OK; }
+    bool IsSupportedArgument(const BaseArgument* p) override
+    {
+        const auto* a = dynamic_cast<const Argument*>(p);
+        return a && IsSupportedArgument(*a);
+    }
+    std::unique_ptr<BaseArgument>
+    MakeArgumentPointer(const void* p_a, const void* p_b0, const void* p_b1, void* p_c, index_t M, index_t N,
+                        index_t K, index_t O, index_t Batch, index_t StrideA, index_t StrideB0, index_t StrideB1,
+                        index_t StrideC, index_t BatchStrideA, index_t BatchStrideB0, index_t BatchStrideB1,
+                        index_t BatchStrideC, AElementwiseOperation, B0ElementwiseOperation,
+                        Acc0ElementwiseOperation, B1ElementwiseOperation, CElementwiseOperation) override
+    {
+        return std::make_unique<Argument>(MakeArgument(
+            static_cast<const half_t*>(p_a), static_cast<const half_t*>(p_b0), static_cast<const half_t*>(p_b1),
+            static_cast<half_t*>(p_c), M, N, K, O, Batch, StrideA, StrideB0, StrideB1, StrideC, BatchStrideA,
+            BatchStrideB0, BatchStrideB1, BatchStrideC));
+    }
+    std::unique_ptr<BaseInvoker> MakeInvokerPointer() override { return std::make_unique<Invoker>(instance_); }
+    std::string GetTypeString() const override
+    {
+        if(instance_ == CKX_INSTANCE_AUTO)
+            return "DeviceBatchedGemmGemm_f16_gmk_gnk_gno_gmo<auto>";
+        return ckx_instance_name(CKX_OP_BATCHED_GEMM_GEMM, instance_);
+    }
+    int instance_;
+};
+
+// ------------------------------------------------------------------ instance factory
+namespace instance {
+
+template <typename DeviceOp>
+struct DeviceOperationInstanceFactory;
+
+template <typename AL, typename BL, typename CL, typename T, typename AOp, typename BOp, typename COp>
+struct DeviceOperationInstanceFactory<DeviceGemm<AL, BL, CL, T, T, T, AOp, BOp, COp>>
+{
+    using DeviceOp = DeviceGemm<AL, BL, CL, T, T, T, AOp, BOp, COp>;
+    static std::vector<std::unique_ptr<DeviceOp>> GetInstances()
+    {
+        std::vector<std::unique_ptr<DeviceOp>> v;
+        const int n = ckx_num_instances(detail::DTypeOf<T>::is_i8 ? CKX_OP_GEMM_I8 : CKX_OP_GEMM_F16);
+        for(int i = 0; i < n; ++i)
+            v.push_back(std::make_unique<DeviceGemmMfma<AL, BL, CL, T, T, T, AOp, BOp, COp>>(i));
+        return v;
+    }
+};
+
+// conv: the interface type carries no data type, so the caller names it
+// (ConvolutionFwdInstances<T,T,T>::Get<2>(), library/include/ck/library/utility/conv_util.hpp:288-397)
+template <typename T, typename InOp, typename WeiOp, typename OutOp>
+std::vector<std::unique_ptr<DeviceConvFwd<InOp, WeiOp, OutOp>>> GetConv2dFwdInstances()
+{
+    std::vector<std::unique_ptr<DeviceConvFwd<InOp, WeiOp, OutOp>>> v;
+    const int n = ckx_num_instances(detail::DTypeOf<T>::is_i8 ? CKX_OP_CONV2D_FWD_I8 : CKX_OP_CONV2D_FWD_F16);
+    for(int i = 0; i < n; ++i)
+        v.push_back(std::make_unique<
+                    DeviceConv2dFwdMfma_Input_N_Hi_Wi_C_Weight_K_Y_X_C_Output_N_Ho_Wo_K<T, T, T, InOp, WeiOp, OutOp>>(
+            i));
+    return v;
+}
+
+} // namespace instance
+} // namespace device
+} // namespace tensor_operation
+} // namespace ck

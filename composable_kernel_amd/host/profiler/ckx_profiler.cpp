@@ -1,0 +1,345 @@
+// ckx_profiler: ckProfiler-style driver (profiler/src/profiler.cpp:48-148) for the operators of
+// this library. Positional arguments follow the reference's conventions
+// (profiler/src/profile_gemm.cpp:27-75, profile_convnd_fwd.cpp:81-115):
+//
+//   ckx_profiler gemm <dtype 1:fp16 3:int8> <layout 1: A[m,k]*B[n,k]> <verify> <init> <log> <time>
+//                     M N K StrideA StrideB StrideC [epilogue 0|1|2] [scale_gemm] [scale_relu] [nrepeat]
+//   ckx_profiler conv2d_fwd <dtype 1|3> <verify> <init> <log> <time>
+//                     N K C Y X Hi Wi Sy Sx Dy Dx LeftPy LeftPx RightPy RightPx [epilogue sg sr] [nrepeat]
+//   ckx_profiler batched_gemm_gemm <verify> <init> <log> <time> M N K O Batch [nrepeat]
+//
+// Every instance of the family is run (DeviceOperationInstanceFactory), one "Perf:" line each
+// and a final "Best Perf:" line, in the reference's format (profile_gemm_impl.hpp:176-177,
+// 246-249), extended with the fraction of the MI355X roofline that binds the problem.
+// verify = 1 checks that all instances agree with the first supported one (bit-exact for
+// int8, rtol = atol = 1e-2 for fp16); comparison against the CPU reference is the job of the
+// test-suite, which regenerates these inputs from the same seeds. If the environment variable
+// CKX_PROFILER_DUMP names a file, the best instance's output tensor is written there.
+#include <cstdlib>
+#include <cstring>
+#include <iomanip>
+#include <iostream>
+
+#include "ckx/device_ops.hpp"
+#include "ckx/host_tensor.hpp"
+
+using namespace ck;
+using namespace ck::tensor_operation;
+using Row  = tensor_layout::gemm::RowMajor;
+using Col  = tensor_layout::gemm::ColumnMajor;
+using Pass = element_wise::PassThrough;
+
+namespace {
+
+constexpr double kPeakF16 = 2516.6, kPeakI8 = 5033.2, kPeakHbmGBs = 8000.0;
+
+struct Best
+{
+    float ms = 0, tflops = 0, gbs = 0;
+    std::string name;
+    int id = -1;
+};
+
+void report(const char* tag, float ms, double flop, double bytes, const std::string& name, bool i8)
+{
+    const double tflops = flop / 1e9 / ms, gbs = bytes / 1e6 / ms;
+    const double fm = tflops / (i8 ? kPeakI8 : kPeakF16), fh = gbs / kPeakHbmGBs;
+    std::cout << tag << std::setw(10) << ms << " ms, " << tflops << " TFlops, " << gbs << " GB/s, " << name << "  ["
+              << std::fixed << std::setprecision(1) << (fm >= fh ? fm : fh) * 100 << "% of "
+              << (fm >= fh ? "MFMA" : "HBM") << " roofline]" << std::defaultfloat << std::setprecision(6)
+              << std::endl;
+}
+
+template <typename T>
+void fill(std::vector<T>& v, int init, uint64_t seed, bool conv)
+{
+    if constexpr(std::is_same_v<T, int8_t>)
+    {
+        if(init == 0)
+            return;
+        ckx::fill_uniform_int8(v, -5, 5, seed);
+    }
+    else
+    {
+        if(init == 0)
+            return;
+        if(init == 1)
+        { // integer values, as the reference's init_method 1
+            std::vector<int8_t> t(v.size());
+            ckx::fill_uniform_int8(t, -5, 5, seed);
+            for(std::size_t i = 0; i < v.size(); ++i)
+                v[i] = (T)(float)t[i];
+        }
+        else
+            ckx::fill_uniform_f16(v, conv ? -1.f : -1.f, 1.f, seed);
+    }
+}
+
+template <typename T, typename Op, typename MakeArg>
+int run_family(std::vector<std::unique_ptr<Op>>& ops, MakeArg make_arg, ckx::DeviceMem& out_dev, std::size_t out_elems,
+               double flop, double bytes, bool verify, bool time_kernel, int nrepeat)
+{
+    constexpr bool i8 = std::is_same_v<T, int8_t>;
+    std::cout << "found " << ops.size() << " instances" << std::endl;
+    Best best;
+    std::vector<T> ref, out(out_elems);
+    bool pass = true;
+    for(std::size_t i = 0; i < ops.size(); ++i)
+    {
+        auto arg = make_arg(*ops[i]);
+        auto inv = ops[i]->MakeInvokerPointer();
+        const std::string name = ops[i]->GetTypeString();
+        if(!ops[i]->IsSupportedArgument(arg.get()))
+        {
+            std::cout << name << " does not support this problem" << std::endl;
+            continue;
+        }
+        out_dev.SetZero();
+        StreamConfig sc{nullptr, time_kernel, nrepeat, nrepeat >= 100 ? nrepeat / 4 : 1};
+        const float ms = inv->Run(arg.get(), sc);
+        ckx::hip_check(hipDeviceSynchronize());
+        if(time_kernel)
+        {
+            report("Perf: ", ms, flop, bytes, name, i8);
+            if(best.id < 0 || ms < best.ms)
+                best = Best{ms, (float)(flop / 1e9 / ms), (float)(bytes / 1e6 / ms), name, (int)i};
+        }
+        else if(best.id < 0)
+            best.id = (int)i, best.name = name;
+        if(verify)
+        {
+            out_dev.FromDevice(out.data());
+            if(ref.empty())
+                ref = out;
+            else
+            {
+                const std::size_t bad = ckx::count_errors(out, ref, 1e-2, 1e-2);
+                if(bad)
+                {
+                    std::cout << "Error: " << name << " disagrees with the first instance on " << bad << " elements"
+                              << std::endl;
+                    pass = false;
+                }
+            }
+        }
+    }
+    if(best.id < 0)
+    {
+        std::cout << "no instance supports this problem" << std::endl;
+        return 1;
+    }
+    if(time_kernel)
+        report("Best Perf: ", best.ms, flop, bytes, best.name, i8);
+    if(const char* path = std::getenv("CKX_PROFILER_DUMP"))
+    {
+        auto arg = make_arg(*ops[best.id]);
+        out_dev.SetZero();
+        ops[best.id]->MakeInvokerPointer()->Run(arg.get(), StreamConfig{});
+        ckx::hip_check(hipDeviceSynchronize());
+        out_dev.FromDevice(out.data());
+        ckx::dump_to_file(path, out);
+    }
+    return pass ? 0 : 1;
+}
+
+template <typename T, typename COp>
+int profile_gemm_t(bool verify, int init, bool time_kernel, int M, int N, int K, int sa, int sb, int sc, COp cop,
+                   int nrepeat)
+{
+    using DeviceOp = device::DeviceGemm<Row, Col, Row, T, T, T, Pass, Pass, COp>;
+    auto ops       = device::instance::DeviceOperationInstanceFactory<DeviceOp>::GetInstances();
+    std::vector<T> a((std::size_t)M * sa), b((std::size_t)N * sb);
+    fill(a, init, 0xC0FFEE, false);
+    fill(b, init, 0xC0FFEE + 1, false);
+    ckx::DeviceMem da(a.size() * sizeof(T)), db(b.size() * sizeof(T)), dc((std::size_t)M * sc * sizeof(T));
+    da.ToDevice(a.data());
+    db.ToDevice(b.data());
+    std::cout << "a_m_k: dim 2, lengths {" << M << ", " << K << "}, strides {" << sa << ", 1}\n"
+              << "b_k_n: dim 2, lengths {" << K << ", " << N << "}, strides {1, " << sb << "}\n"
+              << "c_m_n: dim 2, lengths {" << M << ", " << N << "}, strides {" << sc << ", 1}" << std::endl;
+    const double flop = 2.0 * M * N * K, bytes = sizeof(T) * ((double)M * K + (double)K * N + (double)M * N);
+    return run_family<T>(
+        ops,
+        [&](DeviceOp& op) {
+            return op.MakeArgumentPointer(da.GetDeviceBuffer(), db.GetDeviceBuffer(), dc.GetDeviceBuffer(), M, N, K,
+                                          sa, sb, sc, Pass{}, Pass{}, cop);
+        },
+        dc, (std::size_t)M * sc, flop, bytes, verify, time_kernel, nrepeat);
+}
+
+int profile_gemm(int argc, char* argv[])
+{
+    if(argc < 14)
+    {
+        std::printf("arg1: tensor operation (gemm)\narg2: data type (1: fp16; 3: int8)\n"
+                    "arg3: matrix layout (1: A[m, k] * B[n, k] = C[m, n])\narg4: verification (0: no; 1: yes)\n"
+                    "arg5: initialization (0: no init; 1: integer value; 2: decimal value)\n"
+                    "arg6: print tensor value (0: no; 1: yes)\narg7: time kernel (0=no, 1=yes)\n"
+                    "arg8 to 13: M, N, K, StrideA, StrideB, StrideC\n"
+                    "arg14-16 (int8): epilogue (0 PassThrough, 1 RequantReluRequant, 2 rounded), scale_gemm, scale_relu\n"
+                    "last: nrepeat\n");
+        return 1;
+    }
+    const int dtype = std::atoi(argv[2]), layout = std::atoi(argv[3]);
+    const bool verify = std::atoi(argv[4]), time_kernel = std::atoi(argv[7]);
+    const int init = std::atoi(argv[5]);
+    const int M = std::atoi(argv[8]), N = std::atoi(argv[9]), K = std::atoi(argv[10]);
+    int sa = std::atoi(argv[11]), sb = std::atoi(argv[12]), sc = std::atoi(argv[13]);
+    sa = sa < 0 ? K : sa, sb = sb < 0 ? K : sb, sc = sc < 0 ? N : sc;
+    if(layout != 1)
+    {
+        std::cout << "this data_type & layout is not implemented" << std::endl;
+        return 1;
+    }
+    if(dtype == 1)
+        return profile_gemm_t<half_t>(verify, init, time_kernel, M, N, K, sa, sb, sc, Pass{},
+                                      argc > 14 ? std::atoi(argv[14]) : 10);
+    if(dtype == 3)
+    {
+        const int epi  = argc > 14 ? std::atoi(argv[14]) : 0;
+        const float sg = argc > 15 ? (float)std::atof(argv[15]) : 0.03f;
+        const float sr = argc > 16 ? (float)std::atof(argv[16]) : 1.0f;
+        const int nrep = argc > 17 ? std::atoi(argv[17]) : 10;
+        if(epi == 0)
+            return profile_gemm_t<int8_t>(verify, init, time_kernel, M, N, K, sa, sb, sc, Pass{}, nrep);
+        if(epi == 1)
+            return profile_gemm_t<int8_t>(verify, init, time_kernel, M, N, K, sa, sb, sc,
+                                          element_wise::RequantReluRequant{sg, sr}, nrep);
+        return profile_gemm_t<int8_t>(verify, init, time_kernel, M, N, K, sa, sb, sc,
+                                      element_wise::RequantRoundReluRequantRound{sg, sr}, nrep);
+    }
+    std::cout << "this data_type & layout is not implemented" << std::endl;
+    return 1;
+}
+
+template <typename T, typename OutOp>
+int profile_conv_t(bool verify, int init, bool time_kernel, const int* p, OutOp oop, int nrepeat)
+{
+    const int N = p[0], K = p[1], C = p[2], Y = p[3], X = p[4], Hi = p[5], Wi = p[6], Sy = p[7], Sx = p[8],
+              Dy = p[9], Dx = p[10], LPy = p[11], LPx = p[12], RPy = p[13], RPx = p[14];
+    // conv_util.cpp:103-114
+    const int Ho = (Hi + LPy + RPy - ((Y - 1) * Dy + 1)) / Sy + 1, Wo = (Wi + LPx + RPx - ((X - 1) * Dx + 1)) / Sx + 1;
+    auto ops     = device::instance::GetConv2dFwdInstances<T, Pass, Pass, OutOp>();
+    using Op     = device::DeviceConvFwd<Pass, Pass, OutOp>;
+    std::vector<T> in((std::size_t)N * Hi * Wi * C), wei((std::size_t)K * Y * X * C);
+    fill(in, init, 0xC0FFEE + 2, true);
+    fill(wei, init, 0xC0FFEE + 3, true);
+    const std::size_t out_elems = (std::size_t)N * Ho * Wo * K;
+    ckx::DeviceMem di(in.size() * sizeof(T)), dw(wei.size() * sizeof(T)), dout(out_elems * sizeof(T));
+    di.ToDevice(in.data());
+    dw.ToDevice(wei.data());
+    std::cout << "input: N " << N << " Hi " << Hi << " Wi " << Wi << " C " << C << "; weight: K " << K << " Y " << Y
+              << " X " << X << "; output: Ho " << Ho << " Wo " << Wo << std::endl;
+    // conv_util.cpp:22-39 (flops) and conv_util.hpp:108-136 (bytes: whole input counted)
+    const double flop  = 2.0 * N * K * Ho * Wo * C * Y * X;
+    const double bytes = sizeof(T) * ((double)in.size() + (double)wei.size() + (double)out_elems);
+    return run_family<T>(
+        ops,
+        [&](Op& op) {
+            return op.MakeArgumentPointer(di.GetDeviceBuffer(), dw.GetDeviceBuffer(), dout.GetDeviceBuffer(), N, K, C,
+                                          {Hi, Wi}, {Y, X}, {Ho, Wo}, {Sy, Sx}, {Dy, Dx}, {LPy, LPx}, {RPy, RPx},
+                                          Pass{}, Pass{}, oop);
+        },
+        dout, out_elems, flop, bytes, verify, time_kernel, nrepeat);
+}
+
+int profile_conv(int argc, char* argv[])
+{
+    if(argc < 22)
+    {
+        std::printf("arg1: tensor operation (conv2d_fwd)\narg2: data type (1: fp16; 3: int8)\n"
+                    "arg3: verification\narg4: initialization\narg5: print tensor value\narg6: time kernel\n"
+                    "arg7 to 21: N, K, C, Y, X, Hi, Wi, Sy, Sx, Dy, Dx, LeftPy, LeftPx, RightPy, RightPx\n"
+                    "arg22-24 (int8): epilogue, scale_gemm, scale_relu; last: nrepeat\n");
+        return 1;
+    }
+    const int dtype = std::atoi(argv[2]);
+    const bool verify = std::atoi(argv[3]), time_kernel = std::atoi(argv[6]);
+    const int init = std::atoi(argv[4]);
+    int p[15];
+    for(int i = 0; i < 15; ++i)
+        p[i] = std::atoi(argv[7 + i]);
+    if(dtype == 1)
+        return profile_conv_t<half_t>(verify, init, time_kernel, p, Pass{}, argc > 22 ? std::atoi(argv[22]) : 10);
+    if(dtype == 3)
+    {
+        const int epi  = argc > 22 ? std::atoi(argv[22]) : 0;
+        const float sg = argc > 23 ? (float)std::atof(argv[23]) : 0.03f;
+        const float sr = argc > 24 ? (float)std::atof(argv[24]) : 1.0f;
+        const int nrep = argc > 25 ? std::atoi(argv[25]) : 10;
+        if(epi == 0)
+            return profile_conv_t<int8_t>(verify, init, time_kernel, p, Pass{}, nrep);
+        if(epi == 1)
+            return profile_conv_t<int8_t>(verify, init, time_kernel, p, element_wise::RequantReluRequant{sg, sr}, nrep);
+        return profile_conv_t<int8_t>(verify, init, time_kernel, p, element_wise::RequantRoundReluRequantRound{sg, sr},
+                                      nrep);
+    }
+    std::cout << "this data_type is not implemented" << std::endl;
+    return 1;
+}
+
+int profile_gemm_gemm(int argc, char* argv[])
+{
+    if(argc < 11)
+    {
+        std::printf("arg1: tensor operation (batched_gemm_gemm)\narg2: verification\narg3: initialization\n"
+                    "arg4: print tensor value\narg5: time kernel\narg6 to 10: M, N, K, O, Batch\nlast: nrepeat\n");
+        return 1;
+    }
+    const bool verify = std::atoi(argv[2]), time_kernel = std::atoi(argv[5]);
+    const int init = std::atoi(argv[3]);
+    const int M = std::atoi(argv[6]), N = std::atoi(argv[7]), K = std::atoi(argv[8]), O = std::atoi(argv[9]),
+              G = std::atoi(argv[10]);
+    const int nrepeat = argc > 11 ? std::atoi(argv[11]) : 10;
+    using Op = device::DeviceBatchedGemmGemm<Row, Col, Row, Row, half_t, half_t, half_t, half_t, Pass, Pass, Pass,
+                                             Pass, Pass>;
+    std::vector<std::unique_ptr<Op>> ops;
+    for(int i = 0; i < ckx_num_instances(CKX_OP_BATCHED_GEMM_GEMM); ++i)
+        ops.push_back(std::make_unique<device::DeviceBatchedGemmGemmMfma<>>(i));
+    std::vector<half_t> a((std::size_t)G * M * K), b0((std::size_t)G * N * K), b1((std::size_t)G * N * O);
+    if(init)
+    {
+        ckx::fill_uniform_f16(a, -0.5f, 0.5f, 0xC0FFEE + 4);
+        ckx::fill_uniform_f16(b0, -0.5f, 0.5f, 0xC0FFEE + 5);
+        ckx::fill_uniform_f16(b1, -0.5f, 0.5f, 0xC0FFEE + 6);
+    }
+    const std::size_t out_elems = (std::size_t)G * M * O;
+    ckx::DeviceMem da(a.size() * 2), db0(b0.size() * 2), db1(b1.size() * 2), dc(out_elems * 2);
+    da.ToDevice(a.data());
+    db0.ToDevice(b0.data());
+    db1.ToDevice(b1.data());
+    const double flop  = 2.0 * G * ((double)M * N * K + (double)M * N * O);
+    const double bytes = 2.0 * ((double)a.size() + b0.size() + b1.size() + out_elems);
+    return run_family<half_t>(
+        ops,
+        [&](Op& op) {
+            return op.MakeArgumentPointer(da.GetDeviceBuffer(), db0.GetDeviceBuffer(), db1.GetDeviceBuffer(),
+                                          dc.GetDeviceBuffer(), M, N, K, O, G, K, K, O, O, M * K, N * K, N * O, M * O,
+                                          Pass{}, Pass{}, Pass{}, Pass{}, Pass{});
+        },
+        dc, out_elems, flop, bytes, verify, time_kernel, nrepeat);
+}
+
+} // namespace
+
+int main(int argc, char* argv[])
+{
+    try
+    {
+        if(argc >= 2 && std::strcmp(argv[1], "gemm") == 0)
+            return profile_gemm(argc, argv);
+        if(argc >= 2 && (std::strcmp(argv[1], "conv2d_fwd") == 0 || std::strcmp(argv[1], "conv_fwd") == 0))
+            return profile_conv(argc, argv);
+        if(argc >= 2 && std::strcmp(argv[1], "batched_gemm_gemm") == 0)
+            return profile_gemm_gemm(argc, argv);
+        std::printf("arg1: tensor operation (gemm: GEMM\n"
+                    "                        conv2d_fwd: NHWC/KYXC/NHWK forward convolution\n"
+                    "                        batched_gemm_gemm: batched fused GEMM+GEMM)\n");
+        return 1;
+    }
+    catch(const std::exception& e)
+    {
+        std::cerr << e.what() << std::endl;
+        return 2;
+    }
+}

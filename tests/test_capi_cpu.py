@@ -1,0 +1,102 @@
+"""CPU-only checks of the drop-in boundary: the C-ABI library loads, exports every symbol
+include/ckx.h declares, and its pure-host argument validation behaves like the reference's
+IsSupportedArgument (no kernel is launched here)."""
+import ctypes as C
+import os
+import re
+
+import numpy as np
+import pytest
+
+import composable_kernel_amd as ck
+from composable_kernel_amd import capi
+from composable_kernel_amd.host_tensor import splitmix64, uniform_f16, uniform_int8
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def test_library_exports_every_declared_symbol():
+    hdr = open(os.path.join(ROOT, "include", "ckx.h")).read()
+    hdr = re.sub(r"/\*.*?\*/", "", hdr, flags=re.S)
+    declared = set(re.findall(r"\b(ckx_[a-z0-9_]+)\s*\(", hdr)) - {"ckx_launch_fn"}
+    assert declared == set(capi.SYMBOLS)
+    L = capi.lib()
+    for name in sorted(declared):
+        assert getattr(L, name) is not None
+    assert b"gfx950" in L.ckx_version()
+
+
+def test_instance_factory_lists_named_instances():
+    L = capi.lib()
+    for op in range(5):
+        n = L.ckx_num_instances(op)
+        assert n >= 1
+        names = [L.ckx_instance_name(op, i).decode() for i in range(n)]
+        assert len(set(names)) == n
+        assert L.ckx_instance_name(op, n) is None
+    assert L.ckx_num_instances(99) == 0
+    assert len(ck.DeviceGemmInt8.GetInstances()) == L.ckx_num_instances(capi.OP_GEMM_I8)
+
+
+def test_gemm_argument_validation_is_pure_host_logic():
+    op = ck.DeviceGemmInt8()
+    ok = op.MakeArgumentPointer(0, 0, 0, 1024, 1024, 1024, 1024, 1024, 1024, None, None,
+                                ck.RequantReluRequant(0.5, 0.03, rounded=True))
+    assert op.IsSupportedArgument(ok)
+    # K not a multiple of 16 bytes; stride below K; column-major C; >= 2 GiB operand
+    for bad in [
+        op.MakeArgumentPointer(0, 0, 0, 64, 64, 100, 100, 100, 64),
+        op.MakeArgumentPointer(0, 0, 0, 64, 64, 128, 64, 128, 64),
+        op.MakeArgumentPointer(0, 0, 0, 1 << 16, 64, 1 << 15, 1 << 15, 1 << 15, 64),
+    ]:
+        assert not op.IsSupportedArgument(bad)
+        assert capi.last_error()
+    assert not ck.DeviceGemmInt8(CLayout=ck.ColumnMajor).IsSupportedArgument(ok)
+    assert not ck.DeviceGemmInt8(instance=999).IsSupportedArgument(ok)
+    f16 = ck.DeviceGemmF16()
+    assert f16.IsSupportedArgument(f16.MakeArgumentPointer(0, 0, 0, 4096, 4096, 4096, 4096, 4096, 4096))
+    assert not f16.IsSupportedArgument(f16.MakeArgumentPointer(0, 0, 0, 64, 64, 60, 60, 60, 64))
+    # a functor the fp16 operator does not fuse
+    assert not f16.IsSupportedArgument(
+        f16.MakeArgumentPointer(0, 0, 0, 64, 64, 64, 64, 64, 64, None, None, ck.RequantReluRequant(1, 1)))
+    with pytest.raises(RuntimeError):
+        op.MakeInvokerPointer().Run(op.MakeArgumentPointer(0, 0, 0, 64, 64, 100, 100, 100, 64))
+
+
+def test_conv_argument_validation():
+    op = ck.DeviceConv2dFwdF16()
+    mk = lambda C_, osp: op.MakeArgumentPointer(0, 0, 0, 256, 64, C_, [56, 56], [3, 3], osp, [1, 1], [1, 1],
+                                                [1, 1], [1, 1])
+    assert op.IsSupportedArgument(mk(64, [56, 56]))
+    assert not op.IsSupportedArgument(mk(3, [56, 56]))      # C*2 bytes not a multiple of 16
+    assert not op.IsSupportedArgument(mk(64, [55, 56]))     # output size does not follow from the geometry
+    with pytest.raises(ValueError):
+        op.MakeArgumentPointer(0, 0, 0, 1, 1, 8, [8], [3], [6], [1], [1], [0], [0])   # only 2-D is built
+
+
+def test_gemm_gemm_argument_validation():
+    op = ck.DeviceBatchedGemmGemmF16()
+    mk = lambda K, O: op.MakeArgumentPointer(0, 0, 0, 0, 512, 512, K, O, 64, K, K, O, O, 512 * K, 512 * K,
+                                             512 * O, 512 * O)
+    assert op.IsSupportedArgument(mk(64, 64))
+    assert op.IsSupportedArgument(mk(128, 128))
+    assert not op.IsSupportedArgument(mk(256, 64))
+    assert not op.IsSupportedArgument(mk(60, 64))
+
+
+def test_generators_are_counter_based_and_in_range():
+    # first two outputs of the published splitmix64 generator for seed 1234567
+    z = splitmix64(1234567, 2)
+    assert [int(v) for v in z] == [6457827717110365317, 3203168211198807973]
+    a = uniform_int8((1000,), -5, 5, 7)
+    assert a.min() == -5 and a.max() == 5
+    np.testing.assert_array_equal(uniform_int8((1000,), -5, 5, 7)[:100], uniform_int8((100,), -5, 5, 7))
+    h = uniform_f16((4096,), -1, 1, 9)
+    assert h.dtype == np.float16 and -1 <= h.min() and h.max() <= 1 and abs(float(h.astype(np.float32).mean())) < 0.05
+
+
+def test_missing_library_fails_loudly(tmp_path, monkeypatch):
+    monkeypatch.setattr(capi, "_lib", None)
+    monkeypatch.setattr(capi, "LIB_PATH", str(tmp_path / "libckx.so"))
+    with pytest.raises(FileNotFoundError):
+        capi.lib()

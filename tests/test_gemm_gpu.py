@@ -16,7 +16,7 @@ from oracle import fast, lit
 
 pytestmark = pytest.mark.gpu
 
-N_TILE_INSTANCES = 8
+N_TILE_INSTANCES = 9
 RTOL = ATOL = 1e-2
 
 EPILOGUES = {

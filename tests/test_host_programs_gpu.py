@@ -1,0 +1,98 @@
+"""GPU tests of the C++ host layer: the ckProfiler-style driver and the example that mirrors the
+reference's example 14 run as child processes; the tensors they write are checked against the
+CPU oracle on inputs regenerated here from the same seeds (the generators are counter based)."""
+import os
+import subprocess
+
+import numpy as np
+import pytest
+
+from composable_kernel_amd.host_tensor import uniform_f16, uniform_int8
+from oracle import fast, lit
+
+pytestmark = pytest.mark.gpu
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+BIN = os.path.join(ROOT, "composable_kernel_amd", "bin")
+SEED = 0xC0FFEE
+
+
+def _run(exe, args, dump_var, tmp_path):
+    path = os.path.join(BIN, exe)
+    if not os.path.exists(path):
+        pytest.fail(f"{path} is not built (python -m composable_kernel_amd.build)")
+    dump = str(tmp_path / "out.bin")
+    env = dict(os.environ, **{dump_var: dump})
+    r = subprocess.run([path] + [str(a) for a in args], env=env, stdout=subprocess.PIPE, stderr=subprocess.STDOUT,
+                       text=True, timeout=300)
+    assert r.returncode == 0, r.stdout
+    return r.stdout, dump
+
+
+def test_profiler_int8_requant_gemm_all_instances_agree_and_match_oracle(tmp_path):
+    M, N, K = 1024, 1024, 1024
+    out, dump = _run("ckx_profiler", ["gemm", 3, 1, 1, 1, 0, 1, M, N, K, -1, -1, -1, 2, 0.5, 0.03], "CKX_PROFILER_DUMP",
+                     tmp_path)
+    assert "Best Perf:" in out and "Error" not in out
+    assert out.count("Perf:") >= 8
+    c = np.fromfile(dump, np.int8).reshape(M, N)
+    a = uniform_int8((M, K), -5, 5, SEED)
+    b_nk = uniform_int8((N, K), -5, 5, SEED + 1)
+    np.testing.assert_array_equal(c, lit.gemm_i8(a, b_nk.T, lit.EPI_REQUANT_RND, 0.5, 0.03))
+
+
+def test_profiler_fp16_gemm(tmp_path):
+    M, N, K = 512, 768, 1024
+    out, dump = _run("ckx_profiler", ["gemm", 1, 1, 1, 2, 0, 1, M, N, K, -1, -1, -1], "CKX_PROFILER_DUMP", tmp_path)
+    assert "Best Perf:" in out and "Error" not in out
+    c = np.fromfile(dump, np.float16).reshape(M, N)
+    a = uniform_f16((M, K), -1, 1, SEED)
+    b_nk = uniform_f16((N, K), -1, 1, SEED + 1)
+    bad, max_err = lit.check_err_f16(c, lit.gemm_f16(a, b_nk.T), 1e-2, 1e-2)
+    assert bad == 0, max_err
+
+
+def test_profiler_conv2d_fwd_int8(tmp_path):
+    # N K C Y X Hi Wi Sy Sx Dy Dx LPy LPx RPy RPx (the reference's argument order)
+    geo = [4, 64, 32, 3, 3, 14, 14, 2, 2, 1, 1, 1, 1, 1, 1]
+    out, dump = _run("ckx_profiler", ["conv2d_fwd", 3, 1, 1, 0, 1] + geo, "CKX_PROFILER_DUMP", tmp_path)
+    assert "Best Perf:" in out and "Error" not in out
+    N, K, C, Y, X, Hi, Wi = geo[:7]
+    inp = uniform_int8((N, Hi, Wi, C), -5, 5, SEED + 2)
+    wei = uniform_int8((K, Y, X, C), -5, 5, SEED + 3)
+    want = lit.conv2d_fwd(inp, wei, (2, 2), (1, 1), (1, 1))
+    c = np.fromfile(dump, np.int8).reshape(want.shape)
+    np.testing.assert_array_equal(c, want)
+
+
+def test_profiler_batched_gemm_gemm(tmp_path):
+    M, N, K, O, G = 256, 384, 64, 64, 3
+    out, dump = _run("ckx_profiler", ["batched_gemm_gemm", 1, 1, 0, 1, M, N, K, O, G], "CKX_PROFILER_DUMP", tmp_path)
+    assert "Best Perf:" in out
+    a = uniform_f16((G, M, K), -0.5, 0.5, SEED + 4)
+    b0 = uniform_f16((G, N, K), -0.5, 0.5, SEED + 5)
+    b1 = uniform_f16((G, N, O), -0.5, 0.5, SEED + 6)
+    c = np.fromfile(dump, np.float16).reshape(G, M, O)
+    bad, max_err = lit.check_err_f16(c, lit.batched_gemm_gemm_f16(a, b0.transpose(0, 2, 1), b1), 1e-2, 1e-2)
+    assert bad == 0, max_err
+
+
+def test_profiler_reports_unsupported_problems():
+    path = os.path.join(BIN, "ckx_profiler")
+    r = subprocess.run([path, "gemm", "3", "1", "0", "1", "0", "0", "64", "64", "100", "-1", "-1", "-1"],
+                       stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=120)
+    assert r.returncode == 1
+    assert "does not support this problem" in r.stdout
+
+
+def test_example_gemm_requant_relu_requant_int8(tmp_path):
+    """Same call sequence and defaults as the reference's example 14 (scales 0.03 / 1, literal
+    functor), on a smaller problem."""
+    M, N, K = 768, 512, 1024
+    out, dump = _run("example_gemm_requant_relu_requant_int8", [1, 1, 1, M, N, K, K, K, N], "CKX_EXAMPLE_DUMP", tmp_path)
+    assert "Perf:" in out
+    c = np.fromfile(dump, np.int8).reshape(M, N)
+    a = uniform_int8((M, K), -5, 5, SEED)
+    b_nk = uniform_int8((N, K), -5, 5, SEED + 1)
+    want = lit.gemm_i8(a, b_nk.T, lit.EPI_REQUANT_CK, 0.03, 1.0)
+    np.testing.assert_array_equal(c, want)
+    assert f"sum(C) = {int(want.astype(np.int64).sum())}" in out
