@@ -51,6 +51,12 @@ def lib():
         raise FileNotFoundError(
             f"{LIB_PATH} is missing: build it with `python -m composable_kernel_amd.build` "
             "(there is no CPU fallback)")
+    # In a process that also uses torch (tests, bench), torch's bundled HIP runtime must be the
+    # one that gets loaded: it shares its SONAME with the system copy libckx.so names.
+    try:
+        import torch  # noqa: F401
+    except ImportError:
+        pass
     L = C.CDLL(LIB_PATH)
     i32, f32, vp, i64 = C.c_int32, C.c_float, C.c_void_p, C.c_int64
     L.ckx_version.restype = C.c_char_p
