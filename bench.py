@@ -9,9 +9,13 @@ metric (TFLOP/s and fraction of the dense fp16 MFMA peak) is quoted; the int8 ha
 (4096^3 requant GEMM, TOP/s) and every other config are measured too and attached under "also".
 Prints ONE JSON line on stdout.
 
-Timing: W untimed launches, then K launches between two events recorded on the launch stream
-(torch's current stream, whose handle is what the C ABI receives), bracketed by device
-synchronisation; wall-clock over the same region gives ms_per_step.
+Timing: W untimed launches, then exactly K launches between two events recorded on the launch
+stream (torch's current stream, whose handle is what the C ABI receives), bracketed by device
+synchronisation; wall-clock over the same region gives ms_per_step. The K launches are replayed
+from a HIP graph captured from the same C-ABI calls, so that the GPU runs them back to back
+even for kernels shorter than a Python call (--no-graph launches eagerly). The defaults
+(K = 1000, W = 300) are long enough for the part to reach its operating clocks: the first few
+milliseconds after idle run several hundred MHz lower.
 """
 import argparse
 import json
@@ -66,7 +70,6 @@ def make_launcher(w, instance=-1):
     from composable_kernel_amd import capi
     from composable_kernel_amd.host_tensor import uniform_f16, uniform_int8
 
-    stream = torch.cuda.current_stream().cuda_stream
     keep = []
 
     def dev(a):
@@ -113,7 +116,7 @@ def make_launcher(w, instance=-1):
         raise RuntimeError(f"{w['name']}: not supported: {capi.last_error()}")
 
     def launch():
-        st_ = op._launch(arg, stream)
+        st_ = op._launch(arg, torch.cuda.current_stream().cuda_stream)
         if st_ != 0:
             raise RuntimeError(capi.last_error())
 
@@ -121,17 +124,33 @@ def make_launcher(w, instance=-1):
     return launch
 
 
-def time_workload(w, steps, warmup, instance=-1):
+def time_workload(w, steps, warmup, instance=-1, use_graph=True):
+    """W untimed launches, then exactly K timed ones. The K launches are replayed from a HIP
+    graph (captured once from the same C-ABI calls) so that kernels run back to back on the GPU
+    even when one kernel is shorter than a Python call; use_graph=False launches eagerly."""
     import torch
     launch = make_launcher(w, instance)
     for _ in range(warmup):
         launch()
+    torch.cuda.synchronize()
+    per_graph = max(d for d in range(1, min(steps, 50) + 1) if steps % d == 0)
+    graph = None
+    if use_graph:
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            for _ in range(per_graph):
+                launch()
+        graph.replay()   # one untimed replay
     e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     torch.cuda.synchronize()
     t0 = time.perf_counter()
     e0.record()
-    for _ in range(steps):
-        launch()
+    if graph is not None:
+        for _ in range(steps // per_graph):
+            graph.replay()
+    else:
+        for _ in range(steps):
+            launch()
     e1.record()
     torch.cuda.synchronize()
     wall_ms = (time.perf_counter() - t0) * 1e3 / steps
@@ -178,12 +197,16 @@ def cpu_baseline(w, target_seconds=12.0):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=50)
-    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--steps", type=int, default=1000)
+    ap.add_argument("--warmup", type=int, default=300)
     ap.add_argument("--workload", default="fp16_gemm_4096")
     ap.add_argument("--instance", type=int, default=-1)
     ap.add_argument("--all", action="store_true", help="also time every other config (reported under 'also')")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-graph", action="store_true", help="launch eagerly instead of replaying a HIP graph")
+    ap.add_argument("--copy-probe", action="store_true",
+                    help="also run one 256 MiB device-to-device copy (a kernel of known traffic, used to "
+                         "scale the FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this hot path is a single-GPU kernel library; run with --gpus 1 "
@@ -197,14 +220,19 @@ def main():
     from composable_kernel_amd import capi
     capi.lib()   # fail loudly if the HIP library is missing
 
+    if args.copy_probe:
+        src = torch.empty(256 << 20, dtype=torch.uint8, device="cuda").random_()
+        dst = torch.empty_like(src)
+        dst.copy_(src)
+        torch.cuda.synchronize()
     w = WORKLOADS[args.workload]
-    r = time_workload(w, args.steps, args.warmup, args.instance)
+    r = time_workload(w, args.steps, args.warmup, args.instance, not args.no_graph)
     also = []
     extra = ["int8_requant_gemm_4096"] if args.workload == "fp16_gemm_4096" else []
     if args.all:
         extra = [n for n in WORKLOADS if n != args.workload]
     for n in extra:
-        x = time_workload(WORKLOADS[n], max(10, args.steps // 2), max(3, args.warmup // 2))
+        x = time_workload(WORKLOADS[n], max(10, args.steps // 2), max(3, args.warmup // 2), -1, not args.no_graph)
         also.append({"workload": n, "dtype": x["dtype"], "ms": round(x["ms"], 5),
                      "value": round(x["tput"], 2), "unit": "TOP/s" if x["dtype"] == "i8" else "TFLOP/s",
                      "GB/s": round(x["gbs"], 1), "bound": x["bound"],

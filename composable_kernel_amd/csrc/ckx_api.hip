@@ -11,6 +11,7 @@
 #include "ckx.h"
 #include "gemm_tile.hpp"
 #include "gemm_gemm.hpp"
+#include "gemm_skinny.hpp"
 
 namespace {
 
@@ -64,52 +65,89 @@ hipError_t launch_tile(const ckx::GemmArgs& a, int grid, hipStream_t s)
 struct TileInstance
 {
     const char* name;
-    int bm, bn, threads;
+    int bm, bn, threads, lds;
+    float eff; // measured MFMA throughput of this tile shape relative to the 256x256 one
     tile_launch_fn dense_i8, dense_f16, conv_i8, conv_f16;
 };
 
-#define CKX_TILE(BM, BN, WM, WN, BKB, NST, PP)                                                          \
+#define CKX_TILE(BM, BN, WM, WN, BKB, NST, PP, EFF)                                                     \
     {                                                                                                   \
         "MI355X_Mfma16_Tile<" #BM ", " #BN ", " #BKB "B x" #NST ", waves " #WM "x" #WN ", pp" #PP ">", BM, BN,     \
-            WM* WN * 64, &launch_tile<ckx::DT_I8, BM, BN, WM, WN, BKB, NST, false, PP>,                       \
+            WM* WN * 64, NST*(BM + BN) * BKB, EFF,                                                      \
+            &launch_tile<ckx::DT_I8, BM, BN, WM, WN, BKB, NST, false, PP>,                                   \
             &launch_tile<ckx::DT_F16, BM, BN, WM, WN, BKB, NST, false, PP>,                                 \
             &launch_tile<ckx::DT_I8, BM, BN, WM, WN, BKB, NST, true, PP>,                                   \
             &launch_tile<ckx::DT_F16, BM, BN, WM, WN, BKB, NST, true, PP>                                   \
     }
 
 const TileInstance kTiles[] = {
-    CKX_TILE(256, 256, 2, 4, 128, 2, 0),
-    CKX_TILE(256, 128, 4, 2, 128, 2, 0),
-    CKX_TILE(128, 128, 2, 2, 128, 2, 0),
-    CKX_TILE(128, 64, 4, 1, 128, 2, 0),
-    CKX_TILE(64, 64, 4, 1, 128, 2, 0),
-    CKX_TILE(32, 64, 2, 1, 128, 2, 0),
-    CKX_TILE(16, 64, 1, 1, 128, 2, 0),
-    CKX_TILE(256, 256, 2, 4, 128, 2, 1),
-    CKX_TILE(256, 128, 4, 2, 128, 2, 1),
+    CKX_TILE(256, 256, 2, 4, 128, 2, 0, 1.00f),
+    CKX_TILE(256, 128, 4, 2, 128, 2, 0, 0.84f),
+    CKX_TILE(128, 128, 2, 2, 128, 2, 0, 0.78f),
+    CKX_TILE(128, 64, 4, 1, 128, 2, 0, 0.68f),
+    CKX_TILE(64, 64, 4, 1, 128, 2, 0, 0.55f),
+    CKX_TILE(32, 64, 2, 1, 128, 2, 0, 0.42f),
+    CKX_TILE(16, 64, 1, 1, 128, 2, 0, 0.27f),
+    CKX_TILE(256, 256, 2, 4, 128, 2, 1, 0.97f),
+    CKX_TILE(256, 128, 4, 2, 128, 2, 1, 0.83f),
+    CKX_TILE(256, 64, 8, 1, 128, 2, 0, 0.70f),
 };
 constexpr int kNumTiles = sizeof(kTiles) / sizeof(kTiles[0]);
 
-// Pick the largest tile that still yields enough workgroups to occupy 256 CUs.
-int pick_tile(int M, int N)
+// Instance choice by a small cost model (microseconds on a 256-CU part): workgroups run in
+// rounds of 256 * (workgroups that fit a CU's 160 KB LDS and 2048 threads); a round costs the
+// tile's share of MFMA time, scaled by how well that tile shape feeds the MFMA pipe, plus a
+// fixed prologue/epilogue term that co-resident workgroups overlap.
+int pick_tile(int M, int N, int kbytes)
 {
-    auto tiles = [&](int i) {
-        return (long)((M + kTiles[i].bm - 1) / kTiles[i].bm) * ((N + kTiles[i].bn - 1) / kTiles[i].bn);
-    };
-    const int order[] = {0, 1, 2, 3, 4, 5, 6};
-    for(int i : order)
+    int best       = 0;
+    double best_us = 1e30;
+    const double ktiles = (kbytes + 127) / 128;
+    for(int i = 0; i < kNumTiles; ++i)
     {
-        if(kTiles[i].bm > 16 && M <= kTiles[i].bm / 2)
-            continue; // more than half of the tile rows would be padding
-        if(tiles(i) >= 224)
-            return i;
+        const TileInstance& t = kTiles[i];
+        const long tiles      = (long)((M + t.bm - 1) / t.bm) * ((N + t.bn - 1) / t.bn);
+        int per_cu            = 160 * 1024 / t.lds;
+        per_cu                = per_cu > 2048 / t.threads ? 2048 / t.threads : per_cu;
+        per_cu                = per_cu > 4 ? 4 : per_cu;
+        per_cu                = (long)per_cu * 256 > tiles ? (int)((tiles + 255) / 256) : per_cu;
+        const long rounds     = (tiles + 256l * per_cu - 1) / (256l * per_cu);
+        const double us = rounds * (per_cu * (t.bm * t.bn / 65536.0) / t.eff * ktiles * 1.1 + 6.0 / per_cu + 2.0);
+        if(us < best_us)
+            best_us = us, best = i;
     }
-    // nothing fills the machine: smallest tile that is not mostly padding
-    for(int i = 6; i >= 0; --i)
-        if(M >= kTiles[i].bm || i == 6)
-            return i;
-    return 6;
+    return best;
 }
+
+// ---------------------------------------------------------- skinny instances
+struct SkinnyInstance
+{
+    const char* name;
+    int max_m;
+    tile_launch_fn i8, f16;
+};
+
+template <int DT, int MT, int NW, int KU>
+hipError_t launch_skinny(const ckx::GemmArgs& a, int grid, hipStream_t s)
+{
+    hipLaunchKernelGGL((ckx::gemm_skinny_kernel<DT, MT, NW, KU>), dim3(grid), dim3(NW * 64), 0, s, a);
+    return hipGetLastError();
+}
+
+#define CKX_SKINNY(MT, NW, KU)                                                                 \
+    {                                                                                          \
+        "MI355X_Mfma16_Skinny<rows " #MT "x16, 16 cols, waves " #NW ", unroll " #KU ">", MT * 16, \
+            &launch_skinny<ckx::DT_I8, MT, NW, KU>, &launch_skinny<ckx::DT_F16, MT, NW, KU>       \
+    }
+
+const SkinnyInstance kSkinny[] = {
+    CKX_SKINNY(1, 8, 4),
+    CKX_SKINNY(2, 8, 4),
+    CKX_SKINNY(4, 8, 2),
+    CKX_SKINNY(1, 16, 2),
+};
+constexpr int kNumSkinny    = sizeof(kSkinny) / sizeof(kSkinny[0]);
+constexpr int kNumGemmInsts = kNumTiles + kNumSkinny;
 
 const char* family_prefix(int op)
 {
@@ -130,8 +168,10 @@ int check_gemm_shape(int dt, int M, int N, int K, int sa, int sb, int sc, int al
     const int es = dt == ckx::DT_I8 ? 1 : 2;
     if(M < 0 || N < 0 || K < 0)
         return fail(CKX_INVALID_VALUE, "negative GEMM dimension");
-    if(instance != CKX_INSTANCE_AUTO && (instance < 0 || instance >= kNumTiles))
+    if(instance != CKX_INSTANCE_AUTO && (instance < 0 || instance >= kNumGemmInsts))
         return fail(CKX_INVALID_VALUE, "no such instance");
+    if(instance >= kNumTiles && M > kSkinny[instance - kNumTiles].max_m)
+        return fail(CKX_UNSUPPORTED, "this skinny instance covers fewer rows than M");
     if(epi < CKX_EPI_PASSTHROUGH || epi > CKX_EPI_REQUANT_RND)
         return fail(CKX_INVALID_VALUE, "unknown epilogue");
     if(dt == ckx::DT_F16 && epi != CKX_EPI_PASSTHROUGH)
@@ -160,8 +200,12 @@ int run_gemm(int dt, const void* a, const void* b, void* c, int M, int N, int K,
     if((reinterpret_cast<uintptr_t>(a) | reinterpret_cast<uintptr_t>(b)) & 15)
         return fail(CKX_UNSUPPORTED, "A and B must be 16-byte aligned");
     const int es = dt == ckx::DT_I8 ? 1 : 2;
-    const int ti = instance == CKX_INSTANCE_AUTO ? pick_tile(M, N) : instance;
-    const TileInstance& t = kTiles[ti];
+    int ti = instance;
+    if(instance == CKX_INSTANCE_AUTO)
+    {
+        // a handful of rows against a big weight matrix is an HBM-streaming problem
+        ti = M <= 16 ? kNumTiles + 0 : M <= 32 ? kNumTiles + 1 : M <= 64 ? kNumTiles + 2 : pick_tile(M, N, K * es);
+    }
     ckx::GemmArgs g;
     std::memset(&g, 0, sizeof(g));
     g.a = a, g.b = b, g.c = c;
@@ -169,11 +213,18 @@ int run_gemm(int dt, const void* a, const void* b, void* c, int M, int N, int K,
     g.lda = sa, g.ldb = sb, g.ldc = sc;
     g.a_bytes    = (uint32_t)(((long)(M - 1) * sa + K) * es);
     g.b_bytes    = (uint32_t)(((long)(N - 1) * sb + K) * es);
-    g.tiles_m    = (M + t.bm - 1) / t.bm;
-    g.tiles_n    = (N + t.bn - 1) / t.bn;
     g.epi        = epi;
     g.scale_gemm = sg;
     g.scale_relu = sr;
+    if(ti >= kNumTiles)
+    {
+        const SkinnyInstance& k = kSkinny[ti - kNumTiles];
+        hipError_t e = (dt == ckx::DT_I8 ? k.i8 : k.f16)(g, (N + 15) / 16, (hipStream_t)stream);
+        return e == hipSuccess ? CKX_OK : hip_fail(e, k.name);
+    }
+    const TileInstance& t = kTiles[ti];
+    g.tiles_m    = (M + t.bm - 1) / t.bm;
+    g.tiles_n    = (N + t.bn - 1) / t.bn;
     hipError_t e = (dt == ckx::DT_I8 ? t.dense_i8 : t.dense_f16)(g, g.tiles_m * g.tiles_n, (hipStream_t)stream);
     if(e != hipSuccess)
         return hip_fail(e, t.name);
@@ -227,7 +278,7 @@ int run_conv(int op, const void* in, const void* wei, void* out, const ckx_conv2
         return fail(CKX_INVALID_VALUE, "null operand pointer");
     if((reinterpret_cast<uintptr_t>(in) | reinterpret_cast<uintptr_t>(wei)) & 15)
         return fail(CKX_UNSUPPORTED, "input and weight must be 16-byte aligned");
-    const int ti = instance == CKX_INSTANCE_AUTO ? pick_tile(M, N) : instance;
+    const int ti = instance == CKX_INSTANCE_AUTO ? pick_tile(M, N, K * es) : instance;
     const TileInstance& t = kTiles[ti];
     ckx::GemmArgs g;
     std::memset(&g, 0, sizeof(g));
@@ -263,7 +314,9 @@ const char* ckx_last_error(void) { return g_last_error.c_str(); }
 
 int ckx_num_instances(int op)
 {
-    if(op >= CKX_OP_GEMM_I8 && op <= CKX_OP_CONV2D_FWD_F16)
+    if(op == CKX_OP_GEMM_I8 || op == CKX_OP_GEMM_F16)
+        return kNumGemmInsts;
+    if(op == CKX_OP_CONV2D_FWD_I8 || op == CKX_OP_CONV2D_FWD_F16)
         return kNumTiles;
     if(op == CKX_OP_BATCHED_GEMM_GEMM)
         return ckx::kNumGemmGemmInstances;
@@ -277,7 +330,10 @@ const char* ckx_instance_name(int op, int instance)
     if(!fam || instance < 0 || instance >= ckx_num_instances(op))
         return nullptr;
     s = std::string(fam) + "<" +
-        (op == CKX_OP_BATCHED_GEMM_GEMM ? ckx::gemm_gemm_instance_name(instance) : kTiles[instance].name) + ">";
+        (op == CKX_OP_BATCHED_GEMM_GEMM ? ckx::gemm_gemm_instance_name(instance)
+         : instance >= kNumTiles        ? kSkinny[instance - kNumTiles].name
+                                        : kTiles[instance].name) +
+        ">";
     return s.c_str();
 }
 

@@ -1,0 +1,142 @@
+// Skinny GEMM for gfx950: C[M,N] = epilogue(A[M,K] * B[N,K]^T) with M <= 16*MT (a few token
+// rows against a large weight matrix), int8 or fp16, same layouts as the tile kernel.
+//
+// Such problems are bound by streaming B out of HBM exactly once. Each workgroup owns 16
+// output columns and the WHOLE K extent, split over its waves: a wave loads its K slice of
+// the 16 B rows straight from global memory into registers in the MFMA operand layout (lane
+// l: row l%16, 16 bytes at k-step offset 16*(l/16)) -- there is no reuse across waves, so
+// there is no LDS staging -- multiplies it with the matching A fragments (read through L2),
+// and the per-wave partial tiles are summed through LDS at the end. No split-K workspace, no
+// atomics, and thousands of independent 1 KB loads in flight per CU.
+#pragma once
+
+#include "gemm_tile.hpp"
+
+namespace ckx {
+
+template <int DT, int MT, int NW, int KU>
+__global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(const GemmArgs p)
+{
+    using acc_t = typename std::conditional<DT == DT_I8, i32x4, f32x4>::type;
+    constexpr int ES = DT == DT_I8 ? 1 : 2;
+    __shared__ acc_t red[NW][MT][64];
+
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const uint32_t r = lane & 15, q = lane >> 4;
+    const int n0 = blockIdx.x * 16;
+
+    const uint32_t kbytes = (uint32_t)p.K * ES;
+    const int ksteps      = (int)((kbytes + 63u) >> 6);
+    const int per_wave    = (ksteps + NW - 1) / NW;
+    const int ks_begin    = wave * per_wave;
+    const int ks_end      = ks_begin + per_wave < ksteps ? ks_begin + per_wave : ksteps;
+
+    const __amdgpu_buffer_rsrc_t rsrc_a = make_rsrc(p.a, p.a_bytes);
+    const __amdgpu_buffer_rsrc_t rsrc_b = make_rsrc(p.b, p.b_bytes);
+
+    const uint32_t b_off = (uint32_t)n0 + r < (uint32_t)p.N ? ((uint32_t)n0 + r) * (uint32_t)p.ldb * ES + q * 16 : kOutOfRange;
+    uint32_t a_off[MT];
+#pragma unroll
+    for(int mt = 0; mt < MT; ++mt)
+        a_off[mt] = 16u * mt + r < (uint32_t)p.M ? (16u * mt + r) * (uint32_t)p.lda * ES + q * 16 : kOutOfRange;
+
+    acc_t acc[MT];
+#pragma unroll
+    for(int mt = 0; mt < MT; ++mt)
+        acc[mt] = acc_t{0, 0, 0, 0};
+
+    // one chunk = KU consecutive k-steps (64 bytes of K each); k-steps at or past ks_end and the
+    // K tail read as zeros through an out-of-range buffer offset
+    auto load_chunk = [&](int ks0, i32x4(&bq)[KU], i32x4(&aq)[MT][KU]) {
+#pragma unroll
+        for(int u = 0; u < KU; ++u)
+        {
+            const int ks        = ks0 + u;
+            const uint32_t kb   = (uint32_t)ks * 64u;
+            const bool ok       = ks < ks_end && kb + q * 16 < kbytes;
+            bq[u] = __builtin_bit_cast(i32x4, __builtin_amdgcn_raw_buffer_load_b128(rsrc_b, ok ? b_off + kb : kOutOfRange, 0, 0));
+#pragma unroll
+            for(int mt = 0; mt < MT; ++mt)
+                aq[mt][u] = __builtin_bit_cast(
+                    i32x4, __builtin_amdgcn_raw_buffer_load_b128(rsrc_a, ok ? a_off[mt] + kb : kOutOfRange, 0, 0));
+        }
+    };
+    auto mfma_chunk = [&](const i32x4(&bq)[KU], const i32x4(&aq)[MT][KU]) {
+#pragma unroll
+        for(int u = 0; u < KU; ++u)
+#pragma unroll
+            for(int mt = 0; mt < MT; ++mt)
+            {
+                if constexpr(DT == DT_I8)
+                    acc[mt] = __builtin_amdgcn_mfma_i32_16x16x64_i8(bq[u], aq[mt][u], acc[mt], 0, 0, 0);
+                else
+                    acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, bq[u]),
+                                                                    __builtin_bit_cast(f16x8, aq[mt][u]), acc[mt], 0,
+                                                                    0, 0);
+            }
+    };
+
+    i32x4 b0[KU], a0[MT][KU], b1[KU], a1[MT][KU];
+    load_chunk(ks_begin, b0, a0);
+    for(int ks = ks_begin; ks < ks_end; ks += 2 * KU)
+    {
+        load_chunk(ks + KU, b1, a1);
+        mfma_chunk(b0, a0);
+        load_chunk(ks + 2 * KU, b0, a0);
+        mfma_chunk(b1, a1);
+    }
+
+    // ---- sum the waves' partial tiles, then the epilogue on wave 0 ---------------------
+#pragma unroll
+    for(int mt = 0; mt < MT; ++mt)
+        red[wave][mt][lane] = acc[mt];
+    __syncthreads();
+    if(wave != 0)
+        return;
+#pragma unroll
+    for(int mt = 0; mt < MT; ++mt)
+    {
+        acc_t s = red[0][mt][lane];
+#pragma unroll
+        for(int w = 1; w < NW; ++w)
+        {
+            const acc_t v = red[w][mt][lane];
+            s[0] += v[0], s[1] += v[1], s[2] += v[2], s[3] += v[3];
+        }
+        // lane (m = lane%16, q): columns n0 + 4q .. 4q+3 of row 16*mt + m
+        const int m  = 16 * mt + (int)r;
+        const int nn = n0 + 4 * (int)q;
+        if(m >= p.M || nn >= p.N)
+            continue;
+        if constexpr(DT == DT_I8)
+        {
+            int b[4];
+#pragma unroll
+            for(int j = 0; j < 4; ++j)
+                b[j] = p.epi == EPI_REQUANT_RND  ? requant_rnd(s[j], p.scale_gemm, p.scale_relu)
+                       : p.epi == EPI_REQUANT_CK ? requant_ck(s[j], p.scale_gemm, p.scale_relu)
+                                                 : s[j];
+            int8_t* crow = reinterpret_cast<int8_t*>(p.c) + (size_t)m * p.ldc + nn;
+            if(nn + 4 <= p.N && ((reinterpret_cast<uintptr_t>(crow)) & 3u) == 0)
+                *reinterpret_cast<int*>(crow) = pack4_low_bytes(b[0], b[1], b[2], b[3]);
+            else
+            {
+#pragma unroll
+                for(int j = 0; j < 4; ++j)
+                    if(nn + j < p.N)
+                        crow[j] = (int8_t)b[j];
+            }
+        }
+        else
+        {
+            _Float16* crow = reinterpret_cast<_Float16*>(p.c) + (size_t)m * p.ldc + nn;
+#pragma unroll
+            for(int j = 0; j < 4; ++j)
+                if(nn + j < p.N)
+                    crow[j] = (_Float16)s[j];
+        }
+    }
+}
+
+} // namespace ckx

@@ -15,7 +15,7 @@ def stream():
     return torch.cuda.current_stream().cuda_stream
 
 
-def gemm_i8(a_mk, b_nk, c_op, instance=capi.INSTANCE_AUTO, ldc=None, time_kernel=False):
+def gemm_i8(a_mk, b_nk, c_op, instance=capi.INSTANCE_AUTO, ldc=None, time_kernel=False, allow_unsupported=False):
     """A [M,K] row-major, B given as [N,K] (column-major K x N). Returns int8 [M,N] (and ms)."""
     M, K = a_mk.shape
     N = b_nk.shape[0]
@@ -25,6 +25,8 @@ def gemm_i8(a_mk, b_nk, c_op, instance=capi.INSTANCE_AUTO, ldc=None, time_kernel
     op = ck.DeviceGemmInt8(instance)
     arg = op.MakeArgumentPointer(da, db, dc, M, N, K, a_mk.shape[1], b_nk.shape[1], ldc,
                                  ck.PassThrough(), ck.PassThrough(), c_op)
+    if allow_unsupported and not op.IsSupportedArgument(arg):
+        return None
     assert op.IsSupportedArgument(arg), capi.last_error()
     ms = op.MakeInvokerPointer().Run(arg, ck.StreamConfig(stream(), time_kernel))
     torch.cuda.synchronize()
@@ -34,13 +36,15 @@ def gemm_i8(a_mk, b_nk, c_op, instance=capi.INSTANCE_AUTO, ldc=None, time_kernel
     return (out[:, :N], ms) if time_kernel else out[:, :N]
 
 
-def gemm_f16(a_mk, b_nk, instance=capi.INSTANCE_AUTO, time_kernel=False):
+def gemm_f16(a_mk, b_nk, instance=capi.INSTANCE_AUTO, time_kernel=False, allow_unsupported=False):
     M, K = a_mk.shape
     N = b_nk.shape[0]
     da, db = dev(a_mk), dev(b_nk)
     dc = torch.full((M, N), float("nan"), dtype=torch.float16, device="cuda")
     op = ck.DeviceGemmF16(instance)
     arg = op.MakeArgumentPointer(da, db, dc, M, N, K, K, K, N)
+    if allow_unsupported and not op.IsSupportedArgument(arg):
+        return None
     assert op.IsSupportedArgument(arg), capi.last_error()
     ms = op.MakeInvokerPointer().Run(arg, ck.StreamConfig(stream(), time_kernel))
     torch.cuda.synchronize()
