@@ -30,6 +30,9 @@ sys.path.insert(0, ROOT)
 
 PEAK = {"f16": 2516.6, "i8": 5033.2}   # dense MFMA TFLOP/s / TOP/s, 256 CUs x 2.4 GHz
 HBM_PEAK_GBS = 8000.0
+# Bytes crossing the L2 <-> fabric boundary per launch, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
+# scaled by a 256 MiB copy in the same run (profiles/gemm_tile_fp16_int8_4096_hbm_traffic.md).
+MEASURED_TRAFFIC = {"fp16_gemm_4096": 2.350e8, "int8_requant_gemm_4096": 1.178e8}
 
 
 def _conv_workload(name, dtype, C, K, f, HW, st, pd, N=256):
@@ -241,10 +244,10 @@ def main():
     unit = "TFLOP/s" if w["dtype"] == "f16" else "TOP/s"
     if r["bound"] == "mfma":
         roof = {"bound": "mfma", "achieved": round(r["tput"], 2), "peak": PEAK[w["dtype"]], "unit": unit,
-                "frac": round(r["mfma_frac"], 4), "traffic": None}
+                "frac": round(r["mfma_frac"], 4), "traffic": MEASURED_TRAFFIC.get(w["name"])}
     else:
         roof = {"bound": "hbm", "achieved": round(r["gbs"], 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                "frac": round(r["hbm_frac"], 4), "traffic": None}
+                "frac": round(r["hbm_frac"], 4), "traffic": MEASURED_TRAFFIC.get(w["name"])}
     line = {
         "metric": "int8 TOPS & fp16 TFLOPS at 4096^3 on 1 MI355X; % of dtype MFMA peak",
         "value": round(r["tput"], 2), "unit": unit, "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
