@@ -3,8 +3,9 @@
 // C [G,M,O] row-major (layout gmk_gnk_gno_gmo of upstream's DeviceBatchedGemmGemm; batch
 // offsets as in kernel_batched_gemm_xdlops_v2r3, device_batched_gemm_xdl.hpp:79-88).
 //
-// One workgroup (4 waves) owns 128 rows of one batch and walks N in chunks of 128 columns.
-// The [128 x 128] slice of the intermediate never leaves registers:
+// One workgroup owns 64 or 128 rows of one batch and walks N in steps of 128 columns; the next
+// step's B0 / B1 slices are prefetched into registers while the current one is multiplied.
+// The slice of the intermediate never leaves registers:
 //   gemm0 is issued as S^T = B0_frag x A_frag, so lane (l%16 = m, l/16 = q) holds S[m][n]
 //   for 4 values of n per MFMA tile; the B0 rows fed to a PAIR of tiles are chosen so that
 //   the pair gives the lane n = 32*pair + 8q .. +7, i.e. exactly the eight K-slots that the
@@ -32,28 +33,37 @@ struct GemmGemmArgs
     int M, N, K, O, batch;
     int sa, sb0, sb1, sc;
     int64_t bsa, bsb0, bsb1, bsc;
-    int slabs; // ceil(M / 128)
+    int slabs; // ceil(M / rows per workgroup)
 };
 
-template <int KS, int OG>
+// KS  k-steps of gemm0 (K padded to 32*KS), OG  64-column groups of the output (O padded to 64*OG),
+// MT  16-row MFMA tiles per wave, NW waves: a workgroup owns 16*MT*NW rows of one batch.
+template <int KS, int OG, int MT, int NW>
 struct GemmGemmCfg
 {
-    static constexpr int BM   = 128; // rows per workgroup
+    static constexpr int NT   = 64 * NW;
+    static constexpr int BM   = 16 * MT * NW;
     static constexpr int BNC  = 128; // columns of the intermediate per step
     static constexpr int KP   = KS * 32;
     static constexpr int OP   = OG * 64;
-    static constexpr int AST  = KP * 2 + 16;  // padded LDS row strides (bytes)
+    static constexpr int AST  = KP * 2 + 16;  // padded LDS row strides (bytes): 16 rows hit 16 bank groups
     static constexpr int B1ST = BNC * 2 + 16;
     static constexpr int A_BYTES   = BM * AST;
     static constexpr int B0_BYTES  = BNC * AST;
     static constexpr int B1T_BYTES = OP * B1ST;
     static constexpr int LDS       = A_BYTES + B0_BYTES + B1T_BYTES;
+    static constexpr int KCH = KP / 8; // 16-byte chunks per staged row of A / B0
+    static constexpr int OCH = OP / 8;
+    static constexpr int NB0 = BNC * KCH / NT; // 16-byte loads per thread and step
+    static constexpr int NB1 = BNC * OCH / NT;
+    static_assert(NB0 >= 1 && NB1 >= 1, "too many threads for one step");
 };
 
-template <int KS, int OG>
-__global__ __launch_bounds__(256) void gemm_gemm_kernel(const GemmGemmArgs p)
+template <int KS, int OG, int MT, int NW>
+__global__ __launch_bounds__(NW * 64) void gemm_gemm_kernel(const GemmGemmArgs p)
 {
-    using Cfg = GemmGemmCfg<KS, OG>;
+    using Cfg = GemmGemmCfg<KS, OG, MT, NW>;
+    constexpr int KCH = Cfg::KCH, OCH = Cfg::OCH, NB0 = Cfg::NB0, NB1 = Cfg::NB1, NT = Cfg::NT;
     extern __shared__ __attribute__((aligned(16))) uint8_t gg_smem[];
     uint8_t* sA   = gg_smem;
     uint8_t* sB0  = sA + Cfg::A_BYTES;
@@ -65,19 +75,79 @@ __global__ __launch_bounds__(256) void gemm_gemm_kernel(const GemmGemmArgs p)
     const int fr   = lane & 15; // MFMA row/col index supplied by this lane
     const int q    = lane >> 4; // K-slot group
 
-    const int g    = blockIdx.x / p.slabs;
-    const int m0   = (blockIdx.x - g * p.slabs) * Cfg::BM;
+    // Workgroups of one batch share B0[g] and B1[g]: keep them on one XCD (ids are dealt
+    // round-robin over 8 XCDs) so that those panels are fetched into one L2 only.
+    int g, slab;
+    {
+        const int nb = p.slabs * p.batch;
+        const int bid = blockIdx.x;
+        if((p.batch & 7) == 0)
+        {
+            const int xcd = bid & 7, local = bid >> 3;
+            g    = xcd + 8 * (local / p.slabs);
+            slab = local - (local / p.slabs) * p.slabs;
+        }
+        else
+        {
+            g    = bid / p.slabs;
+            slab = bid - g * p.slabs;
+        }
+        (void)nb;
+    }
+    const int m0       = slab * Cfg::BM;
     const _Float16* A  = p.a + (int64_t)g * p.bsa;
     const _Float16* B0 = p.b0 + (int64_t)g * p.bsb0;
     const _Float16* B1 = p.b1 + (int64_t)g * p.bsb1;
     _Float16* C        = p.c + (int64_t)g * p.bsc;
+    const i32x4 zero4  = {0, 0, 0, 0};
 
-    constexpr int KCH = Cfg::KP / 8; // 16-byte chunks per staged row of A / B0
-    constexpr int OCH = Cfg::OP / 8;
-    const i32x4 zero4 = {0, 0, 0, 0};
+    // ---- register prefetch of one step's B0 / B1 slices ------------------------------------
+    i32x4 rb0[NB0], rb1[NB1];
+    auto load_step = [&](int n0) {
+#pragma unroll
+        for(int i = 0; i < NB0; ++i)
+        {
+            const int idx = tid + NT * i;
+            const int row = idx / KCH, ch = idx - row * KCH;
+            const int n = n0 + row, k = ch * 8;
+            rb0[i] = (n < p.N && k < p.K) ? *reinterpret_cast<const i32x4*>(B0 + (int64_t)n * p.sb0 + k) : zero4;
+        }
+#pragma unroll
+        for(int i = 0; i < NB1; ++i)
+        {
+            // consecutive lanes take consecutive rows n: the transposed 2-byte LDS writes below
+            // then land in consecutive addresses (no bank conflicts); the 16-byte pieces of one
+            // 128-byte line are picked up by the same thread group across i and hit in L1
+            const int idx = tid + NT * i;
+            const int ch = idx / Cfg::BNC, row = idx - ch * Cfg::BNC;
+            const int n = n0 + row, o = ch * 8;
+            rb1[i] = (n < p.N && o < p.O) ? *reinterpret_cast<const i32x4*>(B1 + (int64_t)n * p.sb1 + o) : zero4;
+        }
+    };
+    auto store_step = [&]() {
+#pragma unroll
+        for(int i = 0; i < NB0; ++i)
+        {
+            const int idx = tid + NT * i;
+            const int row = idx / KCH, ch = idx - row * KCH;
+            *reinterpret_cast<i32x4*>(sB0 + row * Cfg::AST + ch * 16) = rb0[i];
+        }
+#pragma unroll
+        for(int i = 0; i < NB1; ++i)
+        {
+            const int idx = tid + NT * i;
+            const int ch = idx / Cfg::BNC, row = idx - ch * Cfg::BNC;
+            const f16x8 v = __builtin_bit_cast(f16x8, rb1[i]);
+#pragma unroll
+            for(int e = 0; e < 8; ++e) // transpose: B1T[o][n]
+                *reinterpret_cast<_Float16*>(sB1T + (ch * 8 + e) * Cfg::B1ST + row * 2) = v[e];
+        }
+    };
+
+    load_step(0);
 
     // ---- A slab -> LDS -> registers (kept for the whole kernel) -----------------------
-    for(int idx = tid; idx < Cfg::BM * KCH; idx += 256)
+    for(int idx = tid; idx < Cfg::BM * KCH; idx += NT)
     {
         const int row = idx / KCH, ch = idx - row * KCH;
         const int m = m0 + row, k = ch * 8;
@@ -87,50 +157,33 @@ __global__ __launch_bounds__(256) void gemm_gemm_kernel(const GemmGemmArgs p)
         *reinterpret_cast<i32x4*>(sA + row * Cfg::AST + ch * 16) = v;
     }
     __syncthreads();
-    f16x8 af[2][KS];
+    f16x8 af[MT][KS];
 #pragma unroll
-    for(int mt = 0; mt < 2; ++mt)
+    for(int mt = 0; mt < MT; ++mt)
 #pragma unroll
         for(int ks = 0; ks < KS; ++ks)
-            af[mt][ks] = *reinterpret_cast<const f16x8*>(sA + (wave * 32 + mt * 16 + fr) * Cfg::AST +
+            af[mt][ks] = *reinterpret_cast<const f16x8*>(sA + (wave * 16 * MT + mt * 16 + fr) * Cfg::AST +
                                                          (ks * 4 + q) * 16);
 
-    f32x4 acc1[2][OG * 4];
+    f32x4 acc1[MT][OG * 4];
 #pragma unroll
-    for(int mt = 0; mt < 2; ++mt)
+    for(int mt = 0; mt < MT; ++mt)
 #pragma unroll
         for(int t = 0; t < OG * 4; ++t)
             acc1[mt][t] = f32x4{0, 0, 0, 0};
 
     for(int n0 = 0; n0 < p.N; n0 += Cfg::BNC)
     {
-        __syncthreads(); // everyone is done reading the previous chunk
-        for(int idx = tid; idx < Cfg::BNC * KCH; idx += 256)
-        {
-            const int row = idx / KCH, ch = idx - row * KCH;
-            const int n = n0 + row, k = ch * 8;
-            i32x4 v = zero4;
-            if(n < p.N && k < p.K)
-                v = *reinterpret_cast<const i32x4*>(B0 + (int64_t)n * p.sb0 + k);
-            *reinterpret_cast<i32x4*>(sB0 + row * Cfg::AST + ch * 16) = v;
-        }
-        for(int idx = tid; idx < Cfg::BNC * OCH; idx += 256)
-        {
-            const int row = idx / OCH, ch = idx - row * OCH;
-            const int n = n0 + row, o = ch * 8;
-            f16x8 v = {0, 0, 0, 0, 0, 0, 0, 0};
-            if(n < p.N && o < p.O)
-                v = *reinterpret_cast<const f16x8*>(B1 + (int64_t)n * p.sb1 + o);
-#pragma unroll
-            for(int e = 0; e < 8; ++e)
-                *reinterpret_cast<_Float16*>(sB1T + (o + e) * Cfg::B1ST + row * 2) = v[e];
-        }
+        __syncthreads(); // everyone is done reading the previous step from LDS
+        store_step();
         __syncthreads();
+        if(n0 + Cfg::BNC < p.N)
+            load_step(n0 + Cfg::BNC); // in flight while this step is multiplied
 
         // ---- gemm0: S^T tiles, 8 tiles of 16 columns, pairs share a 32-column span -----
-        f32x4 s[2][8];
+        f32x4 s[MT][8];
 #pragma unroll
-        for(int mt = 0; mt < 2; ++mt)
+        for(int mt = 0; mt < MT; ++mt)
 #pragma unroll
             for(int t = 0; t < 8; ++t)
                 s[mt][t] = f32x4{0, 0, 0, 0};
@@ -143,14 +196,14 @@ __global__ __launch_bounds__(256) void gemm_gemm_kernel(const GemmGemmArgs p)
                 const f16x8 b0f =
                     *reinterpret_cast<const f16x8*>(sB0 + row * Cfg::AST + (ks * 4 + q) * 16);
 #pragma unroll
-                for(int mt = 0; mt < 2; ++mt)
+                for(int mt = 0; mt < MT; ++mt)
                     s[mt][t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(b0f, af[mt][ks], s[mt][t], 0, 0, 0);
             }
 
         // ---- fp32 -> fp16 (RNE): the pair (2*pr, 2*pr+1) is the gemm1 operand for 32 n ----
-        f16x8 sf[2][4];
+        f16x8 sf[MT][4];
 #pragma unroll
-        for(int mt = 0; mt < 2; ++mt)
+        for(int mt = 0; mt < MT; ++mt)
 #pragma unroll
             for(int pr = 0; pr < 4; ++pr)
 #pragma unroll
@@ -170,7 +223,7 @@ __global__ __launch_bounds__(256) void gemm_gemm_kernel(const GemmGemmArgs p)
                 const f16x8 b1f =
                     *reinterpret_cast<const f16x8*>(sB1T + o * Cfg::B1ST + (32 * pr + 8 * q) * 2);
 #pragma unroll
-                for(int mt = 0; mt < 2; ++mt)
+                for(int mt = 0; mt < MT; ++mt)
                     acc1[mt][ot] =
                         __builtin_amdgcn_mfma_f32_16x16x32_f16(b1f, sf[mt][pr], acc1[mt][ot], 0, 0, 0);
             }
@@ -178,9 +231,9 @@ __global__ __launch_bounds__(256) void gemm_gemm_kernel(const GemmGemmArgs p)
 
     const bool vec_ok = ((reinterpret_cast<uintptr_t>(C) | ((uintptr_t)p.sc * 2)) & 15u) == 0;
 #pragma unroll
-    for(int mt = 0; mt < 2; ++mt)
+    for(int mt = 0; mt < MT; ++mt)
     {
-        const int m = m0 + wave * 32 + mt * 16 + fr;
+        const int m = m0 + wave * 16 * MT + mt * 16 + fr;
         if(m >= p.M)
             continue;
 #pragma unroll
@@ -197,11 +250,13 @@ __global__ __launch_bounds__(256) void gemm_gemm_kernel(const GemmGemmArgs p)
 }
 
 // ---------------------------------------------------------------- host side
-constexpr int kNumGemmGemmInstances = 1;
+constexpr int kNumGemmGemmInstances = 3;
 
-inline const char* gemm_gemm_instance_name(int)
+inline const char* gemm_gemm_instance_name(int i)
 {
-    return "MI355X_Mfma16_GemmGemm<128 rows, 128-col steps, K<=128, O<=128>";
+    return i == 0   ? "MI355X_Mfma16_GemmGemm<128 rows, 4 waves x 32, 128-col steps, K<=128, O<=128>"
+           : i == 1 ? "MI355X_Mfma16_GemmGemm<64 rows, 4 waves x 16, 128-col steps, K<=128, O<=128>"
+                    : "MI355X_Mfma16_GemmGemm<128 rows, 8 waves x 16, 128-col steps, K<=128, O<=128>";
 }
 
 inline bool gemm_gemm_supported(int M, int N, int K, int O, int batch, int sa, int sb0, int sb1, int sc,
@@ -211,7 +266,7 @@ inline bool gemm_gemm_supported(int M, int N, int K, int O, int batch, int sa, i
     (void)bsc;
     if(M < 0 || N < 0 || K < 0 || O < 0 || batch < 0)
         return why = "invalid: negative dimension", false;
-    if(instance != -1 && instance != 0)
+    if(instance < -1 || instance >= kNumGemmGemmInstances)
         return why = "invalid: no such instance", false;
     if(K > 128 || O > 128)
         return why = "K and O above 128 are not built", false;
@@ -219,16 +274,16 @@ inline bool gemm_gemm_supported(int M, int N, int K, int O, int batch, int sa, i
         return why = "K, O and the A/B0/B1 strides must be multiples of 8 elements (16 bytes)", false;
     if(sa < K || sb0 < K || sb1 < O || sc < O)
         return why = "stride smaller than the contiguous extent", false;
-    if((long)((M + 127) / 128) * batch >= (1l << 31))
+    if((long)((M + 63) / 64) * batch >= (1l << 31))
         return why = "grid too large", false;
     return true;
 }
 
-template <int KS, int OG>
-inline hipError_t gemm_gemm_launch_t(const GemmGemmArgs& a, hipStream_t s)
+template <int KS, int OG, int MT, int NW>
+inline hipError_t gemm_gemm_launch_t(GemmGemmArgs a, hipStream_t s)
 {
-    using Cfg  = GemmGemmCfg<KS, OG>;
-    auto* kern = &gemm_gemm_kernel<KS, OG>;
+    using Cfg  = GemmGemmCfg<KS, OG, MT, NW>;
+    auto* kern = &gemm_gemm_kernel<KS, OG, MT, NW>;
     static std::once_flag once;
     static hipError_t attr_err = hipSuccess;
     std::call_once(once, [&] {
@@ -237,27 +292,38 @@ inline hipError_t gemm_gemm_launch_t(const GemmGemmArgs& a, hipStream_t s)
     });
     if(attr_err != hipSuccess)
         return attr_err;
-    hipLaunchKernelGGL(kern, dim3(a.slabs * a.batch), dim3(256), Cfg::LDS, s, a);
+    a.slabs = (a.M + Cfg::BM - 1) / Cfg::BM;
+    hipLaunchKernelGGL(kern, dim3(a.slabs * a.batch), dim3(Cfg::NT), Cfg::LDS, s, a);
     return hipGetLastError();
+}
+
+template <int MT, int NW>
+inline hipError_t gemm_gemm_launch_mt(const GemmGemmArgs& g, hipStream_t s)
+{
+    const int ks = g.K <= 32 ? 1 : (g.K <= 64 ? 2 : 4);
+    const int og = g.O <= 64 ? 1 : 2;
+    if(ks == 1)
+        return og == 1 ? gemm_gemm_launch_t<1, 1, MT, NW>(g, s) : gemm_gemm_launch_t<1, 2, MT, NW>(g, s);
+    if(ks == 2)
+        return og == 1 ? gemm_gemm_launch_t<2, 1, MT, NW>(g, s) : gemm_gemm_launch_t<2, 2, MT, NW>(g, s);
+    return og == 1 ? gemm_gemm_launch_t<4, 1, MT, NW>(g, s) : gemm_gemm_launch_t<4, 2, MT, NW>(g, s);
 }
 
 inline hipError_t gemm_gemm_launch(const void* a, const void* b0, const void* b1, void* c, int M, int N, int K,
                                    int O, int batch, int sa, int sb0, int sb1, int sc, int64_t bsa,
-                                   int64_t bsb0, int64_t bsb1, int64_t bsc, int /*instance*/, hipStream_t s)
+                                   int64_t bsb0, int64_t bsb1, int64_t bsc, int instance, hipStream_t s)
 {
     GemmGemmArgs g;
     g.a = (const _Float16*)a, g.b0 = (const _Float16*)b0, g.b1 = (const _Float16*)b1, g.c = (_Float16*)c;
     g.M = M, g.N = N, g.K = K, g.O = O, g.batch = batch;
     g.sa = sa, g.sb0 = sb0, g.sb1 = sb1, g.sc = sc;
     g.bsa = bsa, g.bsb0 = bsb0, g.bsb1 = bsb1, g.bsc = bsc;
-    g.slabs      = (M + 127) / 128;
-    const int ks = K <= 32 ? 1 : (K <= 64 ? 2 : 4);
-    const int og = O <= 64 ? 1 : 2;
-    if(ks == 1)
-        return og == 1 ? gemm_gemm_launch_t<1, 1>(g, s) : gemm_gemm_launch_t<1, 2>(g, s);
-    if(ks == 2)
-        return og == 1 ? gemm_gemm_launch_t<2, 1>(g, s) : gemm_gemm_launch_t<2, 2>(g, s);
-    return og == 1 ? gemm_gemm_launch_t<4, 1>(g, s) : gemm_gemm_launch_t<4, 2>(g, s);
+    g.slabs = 0;
+    if(instance < 0)
+        instance = 2;
+    return instance == 0 ? gemm_gemm_launch_mt<2, 4>(g, s)
+           : instance == 1 ? gemm_gemm_launch_mt<1, 4>(g, s)
+                           : gemm_gemm_launch_mt<1, 8>(g, s);
 }
 
 } // namespace ckx
