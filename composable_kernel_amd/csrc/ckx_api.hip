@@ -4,6 +4,7 @@
 #include <hip/hip_runtime.h>
 
 #include <cstdio>
+#include <cstdlib>
 #include <cstring>
 #include <mutex>
 #include <string>
@@ -28,6 +29,20 @@ int hip_fail(hipError_t e, const char* what)
     return fail(CKX_HIP_ERROR, std::string(what) + ": " + hipGetErrorString(e));
 }
 
+// int8 outputs at least this large are stored non-temporally (measured on the N256 C256->K512
+// 1x1 s2 conv: int8, 103 MB of output, 68.4 us -> 65.0 us; fp16 outputs get SLOWER, 105 -> 127 us,
+// so they always use plain stores)
+long stream_output_bytes()
+{
+    // CKX_STREAM_OUTPUT_BYTES overrides the threshold (tuning knob; 0 = always, -1 = never)
+    static long v = [] {
+        const char* e = std::getenv("CKX_STREAM_OUTPUT_BYTES");
+        long t        = e ? std::atol(e) : (64l << 20);
+        return t < 0 ? (1l << 62) : t;
+    }();
+    return v;
+}
+
 ckx::MagicDiv make_magic(uint32_t d)
 {
     // include/ck/utility/magic_division.hpp:28-54
@@ -45,11 +60,25 @@ ckx::MagicDiv make_magic(uint32_t d)
 // ------------------------------------------------------------ tile instances
 typedef hipError_t (*tile_launch_fn)(const ckx::GemmArgs&, int grid, hipStream_t);
 
-template <int DT, int BM, int BN, int WM, int WN, int BKB, int NST, bool IM2COL, bool PP>
-hipError_t launch_tile(const ckx::GemmArgs& a, int grid, hipStream_t s)
+int num_cus()
 {
-    using T              = ckx::GemmTile<DT, BM, BN, WM, WN, BKB, NST, IM2COL, PP>;
-    auto* kern           = &ckx::gemm_tile_kernel<DT, BM, BN, WM, WN, BKB, NST, IM2COL, PP>;
+    static int n = [] {
+        int dev = 0, cus = 0;
+        if(hipGetDevice(&dev) != hipSuccess ||
+           hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0)
+            cus = 256;
+        return cus;
+    }();
+    return n;
+}
+
+// Persistent launch: at most (workgroups that fit a CU) x (CUs) workgroups, a multiple of 8 so
+// that workgroup b always lands on XCD b % 8 together with the tiles b, b + grid, ...
+template <int DT, int BM, int BN, int WM, int WN, int BKB, int NST, bool IM2COL>
+hipError_t launch_tile(const ckx::GemmArgs& a, int tiles, hipStream_t s)
+{
+    using T              = ckx::GemmTile<DT, BM, BN, WM, WN, BKB, NST, IM2COL>;
+    auto* kern           = &ckx::gemm_tile_kernel<DT, BM, BN, WM, WN, BKB, NST, IM2COL>;
     static std::once_flag once;
     static hipError_t attr_err = hipSuccess;
     std::call_once(once, [&] {
@@ -58,6 +87,12 @@ hipError_t launch_tile(const ckx::GemmArgs& a, int grid, hipStream_t s)
     });
     if(attr_err != hipSuccess)
         return attr_err;
+    int per_cu = 160 * 1024 / T::LDS;
+    per_cu     = per_cu > 2048 / T::NT ? 2048 / T::NT : per_cu;
+    per_cu     = per_cu < 1 ? 1 : per_cu;
+    int grid   = num_cus() * per_cu;
+    grid -= grid % 8;
+    grid = tiles < grid ? tiles : grid;
     hipLaunchKernelGGL(kern, dim3(grid), dim3(T::NT), T::LDS, s, a);
     return hipGetLastError();
 }
@@ -70,27 +105,24 @@ struct TileInstance
     tile_launch_fn dense_i8, dense_f16, conv_i8, conv_f16;
 };
 
-#define CKX_TILE(BM, BN, WM, WN, BKB, NST, PP, EFF)                                                     \
-    {                                                                                                   \
-        "MI355X_Mfma16_Tile<" #BM ", " #BN ", " #BKB "B x" #NST ", waves " #WM "x" #WN ", pp" #PP ">", BM, BN,     \
-            WM* WN * 64, NST*(BM + BN) * BKB, EFF,                                                      \
-            &launch_tile<ckx::DT_I8, BM, BN, WM, WN, BKB, NST, false, PP>,                                   \
-            &launch_tile<ckx::DT_F16, BM, BN, WM, WN, BKB, NST, false, PP>,                                 \
-            &launch_tile<ckx::DT_I8, BM, BN, WM, WN, BKB, NST, true, PP>,                                   \
-            &launch_tile<ckx::DT_F16, BM, BN, WM, WN, BKB, NST, true, PP>                                   \
+#define CKX_TILE(BM, BN, WM, WN, EFF)                                                              \
+    {                                                                                              \
+        "MI355X_Mfma16_Tile<" #BM ", " #BN ", 128B x2, waves " #WM "x" #WN ">", BM, BN, WM* WN * 64,     \
+            2 * (BM + BN) * 128, EFF, &launch_tile<ckx::DT_I8, BM, BN, WM, WN, 128, 2, false>,           \
+            &launch_tile<ckx::DT_F16, BM, BN, WM, WN, 128, 2, false>,                                 \
+            &launch_tile<ckx::DT_I8, BM, BN, WM, WN, 128, 2, true>,                                   \
+            &launch_tile<ckx::DT_F16, BM, BN, WM, WN, 128, 2, true>                                   \
     }
 
 const TileInstance kTiles[] = {
-    CKX_TILE(256, 256, 2, 4, 128, 2, 0, 1.00f),
-    CKX_TILE(256, 128, 4, 2, 128, 2, 0, 0.84f),
-    CKX_TILE(128, 128, 2, 2, 128, 2, 0, 0.78f),
-    CKX_TILE(128, 64, 4, 1, 128, 2, 0, 0.68f),
-    CKX_TILE(64, 64, 4, 1, 128, 2, 0, 0.55f),
-    CKX_TILE(32, 64, 2, 1, 128, 2, 0, 0.42f),
-    CKX_TILE(16, 64, 1, 1, 128, 2, 0, 0.27f),
-    CKX_TILE(256, 256, 2, 4, 128, 2, 1, 0.97f),
-    CKX_TILE(256, 128, 4, 2, 128, 2, 1, 0.83f),
-    CKX_TILE(256, 64, 8, 1, 128, 2, 0, 0.70f),
+    CKX_TILE(256, 256, 2, 4, 1.00f),
+    CKX_TILE(256, 128, 4, 2, 0.84f),
+    CKX_TILE(128, 128, 2, 2, 0.78f),
+    CKX_TILE(128, 64, 4, 1, 0.68f),
+    CKX_TILE(64, 64, 4, 1, 0.55f),
+    CKX_TILE(32, 64, 2, 1, 0.42f),
+    CKX_TILE(16, 64, 1, 1, 0.27f),
+    CKX_TILE(256, 64, 8, 1, 0.70f),
 };
 constexpr int kNumTiles = sizeof(kTiles) / sizeof(kTiles[0]);
 
@@ -216,6 +248,7 @@ int run_gemm(int dt, const void* a, const void* b, void* c, int M, int N, int K,
     g.epi        = epi;
     g.scale_gemm = sg;
     g.scale_relu = sr;
+    g.nt_store   = es == 1 && (long)M * N * es >= stream_output_bytes();
     if(ti >= kNumTiles)
     {
         const SkinnyInstance& k = kSkinny[ti - kNumTiles];
@@ -246,6 +279,10 @@ int check_conv(int op, const ckx_conv2d_desc* d, int epi, int instance)
        d->Ho < 0 || d->Wo < 0 || d->stride_h <= 0 || d->stride_w <= 0 || d->dilation_h <= 0 ||
        d->dilation_w <= 0 || d->pad_top < 0 || d->pad_left < 0 || d->pad_bottom < 0 || d->pad_right < 0)
         return fail(CKX_INVALID_VALUE, "bad conv geometry");
+    // window coordinates are kept as signed 16-bit pairs in the kernel
+    if(d->Hi > 16384 || d->Wi > 16384 || d->pad_top >= 16384 || d->pad_left >= 16384 ||
+       (long)(d->Y - 1) * d->dilation_h >= 16384 || (long)(d->X - 1) * d->dilation_w >= 16384)
+        return fail(CKX_UNSUPPORTED, "spatial extents above 16384 are not addressed");
     // the output extent has to be what the geometry implies (conv_util.cpp:103-114)
     const int ho = (d->Hi + d->pad_top + d->pad_bottom - ((d->Y - 1) * d->dilation_h + 1)) / d->stride_h + 1;
     const int wo = (d->Wi + d->pad_left + d->pad_right - ((d->X - 1) * d->dilation_w + 1)) / d->stride_w + 1;
@@ -292,6 +329,7 @@ int run_conv(int op, const void* in, const void* wei, void* out, const ckx_conv2
     g.epi        = epi;
     g.scale_gemm = sg;
     g.scale_relu = sr;
+    g.nt_store   = es == 1 && (long)M * N * es >= stream_output_bytes();
     g.cv.Hi = d->Hi, g.cv.Wi = d->Wi, g.cv.C = d->C;
     g.cv.sH = d->stride_h, g.cv.sW = d->stride_w, g.cv.dH = d->dilation_h, g.cv.dW = d->dilation_w;
     g.cv.pT = d->pad_top, g.cv.pL = d->pad_left;

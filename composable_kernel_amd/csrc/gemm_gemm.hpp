@@ -320,7 +320,7 @@ inline hipError_t gemm_gemm_launch(const void* a, const void* b0, const void* b1
     g.bsa = bsa, g.bsb0 = bsb0, g.bsb1 = bsb1, g.bsc = bsc;
     g.slabs = 0;
     if(instance < 0)
-        instance = 2;
+        instance = 0;
     return instance == 0 ? gemm_gemm_launch_mt<2, 4>(g, s)
            : instance == 1 ? gemm_gemm_launch_mt<1, 4>(g, s)
                            : gemm_gemm_launch_mt<1, 8>(g, s);

@@ -52,16 +52,20 @@ enum
 #ifndef CKX_SWZ_SHIFT
 #define CKX_SWZ_SHIFT 0
 #endif
-// C tile stores: plain, or streaming (CKX_NT_STORE) so the lines do not linger dirty in L2
-#ifdef CKX_NT_STORE
-#define CKX_STORE(ptr, val) __builtin_nontemporal_store((val), (ptr))
-#else
-#define CKX_STORE(ptr, val) (*(ptr) = (val))
-#endif
-// which of the two ping-pong groups a wave belongs to: waves w and w+4 share a SIMD
-#ifndef CKX_PP_GROUP
-#define CKX_PP_GROUP(wave) ((wave) >> 2)
-#endif
+// C tile stores: plain, or streaming (non-temporal) when the output is too large to be worth
+// keeping in L2: dirty lines of a streamed output otherwise queue up behind the write-back
+// and the store acknowledgements stall the K pipeline of the next tile.
+// (Written as inline assembly: two stores that differ only in the non-temporal hint get merged
+// into one plain store by the optimiser.)
+template <typename V>
+__device__ __forceinline__ void store_vec(V* ptr, V val, bool nt)
+{
+    static_assert(sizeof(V) == 16, "16-byte vector store");
+    if(nt)
+        asm volatile("global_store_dwordx4 %0, %1, off nt" ::"v"(ptr), "v"(val) : "memory");
+    else
+        *ptr = val;
+}
 
 // q = n / d for 0 <= n < 2^31 (include/ck/utility/magic_division.hpp:28-54,132-137)
 struct MagicDiv
@@ -101,6 +105,7 @@ struct GemmArgs
     int tiles_m, tiles_n;
     int epi;
     float scale_gemm, scale_relu;
+    int nt_store; // stream the C tile past L2 (large outputs)
     ConvGeom cv;
 };
 
@@ -189,7 +194,7 @@ __device__ __forceinline__ int pack4_low_bytes(int b0, int b1, int b2, int b3)
 // 16 consecutive int8 outputs of one row
 template <int EPI>
 __device__ __forceinline__ void store_row16_i8(int8_t* crow, int n0, int N, bool vec_ok, const i32x4 (&v)[4],
-                                               float sg, float sr)
+                                               float sg, float sr, bool nt = false)
 {
     int b[16];
 #pragma unroll
@@ -203,7 +208,7 @@ __device__ __forceinline__ void store_row16_i8(int8_t* crow, int n0, int N, bool
 #pragma unroll
         for(int w = 0; w < 4; ++w)
             pk[w] = pack4_low_bytes(b[4 * w], b[4 * w + 1], b[4 * w + 2], b[4 * w + 3]);
-        CKX_STORE(reinterpret_cast<i32x4*>(crow + n0), pk);
+        store_vec(reinterpret_cast<i32x4*>(crow + n0), pk, nt);
     }
     else
     {
@@ -215,7 +220,7 @@ __device__ __forceinline__ void store_row16_i8(int8_t* crow, int n0, int N, bool
 }
 
 __device__ __forceinline__ void store_row16_f16(_Float16* crow, int n0, int N, bool vec_ok,
-                                                const f32x4 (&v)[4])
+                                                const f32x4 (&v)[4], bool nt = false)
 {
     if(vec_ok && n0 + 16 <= N)
     {
@@ -228,8 +233,8 @@ __device__ __forceinline__ void store_row16_f16(_Float16* crow, int n0, int N, b
             hi[j]     = (_Float16)v[2][j];
             hi[4 + j] = (_Float16)v[3][j];
         }
-        CKX_STORE(reinterpret_cast<f16x8*>(crow + n0), lo);
-        CKX_STORE(reinterpret_cast<f16x8*>(crow + n0 + 8), hi);
+        store_vec(reinterpret_cast<f16x8*>(crow + n0), lo, nt);
+        store_vec(reinterpret_cast<f16x8*>(crow + n0 + 8), hi, nt);
     }
     else
     {
@@ -243,9 +248,12 @@ __device__ __forceinline__ void store_row16_f16(_Float16* crow, int n0, int N, b
 }
 
 // ------------------------------------------------------------------- kernel
-// BKB   bytes of every row staged per K tile (64 or 128)
-// NST   LDS stages; the loads of K tile k+NST-1 are issued while tile k is multiplied
-template <int DT, int BM, int BN, int WM, int WN, int BKB, int NST, bool IM2COL, bool PINGPONG = false>
+// BKB   bytes of every row staged per K tile (128)
+// NST   LDS stages (2)
+// The kernel is PERSISTENT: workgroup b works on tiles b, b + gridDim.x, ... and the K-tile
+// pipeline runs straight across tile boundaries, so the first loads of the next tile are in
+// flight under the last MFMAs, the epilogue arithmetic and the C stores of the current one.
+template <int DT, int BM, int BN, int WM, int WN, int BKB, int NST, bool IM2COL>
 struct GemmTile
 {
     static constexpr int NW      = WM * WN;
@@ -265,22 +273,15 @@ struct GemmTile
     static constexpr int NLA     = BM * CPR / NT; // 16-byte loads per thread and K tile, A
     static constexpr int NLB     = BN * CPR / NT;
     static constexpr int LPT     = NLA + NLB;
-    static_assert(BKB == 64 || BKB == 128, "K tile is 64 or 128 bytes per row");
-    static_assert(NST >= 2 && (NST - 2) * LPT < 64, "vmcnt is a 6-bit counter");
+    static_assert(BKB == 128 && KSTEPS == 2 && NST == 2, "pipeline written for 128-byte K tiles, two stages");
     static_assert(WTM % 16 == 0 && WTN % 64 == 0, "wave tile must be 16k x 64k");
     static_assert((BM * CPR) % NT == 0 && (BN * CPR) % NT == 0, "tile rows must split over the waves");
 
     using acc_t = typename std::conditional<DT == DT_I8, i32x4, f32x4>::type;
 
     // XOR swizzle of the chunk position: the 16 rows read by one MFMA fragment load spread
-    // over all LDS banks.
-    __device__ static __forceinline__ uint32_t swz(uint32_t row)
-    {
-        if constexpr(CPR == 8)
-            return (row >> CKX_SWZ_SHIFT) & 7u;
-        else
-            return (row >> 2) & 3u;
-    }
+    // over all LDS banks (measured: 0 bank conflicts, 256 B/clk).
+    __device__ static __forceinline__ uint32_t swz(uint32_t row) { return (row >> CKX_SWZ_SHIFT) & 7u; }
     __device__ static __forceinline__ uint32_t chunk_offset(uint32_t row, uint32_t chunk)
     {
         return row * BKB + ((chunk ^ swz(row)) << 4);
@@ -294,95 +295,114 @@ struct GemmTile
         const int wm   = wave / WN;
         const int wn   = wave % WN;
 
-        int tm, tn;
-        tile_of_block(blockIdx.x, p.tiles_m, p.tiles_n, tm, tn);
-
+        const int ntiles      = p.tiles_m * p.tiles_n;
+        const int gstride     = (int)gridDim.x;
         const uint32_t kbytes = (uint32_t)p.K * ES;
-        const int nk          = (int)((kbytes + BKB - 1) / BKB);
+        const int nk_real     = (int)((kbytes + BKB - 1) / BKB);
+        const int nk          = nk_real > 0 ? nk_real : 1; // K == 0: one all-zero K tile, C = epilogue(0)
 
         const __amdgpu_buffer_rsrc_t rsrc_a = make_rsrc(p.a, p.a_bytes);
         const __amdgpu_buffer_rsrc_t rsrc_b = make_rsrc(p.b, p.b_bytes);
 
         // ---- per-thread load slots -------------------------------------------------
         // slot j of this thread fills LDS row (j*NW + wave)*RPI + lane/CPR, chunk position lane%CPR
+        // Every slot of a thread sits at the same chunk position: the slot rows differ by
+        // multiples of 8 and the swizzle is row & 7, i.e. lane/8 for all of them.
+        static_assert(CKX_SWZ_SHIFT == 0 && RPI == 8, "one chunk position per thread");
         uint32_t a_off[NLA];  // dense: byte offset of (row, chunk) at K tile 0, or kOutOfRange
-        uint32_t a_kb[NLA];   // byte offset of the chunk inside a K tile
-        int a_hi0[NLA], a_wi0[NLA]; // im2col: top-left input coordinate of the row's window
+        uint32_t a_hw0[NLA]; // im2col: top-left input coordinate of the row's window, (hi0 << 16) | (wi0 & 0xffff)
         uint32_t b_off[NLB];
-        uint32_t b_kb[NLB];
+        const uint32_t kb = ((uint32_t)(lane % CPR) ^ (uint32_t)((lane / CPR) & 7)) << 4; // chunk byte offset in a K tile
+
+        // row / column offsets of the tile the LOAD cursor is on (tile >= ntiles: nothing valid)
+        auto setup_tile = [&](int tile) {
+            int tm = 0, tn = 0;
+            const bool live = tile < ntiles;
+            if(live)
+                tile_of_block(tile, p.tiles_m, p.tiles_n, tm, tn);
 #pragma unroll
-        for(int j = 0; j < NLA; ++j)
-        {
-            const uint32_t r  = (uint32_t)((j * NW + wave) * RPI + lane / CPR);
-            const uint32_t ch = (uint32_t)(lane % CPR) ^ swz(r);
-            a_kb[j]           = ch << 4;
-            const uint32_t gm = (uint32_t)tm * BM + r;
-            if constexpr(!IM2COL)
+            for(int j = 0; j < NLA; ++j)
             {
-                a_off[j] = gm < (uint32_t)p.M ? gm * (uint32_t)p.lda * ES + a_kb[j] : kOutOfRange;
-                a_hi0[j] = a_wi0[j] = 0;
-            }
-            else
-            {
-                if(gm < (uint32_t)p.M)
+                const uint32_t r  = (uint32_t)((j * NW + wave) * RPI + lane / CPR);
+                const uint32_t gm = (uint32_t)tm * BM + r;
+                const bool ok     = live && gm < (uint32_t)p.M;
+                if constexpr(!IM2COL)
                 {
-                    const uint32_t n   = magic_div(gm, p.cv.div_howo);
-                    const uint32_t rem = gm - n * p.cv.div_howo.d;
-                    const uint32_t ho  = magic_div(rem, p.cv.div_wo);
-                    const uint32_t wo  = rem - ho * p.cv.div_wo.d;
-                    a_hi0[j]           = (int)ho * p.cv.sH - p.cv.pT;
-                    a_wi0[j]           = (int)wo * p.cv.sW - p.cv.pL;
-                    a_off[j]           = n * (uint32_t)(p.cv.Hi * p.cv.Wi) * (uint32_t)p.cv.C; // elements
+                    a_off[j] = ok ? gm * (uint32_t)p.lda * ES + kb : kOutOfRange;
+                    a_hw0[j] = 0;
                 }
                 else
                 {
-                    a_hi0[j] = a_wi0[j] = -0x40000000; // every tap out of range
-                    a_off[j]            = 0;
+                    if(ok)
+                    {
+                        const uint32_t n   = magic_div(gm, p.cv.div_howo);
+                        const uint32_t rem = gm - n * p.cv.div_howo.d;
+                        const uint32_t ho  = magic_div(rem, p.cv.div_wo);
+                        const uint32_t wo  = rem - ho * p.cv.div_wo.d;
+                        const int hi0      = (int)ho * p.cv.sH - p.cv.pT;
+                        const int wi0      = (int)wo * p.cv.sW - p.cv.pL;
+                        a_hw0[j]           = ((uint32_t)hi0 << 16) | ((uint32_t)wi0 & 0xffffu);
+                        // byte offset of the window's top-left pixel; may be "negative" (wraps), the
+                        // sum with a valid tap's offset is always inside the tensor
+                        a_off[j] = (uint32_t)(((int)(n * (uint32_t)p.cv.Hi) + hi0) * p.cv.Wi + wi0) *
+                                   (uint32_t)(p.cv.C * ES);
+                    }
+                    else
+                    {
+                        a_hw0[j] = 0xC000C000u; // (-16384, -16384): every tap out of range
+                        a_off[j] = 0;
+                    }
                 }
             }
-        }
 #pragma unroll
-        for(int j = 0; j < NLB; ++j)
-        {
-            const uint32_t r  = (uint32_t)((j * NW + wave) * RPI + lane / CPR);
-            const uint32_t ch = (uint32_t)(lane % CPR) ^ swz(r);
-            b_kb[j]           = ch << 4;
-            const uint32_t gn = (uint32_t)tn * BN + b_row_to_col(r);
-            b_off[j] = gn < (uint32_t)p.N ? gn * (uint32_t)p.ldb * ES + b_kb[j] : kOutOfRange;
-        }
+            for(int j = 0; j < NLB; ++j)
+            {
+                const uint32_t r  = (uint32_t)((j * NW + wave) * RPI + lane / CPR);
+                const uint32_t gn = (uint32_t)tn * BN + b_row_to_col(r);
+                b_off[j] = (live && gn < (uint32_t)p.N) ? gn * (uint32_t)p.ldb * ES + kb : kOutOfRange;
+            }
+        };
 
-        // K tiles at or beyond nk are legal to request: every chunk of them is out of range,
-        // so the hardware writes zeros into a stage nobody reads. This keeps the number of
-        // loads in flight constant, which the vmcnt arithmetic below relies on.
-        auto issue_loads = [&](int kt) {
-            const int stage       = kt % NST;
+        // Direct global->LDS loads of K tile kt of the load cursor's tile into `stage`. Chunks past
+        // K (and whole tiles past the end of the work list) use an out-of-range offset: the
+        // hardware writes zeros, and the number of loads in flight stays constant.
+        auto issue_loads = [&](int kt, int stage) {
             uint8_t* sa           = smem + stage * STAGE;
             uint8_t* sb           = sa + A_TILE;
             const uint32_t k0     = (uint32_t)kt * BKB; // byte offset of the K tile
-            const bool tail       = (k0 + BKB > kbytes);
+            const bool k_ok       = k0 + kb < kbytes; // false only in the K tail (or past the end)
+            // im2col: every load slot of a thread sits at the same chunk position (the swizzle only
+            // depends on lane/8), so the tap (y, x) and channel offset are decoded ONCE per thread
+            // and K tile; a slot then only range-checks its own window.
+            int tap_dh = 0, tap_dw = 0;
+            uint32_t tap_off = 0;
+            bool tap_ok      = true;
+            if constexpr(IM2COL)
+            {
+                const uint32_t ke  = (k0 + kb) / ES; // element index along GEMM-K
+                const uint32_t y   = magic_div(ke, p.cv.div_xc);
+                const uint32_t rem = ke - y * p.cv.div_xc.d;
+                const uint32_t x   = magic_div(rem, p.cv.div_c);
+                const uint32_t cc  = rem - x * p.cv.div_c.d;
+                tap_dh             = (int)y * p.cv.dH;
+                tap_dw             = (int)x * p.cv.dW;
+                tap_off            = ((uint32_t)(tap_dh * p.cv.Wi + tap_dw) * (uint32_t)p.cv.C + cc) * ES;
+                tap_ok             = ke < (uint32_t)p.K;
+            }
 #pragma unroll
             for(int j = 0; j < NLA; ++j)
             {
                 uint32_t voff;
                 if constexpr(!IM2COL)
                 {
-                    voff = a_off[j] + k0;
-                    if(tail && k0 + a_kb[j] >= kbytes)
-                        voff = kOutOfRange;
+                    voff = k_ok ? a_off[j] + k0 : kOutOfRange;
                 }
                 else
                 {
-                    const uint32_t ke  = (k0 + a_kb[j]) / ES; // element index along GEMM-K
-                    const uint32_t y   = magic_div(ke, p.cv.div_xc);
-                    const uint32_t rem = ke - y * p.cv.div_xc.d;
-                    const uint32_t x   = magic_div(rem, p.cv.div_c);
-                    const uint32_t cc  = rem - x * p.cv.div_c.d;
-                    const int hi       = a_hi0[j] + (int)y * p.cv.dH;
-                    const int wi       = a_wi0[j] + (int)x * p.cv.dW;
-                    const bool ok      = (uint32_t)hi < (uint32_t)p.cv.Hi && (uint32_t)wi < (uint32_t)p.cv.Wi &&
-                                    ke < (uint32_t)p.K;
-                    voff = ok ? (a_off[j] + (uint32_t)(hi * p.cv.Wi + wi) * (uint32_t)p.cv.C + cc) * ES
-                              : kOutOfRange;
+                    const int hi0 = (int)a_hw0[j] >> 16, wi0 = (int)(a_hw0[j] << 16) >> 16;
+                    const bool ok = tap_ok && (uint32_t)(hi0 + tap_dh) < (uint32_t)p.cv.Hi &&
+                                    (uint32_t)(wi0 + tap_dw) < (uint32_t)p.cv.Wi;
+                    voff = ok ? a_off[j] + tap_off : kOutOfRange;
                 }
                 __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_a, (lds_ptr_t)(sa + (j * NW + wave) * 1024), 16,
                                                          voff, 0, 0, 0);
@@ -390,11 +410,22 @@ struct GemmTile
 #pragma unroll
             for(int j = 0; j < NLB; ++j)
             {
-                uint32_t voff = b_off[j] + k0;
-                if(tail && k0 + b_kb[j] >= kbytes)
-                    voff = kOutOfRange;
+                const uint32_t voff = k_ok ? b_off[j] + k0 : kOutOfRange;
                 __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_b, (lds_ptr_t)(sb + (j * NW + wave) * 1024), 16,
                                                          voff, 0, 0, 0);
+            }
+        };
+
+        // load cursor: (tile, kt) of the next K tile to request
+        int ld_tile = (int)blockIdx.x, ld_kt = 0;
+        setup_tile(ld_tile);
+        auto issue_next = [&](int stage) {
+            issue_loads(ld_kt, stage);
+            if(++ld_kt == nk)
+            {
+                ld_kt = 0;
+                ld_tile += gstride;
+                setup_tile(ld_tile);
             }
         };
 
@@ -450,145 +481,108 @@ struct GemmTile
             __builtin_amdgcn_sched_group_barrier(0x008, NM - NR * (NM / NR), 0);
         };
 
-        static_assert(KSTEPS == 2 && NST == 2, "pipeline written for 128-byte K tiles, two stages");
-        i32x4 af0[MT], bf0[NG * 4], af1[MT], bf1[NG * 4];
+        // ---- epilogue: registers -> global, 16 consecutive columns per lane -------------
+        const bool vec_ok = ((reinterpret_cast<uintptr_t>(p.c) | ((uintptr_t)p.ldc * ES)) & 15u) == 0;
+        const bool nt     = p.nt_store != 0;
+        auto epilogue = [&](int tile) {
+            int tm, tn;
+            tile_of_block(tile, p.tiles_m, p.tiles_n, tm, tn);
+#pragma unroll
+            for(int i = 0; i < MT; ++i)
+            {
+                const int m = tm * BM + wm * WTM + 16 * i + (lane & 15);
+#pragma unroll
+                for(int g = 0; g < NG; ++g)
+                {
+                    const int n0 = tn * BN + wn * WTN + 64 * g + 16 * (lane >> 4);
+                    if(m < p.M && n0 < p.N)
+                    {
+                        if constexpr(DT == DT_I8)
+                        {
+                            int8_t* crow = reinterpret_cast<int8_t*>(p.c) + (size_t)m * p.ldc;
+                            const i32x4 v[4] = {acc[i][g * 4], acc[i][g * 4 + 1], acc[i][g * 4 + 2],
+                                                acc[i][g * 4 + 3]};
+                            if(p.epi == EPI_REQUANT_RND)
+                                store_row16_i8<EPI_REQUANT_RND>(crow, n0, p.N, vec_ok, v, p.scale_gemm, p.scale_relu, nt);
+                            else if(p.epi == EPI_REQUANT_CK)
+                                store_row16_i8<EPI_REQUANT_CK>(crow, n0, p.N, vec_ok, v, p.scale_gemm, p.scale_relu, nt);
+                            else
+                                store_row16_i8<EPI_PASSTHROUGH>(crow, n0, p.N, vec_ok, v, p.scale_gemm, p.scale_relu, nt);
+                        }
+                        else
+                        {
+                            _Float16* crow   = reinterpret_cast<_Float16*>(p.c) + (size_t)m * p.ldc;
+                            const f32x4 v[4] = {acc[i][g * 4], acc[i][g * 4 + 1], acc[i][g * 4 + 2],
+                                                acc[i][g * 4 + 3]};
+                            store_row16_f16(crow, n0, p.N, vec_ok, v, nt);
+                        }
+                    }
+#pragma unroll
+                    for(int t = 0; t < 4; ++t)
+                        acc[i][g * 4 + t] = acc_t{0, 0, 0, 0};
+                }
+            }
+        };
+
         auto barrier = [&]() {
             __builtin_amdgcn_s_barrier();
             asm volatile("" ::: "memory");
         };
 
-        if constexpr(PINGPONG)
+        // Register double buffer over the two k-steps of a K tile. The barrier sits between
+        // them: by then every wave has pulled ALL of the current K tile into registers, so its
+        // stage can be refilled right away, and the first fragments of the next K tile (of this
+        // or of the next C tile) are read while the second half is still being multiplied.
+        i32x4 af0[MT], bf0[NG * 4], af1[MT], bf1[NG * 4];
+
+        issue_next(0);
+        issue_next(1);
+        asm volatile("s_waitcnt vmcnt(%0)" ::"n"(LPT) : "memory");
+        barrier();
+        read_frags(smem, smem + A_TILE, 0, af0, bf0);
+
+        int kt = 0;
+        int it = 0;
+        for(int tile = (int)blockIdx.x; tile < ntiles;)
         {
-            // Eight waves = two groups of four, one wave of each group per SIMD. The groups run
-            // the same two-segment loop (MEM: pull a whole K tile from LDS into registers;
-            // COMP: 2 x MT x NG*4 MFMAs straight from registers) half an iteration apart, so
-            // that on every SIMD one wave is always inside its MFMA burst while its partner
-            // does LDS reads, global->LDS load issue and waiting. Barrier B(2k) is the point at
-            // which tile k has landed for everybody and nobody reads tile k-1 any more; both
-            // groups issue the loads of tile k+1 right after it.
-            static_assert(NW == 8, "ping-pong needs two waves per SIMD");
-            const int group = CKX_PP_GROUP(wave);
-            issue_loads(0);
-            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-            barrier(); // B0
-            if(group == 0)
-            {
-                for(int kt = 0; kt < nk; ++kt)
-                {
-                    const uint8_t* sa = smem + (kt & 1) * STAGE;
-                    issue_loads(kt + 1);
-                    read_frags(sa, sa + A_TILE, 0, af0, bf0);
-                    read_frags(sa, sa + A_TILE, 1, af1, bf1);
-                    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-                    barrier(); // B(2kt+1)
-                    __builtin_amdgcn_s_setprio(1);
-                    mfma_block(af0, bf0);
-                    mfma_block(af1, bf1);
-                    __builtin_amdgcn_s_setprio(0);
-                    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-                    barrier(); // B(2kt+2)
-                }
-                barrier(); // pairs with the other group's last one
-            }
-            else
-            {
-                issue_loads(1);
-                barrier(); // B1
-                for(int kt = 0; kt < nk; ++kt)
-                {
-                    const uint8_t* sa = smem + (kt & 1) * STAGE;
-                    read_frags(sa, sa + A_TILE, 0, af0, bf0);
-                    read_frags(sa, sa + A_TILE, 1, af1, bf1);
-                    asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
-                    barrier(); // B(2kt+2)
-                    issue_loads(kt + 2);
-                    __builtin_amdgcn_s_setprio(1);
-                    mfma_block(af0, bf0);
-                    mfma_block(af1, bf1);
-                    __builtin_amdgcn_s_setprio(0);
-                    barrier(); // B(2kt+3)
-                }
-            }
-        }
-        else
-        {
-            // Register double buffer over the two k-steps of a K tile. The barrier sits between
-            // them: by then every wave has pulled ALL of tile kt into registers, so the stage of
-            // tile kt can be refilled right away, and the first fragments of tile kt+1 are read
-            // while the second half of tile kt is still being multiplied.
-            issue_loads(0);
-            issue_loads(1);
-            asm volatile("s_waitcnt vmcnt(%0)" ::"n"(LPT) : "memory");
+            const uint8_t* sa  = smem + (it & 1) * STAGE;
+            const uint8_t* sb  = sa + A_TILE;
+            const uint8_t* san = smem + ((it + 1) & 1) * STAGE;
+            const uint8_t* sbn = san + A_TILE;
+
+            read_frags(sa, sb, 1, af1, bf1);
+            mfma_block(af0, bf0);
+            interleave();
+
+            // the next K tile has landed (its loads are the only ones in flight, C stores of an
+            // earlier epilogue aside) and the current one is entirely in registers
+            asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
             barrier();
-            read_frags(smem, smem + A_TILE, 0, af0, bf0);
+            issue_next(it & 1);
 
-            for(int kt = 0; kt < nk; ++kt)
+            read_frags(san, sbn, 0, af0, bf0);
+            mfma_block(af1, bf1);
+            interleave();
+
+            ++it;
+            if(++kt == nk)
             {
-                const uint8_t* sa  = smem + (kt & 1) * STAGE;
-                const uint8_t* sb  = sa + A_TILE;
-                const uint8_t* san = smem + ((kt + 1) & 1) * STAGE;
-                const uint8_t* sbn = san + A_TILE;
-
-                read_frags(sa, sb, 1, af1, bf1);
-                mfma_block(af0, bf0);
-                interleave();
-
-                // tile kt+1 has landed (its loads are the only ones in flight) and tile kt is
-                // entirely in registers
-                asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
-                barrier();
-                issue_loads(kt + 2);
-
-                read_frags(san, sbn, 0, af0, bf0);
-                mfma_block(af1, bf1);
-                interleave();
+                epilogue(tile);
+                kt = 0;
+                tile += gstride;
             }
         }
         // the trailing (all-zero) loads still target LDS: let them retire before the workgroup
         // gives its LDS back
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-
-        // ---- epilogue: registers -> global, 16 consecutive columns per lane -------------
-        const bool vec_ok = ((reinterpret_cast<uintptr_t>(p.c) | ((uintptr_t)p.ldc * ES)) & 15u) == 0;
-#pragma unroll
-        for(int i = 0; i < MT; ++i)
-        {
-            const int m = tm * BM + wm * WTM + 16 * i + (lane & 15);
-            if(m >= p.M)
-                continue;
-#pragma unroll
-            for(int g = 0; g < NG; ++g)
-            {
-                const int n0 = tn * BN + wn * WTN + 64 * g + 16 * (lane >> 4);
-                if(n0 >= p.N)
-                    continue;
-                if constexpr(DT == DT_I8)
-                {
-                    int8_t* crow = reinterpret_cast<int8_t*>(p.c) + (size_t)m * p.ldc;
-                    const i32x4 v[4] = {acc[i][g * 4], acc[i][g * 4 + 1], acc[i][g * 4 + 2], acc[i][g * 4 + 3]};
-                    if(p.epi == EPI_REQUANT_RND)
-                        store_row16_i8<EPI_REQUANT_RND>(crow, n0, p.N, vec_ok, v, p.scale_gemm, p.scale_relu);
-                    else if(p.epi == EPI_REQUANT_CK)
-                        store_row16_i8<EPI_REQUANT_CK>(crow, n0, p.N, vec_ok, v, p.scale_gemm, p.scale_relu);
-                    else
-                        store_row16_i8<EPI_PASSTHROUGH>(crow, n0, p.N, vec_ok, v, p.scale_gemm, p.scale_relu);
-                }
-                else
-                {
-                    _Float16* crow   = reinterpret_cast<_Float16*>(p.c) + (size_t)m * p.ldc;
-                    const f32x4 v[4] = {acc[i][g * 4], acc[i][g * 4 + 1], acc[i][g * 4 + 2], acc[i][g * 4 + 3]};
-                    store_row16_f16(crow, n0, p.N, vec_ok, v);
-                }
-            }
-        }
     }
 };
 
-template <int DT, int BM, int BN, int WM, int WN, int BKB, int NST, bool IM2COL, bool PINGPONG>
+template <int DT, int BM, int BN, int WM, int WN, int BKB, int NST, bool IM2COL>
 __global__ __launch_bounds__(WM* WN * 64) void gemm_tile_kernel(const GemmArgs p)
 {
     extern __shared__ __attribute__((aligned(1024))) uint8_t ckx_smem[];
-    GemmTile<DT, BM, BN, WM, WN, BKB, NST, IM2COL, PINGPONG>::run(p, ckx_smem);
+    GemmTile<DT, BM, BN, WM, WN, BKB, NST, IM2COL>::run(p, ckx_smem);
 }
 
 } // namespace ckx

@@ -39,7 +39,7 @@ def _f16_close(out, ref):
 
 
 @pytest.mark.parametrize("case", SMALL)
-@pytest.mark.parametrize("instance", [capi.INSTANCE_AUTO, 0, 2, 4, 6])
+@pytest.mark.parametrize("instance", [capi.INSTANCE_AUTO, 0, 2, 4, 6, 7])
 def test_conv2d_int8_small_cases_bit_exact(case, instance):
     import gpu_util
     N, C, K, Hi, Wi, Y, X, s, d, p = case
