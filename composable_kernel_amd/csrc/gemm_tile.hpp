@@ -247,6 +247,24 @@ __device__ __forceinline__ void store_row16_f16(_Float16* crow, int n0, int N, b
     }
 }
 
+// Scheduling recipe for one half-iteration that also issues NL direct loads: NL groups of
+// {1 VMEM read, its share of the NR LDS reads, its share of the NM MFMAs}.
+template <int L, int NL, int NR, int NM>
+__device__ __forceinline__ void sched_loads_reads_mfma()
+{
+    if constexpr(L < NL)
+    {
+        constexpr int nr  = NR / NL + (L < NR % NL ? 1 : 0);
+        constexpr int per = NM / NL + (L < NM % NL ? 1 : 0);
+        __builtin_amdgcn_sched_group_barrier(0x010, 1, 0); // VMEM (the direct-to-LDS load counts as load+store)
+        if constexpr(nr > 0)
+            __builtin_amdgcn_sched_group_barrier(0x100, nr, 0); // DS read
+        if constexpr(per > 0)
+            __builtin_amdgcn_sched_group_barrier(0x008, per, 0); // MFMA
+        sched_loads_reads_mfma<L + 1, NL, NR, NM>();
+    }
+}
+
 // ------------------------------------------------------------------- kernel
 // BKB   bytes of every row staged per K tile (128)
 // NST   LDS stages (2)
@@ -363,64 +381,82 @@ struct GemmTile
             }
         };
 
-        // Direct global->LDS loads of K tile kt of the load cursor's tile into `stage`. Chunks past
-        // K (and whole tiles past the end of the work list) use an out-of-range offset: the
-        // hardware writes zeros, and the number of loads in flight stays constant.
-        auto issue_loads = [&](int kt, int stage) {
-            uint8_t* sa           = smem + stage * STAGE;
-            uint8_t* sb           = sa + A_TILE;
-            const uint32_t k0     = (uint32_t)kt * BKB; // byte offset of the K tile
-            const bool k_ok       = k0 + kb < kbytes; // false only in the K tail (or past the end)
-            // im2col: every load slot of a thread sits at the same chunk position (the swizzle only
-            // depends on lane/8), so the tap (y, x) and channel offset are decoded ONCE per thread
-            // and K tile; a slot then only range-checks its own window.
-            int tap_dh = 0, tap_dw = 0;
-            uint32_t tap_off = 0;
-            bool tap_ok      = true;
+        // Direct global->LDS loads of K tile kt of the load cursor's tile into `stage`, one slot at
+        // a time so that the caller can place them between MFMAs. Chunks past K (and whole tiles
+        // past the end of the work list) use an out-of-range offset: the hardware writes zeros,
+        // and the number of loads in flight stays constant.
+        struct LoadCtx
+        {
+            uint8_t* sa;
+            uint8_t* sb;
+            uint32_t k0;      // byte offset of the K tile
+            uint32_t k_oob;   // top bit set for chunks past K: OR-ed into the offset (arithmetic on
+                              // purpose: a select feeding the loads becomes divergent branches)
+            int tap_dh, tap_dw; // im2col: decoded ONCE per thread and K tile, every slot of a thread
+            uint32_t tap_off;   // sits at the same chunk position
+            bool tap_ok;
+        };
+        auto load_ctx = [&](int kt, int stage) {
+            LoadCtx c;
+            c.sa    = smem + stage * STAGE;
+            c.sb    = c.sa + A_TILE;
+            c.k0    = (uint32_t)kt * BKB;
+            c.k_oob = (c.k0 + kb < kbytes) ? 0u : kOutOfRange;
+            c.tap_dh = c.tap_dw = 0;
+            c.tap_off           = 0;
+            c.tap_ok            = true;
             if constexpr(IM2COL)
             {
-                const uint32_t ke  = (k0 + kb) / ES; // element index along GEMM-K
+                const uint32_t ke  = (c.k0 + kb) / ES; // element index along GEMM-K
                 const uint32_t y   = magic_div(ke, p.cv.div_xc);
                 const uint32_t rem = ke - y * p.cv.div_xc.d;
                 const uint32_t x   = magic_div(rem, p.cv.div_c);
                 const uint32_t cc  = rem - x * p.cv.div_c.d;
-                tap_dh             = (int)y * p.cv.dH;
-                tap_dw             = (int)x * p.cv.dW;
-                tap_off            = ((uint32_t)(tap_dh * p.cv.Wi + tap_dw) * (uint32_t)p.cv.C + cc) * ES;
-                tap_ok             = ke < (uint32_t)p.K;
+                c.tap_dh           = (int)y * p.cv.dH;
+                c.tap_dw           = (int)x * p.cv.dW;
+                c.tap_off          = ((uint32_t)(c.tap_dh * p.cv.Wi + c.tap_dw) * (uint32_t)p.cv.C + cc) * ES;
+                c.tap_ok           = ke < (uint32_t)p.K;
             }
-#pragma unroll
-            for(int j = 0; j < NLA; ++j)
+            return c;
+        };
+        auto issue_slot = [&](const LoadCtx& c, int slot) { // slot < NLA: A rows, else B rows
+            if(slot < NLA)
             {
+                const int j = slot;
                 uint32_t voff;
                 if constexpr(!IM2COL)
-                {
-                    voff = k_ok ? a_off[j] + k0 : kOutOfRange;
-                }
+                    voff = (a_off[j] + c.k0) | c.k_oob;
                 else
                 {
                     const int hi0 = (int)a_hw0[j] >> 16, wi0 = (int)(a_hw0[j] << 16) >> 16;
-                    const bool ok = tap_ok && (uint32_t)(hi0 + tap_dh) < (uint32_t)p.cv.Hi &&
-                                    (uint32_t)(wi0 + tap_dw) < (uint32_t)p.cv.Wi;
-                    voff = ok ? a_off[j] + tap_off : kOutOfRange;
+                    const bool ok = c.tap_ok && (uint32_t)(hi0 + c.tap_dh) < (uint32_t)p.cv.Hi &&
+                                    (uint32_t)(wi0 + c.tap_dw) < (uint32_t)p.cv.Wi;
+                    voff = (a_off[j] + c.tap_off) | (ok ? 0u : kOutOfRange);
                 }
-                __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_a, (lds_ptr_t)(sa + (j * NW + wave) * 1024), 16,
+                __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_a, (lds_ptr_t)(c.sa + (j * NW + wave) * 1024), 16,
                                                          voff, 0, 0, 0);
             }
-#pragma unroll
-            for(int j = 0; j < NLB; ++j)
+            else
             {
-                const uint32_t voff = k_ok ? b_off[j] + k0 : kOutOfRange;
-                __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_b, (lds_ptr_t)(sb + (j * NW + wave) * 1024), 16,
+                const int j         = slot - NLA;
+                const uint32_t voff = (b_off[j] + c.k0) | c.k_oob;
+                __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_b, (lds_ptr_t)(c.sb + (j * NW + wave) * 1024), 16,
                                                          voff, 0, 0, 0);
             }
+        };
+        auto issue_loads = [&](int kt, int stage) {
+            const LoadCtx c = load_ctx(kt, stage);
+#pragma unroll
+            for(int sl = 0; sl < LPT; ++sl)
+                issue_slot(c, sl);
         };
 
         // load cursor: (tile, kt) of the next K tile to request
         int ld_tile = (int)blockIdx.x, ld_kt = 0;
         setup_tile(ld_tile);
-        auto issue_next = [&](int stage) {
-            issue_loads(ld_kt, stage);
+        // (kept apart from the issue itself: the branch would split the basic block in which the
+        // loads are interleaved with MFMAs)
+        auto advance_load_cursor = [&]() {
             if(++ld_kt == nk)
             {
                 ld_kt = 0;
@@ -441,44 +477,54 @@ struct GemmTile
         const uint32_t frow = (uint32_t)(lane & 15);
         const uint32_t fq   = (uint32_t)(lane >> 4);
 
+        auto read_one = [&](const uint8_t* sa, const uint8_t* sb, int ks, int r, i32x4(&af)[MT], i32x4(&bf)[NG * 4]) {
+            if(r < MT)
+            {
+                const uint32_t row = (uint32_t)(wm * WTM + 16 * r) + frow;
+                af[r] = *reinterpret_cast<const i32x4*>(sa + chunk_offset(row, ks * 4 + fq));
+            }
+            else
+            {
+                const uint32_t row = (uint32_t)(wn * WTN + 16 * (r - MT)) + frow;
+                bf[r - MT] = *reinterpret_cast<const i32x4*>(sb + chunk_offset(row, ks * 4 + fq));
+            }
+        };
         auto read_frags = [&](const uint8_t* sa, const uint8_t* sb, int ks, i32x4(&af)[MT], i32x4(&bf)[NG * 4]) {
 #pragma unroll
-            for(int i = 0; i < MT; ++i)
-            {
-                const uint32_t row = (uint32_t)(wm * WTM + 16 * i) + frow;
-                af[i] = *reinterpret_cast<const i32x4*>(sa + chunk_offset(row, ks * 4 + fq));
-            }
-#pragma unroll
-            for(int t = 0; t < NG * 4; ++t)
-            {
-                const uint32_t row = (uint32_t)(wn * WTN + 16 * t) + frow;
-                bf[t] = *reinterpret_cast<const i32x4*>(sb + chunk_offset(row, ks * 4 + fq));
-            }
+            for(int r = 0; r < MT + NG * 4; ++r)
+                read_one(sa, sb, ks, r, af, bf);
         };
-        auto mfma_block = [&](const i32x4(&af)[MT], const i32x4(&bf)[NG * 4]) {
-#pragma unroll
-            for(int i = 0; i < MT; ++i)
-#pragma unroll
-                for(int t = 0; t < NG * 4; ++t)
-                {
-                    if constexpr(DT == DT_I8)
-                        acc[i][t] = __builtin_amdgcn_mfma_i32_16x16x64_i8(bf[t], af[i], acc[i][t], 0, 0, 0);
-                    else
-                        acc[i][t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(
-                            __builtin_bit_cast(f16x8, bf[t]), __builtin_bit_cast(f16x8, af[i]), acc[i][t], 0, 0, 0);
-                }
+        auto mfma_one = [&](int m, const i32x4(&af)[MT], const i32x4(&bf)[NG * 4]) {
+            const int i = m / (NG * 4), t = m % (NG * 4);
+            if constexpr(DT == DT_I8)
+                acc[i][t] = __builtin_amdgcn_mfma_i32_16x16x64_i8(bf[t], af[i], acc[i][t], 0, 0, 0);
+            else
+                acc[i][t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, bf[t]),
+                                                                __builtin_bit_cast(f16x8, af[i]), acc[i][t], 0, 0, 0);
         };
-        // Tell the scheduler to keep the order written below: the LDS reads of the NEXT k-step
-        // are spread between the MFMAs of the CURRENT one (1 read : 2 MFMA, then the rest).
-        auto interleave = [&]() {
-            constexpr int NR = MT + NG * 4, NM = MT * NG * 4;
+
+        // One half of a K-tile iteration, written as LPT groups pinned in source order
+        // (sched_barrier): group g = [one direct global->LDS load of the K tile after next]
+        // + [its share of the LDS reads of the NEXT k-step] + [its share of the MFMAs of the CURRENT
+        // k-step]. The loads must not be issued back to back: a burst of eight 1 KB loads per wave
+        // fills the texture-address FIFOs (SQ_VMEM_TA_ADDR/CMD_FIFO_FULL), the in-order wave blocks
+        // on VMEM issue, and its MFMAs wait behind it.
+        auto half_step = [&](auto with_loads, const LoadCtx& lc, const i32x4(&caf)[MT], const i32x4(&cbf)[NG * 4],
+                             const uint8_t* nsa, const uint8_t* nsb, int nks, i32x4(&naf)[MT], i32x4(&nbf)[NG * 4]) {
+            constexpr int NGRP = LPT, NR = MT + NG * 4, NM = MT * NG * 4;
 #pragma unroll
-            for(int r = 0; r < NR; ++r)
+            for(int g = 0; g < NGRP; ++g)
             {
-                __builtin_amdgcn_sched_group_barrier(0x100, 1, 0); // DS read
-                __builtin_amdgcn_sched_group_barrier(0x008, (NM / NR) > 0 ? (NM / NR) : 1, 0); // MFMA
+                if constexpr(decltype(with_loads)::value)
+                    issue_slot(lc, g);
+#pragma unroll
+                for(int r = g * NR / NGRP; r < (g + 1) * NR / NGRP; ++r)
+                    read_one(nsa, nsb, nks, r, naf, nbf);
+#pragma unroll
+                for(int m = g * NM / NGRP; m < (g + 1) * NM / NGRP; ++m)
+                    mfma_one(m, caf, cbf);
+                __builtin_amdgcn_sched_barrier(0);
             }
-            __builtin_amdgcn_sched_group_barrier(0x008, NM - NR * (NM / NR), 0);
         };
 
         // ---- epilogue: registers -> global, 16 consecutive columns per lane -------------
@@ -535,8 +581,10 @@ struct GemmTile
         // or of the next C tile) are read while the second half is still being multiplied.
         i32x4 af0[MT], bf0[NG * 4], af1[MT], bf1[NG * 4];
 
-        issue_next(0);
-        issue_next(1);
+        issue_loads(ld_kt, 0);
+        advance_load_cursor();
+        issue_loads(ld_kt, 1);
+        advance_load_cursor();
         asm volatile("s_waitcnt vmcnt(%0)" ::"n"(LPT) : "memory");
         barrier();
         read_frags(smem, smem + A_TILE, 0, af0, bf0);
@@ -550,19 +598,16 @@ struct GemmTile
             const uint8_t* san = smem + ((it + 1) & 1) * STAGE;
             const uint8_t* sbn = san + A_TILE;
 
-            read_frags(sa, sb, 1, af1, bf1);
-            mfma_block(af0, bf0);
-            interleave();
+            half_step(std::false_type{}, LoadCtx{}, af0, bf0, sa, sb, 1, af1, bf1);
 
             // the next K tile has landed (its loads are the only ones in flight, C stores of an
             // earlier epilogue aside) and the current one is entirely in registers
             asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
             barrier();
-            issue_next(it & 1);
 
-            read_frags(san, sbn, 0, af0, bf0);
-            mfma_block(af1, bf1);
-            interleave();
+            const LoadCtx lc = load_ctx(ld_kt, it & 1);
+            half_step(std::true_type{}, lc, af1, bf1, san, sbn, 0, af0, bf0);
+            advance_load_cursor();
 
             ++it;
             if(++kt == nk)
