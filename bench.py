@@ -117,6 +117,11 @@ def make_launcher(w, instance=-1):
     keep.append(c)
     if not op.IsSupportedArgument(arg):
         raise RuntimeError(f"{w['name']}: not supported: {capi.last_error()}")
+    need = op.GetWorkSpaceSize(arg)
+    if need:   # optional split-K scratch, allocated once outside the timed region
+        ws = torch.empty(need, dtype=torch.uint8, device="cuda")
+        keep.append(ws)
+        op.SetWorkSpacePointer(arg, ws)
 
     def launch():
         st_ = op._launch(arg, torch.cuda.current_stream().cuda_stream)

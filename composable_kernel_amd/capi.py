@@ -20,8 +20,9 @@ INSTANCE_AUTO = -1
 # every symbol include/ckx.h declares
 SYMBOLS = [
     "ckx_version", "ckx_last_error", "ckx_num_instances", "ckx_instance_name",
-    "ckx_gemm_i8_is_supported", "ckx_gemm_i8", "ckx_gemm_f16_is_supported", "ckx_gemm_f16",
-    "ckx_conv2d_fwd_is_supported", "ckx_conv2d_fwd_i8", "ckx_conv2d_fwd_f16",
+    "ckx_gemm_i8_is_supported", "ckx_gemm_i8", "ckx_gemm_i8_workspace_bytes",
+    "ckx_gemm_f16_is_supported", "ckx_gemm_f16", "ckx_gemm_f16_workspace_bytes",
+    "ckx_conv2d_fwd_is_supported", "ckx_conv2d_fwd_i8", "ckx_conv2d_fwd_f16", "ckx_conv2d_fwd_workspace_bytes",
     "ckx_batched_gemm_gemm_f16_is_supported", "ckx_batched_gemm_gemm_f16", "ckx_time_launches",
 ]
 
@@ -66,13 +67,18 @@ def lib():
     L.ckx_instance_name.argtypes = [C.c_int, C.c_int]
     shape = [i32] * 6 + [C.c_int] * 3
     L.ckx_gemm_i8_is_supported.argtypes = shape + [C.c_int, C.c_int]
-    L.ckx_gemm_i8.argtypes = [vp, vp, vp] + shape + [C.c_int, f32, f32, C.c_int, vp]
+    L.ckx_gemm_i8.argtypes = [vp, vp, vp] + shape + [C.c_int, f32, f32, C.c_int, vp, i64, vp]
+    for fn in (L.ckx_gemm_i8_workspace_bytes, L.ckx_gemm_f16_workspace_bytes):
+        fn.restype = i64
+        fn.argtypes = [i32, i32, i32, C.c_int]
     L.ckx_gemm_f16_is_supported.argtypes = shape + [C.c_int]
-    L.ckx_gemm_f16.argtypes = [vp, vp, vp] + shape + [C.c_int, vp]
+    L.ckx_gemm_f16.argtypes = [vp, vp, vp] + shape + [C.c_int, vp, i64, vp]
     dp = C.POINTER(Conv2dDesc)
     L.ckx_conv2d_fwd_is_supported.argtypes = [C.c_int, dp, C.c_int, C.c_int]
-    L.ckx_conv2d_fwd_i8.argtypes = [vp, vp, vp, dp, C.c_int, f32, f32, C.c_int, vp]
-    L.ckx_conv2d_fwd_f16.argtypes = [vp, vp, vp, dp, C.c_int, vp]
+    L.ckx_conv2d_fwd_i8.argtypes = [vp, vp, vp, dp, C.c_int, f32, f32, C.c_int, vp, i64, vp]
+    L.ckx_conv2d_fwd_f16.argtypes = [vp, vp, vp, dp, C.c_int, vp, i64, vp]
+    L.ckx_conv2d_fwd_workspace_bytes.restype = i64
+    L.ckx_conv2d_fwd_workspace_bytes.argtypes = [C.c_int, dp, C.c_int]
     gg = [i32] * 9 + [i64] * 4 + [C.c_int]
     L.ckx_batched_gemm_gemm_f16_is_supported.argtypes = gg
     L.ckx_batched_gemm_gemm_f16.argtypes = [vp] * 4 + gg + [vp]

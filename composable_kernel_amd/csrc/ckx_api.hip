@@ -97,6 +97,14 @@ hipError_t launch_tile(const ckx::GemmArgs& a, int tiles, hipStream_t s)
     return hipGetLastError();
 }
 
+template <int DT>
+hipError_t launch_reduce(const ckx::GemmArgs& a, hipStream_t s)
+{
+    const long groups = (long)a.M * ((a.N + 15) / 16);
+    hipLaunchKernelGGL((ckx::splitk_reduce_kernel<DT>), dim3((unsigned)((groups + 255) / 256)), dim3(256), 0, s, a);
+    return hipGetLastError();
+}
+
 struct TileInstance
 {
     const char* name;
@@ -126,28 +134,71 @@ const TileInstance kTiles[] = {
 };
 constexpr int kNumTiles = sizeof(kTiles) / sizeof(kTiles[0]);
 
-// Instance choice by a small cost model (microseconds on a 256-CU part): workgroups run in
-// rounds of 256 * (workgroups that fit a CU's 160 KB LDS and 2048 threads); a round costs the
-// tile's share of MFMA time, scaled by how well that tile shape feeds the MFMA pipe, plus a
-// fixed prologue/epilogue term that co-resident workgroups overlap.
-int pick_tile(int M, int N, int kbytes)
+// Launch plan: which tile instance, and into how many K runs each C tile is cut (split-K).
+struct Plan
 {
-    int best       = 0;
-    double best_us = 1e30;
-    const double ktiles = (kbytes + 127) / 128;
+    int tile   = 0;
+    int ksplit = 1;
+    int nk_per = 0;
+};
+
+int force_ksplit()
+{
+    // CKX_KSPLIT=n forces n K runs where the problem allows it (tuning / test knob); read per call
+    const char* e = std::getenv("CKX_KSPLIT");
+    return e ? std::atoi(e) : 0;
+}
+
+// Choice by a small cost model (microseconds on a 256-CU part): work units (C tile x K run) are
+// processed in rounds of 256 * (workgroups that fit a CU's 160 KB LDS and 2048 threads); a round
+// costs the unit's share of MFMA time, scaled by how well that tile shape feeds the MFMA pipe,
+// plus a fixed prologue/epilogue term that co-resident workgroups overlap. Split-K adds the
+// second pass (launch + slice traffic) and is only considered when a workspace is available.
+Plan make_plan(int M, int N, int kbytes, int only_tile, long workspace_bytes)
+{
+    Plan best;
+    double best_us  = 1e30;
+    const int nk    = (kbytes + 127) / 128 > 0 ? (kbytes + 127) / 128 : 1;
+    const int force = force_ksplit();
     for(int i = 0; i < kNumTiles; ++i)
     {
+        if(only_tile >= 0 && i != only_tile)
+            continue;
         const TileInstance& t = kTiles[i];
         const long tiles      = (long)((M + t.bm - 1) / t.bm) * ((N + t.bn - 1) / t.bn);
-        int per_cu            = 160 * 1024 / t.lds;
-        per_cu                = per_cu > 2048 / t.threads ? 2048 / t.threads : per_cu;
-        per_cu                = per_cu > 4 ? 4 : per_cu;
-        per_cu                = (long)per_cu * 256 > tiles ? (int)((tiles + 255) / 256) : per_cu;
-        const long rounds     = (tiles + 256l * per_cu - 1) / (256l * per_cu);
-        const double us = rounds * (per_cu * (t.bm * t.bn / 65536.0) / t.eff * ktiles * 1.1 + 6.0 / per_cu + 2.0);
-        if(us < best_us)
-            best_us = us, best = i;
+        for(int sp = 1; sp <= 8; ++sp)
+        {
+            const int nk_per = (nk + sp - 1) / sp;
+            if(sp > 1 && ((long)nk_per * (sp - 1) >= nk || (long)sp * M * N * 4 > workspace_bytes))
+                continue;
+            if(force > 0 && sp != force && !(sp == 1 && ((long)((nk + force - 1) / force) * (force - 1) >= nk ||
+                                                          (long)force * M * N * 4 > workspace_bytes)))
+                continue;
+            const long units = tiles * sp;
+            int per_cu       = 160 * 1024 / t.lds;
+            per_cu           = per_cu > 2048 / t.threads ? 2048 / t.threads : per_cu;
+            per_cu           = per_cu > 4 ? 4 : per_cu;
+            per_cu           = (long)per_cu * 256 > units ? (int)((units + 255) / 256) : per_cu;
+            const long rounds = (units + 256l * per_cu - 1) / (256l * per_cu);
+            // one K-tile iteration costs its MFMA time, but never less than the barrier + load
+            // latency of the two-stage pipeline (~0.42 us measured on small tiles)
+            double iter_us = per_cu * (t.bm * t.bn / 65536.0) / t.eff * 1.1;
+            iter_us        = iter_us < 0.42 ? 0.42 : iter_us;
+            double us      = rounds * (iter_us * nk_per + 6.0 / per_cu + 2.0);
+            if(sp > 1)
+            {
+                // second launch + slice write/read (measured ~2 TB/s effective), and a split has to
+                // promise a clear win: the single-pass estimate is the better calibrated one
+                us += 3.0 + (sp + 0.25) * M * (double)N * 4 / 2.0e6;
+                if(force <= 0)
+                    us *= 1.25;
+            }
+            if(us < best_us)
+                best_us = us, best.tile = i, best.ksplit = sp, best.nk_per = nk_per;
+        }
     }
+    if(best.nk_per == 0)
+        best.nk_per = nk;
     return best;
 }
 
@@ -219,8 +270,19 @@ int check_gemm_shape(int dt, int M, int N, int K, int sa, int sb, int sc, int al
     return CKX_OK;
 }
 
+// workspace need of the launch plan for this GEMM (0: none)
+long gemm_workspace_bytes(int dt, int M, int N, int K, int instance)
+{
+    const int es = dt == ckx::DT_I8 ? 1 : 2;
+    if(M <= 0 || N <= 0 || (instance == CKX_INSTANCE_AUTO && M <= 64) || instance >= kNumTiles)
+        return 0;
+    const Plan pl = make_plan(M, N, K * es, instance, 1l << 60);
+    return pl.ksplit > 1 ? (long)pl.ksplit * M * N * 4 : 0;
+}
+
 int run_gemm(int dt, const void* a, const void* b, void* c, int M, int N, int K, int sa, int sb, int sc,
-             int al, int bl, int cl, int epi, float sg, float sr, int instance, void* stream)
+             int al, int bl, int cl, int epi, float sg, float sr, int instance, void* ws, long ws_bytes,
+             void* stream)
 {
     int st = check_gemm_shape(dt, M, N, K, sa, sb, sc, al, bl, cl, epi, instance);
     if(st != CKX_OK)
@@ -233,10 +295,18 @@ int run_gemm(int dt, const void* a, const void* b, void* c, int M, int N, int K,
         return fail(CKX_UNSUPPORTED, "A and B must be 16-byte aligned");
     const int es = dt == ckx::DT_I8 ? 1 : 2;
     int ti = instance;
-    if(instance == CKX_INSTANCE_AUTO)
+    Plan pl;
+    if(instance == CKX_INSTANCE_AUTO && M <= 64)
     {
         // a handful of rows against a big weight matrix is an HBM-streaming problem
-        ti = M <= 16 ? kNumTiles + 0 : M <= 32 ? kNumTiles + 1 : M <= 64 ? kNumTiles + 2 : pick_tile(M, N, K * es);
+        ti = M <= 16 ? kNumTiles + 0 : M <= 32 ? kNumTiles + 1 : kNumTiles + 2;
+    }
+    else if(instance < kNumTiles)
+    {
+        if(ws && (reinterpret_cast<uintptr_t>(ws) & 15))
+            return fail(CKX_INVALID_VALUE, "workspace must be 16-byte aligned");
+        pl = make_plan(M, N, K * es, instance, ws ? ws_bytes : 0);
+        ti = pl.tile;
     }
     ckx::GemmArgs g;
     std::memset(&g, 0, sizeof(g));
@@ -249,6 +319,7 @@ int run_gemm(int dt, const void* a, const void* b, void* c, int M, int N, int K,
     g.scale_gemm = sg;
     g.scale_relu = sr;
     g.nt_store   = es == 1 && (long)M * N * es >= stream_output_bytes();
+    g.ksplit     = 1;
     if(ti >= kNumTiles)
     {
         const SkinnyInstance& k = kSkinny[ti - kNumTiles];
@@ -258,7 +329,14 @@ int run_gemm(int dt, const void* a, const void* b, void* c, int M, int N, int K,
     const TileInstance& t = kTiles[ti];
     g.tiles_m    = (M + t.bm - 1) / t.bm;
     g.tiles_n    = (N + t.bn - 1) / t.bn;
-    hipError_t e = (dt == ckx::DT_I8 ? t.dense_i8 : t.dense_f16)(g, g.tiles_m * g.tiles_n, (hipStream_t)stream);
+    g.ksplit     = pl.ksplit;
+    g.nk_per     = pl.nk_per;
+    g.ws         = ws;
+    hipError_t e =
+        (dt == ckx::DT_I8 ? t.dense_i8 : t.dense_f16)(g, g.tiles_m * g.tiles_n * g.ksplit, (hipStream_t)stream);
+    if(e == hipSuccess && g.ksplit > 1)
+        e = dt == ckx::DT_I8 ? launch_reduce<ckx::DT_I8>(g, (hipStream_t)stream)
+                             : launch_reduce<ckx::DT_F16>(g, (hipStream_t)stream);
     if(e != hipSuccess)
         return hip_fail(e, t.name);
     return CKX_OK;
@@ -301,8 +379,18 @@ int check_conv(int op, const ckx_conv2d_desc* d, int epi, int instance)
     return CKX_OK;
 }
 
+long conv_workspace_bytes(int op, const ckx_conv2d_desc* d, int instance)
+{
+    const int es = op == CKX_OP_CONV2D_FWD_I8 ? 1 : 2;
+    const long M = (long)d->N * d->Ho * d->Wo;
+    if(M <= 0 || d->K <= 0)
+        return 0;
+    const Plan pl = make_plan((int)M, d->K, d->Y * d->X * d->C * es, instance, 1l << 60);
+    return pl.ksplit > 1 ? (long)pl.ksplit * M * d->K * 4 : 0;
+}
+
 int run_conv(int op, const void* in, const void* wei, void* out, const ckx_conv2d_desc* d, int epi, float sg,
-             float sr, int instance, void* stream)
+             float sr, int instance, void* ws, long ws_bytes, void* stream)
 {
     int st = check_conv(op, d, epi, instance);
     if(st != CKX_OK)
@@ -315,8 +403,10 @@ int run_conv(int op, const void* in, const void* wei, void* out, const ckx_conv2
         return fail(CKX_INVALID_VALUE, "null operand pointer");
     if((reinterpret_cast<uintptr_t>(in) | reinterpret_cast<uintptr_t>(wei)) & 15)
         return fail(CKX_UNSUPPORTED, "input and weight must be 16-byte aligned");
-    const int ti = instance == CKX_INSTANCE_AUTO ? pick_tile(M, N, K * es) : instance;
-    const TileInstance& t = kTiles[ti];
+    if(ws && (reinterpret_cast<uintptr_t>(ws) & 15))
+        return fail(CKX_INVALID_VALUE, "workspace must be 16-byte aligned");
+    const Plan pl = make_plan(M, N, K * es, instance, ws ? ws_bytes : 0);
+    const TileInstance& t = kTiles[pl.tile];
     ckx::GemmArgs g;
     std::memset(&g, 0, sizeof(g));
     g.a = in, g.b = wei, g.c = out;
@@ -337,7 +427,13 @@ int run_conv(int op, const void* in, const void* wei, void* out, const ckx_conv2
     g.cv.div_wo   = make_magic((uint32_t)d->Wo);
     g.cv.div_xc   = make_magic((uint32_t)(d->X * d->C));
     g.cv.div_c    = make_magic((uint32_t)d->C);
-    hipError_t e  = (es == 1 ? t.conv_i8 : t.conv_f16)(g, g.tiles_m * g.tiles_n, (hipStream_t)stream);
+    g.ksplit = pl.ksplit;
+    g.nk_per = pl.nk_per;
+    g.ws     = ws;
+    hipError_t e = (es == 1 ? t.conv_i8 : t.conv_f16)(g, g.tiles_m * g.tiles_n * g.ksplit, (hipStream_t)stream);
+    if(e == hipSuccess && g.ksplit > 1)
+        e = es == 1 ? launch_reduce<ckx::DT_I8>(g, (hipStream_t)stream)
+                    : launch_reduce<ckx::DT_F16>(g, (hipStream_t)stream);
     if(e != hipSuccess)
         return hip_fail(e, t.name);
     return CKX_OK;
@@ -381,12 +477,17 @@ int ckx_gemm_i8_is_supported(int32_t M, int32_t N, int32_t K, int32_t sa, int32_
     return check_gemm_shape(ckx::DT_I8, M, N, K, sa, sb, sc, al, bl, cl, epilogue, instance);
 }
 
+int64_t ckx_gemm_i8_workspace_bytes(int32_t M, int32_t N, int32_t K, int instance)
+{
+    return gemm_workspace_bytes(ckx::DT_I8, M, N, K, instance);
+}
+
 int ckx_gemm_i8(const void* a, const void* b, void* c, int32_t M, int32_t N, int32_t K, int32_t sa,
                 int32_t sb, int32_t sc, int al, int bl, int cl, int epilogue, float scale_gemm,
-                float scale_relu, int instance, void* stream)
+                float scale_relu, int instance, void* workspace, int64_t workspace_bytes, void* stream)
 {
     return run_gemm(ckx::DT_I8, a, b, c, M, N, K, sa, sb, sc, al, bl, cl, epilogue, scale_gemm, scale_relu,
-                    instance, stream);
+                    instance, workspace, workspace_bytes, stream);
 }
 
 int ckx_gemm_f16_is_supported(int32_t M, int32_t N, int32_t K, int32_t sa, int32_t sb, int32_t sc, int al,
@@ -395,11 +496,17 @@ int ckx_gemm_f16_is_supported(int32_t M, int32_t N, int32_t K, int32_t sa, int32
     return check_gemm_shape(ckx::DT_F16, M, N, K, sa, sb, sc, al, bl, cl, CKX_EPI_PASSTHROUGH, instance);
 }
 
+int64_t ckx_gemm_f16_workspace_bytes(int32_t M, int32_t N, int32_t K, int instance)
+{
+    return gemm_workspace_bytes(ckx::DT_F16, M, N, K, instance);
+}
+
 int ckx_gemm_f16(const void* a, const void* b, void* c, int32_t M, int32_t N, int32_t K, int32_t sa,
-                 int32_t sb, int32_t sc, int al, int bl, int cl, int instance, void* stream)
+                 int32_t sb, int32_t sc, int al, int bl, int cl, int instance, void* workspace,
+                 int64_t workspace_bytes, void* stream)
 {
     return run_gemm(ckx::DT_F16, a, b, c, M, N, K, sa, sb, sc, al, bl, cl, CKX_EPI_PASSTHROUGH, 1.0f, 1.0f,
-                    instance, stream);
+                    instance, workspace, workspace_bytes, stream);
 }
 
 int ckx_conv2d_fwd_is_supported(int op, const ckx_conv2d_desc* desc, int epilogue, int instance)
@@ -407,18 +514,26 @@ int ckx_conv2d_fwd_is_supported(int op, const ckx_conv2d_desc* desc, int epilogu
     return check_conv(op, desc, epilogue, instance);
 }
 
+int64_t ckx_conv2d_fwd_workspace_bytes(int op, const ckx_conv2d_desc* desc, int instance)
+{
+    if(check_conv(op, desc, CKX_EPI_PASSTHROUGH, instance) != CKX_OK)
+        return 0;
+    return conv_workspace_bytes(op, desc, instance);
+}
+
 int ckx_conv2d_fwd_i8(const void* in, const void* wei, void* out, const ckx_conv2d_desc* desc, int epilogue,
-                      float scale_gemm, float scale_relu, int instance, void* stream)
+                      float scale_gemm, float scale_relu, int instance, void* workspace, int64_t workspace_bytes,
+                      void* stream)
 {
     return run_conv(CKX_OP_CONV2D_FWD_I8, in, wei, out, desc, epilogue, scale_gemm, scale_relu, instance,
-                    stream);
+                    workspace, workspace_bytes, stream);
 }
 
 int ckx_conv2d_fwd_f16(const void* in, const void* wei, void* out, const ckx_conv2d_desc* desc, int instance,
-                       void* stream)
+                       void* workspace, int64_t workspace_bytes, void* stream)
 {
     return run_conv(CKX_OP_CONV2D_FWD_F16, in, wei, out, desc, CKX_EPI_PASSTHROUGH, 1.0f, 1.0f, instance,
-                    stream);
+                    workspace, workspace_bytes, stream);
 }
 
 int ckx_batched_gemm_gemm_f16_is_supported(int32_t M, int32_t N, int32_t K, int32_t O, int32_t batch,

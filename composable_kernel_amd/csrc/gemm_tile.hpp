@@ -106,6 +106,11 @@ struct GemmArgs
     int epi;
     float scale_gemm, scale_relu;
     int nt_store; // stream the C tile past L2 (large outputs)
+    // split-K: the K tiles of every C tile are cut into `ksplit` runs of `nk_per` K tiles; run s
+    // writes its raw accumulators to slice s of the workspace ([ksplit][M][N] int32 / fp32) and a
+    // second kernel sums the slices and applies the epilogue. ksplit == 1: no workspace.
+    int ksplit, nk_per;
+    void* ws;
     ConvGeom cv;
 };
 
@@ -305,7 +310,7 @@ struct GemmTile
         return row * BKB + ((chunk ^ swz(row)) << 4);
     }
 
-    __device__ static void run(const GemmArgs& p, uint8_t* smem)
+    __device__ static __forceinline__ void run(const GemmArgs& p, uint8_t* smem)
     {
         const int tid  = threadIdx.x;
         const int lane = tid & 63;
@@ -451,17 +456,25 @@ struct GemmTile
                 issue_slot(c, sl);
         };
 
-        // load cursor: (tile, kt) of the next K tile to request
-        int ld_tile = (int)blockIdx.x, ld_kt = 0;
-        setup_tile(ld_tile);
+        // A work unit is (K run s, C tile): unit = s * ntiles + tile, K tiles [s*nk_per, ...).
+        const int nunits = ntiles * p.ksplit;
+        auto unit_k_range = [&](int unit, int& k_begin, int& k_end) {
+            const int sp = unit / ntiles;
+            k_begin      = sp * p.nk_per;
+            k_end        = k_begin + p.nk_per < nk ? k_begin + p.nk_per : nk;
+        };
+        // load cursor: (unit, kt) of the next K tile to request
+        int ld_unit = (int)blockIdx.x, ld_kt = 0, ld_end = nk;
+        unit_k_range(ld_unit, ld_kt, ld_end);
+        setup_tile(ld_unit < nunits ? ld_unit % ntiles : ntiles);
         // (kept apart from the issue itself: the branch would split the basic block in which the
         // loads are interleaved with MFMAs)
         auto advance_load_cursor = [&]() {
-            if(++ld_kt == nk)
+            if(++ld_kt >= ld_end)
             {
-                ld_kt = 0;
-                ld_tile += gstride;
-                setup_tile(ld_tile);
+                ld_unit += gstride;
+                unit_k_range(ld_unit, ld_kt, ld_end);
+                setup_tile(ld_unit < nunits ? ld_unit % ntiles : ntiles);
             }
         };
 
@@ -530,9 +543,11 @@ struct GemmTile
         // ---- epilogue: registers -> global, 16 consecutive columns per lane -------------
         const bool vec_ok = ((reinterpret_cast<uintptr_t>(p.c) | ((uintptr_t)p.ldc * ES)) & 15u) == 0;
         const bool nt     = p.nt_store != 0;
-        auto epilogue = [&](int tile) {
+        auto epilogue = [&](int unit) {
             int tm, tn;
-            tile_of_block(tile, p.tiles_m, p.tiles_n, tm, tn);
+            tile_of_block(unit % ntiles, p.tiles_m, p.tiles_n, tm, tn);
+            acc_t* slice = reinterpret_cast<acc_t*>(reinterpret_cast<uint8_t*>(p.ws) +
+                                                    (size_t)(unit / ntiles) * p.M * p.N * 4);
 #pragma unroll
             for(int i = 0; i < MT; ++i)
             {
@@ -543,7 +558,25 @@ struct GemmTile
                     const int n0 = tn * BN + wn * WTN + 64 * g + 16 * (lane >> 4);
                     if(m < p.M && n0 < p.N)
                     {
-                        if constexpr(DT == DT_I8)
+                        if(p.ksplit > 1)
+                        {
+                            // raw accumulators, 16 consecutive columns = 64 bytes per lane
+                            uint8_t* wrow = reinterpret_cast<uint8_t*>(slice) + ((size_t)m * p.N + n0) * 4;
+                            if(n0 + 16 <= p.N && (p.N & 3) == 0)
+                            {
+#pragma unroll
+                                for(int t = 0; t < 4; ++t)
+                                    reinterpret_cast<acc_t*>(wrow)[t] = acc[i][g * 4 + t];
+                            }
+                            else
+                            {
+#pragma unroll
+                                for(int e = 0; e < 16; ++e)
+                                    if(n0 + e < p.N)
+                                        reinterpret_cast<decltype(acc[0][0][0] + 0)*>(wrow)[e] = acc[i][g * 4 + e / 4][e % 4];
+                            }
+                        }
+                        else if constexpr(DT == DT_I8)
                         {
                             int8_t* crow = reinterpret_cast<int8_t*>(p.c) + (size_t)m * p.ldc;
                             const i32x4 v[4] = {acc[i][g * 4], acc[i][g * 4 + 1], acc[i][g * 4 + 2],
@@ -589,9 +622,10 @@ struct GemmTile
         barrier();
         read_frags(smem, smem + A_TILE, 0, af0, bf0);
 
-        int kt = 0;
+        int kt = 0, kt_end = nk;
         int it = 0;
-        for(int tile = (int)blockIdx.x; tile < ntiles;)
+        unit_k_range((int)blockIdx.x, kt, kt_end);
+        for(int unit = (int)blockIdx.x; unit < nunits;)
         {
             const uint8_t* sa  = smem + (it & 1) * STAGE;
             const uint8_t* sb  = sa + A_TILE;
@@ -610,11 +644,11 @@ struct GemmTile
             advance_load_cursor();
 
             ++it;
-            if(++kt == nk)
+            if(++kt >= kt_end)
             {
-                epilogue(tile);
-                kt = 0;
-                tile += gstride;
+                epilogue(unit);
+                unit += gstride;
+                unit_k_range(unit, kt, kt_end);
             }
         }
         // the trailing (all-zero) loads still target LDS: let them retire before the workgroup
@@ -622,6 +656,62 @@ struct GemmTile
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     }
 };
+
+// Second pass of a split-K launch: C = epilogue(sum over the K runs of the workspace slices).
+// One thread per 16 consecutive columns of a row, slices added in run order (deterministic).
+template <int DT>
+__global__ __launch_bounds__(256) void splitk_reduce_kernel(const GemmArgs p)
+{
+    using acc_t   = typename std::conditional<DT == DT_I8, i32x4, f32x4>::type;
+    constexpr int ES = DT == DT_I8 ? 1 : 2;
+    const int groups_per_row = (p.N + 15) / 16;
+    const long gid = (long)blockIdx.x * 256 + threadIdx.x;
+    if(gid >= (long)p.M * groups_per_row)
+        return;
+    const int m  = (int)(gid / groups_per_row);
+    const int n0 = (int)(gid - (long)m * groups_per_row) * 16;
+    acc_t v[4];
+#pragma unroll
+    for(int t = 0; t < 4; ++t)
+        v[t] = acc_t{0, 0, 0, 0};
+    const bool full = n0 + 16 <= p.N && (p.N & 3) == 0;
+    for(int sp = 0; sp < p.ksplit; ++sp)
+    {
+        const uint8_t* wrow = reinterpret_cast<const uint8_t*>(p.ws) + (((size_t)sp * p.M + m) * p.N + n0) * 4;
+        if(full)
+        {
+#pragma unroll
+            for(int t = 0; t < 4; ++t)
+            {
+                const acc_t w = reinterpret_cast<const acc_t*>(wrow)[t];
+                v[t][0] += w[0], v[t][1] += w[1], v[t][2] += w[2], v[t][3] += w[3];
+            }
+        }
+        else
+        {
+#pragma unroll
+            for(int e = 0; e < 16; ++e)
+                if(n0 + e < p.N)
+                    v[e / 4][e % 4] += reinterpret_cast<const decltype(v[0][0] + 0)*>(wrow)[e];
+        }
+    }
+    const bool vec_ok = ((reinterpret_cast<uintptr_t>(p.c) | ((uintptr_t)p.ldc * ES)) & 15u) == 0;
+    if constexpr(DT == DT_I8)
+    {
+        int8_t* crow = reinterpret_cast<int8_t*>(p.c) + (size_t)m * p.ldc;
+        if(p.epi == EPI_REQUANT_RND)
+            store_row16_i8<EPI_REQUANT_RND>(crow, n0, p.N, vec_ok, v, p.scale_gemm, p.scale_relu);
+        else if(p.epi == EPI_REQUANT_CK)
+            store_row16_i8<EPI_REQUANT_CK>(crow, n0, p.N, vec_ok, v, p.scale_gemm, p.scale_relu);
+        else
+            store_row16_i8<EPI_PASSTHROUGH>(crow, n0, p.N, vec_ok, v, p.scale_gemm, p.scale_relu);
+    }
+    else
+    {
+        _Float16* crow = reinterpret_cast<_Float16*>(p.c) + (size_t)m * p.ldc;
+        store_row16_f16(crow, n0, p.N, vec_ok, v);
+    }
+}
 
 template <int DT, int BM, int BN, int WM, int WN, int BKB, int NST, bool IM2COL>
 __global__ __launch_bounds__(WM* WN * 64) void gemm_tile_kernel(const GemmArgs p)

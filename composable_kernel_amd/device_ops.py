@@ -67,7 +67,9 @@ def _ptr(x):
 
 
 class BaseArgument:
-    p_workspace_ = None
+    p_workspace_ = None       # device pointer (int) set through SetWorkSpacePointer
+    workspace_bytes_ = 0
+    _workspace_owner = None   # keeps a torch tensor alive when one was passed
 
 
 class BaseInvoker:
@@ -104,10 +106,14 @@ class BaseOperator:
         return capi.lib().ckx_instance_name(self.op_family, self.instance).decode()
 
     def GetWorkSpaceSize(self, arg):
+        """Bytes of optional device scratch (split-K); 0 for most problems."""
         return 0
 
-    def SetWorkSpacePointer(self, arg, p):
-        arg.p_workspace_ = p
+    def SetWorkSpacePointer(self, arg, p, nbytes=None):
+        """p: device address or torch CUDA tensor of at least GetWorkSpaceSize(arg) bytes."""
+        arg._workspace_owner = p
+        arg.p_workspace_ = _ptr(p)
+        arg.workspace_bytes_ = int(nbytes if nbytes is not None else self.GetWorkSpaceSize(arg))
 
     def MakeInvokerPointer(self):
         return BaseInvoker(self)
@@ -153,10 +159,14 @@ class DeviceGemmInt8(_DeviceGemm):
         return capi.lib().ckx_gemm_i8_is_supported(a.M, a.N, a.K, a.StrideA, a.StrideB, a.StrideC,
                                                    *self.layouts, a.c_op.epilogue, self.instance)
 
+    def GetWorkSpaceSize(self, a):
+        return int(capi.lib().ckx_gemm_i8_workspace_bytes(a.M, a.N, a.K, self.instance))
+
     def _launch(self, a, stream):
         return capi.lib().ckx_gemm_i8(a.p_a, a.p_b, a.p_c, a.M, a.N, a.K, a.StrideA, a.StrideB, a.StrideC,
                                       *self.layouts, a.c_op.epilogue, a.c_op.scale_gemm, a.c_op.scale_relu,
-                                      self.instance, C.c_void_p(stream or 0))
+                                      self.instance, a.p_workspace_ or 0, a.workspace_bytes_,
+                                      C.c_void_p(stream or 0))
 
 
 class DeviceGemmF16(_DeviceGemm):
@@ -170,9 +180,13 @@ class DeviceGemmF16(_DeviceGemm):
         return capi.lib().ckx_gemm_f16_is_supported(a.M, a.N, a.K, a.StrideA, a.StrideB, a.StrideC,
                                                     *self.layouts, self.instance)
 
+    def GetWorkSpaceSize(self, a):
+        return int(capi.lib().ckx_gemm_f16_workspace_bytes(a.M, a.N, a.K, self.instance))
+
     def _launch(self, a, stream):
         return capi.lib().ckx_gemm_f16(a.p_a, a.p_b, a.p_c, a.M, a.N, a.K, a.StrideA, a.StrideB, a.StrideC,
-                                       *self.layouts, self.instance, C.c_void_p(stream or 0))
+                                       *self.layouts, self.instance, a.p_workspace_ or 0, a.workspace_bytes_,
+                                       C.c_void_p(stream or 0))
 
 
 # -------------------------------------------------------------------- conv
@@ -203,6 +217,9 @@ class _DeviceConvFwd(BaseOperator):
         return capi.lib().ckx_conv2d_fwd_is_supported(self.op_family, C.byref(a.desc), a.out_op.epilogue,
                                                       self.instance)
 
+    def GetWorkSpaceSize(self, a):
+        return int(capi.lib().ckx_conv2d_fwd_workspace_bytes(self.op_family, C.byref(a.desc), self.instance))
+
 
 class DeviceConv2dFwdInt8(_DeviceConvFwd):
     op_family = capi.OP_CONV2D_FWD_I8
@@ -210,7 +227,7 @@ class DeviceConv2dFwdInt8(_DeviceConvFwd):
     def _launch(self, a, stream):
         return capi.lib().ckx_conv2d_fwd_i8(a.p_in, a.p_wei, a.p_out, C.byref(a.desc), a.out_op.epilogue,
                                             a.out_op.scale_gemm, a.out_op.scale_relu, self.instance,
-                                            C.c_void_p(stream or 0))
+                                            a.p_workspace_ or 0, a.workspace_bytes_, C.c_void_p(stream or 0))
 
 
 class DeviceConv2dFwdF16(_DeviceConvFwd):
@@ -218,7 +235,7 @@ class DeviceConv2dFwdF16(_DeviceConvFwd):
 
     def _launch(self, a, stream):
         return capi.lib().ckx_conv2d_fwd_f16(a.p_in, a.p_wei, a.p_out, C.byref(a.desc), self.instance,
-                                             C.c_void_p(stream or 0))
+                                             a.p_workspace_ or 0, a.workspace_bytes_, C.c_void_p(stream or 0))
 
 
 # --------------------------------------------------------------- GEMM-GEMM

@@ -160,7 +160,7 @@ namespace device {
 struct BaseArgument
 {
     virtual ~BaseArgument() {}
-    void* p_workspace_ = nullptr;
+    void* p_workspace_ = nullptr; // optional device scratch, GetWorkSpaceSize() bytes (split-K)
 };
 
 struct BaseInvoker
@@ -327,13 +327,23 @@ struct DeviceGemmMfma : public DeviceGemm<ALayout, BLayout, CLayout, ADataType, 
     }
     static int Launch(const Argument& a, int inst, void* stream)
     {
+        const int64_t ws_bytes = a.p_workspace_ ? WorkSpaceBytes(a, inst) : 0;
         if constexpr(is_i8)
             return ckx_gemm_i8(a.p_a, a.p_b, a.p_c, a.M, a.N, a.K, a.StrideA, a.StrideB, a.StrideC, ALayout::code,
                                BLayout::code, CLayout::code, Epi::kind, Epi::scale_gemm(a.c_element_op),
-                               Epi::scale_relu(a.c_element_op), inst, stream);
+                               Epi::scale_relu(a.c_element_op), inst, a.p_workspace_, ws_bytes, stream);
         else
             return ckx_gemm_f16(a.p_a, a.p_b, a.p_c, a.M, a.N, a.K, a.StrideA, a.StrideB, a.StrideC, ALayout::code,
-                                BLayout::code, CLayout::code, inst, stream);
+                                BLayout::code, CLayout::code, inst, a.p_workspace_, ws_bytes, stream);
+    }
+    static int64_t WorkSpaceBytes(const Argument& a, int inst)
+    {
+        return is_i8 ? ckx_gemm_i8_workspace_bytes(a.M, a.N, a.K, inst) : ckx_gemm_f16_workspace_bytes(a.M, a.N, a.K, inst);
+    }
+    size_t GetWorkSpaceSize(const BaseArgument* p) const override
+    {
+        const auto* a = dynamic_cast<const Argument*>(p);
+        return a ? (size_t)WorkSpaceBytes(*a, instance_) : 0;
     }
     using Invoker = detail::InvokerT<Argument, &Supported, &Launch>;
 
@@ -413,12 +423,18 @@ struct DeviceConv2dFwdMfma_Input_N_Hi_Wi_C_Weight_K_Y_X_C_Output_N_Ho_Wo_K
     }
     static int Launch(const Argument& a, int inst, void* stream)
     {
+        const int64_t ws_bytes = a.p_workspace_ ? ckx_conv2d_fwd_workspace_bytes(op_code, &a.desc, inst) : 0;
         if constexpr(is_i8)
             return ckx_conv2d_fwd_i8(a.p_in, a.p_wei, a.p_out, &a.desc, Epi::kind,
                                      Epi::scale_gemm(a.out_element_op), Epi::scale_relu(a.out_element_op), inst,
-                                     stream);
+                                     a.p_workspace_, ws_bytes, stream);
         else
-            return ckx_conv2d_fwd_f16(a.p_in, a.p_wei, a.p_out, &a.desc, inst, stream);
+            return ckx_conv2d_fwd_f16(a.p_in, a.p_wei, a.p_out, &a.desc, inst, a.p_workspace_, ws_bytes, stream);
+    }
+    size_t GetWorkSpaceSize(const BaseArgument* p) const override
+    {
+        const auto* a = dynamic_cast<const Argument*>(p);
+        return a && a->two_d ? (size_t)ckx_conv2d_fwd_workspace_bytes(op_code, &a->desc, instance_) : 0;
     }
     using Invoker = detail::InvokerT<Argument, &Supported, &Launch>;
 

@@ -7,7 +7,8 @@
  * these calls and carry CK's own interface. All pointers are DEVICE pointers,
  * strides are in ELEMENTS, dimensions are int32 (CK's index_t, include/ck/ck.hpp:176),
  * `stream` is a hipStream_t passed as void* (NULL = default stream). Launches are
- * asynchronous; nothing is allocated, nothing is synchronised.
+ * asynchronous; nothing is allocated, nothing is synchronised. Scratch memory, where a launch
+ * can use it, is the caller's (p_workspace, see ckx_*_workspace_bytes).
  *
  * Return value: 0 on success, a negative ckx_status otherwise; the message for
  * the calling thread's last failure is returned by ckx_last_error().
@@ -89,7 +90,13 @@ int ckx_gemm_i8_is_supported(int32_t M, int32_t N, int32_t K, int32_t stride_a, 
 int ckx_gemm_i8(const void* p_a, const void* p_b, void* p_c, int32_t M, int32_t N, int32_t K,
                 int32_t stride_a, int32_t stride_b, int32_t stride_c, int a_layout, int b_layout,
                 int c_layout, int epilogue, float scale_gemm, float scale_relu, int instance,
-                void* stream);
+                void* p_workspace, int64_t workspace_bytes, void* stream);
+/* BaseOperator::GetWorkSpaceSize (device_base.hpp:47): bytes of device scratch with which the
+ * launch may cut K into several runs (split-K: problems with too few C tiles to occupy the
+ * machine). The workspace is OPTIONAL: with p_workspace == NULL, or fewer bytes than asked for,
+ * the launch uses a plan that needs none. It needs no initialisation and holds nothing between
+ * calls; two launches that share one workspace must not overlap. */
+int64_t ckx_gemm_i8_workspace_bytes(int32_t M, int32_t N, int32_t K, int instance);
 
 /* ---- fp16 GEMM:  C = half(A * B), fp32 accumulation -----------------------
  * Replaces DeviceGemm<..., half_t, half_t, half_t, PassThrough x3>
@@ -98,7 +105,8 @@ int ckx_gemm_f16_is_supported(int32_t M, int32_t N, int32_t K, int32_t stride_a,
                               int32_t stride_c, int a_layout, int b_layout, int c_layout, int instance);
 int ckx_gemm_f16(const void* p_a, const void* p_b, void* p_c, int32_t M, int32_t N, int32_t K,
                  int32_t stride_a, int32_t stride_b, int32_t stride_c, int a_layout, int b_layout,
-                 int c_layout, int instance, void* stream);
+                 int c_layout, int instance, void* p_workspace, int64_t workspace_bytes, void* stream);
+int64_t ckx_gemm_f16_workspace_bytes(int32_t M, int32_t N, int32_t K, int instance);
 
 /* ---- conv2d forward, NHWC input / KYXC weight / NHWK output, implicit GEMM --
  * Replaces DeviceConvFwd<PassThrough, PassThrough, OutOp>::MakeArgumentPointer + Run
@@ -122,9 +130,11 @@ typedef struct ckx_conv2d_desc
 
 int ckx_conv2d_fwd_is_supported(int op, const ckx_conv2d_desc* desc, int epilogue, int instance);
 int ckx_conv2d_fwd_i8(const void* p_in, const void* p_wei, void* p_out, const ckx_conv2d_desc* desc,
-                      int epilogue, float scale_gemm, float scale_relu, int instance, void* stream);
+                      int epilogue, float scale_gemm, float scale_relu, int instance, void* p_workspace,
+                      int64_t workspace_bytes, void* stream);
 int ckx_conv2d_fwd_f16(const void* p_in, const void* p_wei, void* p_out, const ckx_conv2d_desc* desc,
-                       int instance, void* stream);
+                       int instance, void* p_workspace, int64_t workspace_bytes, void* stream);
+int64_t ckx_conv2d_fwd_workspace_bytes(int op, const ckx_conv2d_desc* desc, int instance);
 
 /* ---- batched fused GEMM-GEMM, fp16:  C[g] = half( half(A[g]*B0[g]) * B1[g] ) --
  * The reference snapshot has no such operator; the surface is upstream's

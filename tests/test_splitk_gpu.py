@@ -1,0 +1,122 @@
+"""GPU parity of the split-K plans (C tiles cut into K runs, raw accumulators in a caller
+workspace, second pass sums the runs and applies the epilogue). The run count is chosen by the
+library; CKX_KSPLIT forces it here so that small problems exercise every path. int8 stays
+bit-exact for any split (int32 partial sums); fp16 slices are added in a fixed order."""
+import os
+
+import numpy as np
+import pytest
+
+import composable_kernel_amd as ck
+from composable_kernel_amd import capi
+from composable_kernel_amd.host_tensor import uniform_f16, uniform_int8
+from oracle import fast, lit
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture
+def force_split():
+    def _set(n):
+        if n:
+            os.environ["CKX_KSPLIT"] = str(n)
+        else:
+            os.environ.pop("CKX_KSPLIT", None)
+    yield _set
+    os.environ.pop("CKX_KSPLIT", None)
+
+
+def _run_gemm(op, a, b_nk, c_dtype, c_op=None):
+    import torch
+    import gpu_util
+    M, K = a.shape
+    N = b_nk.shape[0]
+    da, db = gpu_util.dev(a), gpu_util.dev(b_nk)
+    dc = torch.zeros((M, N), dtype=c_dtype, device="cuda")
+    arg = op.MakeArgumentPointer(da, db, dc, M, N, K, K, K, N, None, None, c_op)
+    assert op.IsSupportedArgument(arg)
+    need = op.GetWorkSpaceSize(arg)
+    ws = torch.full((max(need, 16),), 0x7F, dtype=torch.uint8, device="cuda")   # garbage on purpose
+    op.SetWorkSpacePointer(arg, ws)
+    op.MakeInvokerPointer().Run(arg, ck.StreamConfig(gpu_util.stream()))
+    op.MakeInvokerPointer().Run(arg, ck.StreamConfig(gpu_util.stream()))        # idempotent, workspace reusable
+    torch.cuda.synchronize()
+    return dc.cpu().numpy(), need
+
+
+@pytest.mark.parametrize("split", [2, 3, 5, 8])
+@pytest.mark.parametrize("shape", [(128, 320, 4096), (130, 200, 2064), (300, 72, 1040), (256, 256, 1024)])
+@pytest.mark.parametrize("instance", [capi.INSTANCE_AUTO, 0, 3, 6])
+def test_int8_gemm_split_k_bit_exact(force_split, split, shape, instance):
+    M, N, K = shape
+    a = uniform_int8((M, K), -8, 8, 70 + M)
+    b_nk = uniform_int8((N, K), -8, 8, 71 + N)
+    force_split(split)
+    import torch
+    out, need = _run_gemm(ck.DeviceGemmInt8(instance), a, b_nk, torch.int8,
+                          ck.RequantReluRequant(0.02, 0.4, rounded=True))
+    nk = (K + 127) // 128
+    if -(-nk // split) * (split - 1) < nk:
+        assert need == split * M * N * 4        # the forced split was taken
+    np.testing.assert_array_equal(out, fast.gemm_i8(a, b_nk.T, lit.EPI_REQUANT_RND, 0.02, 0.4))
+
+
+@pytest.mark.parametrize("split", [2, 4])
+def test_fp16_gemm_split_k(force_split, split):
+    import torch
+    M, N, K = 136, 264, 2056
+    a = uniform_f16((M, K), -1, 1, 72)
+    b_nk = uniform_f16((N, K), -1, 1, 73)
+    force_split(split)
+    out, need = _run_gemm(ck.DeviceGemmF16(), a, b_nk, torch.float16)
+    assert need == split * M * N * 4
+    bad, max_err = lit.check_err_f16(out, lit.gemm_f16(a, b_nk.T), 1e-2, 1e-2)
+    assert bad == 0, max_err
+    out2, _ = _run_gemm(ck.DeviceGemmF16(), a, b_nk, torch.float16)
+    np.testing.assert_array_equal(out.view(np.uint16), out2.view(np.uint16))   # fixed summation order
+
+
+def test_split_k_without_workspace_falls_back(force_split):
+    import torch
+    import gpu_util
+    M, N, K = 128, 256, 4096
+    a = uniform_int8((M, K), -8, 8, 74)
+    b_nk = uniform_int8((N, K), -8, 8, 75)
+    force_split(4)
+    out = gpu_util.gemm_i8(a, b_nk, ck.PassThrough())        # no workspace attached
+    np.testing.assert_array_equal(out, fast.gemm_i8(a, b_nk.T))
+
+
+@pytest.mark.parametrize("dtype", ["int8", "fp16"])
+def test_conv2d_split_k(force_split, dtype):
+    import torch
+    import gpu_util
+    N, C, K, HW = 3, 64, 96, 7
+    s, d, p = (1, 1), (1, 1), (1, 1)
+    force_split(3)
+    if dtype == "int8":
+        inp = uniform_int8((N, HW, HW, C), -5, 5, 76)
+        wei = uniform_int8((K, 3, 3, C), -5, 5, 77)
+        op, tdt = ck.DeviceConv2dFwdInt8(), torch.int8
+        out_op = ck.RequantReluRequant(0.05, 0.7, rounded=True)
+    else:
+        inp = uniform_f16((N, HW, HW, C), -1, 1, 76)
+        wei = uniform_f16((K, 3, 3, C), -1, 1, 77)
+        op, tdt = ck.DeviceConv2dFwdF16(), torch.float16
+        out_op = None
+    di, dw = gpu_util.dev(inp), gpu_util.dev(wei)
+    do = torch.zeros((N, HW, HW, K), dtype=tdt, device="cuda")
+    arg = op.MakeArgumentPointer(di, dw, do, N, K, C, [HW, HW], [3, 3], [HW, HW], [1, 1], [1, 1], [1, 1], [1, 1],
+                                 None, None, out_op)
+    need = op.GetWorkSpaceSize(arg)
+    assert need == 3 * N * HW * HW * K * 4
+    ws = torch.empty(need, dtype=torch.uint8, device="cuda")
+    op.SetWorkSpacePointer(arg, ws)
+    op.MakeInvokerPointer().Run(arg, ck.StreamConfig(gpu_util.stream()))
+    torch.cuda.synchronize()
+    if dtype == "int8":
+        np.testing.assert_array_equal(
+            do.cpu().numpy(), lit.conv2d_fwd(inp, wei, s, d, p, epi=lit.EPI_REQUANT_RND, scale_gemm=0.05, scale_relu=0.7))
+    else:
+        bad, max_err = lit.check_err_f16(do.cpu().numpy(), lit.conv2d_fwd(inp, wei, s, d, p), 1e-2, 1e-2)
+        assert bad == 0, max_err
