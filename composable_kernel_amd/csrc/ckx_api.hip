@@ -113,24 +113,25 @@ struct TileInstance
     tile_launch_fn dense_i8, dense_f16, conv_i8, conv_f16;
 };
 
-#define CKX_TILE(BM, BN, WM, WN, EFF)                                                              \
+#define CKX_TILE(BM, BN, WM, WN, NST, EFF)                                                         \
     {                                                                                              \
-        "MI355X_Mfma16_Tile<" #BM ", " #BN ", 128B x2, waves " #WM "x" #WN ">", BM, BN, WM* WN * 64,     \
-            2 * (BM + BN) * 128, EFF, &launch_tile<ckx::DT_I8, BM, BN, WM, WN, 128, 2, false>,           \
-            &launch_tile<ckx::DT_F16, BM, BN, WM, WN, 128, 2, false>,                                 \
-            &launch_tile<ckx::DT_I8, BM, BN, WM, WN, 128, 2, true>,                                   \
-            &launch_tile<ckx::DT_F16, BM, BN, WM, WN, 128, 2, true>                                   \
+        "MI355X_Mfma16_Tile<" #BM ", " #BN ", 128B x" #NST ", waves " #WM "x" #WN ">", BM, BN,           \
+            WM* WN * 64, NST*(BM + BN) * 128, EFF, &launch_tile<ckx::DT_I8, BM, BN, WM, WN, 128, NST, false>, \
+            &launch_tile<ckx::DT_F16, BM, BN, WM, WN, 128, NST, false>,                               \
+            &launch_tile<ckx::DT_I8, BM, BN, WM, WN, 128, NST, true>,                                 \
+            &launch_tile<ckx::DT_F16, BM, BN, WM, WN, 128, NST, true>                                 \
     }
 
 const TileInstance kTiles[] = {
-    CKX_TILE(256, 256, 2, 4, 1.00f),
-    CKX_TILE(256, 128, 4, 2, 0.84f),
-    CKX_TILE(128, 128, 2, 2, 0.78f),
-    CKX_TILE(128, 64, 4, 1, 0.68f),
-    CKX_TILE(64, 64, 4, 1, 0.55f),
-    CKX_TILE(32, 64, 2, 1, 0.42f),
-    CKX_TILE(16, 64, 1, 1, 0.27f),
-    CKX_TILE(256, 64, 8, 1, 0.70f),
+    CKX_TILE(256, 256, 2, 4, 2, 1.00f),
+    CKX_TILE(256, 128, 4, 2, 2, 0.84f),
+    CKX_TILE(128, 128, 2, 2, 2, 0.78f),
+    CKX_TILE(128, 64, 4, 1, 2, 0.68f),
+    CKX_TILE(64, 64, 4, 1, 2, 0.55f),
+    CKX_TILE(32, 64, 2, 1, 2, 0.42f),
+    CKX_TILE(16, 64, 1, 1, 2, 0.27f),
+    CKX_TILE(256, 64, 8, 1, 2, 0.70f),
+    CKX_TILE(64, 64, 4, 1, 4, 0.55f),
 };
 constexpr int kNumTiles = sizeof(kTiles) / sizeof(kTiles[0]);
 
@@ -183,7 +184,9 @@ Plan make_plan(int M, int N, int kbytes, int only_tile, long workspace_bytes)
             // one K-tile iteration costs its MFMA time, but never less than the barrier + load
             // latency of the two-stage pipeline (~0.42 us measured on small tiles)
             double iter_us = per_cu * (t.bm * t.bn / 65536.0) / t.eff * 1.1;
-            iter_us        = iter_us < 0.42 ? 0.42 : iter_us;
+            const int nst  = t.lds / ((t.bm + t.bn) * 128);
+            const double floor_us = nst > 2 ? 0.36 : 0.42;
+            iter_us        = iter_us < floor_us ? floor_us : iter_us;
             double us      = rounds * (iter_us * nk_per + 6.0 / per_cu + 2.0);
             if(sp > 1)
             {

@@ -272,7 +272,8 @@ __device__ __forceinline__ void sched_loads_reads_mfma()
 
 // ------------------------------------------------------------------- kernel
 // BKB   bytes of every row staged per K tile (128)
-// NST   LDS stages (2)
+// NST   LDS stages: the loads of K tile k + NST are issued while tile k is multiplied (2: big tiles
+//       that fill the LDS; 4: small tiles of latency-bound problems)
 // The kernel is PERSISTENT: workgroup b works on tiles b, b + gridDim.x, ... and the K-tile
 // pipeline runs straight across tile boundaries, so the first loads of the next tile are in
 // flight under the last MFMAs, the epilogue arithmetic and the C stores of the current one.
@@ -296,7 +297,8 @@ struct GemmTile
     static constexpr int NLA     = BM * CPR / NT; // 16-byte loads per thread and K tile, A
     static constexpr int NLB     = BN * CPR / NT;
     static constexpr int LPT     = NLA + NLB;
-    static_assert(BKB == 128 && KSTEPS == 2 && NST == 2, "pipeline written for 128-byte K tiles, two stages");
+    static_assert(BKB == 128 && KSTEPS == 2, "pipeline written for 128-byte K tiles");
+    static_assert(NST >= 2 && (NST - 2) * LPT < 64, "vmcnt is a 6-bit counter");
     static_assert(WTM % 16 == 0 && WTN % 64 == 0, "wave tile must be 16k x 64k");
     static_assert((BM * CPR) % NT == 0 && (BN * CPR) % NT == 0, "tile rows must split over the waves");
 
@@ -614,39 +616,50 @@ struct GemmTile
         // or of the next C tile) are read while the second half is still being multiplied.
         i32x4 af0[MT], bf0[NG * 4], af1[MT], bf1[NG * 4];
 
-        issue_loads(ld_kt, 0);
-        advance_load_cursor();
-        issue_loads(ld_kt, 1);
-        advance_load_cursor();
-        asm volatile("s_waitcnt vmcnt(%0)" ::"n"(LPT) : "memory");
+#pragma unroll
+        for(int st = 0; st < NST; ++st)
+        {
+            issue_loads(ld_kt, st);
+            advance_load_cursor();
+        }
+        asm volatile("s_waitcnt vmcnt(%0)" ::"n"((NST - 1) * LPT) : "memory");
         barrier();
         read_frags(smem, smem + A_TILE, 0, af0, bf0);
 
         int kt = 0, kt_end = nk;
-        int it = 0;
+        int st_cur = 0;       // stage of the K tile being multiplied
+        bool drain = false;   // C stores are in flight: the next wait cannot count loads
         unit_k_range((int)blockIdx.x, kt, kt_end);
         for(int unit = (int)blockIdx.x; unit < nunits;)
         {
-            const uint8_t* sa  = smem + (it & 1) * STAGE;
+            const int st_next  = st_cur + 1 == NST ? 0 : st_cur + 1;
+            const uint8_t* sa  = smem + st_cur * STAGE;
             const uint8_t* sb  = sa + A_TILE;
-            const uint8_t* san = smem + ((it + 1) & 1) * STAGE;
+            const uint8_t* san = smem + st_next * STAGE;
             const uint8_t* sbn = san + A_TILE;
 
             half_step(std::false_type{}, LoadCtx{}, af0, bf0, sa, sb, 1, af1, bf1);
 
-            // the next K tile has landed (its loads are the only ones in flight, C stores of an
-            // earlier epilogue aside) and the current one is entirely in registers
-            asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+            // The direct loads of a wave retire in order: once at most NST-2 K tiles' worth are in
+            // flight, the next K tile has landed. C stores of an epilogue share the counter and are
+            // not ordered against loads, so the first wait after an epilogue drains everything.
+            // The current K tile is entirely in registers by now (lgkmcnt).
+            if(drain)
+                asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+            else
+                asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" ::"n"((NST - 2) * LPT) : "memory");
+            drain = false;
             barrier();
 
-            const LoadCtx lc = load_ctx(ld_kt, it & 1);
+            const LoadCtx lc = load_ctx(ld_kt, st_cur);
             half_step(std::true_type{}, lc, af1, bf1, san, sbn, 0, af0, bf0);
             advance_load_cursor();
 
-            ++it;
+            st_cur = st_next;
             if(++kt >= kt_end)
             {
                 epilogue(unit);
+                drain = true;
                 unit += gstride;
                 unit_k_range(unit, kt, kt_end);
             }

@@ -39,7 +39,7 @@ def _f16_close(out, ref):
 
 
 @pytest.mark.parametrize("case", SMALL)
-@pytest.mark.parametrize("instance", [capi.INSTANCE_AUTO, 0, 2, 4, 6, 7])
+@pytest.mark.parametrize("instance", [capi.INSTANCE_AUTO, 0, 2, 4, 6, 7, 8])
 def test_conv2d_int8_small_cases_bit_exact(case, instance):
     import gpu_util
     N, C, K, Hi, Wi, Y, X, s, d, p = case
@@ -54,7 +54,7 @@ def test_conv2d_int8_small_cases_bit_exact(case, instance):
 
 
 @pytest.mark.parametrize("case", SMALL)
-@pytest.mark.parametrize("instance", [capi.INSTANCE_AUTO, 1, 3, 5])
+@pytest.mark.parametrize("instance", [capi.INSTANCE_AUTO, 1, 3, 5, 8])
 def test_conv2d_fp16_small_cases(case, instance):
     import gpu_util
     N, C, K, Hi, Wi, Y, X, s, d, p = case

@@ -16,8 +16,8 @@ from oracle import fast, lit
 
 pytestmark = pytest.mark.gpu
 
-N_INSTANCES = 12        # tile instances followed by the skinny (few-row) instances
-SKINNY_MAX_M = {8: 16, 9: 32, 10: 64, 11: 16}
+N_INSTANCES = 13        # tile instances followed by the skinny (few-row) instances
+SKINNY_MAX_M = {9: 16, 10: 32, 11: 64, 12: 16}
 RTOL = ATOL = 1e-2
 
 EPILOGUES = {
