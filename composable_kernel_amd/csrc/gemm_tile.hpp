@@ -492,16 +492,19 @@ struct GemmTile
         const uint32_t frow = (uint32_t)(lane & 15);
         const uint32_t fq   = (uint32_t)(lane >> 4);
 
+        // Fragment r of a k-step, in the order in which the MFMAs of that k-step need them: the B
+        // fragments and the first A fragment feed the first MFMA group, the last A fragment only
+        // the last one, so the LDS latency of the late reads hides under the early groups.
         auto read_one = [&](const uint8_t* sa, const uint8_t* sb, int ks, int r, i32x4(&af)[MT], i32x4(&bf)[NG * 4]) {
-            if(r < MT)
+            if(r < NG * 4)
             {
-                const uint32_t row = (uint32_t)(wm * WTM + 16 * r) + frow;
-                af[r] = *reinterpret_cast<const i32x4*>(sa + chunk_offset(row, ks * 4 + fq));
+                const uint32_t row = (uint32_t)(wn * WTN + 16 * r) + frow;
+                bf[r] = *reinterpret_cast<const i32x4*>(sb + chunk_offset(row, ks * 4 + fq));
             }
             else
             {
-                const uint32_t row = (uint32_t)(wn * WTN + 16 * (r - MT)) + frow;
-                bf[r - MT] = *reinterpret_cast<const i32x4*>(sb + chunk_offset(row, ks * 4 + fq));
+                const uint32_t row = (uint32_t)(wm * WTM + 16 * (r - NG * 4)) + frow;
+                af[r - NG * 4] = *reinterpret_cast<const i32x4*>(sa + chunk_offset(row, ks * 4 + fq));
             }
         };
         auto read_frags = [&](const uint8_t* sa, const uint8_t* sb, int ks, i32x4(&af)[MT], i32x4(&bf)[NG * 4]) {
@@ -526,14 +529,22 @@ struct GemmTile
         // on VMEM issue, and its MFMAs wait behind it.
         auto half_step = [&](auto with_loads, const LoadCtx& lc, const i32x4(&caf)[MT], const i32x4(&cbf)[NG * 4],
                              const uint8_t* nsa, const uint8_t* nsb, int nks, i32x4(&naf)[MT], i32x4(&nbf)[NG * 4]) {
+            // The reads are over two groups before the end of the half, so the next half starts with
+            // every fragment it needs at once already in registers. The first half of an iteration
+            // (top of the loop, where the compiler waits for ALL outstanding LDS reads) starts its
+            // reads one group late: that wait then only covers reads issued long before.
             constexpr int NGRP = LPT, NR = MT + NG * 4, NM = MT * NG * 4;
+            constexpr int RG  = NGRP >= 4 ? NGRP - 2 : NGRP;
+            constexpr int RG0 = (NGRP >= 4 && !decltype(with_loads)::value) ? 1 : 0;
 #pragma unroll
             for(int g = 0; g < NGRP; ++g)
             {
                 if constexpr(decltype(with_loads)::value)
                     issue_slot(lc, g);
+                const int gr = g - RG0 < 0 ? 0 : (g - RG0 > RG ? RG : g - RG0); // read groups done before g
+                const int gn = g + 1 - RG0 < 0 ? 0 : (g + 1 - RG0 > RG ? RG : g + 1 - RG0);
 #pragma unroll
-                for(int r = g * NR / NGRP; r < (g + 1) * NR / NGRP; ++r)
+                for(int r = gr * NR / RG; r < gn * NR / RG; ++r)
                     read_one(nsa, nsb, nks, r, naf, nbf);
 #pragma unroll
                 for(int m = g * NM / NGRP; m < (g + 1) * NM / NGRP; ++m)
