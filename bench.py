@@ -66,8 +66,10 @@ for w in (
     WORKLOADS[w["name"]] = w
 
 
-def make_launcher(w, instance=-1):
-    """Allocates the workload's synthetic operands on the GPU, returns (launch_fn, description)."""
+def make_launcher(w, instance=-1, rotate=1):
+    """Allocates the workload's synthetic operands on the GPU, returns the launch function.
+    rotate > 1 (GEMM workloads): that many distinct copies of the B matrix, used round-robin, so
+    that a weight matrix smaller than the 256 MB Infinity Cache is read from HBM every time."""
     import torch
     import composable_kernel_amd as ck
     from composable_kernel_amd import capi
@@ -93,6 +95,11 @@ def make_launcher(w, instance=-1):
             op = ck.DeviceGemmF16(instance)
             cop = ck.PassThrough()
         arg = op.MakeArgumentPointer(a, b, c, M, N, K, K, K, N, None, None, cop)
+        more_args = []
+        for _ in range(rotate - 1):
+            b2 = b.clone()
+            keep.append(b2)
+            more_args.append(op.MakeArgumentPointer(a, b2, c, M, N, K, K, K, N, None, None, cop))
     elif w["kind"] == "conv":
         N, C, K, f, HW, st, pd = (w[k] for k in ("N", "C", "K", "f", "HW", "st", "pd"))
         Ho = (HW + 2 * pd - f) // st + 1
@@ -122,9 +129,17 @@ def make_launcher(w, instance=-1):
         ws = torch.empty(need, dtype=torch.uint8, device="cuda")
         keep.append(ws)
         op.SetWorkSpacePointer(arg, ws)
+    args = [arg]
+    if w["kind"] == "gemm":
+        for extra in more_args:
+            if need:
+                op.SetWorkSpacePointer(extra, ws)
+            args.append(extra)
+    turn = [0]
 
     def launch():
-        st_ = op._launch(arg, torch.cuda.current_stream().cuda_stream)
+        st_ = op._launch(args[turn[0] % len(args)], torch.cuda.current_stream().cuda_stream)
+        turn[0] += 1
         if st_ != 0:
             raise RuntimeError(capi.last_error())
 
@@ -132,16 +147,18 @@ def make_launcher(w, instance=-1):
     return launch
 
 
-def time_workload(w, steps, warmup, instance=-1, use_graph=True):
+def time_workload(w, steps, warmup, instance=-1, use_graph=True, rotate=1):
     """W untimed launches, then exactly K timed ones. The K launches are replayed from a HIP
     graph (captured once from the same C-ABI calls) so that kernels run back to back on the GPU
     even when one kernel is shorter than a Python call; use_graph=False launches eagerly."""
     import torch
-    launch = make_launcher(w, instance)
+    launch = make_launcher(w, instance, rotate)
     for _ in range(warmup):
         launch()
     torch.cuda.synchronize()
-    per_graph = max(d for d in range(1, min(steps, 50) + 1) if steps % d == 0)
+    # launches per captured graph: a divisor of K that walks the rotation a whole number of times
+    cands = [d for d in range(1, min(steps, 50) + 1) if steps % d == 0 and d % rotate == 0]
+    per_graph = max(cands) if cands else rotate
     graph = None
     if use_graph:
         graph = torch.cuda.CUDAGraph()
@@ -240,11 +257,19 @@ def main():
     if args.all:
         extra = [n for n in WORKLOADS if n != args.workload]
     for n in extra:
-        x = time_workload(WORKLOADS[n], max(10, args.steps // 2), max(3, args.warmup // 2), -1, not args.no_graph)
-        also.append({"workload": n, "dtype": x["dtype"], "ms": round(x["ms"], 5),
-                     "value": round(x["tput"], 2), "unit": "TOP/s" if x["dtype"] == "i8" else "TFLOP/s",
-                     "GB/s": round(x["gbs"], 1), "bound": x["bound"],
-                     "frac_of_bound": round(max(x["mfma_frac"], x["hbm_frac"]), 4)})
+        wl = WORKLOADS[n]
+        k_steps, k_warm = max(16, args.steps // 2), max(3, args.warmup // 2)
+        x = time_workload(wl, k_steps, k_warm, -1, not args.no_graph)
+        row = {"workload": n, "dtype": x["dtype"], "ms": round(x["ms"], 5),
+               "value": round(x["tput"], 2), "unit": "TOP/s" if x["dtype"] == "i8" else "TFLOP/s",
+               "GB/s": round(x["gbs"], 1), "bound": x["bound"],
+               "frac_of_bound": round(max(x["mfma_frac"], x["hbm_frac"]), 4)}
+        if wl["kind"] == "gemm" and x["bound"] == "hbm" and wl["bytes"] < 128e6:
+            # the weight matrix fits the Infinity Cache: also time it cold, 8 copies in turn
+            cold = time_workload(wl, k_steps - k_steps % 8, k_warm, -1, not args.no_graph, rotate=8)
+            row.update({"cold_ms": round(cold["ms"], 5), "cold_GB/s": round(cold["gbs"], 1),
+                        "cold_frac_of_bound": round(cold["hbm_frac"], 4)})
+        also.append(row)
 
     unit = "TFLOP/s" if w["dtype"] == "f16" else "TOP/s"
     if r["bound"] == "mfma":

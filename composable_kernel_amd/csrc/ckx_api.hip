@@ -209,28 +209,32 @@ Plan make_plan(int M, int N, int kbytes, int only_tile, long workspace_bytes)
 struct SkinnyInstance
 {
     const char* name;
-    int max_m;
+    int max_m, cols;
     tile_launch_fn i8, f16;
 };
 
-template <int DT, int MT, int NW, int KU>
+template <int DT, int MT, int NW, int KU, int NT>
 hipError_t launch_skinny(const ckx::GemmArgs& a, int grid, hipStream_t s)
 {
-    hipLaunchKernelGGL((ckx::gemm_skinny_kernel<DT, MT, NW, KU>), dim3(grid), dim3(NW * 64), 0, s, a);
+    hipLaunchKernelGGL((ckx::gemm_skinny_kernel<DT, MT, NW, KU, NT>), dim3(grid), dim3(NW * 64), 0, s, a);
     return hipGetLastError();
 }
 
-#define CKX_SKINNY(MT, NW, KU)                                                                 \
-    {                                                                                          \
-        "MI355X_Mfma16_Skinny<rows " #MT "x16, 16 cols, waves " #NW ", unroll " #KU ">", MT * 16, \
-            &launch_skinny<ckx::DT_I8, MT, NW, KU>, &launch_skinny<ckx::DT_F16, MT, NW, KU>       \
+#define CKX_SKINNY(MT, NW, KU, NT)                                                                          \
+    {                                                                                                       \
+        "MI355X_Mfma16_Skinny<rows " #MT "x16, cols " #NT "x16, waves " #NW ", unroll " #KU ">", MT * 16, NT * 16, \
+            &launch_skinny<ckx::DT_I8, MT, NW, KU, NT>, &launch_skinny<ckx::DT_F16, MT, NW, KU, NT>              \
     }
 
 const SkinnyInstance kSkinny[] = {
-    CKX_SKINNY(1, 8, 4),
-    CKX_SKINNY(2, 8, 4),
-    CKX_SKINNY(4, 8, 2),
-    CKX_SKINNY(1, 16, 2),
+    CKX_SKINNY(1, 8, 4, 1),
+    CKX_SKINNY(2, 8, 4, 1),
+    CKX_SKINNY(4, 8, 2, 1),
+    CKX_SKINNY(1, 16, 2, 1),
+    CKX_SKINNY(1, 8, 2, 4),
+    CKX_SKINNY(1, 8, 2, 2),
+    CKX_SKINNY(2, 8, 2, 4),
+    CKX_SKINNY(2, 8, 2, 2),
 };
 constexpr int kNumSkinny    = sizeof(kSkinny) / sizeof(kSkinny[0]);
 constexpr int kNumGemmInsts = kNumTiles + kNumSkinny;
@@ -277,7 +281,7 @@ int check_gemm_shape(int dt, int M, int N, int K, int sa, int sb, int sc, int al
 long gemm_workspace_bytes(int dt, int M, int N, int K, int instance)
 {
     const int es = dt == ckx::DT_I8 ? 1 : 2;
-    if(M <= 0 || N <= 0 || (instance == CKX_INSTANCE_AUTO && M <= 64) || instance >= kNumTiles)
+    if(M <= 0 || N <= 0 || (instance == CKX_INSTANCE_AUTO && M <= 32) || instance >= kNumTiles)
         return 0;
     const Plan pl = make_plan(M, N, K * es, instance, 1l << 60);
     return pl.ksplit > 1 ? (long)pl.ksplit * M * N * 4 : 0;
@@ -299,10 +303,17 @@ int run_gemm(int dt, const void* a, const void* b, void* c, int M, int N, int K,
     const int es = dt == ckx::DT_I8 ? 1 : 2;
     int ti = instance;
     Plan pl;
-    if(instance == CKX_INSTANCE_AUTO && M <= 64)
+    // 33..64 rows: the tile kernel wins when its C tiles (or C tiles x K runs) fill the machine
+    const bool tile64 = M > 32 && M <= 64 &&
+                        ((N + 63) / 64 >= 160 ||
+                         (ws && !(reinterpret_cast<uintptr_t>(ws) & 15) && make_plan(M, N, K * es, -1, ws_bytes).ksplit > 1));
+    if(instance == CKX_INSTANCE_AUTO && M <= 64 && !tile64)
     {
-        // a handful of rows against a big weight matrix is an HBM-streaming problem
-        ti = M <= 16 ? kNumTiles + 0 : M <= 32 ? kNumTiles + 1 : kNumTiles + 2;
+        // A handful of rows against a big weight matrix is an HBM-streaming problem. Wider
+        // workgroups (32 / 64 columns) re-read A from L2 less often, as long as enough workgroups
+        // remain to keep every CU pulling on HBM; up to 8 rows A is too small to matter.
+        const int wide = M <= 8 ? 0 : (N + 63) / 64 >= 160 ? 2 : (N + 31) / 32 >= 160 ? 1 : 0;
+        ti = kNumTiles + (M <= 16 ? (wide == 2 ? 4 : wide == 1 ? 5 : 0) : M <= 32 ? (wide == 2 ? 6 : wide == 1 ? 7 : 1) : 2);
     }
     else if(instance < kNumTiles)
     {
@@ -326,7 +337,7 @@ int run_gemm(int dt, const void* a, const void* b, void* c, int M, int N, int K,
     if(ti >= kNumTiles)
     {
         const SkinnyInstance& k = kSkinny[ti - kNumTiles];
-        hipError_t e = (dt == ckx::DT_I8 ? k.i8 : k.f16)(g, (N + 15) / 16, (hipStream_t)stream);
+        hipError_t e = (dt == ckx::DT_I8 ? k.i8 : k.f16)(g, (N + k.cols - 1) / k.cols, (hipStream_t)stream);
         return e == hipSuccess ? CKX_OK : hip_fail(e, k.name);
     }
     const TileInstance& t = kTiles[ti];

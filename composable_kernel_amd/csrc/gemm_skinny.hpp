@@ -1,8 +1,9 @@
 // Skinny GEMM for gfx950: C[M,N] = epilogue(A[M,K] * B[N,K]^T) with M <= 16*MT (a few token
 // rows against a large weight matrix), int8 or fp16, same layouts as the tile kernel.
 //
-// Such problems are bound by streaming B out of HBM exactly once. Each workgroup owns 16
-// output columns and the WHOLE K extent, split over its waves: a wave loads its K slice of
+// Such problems are bound by streaming B out of HBM exactly once. Each workgroup owns 16*NT
+// output columns (NT > 1: every A fragment, which comes out of L2, is used NT times) and the
+// WHOLE K extent, split over its waves: a wave loads its K slice of
 // the 16 B rows straight from global memory into registers in the MFMA operand layout (lane
 // l: row l%16, 16 bytes at k-step offset 16*(l/16)) -- there is no reuse across waves, so
 // there is no LDS staging -- multiplies it with the matching A fragments (read through L2),
@@ -14,17 +15,17 @@
 
 namespace ckx {
 
-template <int DT, int MT, int NW, int KU>
+template <int DT, int MT, int NW, int KU, int NT = 1>
 __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(const GemmArgs p)
 {
     using acc_t = typename std::conditional<DT == DT_I8, i32x4, f32x4>::type;
     constexpr int ES = DT == DT_I8 ? 1 : 2;
-    __shared__ acc_t red[NW][MT][64];
+    __shared__ acc_t red[NW][MT][NT][64];
 
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const uint32_t r = lane & 15, q = lane >> 4;
-    const int n0 = blockIdx.x * 16;
+    const int n0 = blockIdx.x * 16 * NT;
 
     const uint32_t kbytes = (uint32_t)p.K * ES;
     const int ksteps      = (int)((kbytes + 63u) >> 6);
@@ -35,49 +36,63 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(const GemmArgs p)
     const __amdgpu_buffer_rsrc_t rsrc_a = make_rsrc(p.a, p.a_bytes);
     const __amdgpu_buffer_rsrc_t rsrc_b = make_rsrc(p.b, p.b_bytes);
 
-    const uint32_t b_off = (uint32_t)n0 + r < (uint32_t)p.N ? ((uint32_t)n0 + r) * (uint32_t)p.ldb * ES + q * 16 : kOutOfRange;
+    uint32_t b_off[NT];
+#pragma unroll
+    for(int nt = 0; nt < NT; ++nt)
+    {
+        const uint32_t n = (uint32_t)n0 + 16u * nt + r;
+        b_off[nt]        = n < (uint32_t)p.N ? n * (uint32_t)p.ldb * ES + q * 16 : kOutOfRange;
+    }
     uint32_t a_off[MT];
 #pragma unroll
     for(int mt = 0; mt < MT; ++mt)
         a_off[mt] = 16u * mt + r < (uint32_t)p.M ? (16u * mt + r) * (uint32_t)p.lda * ES + q * 16 : kOutOfRange;
 
-    acc_t acc[MT];
+    acc_t acc[MT][NT];
 #pragma unroll
     for(int mt = 0; mt < MT; ++mt)
-        acc[mt] = acc_t{0, 0, 0, 0};
+#pragma unroll
+        for(int nt = 0; nt < NT; ++nt)
+            acc[mt][nt] = acc_t{0, 0, 0, 0};
 
     // one chunk = KU consecutive k-steps (64 bytes of K each); k-steps at or past ks_end and the
     // K tail read as zeros through an out-of-range buffer offset
-    auto load_chunk = [&](int ks0, i32x4(&bq)[KU], i32x4(&aq)[MT][KU]) {
+    auto load_chunk = [&](int ks0, i32x4(&bq)[NT][KU], i32x4(&aq)[MT][KU]) {
 #pragma unroll
         for(int u = 0; u < KU; ++u)
         {
             const int ks        = ks0 + u;
             const uint32_t kb   = (uint32_t)ks * 64u;
             const bool ok       = ks < ks_end && kb + q * 16 < kbytes;
-            bq[u] = __builtin_bit_cast(i32x4, __builtin_amdgcn_raw_buffer_load_b128(rsrc_b, ok ? b_off + kb : kOutOfRange, 0, 0));
+#pragma unroll
+            for(int nt = 0; nt < NT; ++nt)
+                bq[nt][u] = __builtin_bit_cast(
+                    i32x4, __builtin_amdgcn_raw_buffer_load_b128(rsrc_b, ok ? b_off[nt] + kb : kOutOfRange, 0, 0));
 #pragma unroll
             for(int mt = 0; mt < MT; ++mt)
                 aq[mt][u] = __builtin_bit_cast(
                     i32x4, __builtin_amdgcn_raw_buffer_load_b128(rsrc_a, ok ? a_off[mt] + kb : kOutOfRange, 0, 0));
         }
     };
-    auto mfma_chunk = [&](const i32x4(&bq)[KU], const i32x4(&aq)[MT][KU]) {
+    auto mfma_chunk = [&](const i32x4(&bq)[NT][KU], const i32x4(&aq)[MT][KU]) {
 #pragma unroll
         for(int u = 0; u < KU; ++u)
 #pragma unroll
             for(int mt = 0; mt < MT; ++mt)
-            {
-                if constexpr(DT == DT_I8)
-                    acc[mt] = __builtin_amdgcn_mfma_i32_16x16x64_i8(bq[u], aq[mt][u], acc[mt], 0, 0, 0);
-                else
-                    acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, bq[u]),
-                                                                    __builtin_bit_cast(f16x8, aq[mt][u]), acc[mt], 0,
-                                                                    0, 0);
-            }
+#pragma unroll
+                for(int nt = 0; nt < NT; ++nt)
+                {
+                    if constexpr(DT == DT_I8)
+                        acc[mt][nt] =
+                            __builtin_amdgcn_mfma_i32_16x16x64_i8(bq[nt][u], aq[mt][u], acc[mt][nt], 0, 0, 0);
+                    else
+                        acc[mt][nt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(
+                            __builtin_bit_cast(f16x8, bq[nt][u]), __builtin_bit_cast(f16x8, aq[mt][u]), acc[mt][nt],
+                            0, 0, 0);
+                }
     };
 
-    i32x4 b0[KU], a0[MT][KU], b1[KU], a1[MT][KU];
+    i32x4 b0[NT][KU], a0[MT][KU], b1[NT][KU], a1[MT][KU];
     load_chunk(ks_begin, b0, a0);
     for(int ks = ks_begin; ks < ks_end; ks += 2 * KU)
     {
@@ -90,23 +105,27 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(const GemmArgs p)
     // ---- sum the waves' partial tiles, then the epilogue on wave 0 ---------------------
 #pragma unroll
     for(int mt = 0; mt < MT; ++mt)
-        red[wave][mt][lane] = acc[mt];
-    __syncthreads();
-    if(wave != 0)
-        return;
 #pragma unroll
-    for(int mt = 0; mt < MT; ++mt)
+        for(int nt = 0; nt < NT; ++nt)
+            red[wave][mt][nt][lane] = acc[mt][nt];
+    __syncthreads();
+    // the (mt, nt) accumulator tiles are dealt round-robin to the waves for the final sum
+#pragma unroll
+    for(int t = 0; t < MT * NT; ++t)
     {
-        acc_t s = red[0][mt][lane];
+        if(t % NW != wave)
+            continue;
+        const int mt = t / NT, nt = t % NT;
+        acc_t s = red[0][mt][nt][lane];
 #pragma unroll
         for(int w = 1; w < NW; ++w)
         {
-            const acc_t v = red[w][mt][lane];
+            const acc_t v = red[w][mt][nt][lane];
             s[0] += v[0], s[1] += v[1], s[2] += v[2], s[3] += v[3];
         }
-        // lane (m = lane%16, q): columns n0 + 4q .. 4q+3 of row 16*mt + m
+        // lane (m = lane%16, q): columns 4q .. 4q+3 of the tile's 16, row 16*mt + m
         const int m  = 16 * mt + (int)r;
-        const int nn = n0 + 4 * (int)q;
+        const int nn = n0 + 16 * nt + 4 * (int)q;
         if(m >= p.M || nn >= p.N)
             continue;
         if constexpr(DT == DT_I8)

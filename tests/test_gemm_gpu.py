@@ -16,8 +16,8 @@ from oracle import fast, lit
 
 pytestmark = pytest.mark.gpu
 
-N_INSTANCES = 13        # tile instances followed by the skinny (few-row) instances
-SKINNY_MAX_M = {9: 16, 10: 32, 11: 64, 12: 16}
+N_INSTANCES = 17        # tile instances followed by the skinny (few-row) instances
+SKINNY_MAX_M = {9: 16, 10: 32, 11: 64, 12: 16, 13: 16, 14: 16, 15: 32, 16: 32}
 RTOL = ATOL = 1e-2
 
 EPILOGUES = {

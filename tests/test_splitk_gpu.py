@@ -120,3 +120,25 @@ def test_conv2d_split_k(force_split, dtype):
     else:
         bad, max_err = lit.check_err_f16(do.cpu().numpy(), lit.conv2d_fwd(inp, wei, s, d, p), 1e-2, 1e-2)
         assert bad == 0, max_err
+
+
+@pytest.mark.parametrize("shape", [(8, 10300, 256), (9, 10300, 256), (16, 5200, 192), (16, 1000, 320), (17, 10300, 128),
+                                   (32, 5200, 256), (33, 10300, 128), (48, 700, 4096), (64, 10304, 192), (65, 700, 2048)])
+def test_auto_instance_few_rows_routing_bit_exact(shape):
+    """Automatic choice for few-row problems: narrow / wide skinny instances up to 32 rows, skinny or
+    tile kernel (with a K split when the workspace is there) up to 64 rows. Every route must give
+    the reference's bits, with and without a workspace."""
+    import torch
+    import gpu_util
+    M, N, K = shape
+    a = uniform_int8((M, K), -8, 8, 90 + M)
+    b_nk = uniform_int8((N, K), -8, 8, 91 + N)
+    c_op = ck.RequantReluRequant(0.02, 0.4, rounded=True)
+    ref = fast.gemm_i8(a, b_nk.T, lit.EPI_REQUANT_RND, 0.02, 0.4)
+    out, _ = _run_gemm(ck.DeviceGemmInt8(), a, b_nk, torch.int8, c_op)
+    np.testing.assert_array_equal(out, ref)
+    np.testing.assert_array_equal(gpu_util.gemm_i8(a, b_nk, c_op), ref)       # no workspace
+    af, bf = uniform_f16((M, K), -1, 1, 92 + M), uniform_f16((N, K), -1, 1, 93 + N)
+    outf, _ = _run_gemm(ck.DeviceGemmF16(), af, bf, torch.float16)
+    reff = fast.gemm_f16(af, bf.T)
+    assert np.all(np.abs(outf.astype(np.float32) - reff.astype(np.float32)) <= 1e-2 + 1e-2 * np.abs(reff.astype(np.float32)))
