@@ -125,7 +125,7 @@ struct TileInstance
 const TileInstance kTiles[] = {
     CKX_TILE(256, 256, 2, 4, 2, 1.00f),
     CKX_TILE(256, 128, 4, 2, 2, 0.84f),
-    CKX_TILE(128, 128, 2, 2, 2, 0.78f),
+    CKX_TILE(128, 128, 2, 2, 2, 0.70f),
     CKX_TILE(128, 64, 4, 1, 2, 0.68f),
     CKX_TILE(64, 64, 4, 1, 2, 0.55f),
     CKX_TILE(32, 64, 2, 1, 2, 0.42f),
