@@ -35,19 +35,23 @@ HBM_PEAK_GBS = 8000.0
 MEASURED_TRAFFIC = {"fp16_gemm_4096": 2.350e8, "int8_requant_gemm_4096": 1.178e8}
 
 
-def _conv_workload(name, dtype, C, K, f, HW, st, pd, N=256):
+def _conv_workload(name, dtype, C, K, f, HW, st, pd, N=256, fused=None):
+    """fused: None, "bias_relu" or "bias_relu_add" (fp16: + bias[K], ReLU, + residual NHWK)."""
     Ho = (HW + 2 * pd - f) // st + 1
     ops = 2.0 * N * K * Ho * Ho * C * f * f
     es = 1 if dtype == "i8" else 2
     touched_in = N * HW * HW * C if st == 1 or f > 1 else N * Ho * Ho * C
-    byts = (touched_in + K * f * f * C + N * Ho * Ho * K) * es
-    return dict(name=name, kind="conv", dtype=dtype, N=N, C=C, K=K, f=f, HW=HW, st=st, pd=pd, ops=ops, bytes=byts)
+    out = N * Ho * Ho * K
+    byts = (touched_in + K * f * f * C + out + (K if fused else 0) + (out if fused == "bias_relu_add" else 0)) * es
+    return dict(name=name, kind="conv", dtype=dtype, N=N, C=C, K=K, f=f, HW=HW, st=st, pd=pd, ops=ops, bytes=byts,
+                fused=fused)
 
 
-def _gemm_workload(name, dtype, M, N, K, values=5, scales=(0.5, 0.03)):
+def _gemm_workload(name, dtype, M, N, K, values=5, scales=(0.5, 0.03), fused=None):
+    """fused: None or "bias_relu" (fp16: E = AddRelu(half(A*B), bias row))."""
     es = 1 if dtype == "i8" else 2
     return dict(name=name, kind="gemm", dtype=dtype, M=M, N=N, K=K, values=values, scales=scales,
-                ops=2.0 * M * N * K, bytes=(M * K + N * K + M * N) * es)
+                ops=2.0 * M * N * K, bytes=(M * K + N * K + M * N + (N if fused else 0)) * es, fused=fused)
 
 
 WORKLOADS = {}
@@ -60,6 +64,9 @@ for w in (
     + [_conv_workload(f"conv_{dt}_c64_k64_3x3_56", dt, 64, 64, 3, 56, 1, 1) for dt in ("f16", "i8")]
     + [_conv_workload(f"conv_{dt}_c256_k512_1x1_56_s2", dt, 256, 512, 1, 56, 2, 0) for dt in ("f16", "i8")]
     + [_conv_workload(f"conv_{dt}_c512_k512_3x3_7", dt, 512, 512, 3, 7, 1, 1) for dt in ("f16", "i8")]
+    + [_gemm_workload("fp16_gemm_bias_relu_4096", "f16", 4096, 4096, 4096, fused="bias_relu"),
+       _conv_workload("conv_f16_c64_k64_3x3_56_bias_relu_add", "f16", 64, 64, 3, 56, 1, 1, fused="bias_relu_add"),
+       _conv_workload("conv_f16_c256_k512_1x1_56_s2_bias_relu", "f16", 256, 512, 1, 56, 2, 0, fused="bias_relu")]
     + [dict(name="gemm_gemm_f16_b64_512x64x512x64", kind="gemm_gemm", dtype="f16", G=64, M=512, N=512, K=64, O=64,
             ops=2.0 * 64 * 512 * 512 * 64 * 2, bytes=4 * 64 * 512 * 64 * 2)]
 ):
@@ -94,12 +101,18 @@ def make_launcher(w, instance=-1, rotate=1):
             c = torch.empty((M, N), dtype=torch.float16, device="cuda")
             op = ck.DeviceGemmF16(instance)
             cop = ck.PassThrough()
-        arg = op.MakeArgumentPointer(a, b, c, M, N, K, K, K, N, None, None, cop)
+        if w.get("fused") == "bias_relu":
+            bias = dev(uniform_f16((N,), -1, 1, 9))
+            op = ck.DeviceGemmMultipleDF16(instance)
+            make = lambda bb: op.MakeArgumentPointer(a, bb, [bias], c, M, N, K, K, K, [0], N, None, None, ck.AddRelu())
+        else:
+            make = lambda bb: op.MakeArgumentPointer(a, bb, c, M, N, K, K, K, N, None, None, cop)
+        arg = make(b)
         more_args = []
         for _ in range(rotate - 1):
             b2 = b.clone()
             keep.append(b2)
-            more_args.append(op.MakeArgumentPointer(a, b2, c, M, N, K, K, K, N, None, None, cop))
+            more_args.append(make(b2))
     elif w["kind"] == "conv":
         N, C, K, f, HW, st, pd = (w[k] for k in ("N", "C", "K", "f", "HW", "st", "pd"))
         Ho = (HW + 2 * pd - f) // st + 1
@@ -113,8 +126,17 @@ def make_launcher(w, instance=-1, rotate=1):
             c = torch.empty((N, Ho, Ho, K), dtype=torch.float16, device="cuda")
             op = ck.DeviceConv2dFwdF16(instance)
             cop = ck.PassThrough()
-        arg = op.MakeArgumentPointer(i, wt, c, N, K, C, [HW, HW], [f, f], [Ho, Ho], [st, st], [1, 1], [pd, pd],
-                                     [pd, pd], None, None, cop)
+        geom = (N, K, C, [HW, HW], [f, f], [Ho, Ho], [st, st], [1, 1], [pd, pd], [pd, pd], None, None)
+        if w.get("fused"):
+            op = ck.DeviceConv2dFwdBiasActivationF16(instance)
+            bias = dev(uniform_f16((K,), -1, 1, 7))
+            if w["fused"] == "bias_relu_add":
+                resi = dev(uniform_f16((N, Ho, Ho, K), -1, 1, 8))
+                arg = op.MakeArgumentPointer(i, wt, c, bias, resi, *geom, ck.AddReluAdd())
+            else:
+                arg = op.MakeArgumentPointer(i, wt, c, bias, *geom, ck.AddRelu())
+        else:
+            arg = op.MakeArgumentPointer(i, wt, c, *geom, cop)
     else:
         G, M, N, K, O = (w[k] for k in ("G", "M", "N", "K", "O"))
         a, b0, b1 = (dev(uniform_f16(s, -0.5, 0.5, 5 + j)) for j, s in enumerate([(G, M, K), (G, N, K), (G, N, O)]))

@@ -14,6 +14,7 @@ LIB_PATH = os.environ.get("CKX_LIB_PATH") or os.path.join(HERE, "lib", "libckx.s
 OK, UNSUPPORTED, INVALID_VALUE, HIP_ERROR = 0, -1, -2, -3
 ROW_MAJOR, COL_MAJOR = 0, 1
 EPI_PASSTHROUGH, EPI_REQUANT_CK, EPI_REQUANT_RND = 0, 1, 2
+EPI_ADD_RELU, EPI_ADD_RELU_ADD, EPI_CSHUFFLE_ADD_RELU = 3, 4, 5
 OP_GEMM_I8, OP_GEMM_F16, OP_CONV2D_FWD_I8, OP_CONV2D_FWD_F16, OP_BATCHED_GEMM_GEMM = range(5)
 INSTANCE_AUTO = -1
 
@@ -22,6 +23,7 @@ SYMBOLS = [
     "ckx_version", "ckx_last_error", "ckx_num_instances", "ckx_instance_name",
     "ckx_gemm_i8_is_supported", "ckx_gemm_i8", "ckx_gemm_i8_workspace_bytes",
     "ckx_gemm_f16_is_supported", "ckx_gemm_f16", "ckx_gemm_f16_workspace_bytes",
+    "ckx_gemm_f16_multiple_d_is_supported", "ckx_gemm_f16_multiple_d", "ckx_conv2d_fwd_bias_activation_f16",
     "ckx_conv2d_fwd_is_supported", "ckx_conv2d_fwd_i8", "ckx_conv2d_fwd_f16", "ckx_conv2d_fwd_workspace_bytes",
     "ckx_batched_gemm_gemm_f16_is_supported", "ckx_batched_gemm_gemm_f16", "ckx_time_launches",
 ]
@@ -73,7 +75,11 @@ def lib():
         fn.argtypes = [i32, i32, i32, C.c_int]
     L.ckx_gemm_f16_is_supported.argtypes = shape + [C.c_int]
     L.ckx_gemm_f16.argtypes = [vp, vp, vp] + shape + [C.c_int, vp, i64, vp]
+    md = [i32] * 8 + [C.c_int] * 3
+    L.ckx_gemm_f16_multiple_d_is_supported.argtypes = md + [C.c_int, C.c_int]
+    L.ckx_gemm_f16_multiple_d.argtypes = [vp] * 5 + md + [C.c_int, C.c_int, vp, i64, vp]
     dp = C.POINTER(Conv2dDesc)
+    L.ckx_conv2d_fwd_bias_activation_f16.argtypes = [vp] * 5 + [dp, C.c_int, C.c_int, vp, i64, vp]
     L.ckx_conv2d_fwd_is_supported.argtypes = [C.c_int, dp, C.c_int, C.c_int]
     L.ckx_conv2d_fwd_i8.argtypes = [vp, vp, vp, dp, C.c_int, f32, f32, C.c_int, vp, i64, vp]
     L.ckx_conv2d_fwd_f16.argtypes = [vp, vp, vp, dp, C.c_int, vp, i64, vp]

@@ -252,6 +252,33 @@ const char* family_prefix(int op)
     }
 }
 
+// Operands of the fused add epilogues (fp16): D0 / D1 are [M,N] row-major, row strides in elements
+struct DOperands
+{
+    const void* d0 = nullptr;
+    const void* d1 = nullptr;
+    int ldd0 = 0, ldd1 = 0;
+};
+
+bool epilogue_fits_dtype(int es, int epi)
+{
+    if(es == 1)
+        return epi >= CKX_EPI_PASSTHROUGH && epi <= CKX_EPI_REQUANT_RND;
+    return epi == CKX_EPI_PASSTHROUGH || (epi >= CKX_EPI_ADD_RELU && epi <= CKX_EPI_CSHUFFLE_ADD_RELU);
+}
+
+int check_d_operands(int epi, int N, const DOperands& d)
+{
+    if(epi < CKX_EPI_ADD_RELU)
+        return CKX_OK;
+    if(!d.d0 || (epi == CKX_EPI_ADD_RELU_ADD && !d.d1))
+        return fail(CKX_INVALID_VALUE, "null D operand pointer");
+    if((d.ldd0 != 0 && d.ldd0 < N) || (epi == CKX_EPI_ADD_RELU_ADD && d.ldd1 != 0 && d.ldd1 < N) || d.ldd0 < 0 ||
+       d.ldd1 < 0)
+        return fail(CKX_UNSUPPORTED, "D stride must be 0 (broadcast row) or at least N");
+    return CKX_OK;
+}
+
 int check_gemm_shape(int dt, int M, int N, int K, int sa, int sb, int sc, int al, int bl, int cl, int epi,
                      int instance)
 {
@@ -262,10 +289,10 @@ int check_gemm_shape(int dt, int M, int N, int K, int sa, int sb, int sc, int al
         return fail(CKX_INVALID_VALUE, "no such instance");
     if(instance >= kNumTiles && M > kSkinny[instance - kNumTiles].max_m)
         return fail(CKX_UNSUPPORTED, "this skinny instance covers fewer rows than M");
-    if(epi < CKX_EPI_PASSTHROUGH || epi > CKX_EPI_REQUANT_RND)
+    if(epi < CKX_EPI_PASSTHROUGH || epi > CKX_EPI_CSHUFFLE_ADD_RELU)
         return fail(CKX_INVALID_VALUE, "unknown epilogue");
-    if(dt == ckx::DT_F16 && epi != CKX_EPI_PASSTHROUGH)
-        return fail(CKX_UNSUPPORTED, "fp16 GEMM only has the PassThrough epilogue");
+    if(!epilogue_fits_dtype(es, epi))
+        return fail(CKX_UNSUPPORTED, "epilogue not available for this dtype");
     if(al != CKX_ROW_MAJOR || bl != CKX_COL_MAJOR || cl != CKX_ROW_MAJOR)
         return fail(CKX_UNSUPPORTED, "only A row-major, B column-major, C row-major (mk_nk_mn) is built");
     if(sa < K || sb < K || sc < N)
@@ -289,10 +316,12 @@ long gemm_workspace_bytes(int dt, int M, int N, int K, int instance)
 
 int run_gemm(int dt, const void* a, const void* b, void* c, int M, int N, int K, int sa, int sb, int sc,
              int al, int bl, int cl, int epi, float sg, float sr, int instance, void* ws, long ws_bytes,
-             void* stream)
+             void* stream, const DOperands& dops = DOperands{})
 {
     int st = check_gemm_shape(dt, M, N, K, sa, sb, sc, al, bl, cl, epi, instance);
     if(st != CKX_OK)
+        return st;
+    if((st = check_d_operands(epi, N, dops)) != CKX_OK)
         return st;
     if(M == 0 || N == 0)
         return CKX_OK;
@@ -333,6 +362,8 @@ int run_gemm(int dt, const void* a, const void* b, void* c, int M, int N, int K,
     g.scale_gemm = sg;
     g.scale_relu = sr;
     g.nt_store   = es == 1 && (long)M * N * es >= stream_output_bytes();
+    g.d0 = dops.d0, g.d1 = epi == CKX_EPI_ADD_RELU_ADD ? dops.d1 : nullptr;
+    g.ldd0 = dops.ldd0, g.ldd1 = dops.ldd1;
     g.ksplit     = 1;
     if(ti >= kNumTiles)
     {
@@ -365,8 +396,9 @@ int check_conv(int op, const ckx_conv2d_desc* d, int epi, int instance)
     const int es = op == CKX_OP_CONV2D_FWD_I8 ? 1 : 2;
     if(instance != CKX_INSTANCE_AUTO && (instance < 0 || instance >= kNumTiles))
         return fail(CKX_INVALID_VALUE, "no such instance");
-    if(epi < CKX_EPI_PASSTHROUGH || epi > CKX_EPI_REQUANT_RND || (es == 2 && epi != CKX_EPI_PASSTHROUGH))
-        return fail(CKX_INVALID_VALUE, "epilogue not available for this dtype");
+    if(epi < CKX_EPI_PASSTHROUGH || epi > CKX_EPI_CSHUFFLE_ADD_RELU || !epilogue_fits_dtype(es, epi) ||
+       epi == CKX_EPI_CSHUFFLE_ADD_RELU)
+        return fail(CKX_INVALID_VALUE, "epilogue not available for this operator");
     if(d->N < 0 || d->K < 0 || d->C < 0 || d->Hi <= 0 || d->Wi <= 0 || d->Y <= 0 || d->X <= 0 ||
        d->Ho < 0 || d->Wo < 0 || d->stride_h <= 0 || d->stride_w <= 0 || d->dilation_h <= 0 ||
        d->dilation_w <= 0 || d->pad_top < 0 || d->pad_left < 0 || d->pad_bottom < 0 || d->pad_right < 0)
@@ -404,10 +436,12 @@ long conv_workspace_bytes(int op, const ckx_conv2d_desc* d, int instance)
 }
 
 int run_conv(int op, const void* in, const void* wei, void* out, const ckx_conv2d_desc* d, int epi, float sg,
-             float sr, int instance, void* ws, long ws_bytes, void* stream)
+             float sr, int instance, void* ws, long ws_bytes, void* stream, const DOperands& dops = DOperands{})
 {
     int st = check_conv(op, d, epi, instance);
     if(st != CKX_OK)
+        return st;
+    if((st = check_d_operands(epi, d->K, dops)) != CKX_OK)
         return st;
     const int es = op == CKX_OP_CONV2D_FWD_I8 ? 1 : 2;
     const int M = d->N * d->Ho * d->Wo, N = d->K, K = d->Y * d->X * d->C;
@@ -434,6 +468,8 @@ int run_conv(int op, const void* in, const void* wei, void* out, const ckx_conv2
     g.scale_gemm = sg;
     g.scale_relu = sr;
     g.nt_store   = es == 1 && (long)M * N * es >= stream_output_bytes();
+    g.d0 = dops.d0, g.d1 = epi == CKX_EPI_ADD_RELU_ADD ? dops.d1 : nullptr;
+    g.ldd0 = dops.ldd0, g.ldd1 = dops.ldd1;
     g.cv.Hi = d->Hi, g.cv.Wi = d->Wi, g.cv.C = d->C;
     g.cv.sH = d->stride_h, g.cv.sW = d->stride_w, g.cv.dH = d->dilation_h, g.cv.dW = d->dilation_w;
     g.cv.pT = d->pad_top, g.cv.pL = d->pad_left;
@@ -521,6 +557,46 @@ int ckx_gemm_f16(const void* a, const void* b, void* c, int32_t M, int32_t N, in
 {
     return run_gemm(ckx::DT_F16, a, b, c, M, N, K, sa, sb, sc, al, bl, cl, CKX_EPI_PASSTHROUGH, 1.0f, 1.0f,
                     instance, workspace, workspace_bytes, stream);
+}
+
+int ckx_gemm_f16_multiple_d_is_supported(int32_t M, int32_t N, int32_t K, int32_t sa, int32_t sb, int32_t sd0,
+                                         int32_t sd1, int32_t se, int al, int bl, int el, int cde_op, int instance)
+{
+    if(cde_op < CKX_EPI_ADD_RELU || cde_op > CKX_EPI_CSHUFFLE_ADD_RELU)
+        return fail(CKX_INVALID_VALUE, "not a CDE element-wise operation");
+    int st = check_gemm_shape(ckx::DT_F16, M, N, K, sa, sb, se, al, bl, el, cde_op, instance);
+    if(st != CKX_OK)
+        return st;
+    DOperands d;
+    d.d0 = d.d1 = &d; // only the strides are under test here
+    d.ldd0 = sd0, d.ldd1 = sd1;
+    return check_d_operands(cde_op, N, d);
+}
+
+int ckx_gemm_f16_multiple_d(const void* a, const void* b, const void* d0, const void* d1, void* e, int32_t M,
+                            int32_t N, int32_t K, int32_t sa, int32_t sb, int32_t sd0, int32_t sd1, int32_t se,
+                            int al, int bl, int el, int cde_op, int instance, void* workspace,
+                            int64_t workspace_bytes, void* stream)
+{
+    if(cde_op < CKX_EPI_ADD_RELU || cde_op > CKX_EPI_CSHUFFLE_ADD_RELU)
+        return fail(CKX_INVALID_VALUE, "not a CDE element-wise operation");
+    DOperands d;
+    d.d0 = d0, d.d1 = d1, d.ldd0 = sd0, d.ldd1 = sd1;
+    return run_gemm(ckx::DT_F16, a, b, e, M, N, K, sa, sb, se, al, bl, el, cde_op, 1.0f, 1.0f, instance, workspace,
+                    workspace_bytes, stream, d);
+}
+
+int ckx_conv2d_fwd_bias_activation_f16(const void* in, const void* wei, void* out, const void* bias,
+                                       const void* resi, const ckx_conv2d_desc* desc, int out_op, int instance,
+                                       void* workspace, int64_t workspace_bytes, void* stream)
+{
+    if(out_op != CKX_EPI_ADD_RELU && out_op != CKX_EPI_ADD_RELU_ADD)
+        return fail(CKX_INVALID_VALUE, "not a bias-activation output operation");
+    DOperands d;
+    d.d0 = bias, d.ldd0 = 0;
+    d.d1 = resi, d.ldd1 = desc ? desc->K : 0;
+    return run_conv(CKX_OP_CONV2D_FWD_F16, in, wei, out, desc, out_op, 1.0f, 1.0f, instance, workspace,
+                    workspace_bytes, stream, d);
 }
 
 int ckx_conv2d_fwd_is_supported(int op, const ckx_conv2d_desc* desc, int epilogue, int instance)

@@ -149,11 +149,19 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(const GemmArgs p)
         }
         else
         {
-            _Float16* crow = reinterpret_cast<_Float16*>(p.c) + (size_t)m * p.ldc + nn;
+            _Float16* crow       = reinterpret_cast<_Float16*>(p.c) + (size_t)m * p.ldc + nn;
+            const _Float16* d0row = reinterpret_cast<const _Float16*>(p.d0) + (size_t)m * p.ldd0 + nn;
+            const _Float16* d1row = reinterpret_cast<const _Float16*>(p.d1) + (size_t)m * p.ldd1 + nn;
 #pragma unroll
             for(int j = 0; j < 4; ++j)
                 if(nn + j < p.N)
-                    crow[j] = (_Float16)s[j];
+                {
+                    float val = s[j];
+                    if(p.epi != EPI_PASSTHROUGH)
+                        val = epi_f16_value(p.epi, val, (float)d0row[j],
+                                            p.epi == EPI_ADD_RELU_ADD ? (float)d1row[j] : 0.0f);
+                    crow[j] = (_Float16)val;
+                }
         }
     }
 }

@@ -46,7 +46,11 @@ enum
 {
     EPI_PASSTHROUGH = 0,
     EPI_REQUANT_CK  = 1,
-    EPI_REQUANT_RND = 2
+    EPI_REQUANT_RND = 2,
+    // fp16 outputs with extra "D" operands (bias row / residual tensor), all arithmetic in fp32:
+    EPI_ADD_RELU          = 3, // e = half(relu(acc + d0))
+    EPI_ADD_RELU_ADD      = 4, // e = half(relu(acc + d0) + d1)
+    EPI_CSHUFFLE_ADD_RELU = 5  // e = relu(half(half(acc) + d0)): C rounded to fp16 before the functor
 };
 
 #ifndef CKX_SWZ_SHIFT
@@ -111,6 +115,11 @@ struct GemmArgs
     // second kernel sums the slices and applies the epilogue. ksplit == 1: no workspace.
     int ksplit, nk_per;
     void* ws;
+    // fp16 "D" operands of the fused add epilogues, [M,N] row-major with row strides ldd0 / ldd1
+    // in elements (0: one row broadcast over M, i.e. a bias vector)
+    const void* d0;
+    const void* d1;
+    int ldd0, ldd1;
     ConvGeom cv;
 };
 
@@ -224,6 +233,28 @@ __device__ __forceinline__ void store_row16_i8(int8_t* crow, int n0, int N, bool
     }
 }
 
+// The fused add epilogues of the fp16 path (element-wise functors AddRelu / AddReluAdd of
+// include/ck/tensor_operation/gpu/element/{binary_,}element_wise_operation.hpp as the host
+// references apply them: reference_conv_fwd_bias_activation[_add].hpp on the fp32 accumulator,
+// example/03_gemm_bias_relu on the accumulator already rounded to fp16).
+__device__ __forceinline__ float epi_f16_value(int mode, float acc, float d0, float d1)
+{
+    if(mode == EPI_CSHUFFLE_ADD_RELU)
+    {
+        const float x = (float)(_Float16)((float)(_Float16)acc + d0);
+        return x > 0.0f ? x : 0.0f;
+    }
+    const float a = acc + d0;
+    const float b = a > 0.0f ? a : 0.0f;
+    return mode == EPI_ADD_RELU_ADD ? b + d1 : b;
+}
+
+// 16 consecutive fp16 outputs of one row with D operands; d0row / d1row point at column 0 of the
+// row's D values (d1row may be null)
+__device__ __forceinline__ void store_row16_f16_fused(_Float16* crow, int n0, int N, bool vec_ok, f32x4 (&v)[4],
+                                                      int mode, const _Float16* d0row, const _Float16* d1row,
+                                                      bool dvec_ok, bool nt);
+
 __device__ __forceinline__ void store_row16_f16(_Float16* crow, int n0, int N, bool vec_ok,
                                                 const f32x4 (&v)[4], bool nt = false)
 {
@@ -250,6 +281,43 @@ __device__ __forceinline__ void store_row16_f16(_Float16* crow, int n0, int N, b
                 if(n0 + t * 4 + j < N)
                     crow[n0 + t * 4 + j] = (_Float16)v[t][j];
     }
+}
+
+__device__ __forceinline__ void store_row16_f16_fused(_Float16* crow, int n0, int N, bool vec_ok, f32x4 (&v)[4],
+                                                      int mode, const _Float16* d0row, const _Float16* d1row,
+                                                      bool dvec_ok, bool nt)
+{
+    const bool has_d1 = mode == EPI_ADD_RELU_ADD;
+    if(dvec_ok && n0 + 16 <= N)
+    {
+        const f16x8 z   = {0, 0, 0, 0, 0, 0, 0, 0};
+        const f16x8 b_lo = *reinterpret_cast<const f16x8*>(d0row + n0);
+        const f16x8 b_hi = *reinterpret_cast<const f16x8*>(d0row + n0 + 8);
+        const f16x8 r_lo = has_d1 ? *reinterpret_cast<const f16x8*>(d1row + n0) : z;
+        const f16x8 r_hi = has_d1 ? *reinterpret_cast<const f16x8*>(d1row + n0 + 8) : z;
+#pragma unroll
+        for(int t = 0; t < 4; ++t)
+#pragma unroll
+            for(int j = 0; j < 4; ++j)
+            {
+                const int e = t * 4 + j;
+                v[t][j]     = epi_f16_value(mode, v[t][j], (float)(e < 8 ? b_lo[e] : b_hi[e - 8]),
+                                            (float)(e < 8 ? r_lo[e] : r_hi[e - 8]));
+            }
+    }
+    else
+    {
+#pragma unroll
+        for(int t = 0; t < 4; ++t)
+#pragma unroll
+            for(int j = 0; j < 4; ++j)
+            {
+                const int n = n0 + t * 4 + j;
+                if(n < N)
+                    v[t][j] = epi_f16_value(mode, v[t][j], (float)d0row[n], has_d1 ? (float)d1row[n] : 0.0f);
+            }
+    }
+    store_row16_f16(crow, n0, N, vec_ok, v, nt);
 }
 
 // Scheduling recipe for one half-iteration that also issues NL direct loads: NL groups of
@@ -556,6 +624,8 @@ struct GemmTile
         // ---- epilogue: registers -> global, 16 consecutive columns per lane -------------
         const bool vec_ok = ((reinterpret_cast<uintptr_t>(p.c) | ((uintptr_t)p.ldc * ES)) & 15u) == 0;
         const bool nt     = p.nt_store != 0;
+        const bool dvec_ok = ((reinterpret_cast<uintptr_t>(p.d0) | ((uintptr_t)p.ldd0 * ES) |
+                               reinterpret_cast<uintptr_t>(p.d1) | ((uintptr_t)p.ldd1 * ES)) & 15u) == 0;
         auto epilogue = [&](int unit) {
             int tm, tn;
             tile_of_block(unit % ntiles, p.tiles_m, p.tiles_n, tm, tn);
@@ -616,6 +686,103 @@ struct GemmTile
             }
         };
 
+        // Epilogue of the fused add / ReLU modes (fp16, no K split). A load issued after a store
+        // has to wait for that store as well (one counter, no ordering between the two kinds), so
+        // the D values are fetched in chunks of CH accumulator rows BEFORE any store of the chunk:
+        // a bias row once for the whole tile, per-row tensors (residual) chunk by chunk.
+        // (which tensors are per-row is a compile-time property of each variant: registers are only
+        // set aside for what is fetched)
+        auto epilogue_fused = [&](int unit, auto chunk_rows, auto d0_row_tensor, auto with_d1) {
+            constexpr int CH          = decltype(chunk_rows)::value < MT ? decltype(chunk_rows)::value : MT;
+            constexpr bool d0_per_row = decltype(d0_row_tensor)::value;
+            constexpr bool has_d1     = decltype(with_d1)::value;
+            int tm, tn;
+            tile_of_block(unit % ntiles, p.tiles_m, p.tiles_n, tm, tn);
+            const _Float16* d0 = reinterpret_cast<const _Float16*>(p.d0);
+            const _Float16* d1 = reinterpret_cast<const _Float16*>(p.d1);
+            const f16x8 zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
+            auto load16 = [&](const _Float16* row, int n0, f16x8& lo, f16x8& hi) {
+                if(dvec_ok && n0 + 16 <= p.N)
+                {
+                    lo = *reinterpret_cast<const f16x8*>(row + n0);
+                    hi = *reinterpret_cast<const f16x8*>(row + n0 + 8);
+                }
+                else
+                {
+#pragma unroll
+                    for(int e = 0; e < 8; ++e)
+                    {
+                        lo[e] = n0 + e < p.N ? row[n0 + e] : (_Float16)0;
+                        hi[e] = n0 + 8 + e < p.N ? row[n0 + 8 + e] : (_Float16)0;
+                    }
+                }
+            };
+            auto col0 = [&](int g) { return tn * BN + wn * WTN + 64 * g + 16 * (lane >> 4); };
+            f16x8 b_lo[NG], b_hi[NG];
+#pragma unroll
+            for(int g = 0; g < NG; ++g)
+            {
+                b_lo[g] = b_hi[g] = zero8;
+                if(!d0_per_row && col0(g) < p.N)
+                    load16(d0, col0(g), b_lo[g], b_hi[g]);
+            }
+#pragma unroll
+            for(int i0 = 0; i0 < MT; i0 += CH)
+            {
+                f16x8 x_lo[d0_per_row ? CH : 1][NG], x_hi[d0_per_row ? CH : 1][NG];
+                f16x8 y_lo[has_d1 ? CH : 1][NG], y_hi[has_d1 ? CH : 1][NG];
+#pragma unroll
+                for(int c = 0; c < CH; ++c)
+#pragma unroll
+                    for(int g = 0; g < NG; ++g)
+                    {
+                        const int m     = tm * BM + wm * WTM + 16 * (i0 + c) + (lane & 15);
+                        const bool live = m < p.M && col0(g) < p.N;
+                        if constexpr(d0_per_row)
+                        {
+                            x_lo[c][g] = x_hi[c][g] = zero8;
+                            if(live)
+                                load16(d0 + (size_t)m * p.ldd0, col0(g), x_lo[c][g], x_hi[c][g]);
+                        }
+                        if constexpr(has_d1)
+                        {
+                            y_lo[c][g] = y_hi[c][g] = zero8;
+                            if(live)
+                                load16(d1 + (size_t)m * p.ldd1, col0(g), y_lo[c][g], y_hi[c][g]);
+                        }
+                    }
+#pragma unroll
+                for(int c = 0; c < CH; ++c)
+#pragma unroll
+                    for(int g = 0; g < NG; ++g)
+                    {
+                        const int i = i0 + c;
+                        const int m = tm * BM + wm * WTM + 16 * i + (lane & 15);
+                        if(m < p.M && col0(g) < p.N)
+                        {
+                            f32x4 v[4];
+#pragma unroll
+                            for(int t = 0; t < 4; ++t)
+#pragma unroll
+                                for(int j = 0; j < 4; ++j)
+                                {
+                                    const int e   = t * 4 + j;
+                                    const int cx  = d0_per_row ? c : 0, cy = has_d1 ? c : 0;
+                                    const float x = d0_per_row ? (float)(e < 8 ? x_lo[cx][g][e & 7] : x_hi[cx][g][e & 7])
+                                                               : (float)(e < 8 ? b_lo[g][e & 7] : b_hi[g][e & 7]);
+                                    const float y = has_d1 ? (float)(e < 8 ? y_lo[cy][g][e & 7] : y_hi[cy][g][e & 7]) : 0.0f;
+                                    v[t][j]       = epi_f16_value(p.epi, acc[i][g * 4 + t][j], x, y);
+                                }
+                            _Float16* crow = reinterpret_cast<_Float16*>(p.c) + (size_t)m * p.ldc;
+                            store_row16_f16(crow, col0(g), p.N, vec_ok, v, nt);
+                        }
+#pragma unroll
+                        for(int t = 0; t < 4; ++t)
+                            acc[i][g * 4 + t] = acc_t{0, 0, 0, 0};
+                    }
+            }
+        };
+
         auto barrier = [&]() {
             __builtin_amdgcn_s_barrier();
             asm volatile("" ::: "memory");
@@ -669,7 +836,28 @@ struct GemmTile
             st_cur = st_next;
             if(++kt >= kt_end)
             {
-                epilogue(unit);
+                if constexpr(DT == DT_F16)
+                {
+                    if(p.epi == EPI_PASSTHROUGH || p.ksplit > 1)
+                        epilogue(unit);
+                    else
+                    {
+                        using std::integral_constant;
+                        using std::false_type;
+                        using std::true_type;
+                        const bool d0_rows = p.ldd0 != 0, resi = p.epi == EPI_ADD_RELU_ADD;
+                        if(!d0_rows && !resi)
+                            epilogue_fused(unit, integral_constant<int, MT>{}, false_type{}, false_type{});
+                        else if(!d0_rows)
+                            epilogue_fused(unit, integral_constant<int, 2>{}, false_type{}, true_type{});
+                        else if(!resi)
+                            epilogue_fused(unit, integral_constant<int, 2>{}, true_type{}, false_type{});
+                        else
+                            epilogue_fused(unit, integral_constant<int, 1>{}, true_type{}, true_type{});
+                    }
+                }
+                else
+                    epilogue(unit);
                 drain = true;
                 unit += gstride;
                 unit_k_range(unit, kt, kt_end);
@@ -733,7 +921,17 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(const GemmArgs p)
     else
     {
         _Float16* crow = reinterpret_cast<_Float16*>(p.c) + (size_t)m * p.ldc;
-        store_row16_f16(crow, n0, p.N, vec_ok, v);
+        if(p.epi == EPI_PASSTHROUGH)
+            store_row16_f16(crow, n0, p.N, vec_ok, v);
+        else
+        {
+            const bool dvec_ok = ((reinterpret_cast<uintptr_t>(p.d0) | ((uintptr_t)p.ldd0 * ES) |
+                                   reinterpret_cast<uintptr_t>(p.d1) | ((uintptr_t)p.ldd1 * ES)) & 15u) == 0;
+            store_row16_f16_fused(crow, n0, p.N, vec_ok, v, p.epi,
+                                  reinterpret_cast<const _Float16*>(p.d0) + (size_t)m * p.ldd0,
+                                  p.d1 ? reinterpret_cast<const _Float16*>(p.d1) + (size_t)m * p.ldd1 : nullptr,
+                                  dvec_ok, false);
+        }
     }
 }
 

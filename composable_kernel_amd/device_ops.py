@@ -41,6 +41,21 @@ class RequantReluRequant:
         self.epilogue = capi.EPI_REQUANT_RND if rounded else capi.EPI_REQUANT_CK
 
 
+class AddRelu:
+    """element_wise::AddRelu (binary_element_wise_operation.hpp:118-146): y = relu(x0 + x1).
+    As an OutElementwiseOperation of the conv operators it acts on the fp32 accumulator
+    (reference_conv_fwd_bias_activation.hpp:118-120); as the CDE operation of DeviceGemmMultipleD it
+    acts on C already rounded to fp16 (example/03_gemm_bias_relu/gemm_bias_relu_xdl_fp16.cpp:31-40)."""
+    epilogue = capi.EPI_ADD_RELU
+    cde_epilogue = capi.EPI_CSHUFFLE_ADD_RELU
+
+
+class AddReluAdd:
+    """element_wise::AddReluAdd (element_wise_operation.hpp:46-81): y = relu(x0 + x1) + x2 in fp32."""
+    epilogue = capi.EPI_ADD_RELU_ADD
+    cde_epilogue = capi.EPI_ADD_RELU_ADD
+
+
 class RowMajor:
     code = capi.ROW_MAJOR
 
@@ -189,6 +204,42 @@ class DeviceGemmF16(_DeviceGemm):
                                        C.c_void_p(stream or 0))
 
 
+class DeviceGemmMultipleDF16(BaseOperator):
+    """DeviceGemmMultipleD<Row, Col, Row, half_t, half_t, Tuple<half_t[, half_t]>, half_t, PassThrough,
+    PassThrough, CDEOp> (device_gemm_multiple_d.hpp:14-55): E = cde_op(A*B, D0[, D1])."""
+    op_family = capi.OP_GEMM_F16
+
+    def __init__(self, instance=capi.INSTANCE_AUTO, ALayout=RowMajor, BLayout=ColumnMajor, DELayout=RowMajor):
+        super().__init__(instance)
+        self.layouts = (ALayout.code, BLayout.code, DELayout.code)
+
+    def MakeArgumentPointer(self, p_a, p_b, p_ds, p_e, M, N, K, StrideA, StrideB, StrideDs, StrideE,
+                            a_element_op=None, b_element_op=None, cde_element_op=None):
+        if not 1 <= len(p_ds) <= 2 or len(StrideDs) != len(p_ds):
+            raise ValueError("one or two D tensors")
+        if not isinstance(cde_element_op, (AddRelu, AddReluAdd)):
+            raise TypeError("CDE element-wise operation not built")
+        a = _GemmArgument(p_a, p_b, p_e, M, N, K, StrideA, StrideB, StrideE, a_element_op or PassThrough(),
+                          b_element_op or PassThrough(), cde_element_op, self.layouts)
+        a.p_ds = [_ptr(p) for p in p_ds] + [0] * (2 - len(p_ds))
+        a.StrideDs = [int(x) for x in StrideDs] + [0] * (2 - len(p_ds))
+        return a
+
+    def _supported(self, a):
+        return capi.lib().ckx_gemm_f16_multiple_d_is_supported(
+            a.M, a.N, a.K, a.StrideA, a.StrideB, a.StrideDs[0], a.StrideDs[1], a.StrideC, *self.layouts,
+            a.c_op.cde_epilogue, self.instance)
+
+    def GetWorkSpaceSize(self, a):
+        return int(capi.lib().ckx_gemm_f16_workspace_bytes(a.M, a.N, a.K, self.instance))
+
+    def _launch(self, a, stream):
+        return capi.lib().ckx_gemm_f16_multiple_d(
+            a.p_a, a.p_b, a.p_ds[0], a.p_ds[1], a.p_c, a.M, a.N, a.K, a.StrideA, a.StrideB, a.StrideDs[0],
+            a.StrideDs[1], a.StrideC, *self.layouts, a.c_op.cde_epilogue, self.instance, a.p_workspace_ or 0,
+            a.workspace_bytes_, C.c_void_p(stream or 0))
+
+
 # -------------------------------------------------------------------- conv
 class _ConvArgument(BaseArgument):
     def __init__(self, p_in, p_wei, p_out, desc, out_op):
@@ -236,6 +287,31 @@ class DeviceConv2dFwdF16(_DeviceConvFwd):
     def _launch(self, a, stream):
         return capi.lib().ckx_conv2d_fwd_f16(a.p_in, a.p_wei, a.p_out, C.byref(a.desc), self.instance,
                                              a.p_workspace_ or 0, a.workspace_bytes_, C.c_void_p(stream or 0))
+
+
+class DeviceConv2dFwdBiasActivationF16(_DeviceConvFwd):
+    """DeviceConvFwdBiasActivation<InOp, WeiOp, AddRelu> and DeviceConvFwdBiasActivationAdd<..., AddReluAdd>
+    (device_conv_fwd_bias_activation.hpp:18-41, device_conv_fwd_bias_activation_add.hpp): p_bias is a
+    [K] vector; p_resi (NHWK, like the output) is given for the Add form only."""
+    op_family = capi.OP_CONV2D_FWD_F16
+
+    def MakeArgumentPointer(self, p_in, p_wei, p_out, p_bias, *rest):
+        # (p_resi,) N, K, C, spatial vectors..., element-wise operations: the Add form has one more pointer
+        p_resi = None
+        if len(rest) == 14:
+            p_resi, rest = rest[0], rest[1:]
+        if len(rest) != 13:
+            raise TypeError("expected N, K, C, 7 vectors and 3 element-wise operations")
+        a = super().MakeArgumentPointer(p_in, p_wei, p_out, *rest)
+        if not isinstance(a.out_op, (AddRelu, AddReluAdd)) or isinstance(a.out_op, AddReluAdd) != (p_resi is not None):
+            raise TypeError("out_element_op must be AddRelu (no residual) or AddReluAdd (with residual)")
+        a.p_bias, a.p_resi = _ptr(p_bias), _ptr(p_resi)
+        return a
+
+    def _launch(self, a, stream):
+        return capi.lib().ckx_conv2d_fwd_bias_activation_f16(
+            a.p_in, a.p_wei, a.p_out, a.p_bias, a.p_resi, C.byref(a.desc), a.out_op.epilogue, self.instance,
+            a.p_workspace_ or 0, a.workspace_bytes_, C.c_void_p(stream or 0))
 
 
 # --------------------------------------------------------------- GEMM-GEMM

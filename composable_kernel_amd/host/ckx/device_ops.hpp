@@ -23,6 +23,7 @@
 #include <hip/hip_runtime.h>
 
 #include <cstdint>
+#include <array>
 #include <memory>
 #include <sstream>
 #include <stdexcept>
@@ -106,8 +107,38 @@ struct RequantRoundReluRequantRound
     float scaleGemm_, scaleRelu_;
 };
 
+// y = relu(x0 + x1) (binary_element_wise_operation.hpp:118-146). On the conv operators x0 is the
+// fp32 accumulator; as the CDE operation of DeviceGemmMultipleD x0 is C already rounded to fp16.
+struct AddRelu
+{
+    template <typename Y, typename X0, typename X1>
+    void operator()(Y& y, const X0& x0, const X1& x1) const
+    {
+        const Y a = static_cast<Y>(x0 + x1);
+        y         = a > Y(0) ? a : Y(0);
+    }
+};
+
+// y = relu(x0 + x1) + x2 in fp32 (element_wise_operation.hpp:46-81)
+struct AddReluAdd
+{
+    template <typename Y, typename X0, typename X1, typename X2>
+    void operator()(Y& y, const X0& x0, const X1& x1, const X2& x2) const
+    {
+        const float a = static_cast<float>(x0) + static_cast<float>(x1);
+        y             = static_cast<Y>((a > 0 ? a : 0) + static_cast<float>(x2));
+    }
+};
+
 } // namespace element_wise
 } // namespace tensor_operation
+
+// ck::Tuple as a type list (include/ck/utility/tuple.hpp): only Size() is needed here
+template <typename... Ts>
+struct Tuple
+{
+    static constexpr index_t Size() { return sizeof...(Ts); }
+};
 } // namespace ck
 
 namespace ckx {
@@ -221,6 +252,51 @@ struct DeviceBatchedGemmGemm : public BaseOperator
                         B0ElementwiseOperation b0_element_op, Acc0ElementwiseOperation acc0_element_op,
                         B1ElementwiseOperation b1_element_op, CElementwiseOperation c_element_op) = 0;
     virtual std::unique_ptr<BaseInvoker> MakeInvokerPointer()                                     = 0;
+};
+
+// device_gemm_multiple_d.hpp:14-55
+template <typename ALayout, typename BLayout, typename DELayout, typename ADataType, typename BDataType,
+          typename DsDataType, typename EDataType, typename AElementwiseOperation, typename BElementwiseOperation,
+          typename CDEElementwiseOperation>
+struct DeviceGemmMultipleD : public BaseOperator
+{
+    static constexpr index_t NumDTensor = DsDataType::Size();
+    virtual std::unique_ptr<BaseArgument>
+    MakeArgumentPointer(const void* p_a, const void* p_b, std::array<const void*, NumDTensor> p_ds, void* p_e,
+                        index_t M, index_t N, index_t K, index_t StrideA, index_t StrideB,
+                        std::array<index_t, NumDTensor> StrideDs, index_t StrideE, AElementwiseOperation a_element_op,
+                        BElementwiseOperation b_element_op, CDEElementwiseOperation cde_element_op) = 0;
+    virtual std::unique_ptr<BaseInvoker> MakeInvokerPointer()                                       = 0;
+};
+
+// device_conv_fwd_bias_activation.hpp:18-41
+template <typename InElementwiseOperation, typename WeiElementwiseOperation, typename OutElementwiseOperation>
+struct DeviceConvFwdBiasActivation : public BaseOperator
+{
+    virtual std::unique_ptr<BaseArgument>
+    MakeArgumentPointer(const void* p_in, const void* p_wei, void* p_out, const void* p_bias, index_t N, index_t K,
+                        index_t C, std::vector<index_t> input_spatial_lengths,
+                        std::vector<index_t> filter_spatial_lengths, std::vector<index_t> output_spatial_lengths,
+                        std::vector<index_t> conv_filter_strides, std::vector<index_t> conv_filter_dilations,
+                        std::vector<index_t> input_left_pads, std::vector<index_t> input_right_pads,
+                        InElementwiseOperation in_element_op, WeiElementwiseOperation wei_element_op,
+                        OutElementwiseOperation out_element_op) = 0;
+    virtual std::unique_ptr<BaseInvoker> MakeInvokerPointer()  = 0;
+};
+
+// device_conv_fwd_bias_activation_add.hpp
+template <typename InElementwiseOperation, typename WeiElementwiseOperation, typename OutElementwiseOperation>
+struct DeviceConvFwdBiasActivationAdd : public BaseOperator
+{
+    virtual std::unique_ptr<BaseArgument>
+    MakeArgumentPointer(const void* p_in, const void* p_wei, void* p_out, const void* p_bias, const void* p_resi,
+                        index_t N, index_t K, index_t C, std::vector<index_t> input_spatial_lengths,
+                        std::vector<index_t> filter_spatial_lengths, std::vector<index_t> output_spatial_lengths,
+                        std::vector<index_t> conv_filter_strides, std::vector<index_t> conv_filter_dilations,
+                        std::vector<index_t> input_left_pads, std::vector<index_t> input_right_pads,
+                        InElementwiseOperation in_element_op, WeiElementwiseOperation wei_element_op,
+                        OutElementwiseOperation out_element_op) = 0;
+    virtual std::unique_ptr<BaseInvoker> MakeInvokerPointer()  = 0;
 };
 
 // ------------------------------------------------------------------- common invoker
@@ -476,6 +552,233 @@ struct DeviceConv2dFwdMfma_Input_N_Hi_Wi_C_Weight_K_Y_X_C_Output_N_Ho_Wo_K
     int instance_;
 };
 
+// ------------------------------------------------ GEMM with fused D operands (fp16)
+// CDE operation: AddRelu (one D: E = relu(half(C) + D0), example 03) or AddReluAdd (two Ds:
+// E = relu(C + D0) + D1 in fp32). A D stride of 0 broadcasts one row (a bias vector).
+template <typename ALayout, typename BLayout, typename DELayout, typename DsDataType,
+          typename CDEElementwiseOperation>
+struct DeviceGemmMultipleDMfma
+    : public DeviceGemmMultipleD<ALayout, BLayout, DELayout, half_t, half_t, DsDataType, half_t,
+                                 element_wise::PassThrough, element_wise::PassThrough, CDEElementwiseOperation>
+{
+    static constexpr index_t NumDTensor = DsDataType::Size();
+    static constexpr bool is_add_relu   = std::is_same_v<CDEElementwiseOperation, element_wise::AddRelu>;
+    static_assert((is_add_relu && NumDTensor == 1) ||
+                      (std::is_same_v<CDEElementwiseOperation, element_wise::AddReluAdd> && NumDTensor == 2),
+                  "built CDE operations: AddRelu with one D tensor, AddReluAdd with two");
+    static constexpr int cde_code = is_add_relu ? CKX_EPI_CSHUFFLE_ADD_RELU : CKX_EPI_ADD_RELU_ADD;
+    using Pass                    = element_wise::PassThrough;
+
+    struct Argument : public BaseArgument
+    {
+        const void *p_a, *p_b, *p_d0, *p_d1;
+        void* p_e;
+        index_t M, N, K, StrideA, StrideB, StrideD0, StrideD1, StrideE;
+    };
+    static int Supported(const Argument& a, int inst)
+    {
+        return ckx_gemm_f16_multiple_d_is_supported(a.M, a.N, a.K, a.StrideA, a.StrideB, a.StrideD0, a.StrideD1,
+                                                    a.StrideE, ALayout::code, BLayout::code, DELayout::code,
+                                                    cde_code, inst);
+    }
+    static int Launch(const Argument& a, int inst, void* stream)
+    {
+        const int64_t ws_bytes = a.p_workspace_ ? ckx_gemm_f16_workspace_bytes(a.M, a.N, a.K, inst) : 0;
+        return ckx_gemm_f16_multiple_d(a.p_a, a.p_b, a.p_d0, a.p_d1, a.p_e, a.M, a.N, a.K, a.StrideA, a.StrideB,
+                                       a.StrideD0, a.StrideD1, a.StrideE, ALayout::code, BLayout::code,
+                                       DELayout::code, cde_code, inst, a.p_workspace_, ws_bytes, stream);
+    }
+    using Invoker = detail::InvokerT<Argument, &Supported, &Launch>;
+
+    explicit DeviceGemmMultipleDMfma(int instance = CKX_INSTANCE_AUTO) : instance_(instance) {}
+    static Argument MakeArgument(const void* p_a, const void* p_b, std::array<const void*, NumDTensor> p_ds,
+                                 void* p_e, index_t M, index_t N, index_t K, index_t StrideA, index_t StrideB,
+                                 std::array<index_t, NumDTensor> StrideDs, index_t StrideE, Pass = {}, Pass = {},
+                                 CDEElementwiseOperation = {})
+    {
+        Argument a;
+        a.p_a = p_a, a.p_b = p_b, a.p_e = p_e;
+        a.p_d0 = p_ds[0], a.StrideD0 = StrideDs[0];
+        a.p_d1 = NumDTensor > 1 ? p_ds[NumDTensor - 1] : nullptr, a.StrideD1 = NumDTensor > 1 ? StrideDs[NumDTensor - 1] : 0;
+        a.M = M, a.N = N, a.K = K, a.StrideA = StrideA, a.StrideB = StrideB, a.StrideE = StrideE;
+        return a;
+    }
+    Invoker MakeInvoker() const { return Invoker{instance_}; }
+    bool IsSupportedArgument(const Argument& a) const { return Supported(a, instance_) == CKX_OK; }
+    bool IsSupportedArgument(const BaseArgument* p) override
+    {
+        const auto* a = dynamic_cast<const Argument*>(p);
+        return a && IsSupportedArgument(*a);
+    }
+    size_t GetWorkSpaceSize(const BaseArgument* p) const override
+    {
+        const auto* a = dynamic_cast<const Argument*>(p);
+        return a ? (size_t)ckx_gemm_f16_workspace_bytes(a->M, a->N, a->K, instance_) : 0;
+    }
+    std::unique_ptr<BaseArgument>
+    MakeArgumentPointer(const void* p_a, const void* p_b, std::array<const void*, NumDTensor> p_ds, void* p_e,
+                        index_t M, index_t N, index_t K, index_t StrideA, index_t StrideB,
+                        std::array<index_t, NumDTensor> StrideDs, index_t StrideE, Pass, Pass,
+                        CDEElementwiseOperation) override
+    {
+        return std::make_unique<Argument>(MakeArgument(p_a, p_b, p_ds, p_e, M, N, K, StrideA, StrideB, StrideDs, StrideE));
+    }
+    std::unique_ptr<BaseInvoker> MakeInvokerPointer() override { return std::make_unique<Invoker>(instance_); }
+    std::string GetTypeString() const override
+    {
+        const std::string base = instance_ == CKX_INSTANCE_AUTO ? std::string("DeviceGemm_f16_f16_f16_mk_nk_mn<auto>")
+                                                                : std::string(ckx_instance_name(CKX_OP_GEMM_F16, instance_));
+        return base + (is_add_relu ? " + AddRelu" : " + AddReluAdd");
+    }
+    int instance_;
+};
+
+// ------------------------------------------ conv2d fwd + bias + ReLU (+ residual), fp16
+namespace detail {
+struct ConvBiasArgument : public BaseArgument
+{
+    const void *p_in, *p_wei, *p_bias, *p_resi;
+    void* p_out;
+    ckx_conv2d_desc desc;
+    bool two_d;
+    int out_op;
+    ConvBiasArgument(const void* in, const void* wei, void* out, const void* bias, const void* resi, int op,
+                     index_t N, index_t K, index_t C, const std::vector<index_t>& isp,
+                     const std::vector<index_t>& fsp, const std::vector<index_t>& osp, const std::vector<index_t>& st,
+                     const std::vector<index_t>& dl, const std::vector<index_t>& lp, const std::vector<index_t>& rp)
+        : p_in(in), p_wei(wei), p_bias(bias), p_resi(resi), p_out(out), desc{}, out_op(op)
+    {
+        two_d = isp.size() == 2 && fsp.size() == 2 && osp.size() == 2 && st.size() == 2 && dl.size() == 2 &&
+                lp.size() == 2 && rp.size() == 2;
+        if(two_d)
+            desc = ckx_conv2d_desc{N,     K,     C,     isp[0], isp[1], fsp[0], fsp[1], osp[0], osp[1],
+                                   st[0], st[1], dl[0], dl[1],  lp[0],  lp[1],  rp[0],  rp[1]};
+    }
+};
+inline int conv_bias_supported(const ConvBiasArgument& a, int inst)
+{
+    return a.two_d ? ckx_conv2d_fwd_is_supported(CKX_OP_CONV2D_FWD_F16, &a.desc, a.out_op, inst) : CKX_UNSUPPORTED;
+}
+inline int conv_bias_launch(const ConvBiasArgument& a, int inst, void* stream)
+{
+    const int64_t ws_bytes = a.p_workspace_ ? ckx_conv2d_fwd_workspace_bytes(CKX_OP_CONV2D_FWD_F16, &a.desc, inst) : 0;
+    return ckx_conv2d_fwd_bias_activation_f16(a.p_in, a.p_wei, a.p_out, a.p_bias, a.p_resi, &a.desc, a.out_op, inst,
+                                              a.p_workspace_, ws_bytes, stream);
+}
+using ConvBiasInvoker = InvokerT<ConvBiasArgument, &conv_bias_supported, &conv_bias_launch>;
+
+// what the two operators share; Derived supplies the interface base class
+template <typename Base>
+struct ConvBiasCommon : public Base
+{
+    using Argument = ConvBiasArgument;
+    using Invoker  = ConvBiasInvoker;
+    explicit ConvBiasCommon(int instance) : instance_(instance) {}
+    Invoker MakeInvoker() const { return Invoker{instance_}; }
+    bool IsSupportedArgument(const Argument& a) const { return conv_bias_supported(a, instance_) == CKX_OK; }
+    bool IsSupportedArgument(const BaseArgument* p) override
+    {
+        const auto* a = dynamic_cast<const Argument*>(p);
+        return a && IsSupportedArgument(*a);
+    }
+    size_t GetWorkSpaceSize(const BaseArgument* p) const override
+    {
+        const auto* a = dynamic_cast<const Argument*>(p);
+        return a && a->two_d ? (size_t)ckx_conv2d_fwd_workspace_bytes(CKX_OP_CONV2D_FWD_F16, &a->desc, instance_) : 0;
+    }
+    std::unique_ptr<BaseInvoker> MakeInvokerPointer() override { return std::make_unique<Invoker>(instance_); }
+    int instance_;
+};
+} // namespace detail
+
+// DeviceConv2dFwdXdl_C_Shuffle_Bias_Activation_Input_N_Hi_Wi_C_Weight_K_Y_X_C_Output_N_Ho_Wo_K (example 06)
+template <typename InElementwiseOperation = element_wise::PassThrough,
+          typename WeiElementwiseOperation = element_wise::PassThrough,
+          typename OutElementwiseOperation = element_wise::AddRelu>
+struct DeviceConv2dFwdBiasActivationMfma_Input_N_Hi_Wi_C_Weight_K_Y_X_C_Output_N_Ho_Wo_K
+    : public detail::ConvBiasCommon<
+          DeviceConvFwdBiasActivation<InElementwiseOperation, WeiElementwiseOperation, OutElementwiseOperation>>
+{
+    static_assert(std::is_same_v<OutElementwiseOperation, element_wise::AddRelu>, "built output operation: AddRelu");
+    using Common = detail::ConvBiasCommon<
+        DeviceConvFwdBiasActivation<InElementwiseOperation, WeiElementwiseOperation, OutElementwiseOperation>>;
+    using Argument = detail::ConvBiasArgument;
+    explicit DeviceConv2dFwdBiasActivationMfma_Input_N_Hi_Wi_C_Weight_K_Y_X_C_Output_N_Ho_Wo_K(
+        int instance = CKX_INSTANCE_AUTO)
+        : Common(instance)
+    {
+    }
+    static Argument MakeArgument(const half_t* p_in, const half_t* p_wei, half_t* p_out, const half_t* p_bias,
+                                 index_t N, index_t K, index_t C, std::vector<index_t> isp, std::vector<index_t> fsp,
+                                 std::vector<index_t> osp, std::vector<index_t> st, std::vector<index_t> dl,
+                                 std::vector<index_t> lp, std::vector<index_t> rp, InElementwiseOperation = {},
+                                 WeiElementwiseOperation = {}, OutElementwiseOperation = {})
+    {
+        return Argument{p_in, p_wei, p_out, p_bias, nullptr, CKX_EPI_ADD_RELU, N, K, C, isp, fsp, osp, st, dl, lp, rp};
+    }
+    std::unique_ptr<BaseArgument>
+    MakeArgumentPointer(const void* p_in, const void* p_wei, void* p_out, const void* p_bias, index_t N, index_t K,
+                        index_t C, std::vector<index_t> isp, std::vector<index_t> fsp, std::vector<index_t> osp,
+                        std::vector<index_t> st, std::vector<index_t> dl, std::vector<index_t> lp,
+                        std::vector<index_t> rp, InElementwiseOperation, WeiElementwiseOperation,
+                        OutElementwiseOperation) override
+    {
+        return std::make_unique<Argument>(p_in, p_wei, p_out, p_bias, nullptr, CKX_EPI_ADD_RELU, N, K, C, isp, fsp, osp,
+                                          st, dl, lp, rp);
+    }
+    std::string GetTypeString() const override
+    {
+        return (this->instance_ == CKX_INSTANCE_AUTO ? std::string("DeviceConv2dFwd_f16_nhwc_kyxc_nhwk<auto>")
+                                                     : std::string(ckx_instance_name(CKX_OP_CONV2D_FWD_F16, this->instance_))) +
+               " + Bias + AddRelu";
+    }
+};
+
+// ..._Bias_Activation_Add_... (example 07)
+template <typename InElementwiseOperation = element_wise::PassThrough,
+          typename WeiElementwiseOperation = element_wise::PassThrough,
+          typename OutElementwiseOperation = element_wise::AddReluAdd>
+struct DeviceConv2dFwdBiasActivationAddMfma_Input_N_Hi_Wi_C_Weight_K_Y_X_C_Output_N_Ho_Wo_K
+    : public detail::ConvBiasCommon<
+          DeviceConvFwdBiasActivationAdd<InElementwiseOperation, WeiElementwiseOperation, OutElementwiseOperation>>
+{
+    static_assert(std::is_same_v<OutElementwiseOperation, element_wise::AddReluAdd>,
+                  "built output operation: AddReluAdd");
+    using Common = detail::ConvBiasCommon<
+        DeviceConvFwdBiasActivationAdd<InElementwiseOperation, WeiElementwiseOperation, OutElementwiseOperation>>;
+    using Argument = detail::ConvBiasArgument;
+    explicit DeviceConv2dFwdBiasActivationAddMfma_Input_N_Hi_Wi_C_Weight_K_Y_X_C_Output_N_Ho_Wo_K(
+        int instance = CKX_INSTANCE_AUTO)
+        : Common(instance)
+    {
+    }
+    static Argument MakeArgument(const half_t* p_in, const half_t* p_wei, half_t* p_out, const half_t* p_bias,
+                                 const half_t* p_resi, index_t N, index_t K, index_t C, std::vector<index_t> isp,
+                                 std::vector<index_t> fsp, std::vector<index_t> osp, std::vector<index_t> st,
+                                 std::vector<index_t> dl, std::vector<index_t> lp, std::vector<index_t> rp,
+                                 InElementwiseOperation = {}, WeiElementwiseOperation = {},
+                                 OutElementwiseOperation = {})
+    {
+        return Argument{p_in, p_wei, p_out, p_bias, p_resi, CKX_EPI_ADD_RELU_ADD, N, K, C, isp, fsp, osp, st, dl, lp, rp};
+    }
+    std::unique_ptr<BaseArgument>
+    MakeArgumentPointer(const void* p_in, const void* p_wei, void* p_out, const void* p_bias, const void* p_resi,
+                        index_t N, index_t K, index_t C, std::vector<index_t> isp, std::vector<index_t> fsp,
+                        std::vector<index_t> osp, std::vector<index_t> st, std::vector<index_t> dl,
+                        std::vector<index_t> lp, std::vector<index_t> rp, InElementwiseOperation,
+                        WeiElementwiseOperation, OutElementwiseOperation) override
+    {
+        return std::make_unique<Argument>(p_in, p_wei, p_out, p_bias, p_resi, CKX_EPI_ADD_RELU_ADD, N, K, C, isp, fsp,
+                                          osp, st, dl, lp, rp);
+    }
+    std::string GetTypeString() const override
+    {
+        return (this->instance_ == CKX_INSTANCE_AUTO ? std::string("DeviceConv2dFwd_f16_nhwc_kyxc_nhwk<auto>")
+                                                     : std::string(ckx_instance_name(CKX_OP_CONV2D_FWD_F16, this->instance_))) +
+               " + Bias + AddReluAdd";
+    }
+};
+
 // -------------------------------------------------------------------- GEMM-GEMM
 template <typename AElementwiseOperation = element_wise::PassThrough,
           typename B0ElementwiseOperation = element_wise::PassThrough,
@@ -593,6 +896,52 @@ std::vector<std::unique_ptr<DeviceConvFwd<InOp, WeiOp, OutOp>>> GetConv2dFwdInst
             i));
     return v;
 }
+
+// instance lists of the fused operators: one per tile configuration (the skinny GEMM instances
+// are included for DeviceGemmMultipleD)
+template <typename AL, typename BL, typename EL, typename Ds, typename CDEOp>
+struct DeviceOperationInstanceFactory<DeviceGemmMultipleD<AL, BL, EL, half_t, half_t, Ds, half_t, element_wise::PassThrough,
+                                                          element_wise::PassThrough, CDEOp>>
+{
+    using DeviceOp = DeviceGemmMultipleD<AL, BL, EL, half_t, half_t, Ds, half_t, element_wise::PassThrough,
+                                         element_wise::PassThrough, CDEOp>;
+    static std::vector<std::unique_ptr<DeviceOp>> GetInstances()
+    {
+        std::vector<std::unique_ptr<DeviceOp>> v;
+        const int n = ckx_num_instances(CKX_OP_GEMM_F16);
+        for(int i = 0; i < n; ++i)
+            v.push_back(std::make_unique<DeviceGemmMultipleDMfma<AL, BL, EL, Ds, CDEOp>>(i));
+        return v;
+    }
+};
+
+template <typename InOp, typename WeiOp, typename OutOp>
+struct DeviceOperationInstanceFactory<DeviceConvFwdBiasActivation<InOp, WeiOp, OutOp>>
+{
+    using DeviceOp = DeviceConvFwdBiasActivation<InOp, WeiOp, OutOp>;
+    static std::vector<std::unique_ptr<DeviceOp>> GetInstances()
+    {
+        std::vector<std::unique_ptr<DeviceOp>> v;
+        for(int i = 0, n = ckx_num_instances(CKX_OP_CONV2D_FWD_F16); i < n; ++i)
+            v.push_back(std::make_unique<
+                        DeviceConv2dFwdBiasActivationMfma_Input_N_Hi_Wi_C_Weight_K_Y_X_C_Output_N_Ho_Wo_K<InOp, WeiOp, OutOp>>(i));
+        return v;
+    }
+};
+
+template <typename InOp, typename WeiOp, typename OutOp>
+struct DeviceOperationInstanceFactory<DeviceConvFwdBiasActivationAdd<InOp, WeiOp, OutOp>>
+{
+    using DeviceOp = DeviceConvFwdBiasActivationAdd<InOp, WeiOp, OutOp>;
+    static std::vector<std::unique_ptr<DeviceOp>> GetInstances()
+    {
+        std::vector<std::unique_ptr<DeviceOp>> v;
+        for(int i = 0, n = ckx_num_instances(CKX_OP_CONV2D_FWD_F16); i < n; ++i)
+            v.push_back(std::make_unique<
+                        DeviceConv2dFwdBiasActivationAddMfma_Input_N_Hi_Wi_C_Weight_K_Y_X_C_Output_N_Ho_Wo_K<InOp, WeiOp, OutOp>>(i));
+        return v;
+    }
+};
 
 } // namespace instance
 } // namespace device

@@ -7,6 +7,11 @@
 //   ckx_profiler conv2d_fwd <dtype 1|3> <verify> <init> <log> <time>
 //                     N K C Y X Hi Wi Sy Sx Dy Dx LeftPy LeftPx RightPy RightPx [epilogue sg sr] [nrepeat]
 //   ckx_profiler batched_gemm_gemm <verify> <init> <log> <time> M N K O Batch [nrepeat]
+//   ckx_profiler conv_fwd_bias_relu | conv_fwd_bias_relu_add <dtype 1> <verify> <init> <log> <time>
+//                     N K C Y X Hi Wi Sy Sx Dy Dx LeftPy LeftPx RightPy RightPx [nrepeat]
+//                     (profiler/src/profile_conv_fwd_bias_relu[_add].cpp; fp16, NHWC/KYXC/NHWK)
+//   ckx_profiler gemm_bias_relu <verify> <init> <log> <time> M N K StrideA StrideB StrideE [nrepeat]
+//                     (example/03_gemm_bias_relu: E = AddRelu(half(A*B), bias row), fp16)
 //
 // Every instance of the family is run (DeviceOperationInstanceFactory), one "Perf:" line each
 // and a final "Best Perf:" line, in the reference's format (profile_gemm_impl.hpp:176-177,
@@ -278,6 +283,111 @@ int profile_conv(int argc, char* argv[])
     return 1;
 }
 
+// conv + bias + ReLU (with_resi: + residual add), fp16
+int profile_conv_bias_relu(int argc, char* argv[], bool with_resi)
+{
+    if(argc < 22 || std::atoi(argv[2]) != 1)
+    {
+        std::printf("arg1: tensor operation (conv_fwd_bias_relu[_add])\narg2: data type (1: fp16)\n"
+                    "arg3: verification\narg4: initialization\narg5: print tensor value\narg6: time kernel\n"
+                    "arg7 to 21: N, K, C, Y, X, Hi, Wi, Sy, Sx, Dy, Dx, LeftPy, LeftPx, RightPy, RightPx\n"
+                    "arg22: nrepeat\n");
+        return 1;
+    }
+    using T = half_t;
+    const bool verify = std::atoi(argv[3]), time_kernel = std::atoi(argv[6]);
+    const int init = std::atoi(argv[4]), nrepeat = argc > 22 ? std::atoi(argv[22]) : 10;
+    int p[15];
+    for(int i = 0; i < 15; ++i)
+        p[i] = std::atoi(argv[7 + i]);
+    const int N = p[0], K = p[1], C = p[2], Y = p[3], X = p[4], Hi = p[5], Wi = p[6], Sy = p[7], Sx = p[8],
+              Dy = p[9], Dx = p[10], LPy = p[11], LPx = p[12], RPy = p[13], RPx = p[14];
+    const int Ho = (Hi + LPy + RPy - ((Y - 1) * Dy + 1)) / Sy + 1, Wo = (Wi + LPx + RPx - ((X - 1) * Dx + 1)) / Sx + 1;
+    const std::size_t out_elems = (std::size_t)N * Ho * Wo * K;
+    std::vector<T> in((std::size_t)N * Hi * Wi * C), wei((std::size_t)K * Y * X * C), bias((std::size_t)K),
+        resi(out_elems);
+    fill(in, init, 0xC0FFEE + 2, true);
+    fill(wei, init, 0xC0FFEE + 3, true);
+    fill(bias, init, 0xC0FFEE + 7, true);
+    fill(resi, init, 0xC0FFEE + 8, true);
+    ckx::DeviceMem di(in.size() * sizeof(T)), dw(wei.size() * sizeof(T)), db(bias.size() * sizeof(T)),
+        dr(resi.size() * sizeof(T)), dout(out_elems * sizeof(T));
+    di.ToDevice(in.data());
+    dw.ToDevice(wei.data());
+    db.ToDevice(bias.data());
+    dr.ToDevice(resi.data());
+    std::cout << "input: N " << N << " Hi " << Hi << " Wi " << Wi << " C " << C << "; weight: K " << K << " Y " << Y
+              << " X " << X << "; output: Ho " << Ho << " Wo " << Wo << std::endl;
+    const double flop  = 2.0 * N * K * Ho * Wo * C * Y * X;
+    const double bytes = sizeof(T) * ((double)in.size() + (double)wei.size() + (double)K +
+                                      (double)out_elems * (with_resi ? 2 : 1));
+    if(with_resi)
+    {
+        using Op = device::DeviceConvFwdBiasActivationAdd<Pass, Pass, element_wise::AddReluAdd>;
+        auto ops = device::instance::DeviceOperationInstanceFactory<Op>::GetInstances();
+        return run_family<T>(
+            ops,
+            [&](Op& op) {
+                return op.MakeArgumentPointer(di.GetDeviceBuffer(), dw.GetDeviceBuffer(), dout.GetDeviceBuffer(),
+                                              db.GetDeviceBuffer(), dr.GetDeviceBuffer(), N, K, C, {Hi, Wi}, {Y, X},
+                                              {Ho, Wo}, {Sy, Sx}, {Dy, Dx}, {LPy, LPx}, {RPy, RPx}, Pass{}, Pass{},
+                                              element_wise::AddReluAdd{});
+            },
+            dout, out_elems, flop, bytes, verify, time_kernel, nrepeat);
+    }
+    using Op = device::DeviceConvFwdBiasActivation<Pass, Pass, element_wise::AddRelu>;
+    auto ops = device::instance::DeviceOperationInstanceFactory<Op>::GetInstances();
+    return run_family<T>(
+        ops,
+        [&](Op& op) {
+            return op.MakeArgumentPointer(di.GetDeviceBuffer(), dw.GetDeviceBuffer(), dout.GetDeviceBuffer(),
+                                          db.GetDeviceBuffer(), N, K, C, {Hi, Wi}, {Y, X}, {Ho, Wo}, {Sy, Sx}, {Dy, Dx},
+                                          {LPy, LPx}, {RPy, RPx}, Pass{}, Pass{}, element_wise::AddRelu{});
+        },
+        dout, out_elems, flop, bytes, verify, time_kernel, nrepeat);
+}
+
+// E = AddRelu(half(A * B), D) with D a bias row (stride 0), as example 03 sets it up
+int profile_gemm_bias_relu(int argc, char* argv[])
+{
+    if(argc < 9)
+    {
+        std::printf("arg1: tensor operation (gemm_bias_relu)\narg2: verification\narg3: initialization\n"
+                    "arg4: print tensor value\narg5: time kernel\narg6 to 11: M, N, K, StrideA, StrideB, StrideE\n"
+                    "arg12: nrepeat\n");
+        return 1;
+    }
+    using T = half_t;
+    const bool verify = std::atoi(argv[2]), time_kernel = std::atoi(argv[5]);
+    const int init = std::atoi(argv[3]);
+    const int M = std::atoi(argv[6]), N = std::atoi(argv[7]), K = std::atoi(argv[8]);
+    int sa = argc > 9 ? std::atoi(argv[9]) : -1, sb = argc > 10 ? std::atoi(argv[10]) : -1,
+        se = argc > 11 ? std::atoi(argv[11]) : -1;
+    sa = sa < 0 ? K : sa, sb = sb < 0 ? K : sb, se = se < 0 ? N : se;
+    const int nrepeat = argc > 12 ? std::atoi(argv[12]) : 10;
+    using Ds       = ck::Tuple<T>;
+    using DeviceOp = device::DeviceGemmMultipleD<Row, Col, Row, T, T, Ds, T, Pass, Pass, element_wise::AddRelu>;
+    auto ops       = device::instance::DeviceOperationInstanceFactory<DeviceOp>::GetInstances();
+    std::vector<T> a((std::size_t)M * sa), b((std::size_t)N * sb), d((std::size_t)N);
+    fill(a, init, 0xC0FFEE, false);
+    fill(b, init, 0xC0FFEE + 1, false);
+    fill(d, init, 0xC0FFEE + 9, false);
+    ckx::DeviceMem da(a.size() * sizeof(T)), db(b.size() * sizeof(T)), dd(d.size() * sizeof(T)),
+        de((std::size_t)M * se * sizeof(T));
+    da.ToDevice(a.data());
+    db.ToDevice(b.data());
+    dd.ToDevice(d.data());
+    const double flop = 2.0 * M * N * K, bytes = sizeof(T) * ((double)M * K + (double)K * N + (double)M * N + N);
+    return run_family<T>(
+        ops,
+        [&](DeviceOp& op) {
+            return op.MakeArgumentPointer(da.GetDeviceBuffer(), db.GetDeviceBuffer(), {dd.GetDeviceBuffer()},
+                                          de.GetDeviceBuffer(), M, N, K, sa, sb, {0}, se, Pass{}, Pass{},
+                                          element_wise::AddRelu{});
+        },
+        de, (std::size_t)M * se, flop, bytes, verify, time_kernel, nrepeat);
+}
+
 int profile_gemm_gemm(int argc, char* argv[])
 {
     if(argc < 11)
@@ -332,9 +442,18 @@ int main(int argc, char* argv[])
             return profile_conv(argc, argv);
         if(argc >= 2 && std::strcmp(argv[1], "batched_gemm_gemm") == 0)
             return profile_gemm_gemm(argc, argv);
+        if(argc >= 2 && std::strcmp(argv[1], "conv_fwd_bias_relu") == 0)
+            return profile_conv_bias_relu(argc, argv, false);
+        if(argc >= 2 && std::strcmp(argv[1], "conv_fwd_bias_relu_add") == 0)
+            return profile_conv_bias_relu(argc, argv, true);
+        if(argc >= 2 && std::strcmp(argv[1], "gemm_bias_relu") == 0)
+            return profile_gemm_bias_relu(argc, argv);
         std::printf("arg1: tensor operation (gemm: GEMM\n"
                     "                        conv2d_fwd: NHWC/KYXC/NHWK forward convolution\n"
-                    "                        batched_gemm_gemm: batched fused GEMM+GEMM)\n");
+                    "                        batched_gemm_gemm: batched fused GEMM+GEMM\n"
+                    "                        conv_fwd_bias_relu: ForwardConvolution+Bias+ReLU\n"
+                    "                        conv_fwd_bias_relu_add: ForwardConvolution+Bias+ReLU+Add\n"
+                    "                        gemm_bias_relu: GEMM+Bias+ReLU)\n");
         return 1;
     }
     catch(const std::exception& e)

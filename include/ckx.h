@@ -51,7 +51,17 @@ enum
 {
     CKX_EPI_PASSTHROUGH = 0,
     CKX_EPI_REQUANT_CK  = 1,
-    CKX_EPI_REQUANT_RND = 2
+    CKX_EPI_REQUANT_RND = 2,
+    /* fp16 outputs with extra fp16 "D" operands, arithmetic in fp32, one rounding at the store:
+     *  ADD_RELU           e = half(relu(acc + d0))          element_wise::AddRelu as applied by
+     *                     ReferenceConvFwd_Bias_Activation (reference_conv_fwd_bias_activation.hpp:75-124)
+     *  ADD_RELU_ADD       e = half(relu(acc + d0) + d1)     element_wise::AddReluAdd
+     *                     (element_wise_operation.hpp:46-81, reference_conv_fwd_bias_activation_add.hpp)
+     *  CSHUFFLE_ADD_RELU  e = relu(half(half(acc) + d0))    AddRelu on the C value already rounded to
+     *                     fp16 (example/03_gemm_bias_relu/gemm_bias_relu_xdl_fp16.cpp:31-40,251-275) */
+    CKX_EPI_ADD_RELU          = 3,
+    CKX_EPI_ADD_RELU_ADD      = 4,
+    CKX_EPI_CSHUFFLE_ADD_RELU = 5
 };
 
 /* Operator families, for the instance queries below. */
@@ -108,6 +118,20 @@ int ckx_gemm_f16(const void* p_a, const void* p_b, void* p_c, int32_t M, int32_t
                  int c_layout, int instance, void* p_workspace, int64_t workspace_bytes, void* stream);
 int64_t ckx_gemm_f16_workspace_bytes(int32_t M, int32_t N, int32_t K, int instance);
 
+/* ---- fp16 GEMM with fused D operands:  E = cde_op(A * B, D0 [, D1]) ----------
+ * Replaces DeviceGemmMultipleD<..., Tuple<half_t[, half_t]>, half_t, PassThrough, PassThrough, CDEOp>
+ * ::MakeArgumentPointer + Run (device_gemm_multiple_d.hpp:14-55) for cde_op in
+ * CKX_EPI_ADD_RELU / _ADD_RELU_ADD / _CSHUFFLE_ADD_RELU. D0, D1 are [M,N] row-major fp16 with row
+ * strides stride_d0 / stride_d1 in elements; stride 0 broadcasts one row (a bias vector), as
+ * example 03 does. p_d1 is ignored unless cde_op uses it. */
+int ckx_gemm_f16_multiple_d_is_supported(int32_t M, int32_t N, int32_t K, int32_t stride_a, int32_t stride_b,
+                                         int32_t stride_d0, int32_t stride_d1, int32_t stride_e, int a_layout,
+                                         int b_layout, int e_layout, int cde_op, int instance);
+int ckx_gemm_f16_multiple_d(const void* p_a, const void* p_b, const void* p_d0, const void* p_d1, void* p_e,
+                            int32_t M, int32_t N, int32_t K, int32_t stride_a, int32_t stride_b, int32_t stride_d0,
+                            int32_t stride_d1, int32_t stride_e, int a_layout, int b_layout, int e_layout,
+                            int cde_op, int instance, void* p_workspace, int64_t workspace_bytes, void* stream);
+
 /* ---- conv2d forward, NHWC input / KYXC weight / NHWK output, implicit GEMM --
  * Replaces DeviceConvFwd<PassThrough, PassThrough, OutOp>::MakeArgumentPointer + Run
  * (device_conv_fwd.hpp:18-39) as implemented by
@@ -135,6 +159,15 @@ int ckx_conv2d_fwd_i8(const void* p_in, const void* p_wei, void* p_out, const ck
 int ckx_conv2d_fwd_f16(const void* p_in, const void* p_wei, void* p_out, const ckx_conv2d_desc* desc,
                        int instance, void* p_workspace, int64_t workspace_bytes, void* stream);
 int64_t ckx_conv2d_fwd_workspace_bytes(int op, const ckx_conv2d_desc* desc, int instance);
+/* conv2d forward + bias + ReLU (+ residual add), fp16: replaces
+ * DeviceConvFwdBiasActivation / DeviceConvFwdBiasActivationAdd ::MakeArgumentPointer + Run
+ * (device_conv_fwd_bias_activation.hpp:18-41, device_conv_fwd_bias_activation_add.hpp).
+ * p_bias is a contiguous [K] vector, p_resi has the output's NHWK layout (ignored for ADD_RELU);
+ * out_op is CKX_EPI_ADD_RELU or CKX_EPI_ADD_RELU_ADD. Supported geometries are those of
+ * ckx_conv2d_fwd_is_supported(CKX_OP_CONV2D_FWD_F16, desc, out_op, instance). */
+int ckx_conv2d_fwd_bias_activation_f16(const void* p_in, const void* p_wei, void* p_out, const void* p_bias,
+                                       const void* p_resi, const ckx_conv2d_desc* desc, int out_op, int instance,
+                                       void* p_workspace, int64_t workspace_bytes, void* stream);
 
 /* ---- batched fused GEMM-GEMM, fp16:  C[g] = half( half(A[g]*B0[g]) * B1[g] ) --
  * The reference snapshot has no such operator; the surface is upstream's

@@ -395,6 +395,49 @@ void cko_conv2d_fwd_i8(const int8_t* in, const int8_t* wei, int8_t* out, int N, 
         [=](std::size_t o, float acc) { out[o] = float_to_i8_trunc_wrap(ep(acc)); });
 }
 
+// conv2d forward + bias + ReLU (+ residual), fp16 tensors: the accumulator stays fp32 through the
+// functor (element_wise::AddRelu / AddReluAdd on floats), one conversion at the store
+// (reference_conv_fwd_bias_activation.hpp:75-124, reference_conv_fwd_bias_activation_add.hpp:78-130,
+// binary_element_wise_operation.hpp:123-129, element_wise_operation.hpp:60-70).
+// bias is [K]; resi has the output's NHWK layout and is null for the two-operand functor.
+void cko_conv2d_fwd_bias_relu_f16(const uint16_t* in, const uint16_t* wei, const uint16_t* bias,
+                                  const uint16_t* resi, uint16_t* out, int N, int K, int C, int Hi, int Wi,
+                                  int Y, int X, int Ho, int Wo, int sH, int sW, int dH, int dW, int pH, int pW,
+                                  int nthreads)
+{
+    conv2d_fwd(
+        N, K, C, Hi, Wi, Y, X, Ho, Wo, sH, sW, dH, dW, pH, pW, nthreads,
+        [=](std::size_t o) { return half_to_float(in[o]); },
+        [=](std::size_t o) { return half_to_float(wei[o]); },
+        [=](std::size_t o, float acc) {
+            const float a = acc + half_to_float(bias[o % (std::size_t)K]);
+            const float b = a > 0.0f ? a : 0.0f;
+            out[o]        = float_to_half(resi ? b + half_to_float(resi[o]) : b);
+        });
+}
+
+// fp16 GEMM + bias row + ReLU the way example 03 verifies it: ReferenceGemm into an fp32 C, then
+// AddRelu on half_t operands, i.e. C is rounded to fp16 when it is passed, the sum is rounded to
+// fp16 again (example/03_gemm_bias_relu/gemm_bias_relu_xdl_fp16.cpp:31-40,251-275).
+// d is [M,N] with element strides (sd_m may be 0: one bias row).
+void cko_gemm_f16_add_relu(const uint16_t* a, const uint16_t* b, const uint16_t* d, uint16_t* e, int M, int N,
+                           int K, int64_t sa_m, int64_t sa_k, int64_t sb_k, int64_t sb_n, int64_t sd_m,
+                           int64_t sd_n, int64_t se_m, int64_t se_n, int nthreads)
+{
+    parallel_for((std::size_t)M * (std::size_t)N, nthreads, [&](std::size_t i0, std::size_t i1) {
+        for(std::size_t i = i0; i < i1; ++i)
+        {
+            const std::size_t m = i / (std::size_t)N, n = i % (std::size_t)N;
+            float acc           = 0;
+            for(int k = 0; k < K; ++k)
+                acc += half_to_float(a[m * sa_m + k * sa_k]) * half_to_float(b[k * sb_k + n * sb_n]);
+            const float c = half_to_float(float_to_half(acc));
+            const float x = half_to_float(float_to_half(c + half_to_float(d[m * sd_m + n * sd_n])));
+            e[m * se_m + n * se_n] = float_to_half(x > 0.0f ? x : 0.0f);
+        }
+    });
+}
+
 // ---- magic-number division (dividend < 2^31, divisor >= 1) ----
 void cko_magic_division_params(uint32_t divisor, uint32_t* multiplier, uint32_t* shift)
 {

@@ -90,6 +90,26 @@ def conv2d_fwd_f16(inp_nhwc, wei_kyxc, strides=(1, 1), dilations=(1, 1), pads=(0
     return out.astype(np.float16).reshape(N, Ho, Wo, K)
 
 
+def conv2d_fwd_bias_relu_f16(inp_nhwc, wei_kyxc, bias_k, resi_nhwk=None, strides=(1, 1), dilations=(1, 1),
+                             pads=(0, 0), right_pads=None):
+    """conv + bias + ReLU (+ residual) in fp32, rounded once to fp16 (BLAS summation order)."""
+    N = inp_nhwc.shape[0]
+    K, Y, X, C = wei_kyxc.shape
+    cols, Ho, Wo = im2col(inp_nhwc, Y, X, strides, dilations, pads, right_pads)
+    acc = cols.astype(np.float32) @ wei_kyxc.reshape(K, Y * X * C).T.astype(np.float32)
+    y = np.maximum(acc + np.asarray(bias_k, np.float32)[None, :], np.float32(0))
+    if resi_nhwk is not None:
+        y = y + np.asarray(resi_nhwk, np.float32).reshape(-1, K)
+    return y.astype(np.float16).reshape(N, Ho, Wo, K)
+
+
+def gemm_f16_add_relu(a_mk, b_kn, d_mn):
+    """relu(half(half(A*B) + D)): the GEMM result is rounded to fp16 before the functor."""
+    c = (np.asarray(a_mk, np.float32) @ np.asarray(b_kn, np.float32)).astype(np.float16)
+    x = (c.astype(np.float32) + np.asarray(d_mn, np.float32)).astype(np.float16)
+    return np.maximum(x, np.float16(0))
+
+
 def batched_gemm_gemm_f16(a_gmk, b0_gkn, b1_gno):
     s = np.matmul(np.asarray(a_gmk, np.float32), np.asarray(b0_gkn, np.float32)).astype(np.float16)
     return np.matmul(s.astype(np.float32), np.asarray(b1_gno, np.float32)).astype(np.float16)

@@ -148,6 +148,38 @@ def conv2d_fwd(inp_nhwc, wei_kyxc, strides=(1, 1), dilations=(1, 1), pads=(0, 0)
     return out
 
 
+def conv2d_fwd_bias_relu_f16(inp_nhwc, wei_kyxc, bias_k, resi_nhwk=None, strides=(1, 1), dilations=(1, 1),
+                             pads=(0, 0), right_pads=None, nthreads=0):
+    """conv + bias + ReLU (+ residual), fp16 tensors, fp32 through the functor, one rounding."""
+    inp = np.ascontiguousarray(inp_nhwc, np.float16)
+    wei = np.ascontiguousarray(wei_kyxc, np.float16)
+    bias = np.ascontiguousarray(bias_k, np.float16)
+    N, Hi, Wi, Cc = inp.shape
+    K, Y, X, _ = wei.shape
+    if right_pads is None:
+        right_pads = pads
+    Ho = conv_out_len(Hi, Y, strides[0], dilations[0], pads[0], right_pads[0])
+    Wo = conv_out_len(Wi, X, strides[1], dilations[1], pads[1], right_pads[1])
+    out = np.empty((N, Ho, Wo, K), np.float16)
+    resi = None if resi_nhwk is None else np.ascontiguousarray(resi_nhwk, np.float16)
+    assert resi is None or resi.shape == out.shape
+    lib().cko_conv2d_fwd_bias_relu_f16(_p(inp), _p(wei), _p(bias), _p(resi) if resi is not None else None,
+                                       _p(out), N, K, Cc, Hi, Wi, Y, X, Ho, Wo, strides[0], strides[1],
+                                       dilations[0], dilations[1], pads[0], pads[1], int(nthreads))
+    return out
+
+
+def gemm_f16_add_relu(a_mk, b_kn, d_mn, nthreads=0):
+    """E = relu(half(half(A*B) + D)) as example 03 verifies it; d_mn may be a broadcast view."""
+    M, K = a_mk.shape
+    _, N = b_kn.shape
+    d = np.broadcast_to(d_mn, (M, N))
+    e = np.empty((M, N), np.float16)
+    lib().cko_gemm_f16_add_relu(_p(a_mk), _p(b_kn), _p(d), _p(e), M, N, K, *_i64(*_estrides(a_mk)),
+                                *_i64(*_estrides(b_kn)), *_i64(*_estrides(d)), *_i64(N, 1), int(nthreads))
+    return e
+
+
 def epilogue_i8(acc, epi, scale_gemm, scale_relu):
     return int(lib().cko_epilogue_i8(int(acc), int(epi), C.c_float(scale_gemm), C.c_float(scale_relu)))
 

@@ -29,6 +29,8 @@
 #include "ck/library/reference_tensor_operation/cpu/reference_gemm.hpp"
 #include "ck/library/reference_tensor_operation/cpu/reference_conv_fwd.hpp"
 #include "ck/library/reference_tensor_operation/cpu/reference_batched_gemm.hpp"
+#include "ck/library/reference_tensor_operation/cpu/reference_conv_fwd_bias_activation.hpp"
+#include "ck/library/reference_tensor_operation/cpu/reference_conv_fwd_bias_activation_add.hpp"
 
 namespace {
 
@@ -185,6 +187,75 @@ void ckref_batched_gemm_f16(const uint16_t* a, const uint16_t* b, uint16_t* c, i
     auto arg = ref.MakeArgument(ta, tb, tc, PassThrough{}, PassThrough{}, PassThrough{});
     inv.Run(arg);
     std::memcpy(c, tc.mData.data(), tc.mData.size() * sizeof(H));
+}
+
+// ReferenceConvFwd_Bias_Activation<half,half,half,Pass,Pass,AddRelu> (example 06) and
+// ReferenceConvFwd_Bias_Activation_Add<..., AddReluAdd> (example 07); resi == null selects the former
+void ckref_conv2d_fwd_bias_relu_f16(const uint16_t* in, const uint16_t* wei, const uint16_t* bias,
+                                    const uint16_t* resi, uint16_t* out, int N, int K, int C, int Hi, int Wi,
+                                    int Y, int X, int Ho, int Wo, int sH, int sW, int dH, int dW, int pH,
+                                    int pW)
+{
+    using T  = ck::half_t;
+    using sz = std::size_t;
+    auto ti  = make_tensor<T>({(sz)N, (sz)C, (sz)Hi, (sz)Wi}, {(sz)C * Hi * Wi, 1, (sz)Wi * C, (sz)C},
+                             reinterpret_cast<const T*>(in));
+    auto tw  = make_tensor<T>({(sz)K, (sz)C, (sz)Y, (sz)X}, {(sz)C * Y * X, 1, (sz)X * C, (sz)C},
+                             reinterpret_cast<const T*>(wei));
+    auto to  = make_tensor<T>({(sz)N, (sz)K, (sz)Ho, (sz)Wo}, {(sz)K * Ho * Wo, 1, (sz)Wo * K, (sz)K},
+                             (const T*)nullptr);
+    auto tb  = make_tensor<T>({(sz)K}, {1}, reinterpret_cast<const T*>(bias));
+    if(resi)
+    {
+        auto tr = make_tensor<T>({(sz)N, (sz)K, (sz)Ho, (sz)Wo}, {(sz)K * Ho * Wo, 1, (sz)Wo * K, (sz)K},
+                                 reinterpret_cast<const T*>(resi));
+        using Op  = ck::tensor_operation::element_wise::AddReluAdd;
+        using Ref = ck::tensor_operation::host::ReferenceConvFwd_Bias_Activation_Add<T, T, T, PassThrough,
+                                                                                     PassThrough, Op>;
+        Ref ref;
+        auto inv = ref.MakeInvoker();
+        auto arg = ref.MakeArgument(ti, tw, to, tb, tr, {sH, sW}, {dH, dW}, {pH, pW}, {pH, pW}, PassThrough{},
+                                    PassThrough{}, Op{});
+        inv.Run(arg);
+    }
+    else
+    {
+        using Op  = ck::tensor_operation::element_wise::AddRelu;
+        using Ref = ck::tensor_operation::host::ReferenceConvFwd_Bias_Activation<T, T, T, PassThrough,
+                                                                                 PassThrough, Op>;
+        Ref ref;
+        auto inv = ref.MakeInvoker();
+        auto arg = ref.MakeArgument(ti, tw, to, tb, {sH, sW}, {dH, dW}, {pH, pW}, {pH, pW}, PassThrough{},
+                                    PassThrough{}, Op{});
+        inv.Run(arg);
+    }
+    std::memcpy(out, to.mData.data(), to.mData.size() * sizeof(T));
+}
+
+// example 03's verification: ReferenceGemm<half,half,float,float,...> then AddRelu on half_t
+void ckref_gemm_f16_add_relu(const uint16_t* a, const uint16_t* b, const uint16_t* d, uint16_t* e, int M, int N,
+                             int K, long sa_m, long sa_k, long sb_k, long sb_n, long sd_m, long sd_n)
+{
+    using T  = ck::half_t;
+    using sz = std::size_t;
+    auto ta  = make_tensor<T>({(sz)M, (sz)K}, {(sz)sa_m, (sz)sa_k}, reinterpret_cast<const T*>(a));
+    auto tb  = make_tensor<T>({(sz)K, (sz)N}, {(sz)sb_k, (sz)sb_n}, reinterpret_cast<const T*>(b));
+    auto tc  = make_tensor<float>({(sz)M, (sz)N}, {(sz)N, 1}, (const float*)nullptr);
+    using Ref =
+        ck::tensor_operation::host::ReferenceGemm<T, T, float, float, PassThrough, PassThrough, PassThrough>;
+    Ref ref;
+    auto inv = ref.MakeInvoker();
+    auto arg = ref.MakeArgument(ta, tb, tc, PassThrough{}, PassThrough{}, PassThrough{});
+    inv.Run(arg);
+    const T* dd = reinterpret_cast<const T*>(d);
+    T* ee       = reinterpret_cast<T*>(e);
+    ck::tensor_operation::element_wise::AddRelu op;
+    for(int m = 0; m < M; ++m)
+        for(int n = 0; n < N; ++n)
+        {
+            const T c = ck::type_convert<T>(tc(m, n));
+            op(ee[(sz)m * N + n], c, dd[(sz)m * sd_m + (sz)n * sd_n]);
+        }
 }
 
 int ckref_conv_out_len(int in_len, int filter_len, int stride, int dilation, int pad_left, int pad_right)

@@ -84,6 +84,30 @@ class _Ref:
            dilations[0], dilations[1], pads[0], pads[1])
         return out
 
+    def conv2d_fwd_bias_relu_f16(self, inp_nhwc, wei_kyxc, bias_k, resi_nhwk=None, strides=(1, 1),
+                                 dilations=(1, 1), pads=(0, 0)):
+        inp = np.ascontiguousarray(inp_nhwc, np.float16)
+        wei = np.ascontiguousarray(wei_kyxc, np.float16)
+        bias = np.ascontiguousarray(bias_k, np.float16)
+        N, Hi, Wi, Cc = inp.shape
+        K, Y, X, _ = wei.shape
+        Ho = self.conv_out_len(Hi, Y, strides[0], dilations[0], pads[0], pads[0])
+        Wo = self.conv_out_len(Wi, X, strides[1], dilations[1], pads[1], pads[1])
+        out = np.zeros((N, Ho, Wo, K), np.float16)
+        resi = None if resi_nhwk is None else np.ascontiguousarray(resi_nhwk, np.float16)
+        self.lib.ckref_conv2d_fwd_bias_relu_f16(_p(inp), _p(wei), _p(bias), _p(resi) if resi is not None else None,
+                                                _p(out), N, K, Cc, Hi, Wi, Y, X, Ho, Wo, strides[0], strides[1],
+                                                dilations[0], dilations[1], pads[0], pads[1])
+        return out
+
+    def gemm_f16_add_relu(self, a_mk, b_kn, d_mn):
+        M, K = a_mk.shape
+        _, N = b_kn.shape
+        d = np.broadcast_to(d_mn, (M, N))
+        e = np.zeros((M, N), np.float16)
+        self.lib.ckref_gemm_f16_add_relu(_p(a_mk), _p(b_kn), _p(d), _p(e), M, N, K, *_es(a_mk), *_es(b_kn), *_es(d))
+        return e
+
     def conv_out_len(self, in_len, filt, stride, dil, pl, pr):
         return int(self.lib.ckref_conv_out_len(in_len, filt, stride, dil, pl, pr))
 

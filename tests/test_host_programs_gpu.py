@@ -96,3 +96,33 @@ def test_example_gemm_requant_relu_requant_int8(tmp_path):
     want = lit.gemm_i8(a, b_nk.T, lit.EPI_REQUANT_CK, 0.03, 1.0)
     np.testing.assert_array_equal(c, want)
     assert f"sum(C) = {int(want.astype(np.int64).sum())}" in out
+
+
+@pytest.mark.parametrize("with_resi", [False, True])
+def test_profiler_conv_fwd_bias_relu_and_add(tmp_path, with_resi):
+    """profile_conv_fwd_bias_relu[_add] of the reference's profiler (the ResNet-50 script's operations)."""
+    geo = [2, 64, 32, 3, 3, 14, 14, 1, 1, 1, 1, 1, 1, 1, 1]
+    op = "conv_fwd_bias_relu_add" if with_resi else "conv_fwd_bias_relu"
+    out, dump = _run("ckx_profiler", [op, 1, 1, 2, 0, 1] + geo, "CKX_PROFILER_DUMP", tmp_path)
+    assert "Best Perf:" in out and "Error" not in out and "AddRelu" in out
+    N, K, C, Y, X, Hi, Wi = geo[:7]
+    inp = uniform_f16((N, Hi, Wi, C), -1, 1, SEED + 2)
+    wei = uniform_f16((K, Y, X, C), -1, 1, SEED + 3)
+    bias = uniform_f16((K,), -1, 1, SEED + 7)
+    resi = uniform_f16((N, 14, 14, K), -1, 1, SEED + 8) if with_resi else None
+    want = lit.conv2d_fwd_bias_relu_f16(inp, wei, bias, resi, (1, 1), (1, 1), (1, 1))
+    c = np.fromfile(dump, np.float16).reshape(want.shape)
+    bad, max_err = lit.check_err_f16(c, want, 1e-2, 1e-2)
+    assert bad == 0, max_err
+
+
+def test_profiler_gemm_bias_relu(tmp_path):
+    M, N, K = 384, 256, 512
+    out, dump = _run("ckx_profiler", ["gemm_bias_relu", 1, 2, 0, 1, M, N, K], "CKX_PROFILER_DUMP", tmp_path)
+    assert "Best Perf:" in out and "Error" not in out
+    a = uniform_f16((M, K), -1, 1, SEED)
+    b_nk = uniform_f16((N, K), -1, 1, SEED + 1)
+    d = uniform_f16((N,), -1, 1, SEED + 9)
+    c = np.fromfile(dump, np.float16).reshape(M, N)
+    bad, max_err = lit.check_err_f16(c, lit.gemm_f16_add_relu(a, b_nk.T, d[None, :]), 1e-2, 1e-2)
+    assert bad == 0, max_err

@@ -326,3 +326,81 @@ def test_conv2d_is_a_gemm_for_1x1():
     wei = _rand_i8(rng, (8, 1, 1, 32))
     out = lit.conv2d_fwd(inp, wei)
     np.testing.assert_array_equal(out.reshape(-1, 8), lit.gemm_i8(inp.reshape(-1, 32), wei.reshape(8, 32).T))
+
+
+# ------------------------------------------------- fused bias / ReLU / residual epilogues
+@pytest.mark.parametrize("case", [c for c in GOLD["cases"] if max(c["expected"]) < 2000 and
+                                  c["left_pads"] == c["right_pads"]])
+def test_conv2d_bias_relu_on_the_reference_golden_vectors(case):
+    """The reference's golden conv outputs (all exactly representable in fp16 for these cases)
+    pushed through AddRelu / AddReluAdd by hand: the bias is chosen so that ReLU cuts part of the
+    outputs, the residual is negative so that relu(acc + b) + r differs from relu(acc + b + r)."""
+    N, K, C = case["N"], case["K"], case["C"]
+    Hi, Wi = case["input"]
+    Y, X = case["filter"]
+    inp = np.arange(N * Hi * Wi * C, dtype=np.float32).reshape(N, Hi, Wi, C).astype(np.float16)
+    wei = np.full((K, Y, X, C), 0.5, np.float16)
+    gold = np.array(case["expected"], np.float32)
+    n, k, ho, wo = case["out_dims_nkhw"]
+    gold = gold.reshape(n, ho, wo, k)
+    assert np.array_equal(gold.astype(np.float16).astype(np.float32), gold)
+    bias = (-np.median(gold) - 0.5 * np.arange(K)).astype(np.float16)
+    resi = np.full(gold.shape, -3.0, np.float16)
+    want = np.maximum(gold + bias.astype(np.float32), 0)
+    out = lit.conv2d_fwd_bias_relu_f16(inp, wei, bias, None, case["strides"], case["dilations"], case["left_pads"])
+    np.testing.assert_array_equal(out, want.astype(np.float16))
+    assert (out == 0).any() and (out > 0).any()
+    out2 = lit.conv2d_fwd_bias_relu_f16(inp, wei, bias, resi, case["strides"], case["dilations"], case["left_pads"])
+    np.testing.assert_array_equal(out2, (want - 3.0).astype(np.float16))
+    assert (out2 == -3).any()
+    np.testing.assert_array_equal(
+        fast.conv2d_fwd_bias_relu_f16(inp, wei, bias, resi, case["strides"], case["dilations"], case["left_pads"]), out2)
+    if REF is not None:
+        np.testing.assert_array_equal(
+            REF.conv2d_fwd_bias_relu_f16(inp, wei, bias, None, case["strides"], case["dilations"], case["left_pads"]), out)
+        np.testing.assert_array_equal(
+            REF.conv2d_fwd_bias_relu_f16(inp, wei, bias, resi, case["strides"], case["dilations"], case["left_pads"]), out2)
+
+
+def test_conv2d_bias_relu_random_lit_fast_ref_agree():
+    rng = np.random.default_rng(5)
+    inp = rng.uniform(-1, 1, (2, 9, 7, 8)).astype(np.float16)
+    wei = rng.uniform(-1, 1, (5, 3, 3, 8)).astype(np.float16)
+    bias = rng.uniform(-2, 2, 5).astype(np.float16)
+    out_shape = (2, 5, 4, 5)
+    resi = rng.uniform(-2, 2, out_shape).astype(np.float16)
+    for r in (None, resi):
+        a = lit.conv2d_fwd_bias_relu_f16(inp, wei, bias, r, (2, 2), (1, 1), (1, 1))
+        assert a.shape == out_shape
+        b = fast.conv2d_fwd_bias_relu_f16(inp, wei, bias, r, (2, 2), (1, 1), (1, 1))
+        assert np.all(np.abs(a.astype(np.float32) - b.astype(np.float32)) <= 2e-3 + 2e-3 * np.abs(b.astype(np.float32)))
+        if REF is not None:
+            np.testing.assert_array_equal(REF.conv2d_fwd_bias_relu_f16(inp, wei, bias, r, (2, 2), (1, 1), (1, 1)), a)
+
+
+def test_gemm_add_relu_rounds_c_to_fp16_before_the_functor():
+    """Example 03 hands the fp32 GEMM result to a functor on half_t operands: C is rounded first.
+    K = 2049 ones give acc = 2049, fp16 2048 (tie to even); + 1 = 2049 -> 2048 again. A single
+    rounding of acc + d = 2050 would give 2050. Negative sums must come out as +0."""
+    a = np.ones((3, 2049), np.float16)
+    b = np.ones((2049, 4), np.float16)
+    d = np.array([1.0, -1.0, -4096.0, 0.0], np.float16)[None, :]
+    e = lit.gemm_f16_add_relu(a, b, d)
+    np.testing.assert_array_equal(e, np.broadcast_to(np.array([2048, 2047, 0, 2048], np.float16), (3, 4)))
+    assert not np.signbit(e).any()
+    np.testing.assert_array_equal(fast.gemm_f16_add_relu(a, b, d), e)
+    if REF is not None:
+        np.testing.assert_array_equal(REF.gemm_f16_add_relu(a, b, d), e)
+
+
+def test_gemm_add_relu_random_lit_ref_bit_exact_and_full_d():
+    rng = np.random.default_rng(8)
+    a = rng.uniform(-1, 1, (17, 96)).astype(np.float16)
+    b = np.asfortranarray(rng.uniform(-1, 1, (96, 23)).astype(np.float16))
+    for d in (rng.uniform(-3, 3, (1, 23)).astype(np.float16), rng.uniform(-3, 3, (17, 23)).astype(np.float16)):
+        e = lit.gemm_f16_add_relu(a, b, d)
+        c = lit.gemm_f16(a, b)
+        x = (c.astype(np.float32) + np.broadcast_to(d, c.shape).astype(np.float32)).astype(np.float16)
+        np.testing.assert_array_equal(e, np.maximum(x, np.float16(0)))
+        if REF is not None:
+            np.testing.assert_array_equal(REF.gemm_f16_add_relu(a, b, d), e)
