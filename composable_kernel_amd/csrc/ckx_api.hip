@@ -155,12 +155,24 @@ int force_ksplit()
 // costs the unit's share of MFMA time, scaled by how well that tile shape feeds the MFMA pipe,
 // plus a fixed prologue/epilogue term that co-resident workgroups overlap. Split-K adds the
 // second pass (launch + slice traffic) and is only considered when a workspace is available.
-Plan make_plan(int M, int N, int kbytes, int only_tile, long workspace_bytes)
+// K runs actually used for a requested KBatch: every run must get at least one 128-byte K tile
+int splitk_runs(int kbytes, int k_batch)
+{
+    const int nk = (kbytes + 127) / 128 > 0 ? (kbytes + 127) / 128 : 1;
+    k_batch      = k_batch > 8 ? 8 : k_batch;
+    for(int sp = k_batch; sp > 1; --sp)
+        if((long)((nk + sp - 1) / sp) * (sp - 1) < nk)
+            return sp;
+    return 1;
+}
+
+// k_batch > 0: the caller fixed the number of K runs (DeviceGemmSplitK's KBatch)
+Plan make_plan(int M, int N, int kbytes, int only_tile, long workspace_bytes, int k_batch = 0)
 {
     Plan best;
     double best_us  = 1e30;
     const int nk    = (kbytes + 127) / 128 > 0 ? (kbytes + 127) / 128 : 1;
-    const int force = force_ksplit();
+    const int force = k_batch > 0 ? splitk_runs(kbytes, k_batch) : force_ksplit();
     for(int i = 0; i < kNumTiles; ++i)
     {
         if(only_tile >= 0 && i != only_tile)
@@ -316,11 +328,15 @@ long gemm_workspace_bytes(int dt, int M, int N, int K, int instance)
 
 int run_gemm(int dt, const void* a, const void* b, void* c, int M, int N, int K, int sa, int sb, int sc,
              int al, int bl, int cl, int epi, float sg, float sr, int instance, void* ws, long ws_bytes,
-             void* stream, const DOperands& dops = DOperands{})
+             void* stream, const DOperands& dops = DOperands{}, int k_batch = 0)
 {
     int st = check_gemm_shape(dt, M, N, K, sa, sb, sc, al, bl, cl, epi, instance);
     if(st != CKX_OK)
         return st;
+    if(k_batch < 0 || k_batch > 8)
+        return fail(CKX_UNSUPPORTED, "KBatch must be 1..8");
+    if(k_batch > 0 && instance >= kNumTiles)
+        return fail(CKX_UNSUPPORTED, "the skinny instances split K over their waves, not over runs");
     if((st = check_d_operands(epi, N, dops)) != CKX_OK)
         return st;
     if(M == 0 || N == 0)
@@ -336,7 +352,7 @@ int run_gemm(int dt, const void* a, const void* b, void* c, int M, int N, int K,
     const bool tile64 = M > 32 && M <= 64 &&
                         ((N + 63) / 64 >= 160 ||
                          (ws && !(reinterpret_cast<uintptr_t>(ws) & 15) && make_plan(M, N, K * es, -1, ws_bytes).ksplit > 1));
-    if(instance == CKX_INSTANCE_AUTO && M <= 64 && !tile64)
+    if(instance == CKX_INSTANCE_AUTO && M <= 64 && !tile64 && k_batch == 0)
     {
         // A handful of rows against a big weight matrix is an HBM-streaming problem. Wider
         // workgroups (32 / 64 columns) re-read A from L2 less often, as long as enough workgroups
@@ -348,7 +364,10 @@ int run_gemm(int dt, const void* a, const void* b, void* c, int M, int N, int K,
     {
         if(ws && (reinterpret_cast<uintptr_t>(ws) & 15))
             return fail(CKX_INVALID_VALUE, "workspace must be 16-byte aligned");
-        pl = make_plan(M, N, K * es, instance, ws ? ws_bytes : 0);
+        if(k_batch > 1 && splitk_runs(K * es, k_batch) > 1 &&
+           (!ws || ws_bytes < (long)splitk_runs(K * es, k_batch) * M * N * 4))
+            return fail(CKX_INVALID_VALUE, "KBatch > 1 needs a workspace of ckx_gemm_splitk_workspace_bytes()");
+        pl = make_plan(M, N, K * es, instance, ws ? ws_bytes : 0, k_batch);
         ti = pl.tile;
     }
     ckx::GemmArgs g;
@@ -557,6 +576,35 @@ int ckx_gemm_f16(const void* a, const void* b, void* c, int32_t M, int32_t N, in
 {
     return run_gemm(ckx::DT_F16, a, b, c, M, N, K, sa, sb, sc, al, bl, cl, CKX_EPI_PASSTHROUGH, 1.0f, 1.0f,
                     instance, workspace, workspace_bytes, stream);
+}
+
+int64_t ckx_gemm_splitk_workspace_bytes(int op, int32_t M, int32_t N, int32_t K, int32_t k_batch)
+{
+    if((op != CKX_OP_GEMM_I8 && op != CKX_OP_GEMM_F16) || M <= 0 || N <= 0 || K < 0 || k_batch < 1)
+        return 0;
+    const int runs = splitk_runs(K * (op == CKX_OP_GEMM_I8 ? 1 : 2), k_batch);
+    return runs > 1 ? (int64_t)runs * M * N * 4 : 0;
+}
+
+int ckx_gemm_i8_splitk(const void* a, const void* b, void* c, int32_t M, int32_t N, int32_t K, int32_t sa,
+                       int32_t sb, int32_t sc, int al, int bl, int cl, int epilogue, float scale_gemm,
+                       float scale_relu, int instance, int32_t k_batch, void* workspace, int64_t workspace_bytes,
+                       void* stream)
+{
+    if(k_batch < 1)
+        return fail(CKX_INVALID_VALUE, "KBatch must be at least 1");
+    return run_gemm(ckx::DT_I8, a, b, c, M, N, K, sa, sb, sc, al, bl, cl, epilogue, scale_gemm, scale_relu,
+                    instance, workspace, workspace_bytes, stream, DOperands{}, k_batch);
+}
+
+int ckx_gemm_f16_splitk(const void* a, const void* b, void* c, int32_t M, int32_t N, int32_t K, int32_t sa,
+                        int32_t sb, int32_t sc, int al, int bl, int cl, int instance, int32_t k_batch,
+                        void* workspace, int64_t workspace_bytes, void* stream)
+{
+    if(k_batch < 1)
+        return fail(CKX_INVALID_VALUE, "KBatch must be at least 1");
+    return run_gemm(ckx::DT_F16, a, b, c, M, N, K, sa, sb, sc, al, bl, cl, CKX_EPI_PASSTHROUGH, 1.0f, 1.0f,
+                    instance, workspace, workspace_bytes, stream, DOperands{}, k_batch);
 }
 
 int ckx_gemm_f16_multiple_d_is_supported(int32_t M, int32_t N, int32_t K, int32_t sa, int32_t sb, int32_t sd0,

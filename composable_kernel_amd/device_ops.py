@@ -204,6 +204,55 @@ class DeviceGemmF16(_DeviceGemm):
                                        C.c_void_p(stream or 0))
 
 
+class _DeviceGemmSplitK(_DeviceGemm):
+    """DeviceGemmSplitK<...> (device_gemm_splitk.hpp:14-39): MakeArgumentPointer takes a trailing KBatch.
+    The workspace (GetWorkSpaceSize) is REQUIRED for KBatch > 1."""
+
+    def MakeArgumentPointer(self, p_a, p_b, p_c, M, N, K, StrideA, StrideB, StrideC, a_element_op=None,
+                            b_element_op=None, c_element_op=None, KBatch=1):
+        a = super().MakeArgumentPointer(p_a, p_b, p_c, M, N, K, StrideA, StrideB, StrideC, a_element_op,
+                                        b_element_op, c_element_op)
+        a.KBatch = int(KBatch)
+        return a
+
+    def GetWorkSpaceSize(self, a):
+        return int(capi.lib().ckx_gemm_splitk_workspace_bytes(self.op_family, a.M, a.N, a.K, a.KBatch))
+
+
+class DeviceGemmSplitKInt8(_DeviceGemmSplitK):
+    op_family = capi.OP_GEMM_I8
+
+    def _supported(self, a):
+        if not 1 <= a.KBatch <= 8 or self.instance >= capi.lib().ckx_num_instances(capi.OP_CONV2D_FWD_I8):
+            capi.lib().ckx_gemm_i8_is_supported(-1, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0)
+            return capi.UNSUPPORTED
+        return capi.lib().ckx_gemm_i8_is_supported(a.M, a.N, a.K, a.StrideA, a.StrideB, a.StrideC,
+                                                   *self.layouts, a.c_op.epilogue, self.instance)
+
+    def _launch(self, a, stream):
+        return capi.lib().ckx_gemm_i8_splitk(a.p_a, a.p_b, a.p_c, a.M, a.N, a.K, a.StrideA, a.StrideB, a.StrideC,
+                                             *self.layouts, a.c_op.epilogue, a.c_op.scale_gemm, a.c_op.scale_relu,
+                                             self.instance, a.KBatch, a.p_workspace_ or 0, a.workspace_bytes_,
+                                             C.c_void_p(stream or 0))
+
+
+class DeviceGemmSplitKF16(_DeviceGemmSplitK):
+    op_family = capi.OP_GEMM_F16
+
+    def _supported(self, a):
+        if (not 1 <= a.KBatch <= 8 or self.instance >= capi.lib().ckx_num_instances(capi.OP_CONV2D_FWD_F16)
+                or not isinstance(a.c_op, PassThrough)):
+            capi.lib().ckx_gemm_f16_is_supported(-1, 0, 0, 0, 0, 0, 0, 0, 0, 0)
+            return capi.UNSUPPORTED
+        return capi.lib().ckx_gemm_f16_is_supported(a.M, a.N, a.K, a.StrideA, a.StrideB, a.StrideC,
+                                                    *self.layouts, self.instance)
+
+    def _launch(self, a, stream):
+        return capi.lib().ckx_gemm_f16_splitk(a.p_a, a.p_b, a.p_c, a.M, a.N, a.K, a.StrideA, a.StrideB, a.StrideC,
+                                              *self.layouts, self.instance, a.KBatch, a.p_workspace_ or 0,
+                                              a.workspace_bytes_, C.c_void_p(stream or 0))
+
+
 class DeviceGemmMultipleDF16(BaseOperator):
     """DeviceGemmMultipleD<Row, Col, Row, half_t, half_t, Tuple<half_t[, half_t]>, half_t, PassThrough,
     PassThrough, CDEOp> (device_gemm_multiple_d.hpp:14-55): E = cde_op(A*B, D0[, D1])."""

@@ -254,6 +254,20 @@ struct DeviceBatchedGemmGemm : public BaseOperator
     virtual std::unique_ptr<BaseInvoker> MakeInvokerPointer()                                     = 0;
 };
 
+// device_gemm_splitk.hpp:14-39
+template <typename ALayout, typename BLayout, typename CLayout, typename ADataType, typename BDataType,
+          typename CDataType, typename AElementwiseOperation, typename BElementwiseOperation,
+          typename CElementwiseOperation>
+struct DeviceGemmSplitK : public BaseOperator
+{
+    virtual std::unique_ptr<BaseArgument>
+    MakeArgumentPointer(const void* p_a, const void* p_b, void* p_c, index_t M, index_t N, index_t K,
+                        index_t StrideA, index_t StrideB, index_t StrideC, AElementwiseOperation a_element_op,
+                        BElementwiseOperation b_element_op, CElementwiseOperation c_element_op,
+                        index_t KBatch)                       = 0;
+    virtual std::unique_ptr<BaseInvoker> MakeInvokerPointer() = 0;
+};
+
 // device_gemm_multiple_d.hpp:14-55
 template <typename ALayout, typename BLayout, typename DELayout, typename ADataType, typename BDataType,
           typename DsDataType, typename EDataType, typename AElementwiseOperation, typename BElementwiseOperation,
@@ -549,6 +563,88 @@ struct DeviceConv2dFwdMfma_Input_N_Hi_Wi_C_Weight_K_Y_X_C_Output_N_Ho_Wo_K
             return is_i8 ? "DeviceConv2dFwd_i8_nhwc_kyxc_nhwk<auto>" : "DeviceConv2dFwd_f16_nhwc_kyxc_nhwk<auto>";
         return ckx_instance_name(op_code, instance_);
     }
+    int instance_;
+};
+
+// ------------------------------------------------------------------ split-K GEMM
+// KBatch runs over K, raw accumulators in the workspace (GetWorkSpaceSize / SetWorkSpacePointer,
+// REQUIRED for KBatch > 1), summed in run order by a second kernel: deterministic, int8 bit-identical
+// to the unsplit operator.
+template <typename ALayout, typename BLayout, typename CLayout, typename ADataType, typename BDataType,
+          typename CDataType, typename AElementwiseOperation, typename BElementwiseOperation,
+          typename CElementwiseOperation>
+struct DeviceGemmSplitKMfma : public DeviceGemmSplitK<ALayout, BLayout, CLayout, ADataType, BDataType, CDataType,
+                                                      AElementwiseOperation, BElementwiseOperation,
+                                                      CElementwiseOperation>
+{
+    using Plain = DeviceGemmMfma<ALayout, BLayout, CLayout, ADataType, BDataType, CDataType, AElementwiseOperation,
+                                 BElementwiseOperation, CElementwiseOperation>;
+    static constexpr bool is_i8 = Plain::is_i8;
+    using Epi                   = typename Plain::Epi;
+    struct Argument : public Plain::Argument
+    {
+        index_t KBatch;
+        Argument(const void* a, const void* b, void* c, index_t m, index_t n, index_t k, index_t sa, index_t sb,
+                 index_t sc, CElementwiseOperation cop, index_t kbatch)
+            : Plain::Argument(a, b, c, m, n, k, sa, sb, sc, cop), KBatch(kbatch)
+        {
+        }
+    };
+    static int64_t WorkSpaceBytes(const Argument& a)
+    {
+        return ckx_gemm_splitk_workspace_bytes(is_i8 ? CKX_OP_GEMM_I8 : CKX_OP_GEMM_F16, a.M, a.N, a.K, a.KBatch);
+    }
+    static int Supported(const Argument& a, int inst)
+    {
+        if(a.KBatch < 1 || a.KBatch > 8 || inst >= ckx_num_instances(CKX_OP_CONV2D_FWD_F16))
+            return CKX_UNSUPPORTED;
+        return Plain::Supported(a, inst);
+    }
+    static int Launch(const Argument& a, int inst, void* stream)
+    {
+        const int64_t ws_bytes = a.p_workspace_ ? WorkSpaceBytes(a) : 0;
+        if constexpr(is_i8)
+            return ckx_gemm_i8_splitk(a.p_a, a.p_b, a.p_c, a.M, a.N, a.K, a.StrideA, a.StrideB, a.StrideC,
+                                      ALayout::code, BLayout::code, CLayout::code, Epi::kind,
+                                      Epi::scale_gemm(a.c_element_op), Epi::scale_relu(a.c_element_op), inst,
+                                      a.KBatch, a.p_workspace_, ws_bytes, stream);
+        else
+            return ckx_gemm_f16_splitk(a.p_a, a.p_b, a.p_c, a.M, a.N, a.K, a.StrideA, a.StrideB, a.StrideC,
+                                       ALayout::code, BLayout::code, CLayout::code, inst, a.KBatch, a.p_workspace_,
+                                       ws_bytes, stream);
+    }
+    using Invoker = detail::InvokerT<Argument, &Supported, &Launch>;
+
+    explicit DeviceGemmSplitKMfma(int instance = CKX_INSTANCE_AUTO) : instance_(instance) {}
+    static Argument MakeArgument(const ADataType* p_a, const BDataType* p_b, CDataType* p_c, index_t M, index_t N,
+                                 index_t K, index_t StrideA, index_t StrideB, index_t StrideC,
+                                 AElementwiseOperation, BElementwiseOperation, CElementwiseOperation c_element_op,
+                                 index_t KBatch)
+    {
+        return Argument{p_a, p_b, p_c, M, N, K, StrideA, StrideB, StrideC, c_element_op, KBatch};
+    }
+    Invoker MakeInvoker() const { return Invoker{instance_}; }
+    bool IsSupportedArgument(const Argument& a) const { return Supported(a, instance_) == CKX_OK; }
+    bool IsSupportedArgument(const BaseArgument* p) override
+    {
+        const auto* a = dynamic_cast<const Argument*>(p);
+        return a && IsSupportedArgument(*a);
+    }
+    size_t GetWorkSpaceSize(const BaseArgument* p) const override
+    {
+        const auto* a = dynamic_cast<const Argument*>(p);
+        return a ? (size_t)WorkSpaceBytes(*a) : 0;
+    }
+    std::unique_ptr<BaseArgument> MakeArgumentPointer(const void* p_a, const void* p_b, void* p_c, index_t M,
+                                                      index_t N, index_t K, index_t StrideA, index_t StrideB,
+                                                      index_t StrideC, AElementwiseOperation,
+                                                      BElementwiseOperation, CElementwiseOperation c_element_op,
+                                                      index_t KBatch) override
+    {
+        return std::make_unique<Argument>(p_a, p_b, p_c, M, N, K, StrideA, StrideB, StrideC, c_element_op, KBatch);
+    }
+    std::unique_ptr<BaseInvoker> MakeInvokerPointer() override { return std::make_unique<Invoker>(instance_); }
+    std::string GetTypeString() const override { return Plain(instance_).GetTypeString() + " + SplitK"; }
     int instance_;
 };
 

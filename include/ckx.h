@@ -118,6 +118,24 @@ int ckx_gemm_f16(const void* p_a, const void* p_b, void* p_c, int32_t M, int32_t
                  int c_layout, int instance, void* p_workspace, int64_t workspace_bytes, void* stream);
 int64_t ckx_gemm_f16_workspace_bytes(int32_t M, int32_t N, int32_t K, int instance);
 
+/* ---- split-K GEMM with a caller-chosen number of K runs ----------------------
+ * Replaces DeviceGemmSplitK<...>::MakeArgumentPointer(..., KBatch) + Run (device_gemm_splitk.hpp:14-39).
+ * The K extent is cut into k_batch (1..8) runs of whole 128-byte K tiles (fewer when K has fewer tiles);
+ * the runs' raw int32 / fp32 accumulators go to the workspace and a second kernel adds them in run
+ * order and applies the epilogue: deterministic, and for int8 bit-identical to the unsplit GEMM
+ * (the reference adds with atomics into a zeroed C instead). k_batch > 1 requires a workspace of
+ * ckx_gemm_splitk_workspace_bytes(op, M, N, K, k_batch) bytes (op = CKX_OP_GEMM_I8 / _F16).
+ * Supported shapes are those of ckx_gemm_*_is_supported with a tile instance (or AUTO). */
+int64_t ckx_gemm_splitk_workspace_bytes(int op, int32_t M, int32_t N, int32_t K, int32_t k_batch);
+int ckx_gemm_i8_splitk(const void* p_a, const void* p_b, void* p_c, int32_t M, int32_t N, int32_t K,
+                       int32_t stride_a, int32_t stride_b, int32_t stride_c, int a_layout, int b_layout,
+                       int c_layout, int epilogue, float scale_gemm, float scale_relu, int instance,
+                       int32_t k_batch, void* p_workspace, int64_t workspace_bytes, void* stream);
+int ckx_gemm_f16_splitk(const void* p_a, const void* p_b, void* p_c, int32_t M, int32_t N, int32_t K,
+                        int32_t stride_a, int32_t stride_b, int32_t stride_c, int a_layout, int b_layout,
+                        int c_layout, int instance, int32_t k_batch, void* p_workspace, int64_t workspace_bytes,
+                        void* stream);
+
 /* ---- fp16 GEMM with fused D operands:  E = cde_op(A * B, D0 [, D1]) ----------
  * Replaces DeviceGemmMultipleD<..., Tuple<half_t[, half_t]>, half_t, PassThrough, PassThrough, CDEOp>
  * ::MakeArgumentPointer + Run (device_gemm_multiple_d.hpp:14-55) for cde_op in

@@ -126,3 +126,15 @@ def test_profiler_gemm_bias_relu(tmp_path):
     c = np.fromfile(dump, np.float16).reshape(M, N)
     bad, max_err = lit.check_err_f16(c, lit.gemm_f16_add_relu(a, b_nk.T, d[None, :]), 1e-2, 1e-2)
     assert bad == 0, max_err
+
+
+def test_profiler_gemm_splitk_int8(tmp_path):
+    """profile_gemm_splitk's argument list (KBatch = arg14); PassThrough int8 output keeps the low byte."""
+    M, N, K = 128, 512, 4096
+    out, dump = _run("ckx_profiler", ["gemm_splitk", 3, 1, 1, 1, 0, 1, M, N, K, -1, -1, -1, 4], "CKX_PROFILER_DUMP",
+                     tmp_path)
+    assert "Best Perf:" in out and "Error" not in out and "SplitK" in out
+    c = np.fromfile(dump, np.int8).reshape(M, N)
+    a = uniform_int8((M, K), -5, 5, SEED)
+    b_nk = uniform_int8((N, K), -5, 5, SEED + 1)
+    np.testing.assert_array_equal(c, fast.gemm_i8(a, b_nk.T))

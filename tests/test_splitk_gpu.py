@@ -142,3 +142,57 @@ def test_auto_instance_few_rows_routing_bit_exact(shape):
     outf, _ = _run_gemm(ck.DeviceGemmF16(), af, bf, torch.float16)
     reff = fast.gemm_f16(af, bf.T)
     assert np.all(np.abs(outf.astype(np.float32) - reff.astype(np.float32)) <= 1e-2 + 1e-2 * np.abs(reff.astype(np.float32)))
+
+
+def _run_splitk(op, a, b_nk, c_dtype, kbatch, c_op=None, give_workspace=True):
+    import torch
+    import gpu_util
+    M, K = a.shape
+    N = b_nk.shape[0]
+    da, db = gpu_util.dev(a), gpu_util.dev(b_nk)
+    dc = torch.zeros((M, N), dtype=c_dtype, device="cuda")
+    arg = op.MakeArgumentPointer(da, db, dc, M, N, K, K, K, N, None, None, c_op, kbatch)
+    if not op.IsSupportedArgument(arg):
+        return None, 0
+    need = op.GetWorkSpaceSize(arg)
+    if give_workspace:
+        ws = torch.full((max(need, 16),), 0x7F, dtype=torch.uint8, device="cuda")
+        op.SetWorkSpacePointer(arg, ws)
+    st = op._launch(arg, gpu_util.stream())
+    torch.cuda.synchronize()
+    return (dc.cpu().numpy() if st == 0 else st), need
+
+
+@pytest.mark.parametrize("kbatch", [1, 2, 4, 8])
+@pytest.mark.parametrize("shape", [(128, 320, 4096), (130, 200, 2064), (16, 64, 256)])
+def test_device_gemm_splitk_kbatch_argument(shape, kbatch):
+    """DeviceGemmSplitK's KBatch (device_gemm_splitk.hpp:14-39): the caller fixes the number of K runs.
+    int8 is bit-identical to the unsplit result for every KBatch; fp16 within tolerance; a K with
+    fewer 128-byte tiles than KBatch uses fewer runs."""
+    import torch
+    M, N, K = shape
+    a = uniform_int8((M, K), -8, 8, 170 + M)
+    b_nk = uniform_int8((N, K), -8, 8, 171 + N)
+    out, need = _run_splitk(ck.DeviceGemmSplitKInt8(), a, b_nk, torch.int8, kbatch,
+                            ck.RequantReluRequant(0.02, 0.4, rounded=True))
+    nk = (K + 127) // 128
+    runs = next(sp for sp in range(min(kbatch, 8), 0, -1) if sp == 1 or -(-nk // sp) * (sp - 1) < nk)
+    assert need == (runs * M * N * 4 if runs > 1 else 0)
+    np.testing.assert_array_equal(out, fast.gemm_i8(a, b_nk.T, lit.EPI_REQUANT_RND, 0.02, 0.4))
+    af, bf = uniform_f16((M, K // 2), -1, 1, 172 + M), uniform_f16((N, K // 2), -1, 1, 173 + N)
+    outf, _ = _run_splitk(ck.DeviceGemmSplitKF16(3), af, bf, torch.float16, kbatch)
+    bad, max_err = lit.check_err_f16(outf, fast.gemm_f16(af, bf.T), 1e-2, 1e-2)
+    assert bad == 0, max_err
+
+
+def test_device_gemm_splitk_rejects_missing_workspace_and_bad_kbatch():
+    import torch
+    a = uniform_int8((64, 1024), -8, 8, 1)
+    b_nk = uniform_int8((64, 1024), -8, 8, 2)
+    st, need = _run_splitk(ck.DeviceGemmSplitKInt8(), a, b_nk, torch.int8, 4, ck.PassThrough(), give_workspace=False)
+    assert need == 4 * 64 * 64 * 4 and st == capi.INVALID_VALUE and "workspace" in capi.last_error()
+    out, _ = _run_splitk(ck.DeviceGemmSplitKInt8(), a, b_nk, torch.int8, 9, ck.PassThrough())
+    assert out is None
+    out, _ = _run_splitk(ck.DeviceGemmSplitKInt8(capi.lib().ckx_num_instances(capi.OP_CONV2D_FWD_I8)), a, b_nk,
+                         torch.int8, 2, ck.PassThrough())
+    assert out is None      # a skinny instance
