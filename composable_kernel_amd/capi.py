@@ -15,7 +15,7 @@ OK, UNSUPPORTED, INVALID_VALUE, HIP_ERROR = 0, -1, -2, -3
 ROW_MAJOR, COL_MAJOR = 0, 1
 EPI_PASSTHROUGH, EPI_REQUANT_CK, EPI_REQUANT_RND = 0, 1, 2
 EPI_ADD_RELU, EPI_ADD_RELU_ADD, EPI_CSHUFFLE_ADD_RELU = 3, 4, 5
-OP_GEMM_I8, OP_GEMM_F16, OP_CONV2D_FWD_I8, OP_CONV2D_FWD_F16, OP_BATCHED_GEMM_GEMM = range(5)
+OP_GEMM_I8, OP_GEMM_F16, OP_CONV2D_FWD_I8, OP_CONV2D_FWD_F16, OP_BATCHED_GEMM_GEMM, OP_GEMM_SPLITK = range(6)
 INSTANCE_AUTO = -1
 
 # every symbol include/ckx.h declares

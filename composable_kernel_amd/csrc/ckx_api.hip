@@ -12,6 +12,7 @@
 #include "ckx.h"
 #include "gemm_tile.hpp"
 #include "gemm_gemm.hpp"
+#include "conv_patch.hpp"
 #include "gemm_skinny.hpp"
 
 namespace {
@@ -260,6 +261,7 @@ const char* family_prefix(int op)
     case CKX_OP_CONV2D_FWD_I8: return "DeviceConv2dFwd_i8_nhwc_kyxc_nhwk";
     case CKX_OP_CONV2D_FWD_F16: return "DeviceConv2dFwd_f16_nhwc_kyxc_nhwk";
     case CKX_OP_BATCHED_GEMM_GEMM: return "DeviceBatchedGemmGemm_f16_gmk_gnk_gno_gmo";
+    case CKX_OP_GEMM_SPLITK: return "DeviceGemmSplitK_mk_nk_mn";
     default: return nullptr;
     }
 }
@@ -406,6 +408,34 @@ int run_gemm(int dt, const void* a, const void* b, void* c, int M, int N, int K,
     return CKX_OK;
 }
 
+// ---------------------------------------------------------- input-patch conv kernel
+const char* const kPatchName = "MI355X_Mfma16_Patch<4 rows x 56, 3x3, C 64, K 64, waves 2x2>";
+
+// shapes the input-patch kernel covers (one instantiation: 3x3 taps, Wo = 56)
+bool conv_patch_applicable(int op, const ckx_conv2d_desc* d, int epi)
+{
+    return op == CKX_OP_CONV2D_FWD_F16 && epi == CKX_EPI_PASSTHROUGH && d->C == 64 && d->K == 64 && d->Y == 3 &&
+           d->X == 3 && d->stride_h == 1 && d->stride_w == 1 && d->dilation_h == 1 && d->dilation_w == 1 &&
+           d->Wo == 56 && d->Ho >= 1 && d->N >= 1 && d->pad_left <= 2 && d->pad_top <= 2;
+}
+
+hipError_t launch_conv_patch(const ckx::ConvPatchArgs& a, hipStream_t s)
+{
+    using T    = ckx::ConvPatch<7, 3, 3>;
+    auto* kern = &ckx::conv_patch_kernel<7, 3, 3>;
+    static std::once_flag once;
+    static hipError_t attr_err = hipSuccess;
+    std::call_once(once, [&] {
+        attr_err = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, T::LDS);
+    });
+    if(attr_err != hipSuccess)
+        return attr_err;
+    const int grid = a.N < num_cus() ? a.N : num_cus();
+    hipLaunchKernelGGL(kern, dim3(grid), dim3(T::NT), T::LDS, s, a);
+    return hipGetLastError();
+}
+
 int check_conv(int op, const ckx_conv2d_desc* d, int epi, int instance)
 {
     if(!d)
@@ -413,7 +443,7 @@ int check_conv(int op, const ckx_conv2d_desc* d, int epi, int instance)
     if(op != CKX_OP_CONV2D_FWD_I8 && op != CKX_OP_CONV2D_FWD_F16)
         return fail(CKX_INVALID_VALUE, "not a conv operator family");
     const int es = op == CKX_OP_CONV2D_FWD_I8 ? 1 : 2;
-    if(instance != CKX_INSTANCE_AUTO && (instance < 0 || instance >= kNumTiles))
+    if(instance != CKX_INSTANCE_AUTO && (instance < 0 || instance >= kNumTiles + (es == 2 ? 1 : 0)))
         return fail(CKX_INVALID_VALUE, "no such instance");
     if(epi < CKX_EPI_PASSTHROUGH || epi > CKX_EPI_CSHUFFLE_ADD_RELU || !epilogue_fits_dtype(es, epi) ||
        epi == CKX_EPI_CSHUFFLE_ADD_RELU)
@@ -441,6 +471,9 @@ int check_conv(int op, const ckx_conv2d_desc* d, int epi, int instance)
     if(in_b >= (1l << 31) || wei_b >= (1l << 31) || out_b >= (1l << 31) ||
        (long)d->N * d->Ho * d->Wo >= (1l << 31))
         return fail(CKX_UNSUPPORTED, "tensors of 2 GiB or more are not addressed");
+    if(instance == kNumTiles && !conv_patch_applicable(op, d, epi))
+        return fail(CKX_UNSUPPORTED, "the input-patch instance covers fp16 3x3 stride-1 layers with C = K = 64, Wo = 56, "
+                                     "PassThrough output");
     return CKX_OK;
 }
 
@@ -449,6 +482,8 @@ long conv_workspace_bytes(int op, const ckx_conv2d_desc* d, int instance)
     const int es = op == CKX_OP_CONV2D_FWD_I8 ? 1 : 2;
     const long M = (long)d->N * d->Ho * d->Wo;
     if(M <= 0 || d->K <= 0)
+        return 0;
+    if(instance == kNumTiles || (instance == CKX_INSTANCE_AUTO && conv_patch_applicable(op, d, CKX_EPI_PASSTHROUGH)))
         return 0;
     const Plan pl = make_plan((int)M, d->K, d->Y * d->X * d->C * es, instance, 1l << 60);
     return pl.ksplit > 1 ? (long)pl.ksplit * M * d->K * 4 : 0;
@@ -472,6 +507,24 @@ int run_conv(int op, const void* in, const void* wei, void* out, const ckx_conv2
         return fail(CKX_UNSUPPORTED, "input and weight must be 16-byte aligned");
     if(ws && (reinterpret_cast<uintptr_t>(ws) & 15))
         return fail(CKX_INVALID_VALUE, "workspace must be 16-byte aligned");
+    if(instance == kNumTiles || (instance == CKX_INSTANCE_AUTO && conv_patch_applicable(op, d, epi) &&
+                                 !(reinterpret_cast<uintptr_t>(out) & 15)))
+    {
+        if(reinterpret_cast<uintptr_t>(out) & 15)
+            return fail(CKX_UNSUPPORTED, "the input-patch instance needs a 16-byte aligned output");
+        ckx::ConvPatchArgs a;
+        std::memset(&a, 0, sizeof(a));
+        a.in = in, a.wei = wei, a.out = out;
+        a.in_bytes  = (uint32_t)((long)d->N * d->Hi * d->Wi * d->C * es);
+        a.wei_bytes = (uint32_t)((long)N * K * es);
+        a.N = d->N, a.Hi = d->Hi, a.Wi = d->Wi, a.Ho = d->Ho, a.Wo = d->Wo;
+        a.pT = d->pad_top, a.pL = d->pad_left;
+        a.nbands = (d->Ho + 3) / 4;
+        a.div_wo = make_magic((uint32_t)d->Wo);
+        a.epi    = epi;
+        hipError_t e = launch_conv_patch(a, (hipStream_t)stream);
+        return e == hipSuccess ? CKX_OK : hip_fail(e, kPatchName);
+    }
     const Plan pl = make_plan(M, N, K * es, instance, ws ? ws_bytes : 0);
     const TileInstance& t = kTiles[pl.tile];
     ckx::GemmArgs g;
@@ -519,8 +572,10 @@ int ckx_num_instances(int op)
 {
     if(op == CKX_OP_GEMM_I8 || op == CKX_OP_GEMM_F16)
         return kNumGemmInsts;
-    if(op == CKX_OP_CONV2D_FWD_I8 || op == CKX_OP_CONV2D_FWD_F16)
+    if(op == CKX_OP_CONV2D_FWD_I8 || op == CKX_OP_GEMM_SPLITK)
         return kNumTiles;
+    if(op == CKX_OP_CONV2D_FWD_F16)
+        return kNumTiles + 1; // + the input-patch kernel
     if(op == CKX_OP_BATCHED_GEMM_GEMM)
         return ckx::kNumGemmGemmInstances;
     return 0;
@@ -534,8 +589,9 @@ const char* ckx_instance_name(int op, int instance)
         return nullptr;
     s = std::string(fam) + "<" +
         (op == CKX_OP_BATCHED_GEMM_GEMM ? ckx::gemm_gemm_instance_name(instance)
-         : instance >= kNumTiles        ? kSkinny[instance - kNumTiles].name
-                                        : kTiles[instance].name) +
+         : op == CKX_OP_CONV2D_FWD_F16 && instance == kNumTiles
+             ? kPatchName
+             : instance >= kNumTiles ? kSkinny[instance - kNumTiles].name : kTiles[instance].name) +
         ">";
     return s.c_str();
 }

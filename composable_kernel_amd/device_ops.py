@@ -223,7 +223,7 @@ class DeviceGemmSplitKInt8(_DeviceGemmSplitK):
     op_family = capi.OP_GEMM_I8
 
     def _supported(self, a):
-        if not 1 <= a.KBatch <= 8 or self.instance >= capi.lib().ckx_num_instances(capi.OP_CONV2D_FWD_I8):
+        if not 1 <= a.KBatch <= 8 or self.instance >= capi.lib().ckx_num_instances(capi.OP_GEMM_SPLITK):
             capi.lib().ckx_gemm_i8_is_supported(-1, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0)
             return capi.UNSUPPORTED
         return capi.lib().ckx_gemm_i8_is_supported(a.M, a.N, a.K, a.StrideA, a.StrideB, a.StrideC,
@@ -240,7 +240,7 @@ class DeviceGemmSplitKF16(_DeviceGemmSplitK):
     op_family = capi.OP_GEMM_F16
 
     def _supported(self, a):
-        if (not 1 <= a.KBatch <= 8 or self.instance >= capi.lib().ckx_num_instances(capi.OP_CONV2D_FWD_F16)
+        if (not 1 <= a.KBatch <= 8 or self.instance >= capi.lib().ckx_num_instances(capi.OP_GEMM_SPLITK)
                 or not isinstance(a.c_op, PassThrough)):
             capi.lib().ckx_gemm_f16_is_supported(-1, 0, 0, 0, 0, 0, 0, 0, 0, 0)
             return capi.UNSUPPORTED

@@ -596,7 +596,7 @@ struct DeviceGemmSplitKMfma : public DeviceGemmSplitK<ALayout, BLayout, CLayout,
     }
     static int Supported(const Argument& a, int inst)
     {
-        if(a.KBatch < 1 || a.KBatch > 8 || inst >= ckx_num_instances(CKX_OP_CONV2D_FWD_F16))
+        if(a.KBatch < 1 || a.KBatch > 8 || inst >= ckx_num_instances(CKX_OP_GEMM_SPLITK))
             return CKX_UNSUPPORTED;
         return Plain::Supported(a, inst);
     }

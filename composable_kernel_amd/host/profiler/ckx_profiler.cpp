@@ -291,7 +291,7 @@ int profile_gemm_splitk_t(bool verify, int init, bool time_kernel, int M, int N,
 {
     using DeviceOp = device::DeviceGemmSplitK<Row, Col, Row, T, T, T, Pass, Pass, Pass>;
     std::vector<std::unique_ptr<DeviceOp>> ops;
-    for(int i = 0, n = ckx_num_instances(CKX_OP_CONV2D_FWD_F16); i < n; ++i) // the tile instances
+    for(int i = 0, n = ckx_num_instances(CKX_OP_GEMM_SPLITK); i < n; ++i)
         ops.push_back(std::make_unique<device::DeviceGemmSplitKMfma<Row, Col, Row, T, T, T, Pass, Pass, Pass>>(i));
     std::vector<T> a((std::size_t)M * sa), b((std::size_t)N * sb);
     fill(a, init, 0xC0FFEE, false);

@@ -71,7 +71,8 @@ enum
     CKX_OP_GEMM_F16          = 1,
     CKX_OP_CONV2D_FWD_I8     = 2,
     CKX_OP_CONV2D_FWD_F16    = 3,
-    CKX_OP_BATCHED_GEMM_GEMM = 4
+    CKX_OP_BATCHED_GEMM_GEMM = 4,
+    CKX_OP_GEMM_SPLITK       = 5 /* instance list of the split-K GEMMs (the tile instances, both dtypes) */
 };
 
 #define CKX_INSTANCE_AUTO (-1)

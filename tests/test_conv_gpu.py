@@ -139,3 +139,49 @@ def test_conv2d_unsupported_arguments_are_refused():
     # output size inconsistent with the geometry
     arg = op.MakeArgumentPointer(d, d, d, 1, 8, 16, [8, 8], [3, 3], [7, 6], [1, 1], [1, 1], [0, 0], [0, 0])
     assert not op.IsSupportedArgument(arg)
+
+
+# (N, Hi, Wi, pads): fp16, C = K = 64, 3x3, stride 1, dilation 1, Wo = 56 -- the input-patch kernel's shapes
+PATCH = [
+    (2, 9, 56, (1, 1)),       # partial last band (Ho = 9)
+    (1, 4, 56, (1, 1)),       # a single band
+    (3, 12, 58, (1, 0)),      # no horizontal padding
+    (2, 7, 54, (0, 2)),       # wide horizontal padding, none vertically (Ho = 5)
+    (1, 56, 56, (1, 1)),      # the ResNet-50 conv2_x layer, one image
+]
+
+
+@pytest.mark.parametrize("case", PATCH)
+@pytest.mark.parametrize("auto", [True, False])
+def test_conv2d_fp16_input_patch_kernel(case, auto):
+    """The LDS-resident input-patch kernel (explicit instance and automatic choice) against the
+    literal oracle; the tile kernel must agree on the same problem."""
+    import gpu_util
+    N, Hi, Wi, p = case
+    inp = uniform_f16((N, Hi, Wi, 64), -1, 1, 900 + Hi)
+    wei = uniform_f16((64, 3, 3, 64), -1, 1, 901 + Wi)
+    patch = capi.lib().ckx_num_instances(capi.OP_CONV2D_FWD_F16) - 1
+    assert b"Patch" in capi.lib().ckx_instance_name(capi.OP_CONV2D_FWD_F16, patch)
+    out = gpu_util.conv2d_fwd(inp, wei, (1, 1), (1, 1), p, instance=capi.INSTANCE_AUTO if auto else patch)
+    ref = lit.conv2d_fwd(inp, wei, (1, 1), (1, 1), p)
+    assert out.shape == ref.shape and out.shape[2] == 56
+    _f16_close(out, ref)
+    _f16_close(gpu_util.conv2d_fwd(inp, wei, (1, 1), (1, 1), p, instance=7), ref)
+
+
+def test_conv2d_fp16_input_patch_kernel_more_images_than_cus():
+    """Workgroups walk several images: 300 images on at most 256 workgroups."""
+    import gpu_util
+    inp = uniform_f16((300, 5, 56, 64), -1, 1, 77)
+    wei = uniform_f16((64, 3, 3, 64), -0.5, 0.5, 78)
+    out = gpu_util.conv2d_fwd(inp, wei, (1, 1), (1, 1), (1, 1))
+    _f16_close(out, fast.conv2d_fwd_f16(inp, wei, (1, 1), (1, 1), (1, 1)))
+
+
+def test_conv2d_input_patch_instance_refuses_other_shapes():
+    import ctypes as C
+    patch = capi.lib().ckx_num_instances(capi.OP_CONV2D_FWD_F16) - 1
+    d = capi.Conv2dDesc(2, 64, 64, 9, 48, 3, 3, 9, 48, 1, 1, 1, 1, 1, 1, 1, 1)     # Wo = 48
+    assert capi.lib().ckx_conv2d_fwd_is_supported(capi.OP_CONV2D_FWD_F16, C.byref(d), 0, patch) == capi.UNSUPPORTED
+    assert capi.lib().ckx_conv2d_fwd_is_supported(capi.OP_CONV2D_FWD_F16, C.byref(d), 0, -1) == capi.OK
+    assert capi.lib().ckx_conv2d_fwd_is_supported(capi.OP_CONV2D_FWD_I8, C.byref(d), 0, patch) == capi.INVALID_VALUE

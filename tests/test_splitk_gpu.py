@@ -193,6 +193,6 @@ def test_device_gemm_splitk_rejects_missing_workspace_and_bad_kbatch():
     assert need == 4 * 64 * 64 * 4 and st == capi.INVALID_VALUE and "workspace" in capi.last_error()
     out, _ = _run_splitk(ck.DeviceGemmSplitKInt8(), a, b_nk, torch.int8, 9, ck.PassThrough())
     assert out is None
-    out, _ = _run_splitk(ck.DeviceGemmSplitKInt8(capi.lib().ckx_num_instances(capi.OP_CONV2D_FWD_I8)), a, b_nk,
+    out, _ = _run_splitk(ck.DeviceGemmSplitKInt8(capi.lib().ckx_num_instances(capi.OP_GEMM_SPLITK)), a, b_nk,
                          torch.int8, 2, ck.PassThrough())
     assert out is None      # a skinny instance
