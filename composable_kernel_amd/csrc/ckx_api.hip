@@ -414,15 +414,17 @@ const char* const kPatchName = "MI355X_Mfma16_Patch<4 rows x 56, 3x3, C 64, K 64
 // shapes the input-patch kernel covers (one instantiation: 3x3 taps, Wo = 56)
 bool conv_patch_applicable(int op, const ckx_conv2d_desc* d, int epi)
 {
-    return op == CKX_OP_CONV2D_FWD_F16 && epi == CKX_EPI_PASSTHROUGH && d->C == 64 && d->K == 64 && d->Y == 3 &&
+    return op == CKX_OP_CONV2D_FWD_F16 &&
+           (epi == CKX_EPI_PASSTHROUGH || epi == CKX_EPI_ADD_RELU || epi == CKX_EPI_ADD_RELU_ADD) && d->C == 64 && d->K == 64 && d->Y == 3 &&
            d->X == 3 && d->stride_h == 1 && d->stride_w == 1 && d->dilation_h == 1 && d->dilation_w == 1 &&
            d->Wo == 56 && d->Ho >= 1 && d->N >= 1 && d->pad_left <= 2 && d->pad_top <= 2;
 }
 
+template <bool FUSED>
 hipError_t launch_conv_patch(const ckx::ConvPatchArgs& a, hipStream_t s)
 {
-    using T    = ckx::ConvPatch<7, 3, 3>;
-    auto* kern = &ckx::conv_patch_kernel<7, 3, 3>;
+    using T    = ckx::ConvPatch<7, 3, 3, FUSED>;
+    auto* kern = &ckx::conv_patch_kernel<7, 3, 3, FUSED>;
     static std::once_flag once;
     static hipError_t attr_err = hipSuccess;
     std::call_once(once, [&] {
@@ -472,8 +474,7 @@ int check_conv(int op, const ckx_conv2d_desc* d, int epi, int instance)
        (long)d->N * d->Ho * d->Wo >= (1l << 31))
         return fail(CKX_UNSUPPORTED, "tensors of 2 GiB or more are not addressed");
     if(instance == kNumTiles && !conv_patch_applicable(op, d, epi))
-        return fail(CKX_UNSUPPORTED, "the input-patch instance covers fp16 3x3 stride-1 layers with C = K = 64, Wo = 56, "
-                                     "PassThrough output");
+        return fail(CKX_UNSUPPORTED, "the input-patch instance covers fp16 3x3 stride-1 layers with C = K = 64, Wo = 56");
     return CKX_OK;
 }
 
@@ -507,11 +508,12 @@ int run_conv(int op, const void* in, const void* wei, void* out, const ckx_conv2
         return fail(CKX_UNSUPPORTED, "input and weight must be 16-byte aligned");
     if(ws && (reinterpret_cast<uintptr_t>(ws) & 15))
         return fail(CKX_INVALID_VALUE, "workspace must be 16-byte aligned");
-    if(instance == kNumTiles || (instance == CKX_INSTANCE_AUTO && conv_patch_applicable(op, d, epi) &&
-                                 !(reinterpret_cast<uintptr_t>(out) & 15)))
+    const bool patch_aligned = !((reinterpret_cast<uintptr_t>(out) | reinterpret_cast<uintptr_t>(dops.d0) |
+                                  (epi == CKX_EPI_ADD_RELU_ADD ? reinterpret_cast<uintptr_t>(dops.d1) : 0)) & 15);
+    if(instance == kNumTiles || (instance == CKX_INSTANCE_AUTO && conv_patch_applicable(op, d, epi) && patch_aligned))
     {
-        if(reinterpret_cast<uintptr_t>(out) & 15)
-            return fail(CKX_UNSUPPORTED, "the input-patch instance needs a 16-byte aligned output");
+        if(!patch_aligned)
+            return fail(CKX_UNSUPPORTED, "the input-patch instance needs 16-byte aligned output, bias and residual");
         ckx::ConvPatchArgs a;
         std::memset(&a, 0, sizeof(a));
         a.in = in, a.wei = wei, a.out = out;
@@ -522,7 +524,9 @@ int run_conv(int op, const void* in, const void* wei, void* out, const ckx_conv2
         a.nbands = (d->Ho + 3) / 4;
         a.div_wo = make_magic((uint32_t)d->Wo);
         a.epi    = epi;
-        hipError_t e = launch_conv_patch(a, (hipStream_t)stream);
+        a.bias = dops.d0, a.resi = epi == CKX_EPI_ADD_RELU_ADD ? dops.d1 : nullptr;
+        hipError_t e = epi == CKX_EPI_PASSTHROUGH ? launch_conv_patch<false>(a, (hipStream_t)stream)
+                                                  : launch_conv_patch<true>(a, (hipStream_t)stream);
         return e == hipSuccess ? CKX_OK : hip_fail(e, kPatchName);
     }
     const Plan pl = make_plan(M, N, K * es, instance, ws ? ws_bytes : 0);

@@ -42,7 +42,9 @@ struct ConvPatchArgs
     const void* resi; // NHWK fp16
 };
 
-template <int MTW, int Y, int X>
+// FUSED: the add / ReLU epilogues (bias, residual) are compiled in; the plain instantiation keeps
+// their registers free
+template <int MTW, int Y, int X, bool FUSED>
 struct ConvPatch
 {
     static constexpr int TH     = 4;                // output rows per band
@@ -105,6 +107,16 @@ struct ConvPatch
                 coff[t][x]        = cc * PXB + ((fq ^ (cc & 7u)) << 4);
             }
         }
+        // fused add / ReLU epilogues: the lane's 8 bias values once, its residual values band by band
+        const bool has_resi = FUSED && p.epi == EPI_ADD_RELU_ADD;
+        f16x8 bias8 = {0, 0, 0, 0, 0, 0, 0, 0};
+        if constexpr(FUSED)
+            bias8 = *reinterpret_cast<const f16x8*>(reinterpret_cast<const _Float16*>(p.bias) + 32 * wn + 8 * (int)fq);
+        f16x8 resi8[FUSED ? MTW : 1];
+#pragma unroll
+        for(int t = 0; t < (FUSED ? MTW : 1); ++t)
+            resi8[t] = f16x8{0, 0, 0, 0, 0, 0, 0, 0};
+
         uint32_t boff[2]; // weight fragment of n-tile j, k-step 0, tap 0
 #pragma unroll
         for(int j = 0; j < 2; ++j)
@@ -182,6 +194,18 @@ struct ConvPatch
                     for(int r = 0; r < MTW + 2; ++r)
                         read_one(0, r);
                 }
+                // residual values of this band: plain loads, issued before the band's direct loads and
+                // waited for with them (a load issued after the stores would have to wait for those)
+                if constexpr(FUSED)
+                  if(has_resi)
+                {
+                    const uint8_t* resi_band = reinterpret_cast<const uint8_t*>(p.resi) +
+                                               ((size_t)n * p.Ho + (size_t)TH * b) * p.Wo * (KO * sizeof(_Float16));
+#pragma unroll
+                    for(int t = 0; t < MTW; ++t)
+                        if(TH * b + (int)rout[t] < p.Ho)
+                            resi8[FUSED ? t : 0] = *reinterpret_cast<const f16x8*>(resi_band + ooff[t]);
+                }
                 // One k-step = MTW groups pinned in source order: [reads of the NEXT k-step, spread over
                 // the first groups and finished two groups early] [one direct load of the next band's
                 // rows] [the 2 MFMAs of one M tile]. With one wave per SIMD nothing else hides the
@@ -244,8 +268,14 @@ struct ConvPatch
 #pragma unroll
                         for(int i = 0; i < 4; ++i)
                         {
-                            o[i]     = (_Float16)acc[t][0][i];
-                            o[4 + i] = (_Float16)acc[t][1][i];
+                            float v0 = acc[t][0][i], v1 = acc[t][1][i];
+                            if constexpr(FUSED)
+                            {
+                                v0 = epi_f16_value(p.epi, v0, (float)bias8[i], (float)resi8[t][i]);
+                                v1 = epi_f16_value(p.epi, v1, (float)bias8[4 + i], (float)resi8[t][4 + i]);
+                            }
+                            o[i]     = (_Float16)v0;
+                            o[4 + i] = (_Float16)v1;
                         }
                         *reinterpret_cast<f16x8*>(reinterpret_cast<uint8_t*>(out_band) + ooff[t]) = o;
                     }
@@ -259,11 +289,11 @@ struct ConvPatch
     }
 };
 
-template <int MTW, int Y, int X>
+template <int MTW, int Y, int X, bool FUSED>
 __global__ __launch_bounds__(256) void conv_patch_kernel(const ConvPatchArgs p)
 {
     extern __shared__ __attribute__((aligned(1024))) uint8_t ckx_patch_smem[];
-    ConvPatch<MTW, Y, X>::run(p, ckx_patch_smem);
+    ConvPatch<MTW, Y, X, FUSED>::run(p, ckx_patch_smem);
 }
 
 } // namespace ckx

@@ -195,3 +195,21 @@ def test_fused_epilogue_argument_checks():
     import ctypes as C
     assert L.ckx_conv2d_fwd_bias_activation_f16(1, 1, 1, 0, 0, C.byref(d), capi.EPI_ADD_RELU, -1, 0, 0, None) == capi.INVALID_VALUE
     assert L.ckx_conv2d_fwd_is_supported(capi.OP_CONV2D_FWD_I8, C.byref(d), capi.EPI_ADD_RELU, -1) != capi.OK
+
+
+@pytest.mark.parametrize("shape", [(2, 9, 56, (1, 1)), (1, 56, 56, (1, 1)), (3, 6, 58, (0, 0))])
+@pytest.mark.parametrize("auto", [True, False])
+def test_conv2d_bias_relu_on_the_input_patch_kernel(shape, auto):
+    """ResNet conv2_x shapes (C = K = 64, 3x3, Wo = 56) take the input-patch kernel, fused functors included."""
+    N, Hi, Wi, p = shape
+    inp = uniform_f16((N, Hi, Wi, 64), -1, 1, 950 + Hi)
+    wei = uniform_f16((64, 3, 3, 64), -0.5, 0.5, 951)
+    bias = uniform_f16((64,), -2, 2, 952)
+    inst = capi.INSTANCE_AUTO if auto else capi.lib().ckx_num_instances(capi.OP_CONV2D_FWD_F16) - 1
+    ref = lit.conv2d_fwd_bias_relu_f16(inp, wei, bias, None, (1, 1), (1, 1), p)
+    out = _conv(inp, wei, bias, None, (1, 1), (1, 1), p, inst)
+    _close(out, ref)
+    assert (out == 0).any() and (out > 0).any()
+    resi = uniform_f16(ref.shape, -2, 2, 953)
+    _close(_conv(inp, wei, bias, resi, (1, 1), (1, 1), p, inst),
+           lit.conv2d_fwd_bias_relu_f16(inp, wei, bias, resi, (1, 1), (1, 1), p))
