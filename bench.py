@@ -47,11 +47,12 @@ def _conv_workload(name, dtype, C, K, f, HW, st, pd, N=256, fused=None):
                 fused=fused)
 
 
-def _gemm_workload(name, dtype, M, N, K, values=5, scales=(0.5, 0.03), fused=None):
-    """fused: None or "bias_relu" (fp16: E = AddRelu(half(A*B), bias row))."""
+def _gemm_workload(name, dtype, M, N, K, values=5, scales=(0.5, 0.03), fused=None, batch=1):
+    """fused: None or "bias_relu" (fp16: E = AddRelu(half(A*B), bias row)); batch > 1: strided batched GEMM."""
     es = 1 if dtype == "i8" else 2
-    return dict(name=name, kind="gemm", dtype=dtype, M=M, N=N, K=K, values=values, scales=scales,
-                ops=2.0 * M * N * K, bytes=(M * K + N * K + M * N + (N if fused else 0)) * es, fused=fused)
+    return dict(name=name, kind="gemm", dtype=dtype, M=M, N=N, K=K, values=values, scales=scales, batch=batch,
+                ops=2.0 * M * N * K * batch, bytes=(M * K + N * K + M * N + (N if fused else 0)) * es * batch,
+                fused=fused)
 
 
 WORKLOADS = {}
@@ -64,6 +65,7 @@ for w in (
     + [_conv_workload(f"conv_{dt}_c64_k64_3x3_56", dt, 64, 64, 3, 56, 1, 1) for dt in ("f16", "i8")]
     + [_conv_workload(f"conv_{dt}_c256_k512_1x1_56_s2", dt, 256, 512, 1, 56, 2, 0) for dt in ("f16", "i8")]
     + [_conv_workload(f"conv_{dt}_c512_k512_3x3_7", dt, 512, 512, 3, 7, 1, 1) for dt in ("f16", "i8")]
+    + [_gemm_workload("fp16_batched_gemm_g16_1024", "f16", 1024, 1024, 1024, batch=16)]
     + [_gemm_workload("fp16_gemm_bias_relu_4096", "f16", 4096, 4096, 4096, fused="bias_relu"),
        _conv_workload("conv_f16_c64_k64_3x3_56_bias_relu_add", "f16", 64, 64, 3, 56, 1, 1, fused="bias_relu_add"),
        _conv_workload("conv_f16_c256_k512_1x1_56_s2_bias_relu", "f16", 256, 512, 1, 56, 2, 0, fused="bias_relu")]
@@ -101,7 +103,13 @@ def make_launcher(w, instance=-1, rotate=1):
             c = torch.empty((M, N), dtype=torch.float16, device="cuda")
             op = ck.DeviceGemmF16(instance)
             cop = ck.PassThrough()
-        if w.get("fused") == "bias_relu":
+        G = w.get("batch", 1)
+        if G > 1:
+            a, b = dev(uniform_f16((G * M, K), -1, 1, 1)), dev(uniform_f16((G * N, K), -1, 1, 2))
+            c = torch.empty((G * M, N), dtype=torch.float16, device="cuda")
+            op = ck.DeviceBatchedGemmF16(instance)
+            make = lambda bb: op.MakeArgumentPointer(a, bb, c, M, N, K, K, K, N, M * K, N * K, M * N, G)
+        elif w.get("fused") == "bias_relu":
             bias = dev(uniform_f16((N,), -1, 1, 9))
             op = ck.DeviceGemmMultipleDF16(instance)
             make = lambda bb: op.MakeArgumentPointer(a, bb, [bias], c, M, N, K, K, K, [0], N, None, None, ck.AddRelu())

@@ -23,6 +23,7 @@ SYMBOLS = [
     "ckx_version", "ckx_last_error", "ckx_num_instances", "ckx_instance_name",
     "ckx_gemm_i8_is_supported", "ckx_gemm_i8", "ckx_gemm_i8_workspace_bytes",
     "ckx_gemm_f16_is_supported", "ckx_gemm_f16", "ckx_gemm_f16_workspace_bytes",
+    "ckx_batched_gemm_is_supported", "ckx_batched_gemm_i8", "ckx_batched_gemm_f16",
     "ckx_gemm_splitk_workspace_bytes", "ckx_gemm_i8_splitk", "ckx_gemm_f16_splitk",
     "ckx_gemm_f16_multiple_d_is_supported", "ckx_gemm_f16_multiple_d", "ckx_conv2d_fwd_bias_activation_f16",
     "ckx_conv2d_fwd_is_supported", "ckx_conv2d_fwd_i8", "ckx_conv2d_fwd_f16", "ckx_conv2d_fwd_workspace_bytes",
@@ -76,6 +77,10 @@ def lib():
         fn.argtypes = [i32, i32, i32, C.c_int]
     L.ckx_gemm_f16_is_supported.argtypes = shape + [C.c_int]
     L.ckx_gemm_f16.argtypes = [vp, vp, vp] + shape + [C.c_int, vp, i64, vp]
+    bshape = [i32] * 6 + [i64] * 3 + [i32] + [C.c_int] * 3
+    L.ckx_batched_gemm_is_supported.argtypes = [C.c_int] + bshape + [C.c_int, C.c_int]
+    L.ckx_batched_gemm_i8.argtypes = [vp, vp, vp] + bshape + [C.c_int, f32, f32, C.c_int, vp]
+    L.ckx_batched_gemm_f16.argtypes = [vp, vp, vp] + bshape + [C.c_int, vp]
     L.ckx_gemm_splitk_workspace_bytes.restype = i64
     L.ckx_gemm_splitk_workspace_bytes.argtypes = [C.c_int, i32, i32, i32, i32]
     L.ckx_gemm_i8_splitk.argtypes = [vp, vp, vp] + shape + [C.c_int, f32, f32, C.c_int, i32, vp, i64, vp]

@@ -328,9 +328,35 @@ long gemm_workspace_bytes(int dt, int M, int N, int K, int instance)
     return pl.ksplit > 1 ? (long)pl.ksplit * M * N * 4 : 0;
 }
 
+// strided-batch part of the argument check (DeviceBatchedGemm)
+int check_batch(int dt, int M, int N, int K, int sa, int sb, int sc, int epi, int instance, int k_batch, int batch,
+                long bsa, long bsb, long bsc)
+{
+    if(batch < 0)
+        return fail(CKX_INVALID_VALUE, "negative batch count");
+    if(batch > 1)
+    {
+        const int es = dt == ckx::DT_I8 ? 1 : 2;
+        if(instance >= kNumTiles)
+            return fail(CKX_UNSUPPORTED, "batched GEMM runs on the tile instances");
+        if(epi >= CKX_EPI_ADD_RELU || k_batch > 1)
+            return fail(CKX_UNSUPPORTED, "batched GEMM has neither D operands nor a K split");
+        if(bsa < 0 || bsb < 0 || bsc < 0 || (bsa * es) % 16 || (bsb * es) % 16)
+            return fail(CKX_UNSUPPORTED, "batch strides of A and B must be non-negative multiples of 16 bytes");
+        if(bsc < (long)(M - 1) * sc + N && M > 0 && N > 0)
+            return fail(CKX_UNSUPPORTED, "C batches overlap");
+        const long ea = ((long)(batch - 1) * bsa + (long)(M - 1) * sa + K) * es;
+        const long eb = ((long)(batch - 1) * bsb + (long)(N - 1) * sb + K) * es;
+        if(ea >= (1l << 31) || eb >= (1l << 31) || ((long)(batch - 1) * bsc + (long)M * sc) * es >= (1l << 31))
+            return fail(CKX_UNSUPPORTED, "operands of 2 GiB or more are not addressed");
+    }
+    return CKX_OK;
+}
+
 int run_gemm(int dt, const void* a, const void* b, void* c, int M, int N, int K, int sa, int sb, int sc,
              int al, int bl, int cl, int epi, float sg, float sr, int instance, void* ws, long ws_bytes,
-             void* stream, const DOperands& dops = DOperands{}, int k_batch = 0)
+             void* stream, const DOperands& dops = DOperands{}, int k_batch = 0, int batch = 1, long bsa = 0,
+             long bsb = 0, long bsc = 0)
 {
     int st = check_gemm_shape(dt, M, N, K, sa, sb, sc, al, bl, cl, epi, instance);
     if(st != CKX_OK)
@@ -339,6 +365,10 @@ int run_gemm(int dt, const void* a, const void* b, void* c, int M, int N, int K,
         return fail(CKX_UNSUPPORTED, "KBatch must be 1..8");
     if(k_batch > 0 && instance >= kNumTiles)
         return fail(CKX_UNSUPPORTED, "the skinny instances split K over their waves, not over runs");
+    if((st = check_batch(dt, M, N, K, sa, sb, sc, epi, instance, k_batch, batch, bsa, bsb, bsc)) != CKX_OK)
+        return st;
+    if(batch == 0)
+        return CKX_OK;
     if((st = check_d_operands(epi, N, dops)) != CKX_OK)
         return st;
     if(M == 0 || N == 0)
@@ -354,7 +384,7 @@ int run_gemm(int dt, const void* a, const void* b, void* c, int M, int N, int K,
     const bool tile64 = M > 32 && M <= 64 &&
                         ((N + 63) / 64 >= 160 ||
                          (ws && !(reinterpret_cast<uintptr_t>(ws) & 15) && make_plan(M, N, K * es, -1, ws_bytes).ksplit > 1));
-    if(instance == CKX_INSTANCE_AUTO && M <= 64 && !tile64 && k_batch == 0)
+    if(instance == CKX_INSTANCE_AUTO && M <= 64 && !tile64 && k_batch == 0 && batch == 1)
     {
         // A handful of rows against a big weight matrix is an HBM-streaming problem. Wider
         // workgroups (32 / 64 columns) re-read A from L2 less often, as long as enough workgroups
@@ -369,7 +399,9 @@ int run_gemm(int dt, const void* a, const void* b, void* c, int M, int N, int K,
         if(k_batch > 1 && splitk_runs(K * es, k_batch) > 1 &&
            (!ws || ws_bytes < (long)splitk_runs(K * es, k_batch) * M * N * 4))
             return fail(CKX_INVALID_VALUE, "KBatch > 1 needs a workspace of ckx_gemm_splitk_workspace_bytes()");
-        pl = make_plan(M, N, K * es, instance, ws ? ws_bytes : 0, k_batch);
+        // a batch multiplies the C tiles: plan for a problem with that many rows, without a K split
+        pl = batch > 1 ? make_plan(M * (batch < 64 ? batch : 64), N, K * es, instance, 0, 1)
+                       : make_plan(M, N, K * es, instance, ws ? ws_bytes : 0, k_batch);
         ti = pl.tile;
     }
     ckx::GemmArgs g;
@@ -377,8 +409,9 @@ int run_gemm(int dt, const void* a, const void* b, void* c, int M, int N, int K,
     g.a = a, g.b = b, g.c = c;
     g.M = M, g.N = N, g.K = K;
     g.lda = sa, g.ldb = sb, g.ldc = sc;
-    g.a_bytes    = (uint32_t)(((long)(M - 1) * sa + K) * es);
-    g.b_bytes    = (uint32_t)(((long)(N - 1) * sb + K) * es);
+    g.a_bytes    = (uint32_t)(((long)(batch - 1) * bsa + (long)(M - 1) * sa + K) * es);
+    g.b_bytes    = (uint32_t)(((long)(batch - 1) * bsb + (long)(N - 1) * sb + K) * es);
+    g.batch = batch, g.bsa = bsa, g.bsb = bsb, g.bsc = bsc;
     g.epi        = epi;
     g.scale_gemm = sg;
     g.scale_relu = sr;
@@ -399,7 +432,7 @@ int run_gemm(int dt, const void* a, const void* b, void* c, int M, int N, int K,
     g.nk_per     = pl.nk_per;
     g.ws         = ws;
     hipError_t e =
-        (dt == ckx::DT_I8 ? t.dense_i8 : t.dense_f16)(g, g.tiles_m * g.tiles_n * g.ksplit, (hipStream_t)stream);
+        (dt == ckx::DT_I8 ? t.dense_i8 : t.dense_f16)(g, g.tiles_m * g.tiles_n * g.ksplit * batch, (hipStream_t)stream);
     if(e == hipSuccess && g.ksplit > 1)
         e = dt == ckx::DT_I8 ? launch_reduce<ckx::DT_I8>(g, (hipStream_t)stream)
                              : launch_reduce<ckx::DT_F16>(g, (hipStream_t)stream);
@@ -665,6 +698,33 @@ int ckx_gemm_f16_splitk(const void* a, const void* b, void* c, int32_t M, int32_
         return fail(CKX_INVALID_VALUE, "KBatch must be at least 1");
     return run_gemm(ckx::DT_F16, a, b, c, M, N, K, sa, sb, sc, al, bl, cl, CKX_EPI_PASSTHROUGH, 1.0f, 1.0f,
                     instance, workspace, workspace_bytes, stream, DOperands{}, k_batch);
+}
+
+int ckx_batched_gemm_is_supported(int op, int32_t M, int32_t N, int32_t K, int32_t sa, int32_t sb, int32_t sc,
+                                  int64_t bsa, int64_t bsb, int64_t bsc, int32_t batch, int al, int bl, int cl,
+                                  int epilogue, int instance)
+{
+    if(op != CKX_OP_GEMM_I8 && op != CKX_OP_GEMM_F16)
+        return fail(CKX_INVALID_VALUE, "not a GEMM operator family");
+    const int dt = op == CKX_OP_GEMM_I8 ? ckx::DT_I8 : ckx::DT_F16;
+    int st       = check_gemm_shape(dt, M, N, K, sa, sb, sc, al, bl, cl, epilogue, instance);
+    return st != CKX_OK ? st : check_batch(dt, M, N, K, sa, sb, sc, epilogue, instance, 0, batch, bsa, bsb, bsc);
+}
+
+int ckx_batched_gemm_i8(const void* a, const void* b, void* c, int32_t M, int32_t N, int32_t K, int32_t sa,
+                        int32_t sb, int32_t sc, int64_t bsa, int64_t bsb, int64_t bsc, int32_t batch, int al, int bl,
+                        int cl, int epilogue, float scale_gemm, float scale_relu, int instance, void* stream)
+{
+    return run_gemm(ckx::DT_I8, a, b, c, M, N, K, sa, sb, sc, al, bl, cl, epilogue, scale_gemm, scale_relu,
+                    instance, nullptr, 0, stream, DOperands{}, 0, batch, bsa, bsb, bsc);
+}
+
+int ckx_batched_gemm_f16(const void* a, const void* b, void* c, int32_t M, int32_t N, int32_t K, int32_t sa,
+                         int32_t sb, int32_t sc, int64_t bsa, int64_t bsb, int64_t bsc, int32_t batch, int al, int bl,
+                         int cl, int instance, void* stream)
+{
+    return run_gemm(ckx::DT_F16, a, b, c, M, N, K, sa, sb, sc, al, bl, cl, CKX_EPI_PASSTHROUGH, 1.0f, 1.0f,
+                    instance, nullptr, 0, stream, DOperands{}, 0, batch, bsa, bsb, bsc);
 }
 
 int ckx_gemm_f16_multiple_d_is_supported(int32_t M, int32_t N, int32_t K, int32_t sa, int32_t sb, int32_t sd0,

@@ -120,6 +120,10 @@ struct GemmArgs
     const void* d0;
     const void* d1;
     int ldd0, ldd1;
+    // strided batch (DeviceBatchedGemm): batch g reads A + g*bsa, B + g*bsb, writes C + g*bsc
+    // (element strides); 0 or 1 = a single GEMM. The byte extents a_bytes / b_bytes span all batches.
+    int batch;
+    long bsa, bsb, bsc;
     ConvGeom cv;
 };
 
@@ -389,6 +393,8 @@ struct GemmTile
         const int wn   = wave % WN;
 
         const int ntiles      = p.tiles_m * p.tiles_n;
+        const int nbatch      = p.batch > 0 ? p.batch : 1;
+        const int ntiles_all  = ntiles * nbatch; // C tiles of all batches: id = batch * ntiles + tile
         const int gstride     = (int)gridDim.x;
         const uint32_t kbytes = (uint32_t)p.K * ES;
         const int nk_real     = (int)((kbytes + BKB - 1) / BKB);
@@ -408,11 +414,13 @@ struct GemmTile
         const uint32_t kb = ((uint32_t)(lane % CPR) ^ (uint32_t)((lane / CPR) & 7)) << 4; // chunk byte offset in a K tile
 
         // row / column offsets of the tile the LOAD cursor is on (tile >= ntiles: nothing valid)
-        auto setup_tile = [&](int tile) {
+        auto setup_tile = [&](int tile_id) {
             int tm = 0, tn = 0;
-            const bool live = tile < ntiles;
+            const bool live = tile_id < ntiles_all;
+            const int g     = live ? tile_id / ntiles : 0;
             if(live)
-                tile_of_block(tile, p.tiles_m, p.tiles_n, tm, tn);
+                tile_of_block(tile_id - g * ntiles, p.tiles_m, p.tiles_n, tm, tn);
+            const uint32_t a_batch = (uint32_t)((long)g * p.bsa * ES), b_batch = (uint32_t)((long)g * p.bsb * ES);
 #pragma unroll
             for(int j = 0; j < NLA; ++j)
             {
@@ -421,7 +429,7 @@ struct GemmTile
                 const bool ok     = live && gm < (uint32_t)p.M;
                 if constexpr(!IM2COL)
                 {
-                    a_off[j] = ok ? gm * (uint32_t)p.lda * ES + kb : kOutOfRange;
+                    a_off[j] = ok ? a_batch + gm * (uint32_t)p.lda * ES + kb : kOutOfRange;
                     a_hw0[j] = 0;
                 }
                 else
@@ -452,7 +460,7 @@ struct GemmTile
             {
                 const uint32_t r  = (uint32_t)((j * NW + wave) * RPI + lane / CPR);
                 const uint32_t gn = (uint32_t)tn * BN + b_row_to_col(r);
-                b_off[j] = (live && gn < (uint32_t)p.N) ? gn * (uint32_t)p.ldb * ES + kb : kOutOfRange;
+                b_off[j] = (live && gn < (uint32_t)p.N) ? b_batch + gn * (uint32_t)p.ldb * ES + kb : kOutOfRange;
             }
         };
 
@@ -526,17 +534,17 @@ struct GemmTile
                 issue_slot(c, sl);
         };
 
-        // A work unit is (K run s, C tile): unit = s * ntiles + tile, K tiles [s*nk_per, ...).
-        const int nunits = ntiles * p.ksplit;
+        // A work unit is (K run s, C tile id): unit = s * ntiles_all + id, K tiles [s*nk_per, ...).
+        const int nunits = ntiles_all * p.ksplit;
         auto unit_k_range = [&](int unit, int& k_begin, int& k_end) {
-            const int sp = unit / ntiles;
+            const int sp = unit / ntiles_all;
             k_begin      = sp * p.nk_per;
             k_end        = k_begin + p.nk_per < nk ? k_begin + p.nk_per : nk;
         };
         // load cursor: (unit, kt) of the next K tile to request
         int ld_unit = (int)blockIdx.x, ld_kt = 0, ld_end = nk;
         unit_k_range(ld_unit, ld_kt, ld_end);
-        setup_tile(ld_unit < nunits ? ld_unit % ntiles : ntiles);
+        setup_tile(ld_unit < nunits ? ld_unit % ntiles_all : ntiles_all);
         // (kept apart from the issue itself: the branch would split the basic block in which the
         // loads are interleaved with MFMAs)
         auto advance_load_cursor = [&]() {
@@ -544,7 +552,7 @@ struct GemmTile
             {
                 ld_unit += gstride;
                 unit_k_range(ld_unit, ld_kt, ld_end);
-                setup_tile(ld_unit < nunits ? ld_unit % ntiles : ntiles);
+                setup_tile(ld_unit < nunits ? ld_unit % ntiles_all : ntiles_all);
             }
         };
 
@@ -622,15 +630,19 @@ struct GemmTile
         };
 
         // ---- epilogue: registers -> global, 16 consecutive columns per lane -------------
-        const bool vec_ok = ((reinterpret_cast<uintptr_t>(p.c) | ((uintptr_t)p.ldc * ES)) & 15u) == 0;
+        const bool vec_ok = ((reinterpret_cast<uintptr_t>(p.c) | ((uintptr_t)p.ldc * ES) |
+                              (nbatch > 1 ? (uintptr_t)p.bsc * ES : 0)) & 15u) == 0;
         const bool nt     = p.nt_store != 0;
         const bool dvec_ok = ((reinterpret_cast<uintptr_t>(p.d0) | ((uintptr_t)p.ldd0 * ES) |
                                reinterpret_cast<uintptr_t>(p.d1) | ((uintptr_t)p.ldd1 * ES)) & 15u) == 0;
         auto epilogue = [&](int unit) {
             int tm, tn;
-            tile_of_block(unit % ntiles, p.tiles_m, p.tiles_n, tm, tn);
+            const int tile_id = unit % ntiles_all, bi = tile_id / ntiles;
+            tile_of_block(tile_id - bi * ntiles, p.tiles_m, p.tiles_n, tm, tn);
+            // (a K split is never combined with a batch: the slices are [run][M][N])
             acc_t* slice = reinterpret_cast<acc_t*>(reinterpret_cast<uint8_t*>(p.ws) +
-                                                    (size_t)(unit / ntiles) * p.M * p.N * 4);
+                                                    (size_t)(unit / ntiles_all) * p.M * p.N * 4);
+            uint8_t* c_batch = reinterpret_cast<uint8_t*>(p.c) + (size_t)bi * p.bsc * ES;
 #pragma unroll
             for(int i = 0; i < MT; ++i)
             {
@@ -661,7 +673,7 @@ struct GemmTile
                         }
                         else if constexpr(DT == DT_I8)
                         {
-                            int8_t* crow = reinterpret_cast<int8_t*>(p.c) + (size_t)m * p.ldc;
+                            int8_t* crow = reinterpret_cast<int8_t*>(c_batch) + (size_t)m * p.ldc;
                             const i32x4 v[4] = {acc[i][g * 4], acc[i][g * 4 + 1], acc[i][g * 4 + 2],
                                                 acc[i][g * 4 + 3]};
                             if(p.epi == EPI_REQUANT_RND)
@@ -673,7 +685,7 @@ struct GemmTile
                         }
                         else
                         {
-                            _Float16* crow   = reinterpret_cast<_Float16*>(p.c) + (size_t)m * p.ldc;
+                            _Float16* crow   = reinterpret_cast<_Float16*>(c_batch) + (size_t)m * p.ldc;
                             const f32x4 v[4] = {acc[i][g * 4], acc[i][g * 4 + 1], acc[i][g * 4 + 2],
                                                 acc[i][g * 4 + 3]};
                             store_row16_f16(crow, n0, p.N, vec_ok, v, nt);

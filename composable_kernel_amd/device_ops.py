@@ -253,6 +253,48 @@ class DeviceGemmSplitKF16(_DeviceGemmSplitK):
                                               a.workspace_bytes_, C.c_void_p(stream or 0))
 
 
+class _DeviceBatchedGemm(_DeviceGemm):
+    """DeviceBatchedGemm<...> (device_batched_gemm.hpp:24-45): strided batch, element strides."""
+
+    def MakeArgumentPointer(self, p_a, p_b, p_c, M, N, K, StrideA, StrideB, StrideC, BatchStrideA, BatchStrideB,
+                            BatchStrideC, Batch, a_element_op=None, b_element_op=None, c_element_op=None):
+        a = super().MakeArgumentPointer(p_a, p_b, p_c, M, N, K, StrideA, StrideB, StrideC, a_element_op,
+                                        b_element_op, c_element_op)
+        a.batch = (int(BatchStrideA), int(BatchStrideB), int(BatchStrideC), int(Batch))
+        return a
+
+    def _supported(self, a):
+        if self.op_family == capi.OP_GEMM_F16 and not isinstance(a.c_op, PassThrough):
+            capi.lib().ckx_gemm_f16_is_supported(-1, 0, 0, 0, 0, 0, 0, 0, 0, 0)
+            return capi.UNSUPPORTED
+        return capi.lib().ckx_batched_gemm_is_supported(self.op_family, a.M, a.N, a.K, a.StrideA, a.StrideB,
+                                                        a.StrideC, *a.batch, *self.layouts, a.c_op.epilogue,
+                                                        self.instance)
+
+    def _launch(self, a, stream):
+        return self._call(a, a.p_a, a.p_b, a.p_c, stream)
+
+
+class DeviceBatchedGemmInt8(_DeviceBatchedGemm):
+    op_family = capi.OP_GEMM_I8
+
+    def _call(self, a, pa, pb, pc, stream):
+        return capi.lib().ckx_batched_gemm_i8(pa, pb, pc, a.M, a.N, a.K, a.StrideA, a.StrideB, a.StrideC, *a.batch,
+                                              *self.layouts, a.c_op.epilogue, a.c_op.scale_gemm, a.c_op.scale_relu,
+                                              self.instance, C.c_void_p(stream or 0))
+
+
+class DeviceBatchedGemmF16(_DeviceBatchedGemm):
+    op_family = capi.OP_GEMM_F16
+
+    def _call(self, a, pa, pb, pc, stream):
+        if not isinstance(a.c_op, PassThrough):
+            capi.lib().ckx_gemm_f16_is_supported(-1, 0, 0, 0, 0, 0, 0, 0, 0, 0)
+            return capi.UNSUPPORTED
+        return capi.lib().ckx_batched_gemm_f16(pa, pb, pc, a.M, a.N, a.K, a.StrideA, a.StrideB, a.StrideC, *a.batch,
+                                               *self.layouts, self.instance, C.c_void_p(stream or 0))
+
+
 class DeviceGemmMultipleDF16(BaseOperator):
     """DeviceGemmMultipleD<Row, Col, Row, half_t, half_t, Tuple<half_t[, half_t]>, half_t, PassThrough,
     PassThrough, CDEOp> (device_gemm_multiple_d.hpp:14-55): E = cde_op(A*B, D0[, D1])."""

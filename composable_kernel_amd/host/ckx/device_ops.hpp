@@ -254,6 +254,21 @@ struct DeviceBatchedGemmGemm : public BaseOperator
     virtual std::unique_ptr<BaseInvoker> MakeInvokerPointer()                                     = 0;
 };
 
+// device_batched_gemm.hpp:24-45
+template <typename ALayout, typename BLayout, typename CLayout, typename ADataType, typename BDataType,
+          typename CDataType, typename AElementwiseOperation, typename BElementwiseOperation,
+          typename CElementwiseOperation>
+struct DeviceBatchedGemm : public BaseOperator
+{
+    virtual std::unique_ptr<BaseArgument>
+    MakeArgumentPointer(const void* p_a, const void* p_b, void* p_c, index_t M, index_t N, index_t K,
+                        index_t StrideA, index_t StrideB, index_t StrideC, index_t BatchStrideA,
+                        index_t BatchStrideB, index_t BatchStrideC, index_t Batch,
+                        AElementwiseOperation a_element_op, BElementwiseOperation b_element_op,
+                        CElementwiseOperation c_element_op)    = 0;
+    virtual std::unique_ptr<BaseInvoker> MakeInvokerPointer() = 0;
+};
+
 // device_gemm_splitk.hpp:14-39
 template <typename ALayout, typename BLayout, typename CLayout, typename ADataType, typename BDataType,
           typename CDataType, typename AElementwiseOperation, typename BElementwiseOperation,
@@ -563,6 +578,79 @@ struct DeviceConv2dFwdMfma_Input_N_Hi_Wi_C_Weight_K_Y_X_C_Output_N_Ho_Wo_K
             return is_i8 ? "DeviceConv2dFwd_i8_nhwc_kyxc_nhwk<auto>" : "DeviceConv2dFwd_f16_nhwc_kyxc_nhwk<auto>";
         return ckx_instance_name(op_code, instance_);
     }
+    int instance_;
+};
+
+// ------------------------------------------------------------------ strided batched GEMM
+// One launch for all batches: the persistent workgroups walk the C tiles of every batch.
+template <typename ALayout, typename BLayout, typename CLayout, typename ADataType, typename BDataType,
+          typename CDataType, typename AElementwiseOperation, typename BElementwiseOperation,
+          typename CElementwiseOperation>
+struct DeviceBatchedGemmMfma : public DeviceBatchedGemm<ALayout, BLayout, CLayout, ADataType, BDataType, CDataType,
+                                                        AElementwiseOperation, BElementwiseOperation,
+                                                        CElementwiseOperation>
+{
+    using Plain = DeviceGemmMfma<ALayout, BLayout, CLayout, ADataType, BDataType, CDataType, AElementwiseOperation,
+                                 BElementwiseOperation, CElementwiseOperation>;
+    static constexpr bool is_i8 = Plain::is_i8;
+    using Epi                   = typename Plain::Epi;
+    struct Argument : public Plain::Argument
+    {
+        index_t BatchStrideA, BatchStrideB, BatchStrideC, Batch;
+        Argument(const void* a, const void* b, void* c, index_t m, index_t n, index_t k, index_t sa, index_t sb,
+                 index_t sc, index_t bsa, index_t bsb, index_t bsc, index_t batch, CElementwiseOperation cop)
+            : Plain::Argument(a, b, c, m, n, k, sa, sb, sc, cop), BatchStrideA(bsa), BatchStrideB(bsb),
+              BatchStrideC(bsc), Batch(batch)
+        {
+        }
+    };
+    static int Supported(const Argument& a, int inst)
+    {
+        return ckx_batched_gemm_is_supported(is_i8 ? CKX_OP_GEMM_I8 : CKX_OP_GEMM_F16, a.M, a.N, a.K, a.StrideA,
+                                             a.StrideB, a.StrideC, a.BatchStrideA, a.BatchStrideB, a.BatchStrideC,
+                                             a.Batch, ALayout::code, BLayout::code, CLayout::code, Epi::kind, inst);
+    }
+    static int Launch(const Argument& a, int inst, void* stream)
+    {
+        if constexpr(is_i8)
+            return ckx_batched_gemm_i8(a.p_a, a.p_b, a.p_c, a.M, a.N, a.K, a.StrideA, a.StrideB, a.StrideC,
+                                       a.BatchStrideA, a.BatchStrideB, a.BatchStrideC, a.Batch, ALayout::code,
+                                       BLayout::code, CLayout::code, Epi::kind, Epi::scale_gemm(a.c_element_op),
+                                       Epi::scale_relu(a.c_element_op), inst, stream);
+        else
+            return ckx_batched_gemm_f16(a.p_a, a.p_b, a.p_c, a.M, a.N, a.K, a.StrideA, a.StrideB, a.StrideC,
+                                        a.BatchStrideA, a.BatchStrideB, a.BatchStrideC, a.Batch, ALayout::code,
+                                        BLayout::code, CLayout::code, inst, stream);
+    }
+    using Invoker = detail::InvokerT<Argument, &Supported, &Launch>;
+
+    explicit DeviceBatchedGemmMfma(int instance = CKX_INSTANCE_AUTO) : instance_(instance) {}
+    static Argument MakeArgument(const ADataType* p_a, const BDataType* p_b, CDataType* p_c, index_t M, index_t N,
+                                 index_t K, index_t StrideA, index_t StrideB, index_t StrideC, index_t BatchStrideA,
+                                 index_t BatchStrideB, index_t BatchStrideC, index_t Batch, AElementwiseOperation,
+                                 BElementwiseOperation, CElementwiseOperation c_element_op)
+    {
+        return Argument{p_a, p_b, p_c, M, N, K, StrideA, StrideB, StrideC, BatchStrideA, BatchStrideB, BatchStrideC,
+                        Batch, c_element_op};
+    }
+    Invoker MakeInvoker() const { return Invoker{instance_}; }
+    bool IsSupportedArgument(const Argument& a) const { return Supported(a, instance_) == CKX_OK; }
+    bool IsSupportedArgument(const BaseArgument* p) override
+    {
+        const auto* a = dynamic_cast<const Argument*>(p);
+        return a && IsSupportedArgument(*a);
+    }
+    std::unique_ptr<BaseArgument>
+    MakeArgumentPointer(const void* p_a, const void* p_b, void* p_c, index_t M, index_t N, index_t K,
+                        index_t StrideA, index_t StrideB, index_t StrideC, index_t BatchStrideA,
+                        index_t BatchStrideB, index_t BatchStrideC, index_t Batch, AElementwiseOperation,
+                        BElementwiseOperation, CElementwiseOperation c_element_op) override
+    {
+        return std::make_unique<Argument>(p_a, p_b, p_c, M, N, K, StrideA, StrideB, StrideC, BatchStrideA,
+                                          BatchStrideB, BatchStrideC, Batch, c_element_op);
+    }
+    std::unique_ptr<BaseInvoker> MakeInvokerPointer() override { return std::make_unique<Invoker>(instance_); }
+    std::string GetTypeString() const override { return Plain(instance_).GetTypeString() + " + Batched"; }
     int instance_;
 };
 

@@ -12,6 +12,8 @@
 //                     (profiler/src/profile_conv_fwd_bias_relu[_add].cpp; fp16, NHWC/KYXC/NHWK)
 //   ckx_profiler gemm_splitk <dtype 1|3> <layout 1> <verify> <init> <log> <time> M N K StrideA StrideB StrideC KBatch
 //                     [nrepeat]   (profiler/src/profile_gemm_splitk.cpp; PassThrough output)
+//   ckx_profiler batched_gemm <dtype 1|3> <layout 1> <verify> <init> <log> <time> M N K StrideA StrideB StrideC
+//                     BatchCount [nrepeat]   (profiler/src/profile_batched_gemm.cpp; dense batch strides)
 //   ckx_profiler gemm_bias_relu <verify> <init> <log> <time> M N K StrideA StrideB StrideE [nrepeat]
 //                     (example/03_gemm_bias_relu: E = AddRelu(half(A*B), bias row), fp16)
 //
@@ -339,6 +341,59 @@ int profile_gemm_splitk(int argc, char* argv[])
                       : profile_gemm_splitk_t<int8_t>(verify, init, time_kernel, M, N, K, sa, sb, sc, kbatch, nrep);
 }
 
+template <typename T>
+int profile_batched_gemm_t(bool verify, int init, bool time_kernel, int M, int N, int K, int sa, int sb, int sc,
+                           int batch, int nrepeat)
+{
+    using DeviceOp = device::DeviceBatchedGemm<Row, Col, Row, T, T, T, Pass, Pass, Pass>;
+    std::vector<std::unique_ptr<DeviceOp>> ops;
+    for(int i = 0, n = ckx_num_instances(CKX_OP_GEMM_SPLITK); i < n; ++i) // the tile instances
+        ops.push_back(std::make_unique<device::DeviceBatchedGemmMfma<Row, Col, Row, T, T, T, Pass, Pass, Pass>>(i));
+    const std::size_t bsa = (std::size_t)M * sa, bsb = (std::size_t)N * sb, bsc = (std::size_t)M * sc;
+    std::vector<T> a(bsa * batch), b(bsb * batch);
+    fill(a, init, 0xC0FFEE, false);
+    fill(b, init, 0xC0FFEE + 1, false);
+    ckx::DeviceMem da(a.size() * sizeof(T)), db(b.size() * sizeof(T)), dc(bsc * batch * sizeof(T));
+    da.ToDevice(a.data());
+    db.ToDevice(b.data());
+    const double flop  = 2.0 * M * N * K * batch;
+    const double bytes = sizeof(T) * ((double)M * K + (double)K * N + (double)M * N) * batch;
+    return run_family<T>(
+        ops,
+        [&](DeviceOp& op) {
+            return op.MakeArgumentPointer(da.GetDeviceBuffer(), db.GetDeviceBuffer(), dc.GetDeviceBuffer(), M, N, K,
+                                          sa, sb, sc, (index_t)bsa, (index_t)bsb, (index_t)bsc, batch, Pass{}, Pass{},
+                                          Pass{});
+        },
+        dc, bsc * batch, flop, bytes, verify, time_kernel, nrepeat);
+}
+
+int profile_batched_gemm(int argc, char* argv[])
+{
+    if(argc < 15)
+    {
+        std::printf("arg1: tensor operation (batched_gemm)\narg2: data type (1: fp16; 3: int8)\n"
+                    "arg3: matrix layout (1: A[g, m, k] * B[g, n, k] = C[g, m, n])\narg4: verification\n"
+                    "arg5: initialization\narg6: print tensor value\narg7: time kernel\n"
+                    "arg8 to 14: M, N, K, StrideA, StrideB, StrideC, BatchCount\n");
+        return 1;
+    }
+    const int dtype = std::atoi(argv[2]), layout = std::atoi(argv[3]);
+    const bool verify = std::atoi(argv[4]), time_kernel = std::atoi(argv[7]);
+    const int init = std::atoi(argv[5]);
+    const int M = std::atoi(argv[8]), N = std::atoi(argv[9]), K = std::atoi(argv[10]);
+    int sa = std::atoi(argv[11]), sb = std::atoi(argv[12]), sc = std::atoi(argv[13]);
+    sa = sa < 0 ? K : sa, sb = sb < 0 ? K : sb, sc = sc < 0 ? N : sc;
+    const int batch = std::atoi(argv[14]), nrep = argc > 15 ? std::atoi(argv[15]) : 10;
+    if(layout != 1 || (dtype != 1 && dtype != 3))
+    {
+        std::cout << "this data_type & layout is not implemented" << std::endl;
+        return 1;
+    }
+    return dtype == 1 ? profile_batched_gemm_t<half_t>(verify, init, time_kernel, M, N, K, sa, sb, sc, batch, nrep)
+                      : profile_batched_gemm_t<int8_t>(verify, init, time_kernel, M, N, K, sa, sb, sc, batch, nrep);
+}
+
 // conv + bias + ReLU (with_resi: + residual add), fp16
 int profile_conv_bias_relu(int argc, char* argv[], bool with_resi)
 {
@@ -502,6 +557,8 @@ int main(int argc, char* argv[])
             return profile_conv_bias_relu(argc, argv, false);
         if(argc >= 2 && std::strcmp(argv[1], "conv_fwd_bias_relu_add") == 0)
             return profile_conv_bias_relu(argc, argv, true);
+        if(argc >= 2 && std::strcmp(argv[1], "batched_gemm") == 0)
+            return profile_batched_gemm(argc, argv);
         if(argc >= 2 && std::strcmp(argv[1], "gemm_splitk") == 0)
             return profile_gemm_splitk(argc, argv);
         if(argc >= 2 && std::strcmp(argv[1], "gemm_bias_relu") == 0)
@@ -511,6 +568,7 @@ int main(int argc, char* argv[])
                     "                        batched_gemm_gemm: batched fused GEMM+GEMM\n"
                     "                        conv_fwd_bias_relu: ForwardConvolution+Bias+ReLU\n"
                     "                        conv_fwd_bias_relu_add: ForwardConvolution+Bias+ReLU+Add\n"
+                    "                        batched_gemm: Batched GEMM\n"
                     "                        gemm_splitk: Split-K GEMM\n"
                     "                        gemm_bias_relu: GEMM+Bias+ReLU)\n");
         return 1;

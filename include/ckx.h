@@ -119,6 +119,26 @@ int ckx_gemm_f16(const void* p_a, const void* p_b, void* p_c, int32_t M, int32_t
                  int c_layout, int instance, void* p_workspace, int64_t workspace_bytes, void* stream);
 int64_t ckx_gemm_f16_workspace_bytes(int32_t M, int32_t N, int32_t K, int instance);
 
+/* ---- strided batched GEMM:  C[g] = c_op(A[g] * B[g]),  g < batch ----------------
+ * Replaces DeviceBatchedGemm<...>::MakeArgumentPointer(..., BatchStrideA, BatchStrideB, BatchStrideC,
+ * Batch, ...) + Run (device_batched_gemm.hpp:24-45; batch offsets as ComputePtrOffsetOfStridedBatch,
+ * device_batched_gemm_xdl.hpp:256-285). Batch strides are in elements. The batches share one launch:
+ * the persistent workgroups walk the C tiles of all batches. Shapes as for ckx_gemm_*_is_supported on a
+ * tile instance (or AUTO); additionally the A / B batch strides must be multiples of 16 bytes, the C
+ * batches must not overlap, and the whole A, B, C extents stay below 2 GiB. */
+int ckx_batched_gemm_is_supported(int op, int32_t M, int32_t N, int32_t K, int32_t stride_a, int32_t stride_b,
+                                  int32_t stride_c, int64_t batch_stride_a, int64_t batch_stride_b,
+                                  int64_t batch_stride_c, int32_t batch, int a_layout, int b_layout, int c_layout,
+                                  int epilogue, int instance);
+int ckx_batched_gemm_i8(const void* p_a, const void* p_b, void* p_c, int32_t M, int32_t N, int32_t K,
+                        int32_t stride_a, int32_t stride_b, int32_t stride_c, int64_t batch_stride_a,
+                        int64_t batch_stride_b, int64_t batch_stride_c, int32_t batch, int a_layout, int b_layout,
+                        int c_layout, int epilogue, float scale_gemm, float scale_relu, int instance, void* stream);
+int ckx_batched_gemm_f16(const void* p_a, const void* p_b, void* p_c, int32_t M, int32_t N, int32_t K,
+                         int32_t stride_a, int32_t stride_b, int32_t stride_c, int64_t batch_stride_a,
+                         int64_t batch_stride_b, int64_t batch_stride_c, int32_t batch, int a_layout, int b_layout,
+                         int c_layout, int instance, void* stream);
+
 /* ---- split-K GEMM with a caller-chosen number of K runs ----------------------
  * Replaces DeviceGemmSplitK<...>::MakeArgumentPointer(..., KBatch) + Run (device_gemm_splitk.hpp:14-39).
  * The K extent is cut into k_batch (1..8) runs of whole 128-byte K tiles (fewer when K has fewer tiles);

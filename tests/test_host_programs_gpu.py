@@ -138,3 +138,17 @@ def test_profiler_gemm_splitk_int8(tmp_path):
     a = uniform_int8((M, K), -5, 5, SEED)
     b_nk = uniform_int8((N, K), -5, 5, SEED + 1)
     np.testing.assert_array_equal(c, fast.gemm_i8(a, b_nk.T))
+
+
+def test_profiler_batched_gemm_fp16(tmp_path):
+    """profile_batched_gemm's argument list (BatchCount = arg14), dense batch strides."""
+    M, N, K, G = 192, 320, 256, 5
+    out, dump = _run("ckx_profiler", ["batched_gemm", 1, 1, 1, 2, 0, 1, M, N, K, -1, -1, -1, G], "CKX_PROFILER_DUMP",
+                     tmp_path)
+    assert "Best Perf:" in out and "Error" not in out and "Batched" in out
+    c = np.fromfile(dump, np.float16).reshape(G, M, N)
+    a = uniform_f16((G, M, K), -1, 1, SEED)
+    b_gnk = uniform_f16((G, N, K), -1, 1, SEED + 1)
+    ref = lit.batched_gemm_f16(a, np.ascontiguousarray(b_gnk.transpose(0, 2, 1)))
+    bad, max_err = lit.check_err_f16(c, ref, 1e-2, 1e-2)
+    assert bad == 0, max_err
