@@ -15,13 +15,15 @@
 //    chunk lands in its slot, which is how the XOR swizzle and the B row permutation are
 //    applied for free. Out-of-range rows / K tail / conv padding use an out-of-range buffer
 //    offset, which the hardware turns into zeros.
-//  * two LDS stages, one barrier per K tile; the loads of tile k+1 are in flight while
-//    tile k is multiplied.
+//  * NST LDS stages in a ring, one barrier per K tile; the kernel is persistent over work units
+//    (C tile x K run x batch) and the loads run ahead of the MFMAs across unit boundaries.
 //  * MFMA is issued as D^T = B_frag x A_frag, so a lane ends up owning, for one row m, the
 //    accumulators of 4 consecutive columns per MFMA tile; the B rows of a 64-column group
 //    are permuted in LDS so that the 4 tiles of the group give the lane 16 CONSECUTIVE
 //    columns. The epilogue (requant, ReLU, saturation, conversion) runs on registers and
 //    each lane stores 16 contiguous outputs: no trip through LDS.
+//  * optional extras of a launch: a K split with raw accumulators in a caller workspace and a
+//    second pass (splitk_reduce_kernel), fp16 add / ReLU epilogues with D operands, a strided batch.
 #pragma once
 
 #include <hip/hip_runtime.h>
@@ -322,24 +324,6 @@ __device__ __forceinline__ void store_row16_f16_fused(_Float16* crow, int n0, in
             }
     }
     store_row16_f16(crow, n0, N, vec_ok, v, nt);
-}
-
-// Scheduling recipe for one half-iteration that also issues NL direct loads: NL groups of
-// {1 VMEM read, its share of the NR LDS reads, its share of the NM MFMAs}.
-template <int L, int NL, int NR, int NM>
-__device__ __forceinline__ void sched_loads_reads_mfma()
-{
-    if constexpr(L < NL)
-    {
-        constexpr int nr  = NR / NL + (L < NR % NL ? 1 : 0);
-        constexpr int per = NM / NL + (L < NM % NL ? 1 : 0);
-        __builtin_amdgcn_sched_group_barrier(0x010, 1, 0); // VMEM (the direct-to-LDS load counts as load+store)
-        if constexpr(nr > 0)
-            __builtin_amdgcn_sched_group_barrier(0x100, nr, 0); // DS read
-        if constexpr(per > 0)
-            __builtin_amdgcn_sched_group_barrier(0x008, per, 0); // MFMA
-        sched_loads_reads_mfma<L + 1, NL, NR, NM>();
-    }
 }
 
 // ------------------------------------------------------------------- kernel
