@@ -28,7 +28,7 @@ import numpy as np
 ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
-PEAK = {"f16": 2516.6, "i8": 5033.2}   # dense MFMA TFLOP/s / TOP/s, 256 CUs x 2.4 GHz
+PEAK = {"f16": 2516.6, "bf16": 2516.6, "i8": 5033.2}   # dense MFMA TFLOP/s / TOP/s, 256 CUs x 2.4 GHz
 HBM_PEAK_GBS = 8000.0
 # Bytes crossing the L2 <-> fabric boundary per launch, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
 # scaled by a 256 MiB copy in the same run (profiles/gemm_tile_fp16_int8_4096_hbm_traffic.md).
@@ -65,7 +65,8 @@ for w in (
     + [_conv_workload(f"conv_{dt}_c64_k64_3x3_56", dt, 64, 64, 3, 56, 1, 1) for dt in ("f16", "i8")]
     + [_conv_workload(f"conv_{dt}_c256_k512_1x1_56_s2", dt, 256, 512, 1, 56, 2, 0) for dt in ("f16", "i8")]
     + [_conv_workload(f"conv_{dt}_c512_k512_3x3_7", dt, 512, 512, 3, 7, 1, 1) for dt in ("f16", "i8")]
-    + [_gemm_workload("fp16_batched_gemm_g16_1024", "f16", 1024, 1024, 1024, batch=16)]
+    + [_gemm_workload("fp16_batched_gemm_g16_1024", "f16", 1024, 1024, 1024, batch=16),
+       _gemm_workload("bf16_gemm_4096", "bf16", 4096, 4096, 4096)]
     + [_gemm_workload("fp16_gemm_bias_relu_4096", "f16", 4096, 4096, 4096, fused="bias_relu"),
        _conv_workload("conv_f16_c64_k64_3x3_56_bias_relu_add", "f16", 64, 64, 3, 56, 1, 1, fused="bias_relu_add"),
        _conv_workload("conv_f16_c256_k512_1x1_56_s2_bias_relu", "f16", 256, 512, 1, 56, 2, 0, fused="bias_relu")]
@@ -104,7 +105,14 @@ def make_launcher(w, instance=-1, rotate=1):
             op = ck.DeviceGemmF16(instance)
             cop = ck.PassThrough()
         G = w.get("batch", 1)
-        if G > 1:
+        if w["dtype"] == "bf16":
+            from composable_kernel_amd.host_tensor import uniform_bf16
+            a = dev(uniform_bf16((M, K), -1, 1, 1).view(np.int16))
+            b = dev(uniform_bf16((N, K), -1, 1, 2).view(np.int16))
+            c = torch.empty((M, N), dtype=torch.int16, device="cuda")
+            op = ck.DeviceGemmBF16(instance)
+            make = lambda bb: op.MakeArgumentPointer(a, bb, c, M, N, K, K, K, N)
+        elif G > 1:
             a, b = dev(uniform_f16((G * M, K), -1, 1, 1)), dev(uniform_f16((G * N, K), -1, 1, 2))
             c = torch.empty((G * M, N), dtype=torch.float16, device="cuda")
             op = ck.DeviceBatchedGemmF16(instance)

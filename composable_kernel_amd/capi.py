@@ -15,7 +15,7 @@ OK, UNSUPPORTED, INVALID_VALUE, HIP_ERROR = 0, -1, -2, -3
 ROW_MAJOR, COL_MAJOR = 0, 1
 EPI_PASSTHROUGH, EPI_REQUANT_CK, EPI_REQUANT_RND = 0, 1, 2
 EPI_ADD_RELU, EPI_ADD_RELU_ADD, EPI_CSHUFFLE_ADD_RELU = 3, 4, 5
-OP_GEMM_I8, OP_GEMM_F16, OP_CONV2D_FWD_I8, OP_CONV2D_FWD_F16, OP_BATCHED_GEMM_GEMM, OP_GEMM_SPLITK = range(6)
+OP_GEMM_I8, OP_GEMM_F16, OP_CONV2D_FWD_I8, OP_CONV2D_FWD_F16, OP_BATCHED_GEMM_GEMM, OP_GEMM_SPLITK, OP_GEMM_BF16 = range(7)
 INSTANCE_AUTO = -1
 
 # every symbol include/ckx.h declares
@@ -23,6 +23,7 @@ SYMBOLS = [
     "ckx_version", "ckx_last_error", "ckx_num_instances", "ckx_instance_name",
     "ckx_gemm_i8_is_supported", "ckx_gemm_i8", "ckx_gemm_i8_workspace_bytes",
     "ckx_gemm_f16_is_supported", "ckx_gemm_f16", "ckx_gemm_f16_workspace_bytes",
+    "ckx_gemm_bf16_is_supported", "ckx_gemm_bf16", "ckx_gemm_bf16_workspace_bytes",
     "ckx_batched_gemm_is_supported", "ckx_batched_gemm_i8", "ckx_batched_gemm_f16",
     "ckx_gemm_splitk_workspace_bytes", "ckx_gemm_i8_splitk", "ckx_gemm_f16_splitk",
     "ckx_gemm_f16_multiple_d_is_supported", "ckx_gemm_f16_multiple_d", "ckx_conv2d_fwd_bias_activation_f16",
@@ -72,11 +73,13 @@ def lib():
     shape = [i32] * 6 + [C.c_int] * 3
     L.ckx_gemm_i8_is_supported.argtypes = shape + [C.c_int, C.c_int]
     L.ckx_gemm_i8.argtypes = [vp, vp, vp] + shape + [C.c_int, f32, f32, C.c_int, vp, i64, vp]
-    for fn in (L.ckx_gemm_i8_workspace_bytes, L.ckx_gemm_f16_workspace_bytes):
+    for fn in (L.ckx_gemm_i8_workspace_bytes, L.ckx_gemm_f16_workspace_bytes, L.ckx_gemm_bf16_workspace_bytes):
         fn.restype = i64
         fn.argtypes = [i32, i32, i32, C.c_int]
     L.ckx_gemm_f16_is_supported.argtypes = shape + [C.c_int]
     L.ckx_gemm_f16.argtypes = [vp, vp, vp] + shape + [C.c_int, vp, i64, vp]
+    L.ckx_gemm_bf16_is_supported.argtypes = shape + [C.c_int]
+    L.ckx_gemm_bf16.argtypes = [vp, vp, vp] + shape + [C.c_int, vp, i64, vp]
     bshape = [i32] * 6 + [i64] * 3 + [i32] + [C.c_int] * 3
     L.ckx_batched_gemm_is_supported.argtypes = [C.c_int] + bshape + [C.c_int, C.c_int]
     L.ckx_batched_gemm_i8.argtypes = [vp, vp, vp] + bshape + [C.c_int, f32, f32, C.c_int, vp]

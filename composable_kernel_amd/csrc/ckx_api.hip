@@ -111,7 +111,7 @@ struct TileInstance
     const char* name;
     int bm, bn, threads, lds;
     float eff; // measured MFMA throughput of this tile shape relative to the 256x256 one
-    tile_launch_fn dense_i8, dense_f16, conv_i8, conv_f16;
+    tile_launch_fn dense_i8, dense_f16, conv_i8, conv_f16, dense_bf16;
 };
 
 #define CKX_TILE(BM, BN, WM, WN, NST, EFF)                                                         \
@@ -120,7 +120,8 @@ struct TileInstance
             WM* WN * 64, NST*(BM + BN) * 128, EFF, &launch_tile<ckx::DT_I8, BM, BN, WM, WN, 128, NST, false>, \
             &launch_tile<ckx::DT_F16, BM, BN, WM, WN, 128, NST, false>,                               \
             &launch_tile<ckx::DT_I8, BM, BN, WM, WN, 128, NST, true>,                                 \
-            &launch_tile<ckx::DT_F16, BM, BN, WM, WN, 128, NST, true>                                 \
+            &launch_tile<ckx::DT_F16, BM, BN, WM, WN, 128, NST, true>,                                \
+            &launch_tile<ckx::DT_BF16, BM, BN, WM, WN, 128, NST, false>                               \
     }
 
 const TileInstance kTiles[] = {
@@ -223,7 +224,7 @@ struct SkinnyInstance
 {
     const char* name;
     int max_m, cols;
-    tile_launch_fn i8, f16;
+    tile_launch_fn i8, f16, bf16;
 };
 
 template <int DT, int MT, int NW, int KU, int NT>
@@ -236,7 +237,8 @@ hipError_t launch_skinny(const ckx::GemmArgs& a, int grid, hipStream_t s)
 #define CKX_SKINNY(MT, NW, KU, NT)                                                                          \
     {                                                                                                       \
         "MI355X_Mfma16_Skinny<rows " #MT "x16, cols " #NT "x16, waves " #NW ", unroll " #KU ">", MT * 16, NT * 16, \
-            &launch_skinny<ckx::DT_I8, MT, NW, KU, NT>, &launch_skinny<ckx::DT_F16, MT, NW, KU, NT>              \
+            &launch_skinny<ckx::DT_I8, MT, NW, KU, NT>, &launch_skinny<ckx::DT_F16, MT, NW, KU, NT>,             \
+            &launch_skinny<ckx::DT_BF16, MT, NW, KU, NT>                                                    \
     }
 
 const SkinnyInstance kSkinny[] = {
@@ -262,6 +264,7 @@ const char* family_prefix(int op)
     case CKX_OP_CONV2D_FWD_F16: return "DeviceConv2dFwd_f16_nhwc_kyxc_nhwk";
     case CKX_OP_BATCHED_GEMM_GEMM: return "DeviceBatchedGemmGemm_f16_gmk_gnk_gno_gmo";
     case CKX_OP_GEMM_SPLITK: return "DeviceGemmSplitK_mk_nk_mn";
+    case CKX_OP_GEMM_BF16: return "DeviceGemm_bf16_bf16_bf16_mk_nk_mn";
     default: return nullptr;
     }
 }
@@ -305,7 +308,7 @@ int check_gemm_shape(int dt, int M, int N, int K, int sa, int sb, int sc, int al
         return fail(CKX_UNSUPPORTED, "this skinny instance covers fewer rows than M");
     if(epi < CKX_EPI_PASSTHROUGH || epi > CKX_EPI_CSHUFFLE_ADD_RELU)
         return fail(CKX_INVALID_VALUE, "unknown epilogue");
-    if(!epilogue_fits_dtype(es, epi))
+    if(!epilogue_fits_dtype(es, epi) || (dt == ckx::DT_BF16 && epi != CKX_EPI_PASSTHROUGH))
         return fail(CKX_UNSUPPORTED, "epilogue not available for this dtype");
     if(al != CKX_ROW_MAJOR || bl != CKX_COL_MAJOR || cl != CKX_ROW_MAJOR)
         return fail(CKX_UNSUPPORTED, "only A row-major, B column-major, C row-major (mk_nk_mn) is built");
@@ -422,7 +425,8 @@ int run_gemm(int dt, const void* a, const void* b, void* c, int M, int N, int K,
     if(ti >= kNumTiles)
     {
         const SkinnyInstance& k = kSkinny[ti - kNumTiles];
-        hipError_t e = (dt == ckx::DT_I8 ? k.i8 : k.f16)(g, (N + k.cols - 1) / k.cols, (hipStream_t)stream);
+        hipError_t e = (dt == ckx::DT_I8 ? k.i8 : dt == ckx::DT_BF16 ? k.bf16 : k.f16)(g, (N + k.cols - 1) / k.cols,
+                                                                                      (hipStream_t)stream);
         return e == hipSuccess ? CKX_OK : hip_fail(e, k.name);
     }
     const TileInstance& t = kTiles[ti];
@@ -432,10 +436,12 @@ int run_gemm(int dt, const void* a, const void* b, void* c, int M, int N, int K,
     g.nk_per     = pl.nk_per;
     g.ws         = ws;
     hipError_t e =
-        (dt == ckx::DT_I8 ? t.dense_i8 : t.dense_f16)(g, g.tiles_m * g.tiles_n * g.ksplit * batch, (hipStream_t)stream);
+        (dt == ckx::DT_I8 ? t.dense_i8 : dt == ckx::DT_BF16 ? t.dense_bf16 : t.dense_f16)(
+            g, g.tiles_m * g.tiles_n * g.ksplit * batch, (hipStream_t)stream);
     if(e == hipSuccess && g.ksplit > 1)
-        e = dt == ckx::DT_I8 ? launch_reduce<ckx::DT_I8>(g, (hipStream_t)stream)
-                             : launch_reduce<ckx::DT_F16>(g, (hipStream_t)stream);
+        e = dt == ckx::DT_I8     ? launch_reduce<ckx::DT_I8>(g, (hipStream_t)stream)
+            : dt == ckx::DT_BF16 ? launch_reduce<ckx::DT_BF16>(g, (hipStream_t)stream)
+                                 : launch_reduce<ckx::DT_F16>(g, (hipStream_t)stream);
     if(e != hipSuccess)
         return hip_fail(e, t.name);
     return CKX_OK;
@@ -607,7 +613,7 @@ const char* ckx_last_error(void) { return g_last_error.c_str(); }
 
 int ckx_num_instances(int op)
 {
-    if(op == CKX_OP_GEMM_I8 || op == CKX_OP_GEMM_F16)
+    if(op == CKX_OP_GEMM_I8 || op == CKX_OP_GEMM_F16 || op == CKX_OP_GEMM_BF16)
         return kNumGemmInsts;
     if(op == CKX_OP_CONV2D_FWD_I8 || op == CKX_OP_GEMM_SPLITK)
         return kNumTiles;
@@ -698,6 +704,25 @@ int ckx_gemm_f16_splitk(const void* a, const void* b, void* c, int32_t M, int32_
         return fail(CKX_INVALID_VALUE, "KBatch must be at least 1");
     return run_gemm(ckx::DT_F16, a, b, c, M, N, K, sa, sb, sc, al, bl, cl, CKX_EPI_PASSTHROUGH, 1.0f, 1.0f,
                     instance, workspace, workspace_bytes, stream, DOperands{}, k_batch);
+}
+
+int ckx_gemm_bf16_is_supported(int32_t M, int32_t N, int32_t K, int32_t sa, int32_t sb, int32_t sc, int al,
+                               int bl, int cl, int instance)
+{
+    return check_gemm_shape(ckx::DT_BF16, M, N, K, sa, sb, sc, al, bl, cl, CKX_EPI_PASSTHROUGH, instance);
+}
+
+int64_t ckx_gemm_bf16_workspace_bytes(int32_t M, int32_t N, int32_t K, int instance)
+{
+    return gemm_workspace_bytes(ckx::DT_BF16, M, N, K, instance);
+}
+
+int ckx_gemm_bf16(const void* a, const void* b, void* c, int32_t M, int32_t N, int32_t K, int32_t sa,
+                  int32_t sb, int32_t sc, int al, int bl, int cl, int instance, void* workspace,
+                  int64_t workspace_bytes, void* stream)
+{
+    return run_gemm(ckx::DT_BF16, a, b, c, M, N, K, sa, sb, sc, al, bl, cl, CKX_EPI_PASSTHROUGH, 1.0f, 1.0f,
+                    instance, workspace, workspace_bytes, stream);
 }
 
 int ckx_batched_gemm_is_supported(int op, int32_t M, int32_t N, int32_t K, int32_t sa, int32_t sb, int32_t sc,

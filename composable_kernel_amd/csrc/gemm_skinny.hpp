@@ -85,6 +85,10 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(const GemmArgs p)
                     if constexpr(DT == DT_I8)
                         acc[mt][nt] =
                             __builtin_amdgcn_mfma_i32_16x16x64_i8(bq[nt][u], aq[mt][u], acc[mt][nt], 0, 0, 0);
+                    else if constexpr(DT == DT_BF16)
+                        acc[mt][nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
+                            __builtin_bit_cast(bf16x8, bq[nt][u]), __builtin_bit_cast(bf16x8, aq[mt][u]), acc[mt][nt],
+                            0, 0, 0);
                     else
                         acc[mt][nt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(
                             __builtin_bit_cast(f16x8, bq[nt][u]), __builtin_bit_cast(f16x8, aq[mt][u]), acc[mt][nt],
@@ -146,6 +150,14 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(const GemmArgs p)
                     if(nn + j < p.N)
                         crow[j] = (int8_t)b[j];
             }
+        }
+        else if constexpr(DT == DT_BF16)
+        {
+            __bf16* crow = reinterpret_cast<__bf16*>(p.c) + (size_t)m * p.ldc + nn;
+#pragma unroll
+            for(int j = 0; j < 4; ++j)
+                if(nn + j < p.N)
+                    crow[j] = (__bf16)s[j];
         }
         else
         {

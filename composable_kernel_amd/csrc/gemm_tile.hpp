@@ -37,11 +37,13 @@ typedef int i32x2 __attribute__((ext_vector_type(2)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
 typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 
 enum
 {
-    DT_I8  = 0,
-    DT_F16 = 1
+    DT_I8   = 0,
+    DT_F16  = 1,
+    DT_BF16 = 2 // bfloat16 operands and output, fp32 accumulation, one round-to-nearest-even conversion
 };
 
 enum
@@ -261,22 +263,25 @@ __device__ __forceinline__ void store_row16_f16_fused(_Float16* crow, int n0, in
                                                       int mode, const _Float16* d0row, const _Float16* d1row,
                                                       bool dvec_ok, bool nt);
 
-__device__ __forceinline__ void store_row16_f16(_Float16* crow, int n0, int N, bool vec_ok,
-                                                const f32x4 (&v)[4], bool nt = false)
+// T = _Float16 or __bf16
+template <typename T>
+__device__ __forceinline__ void store_row16_f16(T* crow, int n0, int N, bool vec_ok, const f32x4 (&v)[4],
+                                                bool nt = false)
 {
+    typedef T tx8 __attribute__((ext_vector_type(8)));
     if(vec_ok && n0 + 16 <= N)
     {
-        f16x8 lo, hi;
+        tx8 lo, hi;
 #pragma unroll
         for(int j = 0; j < 4; ++j)
         {
-            lo[j]     = (_Float16)v[0][j];
-            lo[4 + j] = (_Float16)v[1][j];
-            hi[j]     = (_Float16)v[2][j];
-            hi[4 + j] = (_Float16)v[3][j];
+            lo[j]     = (T)v[0][j];
+            lo[4 + j] = (T)v[1][j];
+            hi[j]     = (T)v[2][j];
+            hi[4 + j] = (T)v[3][j];
         }
-        store_vec(reinterpret_cast<f16x8*>(crow + n0), lo, nt);
-        store_vec(reinterpret_cast<f16x8*>(crow + n0 + 8), hi, nt);
+        store_vec(reinterpret_cast<tx8*>(crow + n0), lo, nt);
+        store_vec(reinterpret_cast<tx8*>(crow + n0 + 8), hi, nt);
     }
     else
     {
@@ -285,7 +290,7 @@ __device__ __forceinline__ void store_row16_f16(_Float16* crow, int n0, int N, b
 #pragma unroll
             for(int j = 0; j < 4; ++j)
                 if(n0 + t * 4 + j < N)
-                    crow[n0 + t * 4 + j] = (_Float16)v[t][j];
+                    crow[n0 + t * 4 + j] = (T)v[t][j];
     }
 }
 
@@ -576,6 +581,9 @@ struct GemmTile
             const int i = m / (NG * 4), t = m % (NG * 4);
             if constexpr(DT == DT_I8)
                 acc[i][t] = __builtin_amdgcn_mfma_i32_16x16x64_i8(bf[t], af[i], acc[i][t], 0, 0, 0);
+            else if constexpr(DT == DT_BF16)
+                acc[i][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, bf[t]),
+                                                                 __builtin_bit_cast(bf16x8, af[i]), acc[i][t], 0, 0, 0);
             else
                 acc[i][t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, bf[t]),
                                                                 __builtin_bit_cast(f16x8, af[i]), acc[i][t], 0, 0, 0);
@@ -669,10 +677,14 @@ struct GemmTile
                         }
                         else
                         {
-                            _Float16* crow   = reinterpret_cast<_Float16*>(c_batch) + (size_t)m * p.ldc;
                             const f32x4 v[4] = {acc[i][g * 4], acc[i][g * 4 + 1], acc[i][g * 4 + 2],
                                                 acc[i][g * 4 + 3]};
-                            store_row16_f16(crow, n0, p.N, vec_ok, v, nt);
+                            if constexpr(DT == DT_BF16)
+                                store_row16_f16(reinterpret_cast<__bf16*>(c_batch) + (size_t)m * p.ldc, n0, p.N, vec_ok,
+                                                v, nt);
+                            else
+                                store_row16_f16(reinterpret_cast<_Float16*>(c_batch) + (size_t)m * p.ldc, n0, p.N,
+                                                vec_ok, v, nt);
                         }
                     }
 #pragma unroll
@@ -914,6 +926,8 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(const GemmArgs p)
         else
             store_row16_i8<EPI_PASSTHROUGH>(crow, n0, p.N, vec_ok, v, p.scale_gemm, p.scale_relu);
     }
+    else if constexpr(DT == DT_BF16)
+        store_row16_f16(reinterpret_cast<__bf16*>(p.c) + (size_t)m * p.ldc, n0, p.N, vec_ok, v);
     else
     {
         _Float16* crow = reinterpret_cast<_Float16*>(p.c) + (size_t)m * p.ldc;

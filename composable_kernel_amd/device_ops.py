@@ -253,6 +253,26 @@ class DeviceGemmSplitKF16(_DeviceGemmSplitK):
                                               a.workspace_bytes_, C.c_void_p(stream or 0))
 
 
+class DeviceGemmBF16(_DeviceGemm):
+    """DeviceGemm<..., bhalf_t, bhalf_t, bhalf_t, PassThrough, PassThrough, PassThrough>"""
+    op_family = capi.OP_GEMM_BF16
+
+    def _supported(self, a):
+        if not isinstance(a.c_op, PassThrough):
+            capi.lib().ckx_gemm_bf16_is_supported(-1, 0, 0, 0, 0, 0, 0, 0, 0, 0)
+            return capi.UNSUPPORTED
+        return capi.lib().ckx_gemm_bf16_is_supported(a.M, a.N, a.K, a.StrideA, a.StrideB, a.StrideC,
+                                                     *self.layouts, self.instance)
+
+    def GetWorkSpaceSize(self, a):
+        return int(capi.lib().ckx_gemm_bf16_workspace_bytes(a.M, a.N, a.K, self.instance))
+
+    def _launch(self, a, stream):
+        return capi.lib().ckx_gemm_bf16(a.p_a, a.p_b, a.p_c, a.M, a.N, a.K, a.StrideA, a.StrideB, a.StrideC,
+                                        *self.layouts, self.instance, a.p_workspace_ or 0, a.workspace_bytes_,
+                                        C.c_void_p(stream or 0))
+
+
 class _DeviceBatchedGemm(_DeviceGemm):
     """DeviceBatchedGemm<...> (device_batched_gemm.hpp:24-45): strided batch, element strides."""
 

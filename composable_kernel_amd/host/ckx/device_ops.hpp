@@ -38,6 +38,7 @@ namespace ck {
 using index_t      = int32_t;
 using long_index_t = int64_t;
 using half_t       = _Float16;
+using bhalf_t      = unsigned short; // bfloat16 bit pattern (include/ck/utility/data_type.hpp:10)
 
 struct StreamConfig
 {
@@ -386,6 +387,11 @@ struct DTypeOf<half_t>
 {
     static constexpr bool is_i8 = false;
 };
+template <>
+struct DTypeOf<bhalf_t>
+{
+    static constexpr bool is_i8 = false;
+};
 
 } // namespace detail
 
@@ -399,11 +405,12 @@ struct DeviceGemmMfma : public DeviceGemm<ALayout, BLayout, CLayout, ADataType, 
                                           AElementwiseOperation, BElementwiseOperation, CElementwiseOperation>
 {
     static_assert(std::is_same_v<ADataType, BDataType> && std::is_same_v<ADataType, CDataType>,
-                  "A, B and C share one data type (int8_t or half_t)");
+                  "A, B and C share one data type (int8_t, half_t or bhalf_t)");
     static_assert(std::is_same_v<AElementwiseOperation, element_wise::PassThrough> &&
                       std::is_same_v<BElementwiseOperation, element_wise::PassThrough>,
                   "A/B element-wise operations other than PassThrough are not built");
-    static constexpr bool is_i8 = detail::DTypeOf<ADataType>::is_i8;
+    static constexpr bool is_i8   = detail::DTypeOf<ADataType>::is_i8;
+    static constexpr bool is_bf16 = std::is_same_v<ADataType, bhalf_t>;
     using Epi                   = ckx::EpilogueOf<CElementwiseOperation>;
     static_assert(is_i8 || Epi::kind == CKX_EPI_PASSTHROUGH, "fp16 GEMM only has the PassThrough epilogue");
 
@@ -426,6 +433,9 @@ struct DeviceGemmMfma : public DeviceGemm<ALayout, BLayout, CLayout, ADataType, 
         if constexpr(is_i8)
             return ckx_gemm_i8_is_supported(a.M, a.N, a.K, a.StrideA, a.StrideB, a.StrideC, ALayout::code,
                                             BLayout::code, CLayout::code, Epi::kind, inst);
+        else if constexpr(is_bf16)
+            return ckx_gemm_bf16_is_supported(a.M, a.N, a.K, a.StrideA, a.StrideB, a.StrideC, ALayout::code,
+                                              BLayout::code, CLayout::code, inst);
         else
             return ckx_gemm_f16_is_supported(a.M, a.N, a.K, a.StrideA, a.StrideB, a.StrideC, ALayout::code,
                                              BLayout::code, CLayout::code, inst);
@@ -437,13 +447,18 @@ struct DeviceGemmMfma : public DeviceGemm<ALayout, BLayout, CLayout, ADataType, 
             return ckx_gemm_i8(a.p_a, a.p_b, a.p_c, a.M, a.N, a.K, a.StrideA, a.StrideB, a.StrideC, ALayout::code,
                                BLayout::code, CLayout::code, Epi::kind, Epi::scale_gemm(a.c_element_op),
                                Epi::scale_relu(a.c_element_op), inst, a.p_workspace_, ws_bytes, stream);
+        else if constexpr(is_bf16)
+            return ckx_gemm_bf16(a.p_a, a.p_b, a.p_c, a.M, a.N, a.K, a.StrideA, a.StrideB, a.StrideC, ALayout::code,
+                                 BLayout::code, CLayout::code, inst, a.p_workspace_, ws_bytes, stream);
         else
             return ckx_gemm_f16(a.p_a, a.p_b, a.p_c, a.M, a.N, a.K, a.StrideA, a.StrideB, a.StrideC, ALayout::code,
                                 BLayout::code, CLayout::code, inst, a.p_workspace_, ws_bytes, stream);
     }
     static int64_t WorkSpaceBytes(const Argument& a, int inst)
     {
-        return is_i8 ? ckx_gemm_i8_workspace_bytes(a.M, a.N, a.K, inst) : ckx_gemm_f16_workspace_bytes(a.M, a.N, a.K, inst);
+        return is_i8     ? ckx_gemm_i8_workspace_bytes(a.M, a.N, a.K, inst)
+               : is_bf16 ? ckx_gemm_bf16_workspace_bytes(a.M, a.N, a.K, inst)
+                         : ckx_gemm_f16_workspace_bytes(a.M, a.N, a.K, inst);
     }
     size_t GetWorkSpaceSize(const BaseArgument* p) const override
     {
@@ -479,9 +494,11 @@ struct DeviceGemmMfma : public DeviceGemm<ALayout, BLayout, CLayout, ADataType, 
     std::unique_ptr<BaseInvoker> MakeInvokerPointer() override { return std::make_unique<Invoker>(instance_); }
     std::string GetTypeString() const override
     {
-        const int op = is_i8 ? CKX_OP_GEMM_I8 : CKX_OP_GEMM_F16;
+        const int op = is_i8 ? CKX_OP_GEMM_I8 : is_bf16 ? CKX_OP_GEMM_BF16 : CKX_OP_GEMM_F16;
         if(instance_ == CKX_INSTANCE_AUTO)
-            return is_i8 ? "DeviceGemm_i8_i8_i8_mk_nk_mn<auto>" : "DeviceGemm_f16_f16_f16_mk_nk_mn<auto>";
+            return is_i8     ? "DeviceGemm_i8_i8_i8_mk_nk_mn<auto>"
+                   : is_bf16 ? "DeviceGemm_bf16_bf16_bf16_mk_nk_mn<auto>"
+                             : "DeviceGemm_f16_f16_f16_mk_nk_mn<auto>";
         return ckx_instance_name(op, instance_);
     }
     int instance_;
@@ -1060,7 +1077,7 @@ struct DeviceOperationInstanceFactory<DeviceGemm<AL, BL, CL, T, T, T, AOp, BOp, 
     static std::vector<std::unique_ptr<DeviceOp>> GetInstances()
     {
         std::vector<std::unique_ptr<DeviceOp>> v;
-        const int n = ckx_num_instances(detail::DTypeOf<T>::is_i8 ? CKX_OP_GEMM_I8 : CKX_OP_GEMM_F16);
+        const int n = ckx_num_instances(CKX_OP_GEMM_F16); // the same list for every data type
         for(int i = 0; i < n; ++i)
             v.push_back(std::make_unique<DeviceGemmMfma<AL, BL, CL, T, T, T, AOp, BOp, COp>>(i));
         return v;

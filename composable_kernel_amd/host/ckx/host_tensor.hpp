@@ -9,6 +9,7 @@
 #include <cmath>
 #include <cstdint>
 #include <cstdio>
+#include <cstring>
 #include <stdexcept>
 #include <string>
 #include <vector>
@@ -61,6 +62,43 @@ inline void fill_uniform_f16(std::vector<_Float16>& v, float lo, float hi, uint6
         const float u = (float)(splitmix64(seed, i) >> 40) * (1.0f / (float)(1 << 24));
         v[i]          = (_Float16)(lo + u * (hi - lo));
     }
+}
+
+// bfloat16 bit patterns: widening is a shift, narrowing rounds to nearest even
+// (type_convert<bhalf_t, float>, include/ck/utility/data_type.hpp:953-993, finite inputs)
+inline float bf16_to_float(unsigned short h)
+{
+    const uint32_t u = (uint32_t)h << 16;
+    float f;
+    std::memcpy(&f, &u, 4);
+    return f;
+}
+inline unsigned short float_to_bf16(float x)
+{
+    uint32_t u;
+    std::memcpy(&u, &x, 4);
+    u += 0x7fffu + ((u >> 16) & 1u);
+    return (unsigned short)(u >> 16);
+}
+inline void fill_uniform_bf16(std::vector<unsigned short>& v, float lo, float hi, uint64_t seed)
+{
+    for(std::size_t i = 0; i < v.size(); ++i)
+    {
+        const float u = (float)(splitmix64(seed, i) >> 40) * (1.0f / (float)(1 << 24));
+        v[i]          = float_to_bf16(lo + u * (hi - lo));
+    }
+}
+inline std::size_t count_errors(const std::vector<unsigned short>& out, const std::vector<unsigned short>& ref,
+                                double rtol, double atol)
+{
+    std::size_t bad = 0;
+    for(std::size_t i = 0; i < ref.size(); ++i)
+    {
+        const double o = bf16_to_float(out[i]), r = bf16_to_float(ref[i]);
+        if(std::fabs(o - r) > atol + rtol * std::fabs(r) || !std::isfinite(o) || !std::isfinite(r))
+            ++bad;
+    }
+    return bad;
 }
 
 // |o - r| <= atol + rtol * |r| and finite, as check_err; returns the number of violations

@@ -2,7 +2,7 @@
 // this library. Positional arguments follow the reference's conventions
 // (profiler/src/profile_gemm.cpp:27-75, profile_convnd_fwd.cpp:81-115):
 //
-//   ckx_profiler gemm <dtype 1:fp16 3:int8> <layout 1: A[m,k]*B[n,k]> <verify> <init> <log> <time>
+//   ckx_profiler gemm <dtype 1:fp16 2:bf16 3:int8> <layout 1: A[m,k]*B[n,k]> <verify> <init> <log> <time>
 //                     M N K StrideA StrideB StrideC [epilogue 0|1|2] [scale_gemm] [scale_relu] [nrepeat]
 //   ckx_profiler conv2d_fwd <dtype 1|3> <verify> <init> <log> <time>
 //                     N K C Y X Hi Wi Sy Sx Dy Dx LeftPy LeftPx RightPy RightPx [epilogue sg sr] [nrepeat]
@@ -67,6 +67,20 @@ void fill(std::vector<T>& v, int init, uint64_t seed, bool conv)
         if(init == 0)
             return;
         ckx::fill_uniform_int8(v, -5, 5, seed);
+    }
+    else if constexpr(std::is_same_v<T, bhalf_t>)
+    {
+        if(init == 0)
+            return;
+        if(init == 1)
+        {
+            std::vector<int8_t> t(v.size());
+            ckx::fill_uniform_int8(t, -5, 5, seed);
+            for(std::size_t i = 0; i < v.size(); ++i)
+                v[i] = ckx::float_to_bf16((float)t[i]);
+        }
+        else
+            ckx::fill_uniform_bf16(v, -1.f, 1.f, seed);
     }
     else
     {
@@ -180,7 +194,7 @@ int profile_gemm(int argc, char* argv[])
 {
     if(argc < 14)
     {
-        std::printf("arg1: tensor operation (gemm)\narg2: data type (1: fp16; 3: int8)\n"
+        std::printf("arg1: tensor operation (gemm)\narg2: data type (1: fp16; 2: bf16; 3: int8)\n"
                     "arg3: matrix layout (1: A[m, k] * B[n, k] = C[m, n])\narg4: verification (0: no; 1: yes)\n"
                     "arg5: initialization (0: no init; 1: integer value; 2: decimal value)\n"
                     "arg6: print tensor value (0: no; 1: yes)\narg7: time kernel (0=no, 1=yes)\n"
@@ -203,6 +217,9 @@ int profile_gemm(int argc, char* argv[])
     if(dtype == 1)
         return profile_gemm_t<half_t>(verify, init, time_kernel, M, N, K, sa, sb, sc, Pass{},
                                       argc > 14 ? std::atoi(argv[14]) : 10);
+    if(dtype == 2)
+        return profile_gemm_t<bhalf_t>(verify, init, time_kernel, M, N, K, sa, sb, sc, Pass{},
+                                       argc > 14 ? std::atoi(argv[14]) : 10);
     if(dtype == 3)
     {
         const int epi  = argc > 14 ? std::atoi(argv[14]) : 0;

@@ -29,3 +29,13 @@ def uniform_f16(shape, lo, hi, seed):
     n = int(np.prod(shape))
     u = (splitmix64(seed, n) >> np.uint64(40)).astype(np.float32) * np.float32(1.0 / (1 << 24))
     return (np.float32(lo) + u * np.float32(hi - lo)).astype(np.float16).reshape(shape)
+
+
+def uniform_bf16(shape, lo, hi, seed):
+    """fp32 uniform in [lo, hi) from 24 random bits, rounded to nearest-even bfloat16; returned as
+    uint16 bit patterns (numpy has no bfloat16)."""
+    n = int(np.prod(shape))
+    u = (splitmix64(seed, n) >> np.uint64(40)).astype(np.float32) * np.float32(1.0 / (1 << 24))
+    x = (np.float32(lo) + u * np.float32(hi - lo)).astype(np.float32)
+    b = x.view(np.uint32).astype(np.uint64)
+    return ((b + 0x7FFF + ((b >> 16) & 1)) >> 16).astype(np.uint16).reshape(shape)

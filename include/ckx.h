@@ -72,7 +72,8 @@ enum
     CKX_OP_CONV2D_FWD_I8     = 2,
     CKX_OP_CONV2D_FWD_F16    = 3,
     CKX_OP_BATCHED_GEMM_GEMM = 4,
-    CKX_OP_GEMM_SPLITK       = 5 /* instance list of the split-K GEMMs (the tile instances, both dtypes) */
+    CKX_OP_GEMM_SPLITK       = 5, /* instance list of the split-K GEMMs (the tile instances, both dtypes) */
+    CKX_OP_GEMM_BF16         = 6
 };
 
 #define CKX_INSTANCE_AUTO (-1)
@@ -118,6 +119,17 @@ int ckx_gemm_f16(const void* p_a, const void* p_b, void* p_c, int32_t M, int32_t
                  int32_t stride_a, int32_t stride_b, int32_t stride_c, int a_layout, int b_layout,
                  int c_layout, int instance, void* p_workspace, int64_t workspace_bytes, void* stream);
 int64_t ckx_gemm_f16_workspace_bytes(int32_t M, int32_t N, int32_t K, int instance);
+
+/* ---- bf16 GEMM:  C = bf16(A * B), fp32 accumulation ------------------------
+ * Replaces DeviceGemm<..., bhalf_t, bhalf_t, bhalf_t, PassThrough x3> (device_gemm.hpp:24-41; the bf16
+ * instances of the reference's gemm family); the conversion is round-to-nearest-even, as
+ * type_convert<bhalf_t, float> (include/ck/utility/data_type.hpp:953-993). */
+int ckx_gemm_bf16_is_supported(int32_t M, int32_t N, int32_t K, int32_t stride_a, int32_t stride_b,
+                               int32_t stride_c, int a_layout, int b_layout, int c_layout, int instance);
+int ckx_gemm_bf16(const void* p_a, const void* p_b, void* p_c, int32_t M, int32_t N, int32_t K,
+                  int32_t stride_a, int32_t stride_b, int32_t stride_c, int a_layout, int b_layout,
+                  int c_layout, int instance, void* p_workspace, int64_t workspace_bytes, void* stream);
+int64_t ckx_gemm_bf16_workspace_bytes(int32_t M, int32_t N, int32_t K, int instance);
 
 /* ---- strided batched GEMM:  C[g] = c_op(A[g] * B[g]),  g < batch ----------------
  * Replaces DeviceBatchedGemm<...>::MakeArgumentPointer(..., BatchStrideA, BatchStrideB, BatchStrideC,

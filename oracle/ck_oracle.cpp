@@ -275,6 +275,44 @@ void cko_gemm_f16(const uint16_t* a, const uint16_t* b, uint16_t* c, int M, int 
     });
 }
 
+// bfloat16 <-> float as type_convert<float, bhalf_t> / type_convert<bhalf_t, float> do it
+// (include/ck/utility/data_type.hpp:940-993): widening is a shift; narrowing rounds to nearest even by
+// adding 0x7fff + lsb unless the exponent is all ones, where a NaN keeps a mantissa bit.
+uint16_t cko_float_to_bf16(float x)
+{
+    uint32_t u;
+    std::memcpy(&u, &x, 4);
+    if(~u & 0x7f800000u)
+        u += 0x7fffu + ((u >> 16) & 1u);
+    else if(u & 0xffffu)
+        u |= 0x10000u;
+    return (uint16_t)(u >> 16);
+}
+
+float cko_bf16_to_float(uint16_t h)
+{
+    const uint32_t u = (uint32_t)h << 16;
+    float f;
+    std::memcpy(&f, &u, 4);
+    return f;
+}
+
+// bf16 GEMM, AccDataType = float, sequential k, PassThrough everywhere (ReferenceGemm with bhalf_t).
+void cko_gemm_bf16(const uint16_t* a, const uint16_t* b, uint16_t* c, int M, int N, int K, int64_t sa_m,
+                   int64_t sa_k, int64_t sb_k, int64_t sb_n, int64_t sc_m, int64_t sc_n, int nthreads)
+{
+    parallel_for((std::size_t)M * (std::size_t)N, nthreads, [&](std::size_t i0, std::size_t i1) {
+        for(std::size_t i = i0; i < i1; ++i)
+        {
+            const std::size_t m = i / (std::size_t)N, n = i % (std::size_t)N;
+            float acc           = 0;
+            for(int k = 0; k < K; ++k)
+                acc += cko_bf16_to_float(a[m * sa_m + k * sa_k]) * cko_bf16_to_float(b[k * sb_k + n * sb_n]);
+            c[m * sc_m + n * sc_n] = cko_float_to_bf16(acc);
+        }
+    });
+}
+
 // Strided batched fp16 GEMM: A [G,M,K], B [G,K,N], C [G,M,N], element strides.
 void cko_batched_gemm_f16(const uint16_t* a, const uint16_t* b, uint16_t* c, int G, int M, int N, int K,
                           int64_t sa_g, int64_t sa_m, int64_t sa_k, int64_t sb_g, int64_t sb_k,

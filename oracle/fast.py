@@ -54,6 +54,23 @@ def gemm_f16(a_mk, b_kn):
     return (np.asarray(a_mk, np.float32) @ np.asarray(b_kn, np.float32)).astype(np.float16)
 
 
+def bf16_to_f32(u16):
+    """uint16 bfloat16 bit patterns -> float32."""
+    return (np.asarray(u16, np.uint16).astype(np.uint32) << 16).view(np.float32)
+
+
+def f32_to_bf16(x):
+    """float32 -> uint16 bfloat16 bit patterns, round to nearest even (finite inputs)."""
+    u = np.asarray(x, np.float32).view(np.uint32).astype(np.uint64)
+    u = u + 0x7FFF + ((u >> 16) & 1)
+    return (u >> 16).astype(np.uint16)
+
+
+def gemm_bf16(a_mk, b_kn):
+    """fp32-accumulated product of bf16 operands rounded once to bf16 (BLAS summation order)."""
+    return f32_to_bf16(bf16_to_f32(a_mk) @ bf16_to_f32(b_kn))
+
+
 def im2col(inp_nhwc, Y, X, strides, dilations, pads, right_pads=None):
     """[N,Hi,Wi,C] -> [N*Ho*Wo, Y*X*C] with (y,x,c) ordering, c fastest; zero padding."""
     if right_pads is None:

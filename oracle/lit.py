@@ -96,6 +96,24 @@ def gemm_f16(a_mk, b_kn, nthreads=0):
     return c
 
 
+def float_to_bf16(x):
+    """float32 array -> uint16 array of bfloat16 bit patterns (the reference's round-to-nearest-even)."""
+    lib().cko_float_to_bf16.restype = C.c_uint16
+    lib().cko_float_to_bf16.argtypes = [C.c_float]
+    flat = np.asarray(x, np.float32).ravel()
+    return np.array([lib().cko_float_to_bf16(float(v)) for v in flat], np.uint16).reshape(np.shape(x))
+
+
+def gemm_bf16(a_mk, b_kn, nthreads=0):
+    """a, b: uint16 arrays of bfloat16 bit patterns; returns uint16 [M,N]."""
+    M, K = a_mk.shape
+    _, N = b_kn.shape
+    c = np.empty((M, N), np.uint16)
+    lib().cko_gemm_bf16(_p(a_mk), _p(b_kn), _p(c), M, N, K, *_i64(*_estrides(a_mk)), *_i64(*_estrides(b_kn)),
+                        *_i64(N, 1), int(nthreads))
+    return c
+
+
 def batched_gemm_f16(a_gmk, b_gkn, nthreads=0):
     G, M, K = a_gmk.shape
     _, _, N = b_gkn.shape

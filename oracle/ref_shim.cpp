@@ -232,6 +232,17 @@ void ckref_conv2d_fwd_bias_relu_f16(const uint16_t* in, const uint16_t* wei, con
     std::memcpy(out, to.mData.data(), to.mData.size() * sizeof(T));
 }
 
+// ReferenceGemm<bhalf_t, bhalf_t, bhalf_t, float, Pass, Pass, Pass> (the reference's bf16 GEMM check)
+void ckref_gemm_bf16(const uint16_t* a, const uint16_t* b, uint16_t* c, int M, int N, int K, long sa_m,
+                     long sa_k, long sb_k, long sb_n, long sc_m, long sc_n)
+{
+    using Ref = ck::tensor_operation::host::ReferenceGemm<ck::bhalf_t, ck::bhalf_t, ck::bhalf_t, float, PassThrough,
+                                                          PassThrough, PassThrough>;
+    run_gemm<Ref, ck::bhalf_t, ck::bhalf_t>(a, b, c, M, N, K, sa_m, sa_k, sb_k, sb_n, sc_m, sc_n, PassThrough{});
+}
+
+uint16_t ckref_float_to_bf16(float x) { return ck::type_convert<ck::bhalf_t>(x); }
+
 // example 03's verification: ReferenceGemm<half,half,float,float,...> then AddRelu on half_t
 void ckref_gemm_f16_add_relu(const uint16_t* a, const uint16_t* b, const uint16_t* d, uint16_t* e, int M, int N,
                              int K, long sa_m, long sa_k, long sb_k, long sb_n, long sd_m, long sd_n)

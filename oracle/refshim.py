@@ -108,6 +108,18 @@ class _Ref:
         self.lib.ckref_gemm_f16_add_relu(_p(a_mk), _p(b_kn), _p(d), _p(e), M, N, K, *_es(a_mk), *_es(b_kn), *_es(d))
         return e
 
+    def gemm_bf16(self, a_mk, b_kn):
+        M, K = a_mk.shape
+        _, N = b_kn.shape
+        c = np.zeros((M, N), np.uint16)
+        self.lib.ckref_gemm_bf16(_p(a_mk), _p(b_kn), _p(c), M, N, K, *_es(a_mk), *_es(b_kn), C.c_long(N), C.c_long(1))
+        return c
+
+    def float_to_bf16(self, x):
+        self.lib.ckref_float_to_bf16.restype = C.c_uint16
+        self.lib.ckref_float_to_bf16.argtypes = [C.c_float]
+        return int(self.lib.ckref_float_to_bf16(float(x)))
+
     def conv_out_len(self, in_len, filt, stride, dil, pl, pr):
         return int(self.lib.ckref_conv_out_len(in_len, filt, stride, dil, pl, pr))
 

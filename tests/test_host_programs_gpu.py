@@ -152,3 +152,16 @@ def test_profiler_batched_gemm_fp16(tmp_path):
     ref = lit.batched_gemm_f16(a, np.ascontiguousarray(b_gnk.transpose(0, 2, 1)))
     bad, max_err = lit.check_err_f16(c, ref, 1e-2, 1e-2)
     assert bad == 0, max_err
+
+
+def test_profiler_bf16_gemm(tmp_path):
+    """data type 2 of the reference profiler's gemm operation (bf16)."""
+    from composable_kernel_amd.host_tensor import uniform_bf16
+    M, N, K = 384, 512, 768
+    out, dump = _run("ckx_profiler", ["gemm", 2, 1, 1, 2, 0, 1, M, N, K, -1, -1, -1], "CKX_PROFILER_DUMP", tmp_path)
+    assert "Best Perf:" in out and "Error" not in out and "bf16" in out
+    c = fast.bf16_to_f32(np.fromfile(dump, np.uint16).reshape(M, N))
+    a = uniform_bf16((M, K), -1, 1, SEED)
+    b_nk = uniform_bf16((N, K), -1, 1, SEED + 1)
+    ref = fast.bf16_to_f32(lit.gemm_bf16(a, np.ascontiguousarray(b_nk.T)))
+    assert np.all(np.abs(c - ref) <= 1e-2 + 1e-2 * np.abs(ref))

@@ -404,3 +404,47 @@ def test_gemm_add_relu_random_lit_ref_bit_exact_and_full_d():
         np.testing.assert_array_equal(e, np.maximum(x, np.float16(0)))
         if REF is not None:
             np.testing.assert_array_equal(REF.gemm_f16_add_relu(a, b, d), e)
+
+
+# ------------------------------------------------------------------------------- bfloat16
+def test_bf16_conversion_is_round_to_nearest_even_like_torch_and_the_reference():
+    """type_convert<bhalf_t, float> (data_type.hpp:953-993): checked against torch's bfloat16 cast (an
+    independent RNE implementation) on random floats, exact ties, the largest finite values and
+    subnormals, and against the reference's own function."""
+    import torch
+    rng = np.random.default_rng(11)
+    x = np.concatenate([
+        rng.standard_normal(4000).astype(np.float32) * np.float32(10.0) ** rng.integers(-30, 30, 4000).astype(np.float32),
+        np.array([1.0, 1.00390625, 1.01171875, 1.0078125, -1.00390625, 3.3895314e38, 3.4028235e38, 1e-40, -1e-45, 0.0,
+                  -0.0, 65280.0, 65408.0], np.float32)])
+    want = torch.from_numpy(x).to(torch.bfloat16).view(torch.int16).numpy().view(np.uint16)
+    got = lit.float_to_bf16(x)
+    np.testing.assert_array_equal(got, want)
+    np.testing.assert_array_equal(fast.f32_to_bf16(x), want)
+    # ties: 1 + 2^-8 is halfway between bf16(1.0) = 0x3F80 and 0x3F81 -> even (0x3F80); 1 + 3*2^-8 -> 0x3F82
+    assert lit.float_to_bf16(np.float32(1.00390625)) == 0x3F80 and lit.float_to_bf16(np.float32(1.01171875)) == 0x3F82
+    np.testing.assert_array_equal(fast.bf16_to_f32(got), torch.from_numpy(x).to(torch.bfloat16).float().numpy())
+    if REF is not None:
+        for v in x[::97]:
+            assert REF.float_to_bf16(v) == int(lit.float_to_bf16(v))
+
+
+def test_gemm_bf16_closed_forms_fast_and_ref():
+    from composable_kernel_amd.host_tensor import uniform_bf16
+    # ones: every entry is K, exact in bf16 up to 256
+    a = np.full((5, 192), 0x3F80, np.uint16)
+    b = np.asfortranarray(np.full((192, 7), 0x3F80, np.uint16))
+    np.testing.assert_array_equal(lit.gemm_bf16(a, b), np.full((5, 7), lit.float_to_bf16(np.float32(192.0)), np.uint16))
+    # K = 257 ones -> 257 is not a bf16 (8 significant bits): tie between 256 and 258 -> 256
+    a = np.full((2, 257), 0x3F80, np.uint16)
+    b = np.asfortranarray(np.full((257, 3), 0x3F80, np.uint16))
+    assert np.all(fast.bf16_to_f32(lit.gemm_bf16(a, b)) == 256.0)
+    a = uniform_bf16((33, 160), -1, 1, 21)
+    b = np.asfortranarray(uniform_bf16((160, 29), -1, 1, 22))
+    c = lit.gemm_bf16(a, b)
+    exact = fast.bf16_to_f32(a).astype(np.float64) @ fast.bf16_to_f32(b).astype(np.float64)
+    assert np.all(np.abs(fast.bf16_to_f32(c) - exact) <= 2.0 ** -8 * np.abs(exact) + 1e-4)
+    f = fast.bf16_to_f32(fast.gemm_bf16(a, b))
+    assert np.all(np.abs(fast.bf16_to_f32(c) - f) <= 1e-2 + 1e-2 * np.abs(f))
+    if REF is not None:
+        np.testing.assert_array_equal(REF.gemm_bf16(a, b), c)
