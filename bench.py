@@ -47,10 +47,12 @@ def _conv_workload(name, dtype, C, K, f, HW, st, pd, N=256, fused=None):
                 fused=fused)
 
 
-def _gemm_workload(name, dtype, M, N, K, values=5, scales=(0.5, 0.03), fused=None, batch=1):
-    """fused: None or "bias_relu" (fp16: E = AddRelu(half(A*B), bias row)); batch > 1: strided batched GEMM."""
+def _gemm_workload(name, dtype, M, N, K, values=5, scales=(0.5, 0.03), fused=None, batch=1, layout="mk_nk"):
+    """fused: None or "bias_relu" (fp16: E = AddRelu(half(A*B), bias row)); batch > 1: strided batched GEMM;
+    layout: how A ("mk" row-major / "km" column-major) and B ("nk" column-major / "kn" row-major) are stored."""
     es = 1 if dtype == "i8" else 2
     return dict(name=name, kind="gemm", dtype=dtype, M=M, N=N, K=K, values=values, scales=scales, batch=batch,
+                layout=layout,
                 ops=2.0 * M * N * K * batch, bytes=(M * K + N * K + M * N + (N if fused else 0)) * es * batch,
                 fused=fused)
 
@@ -67,6 +69,8 @@ for w in (
     + [_conv_workload(f"conv_{dt}_c512_k512_3x3_7", dt, 512, 512, 3, 7, 1, 1) for dt in ("f16", "i8")]
     + [_gemm_workload("fp16_batched_gemm_g16_1024", "f16", 1024, 1024, 1024, batch=16),
        _gemm_workload("bf16_gemm_4096", "bf16", 4096, 4096, 4096)]
+    + [_gemm_workload(f"fp16_gemm_4096_{lay}", "f16", 4096, 4096, 4096, layout=lay) for lay in ("km_kn", "km_nk", "mk_kn")]
+    + [_gemm_workload(f"int8_requant_gemm_4096_{lay}", "i8", 4096, 4096, 4096, layout=lay) for lay in ("km_kn", "km_nk", "mk_kn")]
     + [_gemm_workload("fp16_gemm_bias_relu_4096", "f16", 4096, 4096, 4096, fused="bias_relu"),
        _conv_workload("conv_f16_c64_k64_3x3_56_bias_relu_add", "f16", 64, 64, 3, 56, 1, 1, fused="bias_relu_add"),
        _conv_workload("conv_f16_c256_k512_1x1_56_s2_bias_relu", "f16", 256, 512, 1, 56, 2, 0, fused="bias_relu")]
@@ -94,15 +98,19 @@ def make_launcher(w, instance=-1, rotate=1):
 
     if w["kind"] == "gemm":
         M, N, K = w["M"], w["N"], w["K"]
+        la, lb = w.get("layout", "mk_nk").split("_")
+        a_shape, b_shape = ((M, K) if la == "mk" else (K, M)), ((N, K) if lb == "nk" else (K, N))
+        lay = dict(ALayout=ck.RowMajor if la == "mk" else ck.ColumnMajor, BLayout=ck.ColumnMajor if lb == "nk" else ck.RowMajor)
+        sa, sb = a_shape[1], b_shape[1]
         if w["dtype"] == "i8":
-            a, b = dev(uniform_int8((M, K), -w["values"], w["values"], 1)), dev(uniform_int8((N, K), -w["values"], w["values"], 2))
+            a, b = dev(uniform_int8(a_shape, -w["values"], w["values"], 1)), dev(uniform_int8(b_shape, -w["values"], w["values"], 2))
             c = torch.empty((M, N), dtype=torch.int8, device="cuda")
-            op = ck.DeviceGemmInt8(instance)
+            op = ck.DeviceGemmInt8(instance, **lay)
             cop = ck.RequantReluRequant(w["scales"][0], w["scales"][1], rounded=True)
         else:
-            a, b = dev(uniform_f16((M, K), -1, 1, 1)), dev(uniform_f16((N, K), -1, 1, 2))
+            a, b = dev(uniform_f16(a_shape, -1, 1, 1)), dev(uniform_f16(b_shape, -1, 1, 2))
             c = torch.empty((M, N), dtype=torch.float16, device="cuda")
-            op = ck.DeviceGemmF16(instance)
+            op = ck.DeviceGemmF16(instance, **lay)
             cop = ck.PassThrough()
         G = w.get("batch", 1)
         if w["dtype"] == "bf16":
@@ -122,7 +130,7 @@ def make_launcher(w, instance=-1, rotate=1):
             op = ck.DeviceGemmMultipleDF16(instance)
             make = lambda bb: op.MakeArgumentPointer(a, bb, [bias], c, M, N, K, K, K, [0], N, None, None, ck.AddRelu())
         else:
-            make = lambda bb: op.MakeArgumentPointer(a, bb, c, M, N, K, K, K, N, None, None, cop)
+            make = lambda bb: op.MakeArgumentPointer(a, bb, c, M, N, K, sa, sb, N, None, None, cop)
         arg = make(b)
         more_args = []
         for _ in range(rotate - 1):

@@ -34,20 +34,30 @@ def stale():
 
 
 def build_lib(force=False, verbose=False, extra_flags=()):
-    """Compile csrc/*.hip into lib/libckx.so. Returns the library path."""
+    """Compile csrc/*.hip (side by side) into objects and link lib/libckx.so. Returns the library path."""
     if not force and not stale():
         return LIB
+    from concurrent.futures import ThreadPoolExecutor
     os.makedirs(LIBDIR, exist_ok=True)
-    cmd = [HIPCC] + DEVICE_FLAGS + list(extra_flags) + ["-fPIC", "-shared", "-I" + os.path.join(ROOT, "include"),
-                                                        "-I" + CSRC, os.path.join(CSRC, "ckx_api.hip"), "-o", LIB]
-    if verbose:
-        print(" ".join(cmd))
-    r = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
-    out = "\n".join(l for l in r.stdout.splitlines() if "packed-fp32-ops" not in l)
-    if r.returncode != 0:
-        raise RuntimeError("hipcc failed:\n" + out)
-    if verbose and out.strip():
-        print(out)
+    units = [f for f in sources() if f.endswith(".hip")]
+    objs = [os.path.join(LIBDIR, os.path.basename(u)[:-4] + ".o") for u in units]
+
+    def run(cmd):
+        if verbose:
+            print(" ".join(cmd))
+        r = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+        out = "\n".join(l for l in r.stdout.splitlines() if "packed-fp32-ops" not in l)
+        if r.returncode != 0:
+            raise RuntimeError("hipcc failed:\n" + out)
+        if verbose and out.strip():
+            print(out)
+
+    common = [HIPCC] + DEVICE_FLAGS + list(extra_flags) + ["-fPIC", "-I" + os.path.join(ROOT, "include"), "-I" + CSRC]
+    with ThreadPoolExecutor(max_workers=len(units)) as pool:
+        list(pool.map(lambda uo: run(common + ["-c", uo[0], "-o", uo[1]]), zip(units, objs)))
+    run([HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC"] + objs + ["-o", LIB])
+    for o in objs:
+        os.remove(o)
     return LIB
 
 

@@ -11,6 +11,7 @@
 
 #include "ckx.h"
 #include "gemm_tile.hpp"
+#include "tile_launch.hpp"
 #include "gemm_gemm.hpp"
 #include "conv_patch.hpp"
 #include "gemm_skinny.hpp"
@@ -59,44 +60,9 @@ ckx::MagicDiv make_magic(uint32_t d)
 }
 
 // ------------------------------------------------------------ tile instances
-typedef hipError_t (*tile_launch_fn)(const ckx::GemmArgs&, int grid, hipStream_t);
-
-int num_cus()
-{
-    static int n = [] {
-        int dev = 0, cus = 0;
-        if(hipGetDevice(&dev) != hipSuccess ||
-           hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0)
-            cus = 256;
-        return cus;
-    }();
-    return n;
-}
-
-// Persistent launch: at most (workgroups that fit a CU) x (CUs) workgroups, a multiple of 8 so
-// that workgroup b always lands on XCD b % 8 together with the tiles b, b + grid, ...
-template <int DT, int BM, int BN, int WM, int WN, int BKB, int NST, bool IM2COL>
-hipError_t launch_tile(const ckx::GemmArgs& a, int tiles, hipStream_t s)
-{
-    using T              = ckx::GemmTile<DT, BM, BN, WM, WN, BKB, NST, IM2COL>;
-    auto* kern           = &ckx::gemm_tile_kernel<DT, BM, BN, WM, WN, BKB, NST, IM2COL>;
-    static std::once_flag once;
-    static hipError_t attr_err = hipSuccess;
-    std::call_once(once, [&] {
-        attr_err = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, T::LDS);
-    });
-    if(attr_err != hipSuccess)
-        return attr_err;
-    int per_cu = 160 * 1024 / T::LDS;
-    per_cu     = per_cu > 2048 / T::NT ? 2048 / T::NT : per_cu;
-    per_cu     = per_cu < 1 ? 1 : per_cu;
-    int grid   = num_cus() * per_cu;
-    grid -= grid % 8;
-    grid = tiles < grid ? tiles : grid;
-    hipLaunchKernelGGL(kern, dim3(grid), dim3(T::NT), T::LDS, s, a);
-    return hipGetLastError();
-}
+using ckx::launch_tile;
+using ckx::num_cus;
+using ckx::tile_launch_fn;
 
 template <int DT>
 hipError_t launch_reduce(const ckx::GemmArgs& a, hipStream_t s)
@@ -112,29 +78,22 @@ struct TileInstance
     int bm, bn, threads, lds;
     float eff; // measured MFMA throughput of this tile shape relative to the 256x256 one
     tile_launch_fn dense_i8, dense_f16, conv_i8, conv_f16, dense_bf16;
+    tile_launch_fn dense_f16_fused, conv_f16_fused; // fp16 with the add / ReLU epilogues and D operands
 };
 
 #define CKX_TILE(BM, BN, WM, WN, NST, EFF)                                                         \
-    {                                                                                              \
+    TileInstance{                                                                                  \
         "MI355X_Mfma16_Tile<" #BM ", " #BN ", 128B x" #NST ", waves " #WM "x" #WN ">", BM, BN,           \
             WM* WN * 64, NST*(BM + BN) * 128, EFF, &launch_tile<ckx::DT_I8, BM, BN, WM, WN, 128, NST, false>, \
             &launch_tile<ckx::DT_F16, BM, BN, WM, WN, 128, NST, false>,                               \
             &launch_tile<ckx::DT_I8, BM, BN, WM, WN, 128, NST, true>,                                 \
             &launch_tile<ckx::DT_F16, BM, BN, WM, WN, 128, NST, true>,                                \
-            &launch_tile<ckx::DT_BF16, BM, BN, WM, WN, 128, NST, false>                               \
-    }
+            &launch_tile<ckx::DT_BF16, BM, BN, WM, WN, 128, NST, false>,                              \
+            &launch_tile<ckx::DT_F16, BM, BN, WM, WN, 128, NST, false, false, false, true>,           \
+            &launch_tile<ckx::DT_F16, BM, BN, WM, WN, 128, NST, true, false, false, true>             \
+    },
 
-const TileInstance kTiles[] = {
-    CKX_TILE(256, 256, 2, 4, 2, 1.00f),
-    CKX_TILE(256, 128, 4, 2, 2, 0.84f),
-    CKX_TILE(128, 128, 2, 2, 2, 0.70f),
-    CKX_TILE(128, 64, 4, 1, 2, 0.68f),
-    CKX_TILE(64, 64, 4, 1, 2, 0.55f),
-    CKX_TILE(32, 64, 2, 1, 2, 0.42f),
-    CKX_TILE(16, 64, 1, 1, 2, 0.27f),
-    CKX_TILE(256, 64, 8, 1, 2, 0.70f),
-    CKX_TILE(64, 64, 4, 1, 4, 0.55f),
-};
+const TileInstance kTiles[] = {CKX_FOR_EACH_TILE(CKX_TILE)};
 constexpr int kNumTiles = sizeof(kTiles) / sizeof(kTiles[0]);
 
 // Launch plan: which tile instance, and into how many K runs each C tile is cut (split-K).
@@ -169,7 +128,8 @@ int splitk_runs(int kbytes, int k_batch)
 }
 
 // k_batch > 0: the caller fixed the number of K runs (DeviceGemmSplitK's KBatch)
-Plan make_plan(int M, int N, int kbytes, int only_tile, long workspace_bytes, int k_batch = 0)
+// kmajor: a K-major operand (A column-major / B row-major) -- only the tiles of 64 rows and more
+Plan make_plan(int M, int N, int kbytes, int only_tile, long workspace_bytes, int k_batch = 0, bool kmajor = false)
 {
     Plan best;
     double best_us  = 1e30;
@@ -180,6 +140,8 @@ Plan make_plan(int M, int N, int kbytes, int only_tile, long workspace_bytes, in
         if(only_tile >= 0 && i != only_tile)
             continue;
         const TileInstance& t = kTiles[i];
+        if(kmajor && t.bm < 64)
+            continue;
         const long tiles      = (long)((M + t.bm - 1) / t.bm) * ((N + t.bn - 1) / t.bn);
         for(int sp = 1; sp <= 8; ++sp)
         {
@@ -310,13 +272,23 @@ int check_gemm_shape(int dt, int M, int N, int K, int sa, int sb, int sc, int al
         return fail(CKX_INVALID_VALUE, "unknown epilogue");
     if(!epilogue_fits_dtype(es, epi) || (dt == ckx::DT_BF16 && epi != CKX_EPI_PASSTHROUGH))
         return fail(CKX_UNSUPPORTED, "epilogue not available for this dtype");
-    if(al != CKX_ROW_MAJOR || bl != CKX_COL_MAJOR || cl != CKX_ROW_MAJOR)
-        return fail(CKX_UNSUPPORTED, "only A row-major, B column-major, C row-major (mk_nk_mn) is built");
-    if(sa < K || sb < K || sc < N)
+    if((al != CKX_ROW_MAJOR && al != CKX_COL_MAJOR) || (bl != CKX_ROW_MAJOR && bl != CKX_COL_MAJOR))
+        return fail(CKX_INVALID_VALUE, "unknown layout");
+    if(cl != CKX_ROW_MAJOR)
+        return fail(CKX_UNSUPPORTED, "C is row-major in every instance (as in the reference's instance lists)");
+    // K-major operands: A column-major (element (m,k) at k*sa + m), B row-major ((k,n) at k*sb + n)
+    const bool ta = al == CKX_COL_MAJOR, tb = bl == CKX_ROW_MAJOR;
+    if((ta || tb) && epi >= CKX_EPI_ADD_RELU)
+        return fail(CKX_UNSUPPORTED, "the D-operand epilogues are built for A row-major, B column-major");
+    if((ta || tb) && instance != CKX_INSTANCE_AUTO && !ckx::layout_tile(dt, instance, ta, tb))
+        return fail(CKX_UNSUPPORTED, "this instance has no variant for a K-major operand (tiles of 64 rows and more do)");
+    if(sa < (ta ? M : K) || sb < (tb ? N : K) || sc < N)
         return fail(CKX_UNSUPPORTED, "stride smaller than the contiguous extent");
-    if(((long)K * es) % 16 || ((long)sa * es) % 16 || ((long)sb * es) % 16)
-        return fail(CKX_UNSUPPORTED, "K and the A/B strides must be multiples of 16 bytes");
-    if((long)M * sa * es >= (1l << 31) || (long)N * sb * es >= (1l << 31) || (long)M * sc * es >= (1l << 31))
+    if(((long)(ta ? M : K) * es) % 16 || ((long)(tb ? N : K) * es) % 16 || ((long)sa * es) % 16 ||
+       ((long)sb * es) % 16)
+        return fail(CKX_UNSUPPORTED, "the contiguous extents of A and B and their strides must be multiples of 16 bytes");
+    if((long)(ta ? K : M) * sa * es >= (1l << 31) || (long)(tb ? K : N) * sb * es >= (1l << 31) ||
+       (long)M * sc * es >= (1l << 31))
         return fail(CKX_UNSUPPORTED, "operands of 2 GiB or more are not addressed");
     return CKX_OK;
 }
@@ -332,8 +304,14 @@ long gemm_workspace_bytes(int dt, int M, int N, int K, int instance)
 }
 
 // strided-batch part of the argument check (DeviceBatchedGemm)
-int check_batch(int dt, int M, int N, int K, int sa, int sb, int sc, int epi, int instance, int k_batch, int batch,
-                long bsa, long bsb, long bsc)
+// bytes from the first to one past the last element of an operand of `rows` rows of `cols` contiguous elements
+long operand_extent(int batch, long bs, int rows, int cols, int stride, int es)
+{
+    return rows > 0 && cols > 0 ? ((long)(batch - 1) * bs + (long)(rows - 1) * stride + cols) * es : 0;
+}
+
+int check_batch(int dt, int M, int N, int K, int sa, int sb, int sc, bool ta, bool tb, int epi, int instance,
+                int k_batch, int batch, long bsa, long bsb, long bsc)
 {
     if(batch < 0)
         return fail(CKX_INVALID_VALUE, "negative batch count");
@@ -348,8 +326,8 @@ int check_batch(int dt, int M, int N, int K, int sa, int sb, int sc, int epi, in
             return fail(CKX_UNSUPPORTED, "batch strides of A and B must be non-negative multiples of 16 bytes");
         if(bsc < (long)(M - 1) * sc + N && M > 0 && N > 0)
             return fail(CKX_UNSUPPORTED, "C batches overlap");
-        const long ea = ((long)(batch - 1) * bsa + (long)(M - 1) * sa + K) * es;
-        const long eb = ((long)(batch - 1) * bsb + (long)(N - 1) * sb + K) * es;
+        const long ea = operand_extent(batch, bsa, ta ? K : M, ta ? M : K, sa, es);
+        const long eb = operand_extent(batch, bsb, tb ? K : N, tb ? N : K, sb, es);
         if(ea >= (1l << 31) || eb >= (1l << 31) || ((long)(batch - 1) * bsc + (long)M * sc) * es >= (1l << 31))
             return fail(CKX_UNSUPPORTED, "operands of 2 GiB or more are not addressed");
     }
@@ -368,7 +346,8 @@ int run_gemm(int dt, const void* a, const void* b, void* c, int M, int N, int K,
         return fail(CKX_UNSUPPORTED, "KBatch must be 1..8");
     if(k_batch > 0 && instance >= kNumTiles)
         return fail(CKX_UNSUPPORTED, "the skinny instances split K over their waves, not over runs");
-    if((st = check_batch(dt, M, N, K, sa, sb, sc, epi, instance, k_batch, batch, bsa, bsb, bsc)) != CKX_OK)
+    const bool ta = al == CKX_COL_MAJOR, tb = bl == CKX_ROW_MAJOR, kmajor = ta || tb;
+    if((st = check_batch(dt, M, N, K, sa, sb, sc, ta, tb, epi, instance, k_batch, batch, bsa, bsb, bsc)) != CKX_OK)
         return st;
     if(batch == 0)
         return CKX_OK;
@@ -384,11 +363,13 @@ int run_gemm(int dt, const void* a, const void* b, void* c, int M, int N, int K,
     int ti = instance;
     Plan pl;
     // 33..64 rows: the tile kernel wins when its C tiles (or C tiles x K runs) fill the machine
-    const bool tile64 = M > 32 && M <= 64 &&
-                        ((N + 63) / 64 >= 160 ||
-                         (ws && !(reinterpret_cast<uintptr_t>(ws) & 15) && make_plan(M, N, K * es, -1, ws_bytes).ksplit > 1));
+    const bool tile64 = kmajor || (M > 32 && M <= 64 &&
+                                   ((N + 63) / 64 >= 160 ||
+                                    (ws && !(reinterpret_cast<uintptr_t>(ws) & 15) &&
+                                     make_plan(M, N, K * es, -1, ws_bytes).ksplit > 1)));
     if(instance == CKX_INSTANCE_AUTO && M <= 64 && !tile64 && k_batch == 0 && batch == 1)
     {
+        // (the skinny kernels read both operands K-contiguous: other layouts always take the tile kernel)
         // A handful of rows against a big weight matrix is an HBM-streaming problem. Wider
         // workgroups (32 / 64 columns) re-read A from L2 less often, as long as enough workgroups
         // remain to keep every CU pulling on HBM; up to 8 rows A is too small to matter.
@@ -403,8 +384,8 @@ int run_gemm(int dt, const void* a, const void* b, void* c, int M, int N, int K,
            (!ws || ws_bytes < (long)splitk_runs(K * es, k_batch) * M * N * 4))
             return fail(CKX_INVALID_VALUE, "KBatch > 1 needs a workspace of ckx_gemm_splitk_workspace_bytes()");
         // a batch multiplies the C tiles: plan for a problem with that many rows, without a K split
-        pl = batch > 1 ? make_plan(M * (batch < 64 ? batch : 64), N, K * es, instance, 0, 1)
-                       : make_plan(M, N, K * es, instance, ws ? ws_bytes : 0, k_batch);
+        pl = batch > 1 ? make_plan(M * (batch < 64 ? batch : 64), N, K * es, instance, 0, 1, kmajor)
+                       : make_plan(M, N, K * es, instance, ws ? ws_bytes : 0, k_batch, kmajor);
         ti = pl.tile;
     }
     ckx::GemmArgs g;
@@ -412,8 +393,8 @@ int run_gemm(int dt, const void* a, const void* b, void* c, int M, int N, int K,
     g.a = a, g.b = b, g.c = c;
     g.M = M, g.N = N, g.K = K;
     g.lda = sa, g.ldb = sb, g.ldc = sc;
-    g.a_bytes    = (uint32_t)(((long)(batch - 1) * bsa + (long)(M - 1) * sa + K) * es);
-    g.b_bytes    = (uint32_t)(((long)(batch - 1) * bsb + (long)(N - 1) * sb + K) * es);
+    g.a_bytes    = (uint32_t)operand_extent(batch, bsa, ta ? K : M, ta ? M : K, sa, es);
+    g.b_bytes    = (uint32_t)operand_extent(batch, bsb, tb ? K : N, tb ? N : K, sb, es);
     g.batch = batch, g.bsa = bsa, g.bsb = bsb, g.bsc = bsc;
     g.epi        = epi;
     g.scale_gemm = sg;
@@ -435,9 +416,15 @@ int run_gemm(int dt, const void* a, const void* b, void* c, int M, int N, int K,
     g.ksplit     = pl.ksplit;
     g.nk_per     = pl.nk_per;
     g.ws         = ws;
-    hipError_t e =
-        (dt == ckx::DT_I8 ? t.dense_i8 : dt == ckx::DT_BF16 ? t.dense_bf16 : t.dense_f16)(
-            g, g.tiles_m * g.tiles_n * g.ksplit * batch, (hipStream_t)stream);
+    const bool fused            = epi >= CKX_EPI_ADD_RELU && g.ksplit == 1; // (after a K split the second pass applies it)
+    const tile_launch_fn launch = kmajor               ? ckx::layout_tile(dt, ti, ta, tb)
+                                  : dt == ckx::DT_I8   ? t.dense_i8
+                                  : dt == ckx::DT_BF16 ? t.dense_bf16
+                                  : fused              ? t.dense_f16_fused
+                                                       : t.dense_f16;
+    if(!launch)
+        return fail(CKX_UNSUPPORTED, "no kernel variant for this layout");
+    hipError_t e = launch(g, g.tiles_m * g.tiles_n * g.ksplit * batch, (hipStream_t)stream);
     if(e == hipSuccess && g.ksplit > 1)
         e = dt == ckx::DT_I8     ? launch_reduce<ckx::DT_I8>(g, (hipStream_t)stream)
             : dt == ckx::DT_BF16 ? launch_reduce<ckx::DT_BF16>(g, (hipStream_t)stream)
@@ -595,7 +582,9 @@ int run_conv(int op, const void* in, const void* wei, void* out, const ckx_conv2
     g.ksplit = pl.ksplit;
     g.nk_per = pl.nk_per;
     g.ws     = ws;
-    hipError_t e = (es == 1 ? t.conv_i8 : t.conv_f16)(g, g.tiles_m * g.tiles_n * g.ksplit, (hipStream_t)stream);
+    const bool fused = epi >= CKX_EPI_ADD_RELU && g.ksplit == 1;
+    hipError_t e     = (es == 1 ? t.conv_i8 : fused ? t.conv_f16_fused : t.conv_f16)(g, g.tiles_m * g.tiles_n * g.ksplit,
+                                                                                 (hipStream_t)stream);
     if(e == hipSuccess && g.ksplit > 1)
         e = es == 1 ? launch_reduce<ckx::DT_I8>(g, (hipStream_t)stream)
                     : launch_reduce<ckx::DT_F16>(g, (hipStream_t)stream);
@@ -733,7 +722,8 @@ int ckx_batched_gemm_is_supported(int op, int32_t M, int32_t N, int32_t K, int32
         return fail(CKX_INVALID_VALUE, "not a GEMM operator family");
     const int dt = op == CKX_OP_GEMM_I8 ? ckx::DT_I8 : ckx::DT_F16;
     int st       = check_gemm_shape(dt, M, N, K, sa, sb, sc, al, bl, cl, epilogue, instance);
-    return st != CKX_OK ? st : check_batch(dt, M, N, K, sa, sb, sc, epilogue, instance, 0, batch, bsa, bsb, bsc);
+    return st != CKX_OK ? st : check_batch(dt, M, N, K, sa, sb, sc, al == CKX_COL_MAJOR, bl == CKX_ROW_MAJOR, epilogue, instance, 0, batch,
+                                         bsa, bsb, bsc);
 }
 
 int ckx_batched_gemm_i8(const void* a, const void* b, void* c, int32_t M, int32_t N, int32_t K, int32_t sa,

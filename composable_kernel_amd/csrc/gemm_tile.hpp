@@ -29,6 +29,7 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 #include <type_traits>
+#include <utility>
 
 namespace ckx {
 
@@ -57,9 +58,6 @@ enum
     EPI_CSHUFFLE_ADD_RELU = 5  // e = relu(half(half(acc) + d0)): C rounded to fp16 before the functor
 };
 
-#ifndef CKX_SWZ_SHIFT
-#define CKX_SWZ_SHIFT 0
-#endif
 // C tile stores: plain, or streaming (non-temporal) when the output is too large to be worth
 // keeping in L2: dirty lines of a streamed output otherwise queue up behind the write-back
 // and the store acknowledgements stall the K pipeline of the next tile.
@@ -168,6 +166,47 @@ __device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* p, uint3
 }
 
 typedef __attribute__((address_space(3))) void* lds_ptr_t;
+
+// compile-time loop: f(integral_constant<int, 0>) ... f(integral_constant<int, N - 1>)
+template <typename F, int... I>
+__device__ __forceinline__ void static_for_impl(F&& f, std::integer_sequence<int, I...>)
+{
+    (f(std::integral_constant<int, I>{}), ...);
+}
+template <int N, typename F>
+__device__ __forceinline__ void static_for(F&& f)
+{
+    static_for_impl(static_cast<F&&>(f), std::make_integer_sequence<int, N>{});
+}
+
+// LDS fragment reads as inline assembly. The compiler orders every LDS read it knows about after ALL
+// outstanding direct global->LDS loads (s_waitcnt vmcnt(0): it cannot tell which stage they fill),
+// which would hold the first reads of a K tile until the prefetch of the tile after next has landed.
+// Reads it does not know about are not counted in lgkmcnt either: the kernel waits for them itself
+// (s_waitcnt lgkmcnt(0) followed by a scheduling barrier) before the first instruction that uses them.
+// (No "memory" clobber: that alone makes the statement a possible LDS access and brings the wait back.
+// volatile keeps the statements in program order among themselves and with the loads and stores.)
+template <int IMM>
+__device__ __forceinline__ i32x4 lds_read_b128(uint32_t addr)
+{
+    static_assert(IMM >= 0 && IMM < 65536, "16-bit offset field");
+    i32x4 v;
+    asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(v) : "v"(addr), "n"(IMM));
+    return v;
+}
+// transposing reads (gfx950): 16 lanes x 8 bytes = a 4 x 16 block of 16-bit (8 x 16 of 8-bit) elements,
+// each lane ends up with one column of it
+template <int ES, int IMM>
+__device__ __forceinline__ i32x2 lds_read_tr_b64(uint32_t addr)
+{
+    static_assert(IMM >= 0 && IMM < 65536, "16-bit offset field");
+    i32x2 v;
+    if constexpr(ES == 2)
+        asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2" : "=v"(v) : "v"(addr), "n"(IMM));
+    else
+        asm volatile("ds_read_b64_tr_b8 %0, %1 offset:%2" : "=v"(v) : "v"(addr), "n"(IMM));
+    return v;
+}
 
 // ---------------------------------------------------------------- epilogues
 // All in fp32 on the exactly converted int32 accumulator; the two multiplies are separate
@@ -338,7 +377,22 @@ __device__ __forceinline__ void store_row16_f16_fused(_Float16* crow, int n0, in
 // The kernel is PERSISTENT: workgroup b works on tiles b, b + gridDim.x, ... and the K-tile
 // pipeline runs straight across tile boundaries, so the first loads of the next tile are in
 // flight under the last MFMAs, the epilogue arithmetic and the C stores of the current one.
-template <int DT, int BM, int BN, int WM, int WN, int BKB, int NST, bool IM2COL>
+//
+// TA / TB: the operand is stored K-MAJOR (A column-major "km": element (m,k) at k*lda + m; B row-major
+// "kn": element (k,n) at k*ldb + n). Its staged tile is then [k row][m or n], 16-byte chunks of 8 fp16 /
+// 16 int8 consecutive m (n), and the MFMA fragments come out of LDS through the transposing reads
+// ds_read_b64_tr_b16 / _b8: within 16 lanes, lane 4e+j (b16; 2e+j for b8) points at 4 (8) consecutive
+// elements of k row e, and lane i receives element i of every one of the 4 (8) rows -- four (eight)
+// consecutive k of ONE m, i.e. half an MFMA operand. A K-major B tile keeps its columns in natural
+// order (the transposing read has no room for the column permutation of the K-contiguous path), and
+// the epilogue moves accumulators between the four 16-lane rows instead (transpose_acc).
+//
+// FUSED (fp16): the variant with the add / ReLU epilogues and their D operands. A kernel of its own: the
+// D loads of that epilogue leave the compiler with "some global load may be outstanding" at the top of
+// the K loop, which it answers with s_waitcnt vmcnt(0) in every iteration -- also for launches that
+// never run that epilogue -- and that wait holds the loop until the prefetched K tile has landed.
+template <int DT, int BM, int BN, int WM, int WN, int BKB, int NST, bool IM2COL, bool TA = false, bool TB = false,
+          bool FUSED = false>
 struct GemmTile
 {
     static constexpr int NW      = WM * WN;
@@ -363,15 +417,39 @@ struct GemmTile
     static_assert(WTM % 16 == 0 && WTN % 64 == 0, "wave tile must be 16k x 64k");
     static_assert((BM * CPR) % NT == 0 && (BN * CPR) % NT == 0, "tile rows must split over the waves");
 
+    static_assert(!(IM2COL && (TA || TB)), "the im2col view is K-contiguous");
+    static_assert(!FUSED || (DT == DT_F16 && !TA && !TB), "D-operand epilogues: fp16, K-contiguous operands");
+    static_assert((!TA || (BM >= 64 && BM * ES <= 1024)) && (!TB || (BN >= 64 && BN * ES <= 1024)),
+                  "a K-major tile row is 64..1024 bytes");
+    static constexpr int KE = BKB / ES; // k rows of a K tile
+
     using acc_t = typename std::conditional<DT == DT_I8, i32x4, f32x4>::type;
 
-    // XOR swizzle of the chunk position: the 16 rows read by one MFMA fragment load spread
-    // over all LDS banks (measured: 0 bank conflicts, 256 B/clk).
-    __device__ static __forceinline__ uint32_t swz(uint32_t row) { return (row >> CKX_SWZ_SHIFT) & 7u; }
-    __device__ static __forceinline__ uint32_t chunk_offset(uint32_t row, uint32_t chunk)
+    // K-major tiles: k row r of a tile of BX columns sits at r * BX * ES, and its 16-element segments
+    // are XOR-ed with bits of r so that the rows touched by one transposing read (fp16: r = 8q + e,
+    // e < 4; int8: r = 16q + e, e < 8; the 32 lanes q = 0,1 or q = 2,3 share a pass) fall on distinct banks.
+    template <int BX>
+    __device__ static __forceinline__ uint32_t tswz(uint32_t r)
     {
-        return row * BKB + ((chunk ^ swz(row)) << 4);
+        constexpr int P  = BX * ES;
+        constexpr int LB = P >= 256 ? 0 : (P == 128 ? 1 : 2); // row bits the pitch already spreads
+        const uint32_t full = ES == 2 ? ((r & 3u) | (((r >> 3) & 1u) << 2)) : ((r & 7u) | (((r >> 4) & 1u) << 3));
+        return full >> LB;
     }
+    // slot j of a thread in a K-major tile: k row and first column of its 16-byte chunk
+    template <int BX>
+    __device__ static __forceinline__ void tslot(int j, int wave, int lane, uint32_t& r, uint32_t& x)
+    {
+        constexpr int CPRT = BX * ES / 16, RPW = 64 / CPRT;
+        r                  = (uint32_t)((j * NW + wave) * RPW + lane / CPRT);
+        const uint32_t pc  = (uint32_t)(lane % CPRT);
+        const uint32_t seg = (pc / ES) ^ tswz<BX>(r);
+        x                  = seg * 16 + (pc % ES) * (16 / ES);
+    }
+
+    // K-contiguous tiles: the 16-byte chunk at position c of staged row r holds chunk c ^ (r & 7) of that
+    // row, so the 16 rows read by one MFMA fragment load spread over all LDS banks (measured: no bank
+    // conflicts, 256 B/clk).
 
     __device__ static __forceinline__ void run(const GemmArgs& p, uint8_t* smem)
     {
@@ -396,11 +474,14 @@ struct GemmTile
         // slot j of this thread fills LDS row (j*NW + wave)*RPI + lane/CPR, chunk position lane%CPR
         // Every slot of a thread sits at the same chunk position: the slot rows differ by
         // multiples of 8 and the swizzle is row & 7, i.e. lane/8 for all of them.
-        static_assert(CKX_SWZ_SHIFT == 0 && RPI == 8, "one chunk position per thread");
+        static_assert(RPI == 8, "one chunk position per thread");
         uint32_t a_off[NLA];  // dense: byte offset of (row, chunk) at K tile 0, or kOutOfRange
         uint32_t a_hw0[NLA]; // im2col: top-left input coordinate of the row's window, (hi0 << 16) | (wi0 & 0xffff)
         uint32_t b_off[NLB];
         const uint32_t kb = ((uint32_t)(lane % CPR) ^ (uint32_t)((lane / CPR) & 7)) << 4; // chunk byte offset in a K tile
+        // K-major operands: k row (within a K tile) of this thread's slot 0; slot j is j * NW * rows-per-load further
+        const uint32_t trow_a = TA ? (uint32_t)(wave * (1024 / (BM * ES)) + lane / (BM * ES / 16)) : 0u;
+        const uint32_t trow_b = TB ? (uint32_t)(wave * (1024 / (BN * ES)) + lane / (BN * ES / 16)) : 0u;
 
         // row / column offsets of the tile the LOAD cursor is on (tile >= ntiles: nothing valid)
         auto setup_tile = [&](int tile_id) {
@@ -413,6 +494,15 @@ struct GemmTile
 #pragma unroll
             for(int j = 0; j < NLA; ++j)
             {
+                if constexpr(TA)
+                {
+                    uint32_t r, x;
+                    tslot<BM>(j, wave, lane, r, x);
+                    const uint32_t gx = (uint32_t)tm * BM + x;
+                    a_off[j] = (live && gx < (uint32_t)p.M) ? a_batch + (r * (uint32_t)p.lda + gx) * ES : kOutOfRange;
+                    a_hw0[j] = 0;
+                    continue;
+                }
                 const uint32_t r  = (uint32_t)((j * NW + wave) * RPI + lane / CPR);
                 const uint32_t gm = (uint32_t)tm * BM + r;
                 const bool ok     = live && gm < (uint32_t)p.M;
@@ -447,6 +537,14 @@ struct GemmTile
 #pragma unroll
             for(int j = 0; j < NLB; ++j)
             {
+                if constexpr(TB)
+                {
+                    uint32_t r, x;
+                    tslot<BN>(j, wave, lane, r, x);
+                    const uint32_t gx = (uint32_t)tn * BN + x;
+                    b_off[j] = (live && gx < (uint32_t)p.N) ? b_batch + (r * (uint32_t)p.ldb + gx) * ES : kOutOfRange;
+                    continue;
+                }
                 const uint32_t r  = (uint32_t)((j * NW + wave) * RPI + lane / CPR);
                 const uint32_t gn = (uint32_t)tn * BN + b_row_to_col(r);
                 b_off[j] = (live && gn < (uint32_t)p.N) ? b_batch + gn * (uint32_t)p.ldb * ES + kb : kOutOfRange;
@@ -462,6 +560,8 @@ struct GemmTile
             uint8_t* sa;
             uint8_t* sb;
             uint32_t k0;      // byte offset of the K tile
+            uint32_t k0a, k0b; // K-major operands: byte offset of the K tile's first k row
+            int klim;          // K-major operands: k rows of this K tile that exist
             uint32_t k_oob;   // top bit set for chunks past K: OR-ed into the offset (arithmetic on
                               // purpose: a select feeding the loads becomes divergent branches)
             int tap_dh, tap_dw; // im2col: decoded ONCE per thread and K tile, every slot of a thread
@@ -474,6 +574,9 @@ struct GemmTile
             c.sb    = c.sa + A_TILE;
             c.k0    = (uint32_t)kt * BKB;
             c.k_oob = (c.k0 + kb < kbytes) ? 0u : kOutOfRange;
+            c.k0a   = TA ? (uint32_t)kt * KE * (uint32_t)p.lda * ES : 0u;
+            c.k0b   = TB ? (uint32_t)kt * KE * (uint32_t)p.ldb * ES : 0u;
+            c.klim  = p.K - kt * KE;
             c.tap_dh = c.tap_dw = 0;
             c.tap_off           = 0;
             c.tap_ok            = true;
@@ -496,7 +599,9 @@ struct GemmTile
             {
                 const int j = slot;
                 uint32_t voff;
-                if constexpr(!IM2COL)
+                if constexpr(TA)
+                    voff = (a_off[j] + c.k0a) | (~(uint32_t)((int)(trow_a + j * NW * (1024 / (BM * ES))) - c.klim) & kOutOfRange);
+                else if constexpr(!IM2COL)
                     voff = (a_off[j] + c.k0) | c.k_oob;
                 else
                 {
@@ -511,7 +616,9 @@ struct GemmTile
             else
             {
                 const int j         = slot - NLA;
-                const uint32_t voff = (b_off[j] + c.k0) | c.k_oob;
+                const uint32_t voff =
+                    TB ? (b_off[j] + c.k0b) | (~(uint32_t)((int)(trow_b + j * NW * (1024 / (BN * ES))) - c.klim) & kOutOfRange)
+                       : (b_off[j] + c.k0) | c.k_oob;
                 __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_b, (lds_ptr_t)(c.sb + (j * NW + wave) * 1024), 16,
                                                          voff, 0, 0, 0);
             }
@@ -560,22 +667,68 @@ struct GemmTile
         // Fragment r of a k-step, in the order in which the MFMAs of that k-step need them: the B
         // fragments and the first A fragment feed the first MFMA group, the last A fragment only
         // the last one, so the LDS latency of the late reads hides under the early groups.
-        auto read_one = [&](const uint8_t* sa, const uint8_t* sb, int ks, int r, i32x4(&af)[MT], i32x4(&bf)[NG * 4]) {
-            if(r < NG * 4)
+        // Per-lane parts of the fragment addresses (LDS byte addresses relative to a stage), fixed for the
+        // whole kernel; the fragment index and the k-step only add an immediate offset (and, in a K-major
+        // tile, flip segment bits: the swizzle is an XOR).
+        //   K-contiguous tile: row = wave rows + 16 * fragment + lane % 16, chunk = 4 * ks + lane / 16
+        //   K-major tile:      k row = 32 * ks + 8 * (lane / 16) + 4 * h + (lane % 16) / 4   (fp16; h = 0,1)
+        //                              64 * ks + 16 * (lane / 16) + 8 * h + (lane % 16) / 2  (int8)
+        constexpr int SEGSH = ES == 2 ? 5 : 4;                       // log2 bytes of a 16-element segment
+        constexpr int TKS = ES == 2 ? 32 : 64, THALF = ES == 2 ? 4 : 8; // k rows per k-step / per transposing read
+        const uint32_t smem_lds = (uint32_t)(uintptr_t)(lds_ptr_t)smem;
+        auto kcontig_part = [&](int wave_row0, int ks) {
+            return (uint32_t)(wave_row0 + (int)frow) * BKB + ((((uint32_t)ks * 4 + fq) ^ (frow & 7u)) << 4);
+        };
+        auto kmajor_part = [&](auto bx, int wave_col0) {
+            constexpr int BX = decltype(bx)::value, P = BX * ES;
+            const uint32_t e = ES == 2 ? frow >> 2 : frow >> 1, j = ES == 2 ? (frow & 3u) : (frow & 1u);
+            const uint32_t r = (ES == 2 ? 8u : 16u) * fq + e;
+            return r * P + ((((uint32_t)wave_col0 >> 4) ^ tswz<BX>(r)) << SEGSH) + (j << 3);
+        };
+        const uint32_t fa0 = TA ? kmajor_part(std::integral_constant<int, BM>{}, wm * WTM) : kcontig_part(wm * WTM, 0);
+        const uint32_t fa1 = TA ? fa0 : kcontig_part(wm * WTM, 1);
+        const uint32_t fb0 = TB ? kmajor_part(std::integral_constant<int, BN>{}, wn * WTN) : kcontig_part(wn * WTN, 0);
+        const uint32_t fb1 = TB ? fb0 : kcontig_part(wn * WTN, 1);
+        static_assert((MT & (MT - 1)) == 0 && ((NG * 4) & (NG * 4 - 1)) == 0, "fragment index is XOR-ed into the address");
+
+        // Fragment R of k-step KS, in the order in which the MFMAs of that k-step need them: the B
+        // fragments and the first A fragment feed the first MFMA group, the last A fragment only
+        // the last one, so the LDS latency of the late reads hides under the early groups.
+        // stage_lds: LDS address of the stage.
+        auto read_one = [&](uint32_t stage_lds, auto ks_c, auto r_c, i32x4(&af)[MT], i32x4(&bf)[NG * 4]) {
+            constexpr int KS = decltype(ks_c)::value, R = decltype(r_c)::value;
+            if constexpr(R < NG * 4)
             {
-                const uint32_t row = (uint32_t)(wn * WTN + 16 * r) + frow;
-                bf[r] = *reinterpret_cast<const i32x4*>(sb + chunk_offset(row, ks * 4 + fq));
+                const uint32_t base = stage_lds + (KS ? fb1 : fb0);
+                if constexpr(TB)
+                {
+                    const uint32_t a = base ^ ((uint32_t)R << SEGSH);
+                    const i32x2 lo   = lds_read_tr_b64<ES, A_TILE + KS * TKS * BN * ES>(a);
+                    const i32x2 hi   = lds_read_tr_b64<ES, A_TILE + (KS * TKS + THALF) * BN * ES>(a);
+                    bf[R]            = i32x4{lo[0], lo[1], hi[0], hi[1]};
+                }
+                else
+                    bf[R] = lds_read_b128<A_TILE + R * 16 * BKB>(base);
             }
             else
             {
-                const uint32_t row = (uint32_t)(wm * WTM + 16 * (r - NG * 4)) + frow;
-                af[r - NG * 4] = *reinterpret_cast<const i32x4*>(sa + chunk_offset(row, ks * 4 + fq));
+                constexpr int I     = R - NG * 4;
+                const uint32_t base = stage_lds + (KS ? fa1 : fa0);
+                if constexpr(TA)
+                {
+                    const uint32_t a = base ^ ((uint32_t)I << SEGSH);
+                    const i32x2 lo   = lds_read_tr_b64<ES, KS * TKS * BM * ES>(a);
+                    const i32x2 hi   = lds_read_tr_b64<ES, (KS * TKS + THALF) * BM * ES>(a);
+                    af[I]            = i32x4{lo[0], lo[1], hi[0], hi[1]};
+                }
+                else
+                    af[I] = lds_read_b128<I * 16 * BKB>(base);
             }
         };
-        auto read_frags = [&](const uint8_t* sa, const uint8_t* sb, int ks, i32x4(&af)[MT], i32x4(&bf)[NG * 4]) {
-#pragma unroll
-            for(int r = 0; r < MT + NG * 4; ++r)
-                read_one(sa, sb, ks, r, af, bf);
+        // the kernel's own wait for its fragment reads; nothing may be scheduled across it
+        auto wait_frags = [&]() {
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+            __builtin_amdgcn_sched_barrier(0);
         };
         auto mfma_one = [&](int m, const i32x4(&af)[MT], const i32x4(&bf)[NG * 4]) {
             const int i = m / (NG * 4), t = m % (NG * 4);
@@ -596,29 +749,27 @@ struct GemmTile
         // fills the texture-address FIFOs (SQ_VMEM_TA_ADDR/CMD_FIFO_FULL), the in-order wave blocks
         // on VMEM issue, and its MFMAs wait behind it.
         auto half_step = [&](auto with_loads, const LoadCtx& lc, const i32x4(&caf)[MT], const i32x4(&cbf)[NG * 4],
-                             const uint8_t* nsa, const uint8_t* nsb, int nks, i32x4(&naf)[MT], i32x4(&nbf)[NG * 4]) {
-            // The reads are over two groups before the end of the half, so the next half starts with
-            // every fragment it needs at once already in registers. The first half of an iteration
-            // (top of the loop, where the compiler waits for ALL outstanding LDS reads) starts its
-            // reads one group late: that wait then only covers reads issued long before.
+                             uint32_t nstage_lds, auto nks, i32x4(&naf)[MT], i32x4(&nbf)[NG * 4]) {
+            // The reads are over two groups before the end of the half; the first half of an iteration
+            // starts its reads one group late.
             constexpr int NGRP = LPT, NR = MT + NG * 4, NM = MT * NG * 4;
             constexpr int RG  = NGRP >= 4 ? NGRP - 2 : NGRP;
             constexpr int RG0 = (NGRP >= 4 && !decltype(with_loads)::value) ? 1 : 0;
-#pragma unroll
-            for(int g = 0; g < NGRP; ++g)
-            {
+            static_for<NGRP>([&](auto g_c) {
+                constexpr int g = decltype(g_c)::value;
                 if constexpr(decltype(with_loads)::value)
                     issue_slot(lc, g);
-                const int gr = g - RG0 < 0 ? 0 : (g - RG0 > RG ? RG : g - RG0); // read groups done before g
-                const int gn = g + 1 - RG0 < 0 ? 0 : (g + 1 - RG0 > RG ? RG : g + 1 - RG0);
-#pragma unroll
-                for(int r = gr * NR / RG; r < gn * NR / RG; ++r)
-                    read_one(nsa, nsb, nks, r, naf, nbf);
+                constexpr int gr = g - RG0 < 0 ? 0 : (g - RG0 > RG ? RG : g - RG0); // read groups done before g
+                constexpr int gn = g + 1 - RG0 < 0 ? 0 : (g + 1 - RG0 > RG ? RG : g + 1 - RG0);
+                constexpr int r0 = gr * NR / RG, r1 = gn * NR / RG;
+                static_for<r1 - r0>([&](auto r_c) {
+                    read_one(nstage_lds, nks, std::integral_constant<int, r0 + decltype(r_c)::value>{}, naf, nbf);
+                });
 #pragma unroll
                 for(int m = g * NM / NGRP; m < (g + 1) * NM / NGRP; ++m)
                     mfma_one(m, caf, cbf);
                 __builtin_amdgcn_sched_barrier(0);
-            }
+            });
         };
 
         // ---- epilogue: registers -> global, 16 consecutive columns per lane -------------
@@ -791,6 +942,40 @@ struct GemmTile
             }
         };
 
+        // K-major B: MFMA tile t of a 64-column group covered columns 16t..16t+15, so the lane in 16-lane
+        // row q holds columns 16t + 4q + (0..3). A 4x4 transpose between t and q (two butterfly stages of
+        // v_permlane32_swap / v_permlane16_swap) gives lane row q the columns 16q + 4t + (0..3) -- the
+        // ownership the epilogues are written for.
+        auto transpose_acc = [&]() {
+#pragma unroll
+            for(int i = 0; i < MT; ++i)
+#pragma unroll
+                for(int g = 0; g < NG; ++g)
+#pragma unroll
+                    for(int e = 0; e < 4; ++e)
+                    {
+                        uint32_t x[4];
+#pragma unroll
+                        for(int t = 0; t < 4; ++t)
+                        {
+                            // (through a scalar temporary: a bit cast applied directly to a vector-element
+                            // lvalue reads element 0)
+                            const auto v = acc[i][g * 4 + t][e];
+                            x[t]         = __builtin_bit_cast(uint32_t, v);
+                        }
+                        // rows 2,3 of x[t] <-> rows 0,1 of x[t + 2]
+                        auto s02 = __builtin_amdgcn_permlane32_swap(x[0], x[2], false, false);
+                        auto s13 = __builtin_amdgcn_permlane32_swap(x[1], x[3], false, false);
+                        // odd rows of the first <-> even rows of the second
+                        auto u01 = __builtin_amdgcn_permlane16_swap(s02[0], s13[0], false, false);
+                        auto u23 = __builtin_amdgcn_permlane16_swap(s02[1], s13[1], false, false);
+                        x[0] = u01[0], x[1] = u01[1], x[2] = u23[0], x[3] = u23[1];
+#pragma unroll
+                        for(int t = 0; t < 4; ++t)
+                            acc[i][g * 4 + t][e] = __builtin_bit_cast(decltype(acc[0][0][0] + 0), x[t]);
+                    }
+        };
+
         auto barrier = [&]() {
             __builtin_amdgcn_s_barrier();
             asm volatile("" ::: "memory");
@@ -810,7 +995,7 @@ struct GemmTile
         }
         asm volatile("s_waitcnt vmcnt(%0)" ::"n"((NST - 1) * LPT) : "memory");
         barrier();
-        read_frags(smem, smem + A_TILE, 0, af0, bf0);
+        static_for<MT + NG * 4>([&](auto r_c) { read_one(smem_lds, std::integral_constant<int, 0>{}, r_c, af0, bf0); });
 
         int kt = 0, kt_end = nk;
         int st_cur = 0;       // stage of the K tile being multiplied
@@ -819,12 +1004,10 @@ struct GemmTile
         for(int unit = (int)blockIdx.x; unit < nunits;)
         {
             const int st_next  = st_cur + 1 == NST ? 0 : st_cur + 1;
-            const uint8_t* sa  = smem + st_cur * STAGE;
-            const uint8_t* sb  = sa + A_TILE;
-            const uint8_t* san = smem + st_next * STAGE;
-            const uint8_t* sbn = san + A_TILE;
-
-            half_step(std::false_type{}, LoadCtx{}, af0, bf0, sa, sb, 1, af1, bf1);
+            // first fragments of this K tile (read in the previous half-iteration / the prologue)
+            wait_frags();
+            half_step(std::false_type{}, LoadCtx{}, af0, bf0, smem_lds + (uint32_t)(st_cur * STAGE),
+                      std::integral_constant<int, 1>{}, af1, bf1);
 
             // The direct loads of a wave retire in order: once at most NST-2 K tiles' worth are in
             // flight, the next K tile has landed. C stores of an epilogue share the counter and are
@@ -834,17 +1017,21 @@ struct GemmTile
                 asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
             else
                 asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" ::"n"((NST - 2) * LPT) : "memory");
+            __builtin_amdgcn_sched_barrier(0);
             drain = false;
             barrier();
 
             const LoadCtx lc = load_ctx(ld_kt, st_cur);
-            half_step(std::true_type{}, lc, af1, bf1, san, sbn, 0, af0, bf0);
+            half_step(std::true_type{}, lc, af1, bf1, smem_lds + (uint32_t)(st_next * STAGE),
+                      std::integral_constant<int, 0>{}, af0, bf0);
             advance_load_cursor();
 
             st_cur = st_next;
             if(++kt >= kt_end)
             {
-                if constexpr(DT == DT_F16)
+                if constexpr(TB)
+                    transpose_acc();
+                if constexpr(FUSED)
                 {
                     if(p.epi == EPI_PASSTHROUGH || p.ksplit > 1)
                         epilogue(unit);
@@ -945,11 +1132,12 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(const GemmArgs p)
     }
 }
 
-template <int DT, int BM, int BN, int WM, int WN, int BKB, int NST, bool IM2COL>
+template <int DT, int BM, int BN, int WM, int WN, int BKB, int NST, bool IM2COL, bool TA = false, bool TB = false,
+          bool FUSED = false>
 __global__ __launch_bounds__(WM* WN * 64) void gemm_tile_kernel(const GemmArgs p)
 {
     extern __shared__ __attribute__((aligned(1024))) uint8_t ckx_smem[];
-    GemmTile<DT, BM, BN, WM, WN, BKB, NST, IM2COL>::run(p, ckx_smem);
+    GemmTile<DT, BM, BN, WM, WN, BKB, NST, IM2COL, TA, TB, FUSED>::run(p, ckx_smem);
 }
 
 } // namespace ckx

@@ -129,8 +129,8 @@ def test_int8_gemm_unsupported_arguments_are_refused():
     assert not op.IsSupportedArgument(arg)
     with pytest.raises(RuntimeError):
         op.MakeInvokerPointer().Run(arg)
-    # row-major B is not built
-    op2 = ck.DeviceGemmInt8(ALayout=ck.RowMajor, BLayout=ck.RowMajor)
+    # column-major C is not built (nor is it in the reference's instance lists)
+    op2 = ck.DeviceGemmInt8(CLayout=ck.ColumnMajor)
     assert not op2.IsSupportedArgument(op2.MakeArgumentPointer(d, d, d, 64, 64, 64, 64, 64, 64))
     # empty problem is a no-op
     arg = op.MakeArgumentPointer(d, d, d, 0, 64, 64, 64, 64, 64)
