@@ -495,11 +495,17 @@ struct DeviceGemmMfma : public DeviceGemm<ALayout, BLayout, CLayout, ADataType, 
     std::string GetTypeString() const override
     {
         const int op = is_i8 ? CKX_OP_GEMM_I8 : is_bf16 ? CKX_OP_GEMM_BF16 : CKX_OP_GEMM_F16;
-        if(instance_ == CKX_INSTANCE_AUTO)
-            return is_i8     ? "DeviceGemm_i8_i8_i8_mk_nk_mn<auto>"
-                   : is_bf16 ? "DeviceGemm_bf16_bf16_bf16_mk_nk_mn<auto>"
-                             : "DeviceGemm_f16_f16_f16_mk_nk_mn<auto>";
-        return ckx_instance_name(op, instance_);
+        std::string name = instance_ == CKX_INSTANCE_AUTO ? is_i8     ? "DeviceGemm_i8_i8_i8_mk_nk_mn<auto>"
+                                                            : is_bf16 ? "DeviceGemm_bf16_bf16_bf16_mk_nk_mn<auto>"
+                                                                      : "DeviceGemm_f16_f16_f16_mk_nk_mn<auto>"
+                                                          : ckx_instance_name(op, instance_);
+        // the library lists one set of instances for all A / B layouts: put this operator's layouts in the name
+        const std::string tag = std::string(std::is_same_v<ALayout, tensor_layout::gemm::RowMajor> ? "mk_" : "km_") +
+                                (std::is_same_v<BLayout, tensor_layout::gemm::RowMajor> ? "kn" : "nk");
+        const auto pos = name.find("mk_nk");
+        if(pos != std::string::npos)
+            name.replace(pos, 5, tag);
+        return name;
     }
     int instance_;
 };

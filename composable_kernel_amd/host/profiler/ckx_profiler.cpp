@@ -2,7 +2,7 @@
 // this library. Positional arguments follow the reference's conventions
 // (profiler/src/profile_gemm.cpp:27-75, profile_convnd_fwd.cpp:81-115):
 //
-//   ckx_profiler gemm <dtype 1:fp16 2:bf16 3:int8> <layout 1: A[m,k]*B[n,k]> <verify> <init> <log> <time>
+//   ckx_profiler gemm <dtype 1:fp16 2:bf16 3:int8> <layout 0:mk_kn 1:mk_nk 2:km_kn 3:km_nk> <verify> <init> <log> <time>
 //                     M N K StrideA StrideB StrideC [epilogue 0|1|2] [scale_gemm] [scale_relu] [nrepeat]
 //   ckx_profiler conv2d_fwd <dtype 1|3> <verify> <init> <log> <time>
 //                     N K C Y X Hi Wi Sy Sx Dy Dx LeftPy LeftPx RightPy RightPx [epilogue sg sr] [nrepeat]
@@ -165,20 +165,33 @@ int run_family(std::vector<std::unique_ptr<Op>>& ops, MakeArg make_arg, ckx::Dev
     return pass ? 0 : 1;
 }
 
-template <typename T, typename COp>
-int profile_gemm_t(bool verify, int init, bool time_kernel, int M, int N, int K, int sa, int sb, int sc, COp cop,
+// layout codes of the reference's profiler (profiler/src/profile_gemm.cpp:13-19)
+enum GemmMatrixLayout
+{
+    MK_KN_MN = 0,
+    MK_NK_MN = 1,
+    KM_KN_MN = 2,
+    KM_NK_MN = 3
+};
+
+template <typename T, typename COp, typename AL, typename BL>
+int profile_gemm_l(bool verify, int init, bool time_kernel, int M, int N, int K, int sa, int sb, int sc, COp cop,
                    int nrepeat)
 {
-    using DeviceOp = device::DeviceGemm<Row, Col, Row, T, T, T, Pass, Pass, COp>;
+    using DeviceOp = device::DeviceGemm<AL, BL, Row, T, T, T, Pass, Pass, COp>;
     auto ops       = device::instance::DeviceOperationInstanceFactory<DeviceOp>::GetInstances();
-    std::vector<T> a((std::size_t)M * sa), b((std::size_t)N * sb);
+    constexpr bool a_row = std::is_same_v<AL, Row>, b_row = std::is_same_v<BL, Row>;
+    sa = sa < 0 ? (a_row ? K : M) : sa, sb = sb < 0 ? (b_row ? N : K) : sb, sc = sc < 0 ? N : sc;
+    std::vector<T> a((std::size_t)(a_row ? M : K) * sa), b((std::size_t)(b_row ? K : N) * sb);
     fill(a, init, 0xC0FFEE, false);
     fill(b, init, 0xC0FFEE + 1, false);
     ckx::DeviceMem da(a.size() * sizeof(T)), db(b.size() * sizeof(T)), dc((std::size_t)M * sc * sizeof(T));
     da.ToDevice(a.data());
     db.ToDevice(b.data());
-    std::cout << "a_m_k: dim 2, lengths {" << M << ", " << K << "}, strides {" << sa << ", 1}\n"
-              << "b_k_n: dim 2, lengths {" << K << ", " << N << "}, strides {1, " << sb << "}\n"
+    std::cout << "a_m_k: dim 2, lengths {" << M << ", " << K << "}, strides {" << (a_row ? sa : 1) << ", "
+              << (a_row ? 1 : sa) << "}\n"
+              << "b_k_n: dim 2, lengths {" << K << ", " << N << "}, strides {" << (b_row ? sb : 1) << ", "
+              << (b_row ? 1 : sb) << "}\n"
               << "c_m_n: dim 2, lengths {" << M << ", " << N << "}, strides {" << sc << ", 1}" << std::endl;
     const double flop = 2.0 * M * N * K, bytes = sizeof(T) * ((double)M * K + (double)K * N + (double)M * N);
     return run_family<T>(
@@ -190,15 +203,34 @@ int profile_gemm_t(bool verify, int init, bool time_kernel, int M, int N, int K,
         dc, (std::size_t)M * sc, flop, bytes, verify, time_kernel, nrepeat);
 }
 
+template <typename T, typename COp>
+int profile_gemm_t(int layout, bool verify, int init, bool time_kernel, int M, int N, int K, int sa, int sb, int sc,
+                   COp cop, int nrepeat)
+{
+    switch(layout)
+    {
+    case MK_KN_MN: return profile_gemm_l<T, COp, Row, Row>(verify, init, time_kernel, M, N, K, sa, sb, sc, cop, nrepeat);
+    case MK_NK_MN: return profile_gemm_l<T, COp, Row, Col>(verify, init, time_kernel, M, N, K, sa, sb, sc, cop, nrepeat);
+    case KM_KN_MN: return profile_gemm_l<T, COp, Col, Row>(verify, init, time_kernel, M, N, K, sa, sb, sc, cop, nrepeat);
+    case KM_NK_MN: return profile_gemm_l<T, COp, Col, Col>(verify, init, time_kernel, M, N, K, sa, sb, sc, cop, nrepeat);
+    }
+    std::cout << "this data_type & layout is not implemented" << std::endl;
+    return 1;
+}
+
 int profile_gemm(int argc, char* argv[])
 {
     if(argc < 14)
     {
         std::printf("arg1: tensor operation (gemm)\narg2: data type (1: fp16; 2: bf16; 3: int8)\n"
-                    "arg3: matrix layout (1: A[m, k] * B[n, k] = C[m, n])\narg4: verification (0: no; 1: yes)\n"
+                    "arg3: matrix layout (0: A[m, k] * B[k, n] = C[m, n];\n"
+                    "                     1: A[m, k] * B[n, k] = C[m, n];\n"
+                    "                     2: A[k, m] * B[k, n] = C[m, n];\n"
+                    "                     3: A[k, m] * B[n, k] = C[m, n])\n"
+                    "arg4: verification (0: no; 1: yes)\n"
                     "arg5: initialization (0: no init; 1: integer value; 2: decimal value)\n"
                     "arg6: print tensor value (0: no; 1: yes)\narg7: time kernel (0=no, 1=yes)\n"
-                    "arg8 to 13: M, N, K, StrideA, StrideB, StrideC\n"
+                    "arg8 to 13: M, N, K, StrideA, StrideB, StrideC (negative: packed)\n"
                     "arg14-16 (int8): epilogue (0 PassThrough, 1 RequantReluRequant, 2 rounded), scale_gemm, scale_relu\n"
                     "last: nrepeat\n");
         return 1;
@@ -208,17 +240,11 @@ int profile_gemm(int argc, char* argv[])
     const int init = std::atoi(argv[5]);
     const int M = std::atoi(argv[8]), N = std::atoi(argv[9]), K = std::atoi(argv[10]);
     int sa = std::atoi(argv[11]), sb = std::atoi(argv[12]), sc = std::atoi(argv[13]);
-    sa = sa < 0 ? K : sa, sb = sb < 0 ? K : sb, sc = sc < 0 ? N : sc;
-    if(layout != 1)
-    {
-        std::cout << "this data_type & layout is not implemented" << std::endl;
-        return 1;
-    }
     if(dtype == 1)
-        return profile_gemm_t<half_t>(verify, init, time_kernel, M, N, K, sa, sb, sc, Pass{},
+        return profile_gemm_t<half_t>(layout, verify, init, time_kernel, M, N, K, sa, sb, sc, Pass{},
                                       argc > 14 ? std::atoi(argv[14]) : 10);
     if(dtype == 2)
-        return profile_gemm_t<bhalf_t>(verify, init, time_kernel, M, N, K, sa, sb, sc, Pass{},
+        return profile_gemm_t<bhalf_t>(layout, verify, init, time_kernel, M, N, K, sa, sb, sc, Pass{},
                                        argc > 14 ? std::atoi(argv[14]) : 10);
     if(dtype == 3)
     {
@@ -227,11 +253,11 @@ int profile_gemm(int argc, char* argv[])
         const float sr = argc > 16 ? (float)std::atof(argv[16]) : 1.0f;
         const int nrep = argc > 17 ? std::atoi(argv[17]) : 10;
         if(epi == 0)
-            return profile_gemm_t<int8_t>(verify, init, time_kernel, M, N, K, sa, sb, sc, Pass{}, nrep);
+            return profile_gemm_t<int8_t>(layout, verify, init, time_kernel, M, N, K, sa, sb, sc, Pass{}, nrep);
         if(epi == 1)
-            return profile_gemm_t<int8_t>(verify, init, time_kernel, M, N, K, sa, sb, sc,
+            return profile_gemm_t<int8_t>(layout, verify, init, time_kernel, M, N, K, sa, sb, sc,
                                           element_wise::RequantReluRequant{sg, sr}, nrep);
-        return profile_gemm_t<int8_t>(verify, init, time_kernel, M, N, K, sa, sb, sc,
+        return profile_gemm_t<int8_t>(layout, verify, init, time_kernel, M, N, K, sa, sb, sc,
                                       element_wise::RequantRoundReluRequantRound{sg, sr}, nrep);
     }
     std::cout << "this data_type & layout is not implemented" << std::endl;

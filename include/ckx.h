@@ -95,7 +95,15 @@ const char* ckx_instance_name(int op, int instance);
  * ::MakeArgumentPointer + Invoker::Run (device_gemm.hpp:24-41,
  * device_gemm_xdl_cshuffle.hpp:399-556) and kernel_gemm_xdl_cshuffle_v1
  * (gridwise_gemm_xdl_cshuffle_v1.hpp:32-74).
- * A is [M,K], B is [K,N], C is [M,N]; *_layout selects which stride is 1. */
+ * A is [M,K], B is [K,N], C is [M,N]; *_layout selects which stride is 1:
+ *   a_layout CKX_ROW_MAJOR  "mk": A(m,k) at m*stride_a + k      CKX_COL_MAJOR "km": at k*stride_a + m
+ *   b_layout CKX_COL_MAJOR  "nk": B(k,n) at n*stride_b + k      CKX_ROW_MAJOR "kn": at k*stride_b + n
+ *   c_layout CKX_ROW_MAJOR only (as in the reference's instance lists
+ *   device_gemm_xdl_*_{mk_kn,mk_nk,km_kn,km_nk}_mn_instance.cpp).
+ * The contiguous extent of A and of B and both strides must be whole 16-byte vectors. mk_nk runs on
+ * every instance; a K-major operand (km / kn) on the tile instances of 64 rows and more (others report
+ * CKX_UNSUPPORTED), with the PassThrough / requant epilogues. This holds for every ckx_gemm_* and
+ * ckx_batched_gemm_* entry point below. */
 int ckx_gemm_i8_is_supported(int32_t M, int32_t N, int32_t K, int32_t stride_a, int32_t stride_b,
                              int32_t stride_c, int a_layout, int b_layout, int c_layout, int epilogue,
                              int instance);

@@ -165,3 +165,28 @@ def test_profiler_bf16_gemm(tmp_path):
     b_nk = uniform_bf16((N, K), -1, 1, SEED + 1)
     ref = fast.bf16_to_f32(lit.gemm_bf16(a, np.ascontiguousarray(b_nk.T)))
     assert np.all(np.abs(c - ref) <= 1e-2 + 1e-2 * np.abs(ref))
+
+
+@pytest.mark.parametrize("layout", [0, 2, 3])     # mk_kn, km_kn, km_nk (profiler/src/profile_gemm.cpp:13-19)
+def test_profiler_gemm_other_layouts(tmp_path, layout):
+    """The layouts with a K-major operand through the C++ operator templates: A stored [K,M] for km, B stored
+    [K,N] for kn, the generators filling the stored arrays in order."""
+    M, N, K = 384, 512, 640
+    out, dump = _run("ckx_profiler", ["gemm", 3, layout, 1, 1, 0, 1, M, N, K, -1, -1, -1, 2, 0.05, 0.4],
+                     "CKX_PROFILER_DUMP", tmp_path)
+    assert "Best Perf:" in out and "Error" not in out
+    assert out.count("does not support this problem") >= 8      # skinny and few-row tile instances
+    a_st = uniform_int8((K, M) if layout >= 2 else (M, K), -5, 5, SEED)
+    b_st = uniform_int8((K, N) if layout in (0, 2) else (N, K), -5, 5, SEED + 1)
+    a_mk = a_st.T if layout >= 2 else a_st
+    b_kn = b_st if layout in (0, 2) else b_st.T
+    c = np.fromfile(dump, np.int8).reshape(M, N)
+    np.testing.assert_array_equal(c, lit.gemm_i8(a_mk, b_kn, lit.EPI_REQUANT_RND, 0.05, 0.4))
+    out, dump = _run("ckx_profiler", ["gemm", 1, layout, 1, 2, 0, 1, M, N, K, -1, -1, -1], "CKX_PROFILER_DUMP", tmp_path)
+    assert "Best Perf:" in out and "Error" not in out
+    a_st = uniform_f16((K, M) if layout >= 2 else (M, K), -1, 1, SEED)
+    b_st = uniform_f16((K, N) if layout in (0, 2) else (N, K), -1, 1, SEED + 1)
+    c = np.fromfile(dump, np.float16).reshape(M, N)
+    bad, max_err = lit.check_err_f16(c, lit.gemm_f16(a_st.T if layout >= 2 else a_st, b_st if layout in (0, 2) else b_st.T),
+                                     1e-2, 1e-2)
+    assert bad == 0, max_err
