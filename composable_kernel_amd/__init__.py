@@ -8,7 +8,7 @@
 """
 from . import capi, device_ops, host_tensor  # noqa: F401
 from .device_ops import (  # noqa: F401
-    PassThrough, RequantReluRequant, AddRelu, AddReluAdd, RowMajor, ColumnMajor, StreamConfig,
+    PassThrough, Scale, RequantReluRequant, AddRelu, AddReluAdd, RowMajor, ColumnMajor, StreamConfig,
     DeviceGemmInt8, DeviceGemmF16, DeviceGemmBF16, DeviceGemmSplitKInt8, DeviceGemmSplitKF16, DeviceBatchedGemmInt8, DeviceBatchedGemmF16, DeviceGemmMultipleDF16, DeviceConv2dFwdInt8, DeviceConv2dFwdF16,
-    DeviceConv2dFwdBiasActivationF16, DeviceBatchedGemmGemmF16,
+    DeviceConv2dFwdBiasActivationF16, DeviceBatchedGemmGemmF16, DeviceBatchedGemmSoftmaxGemmF16,
 )

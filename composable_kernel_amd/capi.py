@@ -15,7 +15,8 @@ OK, UNSUPPORTED, INVALID_VALUE, HIP_ERROR = 0, -1, -2, -3
 ROW_MAJOR, COL_MAJOR = 0, 1
 EPI_PASSTHROUGH, EPI_REQUANT_CK, EPI_REQUANT_RND = 0, 1, 2
 EPI_ADD_RELU, EPI_ADD_RELU_ADD, EPI_CSHUFFLE_ADD_RELU = 3, 4, 5
-OP_GEMM_I8, OP_GEMM_F16, OP_CONV2D_FWD_I8, OP_CONV2D_FWD_F16, OP_BATCHED_GEMM_GEMM, OP_GEMM_SPLITK, OP_GEMM_BF16 = range(7)
+(OP_GEMM_I8, OP_GEMM_F16, OP_CONV2D_FWD_I8, OP_CONV2D_FWD_F16, OP_BATCHED_GEMM_GEMM, OP_GEMM_SPLITK, OP_GEMM_BF16,
+ OP_BATCHED_GEMM_SOFTMAX_GEMM) = range(8)
 INSTANCE_AUTO = -1
 
 # every symbol include/ckx.h declares
@@ -29,6 +30,7 @@ SYMBOLS = [
     "ckx_gemm_f16_multiple_d_is_supported", "ckx_gemm_f16_multiple_d", "ckx_conv2d_fwd_bias_activation_f16",
     "ckx_conv2d_fwd_is_supported", "ckx_conv2d_fwd_i8", "ckx_conv2d_fwd_f16", "ckx_conv2d_fwd_workspace_bytes",
     "ckx_batched_gemm_gemm_f16_is_supported", "ckx_batched_gemm_gemm_f16", "ckx_time_launches",
+    "ckx_batched_gemm_softmax_gemm_f16_is_supported", "ckx_batched_gemm_softmax_gemm_f16",
 ]
 
 
@@ -101,6 +103,9 @@ def lib():
     gg = [i32] * 9 + [i64] * 4 + [C.c_int]
     L.ckx_batched_gemm_gemm_f16_is_supported.argtypes = gg
     L.ckx_batched_gemm_gemm_f16.argtypes = [vp] * 4 + gg + [vp]
+    gsg = [i32] * 9 + [i64] * 4 + [f32, C.c_int, C.c_int]
+    L.ckx_batched_gemm_softmax_gemm_f16_is_supported.argtypes = gsg
+    L.ckx_batched_gemm_softmax_gemm_f16.argtypes = [vp] * 4 + gsg + [vp]
     L.ckx_time_launches.argtypes = [LAUNCH_FN, vp, C.c_int, C.c_int, vp, C.POINTER(C.c_float)]
     _lib = L
     return L

@@ -225,6 +225,7 @@ const char* family_prefix(int op)
     case CKX_OP_CONV2D_FWD_I8: return "DeviceConv2dFwd_i8_nhwc_kyxc_nhwk";
     case CKX_OP_CONV2D_FWD_F16: return "DeviceConv2dFwd_f16_nhwc_kyxc_nhwk";
     case CKX_OP_BATCHED_GEMM_GEMM: return "DeviceBatchedGemmGemm_f16_gmk_gnk_gno_gmo";
+    case CKX_OP_BATCHED_GEMM_SOFTMAX_GEMM: return "DeviceBatchedGemmSoftmaxGemm_f16_gmk_gnk_gno_gmo";
     case CKX_OP_GEMM_SPLITK: return "DeviceGemmSplitK_mk_nk_mn";
     case CKX_OP_GEMM_BF16: return "DeviceGemm_bf16_bf16_bf16_mk_nk_mn";
     default: return nullptr;
@@ -608,7 +609,7 @@ int ckx_num_instances(int op)
         return kNumTiles;
     if(op == CKX_OP_CONV2D_FWD_F16)
         return kNumTiles + 1; // + the input-patch kernel
-    if(op == CKX_OP_BATCHED_GEMM_GEMM)
+    if(op == CKX_OP_BATCHED_GEMM_GEMM || op == CKX_OP_BATCHED_GEMM_SOFTMAX_GEMM)
         return ckx::kNumGemmGemmInstances;
     return 0;
 }
@@ -620,7 +621,8 @@ const char* ckx_instance_name(int op, int instance)
     if(!fam || instance < 0 || instance >= ckx_num_instances(op))
         return nullptr;
     s = std::string(fam) + "<" +
-        (op == CKX_OP_BATCHED_GEMM_GEMM ? ckx::gemm_gemm_instance_name(instance)
+        (op == CKX_OP_BATCHED_GEMM_GEMM || op == CKX_OP_BATCHED_GEMM_SOFTMAX_GEMM
+             ? ckx::gemm_gemm_instance_name(instance)
          : op == CKX_OP_CONV2D_FWD_F16 && instance == kNumTiles
              ? kPatchName
              : instance >= kNumTiles ? kSkinny[instance - kNumTiles].name : kTiles[instance].name) +
@@ -830,7 +832,7 @@ int ckx_batched_gemm_gemm_f16(const void* a, const void* b0, const void* b1, voi
         return st;
     if(M == 0 || O == 0 || batch == 0)
         return CKX_OK;
-    if(!a || !b0 || !b1 || !c)
+    if(!a || !c || (N > 0 && (!b0 || !b1))) // (N == 0: B0 and B1 are empty, C = 0)
         return fail(CKX_INVALID_VALUE, "null operand pointer");
     if((reinterpret_cast<uintptr_t>(a) | reinterpret_cast<uintptr_t>(b0) | reinterpret_cast<uintptr_t>(b1) |
         reinterpret_cast<uintptr_t>(c)) & 15)
@@ -839,6 +841,41 @@ int ckx_batched_gemm_gemm_f16(const void* a, const void* b0, const void* b1, voi
                                          instance, (hipStream_t)stream);
     if(e != hipSuccess)
         return hip_fail(e, "batched_gemm_gemm");
+    return CKX_OK;
+}
+
+int ckx_batched_gemm_softmax_gemm_f16_is_supported(int32_t M, int32_t N, int32_t K, int32_t O, int32_t batch,
+                                                   int32_t sa, int32_t sb0, int32_t sb1, int32_t sc, int64_t bsa,
+                                                   int64_t bsb0, int64_t bsb1, int64_t bsc, float acc0_scale,
+                                                   int mask_out_upper_triangle, int instance)
+{
+    if(!(acc0_scale == acc0_scale) || acc0_scale - acc0_scale != 0.0f)
+        return fail(CKX_INVALID_VALUE, "the score scale must be finite");
+    if(mask_out_upper_triangle != 0 && mask_out_upper_triangle != 1)
+        return fail(CKX_INVALID_VALUE, "mask_out_upper_triangle is 0 or 1");
+    return ckx_batched_gemm_gemm_f16_is_supported(M, N, K, O, batch, sa, sb0, sb1, sc, bsa, bsb0, bsb1, bsc, instance);
+}
+
+int ckx_batched_gemm_softmax_gemm_f16(const void* a, const void* b0, const void* b1, void* c, int32_t M, int32_t N,
+                                      int32_t K, int32_t O, int32_t batch, int32_t sa, int32_t sb0, int32_t sb1,
+                                      int32_t sc, int64_t bsa, int64_t bsb0, int64_t bsb1, int64_t bsc,
+                                      float acc0_scale, int mask_out_upper_triangle, int instance, void* stream)
+{
+    int st = ckx_batched_gemm_softmax_gemm_f16_is_supported(M, N, K, O, batch, sa, sb0, sb1, sc, bsa, bsb0, bsb1, bsc,
+                                                            acc0_scale, mask_out_upper_triangle, instance);
+    if(st != CKX_OK)
+        return st;
+    if(M == 0 || O == 0 || batch == 0)
+        return CKX_OK;
+    if(!a || !c || (N > 0 && (!b0 || !b1))) // (N == 0: B0 and B1 are empty, C = 0)
+        return fail(CKX_INVALID_VALUE, "null operand pointer");
+    if((reinterpret_cast<uintptr_t>(a) | reinterpret_cast<uintptr_t>(b0) | reinterpret_cast<uintptr_t>(b1) |
+        reinterpret_cast<uintptr_t>(c)) & 15)
+        return fail(CKX_UNSUPPORTED, "operands must be 16-byte aligned");
+    hipError_t e = ckx::gemm_gemm_launch(a, b0, b1, c, M, N, K, O, batch, sa, sb0, sb1, sc, bsa, bsb0, bsb1, bsc,
+                                         instance, (hipStream_t)stream, true, acc0_scale, mask_out_upper_triangle != 0);
+    if(e != hipSuccess)
+        return hip_fail(e, "batched_gemm_softmax_gemm");
     return CKX_OK;
 }
 

@@ -12,6 +12,15 @@
 //   same lane must supply as the second operand of gemm1 (C^T = B1T_frag x S_frag) after a
 //   round-to-nearest-even conversion to fp16. B1 is transposed while it is staged into LDS
 //   so that its fragment is one 16-byte read as well.
+//
+// SOFTMAX variant (upstream's DeviceBatchedGemmSoftmaxGemm, "attention"):
+//   C[g] = half( half(softmax_n(scale * A[g] * B0[g], masked)) * B1[g] )
+// with the softmax along N in one pass over N (running row maximum and running sum): a step's
+// scores become p = exp(s - running max), the output accumulators and the running sum are rescaled
+// whenever the maximum grows, and the division by the sum happens once at the end. A row's 128
+// scores of a step sit in four lanes (l%16 = row, l/16 = q), 32 each: the row maximum and the final
+// sum cross those lanes with v_permlane16_swap / v_permlane32_swap. Columns past N and, with the
+// upper-triangle mask, columns n > m count as -infinity; masked-out steps are skipped altogether.
 #pragma once
 
 #include <hip/hip_runtime.h>
@@ -34,7 +43,29 @@ struct GemmGemmArgs
     int sa, sb0, sb1, sc;
     int64_t bsa, bsb0, bsb1, bsc;
     int slabs; // ceil(M / rows per workgroup)
+    float scale;   // softmax variant: scores are scale * (A * B0)
+    int mask_upper; // softmax variant: scores with n > m are masked out
 };
+
+// maximum / sum over the four lanes l, l^16, l^32, l^48 (every one of them gets the result)
+__device__ __forceinline__ float quad_rows_max(float x)
+{
+    auto a = __builtin_amdgcn_permlane16_swap(__builtin_bit_cast(uint32_t, x), __builtin_bit_cast(uint32_t, x), false, false);
+    const uint32_t a0 = a[0], a1 = a[1];
+    x      = __builtin_fmaxf(__builtin_bit_cast(float, a0), __builtin_bit_cast(float, a1));
+    auto b = __builtin_amdgcn_permlane32_swap(__builtin_bit_cast(uint32_t, x), __builtin_bit_cast(uint32_t, x), false, false);
+    const uint32_t b0 = b[0], b1 = b[1];
+    return __builtin_fmaxf(__builtin_bit_cast(float, b0), __builtin_bit_cast(float, b1));
+}
+__device__ __forceinline__ float quad_rows_sum(float x)
+{
+    auto a = __builtin_amdgcn_permlane16_swap(__builtin_bit_cast(uint32_t, x), __builtin_bit_cast(uint32_t, x), false, false);
+    const uint32_t a0 = a[0], a1 = a[1];
+    x      = __builtin_bit_cast(float, a0) + __builtin_bit_cast(float, a1);
+    auto b = __builtin_amdgcn_permlane32_swap(__builtin_bit_cast(uint32_t, x), __builtin_bit_cast(uint32_t, x), false, false);
+    const uint32_t b0 = b[0], b1 = b[1];
+    return __builtin_bit_cast(float, b0) + __builtin_bit_cast(float, b1);
+}
 
 // KS  k-steps of gemm0 (K padded to 32*KS), OG  64-column groups of the output (O padded to 64*OG),
 // MT  16-row MFMA tiles per wave, NW waves: a workgroup owns 16*MT*NW rows of one batch.
@@ -59,7 +90,7 @@ struct GemmGemmCfg
     static_assert(NB0 >= 1 && NB1 >= 1, "too many threads for one step");
 };
 
-template <int KS, int OG, int MT, int NW>
+template <int KS, int OG, int MT, int NW, bool SOFTMAX = false>
 __global__ __launch_bounds__(NW * 64) void gemm_gemm_kernel(const GemmGemmArgs p)
 {
     using Cfg = GemmGemmCfg<KS, OG, MT, NW>;
@@ -172,12 +203,23 @@ __global__ __launch_bounds__(NW * 64) void gemm_gemm_kernel(const GemmGemmArgs p
         for(int t = 0; t < OG * 4; ++t)
             acc1[mt][t] = f32x4{0, 0, 0, 0};
 
-    for(int n0 = 0; n0 < p.N; n0 += Cfg::BNC)
+    // softmax state of the MT rows this lane holds scores of (identical in the four lanes of a row,
+    // except row_sum, which is each lane's share until the end)
+    constexpr float kLog2e = 1.4426950408889634f;
+    const float ninf       = -__builtin_inff();
+    float row_max[MT], row_sum[MT];
+#pragma unroll
+    for(int mt = 0; mt < MT; ++mt)
+        row_max[mt] = ninf, row_sum[mt] = 0.0f;
+    // with the upper-triangle mask, columns past the slab's last row are masked for every row of it
+    const int n_end = (SOFTMAX && p.mask_upper && m0 + Cfg::BM < p.N) ? m0 + Cfg::BM : p.N;
+
+    for(int n0 = 0; n0 < n_end; n0 += Cfg::BNC)
     {
         __syncthreads(); // everyone is done reading the previous step from LDS
         store_step();
         __syncthreads();
-        if(n0 + Cfg::BNC < p.N)
+        if(n0 + Cfg::BNC < n_end)
             load_step(n0 + Cfg::BNC); // in flight while this step is multiplied
 
         // ---- gemm0: S^T tiles, 8 tiles of 16 columns, pairs share a 32-column span -----
@@ -199,6 +241,47 @@ __global__ __launch_bounds__(NW * 64) void gemm_gemm_kernel(const GemmGemmArgs p
                 for(int mt = 0; mt < MT; ++mt)
                     s[mt][t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(b0f, af[mt][ks], s[mt][t], 0, 0, 0);
             }
+
+        if constexpr(SOFTMAX)
+        {
+            // s[mt][t][j] is the score of row m0 + wave*16*MT + 16*mt + fr, column n0 + 32*(t/2) + 8q + 4*(t%2) + j
+#pragma unroll
+            for(int mt = 0; mt < MT; ++mt)
+            {
+                const int m = m0 + wave * 16 * MT + mt * 16 + fr;
+                const int n_lim = (p.mask_upper && m + 1 < p.N) ? m + 1 : p.N; // columns >= n_lim are masked
+                float mx = ninf;
+#pragma unroll
+                for(int t = 0; t < 8; ++t)
+#pragma unroll
+                    for(int j = 0; j < 4; ++j)
+                    {
+                        const int n  = n0 + 32 * (t >> 1) + 8 * q + 4 * (t & 1) + j;
+                        const float v = n < n_lim ? s[mt][t][j] * p.scale : ninf;
+                        s[mt][t][j]  = v;
+                        mx           = __builtin_fmaxf(mx, v);
+                    }
+                mx                 = quad_rows_max(mx);
+                const float m_new  = __builtin_fmaxf(row_max[mt], mx);
+                const float m_safe = m_new == ninf ? 0.0f : m_new; // a row with nothing unmasked yet: every p is 0
+                const float corr   = __builtin_amdgcn_exp2f((row_max[mt] - m_safe) * kLog2e);
+                row_max[mt]        = m_new;
+                float part         = 0.0f;
+#pragma unroll
+                for(int t = 0; t < 8; ++t)
+#pragma unroll
+                    for(int j = 0; j < 4; ++j)
+                    {
+                        const float e = __builtin_amdgcn_exp2f((s[mt][t][j] - m_safe) * kLog2e);
+                        s[mt][t][j]   = e;
+                        part += e;
+                    }
+                row_sum[mt] = row_sum[mt] * corr + part;
+#pragma unroll
+                for(int ot = 0; ot < OG * 4; ++ot)
+                    acc1[mt][ot] = acc1[mt][ot] * corr;
+            }
+        }
 
         // ---- fp32 -> fp16 (RNE): the pair (2*pr, 2*pr+1) is the gemm1 operand for 32 n ----
         f16x8 sf[MT][4];
@@ -230,6 +313,18 @@ __global__ __launch_bounds__(NW * 64) void gemm_gemm_kernel(const GemmGemmArgs p
     }
 
     const bool vec_ok = ((reinterpret_cast<uintptr_t>(C) | ((uintptr_t)p.sc * 2)) & 15u) == 0;
+    if constexpr(SOFTMAX)
+    {
+#pragma unroll
+        for(int mt = 0; mt < MT; ++mt)
+        {
+            const float total = quad_rows_sum(row_sum[mt]);
+            const float inv   = total > 0.0f ? 1.0f / total : 0.0f; // N == 0: an empty sum, C = 0
+#pragma unroll
+            for(int ot = 0; ot < OG * 4; ++ot)
+                acc1[mt][ot] = acc1[mt][ot] * inv;
+        }
+    }
 #pragma unroll
     for(int mt = 0; mt < MT; ++mt)
     {
@@ -279,11 +374,11 @@ inline bool gemm_gemm_supported(int M, int N, int K, int O, int batch, int sa, i
     return true;
 }
 
-template <int KS, int OG, int MT, int NW>
+template <int KS, int OG, int MT, int NW, bool SOFTMAX>
 inline hipError_t gemm_gemm_launch_t(GemmGemmArgs a, hipStream_t s)
 {
     using Cfg  = GemmGemmCfg<KS, OG, MT, NW>;
-    auto* kern = &gemm_gemm_kernel<KS, OG, MT, NW>;
+    auto* kern = &gemm_gemm_kernel<KS, OG, MT, NW, SOFTMAX>;
     static std::once_flag once;
     static hipError_t attr_err = hipSuccess;
     std::call_once(once, [&] {
@@ -297,21 +392,23 @@ inline hipError_t gemm_gemm_launch_t(GemmGemmArgs a, hipStream_t s)
     return hipGetLastError();
 }
 
-template <int MT, int NW>
+template <int MT, int NW, bool SOFTMAX>
 inline hipError_t gemm_gemm_launch_mt(const GemmGemmArgs& g, hipStream_t s)
 {
     const int ks = g.K <= 32 ? 1 : (g.K <= 64 ? 2 : 4);
     const int og = g.O <= 64 ? 1 : 2;
     if(ks == 1)
-        return og == 1 ? gemm_gemm_launch_t<1, 1, MT, NW>(g, s) : gemm_gemm_launch_t<1, 2, MT, NW>(g, s);
+        return og == 1 ? gemm_gemm_launch_t<1, 1, MT, NW, SOFTMAX>(g, s) : gemm_gemm_launch_t<1, 2, MT, NW, SOFTMAX>(g, s);
     if(ks == 2)
-        return og == 1 ? gemm_gemm_launch_t<2, 1, MT, NW>(g, s) : gemm_gemm_launch_t<2, 2, MT, NW>(g, s);
-    return og == 1 ? gemm_gemm_launch_t<4, 1, MT, NW>(g, s) : gemm_gemm_launch_t<4, 2, MT, NW>(g, s);
+        return og == 1 ? gemm_gemm_launch_t<2, 1, MT, NW, SOFTMAX>(g, s) : gemm_gemm_launch_t<2, 2, MT, NW, SOFTMAX>(g, s);
+    return og == 1 ? gemm_gemm_launch_t<4, 1, MT, NW, SOFTMAX>(g, s) : gemm_gemm_launch_t<4, 2, MT, NW, SOFTMAX>(g, s);
 }
 
+// softmax: the attention variant with scores scale * (A * B0) and the optional upper-triangle mask
 inline hipError_t gemm_gemm_launch(const void* a, const void* b0, const void* b1, void* c, int M, int N, int K,
                                    int O, int batch, int sa, int sb0, int sb1, int sc, int64_t bsa,
-                                   int64_t bsb0, int64_t bsb1, int64_t bsc, int instance, hipStream_t s)
+                                   int64_t bsb0, int64_t bsb1, int64_t bsc, int instance, hipStream_t s,
+                                   bool softmax = false, float scale = 1.0f, bool mask_upper = false)
 {
     GemmGemmArgs g;
     g.a = (const _Float16*)a, g.b0 = (const _Float16*)b0, g.b1 = (const _Float16*)b1, g.c = (_Float16*)c;
@@ -319,11 +416,16 @@ inline hipError_t gemm_gemm_launch(const void* a, const void* b0, const void* b1
     g.sa = sa, g.sb0 = sb0, g.sb1 = sb1, g.sc = sc;
     g.bsa = bsa, g.bsb0 = bsb0, g.bsb1 = bsb1, g.bsc = bsc;
     g.slabs = 0;
+    g.scale = scale, g.mask_upper = mask_upper;
     if(instance < 0)
         instance = 0;
-    return instance == 0 ? gemm_gemm_launch_mt<2, 4>(g, s)
-           : instance == 1 ? gemm_gemm_launch_mt<1, 4>(g, s)
-                           : gemm_gemm_launch_mt<1, 8>(g, s);
+    if(softmax)
+        return instance == 0 ? gemm_gemm_launch_mt<2, 4, true>(g, s)
+               : instance == 1 ? gemm_gemm_launch_mt<1, 4, true>(g, s)
+                               : gemm_gemm_launch_mt<1, 8, true>(g, s);
+    return instance == 0 ? gemm_gemm_launch_mt<2, 4, false>(g, s)
+           : instance == 1 ? gemm_gemm_launch_mt<1, 4, false>(g, s)
+                           : gemm_gemm_launch_mt<1, 8, false>(g, s);
 }
 
 } // namespace ckx

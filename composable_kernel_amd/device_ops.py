@@ -30,6 +30,13 @@ class PassThrough:
     scale_relu = 1.0
 
 
+class Scale:
+    """element_wise::Scale (unary_element_wise_operation.hpp:27-41): y = scale * x"""
+
+    def __init__(self, scale):
+        self.scale = float(scale)
+
+
 class RequantReluRequant:
     """example/14_gemm_xdl_requant_relu_requant/gemm_xdl_requant_relu_requant_int8.cpp:21-39.
     rounded=False is the literal functor (no rounding, truncating cast);
@@ -452,3 +459,37 @@ class DeviceBatchedGemmGemmF16(BaseOperator):
 
     def _launch(self, a, stream):
         return capi.lib().ckx_batched_gemm_gemm_f16(*a.ptrs, *a.dims, self.instance, C.c_void_p(stream or 0))
+
+
+class DeviceBatchedGemmSoftmaxGemmF16(BaseOperator):
+    """DeviceBatchedGemmSoftmaxGemm<Row, Col, Row, Row, half x4, PassThrough, PassThrough, Scale, PassThrough,
+    PassThrough, MaskOutUpperTriangle> (upstream's device_batched_gemm_softmax_gemm.hpp:29-62):
+    C[g] = half(half(softmax_n(mask(scale * A[g] B0[g]))) B1[g])."""
+    op_family = capi.OP_BATCHED_GEMM_SOFTMAX_GEMM
+
+    def __init__(self, instance=capi.INSTANCE_AUTO, MaskOutUpperTriangle=False):
+        super().__init__(instance)
+        self.mask = bool(MaskOutUpperTriangle)
+
+    def MakeArgumentPointer(self, p_a, p_b0, p_b1, p_c, M, N, K, O, Batch, StrideA, StrideB0, StrideB1,
+                            StrideC, BatchStrideA, BatchStrideB0, BatchStrideB1, BatchStrideC,
+                            a_element_op=None, b0_element_op=None, acc0_element_op=None,
+                            b1_element_op=None, c_element_op=None):
+        for op in (a_element_op, b0_element_op, b1_element_op, c_element_op):
+            if op is not None and not isinstance(op, PassThrough):
+                raise TypeError("only PassThrough element-wise operations are built for A, B0, B1 and C")
+        if acc0_element_op is not None and not isinstance(acc0_element_op, (Scale, PassThrough)):
+            raise TypeError("the score operation is Scale or PassThrough")
+        a = _GemmGemmArgument()
+        a.ptrs = (_ptr(p_a), _ptr(p_b0), _ptr(p_b1), _ptr(p_c))
+        a.dims = (int(M), int(N), int(K), int(O), int(Batch), int(StrideA), int(StrideB0), int(StrideB1),
+                  int(StrideC), int(BatchStrideA), int(BatchStrideB0), int(BatchStrideB1), int(BatchStrideC))
+        a.scale = acc0_element_op.scale if isinstance(acc0_element_op, Scale) else 1.0
+        return a
+
+    def _supported(self, a):
+        return capi.lib().ckx_batched_gemm_softmax_gemm_f16_is_supported(*a.dims, a.scale, int(self.mask), self.instance)
+
+    def _launch(self, a, stream):
+        return capi.lib().ckx_batched_gemm_softmax_gemm_f16(*a.ptrs, *a.dims, a.scale, int(self.mask), self.instance,
+                                                            C.c_void_p(stream or 0))

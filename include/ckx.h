@@ -73,7 +73,8 @@ enum
     CKX_OP_CONV2D_FWD_F16    = 3,
     CKX_OP_BATCHED_GEMM_GEMM = 4,
     CKX_OP_GEMM_SPLITK       = 5, /* instance list of the split-K GEMMs (the tile instances, both dtypes) */
-    CKX_OP_GEMM_BF16         = 6
+    CKX_OP_GEMM_BF16         = 6,
+    CKX_OP_BATCHED_GEMM_SOFTMAX_GEMM = 7
 };
 
 #define CKX_INSTANCE_AUTO (-1)
@@ -245,6 +246,31 @@ int ckx_batched_gemm_gemm_f16(const void* p_a, const void* p_b0, const void* p_b
                               int32_t stride_b0, int32_t stride_b1, int32_t stride_c,
                               int64_t batch_stride_a, int64_t batch_stride_b0, int64_t batch_stride_b1,
                               int64_t batch_stride_c, int instance, void* stream);
+
+/* ---- batched fused GEMM + softmax + GEMM ("attention"), fp16 ------------------
+ *   C[g] = half( half(softmax_n(mask(acc0_scale * (A[g] * B0[g])))) * B1[g] )
+ * The surface is upstream's DeviceBatchedGemmSoftmaxGemm::MakeArgumentPointer
+ * (device_batched_gemm_softmax_gemm.hpp:29-62 of later Composable Kernel releases) with
+ * Acc0ElementwiseOperation = Scale{acc0_scale}, every other functor PassThrough, and the class's
+ * MaskOutUpperTriangle parameter as an argument (scores with n > m count as -infinity). The pieces
+ * are the reference's: ReferenceBatchedGemm (reference_batched_gemm.hpp:56-88) and ReferenceSoftmax
+ * over n in fp32 (reference_softmax.hpp:61-113: exp(x - max) / sum). Layouts and limits as for
+ * ckx_batched_gemm_gemm_f16; neither the scores nor the probabilities leave the chip. The softmax
+ * is computed in one pass with a running maximum, so the probabilities are rounded to fp16 BEFORE
+ * the division by the row sum (the reference rounds after it): results agree within fp16 rounding
+ * of the probabilities, not bit for bit. N == 0 gives C = 0. */
+int ckx_batched_gemm_softmax_gemm_f16_is_supported(int32_t M, int32_t N, int32_t K, int32_t O, int32_t batch,
+                                                   int32_t stride_a, int32_t stride_b0, int32_t stride_b1,
+                                                   int32_t stride_c, int64_t batch_stride_a,
+                                                   int64_t batch_stride_b0, int64_t batch_stride_b1,
+                                                   int64_t batch_stride_c, float acc0_scale,
+                                                   int mask_out_upper_triangle, int instance);
+int ckx_batched_gemm_softmax_gemm_f16(const void* p_a, const void* p_b0, const void* p_b1, void* p_c, int32_t M,
+                                      int32_t N, int32_t K, int32_t O, int32_t batch, int32_t stride_a,
+                                      int32_t stride_b0, int32_t stride_b1, int32_t stride_c,
+                                      int64_t batch_stride_a, int64_t batch_stride_b0, int64_t batch_stride_b1,
+                                      int64_t batch_stride_c, float acc0_scale, int mask_out_upper_triangle,
+                                      int instance, void* stream);
 
 /* ---- timing helper --------------------------------------------------------
  * launch_and_time_kernel (include/ck/device_utility/kernel_launch.hpp:13-74):

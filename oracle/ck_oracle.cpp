@@ -14,6 +14,13 @@
 //       fp16 intermediate (the fused operator does not exist in the reference
 //       snapshot: parity UNPINNED by reference vectors, pinned by brute force
 //       and closed forms in tests/test_oracle.py)
+//   cko_batched_gemm_softmax_gemm_f16  ReferenceBatchedGemm (fp32 scores, element_wise::Scale,
+//       unary_element_wise_operation.hpp:27-41) -> upper-triangle mask -> ReferenceSoftmax over n
+//       (reference_softmax.hpp:56-117: max, exp(x - max), sum, alpha * e / sum + beta * out with
+//       alpha = 1, beta = 0; float in, half out) -> ReferenceBatchedGemm: the verification chain of
+//       upstream's batched_gemm_scale_softmax_gemm example. The fused operator is not in the
+//       reference snapshot; every piece is, and the chain is pinned against those pieces compiled
+//       from the reference (oracle/_ref), closed forms and scipy's softmax in tests/test_oracle.py.
 //   epilogue functors                RequantReluRequant
 //       example/14_gemm_xdl_requant_relu_requant/gemm_xdl_requant_relu_requant_int8.cpp:21-39
 //       PassThrough include/ck/tensor_operation/gpu/element/unary_element_wise_operation.hpp:13-25
@@ -37,6 +44,7 @@
 #include <cstdint>
 #include <cstring>
 #include <functional>
+#include <limits>
 #include <thread>
 #include <vector>
 
@@ -345,6 +353,49 @@ void cko_batched_gemm_gemm_f16(const uint16_t* a, const uint16_t* b0, const uint
                          (int64_t)M * N, N, 1, nthreads);
     cko_batched_gemm_f16(s.data(), b1, c, G, M, O, N, (int64_t)M * N, N, 1, sb1_g, sb1_n, sb1_o, sc_g,
                          sc_m, sc_o, nthreads);
+}
+
+// C[g] = fp16( fp16(softmax_n(mask(scale * (A[g] * B0[g])))) * B1[g] ): A [G,M,K], B0 logical [G,K,N],
+// B1 logical [G,N,O], C [G,M,O]. mask_upper: scores with n > m are -infinity before the softmax.
+void cko_batched_gemm_softmax_gemm_f16(const uint16_t* a, const uint16_t* b0, const uint16_t* b1, uint16_t* c,
+                                       int G, int M, int N, int K, int O, int64_t sa_g, int64_t sa_m,
+                                       int64_t sa_k, int64_t sb0_g, int64_t sb0_k, int64_t sb0_n,
+                                       int64_t sb1_g, int64_t sb1_n, int64_t sb1_o, int64_t sc_g, int64_t sc_m,
+                                       int64_t sc_o, float scale, int mask_upper, int nthreads)
+{
+    std::vector<uint16_t> prob((std::size_t)G * M * N);
+    parallel_for((std::size_t)G * M, nthreads, [&](std::size_t i0, std::size_t i1) {
+        std::vector<float> x((std::size_t)N);
+        for(std::size_t i = i0; i < i1; ++i)
+        {
+            const std::size_t g = i / (std::size_t)M, m = i % (std::size_t)M;
+            // gemm0: fp32 accumulation over k in order, then c_op = Scale: y = scale * x
+            for(int n = 0; n < N; ++n)
+            {
+                float acc = 0;
+                for(int k = 0; k < K; ++k)
+                    acc += half_to_float(a[g * sa_g + m * sa_m + k * sa_k]) *
+                           half_to_float(b0[g * sb0_g + k * sb0_k + n * sb0_n]);
+                x[n] = scale * acc;
+                if(mask_upper && (std::size_t)n > m)
+                    x[n] = -std::numeric_limits<float>::infinity();
+            }
+            // softmax over n: max (from lowest()), exp(x - max), sum in n order, e / sum
+            float mx = std::numeric_limits<float>::lowest();
+            for(int n = 0; n < N; ++n)
+                mx = std::max(mx, x[n]);
+            float sum = 0;
+            for(int n = 0; n < N; ++n)
+            {
+                x[n] = std::exp(x[n] - mx);
+                sum += x[n];
+            }
+            for(int n = 0; n < N; ++n)
+                prob[(g * M + m) * N + n] = float_to_half(1.0f * x[n] / sum + 0.0f * 0.0f);
+        }
+    });
+    cko_batched_gemm_f16(prob.data(), b1, c, G, M, O, N, (int64_t)M * N, N, 1, sb1_g, sb1_n, sb1_o, sc_g, sc_m,
+                         sc_o, nthreads);
 }
 
 // conv output length along one spatial dimension

@@ -130,3 +130,14 @@ def gemm_f16_add_relu(a_mk, b_kn, d_mn):
 def batched_gemm_gemm_f16(a_gmk, b0_gkn, b1_gno):
     s = np.matmul(np.asarray(a_gmk, np.float32), np.asarray(b0_gkn, np.float32)).astype(np.float16)
     return np.matmul(s.astype(np.float32), np.asarray(b1_gno, np.float32)).astype(np.float16)
+
+
+def batched_gemm_softmax_gemm_f16(a_gmk, b0_gkn, b1_gno, scale=1.0, mask_upper=False):
+    """numpy form of lit.batched_gemm_softmax_gemm_f16 (fp32 BLAS sums: within tolerance, not bit-equal)."""
+    x = np.float32(scale) * np.matmul(np.asarray(a_gmk, np.float32), np.asarray(b0_gkn, np.float32))
+    if mask_upper:
+        M, N = x.shape[1:]
+        x = np.where(np.arange(N)[None, None, :] > np.arange(M)[None, :, None], -np.inf, x).astype(np.float32)
+    e = np.exp(x - x.max(axis=2, keepdims=True))
+    p = (e / e.sum(axis=2, keepdims=True, dtype=np.float32)).astype(np.float16)
+    return np.matmul(p.astype(np.float32), np.asarray(b1_gno, np.float32)).astype(np.float16)

@@ -135,6 +135,19 @@ def batched_gemm_gemm_f16(a_gmk, b0_gkn, b1_gno, nthreads=0):
     return c
 
 
+def batched_gemm_softmax_gemm_f16(a_gmk, b0_gkn, b1_gno, scale=1.0, mask_upper=False, nthreads=0):
+    """C[g] = half(half(softmax_n(mask(scale * A[g] B0[g]))) B1[g]); mask_upper: scores with n > m are masked."""
+    G, M, K = a_gmk.shape
+    _, _, N = b0_gkn.shape
+    _, _, O = b1_gno.shape
+    c = np.empty((G, M, O), np.float16)
+    sa, sb0, sb1 = _estrides(a_gmk), _estrides(b0_gkn), _estrides(b1_gno)
+    lib().cko_batched_gemm_softmax_gemm_f16(_p(a_gmk), _p(b0_gkn), _p(b1_gno), _p(c), G, M, N, K, O,
+                                            *_i64(*sa, *sb0, *sb1, M * O, O, 1), C.c_float(scale),
+                                            int(bool(mask_upper)), int(nthreads))
+    return c
+
+
 def conv_out_len(in_len, filt, stride, dil, pl, pr):
     return int(lib().cko_conv_out_len(in_len, filt, stride, dil, pl, pr))
 

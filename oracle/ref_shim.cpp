@@ -9,6 +9,8 @@
 //   ReferenceGemm<half,half,half,float,Pass,Pass,Pass>                 (example 01 fp16)
 //   ReferenceConvFwd<T,T,T,Pass,Pass,Pass,2> for float / half / int8
 //   ReferenceBatchedGemm<half,half,half,Pass,Pass,Pass>
+//   ReferenceBatchedGemm<half,half,float,Pass,Pass,Scale> -> ReferenceSoftmax<float,half,float> ->
+//   ReferenceBatchedGemm<half,half,half,...>: the pieces of the fused GEMM + softmax + GEMM check
 //
 // RequantReluRequant lives inside the example's translation unit
 // (example/14_.../gemm_xdl_requant_relu_requant_int8.cpp:21-39), which also pulls
@@ -20,6 +22,7 @@
 #include <cmath>
 #include <cstdint>
 #include <cstring>
+#include <limits>
 #include <vector>
 
 #include "ck/utility/magic_division.hpp"
@@ -29,6 +32,7 @@
 #include "ck/library/reference_tensor_operation/cpu/reference_gemm.hpp"
 #include "ck/library/reference_tensor_operation/cpu/reference_conv_fwd.hpp"
 #include "ck/library/reference_tensor_operation/cpu/reference_batched_gemm.hpp"
+#include "ck/library/reference_tensor_operation/cpu/reference_softmax.hpp"
 #include "ck/library/reference_tensor_operation/cpu/reference_conv_fwd_bias_activation.hpp"
 #include "ck/library/reference_tensor_operation/cpu/reference_conv_fwd_bias_activation_add.hpp"
 
@@ -186,6 +190,52 @@ void ckref_batched_gemm_f16(const uint16_t* a, const uint16_t* b, uint16_t* c, i
     auto inv = ref.MakeInvoker();
     auto arg = ref.MakeArgument(ta, tb, tc, PassThrough{}, PassThrough{}, PassThrough{});
     inv.Run(arg);
+    std::memcpy(c, tc.mData.data(), tc.mData.size() * sizeof(H));
+}
+
+// scores = Scale(A * B0) in fp32 (the reference's ReferenceBatchedGemm and element_wise::Scale), optional
+// upper-triangle mask, the reference's ReferenceSoftmax over n (float in, half out, alpha 1, beta 0),
+// then the reference's ReferenceBatchedGemm with B1
+void ckref_batched_gemm_softmax_gemm_f16(const uint16_t* a, const uint16_t* b0, const uint16_t* b1, uint16_t* c,
+                                         int G, int M, int N, int K, int O, long sa_g, long sa_m, long sa_k,
+                                         long sb0_g, long sb0_k, long sb0_n, long sb1_g, long sb1_n, long sb1_o,
+                                         float scale, int mask_upper)
+{
+    using H     = ck::half_t;
+    using sz    = std::size_t;
+    using Scale = ck::tensor_operation::element_wise::Scale;
+    auto ta  = make_tensor<H>({(sz)G, (sz)M, (sz)K}, {(sz)sa_g, (sz)sa_m, (sz)sa_k}, (const H*)a);
+    auto tb0 = make_tensor<H>({(sz)G, (sz)K, (sz)N}, {(sz)sb0_g, (sz)sb0_k, (sz)sb0_n}, (const H*)b0);
+    auto tb1 = make_tensor<H>({(sz)G, (sz)N, (sz)O}, {(sz)sb1_g, (sz)sb1_n, (sz)sb1_o}, (const H*)b1);
+    Tensor<float> acc0(HostTensorDescriptor(std::vector<sz>{(sz)G, (sz)M, (sz)N}));
+    Tensor<H> prob(HostTensorDescriptor(std::vector<sz>{(sz)G, (sz)M, (sz)N}));
+    Tensor<H> tc(HostTensorDescriptor(std::vector<sz>{(sz)G, (sz)M, (sz)O}));
+    {
+        using Ref = ck::tensor_operation::host::ReferenceBatchedGemm<H, H, float, PassThrough, PassThrough, Scale>;
+        Ref ref;
+        auto inv = ref.MakeInvoker();
+        auto arg = ref.MakeArgument(ta, tb0, acc0, PassThrough{}, PassThrough{}, Scale{scale});
+        inv.Run(arg);
+    }
+    if(mask_upper)
+        acc0.ForEach([&](auto& self, auto idx) {
+            if(idx[2] > idx[1])
+                self(idx) = -std::numeric_limits<float>::infinity();
+        });
+    {
+        using Ref = ck::tensor_operation::host::ReferenceSoftmax<float, H, float>;
+        Ref ref;
+        auto inv = ref.MakeInvoker();
+        auto arg = ref.MakeArgument(acc0, prob, 1.0f, 0.0f, {2});
+        inv.Run(arg);
+    }
+    {
+        using Ref = ck::tensor_operation::host::ReferenceBatchedGemm<H, H, H, PassThrough, PassThrough, PassThrough>;
+        Ref ref;
+        auto inv = ref.MakeInvoker();
+        auto arg = ref.MakeArgument(prob, tb1, tc, PassThrough{}, PassThrough{}, PassThrough{});
+        inv.Run(arg);
+    }
     std::memcpy(c, tc.mData.data(), tc.mData.size() * sizeof(H));
 }
 

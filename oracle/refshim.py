@@ -69,6 +69,16 @@ class _Ref:
                                         *_es(b_gkn), C.c_long(M * N), C.c_long(N), C.c_long(1))
         return c
 
+    def batched_gemm_softmax_gemm_f16(self, a_gmk, b0_gkn, b1_gno, scale=1.0, mask_upper=False):
+        G, M, K = a_gmk.shape
+        _, _, N = b0_gkn.shape
+        _, _, O = b1_gno.shape
+        c = np.zeros((G, M, O), np.float16)
+        self.lib.ckref_batched_gemm_softmax_gemm_f16(_p(a_gmk), _p(b0_gkn), _p(b1_gno), _p(c), G, M, N, K, O,
+                                                     *_es(a_gmk), *_es(b0_gkn), *_es(b1_gno), C.c_float(scale),
+                                                     int(bool(mask_upper)))
+        return c
+
     def conv2d_fwd(self, inp_nhwc, wei_kyxc, strides=(1, 1), dilations=(1, 1), pads=(0, 0)):
         inp = np.ascontiguousarray(inp_nhwc)
         wei = np.ascontiguousarray(wei_kyxc)

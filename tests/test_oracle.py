@@ -12,6 +12,7 @@ import numpy as np
 import pytest
 
 import oracle
+from composable_kernel_amd.host_tensor import uniform_f16
 from oracle import lit, fast
 
 HERE = os.path.dirname(os.path.abspath(__file__))
@@ -448,3 +449,55 @@ def test_gemm_bf16_closed_forms_fast_and_ref():
     assert np.all(np.abs(fast.bf16_to_f32(c) - f) <= 1e-2 + 1e-2 * np.abs(f))
     if REF is not None:
         np.testing.assert_array_equal(REF.gemm_bf16(a, b), c)
+
+
+def test_gemm_softmax_gemm_closed_forms():
+    """What the mathematics fixes: zero scores give the uniform distribution; under the upper-triangle mask
+    row 0 sees only column 0; a dominant score selects its row of B1; the scale multiplies the scores."""
+    G, M, N, K, O = 2, 24, 32, 16, 8
+    b1 = (np.arange(G * N * O).reshape(G, N, O) % 7).astype(np.float16)
+    a0 = np.zeros((G, M, K), np.float16)
+    b0 = uniform_f16((G, K, N), -1, 1, 71)
+    # uniform: p = half(1/32) = 2^-5 exactly, C = mean over n of B1 (small integers / 32: exact in fp16)
+    np.testing.assert_array_equal(lit.batched_gemm_softmax_gemm_f16(a0, b0, b1),
+                                  np.broadcast_to(b1.astype(np.float32).mean(axis=1, keepdims=True), (G, M, O)).astype(np.float16))
+    # mask: row m averages rows 0..m of B1; row 0 is B1[0] exactly, row 3 the mean of four rows
+    c = lit.batched_gemm_softmax_gemm_f16(a0, b0, b1, mask_upper=True)
+    np.testing.assert_array_equal(c[:, 0], b1[:, 0])
+    np.testing.assert_array_equal(c[:, 3], b1[:, :4].astype(np.float32).mean(axis=1).astype(np.float16))
+    # dominant score: A = e_k rows, B0 = 40 * identity-like -> softmax is one-hot to within exp(-40)
+    a = np.zeros((G, M, K), np.float16)
+    a[:, np.arange(M), np.arange(M) % K] = 1
+    b0h = np.zeros((G, K, N), np.float16)
+    b0h[:, np.arange(K), (np.arange(K) * 2) % N] = 40
+    c = lit.batched_gemm_softmax_gemm_f16(a, b0h, b1)
+    np.testing.assert_array_equal(c, b1[:, ((np.arange(M) % K) * 2) % N])
+    # the scale acts on the scores: scale 0 is the uniform case whatever A and B0 hold
+    an = uniform_f16((G, M, K), -1, 1, 72)
+    np.testing.assert_array_equal(lit.batched_gemm_softmax_gemm_f16(an, b0, b1, scale=0.0),
+                                  lit.batched_gemm_softmax_gemm_f16(a0, b0, b1))
+
+
+@pytest.mark.parametrize("mask", [False, True])
+def test_gemm_softmax_gemm_against_scipy_fast_and_ref(mask):
+    """float64 softmax (scipy) with an fp16 rounding of the probabilities, the numpy form, and -- bit for bit --
+    the reference's own ReferenceBatchedGemm / Scale / ReferenceSoftmax chain where it is built."""
+    from scipy.special import softmax
+    for (G, M, N, K, O), scale in [((3, 40, 72, 24, 16), 0.125), ((2, 65, 33, 64, 40), 1.0), ((1, 7, 130, 8, 8), 0.5)]:
+        a = uniform_f16((G, M, K), -1, 1, 80 + M)
+        b0 = uniform_f16((G, N, K), -1, 1, 81 + N).transpose(0, 2, 1)      # stored [G,N,K]
+        b1 = uniform_f16((G, N, O), -1, 1, 82 + O)
+        c = lit.batched_gemm_softmax_gemm_f16(a, b0, b1, scale, mask)
+        x = scale * np.matmul(a.astype(np.float64), b0.astype(np.float64))
+        if mask:
+            x = np.where(np.arange(N)[None, None, :] > np.arange(M)[None, :, None], -np.inf, x)
+        p = softmax(x, axis=2).astype(np.float16)
+        want = np.matmul(p.astype(np.float64), b1.astype(np.float64))
+        assert np.abs(c.astype(np.float64) - want).max() < 2e-3
+        bad, max_err = lit.check_err_f16(fast.batched_gemm_softmax_gemm_f16(a, b0, b1, scale, mask), c, 1e-2, 1e-2)
+        assert bad == 0, max_err
+        if REF is not None:
+            np.testing.assert_array_equal(REF.batched_gemm_softmax_gemm_f16(a, b0, b1, scale, mask).view(np.uint16),
+                                          c.view(np.uint16))
+        # thread count is unobservable
+        np.testing.assert_array_equal(lit.batched_gemm_softmax_gemm_f16(a, b0, b1, scale, mask, nthreads=1), c)
