@@ -75,7 +75,12 @@ for w in (
        _conv_workload("conv_f16_c64_k64_3x3_56_bias_relu_add", "f16", 64, 64, 3, 56, 1, 1, fused="bias_relu_add"),
        _conv_workload("conv_f16_c256_k512_1x1_56_s2_bias_relu", "f16", 256, 512, 1, 56, 2, 0, fused="bias_relu")]
     + [dict(name="gemm_gemm_f16_b64_512x64x512x64", kind="gemm_gemm", dtype="f16", G=64, M=512, N=512, K=64, O=64,
-            ops=2.0 * 64 * 512 * 512 * 64 * 2, bytes=4 * 64 * 512 * 64 * 2)]
+            ops=2.0 * 64 * 512 * 512 * 64 * 2, bytes=4 * 64 * 512 * 64 * 2),
+       # the same shapes with a softmax between the GEMMs (attention): 64 heads of 512 x 512 scores, and a long one
+       dict(name="gemm_softmax_gemm_f16_b64_512x64x512x64", kind="gemm_gemm", softmax=True, dtype="f16", G=64, M=512,
+            N=512, K=64, O=64, ops=2.0 * 64 * 512 * 512 * 64 * 2, bytes=4 * 64 * 512 * 64 * 2),
+       dict(name="gemm_softmax_gemm_f16_b64_4096x64x4096x64", kind="gemm_gemm", softmax=True, dtype="f16", G=64, M=4096,
+            N=4096, K=64, O=64, ops=2.0 * 64 * 4096 * 4096 * 64 * 2, bytes=4 * 64 * 4096 * 64 * 2)]
 ):
     WORKLOADS[w["name"]] = w
 
@@ -165,8 +170,13 @@ def make_launcher(w, instance=-1, rotate=1):
         G, M, N, K, O = (w[k] for k in ("G", "M", "N", "K", "O"))
         a, b0, b1 = (dev(uniform_f16(s, -0.5, 0.5, 5 + j)) for j, s in enumerate([(G, M, K), (G, N, K), (G, N, O)]))
         c = torch.empty((G, M, O), dtype=torch.float16, device="cuda")
-        op = ck.DeviceBatchedGemmGemmF16(instance)
-        arg = op.MakeArgumentPointer(a, b0, b1, c, M, N, K, O, G, K, K, O, O, M * K, N * K, N * O, M * O)
+        if w.get("softmax"):
+            op = ck.DeviceBatchedGemmSoftmaxGemmF16(instance)
+            arg = op.MakeArgumentPointer(a, b0, b1, c, M, N, K, O, G, K, K, O, O, M * K, N * K, N * O, M * O,
+                                         None, None, ck.Scale(K ** -0.5))
+        else:
+            op = ck.DeviceBatchedGemmGemmF16(instance)
+            arg = op.MakeArgumentPointer(a, b0, b1, c, M, N, K, O, G, K, K, O, O, M * K, N * K, N * O, M * O)
     keep.append(c)
     if not op.IsSupportedArgument(arg):
         raise RuntimeError(f"{w['name']}: not supported: {capi.last_error()}")

@@ -91,7 +91,11 @@ struct GemmGemmCfg
 };
 
 template <int KS, int OG, int MT, int NW, bool SOFTMAX = false>
-__global__ __launch_bounds__(NW * 64) void gemm_gemm_kernel(const GemmGemmArgs p)
+// (the 32-row-per-wave softmax variant for small K and O is held to 256 registers, two waves per SIMD: one
+// wave's exponentials then overlap the other's MFMAs; left alone the compiler takes 340 and runs one)
+__global__ __launch_bounds__(NW * 64)
+    __attribute__((amdgpu_waves_per_eu(SOFTMAX && MT == 2 && KS <= 2 && OG == 1 ? 2 : 1))) void gemm_gemm_kernel(
+        const GemmGemmArgs p)
 {
     using Cfg = GemmGemmCfg<KS, OG, MT, NW>;
     constexpr int KCH = Cfg::KCH, OCH = Cfg::OCH, NB0 = Cfg::NB0, NB1 = Cfg::NB1, NT = Cfg::NT;
@@ -244,27 +248,45 @@ __global__ __launch_bounds__(NW * 64) void gemm_gemm_kernel(const GemmGemmArgs p
 
         if constexpr(SOFTMAX)
         {
-            // s[mt][t][j] is the score of row m0 + wave*16*MT + 16*mt + fr, column n0 + 32*(t/2) + 8q + 4*(t%2) + j
+            // s[mt][t][j] is the score of row m0 + wave*16*MT + 16*mt + fr, column n0 + 32*(t/2) + 8q + 4*(t%2) + j.
+            // Everything below works on x = score * scale * log2(e), so that exp(score - max) is one
+            // v_exp_f32 of a difference.
+            const float c2 = p.scale * kLog2e;
+            // does this step hold masked columns for any row of this wave? (wave-uniform: the plain path
+            // skips the per-element compare and select)
+            const int wave_m0    = m0 + wave * 16 * MT;
+            const bool step_mask = n0 + Cfg::BNC > p.N || (p.mask_upper && n0 + Cfg::BNC > wave_m0 + 1);
 #pragma unroll
             for(int mt = 0; mt < MT; ++mt)
             {
-                const int m = m0 + wave * 16 * MT + mt * 16 + fr;
+                const int m     = wave_m0 + mt * 16 + fr;
                 const int n_lim = (p.mask_upper && m + 1 < p.N) ? m + 1 : p.N; // columns >= n_lim are masked
                 float mx = ninf;
+                if(step_mask)
+                {
+#pragma unroll
+                    for(int t = 0; t < 8; ++t)
+#pragma unroll
+                        for(int j = 0; j < 4; ++j)
+                        {
+                            const int n = n0 + 32 * (t >> 1) + 8 * q + 4 * (t & 1) + j;
+                            s[mt][t][j] = n < n_lim ? s[mt][t][j] * c2 : ninf;
+                        }
+                }
+                else
+                {
+#pragma unroll
+                    for(int t = 0; t < 8; ++t)
+                        s[mt][t] = s[mt][t] * c2;
+                }
 #pragma unroll
                 for(int t = 0; t < 8; ++t)
-#pragma unroll
-                    for(int j = 0; j < 4; ++j)
-                    {
-                        const int n  = n0 + 32 * (t >> 1) + 8 * q + 4 * (t & 1) + j;
-                        const float v = n < n_lim ? s[mt][t][j] * p.scale : ninf;
-                        s[mt][t][j]  = v;
-                        mx           = __builtin_fmaxf(mx, v);
-                    }
+                    mx = __builtin_fmaxf(__builtin_fmaxf(mx, __builtin_fmaxf(s[mt][t][0], s[mt][t][1])),
+                                         __builtin_fmaxf(s[mt][t][2], s[mt][t][3]));
                 mx                 = quad_rows_max(mx);
                 const float m_new  = __builtin_fmaxf(row_max[mt], mx);
                 const float m_safe = m_new == ninf ? 0.0f : m_new; // a row with nothing unmasked yet: every p is 0
-                const float corr   = __builtin_amdgcn_exp2f((row_max[mt] - m_safe) * kLog2e);
+                const float corr   = __builtin_amdgcn_exp2f(row_max[mt] - m_safe);
                 row_max[mt]        = m_new;
                 float part         = 0.0f;
 #pragma unroll
@@ -272,14 +294,18 @@ __global__ __launch_bounds__(NW * 64) void gemm_gemm_kernel(const GemmGemmArgs p
 #pragma unroll
                     for(int j = 0; j < 4; ++j)
                     {
-                        const float e = __builtin_amdgcn_exp2f((s[mt][t][j] - m_safe) * kLog2e);
+                        const float e = __builtin_amdgcn_exp2f(s[mt][t][j] - m_safe);
                         s[mt][t][j]   = e;
                         part += e;
                     }
                 row_sum[mt] = row_sum[mt] * corr + part;
+                // (wave-uniform skip: once the running maxima have settled, corr is 1 in every lane)
+                if(__builtin_amdgcn_ballot_w64(corr != 1.0f) != 0)
+                {
 #pragma unroll
-                for(int ot = 0; ot < OG * 4; ++ot)
-                    acc1[mt][ot] = acc1[mt][ot] * corr;
+                    for(int ot = 0; ot < OG * 4; ++ot)
+                        acc1[mt][ot] = acc1[mt][ot] * corr;
+                }
             }
         }
 
@@ -418,7 +444,10 @@ inline hipError_t gemm_gemm_launch(const void* a, const void* b0, const void* b1
     g.slabs = 0;
     g.scale = scale, g.mask_upper = mask_upper;
     if(instance < 0)
-        instance = 0;
+        // softmax: many short waves overlap one wave's exponentials with another's MFMAs (8 x 16 rows: 13.4 vs
+        // 14.8 us at batch 64, 512 x 512 scores); over a long N the 32-row waves of the register-capped variant
+        // read B0 / B1 fragments half as often per row and win (434 vs 581 us at 4096 x 4096)
+        instance = !softmax ? 0 : (K <= 64 && O <= 64 && N >= 1024) ? 0 : 2;
     if(softmax)
         return instance == 0 ? gemm_gemm_launch_mt<2, 4, true>(g, s)
                : instance == 1 ? gemm_gemm_launch_mt<1, 4, true>(g, s)

@@ -84,6 +84,14 @@ struct PassThrough
     }
 };
 
+// y = scale * x (unary_element_wise_operation.hpp:27-41)
+struct Scale
+{
+    Scale(float scale = 1.0f) : scale_(scale) {}
+    void operator()(float& y, const float& x) const { y = scale_ * x; }
+    float scale_;
+};
+
 // y = clamp(scaleRelu * relu(scaleGemm * x), -128, 127); the int8 cast truncates
 // (example/14_gemm_xdl_requant_relu_requant/gemm_xdl_requant_relu_requant_int8.cpp:21-39)
 struct RequantReluRequant
@@ -244,6 +252,23 @@ template <typename ALayout, typename B0Layout, typename B1Layout, typename CLayo
           typename B0ElementwiseOperation, typename Acc0ElementwiseOperation, typename B1ElementwiseOperation,
           typename CElementwiseOperation>
 struct DeviceBatchedGemmGemm : public BaseOperator
+{
+    virtual std::unique_ptr<BaseArgument>
+    MakeArgumentPointer(const void* p_a, const void* p_b0, const void* p_b1, void* p_c, index_t M, index_t N,
+                        index_t K, index_t O, index_t Batch, index_t StrideA, index_t StrideB0, index_t StrideB1,
+                        index_t StrideC, index_t BatchStrideA, index_t BatchStrideB0, index_t BatchStrideB1,
+                        index_t BatchStrideC, AElementwiseOperation a_element_op,
+                        B0ElementwiseOperation b0_element_op, Acc0ElementwiseOperation acc0_element_op,
+                        B1ElementwiseOperation b1_element_op, CElementwiseOperation c_element_op) = 0;
+    virtual std::unique_ptr<BaseInvoker> MakeInvokerPointer()                                     = 0;
+};
+
+// upstream device_batched_gemm_softmax_gemm.hpp:15-62
+template <typename ALayout, typename B0Layout, typename B1Layout, typename CLayout, typename ADataType,
+          typename B0DataType, typename B1DataType, typename CDataType, typename AElementwiseOperation,
+          typename B0ElementwiseOperation, typename Acc0ElementwiseOperation, typename B1ElementwiseOperation,
+          typename CElementwiseOperation, bool MaskOutUpperTriangle>
+struct DeviceBatchedGemmSoftmaxGemm : public BaseOperator
 {
     virtual std::unique_ptr<BaseArgument>
     MakeArgumentPointer(const void* p_a, const void* p_b0, const void* p_b1, void* p_c, index_t M, index_t N,
@@ -1066,6 +1091,90 @@ struct DeviceBatchedGemmGemmMfma
         if(instance_ == CKX_INSTANCE_AUTO)
             return "DeviceBatchedGemmGemm_f16_gmk_gnk_gno_gmo<auto>";
         return ckx_instance_name(CKX_OP_BATCHED_GEMM_GEMM, instance_);
+    }
+    int instance_;
+};
+
+// ------------------------------------------------------------- GEMM + softmax + GEMM
+// Acc0ElementwiseOperation: element_wise::Scale (or PassThrough = scale 1); MaskOutUpperTriangle as in upstream
+template <typename Acc0ElementwiseOperation = element_wise::Scale, bool MaskOutUpperTriangle = false>
+struct DeviceBatchedGemmSoftmaxGemmMfma
+    : public DeviceBatchedGemmSoftmaxGemm<tensor_layout::gemm::RowMajor, tensor_layout::gemm::ColumnMajor,
+                                          tensor_layout::gemm::RowMajor, tensor_layout::gemm::RowMajor, half_t, half_t,
+                                          half_t, half_t, element_wise::PassThrough, element_wise::PassThrough,
+                                          Acc0ElementwiseOperation, element_wise::PassThrough,
+                                          element_wise::PassThrough, MaskOutUpperTriangle>
+{
+    using Pass = element_wise::PassThrough;
+    static_assert(std::is_same_v<Acc0ElementwiseOperation, element_wise::Scale> ||
+                      std::is_same_v<Acc0ElementwiseOperation, Pass>,
+                  "the score operation is Scale or PassThrough");
+    struct Argument : public BaseArgument
+    {
+        const void *p_a, *p_b0, *p_b1;
+        void* p_c;
+        index_t M, N, K, O, Batch, StrideA, StrideB0, StrideB1, StrideC;
+        int64_t BatchStrideA, BatchStrideB0, BatchStrideB1, BatchStrideC;
+        float scale;
+    };
+    static float ScaleOf(const element_wise::Scale& op) { return op.scale_; }
+    static float ScaleOf(const Pass&) { return 1.0f; }
+    static int Supported(const Argument& a, int inst)
+    {
+        return ckx_batched_gemm_softmax_gemm_f16_is_supported(a.M, a.N, a.K, a.O, a.Batch, a.StrideA, a.StrideB0,
+                                                              a.StrideB1, a.StrideC, a.BatchStrideA, a.BatchStrideB0,
+                                                              a.BatchStrideB1, a.BatchStrideC, a.scale,
+                                                              MaskOutUpperTriangle ? 1 : 0, inst);
+    }
+    static int Launch(const Argument& a, int inst, void* stream)
+    {
+        return ckx_batched_gemm_softmax_gemm_f16(a.p_a, a.p_b0, a.p_b1, a.p_c, a.M, a.N, a.K, a.O, a.Batch, a.StrideA,
+                                                 a.StrideB0, a.StrideB1, a.StrideC, a.BatchStrideA, a.BatchStrideB0,
+                                                 a.BatchStrideB1, a.BatchStrideC, a.scale,
+                                                 MaskOutUpperTriangle ? 1 : 0, inst, stream);
+    }
+    using Invoker = detail::InvokerT<Argument, &Supported, &Launch>;
+
+    explicit DeviceBatchedGemmSoftmaxGemmMfma(int instance = CKX_INSTANCE_AUTO) : instance_(instance) {}
+    static Argument MakeArgument(const half_t* p_a, const half_t* p_b0, const half_t* p_b1, half_t* p_c, index_t M,
+                                 index_t N, index_t K, index_t O, index_t Batch, index_t StrideA, index_t StrideB0,
+                                 index_t StrideB1, index_t StrideC, index_t BatchStrideA, index_t BatchStrideB0,
+                                 index_t BatchStrideB1, index_t BatchStrideC, Pass = {}, Pass = {},
+                                 Acc0ElementwiseOperation acc0_element_op = {}, Pass = {}, Pass = {})
+    {
+        Argument a;
+        a.p_a = p_a, a.p_b0 = p_b0, a.p_b1 = p_b1, a.p_c = p_c;
+        a.M = M, a.N = N, a.K = K, a.O = O, a.Batch = Batch;
+        a.StrideA = StrideA, a.StrideB0 = StrideB0, a.StrideB1 = StrideB1, a.StrideC = StrideC;
+        a.BatchStrideA = BatchStrideA, a.BatchStrideB0 = BatchStrideB0, a.BatchStrideB1 = BatchStrideB1,
+        a.BatchStrideC = BatchStrideC;
+        a.scale        = ScaleOf(acc0_element_op);
+        return a;
+    }
+    Invoker MakeInvoker() const { return Invoker{instance_}; }
+    bool IsSupportedArgument(const Argument& a) const { return Supported(a, instance_) == CKX_OK; }
+    bool IsSupportedArgument(const BaseArgument* p) override
+    {
+        const auto* a = dynamic_cast<const Argument*>(p);
+        return a && IsSupportedArgument(*a);
+    }
+    std::unique_ptr<BaseArgument>
+    MakeArgumentPointer(const void* p_a, const void* p_b0, const void* p_b1, void* p_c, index_t M, index_t N,
+                        index_t K, index_t O, index_t Batch, index_t StrideA, index_t StrideB0, index_t StrideB1,
+                        index_t StrideC, index_t BatchStrideA, index_t BatchStrideB0, index_t BatchStrideB1,
+                        index_t BatchStrideC, Pass, Pass, Acc0ElementwiseOperation acc0_element_op, Pass, Pass) override
+    {
+        return std::make_unique<Argument>(MakeArgument(
+            static_cast<const half_t*>(p_a), static_cast<const half_t*>(p_b0), static_cast<const half_t*>(p_b1),
+            static_cast<half_t*>(p_c), M, N, K, O, Batch, StrideA, StrideB0, StrideB1, StrideC, BatchStrideA,
+            BatchStrideB0, BatchStrideB1, BatchStrideC, Pass{}, Pass{}, acc0_element_op));
+    }
+    std::unique_ptr<BaseInvoker> MakeInvokerPointer() override { return std::make_unique<Invoker>(instance_); }
+    std::string GetTypeString() const override
+    {
+        if(instance_ == CKX_INSTANCE_AUTO)
+            return "DeviceBatchedGemmSoftmaxGemm_f16_gmk_gnk_gno_gmo<auto>";
+        return ckx_instance_name(CKX_OP_BATCHED_GEMM_SOFTMAX_GEMM, instance_);
     }
     int instance_;
 };

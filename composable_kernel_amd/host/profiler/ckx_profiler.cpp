@@ -7,6 +7,7 @@
 //   ckx_profiler conv2d_fwd <dtype 1|3> <verify> <init> <log> <time>
 //                     N K C Y X Hi Wi Sy Sx Dy Dx LeftPy LeftPx RightPy RightPx [epilogue sg sr] [nrepeat]
 //   ckx_profiler batched_gemm_gemm <verify> <init> <log> <time> M N K O Batch [nrepeat]
+//   ckx_profiler batched_gemm_softmax_gemm <verify> <init> <log> <time> M N K O Batch [scale] [mask 0|1] [nrepeat]
 //   ckx_profiler conv_fwd_bias_relu | conv_fwd_bias_relu_add <dtype 1> <verify> <init> <log> <time>
 //                     N K C Y X Hi Wi Sy Sx Dy Dx LeftPy LeftPx RightPy RightPx [nrepeat]
 //                     (profiler/src/profile_conv_fwd_bias_relu[_add].cpp; fp16, NHWC/KYXC/NHWK)
@@ -584,6 +585,61 @@ int profile_gemm_gemm(int argc, char* argv[])
         dc, out_elems, flop, bytes, verify, time_kernel, nrepeat);
 }
 
+// batched_gemm_softmax_gemm <verify> <init> <log> <time> M N K O Batch [scale] [mask_out_upper_triangle] [nrepeat]
+template <bool Mask>
+int profile_gemm_softmax_gemm_t(bool verify, int init, bool time_kernel, int M, int N, int K, int O, int G, float scale,
+                                int nrepeat)
+{
+    using Scale = element_wise::Scale;
+    using Op = device::DeviceBatchedGemmSoftmaxGemm<Row, Col, Row, Row, half_t, half_t, half_t, half_t, Pass, Pass, Scale,
+                                                    Pass, Pass, Mask>;
+    std::vector<std::unique_ptr<Op>> ops;
+    for(int i = 0; i < ckx_num_instances(CKX_OP_BATCHED_GEMM_SOFTMAX_GEMM); ++i)
+        ops.push_back(std::make_unique<device::DeviceBatchedGemmSoftmaxGemmMfma<Scale, Mask>>(i));
+    std::vector<half_t> a((std::size_t)G * M * K), b0((std::size_t)G * N * K), b1((std::size_t)G * N * O);
+    if(init)
+    {
+        ckx::fill_uniform_f16(a, -1.0f, 1.0f, 0xC0FFEE + 7);
+        ckx::fill_uniform_f16(b0, -1.0f, 1.0f, 0xC0FFEE + 8);
+        ckx::fill_uniform_f16(b1, -1.0f, 1.0f, 0xC0FFEE + 9);
+    }
+    const std::size_t out_elems = (std::size_t)G * M * O;
+    ckx::DeviceMem da(a.size() * 2), db0(b0.size() * 2), db1(b1.size() * 2), dc(out_elems * 2);
+    da.ToDevice(a.data());
+    db0.ToDevice(b0.data());
+    db1.ToDevice(b1.data());
+    const double flop  = 2.0 * G * ((double)M * N * K + (double)M * N * O);
+    const double bytes = 2.0 * ((double)a.size() + b0.size() + b1.size() + out_elems);
+    return run_family<half_t>(
+        ops,
+        [&](Op& op) {
+            return op.MakeArgumentPointer(da.GetDeviceBuffer(), db0.GetDeviceBuffer(), db1.GetDeviceBuffer(),
+                                          dc.GetDeviceBuffer(), M, N, K, O, G, K, K, O, O, M * K, N * K, N * O, M * O,
+                                          Pass{}, Pass{}, Scale{scale}, Pass{}, Pass{});
+        },
+        dc, out_elems, flop, bytes, verify, time_kernel, nrepeat);
+}
+
+int profile_gemm_softmax_gemm(int argc, char* argv[])
+{
+    if(argc < 11)
+    {
+        std::printf("arg1: tensor operation (batched_gemm_softmax_gemm)\narg2: verification\narg3: initialization\n"
+                    "arg4: print tensor value\narg5: time kernel\narg6 to 10: M, N, K, O, Batch\n"
+                    "arg11: score scale (default 1/sqrt(K))\narg12: mask out the upper triangle (0 | 1)\nlast: nrepeat\n");
+        return 1;
+    }
+    const bool verify = std::atoi(argv[2]), time_kernel = std::atoi(argv[5]);
+    const int init = std::atoi(argv[3]);
+    const int M = std::atoi(argv[6]), N = std::atoi(argv[7]), K = std::atoi(argv[8]), O = std::atoi(argv[9]),
+              G = std::atoi(argv[10]);
+    const float scale = argc > 11 ? (float)std::atof(argv[11]) : 1.0f / std::sqrt((float)(K > 0 ? K : 1));
+    const bool mask   = argc > 12 && std::atoi(argv[12]);
+    const int nrepeat = argc > 13 ? std::atoi(argv[13]) : 10;
+    return mask ? profile_gemm_softmax_gemm_t<true>(verify, init, time_kernel, M, N, K, O, G, scale, nrepeat)
+                : profile_gemm_softmax_gemm_t<false>(verify, init, time_kernel, M, N, K, O, G, scale, nrepeat);
+}
+
 } // namespace
 
 int main(int argc, char* argv[])
@@ -596,6 +652,8 @@ int main(int argc, char* argv[])
             return profile_conv(argc, argv);
         if(argc >= 2 && std::strcmp(argv[1], "batched_gemm_gemm") == 0)
             return profile_gemm_gemm(argc, argv);
+        if(argc >= 2 && std::strcmp(argv[1], "batched_gemm_softmax_gemm") == 0)
+            return profile_gemm_softmax_gemm(argc, argv);
         if(argc >= 2 && std::strcmp(argv[1], "conv_fwd_bias_relu") == 0)
             return profile_conv_bias_relu(argc, argv, false);
         if(argc >= 2 && std::strcmp(argv[1], "conv_fwd_bias_relu_add") == 0)
@@ -609,6 +667,7 @@ int main(int argc, char* argv[])
         std::printf("arg1: tensor operation (gemm: GEMM\n"
                     "                        conv2d_fwd: NHWC/KYXC/NHWK forward convolution\n"
                     "                        batched_gemm_gemm: batched fused GEMM+GEMM\n"
+                    "                        batched_gemm_softmax_gemm: batched fused GEMM+Softmax+GEMM\n"
                     "                        conv_fwd_bias_relu: ForwardConvolution+Bias+ReLU\n"
                     "                        conv_fwd_bias_relu_add: ForwardConvolution+Bias+ReLU+Add\n"
                     "                        batched_gemm: Batched GEMM\n"

@@ -190,3 +190,18 @@ def test_profiler_gemm_other_layouts(tmp_path, layout):
     bad, max_err = lit.check_err_f16(c, lit.gemm_f16(a_st.T if layout >= 2 else a_st, b_st if layout in (0, 2) else b_st.T),
                                      1e-2, 1e-2)
     assert bad == 0, max_err
+
+
+@pytest.mark.parametrize("mask", [0, 1])
+def test_profiler_batched_gemm_softmax_gemm(tmp_path, mask):
+    M, N, K, O, G = 256, 384, 64, 64, 3
+    out, dump = _run("ckx_profiler", ["batched_gemm_softmax_gemm", 1, 1, 0, 1, M, N, K, O, G, 0.125, mask],
+                     "CKX_PROFILER_DUMP", tmp_path)
+    assert "Best Perf:" in out and "Error" not in out and "SoftmaxGemm" in out
+    a = uniform_f16((G, M, K), -1, 1, SEED + 7)
+    b0 = uniform_f16((G, N, K), -1, 1, SEED + 8)
+    b1 = uniform_f16((G, N, O), -1, 1, SEED + 9)
+    c = np.fromfile(dump, np.float16).reshape(G, M, O)
+    want = lit.batched_gemm_softmax_gemm_f16(a, b0.transpose(0, 2, 1), b1, 0.125, bool(mask))
+    bad, max_err = lit.check_err_f16(c, want, 1e-2, 1e-2)
+    assert bad == 0, max_err
