@@ -4,7 +4,7 @@
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--all] [--no-cpu]
 
 A "step" is one launch of the workload's kernel over synthetic inputs that are already resident
-in HBM. The default workload is BASELINE.json's configs[1], the fp16 GEMM at 4096^3 on which the
+in HBM. The default workload is the fp16 GEMM at 4096^3 on which the
 metric (TFLOP/s and fraction of the dense fp16 MFMA peak) is quoted; the int8 half of the metric
 (4096^3 requant GEMM, TOP/s) and every other config are measured too and attached under "also".
 Prints ONE JSON line on stdout.
@@ -291,7 +291,7 @@ def main():
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this hot path is a single-GPU kernel library; run with --gpus 1 "
-              "(sharding is over independent output tiles, see DESIGN.md)", file=sys.stderr)
+              "(a larger problem would shard over independent output tiles, one launch per GPU)", file=sys.stderr)
         sys.exit(2)
 
     import torch

@@ -2,7 +2,7 @@
 
 Parameter sets follow the reference's test/convnd_fwd/conv2d_fwd.cpp:104-115,187-266
 (default 3x3 stride 2 dilation 2 pad 2; 1x1 stride 1 pad 0; 1x1 stride 2 pad 0) and its golden
-vectors (test/reference_conv_fwd/reference_conv_fwd.cpp:94-154), plus BASELINE config 4's
+vectors (test/reference_conv_fwd/reference_conv_fwd.cpp:94-154), plus benchmark configuration 4's
 ResNet-50 layers on a reduced batch (full batch through the im2col/BLAS form).
 int8 is bit-exact (PassThrough keeps the low byte, as the reference's int8 conv does);
 fp16 within rtol = atol = 1e-2.
@@ -85,7 +85,7 @@ def test_conv2d_reference_golden_vectors_fp16():
 
 
 RESNET = [
-    # BASELINE config 4 (C, K, filter, HW, stride, pad)
+    # benchmark configuration 4 (C, K, filter, HW, stride, pad)
     (64, 64, 3, 56, 1, 1),
     (256, 512, 1, 56, 2, 0),
     (512, 512, 3, 7, 1, 1),

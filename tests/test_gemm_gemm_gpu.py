@@ -42,7 +42,7 @@ def test_gemm_gemm_closed_form():
 
 
 def test_gemm_gemm_config5():
-    """BASELINE config 5: batch 64, (512x64)(64x512)(512x64), U[-0.5, 0.5]."""
+    """Benchmark configuration 5: batch 64, (512x64)(64x512)(512x64), U[-0.5, 0.5]."""
     import gpu_util
     G, M, N, K, O = 64, 512, 512, 64, 64
     a = uniform_f16((G, M, K), -0.5, 0.5, 910)

@@ -35,7 +35,7 @@ def _assert_f16_close(out, ref, rtol=RTOL, atol=ATOL):
 
 @pytest.mark.parametrize("epi", list(EPILOGUES))
 def test_int8_gemm_config1_1024_cubed_bit_exact(epi):
-    """BASELINE config 1: M=N=K=1024, int8 in [-5,5], literal ReferenceGemm oracle."""
+    """Benchmark configuration 1: M=N=K=1024, int8 in [-5,5], literal ReferenceGemm oracle."""
     import gpu_util
     c_op, kind, sg, sr = EPILOGUES[epi]
     a = uniform_int8((1024, 1024), -5, 5, 0xC0FFEE)
@@ -165,7 +165,7 @@ def test_fp16_gemm_closed_forms():
 
 
 def test_fp16_gemm_config2_4096_cubed_within_tolerance():
-    """BASELINE config 2. Full output against the fp32 BLAS form, a sample of rows against the
+    """Benchmark configuration 2 (fp16, 4096^3). Full output against the fp32 BLAS form, a sample of rows against the
     literal sequential-k oracle."""
     import gpu_util
     M = N = K = 4096
@@ -196,7 +196,7 @@ def test_int8_gemm_4096_cubed_bit_exact():
 @pytest.mark.parametrize("M", [1, 16, 128, 4096])
 @pytest.mark.parametrize("NK", [(11008, 4096), (4096, 11008)])
 def test_int8_gemm_config3_llm_shapes_bit_exact(M, NK):
-    """BASELINE config 3: tokens x N x K, int8 in [-8,8], scales 0.02 / 0.4, rounded mode."""
+    """Benchmark configuration 3: tokens x N x K, int8 in [-8,8], scales 0.02 / 0.4, rounded mode."""
     import gpu_util
     N, K = NK
     a = uniform_int8((M, K), -8, 8, 61 + M)

@@ -126,7 +126,7 @@ def test_gemm_softmax_gemm_padded_strides_and_scale_zero():
 
 @pytest.mark.parametrize("mask", [False, True])
 def test_gemm_softmax_gemm_config5_shape(mask):
-    """BASELINE config 5's shapes with the softmax in between: batch 64, 512 x 512 scores, K = O = 64."""
+    """Benchmark configuration 5's shapes with the softmax in between: batch 64, 512 x 512 scores, K = O = 64."""
     G, M, N, K, O = 64, 512, 512, 64, 64
     a = uniform_f16((G, M, K), -1, 1, 1910)
     b0_gnk = uniform_f16((G, N, K), -1, 1, 1911)
