@@ -18,8 +18,8 @@
 // with the softmax along N in one pass over N (running row maximum and running sum): a step's
 // scores become p = exp(s - running max), the output accumulators and the running sum are rescaled
 // whenever the maximum grows, and the division by the sum happens once at the end. A row's 128
-// scores of a step sit in four lanes (l%16 = row, l/16 = q), 32 each: the row maximum and the final
-// sum cross those lanes with v_permlane16_swap / v_permlane32_swap. Columns past N and, with the
+// scores of a step sit in four lanes (l%16 = row, l/16 = q), 32 each: the row maximum crosses those
+// lanes with v_permlane16_swap / v_permlane32_swap, and so does the final sum. Columns past N and, with the
 // upper-triangle mask, columns n > m count as -infinity; masked-out steps are skipped altogether.
 #pragma once
 
@@ -48,15 +48,6 @@ struct GemmGemmArgs
 };
 
 // maximum / sum over the four lanes l, l^16, l^32, l^48 (every one of them gets the result)
-__device__ __forceinline__ float quad_rows_max(float x)
-{
-    auto a = __builtin_amdgcn_permlane16_swap(__builtin_bit_cast(uint32_t, x), __builtin_bit_cast(uint32_t, x), false, false);
-    const uint32_t a0 = a[0], a1 = a[1];
-    x      = __builtin_fmaxf(__builtin_bit_cast(float, a0), __builtin_bit_cast(float, a1));
-    auto b = __builtin_amdgcn_permlane32_swap(__builtin_bit_cast(uint32_t, x), __builtin_bit_cast(uint32_t, x), false, false);
-    const uint32_t b0 = b[0], b1 = b[1];
-    return __builtin_fmaxf(__builtin_bit_cast(float, b0), __builtin_bit_cast(float, b1));
-}
 __device__ __forceinline__ float quad_rows_sum(float x)
 {
     auto a = __builtin_amdgcn_permlane16_swap(__builtin_bit_cast(uint32_t, x), __builtin_bit_cast(uint32_t, x), false, false);
@@ -65,6 +56,15 @@ __device__ __forceinline__ float quad_rows_sum(float x)
     auto b = __builtin_amdgcn_permlane32_swap(__builtin_bit_cast(uint32_t, x), __builtin_bit_cast(uint32_t, x), false, false);
     const uint32_t b0 = b[0], b1 = b[1];
     return __builtin_bit_cast(float, b0) + __builtin_bit_cast(float, b1);
+}
+__device__ __forceinline__ float quad_rows_max(float x)
+{
+    auto a = __builtin_amdgcn_permlane16_swap(__builtin_bit_cast(uint32_t, x), __builtin_bit_cast(uint32_t, x), false, false);
+    const uint32_t a0 = a[0], a1 = a[1];
+    x      = __builtin_fmaxf(__builtin_bit_cast(float, a0), __builtin_bit_cast(float, a1));
+    auto b = __builtin_amdgcn_permlane32_swap(__builtin_bit_cast(uint32_t, x), __builtin_bit_cast(uint32_t, x), false, false);
+    const uint32_t b0 = b[0], b1 = b[1];
+    return __builtin_fmaxf(__builtin_bit_cast(float, b0), __builtin_bit_cast(float, b1));
 }
 
 // KS  k-steps of gemm0 (K padded to 32*KS), OG  64-column groups of the output (O padded to 64*OG),
@@ -215,6 +215,18 @@ __global__ __launch_bounds__(NW * 64)
 #pragma unroll
     for(int mt = 0; mt < MT; ++mt)
         row_max[mt] = ninf, row_sum[mt] = 0.0f;
+    // (never exactly 0: a masked score is -inf, and -inf * 0 would be a NaN; with the smallest normal number
+    // instead, scale 0 still turns every unmasked score into 0)
+    const float c2 = __builtin_fmaxf(__builtin_fabsf(p.scale) * kLog2e, 1.17549435e-38f);
+    if(SOFTMAX && p.scale < 0.0f)
+    {
+        // scores = scale * (A * B0) = |scale| * ((-A) * B0): flip the sign bits of the A fragments once
+#pragma unroll
+        for(int mt = 0; mt < MT; ++mt)
+#pragma unroll
+            for(int ks = 0; ks < KS; ++ks)
+                af[mt][ks] = __builtin_bit_cast(f16x8, __builtin_bit_cast(i32x4, af[mt][ks]) ^ (int)0x80008000);
+    }
     // with the upper-triangle mask, columns past the slab's last row are masked for every row of it
     const int n_end = (SOFTMAX && p.mask_upper && m0 + Cfg::BM < p.N) ? m0 + Cfg::BM : p.N;
 
@@ -249,10 +261,10 @@ __global__ __launch_bounds__(NW * 64)
         if constexpr(SOFTMAX)
         {
             // s[mt][t][j] is the score of row m0 + wave*16*MT + 16*mt + fr, column n0 + 32*(t/2) + 8q + 4*(t%2) + j.
-            // Everything below works on x = score * scale * log2(e), so that exp(score - max) is one
-            // v_exp_f32 of a difference.
-            const float c2 = p.scale * kLog2e;
-            // does this step hold masked columns for any row of this wave? (wave-uniform: the plain path
+            // The running maximum is kept as x = score * |scale| * log2(e), so that exp(score - max) is one
+            // fused multiply-add and one v_exp_f32 (a negative scale has been moved into A's sign above, which
+            // lets the maximum be taken over the raw scores).
+            // Does this step hold masked columns for any row of this wave? (wave-uniform: the plain path
             // skips the per-element compare and select)
             const int wave_m0    = m0 + wave * 16 * MT;
             const bool step_mask = n0 + Cfg::BNC > p.N || (p.mask_upper && n0 + Cfg::BNC > wave_m0 + 1);
@@ -261,7 +273,6 @@ __global__ __launch_bounds__(NW * 64)
             {
                 const int m     = wave_m0 + mt * 16 + fr;
                 const int n_lim = (p.mask_upper && m + 1 < p.N) ? m + 1 : p.N; // columns >= n_lim are masked
-                float mx = ninf;
                 if(step_mask)
                 {
 #pragma unroll
@@ -270,31 +281,27 @@ __global__ __launch_bounds__(NW * 64)
                         for(int j = 0; j < 4; ++j)
                         {
                             const int n = n0 + 32 * (t >> 1) + 8 * q + 4 * (t & 1) + j;
-                            s[mt][t][j] = n < n_lim ? s[mt][t][j] * c2 : ninf;
+                            s[mt][t][j] = n < n_lim ? s[mt][t][j] : ninf;
                         }
                 }
-                else
-                {
-#pragma unroll
-                    for(int t = 0; t < 8; ++t)
-                        s[mt][t] = s[mt][t] * c2;
-                }
+                float mx = ninf;
 #pragma unroll
                 for(int t = 0; t < 8; ++t)
                     mx = __builtin_fmaxf(__builtin_fmaxf(mx, __builtin_fmaxf(s[mt][t][0], s[mt][t][1])),
                                          __builtin_fmaxf(s[mt][t][2], s[mt][t][3]));
-                mx                 = quad_rows_max(mx);
-                const float m_new  = __builtin_fmaxf(row_max[mt], mx);
+                mx = quad_rows_max(mx);
+                // (c2 > 0: the maximum commutes with the scaling, and -inf stays -inf)
+                const float m_new  = __builtin_fmaxf(row_max[mt], mx * c2);
                 const float m_safe = m_new == ninf ? 0.0f : m_new; // a row with nothing unmasked yet: every p is 0
                 const float corr   = __builtin_amdgcn_exp2f(row_max[mt] - m_safe);
                 row_max[mt]        = m_new;
-                float part         = 0.0f;
+                float part = 0.0f;
 #pragma unroll
                 for(int t = 0; t < 8; ++t)
 #pragma unroll
                     for(int j = 0; j < 4; ++j)
                     {
-                        const float e = __builtin_amdgcn_exp2f(s[mt][t][j] - m_safe);
+                        const float e = __builtin_amdgcn_exp2f(__builtin_fmaf(s[mt][t][j], c2, -m_safe));
                         s[mt][t][j]   = e;
                         part += e;
                     }

@@ -112,6 +112,19 @@ def test_gemm_softmax_gemm_running_maximum_is_rescaled():
         np.testing.assert_array_equal(out[0], np.broadcast_to(b1[0, int(np.argmax(b0[0, :, 0]))], (M, O)))
 
 
+def test_gemm_softmax_gemm_negative_scale():
+    """A negative scale turns the softmax towards the SMALLEST raw score (the kernel moves the sign into A)."""
+    G, M, N, K, O = 2, 96, 300, 32, 32
+    a = uniform_f16((G, M, K), -1, 1, 21)
+    b0_gnk = uniform_f16((G, N, K), -1, 1, 22)
+    b1 = uniform_f16((G, N, O), -1, 1, 23)
+    for mask in (False, True):
+        out = _run(a, b0_gnk, b1, -0.7, mask)
+        _close(out, lit.batched_gemm_softmax_gemm_f16(a, b0_gnk.transpose(0, 2, 1), b1, -0.7, mask))
+        # same as a positive scale on the negated A
+        np.testing.assert_array_equal(out.view(np.uint16), _run(-a, b0_gnk, b1, 0.7, mask).view(np.uint16))
+
+
 def test_gemm_softmax_gemm_padded_strides_and_scale_zero():
     G, M, N, K, O = 3, 72, 200, 64, 48
     a = uniform_f16((G, M, K), -1, 1, 11)
