@@ -438,20 +438,22 @@ int run_gemm(int dt, const void* a, const void* b, void* c, int M, int N, int K,
 // ---------------------------------------------------------- input-patch conv kernel
 const char* const kPatchName = "MI355X_Mfma16_Patch<4 rows x 56, 3x3, C 64, K 64, waves 2x2>";
 
-// shapes the input-patch kernel covers (one instantiation: 3x3 taps, Wo = 56)
+// shapes the input-patch kernel covers (one instantiation per data type: 3x3 taps, Wo = 56)
 bool conv_patch_applicable(int op, const ckx_conv2d_desc* d, int epi)
 {
-    return op == CKX_OP_CONV2D_FWD_F16 &&
-           (epi == CKX_EPI_PASSTHROUGH || epi == CKX_EPI_ADD_RELU || epi == CKX_EPI_ADD_RELU_ADD) && d->C == 64 && d->K == 64 && d->Y == 3 &&
+    const bool epi_ok = op == CKX_OP_CONV2D_FWD_F16
+                            ? (epi == CKX_EPI_PASSTHROUGH || epi == CKX_EPI_ADD_RELU || epi == CKX_EPI_ADD_RELU_ADD)
+                            : (epi == CKX_EPI_PASSTHROUGH || epi == CKX_EPI_REQUANT_CK || epi == CKX_EPI_REQUANT_RND);
+    return (op == CKX_OP_CONV2D_FWD_F16 || op == CKX_OP_CONV2D_FWD_I8) && epi_ok && d->C == 64 && d->K == 64 && d->Y == 3 &&
            d->X == 3 && d->stride_h == 1 && d->stride_w == 1 && d->dilation_h == 1 && d->dilation_w == 1 &&
            d->Wo == 56 && d->Ho >= 1 && d->N >= 1 && d->pad_left <= 2 && d->pad_top <= 2;
 }
 
-template <bool FUSED>
+template <int DT, bool FUSED>
 hipError_t launch_conv_patch(const ckx::ConvPatchArgs& a, hipStream_t s)
 {
-    using T    = ckx::ConvPatch<7, 3, 3, FUSED>;
-    auto* kern = &ckx::conv_patch_kernel<7, 3, 3, FUSED>;
+    using T    = ckx::ConvPatch<DT, 7, 3, 3, FUSED>;
+    auto* kern = &ckx::conv_patch_kernel<DT, 7, 3, 3, FUSED>;
     static std::once_flag once;
     static hipError_t attr_err = hipSuccess;
     std::call_once(once, [&] {
@@ -472,7 +474,7 @@ int check_conv(int op, const ckx_conv2d_desc* d, int epi, int instance)
     if(op != CKX_OP_CONV2D_FWD_I8 && op != CKX_OP_CONV2D_FWD_F16)
         return fail(CKX_INVALID_VALUE, "not a conv operator family");
     const int es = op == CKX_OP_CONV2D_FWD_I8 ? 1 : 2;
-    if(instance != CKX_INSTANCE_AUTO && (instance < 0 || instance >= kNumTiles + (es == 2 ? 1 : 0)))
+    if(instance != CKX_INSTANCE_AUTO && (instance < 0 || instance > kNumTiles))
         return fail(CKX_INVALID_VALUE, "no such instance");
     if(epi < CKX_EPI_PASSTHROUGH || epi > CKX_EPI_CSHUFFLE_ADD_RELU || !epilogue_fits_dtype(es, epi) ||
        epi == CKX_EPI_CSHUFFLE_ADD_RELU)
@@ -501,7 +503,7 @@ int check_conv(int op, const ckx_conv2d_desc* d, int epi, int instance)
        (long)d->N * d->Ho * d->Wo >= (1l << 31))
         return fail(CKX_UNSUPPORTED, "tensors of 2 GiB or more are not addressed");
     if(instance == kNumTiles && !conv_patch_applicable(op, d, epi))
-        return fail(CKX_UNSUPPORTED, "the input-patch instance covers fp16 3x3 stride-1 layers with C = K = 64, Wo = 56");
+        return fail(CKX_UNSUPPORTED, "the input-patch instance covers 3x3 stride-1 layers with C = K = 64, Wo = 56");
     return CKX_OK;
 }
 
@@ -552,8 +554,10 @@ int run_conv(int op, const void* in, const void* wei, void* out, const ckx_conv2
         a.div_wo = make_magic((uint32_t)d->Wo);
         a.epi    = epi;
         a.bias = dops.d0, a.resi = epi == CKX_EPI_ADD_RELU_ADD ? dops.d1 : nullptr;
-        hipError_t e = epi == CKX_EPI_PASSTHROUGH ? launch_conv_patch<false>(a, (hipStream_t)stream)
-                                                  : launch_conv_patch<true>(a, (hipStream_t)stream);
+        a.scale_gemm = sg, a.scale_relu = sr;
+        hipError_t e = es == 1                     ? launch_conv_patch<ckx::DT_I8, false>(a, (hipStream_t)stream)
+                       : epi == CKX_EPI_PASSTHROUGH ? launch_conv_patch<ckx::DT_F16, false>(a, (hipStream_t)stream)
+                                                    : launch_conv_patch<ckx::DT_F16, true>(a, (hipStream_t)stream);
         return e == hipSuccess ? CKX_OK : hip_fail(e, kPatchName);
     }
     const Plan pl = make_plan(M, N, K * es, instance, ws ? ws_bytes : 0);
@@ -605,9 +609,9 @@ int ckx_num_instances(int op)
 {
     if(op == CKX_OP_GEMM_I8 || op == CKX_OP_GEMM_F16 || op == CKX_OP_GEMM_BF16)
         return kNumGemmInsts;
-    if(op == CKX_OP_CONV2D_FWD_I8 || op == CKX_OP_GEMM_SPLITK)
+    if(op == CKX_OP_GEMM_SPLITK)
         return kNumTiles;
-    if(op == CKX_OP_CONV2D_FWD_F16)
+    if(op == CKX_OP_CONV2D_FWD_F16 || op == CKX_OP_CONV2D_FWD_I8)
         return kNumTiles + 1; // + the input-patch kernel
     if(op == CKX_OP_BATCHED_GEMM_GEMM || op == CKX_OP_BATCHED_GEMM_SOFTMAX_GEMM)
         return ckx::kNumGemmGemmInstances;
@@ -623,7 +627,7 @@ const char* ckx_instance_name(int op, int instance)
     s = std::string(fam) + "<" +
         (op == CKX_OP_BATCHED_GEMM_GEMM || op == CKX_OP_BATCHED_GEMM_SOFTMAX_GEMM
              ? ckx::gemm_gemm_instance_name(instance)
-         : op == CKX_OP_CONV2D_FWD_F16 && instance == kNumTiles
+         : (op == CKX_OP_CONV2D_FWD_F16 || op == CKX_OP_CONV2D_FWD_I8) && instance == kNumTiles
              ? kPatchName
              : instance >= kNumTiles ? kSkinny[instance - kNumTiles].name : kTiles[instance].name) +
         ">";

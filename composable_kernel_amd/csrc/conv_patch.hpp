@@ -1,23 +1,25 @@
-// Input-patch conv2d forward for gfx950, fp16, NHWC / KYXC / NHWK: the 3x3-class layers with few
+// Input-patch conv2d forward for gfx950, fp16 and int8, NHWC / KYXC / NHWK: the 3x3-class layers with few
 // channels (ResNet conv2_x: C = 64, K = 64, 56 x 56), where the implicit-GEMM tile kernel re-reads
 // every input pixel once per filter tap out of L2 and is bound by that.
 //
 // Takes the place of the same reference kernel as the tile kernel
 // (DeviceConv2dFwdXdl_Input_N_Hi_Wi_C_Weight_K_Y_X_C_Output_N_Ho_Wo_K,
 // device_conv2d_fwd_xdl_nhwc_kyxc_nhwk.hpp:57-720) for the shapes it covers:
-//   C * 2 bytes = 128 (one pixel = one 128-byte LDS row = one tap's K tile), K = 64,
+//   C = 64 (one pixel = one LDS row of 128 bytes fp16 / 64 bytes int8 = one tap's K tile), K = 64,
 //   Y x X taps, stride 1, dilation 1, Wo = 8 * MTW <= 56, Wo + X - 1 <= 64.
+// int8: one pixel is exactly one MFMA k-step (16x16x64), half the LDS reads and MFMAs per tap of fp16;
+// the epilogue is the requant / PassThrough family of the GEMM, 8 consecutive int8 channels per lane.
 //
 //  * A workgroup (4 waves) owns whole images and walks them in bands of 4 output rows. The
-//    input rows a band needs (4 + Y - 1) live in LDS in a RING of 10 rows x 64 pixels x 128 B;
+//    input rows a band needs (4 + Y - 1) live in LDS in a RING of 10 rows x 64 pixels x 128 (64) B;
 //    while band b is multiplied, the 4 new rows of band b + 1 are fetched into the ring slots
 //    that band b - 1 has finished with. Every input pixel is read from memory ONCE.
 //  * All Y * X * 64 weight rows (72 KB) are LDS-resident for the life of the workgroup.
 //  * The A fragment of tap (y, x) for 16 consecutive output pixels is the patch shifted by
 //    (y rows, x pixels): the same 128-byte rows, another base address. A lane keeps one
 //    precomputed byte offset per (M tile, x) and one per (M tile, y): a fragment address is one add.
-//  * 16-byte chunks are swizzled by the patch COLUMN (chunk ^ (col & 7)), so the 16 pixels of a
-//    fragment read spread over the banks exactly as the 16 rows of a GEMM fragment do.
+//  * 16-byte chunks are swizzled by the patch COLUMN (fp16: chunk ^ (col & 7); int8, 4 chunks per pixel:
+//    chunk ^ ((col >> 2) & 3)), so the 16 pixels of a fragment read spread over all banks.
 //  * 2 x 2 waves: a wave multiplies 16 * MTW pixels x 32 output channels; D^T = B_frag x A_frag with
 //    the weight rows permuted in LDS so that a lane ends up with 8 consecutive channels of one
 //    pixel: one 16-byte store, no trip through LDS.
@@ -37,20 +39,29 @@ struct ConvPatchArgs
     int pT, pL;
     int nbands; // ceil(Ho / 4)
     MagicDiv div_wo;
-    int epi; // EPI_PASSTHROUGH, EPI_ADD_RELU, EPI_ADD_RELU_ADD
+    int epi; // fp16: EPI_PASSTHROUGH, EPI_ADD_RELU, EPI_ADD_RELU_ADD; int8: EPI_PASSTHROUGH, EPI_REQUANT_CK, EPI_REQUANT_RND
     const void* bias; // [64] fp16
     const void* resi; // NHWK fp16
+    float scale_gemm, scale_relu; // int8 requant epilogues
 };
 
 // FUSED: the add / ReLU epilogues (bias, residual) are compiled in; the plain instantiation keeps
 // their registers free
-template <int MTW, int Y, int X, bool FUSED>
+template <int DT, int MTW, int Y, int X, bool FUSED>
 struct ConvPatch
 {
+    static constexpr int ES     = DT == DT_I8 ? 1 : 2;
     static constexpr int TH     = 4;                // output rows per band
-    static constexpr int RING   = 2 * TH + 2;       // ring rows (Y <= 3)
+    // bands of input rows in flight ahead of the band being multiplied. fp16 rows fill the LDS with one; int8
+    // rows are half as large, and three bands of head start take the HBM latency out of the band loop (one
+    // image per workgroup at a time: nothing else would hide it)
+    static constexpr int AHEAD  = ES == 1 ? 3 : 1;
+    static constexpr int RING   = (AHEAD + 1) * TH + 2; // ring rows (Y <= 3)
     static constexpr int PITCH  = 64;               // pixels per ring row
-    static constexpr int PXB    = 128;              // bytes per pixel (C * 2)
+    static constexpr int PXB    = 64 * ES;          // bytes per pixel (C * element size)
+    static constexpr int CPP    = PXB / 16;         // 16-byte chunks per pixel (8 / 4)
+    static constexpr int PPI    = 64 / CPP;         // pixels (or weight rows) covered by one wave-wide direct load
+    static constexpr int KSP    = PXB / 64;         // MFMA k-steps per tap (2 / 1)
     static constexpr int KO     = 64;               // output channels
     static constexpr int TAPS   = Y * X;
     static constexpr int RING_BYTES = RING * PITCH * PXB;
@@ -59,6 +70,10 @@ struct ConvPatch
     static constexpr int NT         = 256;
     static constexpr int NEED_ROWS  = TH + Y - 1;   // input rows of one band
     static_assert(Y >= 1 && Y <= 3 && X >= 1 && X <= 3 && MTW >= 1 && MTW <= 7, "covered shapes");
+    static_assert(DT == DT_F16 || (DT == DT_I8 && !FUSED), "fp16 (optionally with the add / ReLU epilogues) or int8");
+    using acc_t = typename std::conditional<DT == DT_I8, i32x4, f32x4>::type;
+    // swizzle key of a pixel column / weight row: the 16 rows of a fragment read must land on distinct banks
+    __device__ static __forceinline__ uint32_t key(uint32_t r) { return CPP == 8 ? (r & 7u) : ((r >> 2) & 3u); }
 
     __device__ static __forceinline__ void run(const ConvPatchArgs& p, uint8_t* smem)
     {
@@ -74,15 +89,16 @@ struct ConvPatch
 
         // ---- weights: LDS row tap*64 + r holds output channel w_row_to_ch(r), swizzled by r & 7
         {
-            const uint32_t rl  = (uint32_t)(lane >> 3);  // row within the 8-row block = its swizzle key
-            const uint32_t pos = (uint32_t)(lane & 7);
-            for(int k = wave; k < TAPS * 8; k += 4)
+            constexpr int BPT  = KO / PPI;                 // wave-wide loads per tap (8 / 4)
+            const uint32_t rl  = (uint32_t)(lane / CPP);   // row within the block of PPI rows
+            const uint32_t pos = (uint32_t)(lane % CPP);
+            for(int k = wave; k < TAPS * BPT; k += 4)
             {
-                const uint32_t tap = (uint32_t)k >> 3;
-                const uint32_t r   = (((uint32_t)k & 7u) << 3) + rl; // 0..63
+                const uint32_t tap = (uint32_t)k / BPT;
+                const uint32_t r   = ((uint32_t)k % BPT) * PPI + rl; // 0..63
                 // within a 32-row group, row 16j + 4q + i holds channel 8q + 4j + i
                 const uint32_t ch = (r & ~31u) | (((r >> 2) & 3u) << 3) | (((r >> 4) & 1u) << 2) | (r & 3u);
-                const uint32_t voff = (ch * TAPS + tap) * PXB + ((pos ^ rl) << 4);
+                const uint32_t voff = (ch * TAPS + tap) * PXB + ((pos ^ key(r)) << 4);
                 __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_wei, (lds_ptr_t)(wlds + (size_t)k * 1024), 16, voff, 0,
                                                          0, 0);
             }
@@ -99,12 +115,12 @@ struct ConvPatch
             const uint32_t r = magic_div(q, p.div_wo);
             const uint32_t w = q - r * (uint32_t)p.Wo;
             rout[t]          = r;
-            ooff[t]          = ((r * (uint32_t)p.Wo + w) * KO + (uint32_t)(32 * wn) + 8u * fq) * 2u;
+            ooff[t]          = ((r * (uint32_t)p.Wo + w) * KO + (uint32_t)(32 * wn) + 8u * fq) * ES;
 #pragma unroll
             for(int x = 0; x < X; ++x)
             {
                 const uint32_t cc = w + (uint32_t)x;
-                coff[t][x]        = cc * PXB + ((fq ^ (cc & 7u)) << 4);
+                coff[t][x]        = cc * PXB + ((fq ^ key(cc)) << 4);
             }
         }
         // fused add / ReLU epilogues: the lane's 8 bias values once, its residual values band by band
@@ -120,26 +136,27 @@ struct ConvPatch
         uint32_t boff[2]; // weight fragment of n-tile j, k-step 0, tap 0
 #pragma unroll
         for(int j = 0; j < 2; ++j)
-            boff[j] = (uint32_t)(32 * wn + 16 * j + (int)frow) * PXB + ((fq ^ (frow & 7u)) << 4);
+            boff[j] = (uint32_t)(32 * wn + 16 * j + (int)frow) * PXB + ((fq ^ key(frow)) << 4);
 
-        // ---- input rows -> ring: block k = (row j, 8-pixel column group cg) ------------------
-        // lane: patch column 8*cg + lane/8, LDS chunk position lane%8 <- global chunk pos ^ (col & 7)
+        // ---- input rows -> ring: block k = (row j, PPI-pixel column group cg) ------------------
+        // lane: patch column PPI*cg + lane/CPP, LDS chunk position lane%CPP <- global chunk pos ^ key(col)
+        constexpr int BPR = PITCH / PPI; // blocks per ring row (8 / 4)
         auto load_block = [&](int n, int j, int cg) {
-            const int cc = 8 * cg + (lane >> 3);
+            const int cc = PPI * cg + lane / CPP;
             const int wi = cc - p.pL, hi = j - p.pT;
             const bool ok = (uint32_t)hi < (uint32_t)p.Hi && (uint32_t)wi < (uint32_t)p.Wi && n < p.N;
-            const uint32_t chunk = (uint32_t)(lane & 7) ^ (uint32_t)(lane >> 3);
+            const uint32_t chunk = (uint32_t)(lane % CPP) ^ key((uint32_t)cc);
             const uint32_t voff =
                 ((uint32_t)((n * p.Hi + hi) * p.Wi + wi) * PXB + (chunk << 4)) | (ok ? 0u : kOutOfRange);
             const int slot = j % RING;
-            __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_in, (lds_ptr_t)(ring + (size_t)(slot * PITCH + 8 * cg) * PXB),
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_in, (lds_ptr_t)(ring + (size_t)(slot * PITCH + PPI * cg) * PXB),
                                                      16, voff, 0, 0, 0);
         };
 
-        f32x4 acc[MTW][2];
+        acc_t acc[MTW][2];
 #pragma unroll
         for(int t = 0; t < MTW; ++t)
-            acc[t][0] = acc[t][1] = f32x4{0, 0, 0, 0};
+            acc[t][0] = acc[t][1] = acc_t{0, 0, 0, 0};
 
         auto barrier = [&]() {
             __builtin_amdgcn_s_barrier();
@@ -151,8 +168,8 @@ struct ConvPatch
         for(int n = (int)blockIdx.x; n < p.N; n += (int)gridDim.x)
         {
             // rows of the first band (every wave has passed the barrier that ended the previous image)
-            for(int k = wave; k < NEED_ROWS * 8; k += 4)
-                load_block(n, k >> 3, k & 7);
+            for(int k = wave; k < (NEED_ROWS + TH * (AHEAD - 1)) * BPR; k += 4)
+                load_block(n, k / BPR, k % BPR);
             asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
             barrier();
 
@@ -168,10 +185,10 @@ struct ConvPatch
                             roff[t][y] = (rout[t] + (uint32_t)y) * (PITCH * PXB);
                 }
 
-                // fragment r of k-step s = (tap, half): r = 0, 1 the two weight tiles, then the M tiles
-                // in the order in which the MFMAs use them
+                // fragment r of k-step s = (tap, half) (int8: s = tap): r = 0, 1 the two weight tiles, then the
+                // M tiles in the order in which the MFMAs use them
                 auto read_one = [&](int s, int r) {
-                    const int buf = s & 1, tap = s >> 1, ks = s & 1, y = tap / X, x = tap % X;
+                    const int buf = s & 1, tap = s / KSP, ks = s % KSP, y = tap / X, x = tap % X;
                     if(r < 2)
                         bf[buf][r] = *reinterpret_cast<const i32x4*>(wlds + tap * (KO * PXB) +
                                                                      (boff[r] ^ (uint32_t)(ks * 64)));
@@ -183,9 +200,14 @@ struct ConvPatch
                     const int buf = s & 1;
 #pragma unroll
                     for(int j = 0; j < 2; ++j)
-                        acc[t][j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, bf[buf][j]),
-                                                                        __builtin_bit_cast(f16x8, af[buf][t]),
-                                                                        acc[t][j], 0, 0, 0);
+                    {
+                        if constexpr(DT == DT_I8)
+                            acc[t][j] = __builtin_amdgcn_mfma_i32_16x16x64_i8(bf[buf][j], af[buf][t], acc[t][j], 0, 0, 0);
+                        else
+                            acc[t][j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, bf[buf][j]),
+                                                                            __builtin_bit_cast(f16x8, af[buf][t]),
+                                                                            acc[t][j], 0, 0, 0);
+                    }
                 };
 
                 if(b == 0)
@@ -211,32 +233,37 @@ struct ConvPatch
                 // rows] [the 2 MFMAs of one M tile]. With one wave per SIMD nothing else hides the
                 // issue slots of the reads, so they go between the MFMAs.
                 constexpr int NR = MTW + 2, RG = MTW > 2 ? MTW - 2 : MTW;
+                constexpr int NS = KSP * TAPS;           // k-steps of a band
+                constexpr int NBLK = TH * BPR / 4;       // direct loads per wave for the next band's rows
+                static_assert(NBLK <= NS, "one direct load per k-step");
 #pragma unroll
-                for(int s = 0; s < 2 * TAPS; ++s)
+                for(int s = 0; s < NS; ++s)
                 {
 #pragma unroll
                     for(int g = 0; g < MTW; ++g)
                     {
-                        if(s + 1 < 2 * TAPS)
+                        if(s + 1 < NS)
                         {
 #pragma unroll
                             for(int r = (g < RG ? g : RG) * NR / RG; r < (g + 1 < RG ? g + 1 : RG) * NR / RG; ++r)
                                 read_one(s + 1, r);
                         }
-                        // the 4 new input rows of the next band: 32 blocks, 8 per wave, one per k-step
-                        if(s < 8 && g == MTW - 1)
+                        // the 4 new input rows of the next band: TH * BPR blocks, NBLK per wave, one per k-step
+                        if(s < NBLK && g == MTW - 1)
                         {
                             const int k = wave + 4 * s;
-                            load_block(n, j0 + NEED_ROWS + (k >> 3), k & 7);
+                            load_block(n, j0 + NEED_ROWS + TH * (AHEAD - 1) + k / BPR, k % BPR);
                         }
                         mfma_pair(s, g);
                         __builtin_amdgcn_sched_barrier(0);
                     }
                 }
 
-                // the next band's rows have landed (this wave's share) before the stores go out:
-                // stores share the counter with loads and are not ordered against them
-                asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+                // the next band's rows have landed (this wave's share) before the stores go out. Loads retire in
+                // order among themselves, so "at most the loads of the AHEAD - 1 later bands outstanding" implies
+                // it; stores share the counter and are not ordered against loads, which can only make this
+                // wait longer, never too short
+                asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" ::"n"((AHEAD - 1) * NBLK) : "memory");
                 // every wave is through with this band's rows, and the next band's rows are visible:
                 // its first fragments are read under the epilogue
                 barrier();
@@ -258,28 +285,79 @@ struct ConvPatch
                 }
 
                 // ---- epilogue: 8 consecutive channels of one pixel per lane and M tile ----------
-                _Float16* out_band = reinterpret_cast<_Float16*>(p.out) + ((size_t)n * p.Ho + (size_t)TH * b) * p.Wo * KO;
-#pragma unroll
-                for(int t = 0; t < MTW; ++t)
+                uint8_t* out_band = reinterpret_cast<uint8_t*>(p.out) + ((size_t)n * p.Ho + (size_t)TH * b) * p.Wo * (KO * ES);
+                if constexpr(DT == DT_I8)
                 {
-                    if(TH * b + (int)rout[t] < p.Ho)
-                    {
-                        f16x8 o;
+                    // 8 consecutive int8 channels per lane and M tile: the requant / PassThrough family of the GEMM
+                    // epilogue. The mode is dispatched ONCE per band (a compile-time parameter of the body): tested
+                    // per value it turns the epilogue into hundreds of scalar branches, which cost more than the
+                    // whole K loop.
+                    auto store_band = [&](auto epi_c) {
+                        constexpr int EPI = decltype(epi_c)::value;
 #pragma unroll
-                        for(int i = 0; i < 4; ++i)
+                        for(int t = 0; t < MTW; ++t)
                         {
-                            float v0 = acc[t][0][i], v1 = acc[t][1][i];
-                            if constexpr(FUSED)
+                            if(TH * b + (int)rout[t] < p.Ho)
                             {
-                                v0 = epi_f16_value(p.epi, v0, (float)bias8[i], (float)resi8[t][i]);
-                                v1 = epi_f16_value(p.epi, v1, (float)bias8[4 + i], (float)resi8[t][4 + i]);
+                                int v[8];
+#pragma unroll
+                                for(int i = 0; i < 4; ++i)
+                                {
+                                    v[i]     = epilogue_i8<EPI>(acc[t][0][i], p.scale_gemm, p.scale_relu);
+                                    v[4 + i] = epilogue_i8<EPI>(acc[t][1][i], p.scale_gemm, p.scale_relu);
+                                }
+                                i32x2 o;
+                                o[0] = pack4_low_bytes(v[0], v[1], v[2], v[3]);
+                                o[1] = pack4_low_bytes(v[4], v[5], v[6], v[7]);
+                                *reinterpret_cast<i32x2*>(out_band + ooff[t]) = o;
                             }
-                            o[i]     = (_Float16)v0;
-                            o[4 + i] = (_Float16)v1;
+                            acc[t][0] = acc[t][1] = acc_t{0, 0, 0, 0};
                         }
-                        *reinterpret_cast<f16x8*>(reinterpret_cast<uint8_t*>(out_band) + ooff[t]) = o;
+                    };
+                    if(p.epi == EPI_REQUANT_RND)
+                        store_band(std::integral_constant<int, EPI_REQUANT_RND>{});
+                    else if(p.epi == EPI_REQUANT_CK)
+                        store_band(std::integral_constant<int, EPI_REQUANT_CK>{});
+                    else
+                        store_band(std::integral_constant<int, EPI_PASSTHROUGH>{});
+                }
+                else
+                {
+                    // (fused variant: the functor is a compile-time parameter of the body as well)
+                    auto store_band = [&](auto epi_c) {
+                        constexpr int EPI = decltype(epi_c)::value;
+#pragma unroll
+                        for(int t = 0; t < MTW; ++t)
+                        {
+                            if(TH * b + (int)rout[t] < p.Ho)
+                            {
+                                f16x8 o;
+#pragma unroll
+                                for(int i = 0; i < 4; ++i)
+                                {
+                                    float v0 = acc[t][0][i], v1 = acc[t][1][i];
+                                    if constexpr(EPI != EPI_PASSTHROUGH)
+                                    {
+                                        v0 = epi_f16_value(EPI, v0, (float)bias8[i], (float)resi8[FUSED ? t : 0][i]);
+                                        v1 = epi_f16_value(EPI, v1, (float)bias8[4 + i], (float)resi8[FUSED ? t : 0][4 + i]);
+                                    }
+                                    o[i]     = (_Float16)v0;
+                                    o[4 + i] = (_Float16)v1;
+                                }
+                                *reinterpret_cast<f16x8*>(out_band + ooff[t]) = o;
+                            }
+                            acc[t][0] = acc[t][1] = acc_t{0, 0, 0, 0};
+                        }
+                    };
+                    if constexpr(FUSED)
+                    {
+                        if(p.epi == EPI_ADD_RELU_ADD)
+                            store_band(std::integral_constant<int, EPI_ADD_RELU_ADD>{});
+                        else
+                            store_band(std::integral_constant<int, EPI_ADD_RELU>{});
                     }
-                    acc[t][0] = acc[t][1] = f32x4{0, 0, 0, 0};
+                    else
+                        store_band(std::integral_constant<int, EPI_PASSTHROUGH>{});
                 }
             }
             barrier(); // the ring is free for the next image's first rows
@@ -289,11 +367,11 @@ struct ConvPatch
     }
 };
 
-template <int MTW, int Y, int X, bool FUSED>
+template <int DT, int MTW, int Y, int X, bool FUSED>
 __global__ __launch_bounds__(256) void conv_patch_kernel(const ConvPatchArgs p)
 {
     extern __shared__ __attribute__((aligned(1024))) uint8_t ckx_patch_smem[];
-    ConvPatch<MTW, Y, X, FUSED>::run(p, ckx_patch_smem);
+    ConvPatch<DT, MTW, Y, X, FUSED>::run(p, ckx_patch_smem);
 }
 
 } // namespace ckx

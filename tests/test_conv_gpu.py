@@ -184,4 +184,40 @@ def test_conv2d_input_patch_instance_refuses_other_shapes():
     d = capi.Conv2dDesc(2, 64, 64, 9, 48, 3, 3, 9, 48, 1, 1, 1, 1, 1, 1, 1, 1)     # Wo = 48
     assert capi.lib().ckx_conv2d_fwd_is_supported(capi.OP_CONV2D_FWD_F16, C.byref(d), 0, patch) == capi.UNSUPPORTED
     assert capi.lib().ckx_conv2d_fwd_is_supported(capi.OP_CONV2D_FWD_F16, C.byref(d), 0, -1) == capi.OK
-    assert capi.lib().ckx_conv2d_fwd_is_supported(capi.OP_CONV2D_FWD_I8, C.byref(d), 0, patch) == capi.INVALID_VALUE
+    assert capi.lib().ckx_conv2d_fwd_is_supported(capi.OP_CONV2D_FWD_I8, C.byref(d), 0, patch) == capi.UNSUPPORTED
+    assert capi.lib().ckx_conv2d_fwd_is_supported(capi.OP_CONV2D_FWD_I8, C.byref(d), 0, patch + 1) == capi.INVALID_VALUE
+
+
+@pytest.mark.parametrize("case", PATCH)
+@pytest.mark.parametrize("auto", [True, False])
+def test_conv2d_int8_input_patch_kernel_bit_exact(case, auto):
+    """The int8 form of the input-patch kernel (a pixel = 64 bytes = one MFMA k-step): PassThrough (low byte)
+    and both requant epilogues, bit for bit against the literal oracle; the tile kernel must agree."""
+    import gpu_util
+    N, Hi, Wi, p = case
+    inp = uniform_int8((N, Hi, Wi, 64), -5, 5, 950 + Hi)
+    wei = uniform_int8((64, 3, 3, 64), -5, 5, 951 + Wi)
+    patch = capi.lib().ckx_num_instances(capi.OP_CONV2D_FWD_I8) - 1
+    assert b"Patch" in capi.lib().ckx_instance_name(capi.OP_CONV2D_FWD_I8, patch)
+    inst = capi.INSTANCE_AUTO if auto else patch
+    out = gpu_util.conv2d_fwd(inp, wei, (1, 1), (1, 1), p, instance=inst)
+    ref = lit.conv2d_fwd(inp, wei, (1, 1), (1, 1), p)
+    assert out.shape == ref.shape and out.shape[2] == 56
+    np.testing.assert_array_equal(out, ref)
+    for rq, kind in ((ck.RequantReluRequant(0.05, 0.7, rounded=True), lit.EPI_REQUANT_RND),
+                     (ck.RequantReluRequant(0.03, 1.0), lit.EPI_REQUANT_CK)):
+        out = gpu_util.conv2d_fwd(inp, wei, (1, 1), (1, 1), p, out_op=rq, instance=inst)
+        ref = lit.conv2d_fwd(inp, wei, (1, 1), (1, 1), p, epi=kind, scale_gemm=rq.scale_gemm, scale_relu=rq.scale_relu)
+        np.testing.assert_array_equal(out, ref)
+        np.testing.assert_array_equal(gpu_util.conv2d_fwd(inp, wei, (1, 1), (1, 1), p, out_op=rq, instance=7), ref)
+        assert out.max() > 0
+
+
+def test_conv2d_int8_input_patch_kernel_full_range_and_many_images():
+    """Full-range int8 values (the int32 sums wrap into the low byte under PassThrough) and more images than
+    workgroups."""
+    import gpu_util
+    inp = uniform_int8((300, 5, 56, 64), -128, 127, 87)
+    wei = uniform_int8((64, 3, 3, 64), -128, 127, 88)
+    out = gpu_util.conv2d_fwd(inp, wei, (1, 1), (1, 1), (1, 1))
+    np.testing.assert_array_equal(out, fast.conv2d_fwd_i8(inp, wei, (1, 1), (1, 1), (1, 1)))
