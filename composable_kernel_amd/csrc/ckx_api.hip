@@ -436,7 +436,7 @@ int run_gemm(int dt, const void* a, const void* b, void* c, int M, int N, int K,
 }
 
 // ---------------------------------------------------------- input-patch conv kernel
-const char* const kPatchName = "MI355X_Mfma16_Patch<4 rows x 56, 3x3, C 64, K 64, waves 2x2>";
+const char* const kPatchName = "MI355X_Mfma16_Patch<rows x 56, 3x3, C 64, K 64, 4 waves>";
 
 // shapes the input-patch kernel covers (one instantiation per data type: 3x3 taps, Wo = 56)
 bool conv_patch_applicable(int op, const ckx_conv2d_desc* d, int epi)
@@ -550,7 +550,6 @@ int run_conv(int op, const void* in, const void* wei, void* out, const ckx_conv2
         a.wei_bytes = (uint32_t)((long)N * K * es);
         a.N = d->N, a.Hi = d->Hi, a.Wi = d->Wi, a.Ho = d->Ho, a.Wo = d->Wo;
         a.pT = d->pad_top, a.pL = d->pad_left;
-        a.nbands = (d->Ho + 3) / 4;
         a.div_wo = make_magic((uint32_t)d->Wo);
         a.epi    = epi;
         a.bias = dops.d0, a.resi = epi == CKX_EPI_ADD_RELU_ADD ? dops.d1 : nullptr;

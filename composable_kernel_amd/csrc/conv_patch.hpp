@@ -37,7 +37,6 @@ struct ConvPatchArgs
     uint32_t in_bytes, wei_bytes;
     int N, Hi, Wi, Ho, Wo;
     int pT, pL;
-    int nbands; // ceil(Ho / 4)
     MagicDiv div_wo;
     int epi; // fp16: EPI_PASSTHROUGH, EPI_ADD_RELU, EPI_ADD_RELU_ADD; int8: EPI_PASSTHROUGH, EPI_REQUANT_CK, EPI_REQUANT_RND
     const void* bias; // [64] fp16
@@ -47,15 +46,22 @@ struct ConvPatchArgs
 
 // FUSED: the add / ReLU epilogues (bias, residual) are compiled in; the plain instantiation keeps
 // their registers free
-template <int DT, int MTW, int Y, int X, bool FUSED>
+// TH output rows per band, WMW x (4 / WMW) waves: a wave multiplies 16 * MTW pixels x 64 / (4 / WMW) channels.
+// fp16: 4 rows, 2 x 2 waves (the LDS holds no deeper ring beside the weights); int8: 8 rows, 4 x 1 waves -- every
+// wave then owns all 64 channels of its pixels (one 16-byte store per pixel and lane, whole 64-byte pixels per
+// four lanes) and reads 11 fragments per 28 MFMAs instead of 9 per 14.
+template <int DT, int MTW, int Y, int X, bool FUSED, int TH_ = (DT == DT_I8 ? 8 : 4), int WMW = (DT == DT_I8 ? 4 : 2)>
 struct ConvPatch
 {
     static constexpr int ES     = DT == DT_I8 ? 1 : 2;
-    static constexpr int TH     = 4;                // output rows per band
+    static constexpr int TH     = TH_;              // output rows per band
+    static constexpr int WNW    = 4 / WMW;          // waves along the output channels
+    static constexpr int NBT    = 4 / WNW;          // 16-channel weight tiles per wave (2 / 4)
+    static constexpr int CPW    = 16 * NBT;         // channels per wave
     // bands of input rows in flight ahead of the band being multiplied. fp16 rows fill the LDS with one; int8
     // rows are half as large, and three bands of head start take the HBM latency out of the band loop (one
     // image per workgroup at a time: nothing else would hide it)
-    static constexpr int AHEAD  = ES == 1 ? 3 : 1;
+    static constexpr int AHEAD  = ES == 1 ? 2 : 1;
     static constexpr int RING   = (AHEAD + 1) * TH + 2; // ring rows (Y <= 3)
     static constexpr int PITCH  = 64;               // pixels per ring row
     static constexpr int PXB    = 64 * ES;          // bytes per pixel (C * element size)
@@ -71,6 +77,8 @@ struct ConvPatch
     static constexpr int NEED_ROWS  = TH + Y - 1;   // input rows of one band
     static_assert(Y >= 1 && Y <= 3 && X >= 1 && X <= 3 && MTW >= 1 && MTW <= 7, "covered shapes");
     static_assert(DT == DT_F16 || (DT == DT_I8 && !FUSED), "fp16 (optionally with the add / ReLU epilogues) or int8");
+    static_assert((WMW == 2 || WMW == 4) && (NBT == 2 || DT == DT_I8), "wave arrangements built");
+    static_assert(LDS <= 160 * 1024, "ring + weights fit the LDS");
     using acc_t = typename std::conditional<DT == DT_I8, i32x4, f32x4>::type;
     // swizzle key of a pixel column / weight row: the 16 rows of a fragment read must land on distinct banks
     __device__ static __forceinline__ uint32_t key(uint32_t r) { return CPP == 8 ? (r & 7u) : ((r >> 2) & 3u); }
@@ -79,7 +87,7 @@ struct ConvPatch
     {
         const int lane = threadIdx.x & 63;
         const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-        const int wm = wave >> 1, wn = wave & 1;
+        const int wm = wave / WNW, wn = wave % WNW;
         const uint32_t frow = (uint32_t)(lane & 15), fq = (uint32_t)(lane >> 4);
         uint8_t* ring = smem;
         uint8_t* wlds = smem + RING_BYTES;
@@ -96,8 +104,9 @@ struct ConvPatch
             {
                 const uint32_t tap = (uint32_t)k / BPT;
                 const uint32_t r   = ((uint32_t)k % BPT) * PPI + rl; // 0..63
-                // within a 32-row group, row 16j + 4q + i holds channel 8q + 4j + i
-                const uint32_t ch = (r & ~31u) | (((r >> 2) & 3u) << 3) | (((r >> 4) & 1u) << 2) | (r & 3u);
+                // within a wave's group of CPW rows, row 16j + 4q + i holds channel 4*NBT*q + 4j + i
+                const uint32_t rr = r % CPW;
+                const uint32_t ch = (r - rr) + (4 * NBT) * ((rr >> 2) & 3u) + 4 * (rr >> 4) + (rr & 3u);
                 const uint32_t voff = (ch * TAPS + tap) * PXB + ((pos ^ key(r)) << 4);
                 __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_wei, (lds_ptr_t)(wlds + (size_t)k * 1024), 16, voff, 0,
                                                          0, 0);
@@ -115,7 +124,7 @@ struct ConvPatch
             const uint32_t r = magic_div(q, p.div_wo);
             const uint32_t w = q - r * (uint32_t)p.Wo;
             rout[t]          = r;
-            ooff[t]          = ((r * (uint32_t)p.Wo + w) * KO + (uint32_t)(32 * wn) + 8u * fq) * ES;
+            ooff[t]          = ((r * (uint32_t)p.Wo + w) * KO + (uint32_t)(CPW * wn) + (uint32_t)(4 * NBT) * fq) * ES;
 #pragma unroll
             for(int x = 0; x < X; ++x)
             {
@@ -127,16 +136,16 @@ struct ConvPatch
         const bool has_resi = FUSED && p.epi == EPI_ADD_RELU_ADD;
         f16x8 bias8 = {0, 0, 0, 0, 0, 0, 0, 0};
         if constexpr(FUSED)
-            bias8 = *reinterpret_cast<const f16x8*>(reinterpret_cast<const _Float16*>(p.bias) + 32 * wn + 8 * (int)fq);
+            bias8 = *reinterpret_cast<const f16x8*>(reinterpret_cast<const _Float16*>(p.bias) + CPW * wn + 4 * NBT * (int)fq);
         f16x8 resi8[FUSED ? MTW : 1];
 #pragma unroll
         for(int t = 0; t < (FUSED ? MTW : 1); ++t)
             resi8[t] = f16x8{0, 0, 0, 0, 0, 0, 0, 0};
 
-        uint32_t boff[2]; // weight fragment of n-tile j, k-step 0, tap 0
+        uint32_t boff[NBT]; // weight fragment of n-tile j, k-step 0, tap 0
 #pragma unroll
-        for(int j = 0; j < 2; ++j)
-            boff[j] = (uint32_t)(32 * wn + 16 * j + (int)frow) * PXB + ((fq ^ key(frow)) << 4);
+        for(int j = 0; j < NBT; ++j)
+            boff[j] = (uint32_t)(CPW * wn + 16 * j + (int)frow) * PXB + ((fq ^ key(frow)) << 4);
 
         // ---- input rows -> ring: block k = (row j, PPI-pixel column group cg) ------------------
         // lane: patch column PPI*cg + lane/CPP, LDS chunk position lane%CPP <- global chunk pos ^ key(col)
@@ -153,10 +162,12 @@ struct ConvPatch
                                                      16, voff, 0, 0, 0);
         };
 
-        acc_t acc[MTW][2];
+        acc_t acc[MTW][NBT];
 #pragma unroll
         for(int t = 0; t < MTW; ++t)
-            acc[t][0] = acc[t][1] = acc_t{0, 0, 0, 0};
+#pragma unroll
+            for(int j = 0; j < NBT; ++j)
+                acc[t][j] = acc_t{0, 0, 0, 0};
 
         auto barrier = [&]() {
             __builtin_amdgcn_s_barrier();
@@ -164,7 +175,8 @@ struct ConvPatch
         };
 
         uint32_t roff[MTW][Y]; // ring byte offset of (M tile's output row + y) for the current band
-        i32x4 af[2][MTW], bf[2][2];
+        i32x4 af[2][MTW], bf[2][NBT];
+        const int nbands = (p.Ho + TH - 1) / TH;
         for(int n = (int)blockIdx.x; n < p.N; n += (int)gridDim.x)
         {
             // rows of the first band (every wave has passed the barrier that ended the previous image)
@@ -173,7 +185,7 @@ struct ConvPatch
             asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
             barrier();
 
-            for(int b = 0; b < p.nbands; ++b)
+            for(int b = 0; b < nbands; ++b)
             {
                 const int j0 = TH * b; // first ring row index (before the modulo) of this band
                 if(b == 0)
@@ -189,17 +201,17 @@ struct ConvPatch
                 // M tiles in the order in which the MFMAs use them
                 auto read_one = [&](int s, int r) {
                     const int buf = s & 1, tap = s / KSP, ks = s % KSP, y = tap / X, x = tap % X;
-                    if(r < 2)
+                    if(r < NBT)
                         bf[buf][r] = *reinterpret_cast<const i32x4*>(wlds + tap * (KO * PXB) +
                                                                      (boff[r] ^ (uint32_t)(ks * 64)));
                     else
-                        af[buf][r - 2] = *reinterpret_cast<const i32x4*>(ring + roff[r - 2][y] +
-                                                                         (coff[r - 2][x] ^ (uint32_t)(ks * 64)));
+                        af[buf][r - NBT] = *reinterpret_cast<const i32x4*>(ring + roff[r - NBT][y] +
+                                                                           (coff[r - NBT][x] ^ (uint32_t)(ks * 64)));
                 };
                 auto mfma_pair = [&](int s, int t) {
                     const int buf = s & 1;
 #pragma unroll
-                    for(int j = 0; j < 2; ++j)
+                    for(int j = 0; j < NBT; ++j)
                     {
                         if constexpr(DT == DT_I8)
                             acc[t][j] = __builtin_amdgcn_mfma_i32_16x16x64_i8(bf[buf][j], af[buf][t], acc[t][j], 0, 0, 0);
@@ -213,7 +225,7 @@ struct ConvPatch
                 if(b == 0)
                 {
 #pragma unroll
-                    for(int r = 0; r < MTW + 2; ++r)
+                    for(int r = 0; r < MTW + NBT; ++r)
                         read_one(0, r);
                 }
                 // residual values of this band: plain loads, issued before the band's direct loads and
@@ -232,7 +244,7 @@ struct ConvPatch
                 // the first groups and finished two groups early] [one direct load of the next band's
                 // rows] [the 2 MFMAs of one M tile]. With one wave per SIMD nothing else hides the
                 // issue slots of the reads, so they go between the MFMAs.
-                constexpr int NR = MTW + 2, RG = MTW > 2 ? MTW - 2 : MTW;
+                constexpr int NR = MTW + NBT, RG = MTW > 2 ? MTW - 2 : MTW;
                 constexpr int NS = KSP * TAPS;           // k-steps of a band
                 constexpr int NBLK = TH * BPR / 4;       // direct loads per wave for the next band's rows
                 static_assert(NBLK <= NS, "one direct load per k-step");
@@ -267,7 +279,7 @@ struct ConvPatch
                 // every wave is through with this band's rows, and the next band's rows are visible:
                 // its first fragments are read under the epilogue
                 barrier();
-                if(b + 1 < p.nbands)
+                if(b + 1 < nbands)
                 {
                     const int j1 = j0 + TH;
 #pragma unroll
@@ -280,7 +292,7 @@ struct ConvPatch
                             roff[t][y]  = sl * (PITCH * PXB);
                         }
 #pragma unroll
-                    for(int r = 0; r < MTW + 2; ++r)
+                    for(int r = 0; r < MTW + NBT; ++r)
                         read_one(0, r);
                 }
 
@@ -299,19 +311,21 @@ struct ConvPatch
                         {
                             if(TH * b + (int)rout[t] < p.Ho)
                             {
-                                int v[8];
+                                int o[NBT];
 #pragma unroll
-                                for(int i = 0; i < 4; ++i)
-                                {
-                                    v[i]     = epilogue_i8<EPI>(acc[t][0][i], p.scale_gemm, p.scale_relu);
-                                    v[4 + i] = epilogue_i8<EPI>(acc[t][1][i], p.scale_gemm, p.scale_relu);
-                                }
-                                i32x2 o;
-                                o[0] = pack4_low_bytes(v[0], v[1], v[2], v[3]);
-                                o[1] = pack4_low_bytes(v[4], v[5], v[6], v[7]);
-                                *reinterpret_cast<i32x2*>(out_band + ooff[t]) = o;
+                                for(int j = 0; j < NBT; ++j)
+                                    o[j] = pack4_low_bytes(epilogue_i8<EPI>(acc[t][j][0], p.scale_gemm, p.scale_relu),
+                                                           epilogue_i8<EPI>(acc[t][j][1], p.scale_gemm, p.scale_relu),
+                                                           epilogue_i8<EPI>(acc[t][j][2], p.scale_gemm, p.scale_relu),
+                                                           epilogue_i8<EPI>(acc[t][j][3], p.scale_gemm, p.scale_relu));
+                                if constexpr(NBT == 4)
+                                    *reinterpret_cast<i32x4*>(out_band + ooff[t]) = i32x4{o[0], o[1], o[2], o[3]};
+                                else
+                                    *reinterpret_cast<i32x2*>(out_band + ooff[t]) = i32x2{o[0], o[1]};
                             }
-                            acc[t][0] = acc[t][1] = acc_t{0, 0, 0, 0};
+#pragma unroll
+                            for(int j = 0; j < NBT; ++j)
+                                acc[t][j] = acc_t{0, 0, 0, 0};
                         }
                     };
                     if(p.epi == EPI_REQUANT_RND)
