@@ -14,6 +14,7 @@
 #include "tile_launch.hpp"
 #include "gemm_gemm.hpp"
 #include "conv_patch.hpp"
+#include "conv_pointwise.hpp"
 #include "gemm_skinny.hpp"
 
 namespace {
@@ -449,6 +450,29 @@ bool conv_patch_applicable(int op, const ckx_conv2d_desc* d, int epi)
            d->Wo == 56 && d->Ho >= 1 && d->N >= 1 && d->pad_left <= 2 && d->pad_top <= 2;
 }
 
+// ---------------------------------------------------------- weight-stationary pointwise conv kernel
+const char* const kPointwiseName = "MI355X_Mfma16_Pointwise<1x1, C 256/512 bytes, K 512 per workgroup, 8 waves>";
+constexpr int kConvPatchInstance = kNumTiles, kConvPointwiseInstance = kNumTiles + 1, kNumConvInsts = kNumTiles + 2;
+
+// shapes the pointwise kernel covers: 1x1 filters without padding, a pixel of 256 or 512 bytes, output channels in
+// whole blocks of 512
+bool conv_pointwise_applicable(int op, const ckx_conv2d_desc* d, int epi)
+{
+    const int es      = op == CKX_OP_CONV2D_FWD_I8 ? 1 : 2;
+    const bool epi_ok = op == CKX_OP_CONV2D_FWD_F16
+                            ? (epi == CKX_EPI_PASSTHROUGH || epi == CKX_EPI_ADD_RELU)
+                            : (epi == CKX_EPI_PASSTHROUGH || epi == CKX_EPI_REQUANT_CK || epi == CKX_EPI_REQUANT_RND);
+    return (op == CKX_OP_CONV2D_FWD_F16 || op == CKX_OP_CONV2D_FWD_I8) && epi_ok && d->Y == 1 && d->X == 1 &&
+           d->pad_top == 0 && d->pad_left == 0 && d->pad_bottom == 0 && d->pad_right == 0 &&
+           (d->C * es == 256 || d->C * es == 512) && d->K >= 512 && d->K % 512 == 0 && d->N >= 1 && d->Ho >= 1 &&
+           d->Wo >= 1;
+}
+// ... and the ones it is chosen for: enough pixels for every workgroup to amortise loading its weight slice
+bool conv_pointwise_preferred(int op, const ckx_conv2d_desc* d, int epi)
+{
+    return conv_pointwise_applicable(op, d, epi) && (long)d->N * d->Ho * d->Wo * (d->K / 512) >= 64 * 1024;
+}
+
 template <int DT, bool FUSED>
 hipError_t launch_conv_patch(const ckx::ConvPatchArgs& a, hipStream_t s)
 {
@@ -474,7 +498,7 @@ int check_conv(int op, const ckx_conv2d_desc* d, int epi, int instance)
     if(op != CKX_OP_CONV2D_FWD_I8 && op != CKX_OP_CONV2D_FWD_F16)
         return fail(CKX_INVALID_VALUE, "not a conv operator family");
     const int es = op == CKX_OP_CONV2D_FWD_I8 ? 1 : 2;
-    if(instance != CKX_INSTANCE_AUTO && (instance < 0 || instance > kNumTiles))
+    if(instance != CKX_INSTANCE_AUTO && (instance < 0 || instance >= kNumConvInsts))
         return fail(CKX_INVALID_VALUE, "no such instance");
     if(epi < CKX_EPI_PASSTHROUGH || epi > CKX_EPI_CSHUFFLE_ADD_RELU || !epilogue_fits_dtype(es, epi) ||
        epi == CKX_EPI_CSHUFFLE_ADD_RELU)
@@ -502,8 +526,11 @@ int check_conv(int op, const ckx_conv2d_desc* d, int epi, int instance)
     if(in_b >= (1l << 31) || wei_b >= (1l << 31) || out_b >= (1l << 31) ||
        (long)d->N * d->Ho * d->Wo >= (1l << 31))
         return fail(CKX_UNSUPPORTED, "tensors of 2 GiB or more are not addressed");
-    if(instance == kNumTiles && !conv_patch_applicable(op, d, epi))
+    if(instance == kConvPatchInstance && !conv_patch_applicable(op, d, epi))
         return fail(CKX_UNSUPPORTED, "the input-patch instance covers 3x3 stride-1 layers with C = K = 64, Wo = 56");
+    if(instance == kConvPointwiseInstance && !conv_pointwise_applicable(op, d, epi))
+        return fail(CKX_UNSUPPORTED, "the pointwise instance covers 1x1 layers without padding, C of 256 or 512 bytes, "
+                                     "K a multiple of 512, PassThrough / requant / bias + ReLU epilogues");
     return CKX_OK;
 }
 
@@ -513,7 +540,9 @@ long conv_workspace_bytes(int op, const ckx_conv2d_desc* d, int instance)
     const long M = (long)d->N * d->Ho * d->Wo;
     if(M <= 0 || d->K <= 0)
         return 0;
-    if(instance == kNumTiles || (instance == CKX_INSTANCE_AUTO && conv_patch_applicable(op, d, CKX_EPI_PASSTHROUGH)))
+    if(instance == kConvPatchInstance || instance == kConvPointwiseInstance ||
+       (instance == CKX_INSTANCE_AUTO &&
+        (conv_patch_applicable(op, d, CKX_EPI_PASSTHROUGH) || conv_pointwise_preferred(op, d, CKX_EPI_PASSTHROUGH))))
         return 0;
     const Plan pl = make_plan((int)M, d->K, d->Y * d->X * d->C * es, instance, 1l << 60);
     return pl.ksplit > 1 ? (long)pl.ksplit * M * d->K * 4 : 0;
@@ -539,7 +568,7 @@ int run_conv(int op, const void* in, const void* wei, void* out, const ckx_conv2
         return fail(CKX_INVALID_VALUE, "workspace must be 16-byte aligned");
     const bool patch_aligned = !((reinterpret_cast<uintptr_t>(out) | reinterpret_cast<uintptr_t>(dops.d0) |
                                   (epi == CKX_EPI_ADD_RELU_ADD ? reinterpret_cast<uintptr_t>(dops.d1) : 0)) & 15);
-    if(instance == kNumTiles || (instance == CKX_INSTANCE_AUTO && conv_patch_applicable(op, d, epi) && patch_aligned))
+    if(instance == kConvPatchInstance || (instance == CKX_INSTANCE_AUTO && conv_patch_applicable(op, d, epi) && patch_aligned))
     {
         if(!patch_aligned)
             return fail(CKX_UNSUPPORTED, "the input-patch instance needs 16-byte aligned output, bias and residual");
@@ -558,6 +587,28 @@ int run_conv(int op, const void* in, const void* wei, void* out, const ckx_conv2
                        : epi == CKX_EPI_PASSTHROUGH ? launch_conv_patch<ckx::DT_F16, false>(a, (hipStream_t)stream)
                                                     : launch_conv_patch<ckx::DT_F16, true>(a, (hipStream_t)stream);
         return e == hipSuccess ? CKX_OK : hip_fail(e, kPatchName);
+    }
+    if(instance == kConvPointwiseInstance ||
+       (instance == CKX_INSTANCE_AUTO && conv_pointwise_preferred(op, d, epi) && patch_aligned && dops.ldd0 == 0))
+    {
+        if(!patch_aligned)
+            return fail(CKX_UNSUPPORTED, "the pointwise instance needs 16-byte aligned output and bias");
+        if(epi == CKX_EPI_ADD_RELU && dops.ldd0 != 0)
+            return fail(CKX_UNSUPPORTED, "the pointwise instance adds a bias row (D0 row stride 0) only");
+        ckx::ConvPointwiseArgs a;
+        std::memset(&a, 0, sizeof(a));
+        a.in = in, a.wei = wei, a.out = out;
+        a.in_bytes = (uint32_t)((long)d->N * d->Hi * d->Wi * d->C * es);
+        a.M = M, a.Kout = N;
+        a.Hi = d->Hi, a.Wi = d->Wi, a.Wo = d->Wo, a.HoWo = d->Ho * d->Wo, a.sH = d->stride_h, a.sW = d->stride_w;
+        a.div_howo = make_magic((uint32_t)(d->Ho * d->Wo));
+        a.div_wo   = make_magic((uint32_t)d->Wo);
+        a.epi = epi, a.bias = dops.d0;
+        a.scale_gemm = sg, a.scale_relu = sr;
+        a.nt_store   = (long)M * N * es >= stream_output_bytes();
+        hipError_t e = ckx::launch_conv_pointwise(es == 1 ? ckx::DT_I8 : ckx::DT_F16, d->C * es, epi == CKX_EPI_ADD_RELU, a,
+                                                  (hipStream_t)stream);
+        return e == hipSuccess ? CKX_OK : hip_fail(e, kPointwiseName);
     }
     const Plan pl = make_plan(M, N, K * es, instance, ws ? ws_bytes : 0);
     const TileInstance& t = kTiles[pl.tile];
@@ -611,7 +662,7 @@ int ckx_num_instances(int op)
     if(op == CKX_OP_GEMM_SPLITK)
         return kNumTiles;
     if(op == CKX_OP_CONV2D_FWD_F16 || op == CKX_OP_CONV2D_FWD_I8)
-        return kNumTiles + 1; // + the input-patch kernel
+        return kNumConvInsts; // + the input-patch and the pointwise kernel
     if(op == CKX_OP_BATCHED_GEMM_GEMM || op == CKX_OP_BATCHED_GEMM_SOFTMAX_GEMM)
         return ckx::kNumGemmGemmInstances;
     return 0;
@@ -626,8 +677,8 @@ const char* ckx_instance_name(int op, int instance)
     s = std::string(fam) + "<" +
         (op == CKX_OP_BATCHED_GEMM_GEMM || op == CKX_OP_BATCHED_GEMM_SOFTMAX_GEMM
              ? ckx::gemm_gemm_instance_name(instance)
-         : (op == CKX_OP_CONV2D_FWD_F16 || op == CKX_OP_CONV2D_FWD_I8) && instance == kNumTiles
-             ? kPatchName
+         : (op == CKX_OP_CONV2D_FWD_F16 || op == CKX_OP_CONV2D_FWD_I8) && instance >= kNumTiles
+             ? (instance == kConvPatchInstance ? kPatchName : kPointwiseName)
              : instance >= kNumTiles ? kSkinny[instance - kNumTiles].name : kTiles[instance].name) +
         ">";
     return s.c_str();

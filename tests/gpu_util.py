@@ -52,6 +52,14 @@ def gemm_f16(a_mk, b_nk, instance=capi.INSTANCE_AUTO, time_kernel=False, allow_u
     return (out, ms) if time_kernel else out
 
 
+def conv_instance(op, tag):
+    """Index of the conv instance of family `op` (capi.OP_CONV2D_FWD_*) whose name contains `tag`."""
+    L = capi.lib()
+    hits = [i for i in range(L.ckx_num_instances(op)) if tag.encode() in L.ckx_instance_name(op, i)]
+    assert len(hits) == 1, (tag, hits)
+    return hits[0]
+
+
 def conv2d_fwd(inp_nhwc, wei_kyxc, strides, dilations, pads, out_op=None, instance=capi.INSTANCE_AUTO,
                right_pads=None):
     N, Hi, Wi, C = inp_nhwc.shape

@@ -160,8 +160,7 @@ def test_conv2d_fp16_input_patch_kernel(case, auto):
     N, Hi, Wi, p = case
     inp = uniform_f16((N, Hi, Wi, 64), -1, 1, 900 + Hi)
     wei = uniform_f16((64, 3, 3, 64), -1, 1, 901 + Wi)
-    patch = capi.lib().ckx_num_instances(capi.OP_CONV2D_FWD_F16) - 1
-    assert b"Patch" in capi.lib().ckx_instance_name(capi.OP_CONV2D_FWD_F16, patch)
+    patch = gpu_util.conv_instance(capi.OP_CONV2D_FWD_F16, "Patch")
     out = gpu_util.conv2d_fwd(inp, wei, (1, 1), (1, 1), p, instance=capi.INSTANCE_AUTO if auto else patch)
     ref = lit.conv2d_fwd(inp, wei, (1, 1), (1, 1), p)
     assert out.shape == ref.shape and out.shape[2] == 56
@@ -180,12 +179,14 @@ def test_conv2d_fp16_input_patch_kernel_more_images_than_cus():
 
 def test_conv2d_input_patch_instance_refuses_other_shapes():
     import ctypes as C
-    patch = capi.lib().ckx_num_instances(capi.OP_CONV2D_FWD_F16) - 1
+    import gpu_util
+    patch = gpu_util.conv_instance(capi.OP_CONV2D_FWD_F16, "Patch")
     d = capi.Conv2dDesc(2, 64, 64, 9, 48, 3, 3, 9, 48, 1, 1, 1, 1, 1, 1, 1, 1)     # Wo = 48
     assert capi.lib().ckx_conv2d_fwd_is_supported(capi.OP_CONV2D_FWD_F16, C.byref(d), 0, patch) == capi.UNSUPPORTED
     assert capi.lib().ckx_conv2d_fwd_is_supported(capi.OP_CONV2D_FWD_F16, C.byref(d), 0, -1) == capi.OK
     assert capi.lib().ckx_conv2d_fwd_is_supported(capi.OP_CONV2D_FWD_I8, C.byref(d), 0, patch) == capi.UNSUPPORTED
-    assert capi.lib().ckx_conv2d_fwd_is_supported(capi.OP_CONV2D_FWD_I8, C.byref(d), 0, patch + 1) == capi.INVALID_VALUE
+    n = capi.lib().ckx_num_instances(capi.OP_CONV2D_FWD_I8)
+    assert capi.lib().ckx_conv2d_fwd_is_supported(capi.OP_CONV2D_FWD_I8, C.byref(d), 0, n) == capi.INVALID_VALUE
 
 
 @pytest.mark.parametrize("case", PATCH)
@@ -197,8 +198,7 @@ def test_conv2d_int8_input_patch_kernel_bit_exact(case, auto):
     N, Hi, Wi, p = case
     inp = uniform_int8((N, Hi, Wi, 64), -5, 5, 950 + Hi)
     wei = uniform_int8((64, 3, 3, 64), -5, 5, 951 + Wi)
-    patch = capi.lib().ckx_num_instances(capi.OP_CONV2D_FWD_I8) - 1
-    assert b"Patch" in capi.lib().ckx_instance_name(capi.OP_CONV2D_FWD_I8, patch)
+    patch = gpu_util.conv_instance(capi.OP_CONV2D_FWD_I8, "Patch")
     inst = capi.INSTANCE_AUTO if auto else patch
     out = gpu_util.conv2d_fwd(inp, wei, (1, 1), (1, 1), p, instance=inst)
     ref = lit.conv2d_fwd(inp, wei, (1, 1), (1, 1), p)
@@ -221,3 +221,85 @@ def test_conv2d_int8_input_patch_kernel_full_range_and_many_images():
     wei = uniform_int8((64, 3, 3, 64), -128, 127, 88)
     out = gpu_util.conv2d_fwd(inp, wei, (1, 1), (1, 1), (1, 1))
     np.testing.assert_array_equal(out, fast.conv2d_fwd_i8(inp, wei, (1, 1), (1, 1), (1, 1)))
+
+
+# (N, C, K, Hi, Wi, strides): 1x1 filters, no padding, a pixel of 256 or 512 bytes, K in blocks of 512 -- the
+# weight-stationary pointwise kernel's shapes (the reference's Filter1x1Pad0 / Filter1x1Stride1Pad0 specialisations)
+POINTWISE_F16 = [
+    (1, 256, 512, 4, 8, (1, 1)),        # one band exactly
+    (3, 256, 512, 7, 5, (1, 1)),        # pixel count not a multiple of the band (105)
+    (2, 128, 1024, 9, 9, (2, 2)),       # 256-byte pixels, two blocks of output channels, stride 2
+    (2, 256, 512, 11, 13, (2, 1)),      # different strides along h and w
+    (1, 128, 512, 1, 3, (1, 1)),        # fewer pixels than one MFMA tile
+]
+POINTWISE_I8 = [
+    (1, 256, 512, 4, 8, (1, 1)),
+    (3, 512, 512, 7, 5, (1, 1)),        # 512-byte pixels
+    (2, 256, 1024, 9, 9, (2, 2)),
+    (2, 512, 512, 11, 13, (1, 2)),
+]
+
+
+@pytest.mark.parametrize("case", POINTWISE_F16)
+def test_conv2d_fp16_pointwise_kernel(case):
+    """The weight-stationary 1x1 kernel (weights in registers, pixels through an LDS ring) against the literal
+    oracle; the tile kernel must agree on the same problem."""
+    import gpu_util
+    N, C, K, Hi, Wi, s = case
+    inp = uniform_f16((N, Hi, Wi, C), -1, 1, 1000 + Hi)
+    wei = uniform_f16((K, 1, 1, C), -1, 1, 1001 + Wi)
+    pw = gpu_util.conv_instance(capi.OP_CONV2D_FWD_F16, "Pointwise")
+    ref = lit.conv2d_fwd(inp, wei, s, (1, 1), (0, 0))
+    _f16_close(gpu_util.conv2d_fwd(inp, wei, s, (1, 1), (0, 0), instance=pw), ref)
+    _f16_close(gpu_util.conv2d_fwd(inp, wei, s, (1, 1), (0, 0), instance=0), ref)
+
+
+@pytest.mark.parametrize("case", POINTWISE_I8)
+def test_conv2d_int8_pointwise_kernel_bit_exact(case):
+    import gpu_util
+    N, C, K, Hi, Wi, s = case
+    inp = uniform_int8((N, Hi, Wi, C), -5, 5, 1010 + Hi)
+    wei = uniform_int8((K, 1, 1, C), -5, 5, 1011 + Wi)
+    pw = gpu_util.conv_instance(capi.OP_CONV2D_FWD_I8, "Pointwise")
+    np.testing.assert_array_equal(gpu_util.conv2d_fwd(inp, wei, s, (1, 1), (0, 0), instance=pw),
+                                  lit.conv2d_fwd(inp, wei, s, (1, 1), (0, 0)))
+    for rq, kind in ((ck.RequantReluRequant(0.02, 0.7, rounded=True), lit.EPI_REQUANT_RND),
+                     (ck.RequantReluRequant(0.03, 1.0), lit.EPI_REQUANT_CK)):
+        out = gpu_util.conv2d_fwd(inp, wei, s, (1, 1), (0, 0), out_op=rq, instance=pw)
+        np.testing.assert_array_equal(
+            out, lit.conv2d_fwd(inp, wei, s, (1, 1), (0, 0), epi=kind, scale_gemm=rq.scale_gemm, scale_relu=rq.scale_relu))
+        assert out.max() > 0
+
+
+@pytest.mark.parametrize("dtype", ["f16", "i8"])
+def test_conv2d_pointwise_kernel_long_runs_of_bands(dtype):
+    """Enough pixels for every workgroup to go round its ring of bands several times (the automatic choice for such
+    layers), full-range int8 values included (the int32 sums wrap into the low byte under PassThrough)."""
+    import gpu_util
+    if dtype == "f16":
+        inp = uniform_f16((36, 56, 56, 256), -1, 1, 1020)
+        wei = uniform_f16((512, 1, 1, 256), -1, 1, 1021)
+        out = gpu_util.conv2d_fwd(inp, wei, (1, 1), (1, 1), (0, 0))
+        _f16_close(out, fast.conv2d_fwd_f16(inp, wei, (1, 1), (1, 1), (0, 0)))
+    else:
+        inp = uniform_int8((256, 57, 55, 256), -128, 127, 1022)
+        wei = uniform_int8((512, 1, 1, 256), -128, 127, 1023)
+        out = gpu_util.conv2d_fwd(inp, wei, (2, 2), (1, 1), (0, 0))
+        np.testing.assert_array_equal(out, fast.conv2d_fwd_i8(inp, wei, (2, 2), (1, 1), (0, 0)))
+
+
+def test_conv2d_pointwise_instance_refuses_other_shapes():
+    import ctypes as C
+    import gpu_util
+    L = capi.lib()
+    pw = gpu_util.conv_instance(capi.OP_CONV2D_FWD_F16, "Pointwise")
+    ok = capi.Conv2dDesc(2, 512, 256, 8, 8, 1, 1, 8, 8, 1, 1, 1, 1, 0, 0, 0, 0)
+    assert L.ckx_conv2d_fwd_is_supported(capi.OP_CONV2D_FWD_F16, C.byref(ok), 0, pw) == capi.OK
+    for d in (capi.Conv2dDesc(2, 256, 256, 8, 8, 1, 1, 8, 8, 1, 1, 1, 1, 0, 0, 0, 0),      # K = 256
+              capi.Conv2dDesc(2, 512, 64, 8, 8, 1, 1, 8, 8, 1, 1, 1, 1, 0, 0, 0, 0),       # 128-byte pixels
+              capi.Conv2dDesc(2, 512, 256, 8, 8, 1, 1, 10, 10, 1, 1, 1, 1, 1, 1, 1, 1),    # padded
+              capi.Conv2dDesc(2, 512, 256, 8, 8, 3, 3, 6, 6, 1, 1, 1, 1, 0, 0, 0, 0)):     # 3x3
+        assert L.ckx_conv2d_fwd_is_supported(capi.OP_CONV2D_FWD_F16, C.byref(d), 0, pw) == capi.UNSUPPORTED
+        assert L.ckx_conv2d_fwd_is_supported(capi.OP_CONV2D_FWD_F16, C.byref(d), 0, -1) == capi.OK
+    # the residual functor stays with the tile kernel
+    assert L.ckx_conv2d_fwd_is_supported(capi.OP_CONV2D_FWD_F16, C.byref(ok), capi.EPI_ADD_RELU_ADD, pw) == capi.UNSUPPORTED

@@ -205,7 +205,8 @@ def test_conv2d_bias_relu_on_the_input_patch_kernel(shape, auto):
     inp = uniform_f16((N, Hi, Wi, 64), -1, 1, 950 + Hi)
     wei = uniform_f16((64, 3, 3, 64), -0.5, 0.5, 951)
     bias = uniform_f16((64,), -2, 2, 952)
-    inst = capi.INSTANCE_AUTO if auto else capi.lib().ckx_num_instances(capi.OP_CONV2D_FWD_F16) - 1
+    import gpu_util
+    inst = capi.INSTANCE_AUTO if auto else gpu_util.conv_instance(capi.OP_CONV2D_FWD_F16, "Patch")
     ref = lit.conv2d_fwd_bias_relu_f16(inp, wei, bias, None, (1, 1), (1, 1), p)
     out = _conv(inp, wei, bias, None, (1, 1), (1, 1), p, inst)
     _close(out, ref)
@@ -213,3 +214,20 @@ def test_conv2d_bias_relu_on_the_input_patch_kernel(shape, auto):
     resi = uniform_f16(ref.shape, -2, 2, 953)
     _close(_conv(inp, wei, bias, resi, (1, 1), (1, 1), p, inst),
            lit.conv2d_fwd_bias_relu_f16(inp, wei, bias, resi, (1, 1), (1, 1), p))
+
+
+@pytest.mark.parametrize("shape", [(3, 256, 512, 7, 5, (1, 1)), (2, 128, 1024, 9, 9, (2, 2)), (40, 256, 512, 56, 56, (2, 2))])
+def test_conv2d_bias_relu_on_the_pointwise_kernel(shape):
+    """1x1 layers on the weight-stationary kernel with the bias + ReLU functor compiled in (explicit instance for the
+    small shapes, the automatic choice for the large one)."""
+    import gpu_util
+    N, C, K, Hi, Wi, s = shape
+    inp = uniform_f16((N, Hi, Wi, C), -1, 1, 960 + Hi)
+    wei = uniform_f16((K, 1, 1, C), -0.5, 0.5, 961)
+    bias = uniform_f16((K,), -2, 2, 962)
+    big = N * Hi * Wi > 100000
+    inst = capi.INSTANCE_AUTO if big else gpu_util.conv_instance(capi.OP_CONV2D_FWD_F16, "Pointwise")
+    ref = (fast if big else lit).conv2d_fwd_bias_relu_f16(inp, wei, bias, None, s, (1, 1), (0, 0))
+    out = _conv(inp, wei, bias, None, s, (1, 1), (0, 0), inst)
+    _close(out, ref)
+    assert (out == 0).any() and (out > 0).any()
