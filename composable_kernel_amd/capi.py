@@ -29,6 +29,7 @@ SYMBOLS = [
     "ckx_gemm_splitk_workspace_bytes", "ckx_gemm_i8_splitk", "ckx_gemm_f16_splitk",
     "ckx_gemm_f16_multiple_d_is_supported", "ckx_gemm_f16_multiple_d", "ckx_conv2d_fwd_bias_activation_f16",
     "ckx_conv2d_fwd_is_supported", "ckx_conv2d_fwd_i8", "ckx_conv2d_fwd_f16", "ckx_conv2d_fwd_workspace_bytes",
+    "ckx_convnd_fwd_is_supported", "ckx_convnd_fwd", "ckx_convnd_fwd_workspace_bytes",
     "ckx_batched_gemm_gemm_f16_is_supported", "ckx_batched_gemm_gemm_f16", "ckx_time_launches",
     "ckx_batched_gemm_softmax_gemm_f16_is_supported", "ckx_batched_gemm_softmax_gemm_f16",
 ]
@@ -38,6 +39,21 @@ class Conv2dDesc(C.Structure):
     _fields_ = [(n, C.c_int32) for n in (
         "N", "K", "C", "Hi", "Wi", "Y", "X", "Ho", "Wo", "stride_h", "stride_w", "dilation_h",
         "dilation_w", "pad_top", "pad_left", "pad_bottom", "pad_right")]
+
+
+class ConvNdDesc(C.Structure):
+    """ckx_convnd_desc: the first ndim entries of every array are used, slowest dimension first."""
+    _fields_ = [("ndim", C.c_int32), ("N", C.c_int32), ("K", C.c_int32), ("C", C.c_int32)] + [
+        (n, C.c_int32 * 3) for n in ("in_", "filter", "out", "stride", "dilation", "pad_left", "pad_right")]
+
+    @classmethod
+    def make(cls, N, K, C_, in_len, filt, out_len, strides, dilations, left_pads, right_pads):
+        nd = len(in_len)
+        if nd not in (1, 2, 3) or any(len(v) != nd for v in (filt, out_len, strides, dilations, left_pads, right_pads)):
+            raise ValueError("1, 2 or 3 spatial dimensions, every vector of that length")
+        arr = lambda v: (C.c_int32 * 3)(*([int(x) for x in v] + [0] * (3 - nd)))
+        return cls(nd, int(N), int(K), int(C_), arr(in_len), arr(filt), arr(out_len), arr(strides), arr(dilations),
+                   arr(left_pads), arr(right_pads))
 
 
 LAUNCH_FN = C.CFUNCTYPE(C.c_int, C.c_void_p)
@@ -100,6 +116,11 @@ def lib():
     L.ckx_conv2d_fwd_f16.argtypes = [vp, vp, vp, dp, C.c_int, vp, i64, vp]
     L.ckx_conv2d_fwd_workspace_bytes.restype = i64
     L.ckx_conv2d_fwd_workspace_bytes.argtypes = [C.c_int, dp, C.c_int]
+    ndp = C.POINTER(ConvNdDesc)
+    L.ckx_convnd_fwd_is_supported.argtypes = [C.c_int, ndp, C.c_int, C.c_int]
+    L.ckx_convnd_fwd.argtypes = [C.c_int, vp, vp, vp, ndp, C.c_int, f32, f32, C.c_int, vp, i64, vp]
+    L.ckx_convnd_fwd_workspace_bytes.restype = i64
+    L.ckx_convnd_fwd_workspace_bytes.argtypes = [C.c_int, ndp, C.c_int]
     gg = [i32] * 9 + [i64] * 4 + [C.c_int]
     L.ckx_batched_gemm_gemm_f16_is_supported.argtypes = gg
     L.ckx_batched_gemm_gemm_f16.argtypes = [vp] * 4 + gg + [vp]

@@ -648,6 +648,160 @@ int run_conv(int op, const void* in, const void* wei, void* out, const ckx_conv2
     return CKX_OK;
 }
 
+// ---------------------------------------------------------- conv forward, 1 / 2 / 3 spatial dimensions
+// One and two dimensions are the 2-D problem (a 1-D conv is a 2-D conv on images one pixel high: same taps in
+// the same order); so is a 3-D problem whose depth axis is not convolved (one tap, stride 1, no padding):
+// N * D images.
+bool convnd_as_2d(const ckx_convnd_desc* d, ckx_conv2d_desc& o)
+{
+    std::memset(&o, 0, sizeof(o));
+    o.N = d->N, o.K = d->K, o.C = d->C;
+    if(d->ndim == 1)
+    {
+        o.Hi = 1, o.Y = 1, o.Ho = 1, o.stride_h = 1, o.dilation_h = 1;
+        o.Wi = d->in[0], o.X = d->filter[0], o.Wo = d->out[0], o.stride_w = d->stride[0];
+        o.dilation_w = d->dilation[0], o.pad_left = d->pad_left[0], o.pad_right = d->pad_right[0];
+        return true;
+    }
+    const int h = d->ndim - 2; // index of the H entries
+    if(d->ndim == 3)
+    {
+        if(d->filter[0] != 1 || d->stride[0] != 1 || d->pad_left[0] != 0 || d->pad_right[0] != 0 ||
+           d->in[0] != d->out[0] || d->in[0] <= 0 || (long)d->N * d->in[0] >= (1l << 31))
+            return false;
+        o.N = d->N * d->in[0];
+    }
+    o.Hi = d->in[h], o.Wi = d->in[h + 1], o.Y = d->filter[h], o.X = d->filter[h + 1];
+    o.Ho = d->out[h], o.Wo = d->out[h + 1], o.stride_h = d->stride[h], o.stride_w = d->stride[h + 1];
+    o.dilation_h = d->dilation[h], o.dilation_w = d->dilation[h + 1];
+    o.pad_top = d->pad_left[h], o.pad_left = d->pad_left[h + 1];
+    o.pad_bottom = d->pad_right[h], o.pad_right = d->pad_right[h + 1];
+    return true;
+}
+
+int check_convnd(int op, const ckx_convnd_desc* d, int epi, int instance, ckx_conv2d_desc& as2d, bool& is2d)
+{
+    is2d = false;
+    if(!d)
+        return fail(CKX_INVALID_VALUE, "null conv descriptor");
+    if(op != CKX_OP_CONV2D_FWD_I8 && op != CKX_OP_CONV2D_FWD_F16)
+        return fail(CKX_INVALID_VALUE, "not a conv operator family");
+    if(d->ndim < 1 || d->ndim > 3)
+        return fail(CKX_INVALID_VALUE, "1, 2 or 3 spatial dimensions");
+    if((is2d = convnd_as_2d(d, as2d)))
+        return check_conv(op, &as2d, epi, instance);
+    // three convolved dimensions: the tile instances
+    const int es = op == CKX_OP_CONV2D_FWD_I8 ? 1 : 2;
+    if(instance != CKX_INSTANCE_AUTO && (instance < 0 || instance >= kNumConvInsts))
+        return fail(CKX_INVALID_VALUE, "no such instance");
+    if(instance >= kNumTiles)
+        return fail(CKX_UNSUPPORTED, "the input-patch and pointwise instances cover two spatial dimensions");
+    if(epi < CKX_EPI_PASSTHROUGH || epi > CKX_EPI_REQUANT_RND || !epilogue_fits_dtype(es, epi))
+        return fail(CKX_INVALID_VALUE, "epilogue not available for this operator");
+    if(d->N < 0 || d->K < 0 || d->C < 0)
+        return fail(CKX_INVALID_VALUE, "bad conv geometry");
+    long in_px = d->N, out_px = d->N, taps = 1;
+    for(int i = 0; i < 3; ++i)
+    {
+        if(d->in[i] <= 0 || d->filter[i] <= 0 || d->out[i] < 0 || d->stride[i] <= 0 || d->dilation[i] <= 0 ||
+           d->pad_left[i] < 0 || d->pad_right[i] < 0)
+            return fail(CKX_INVALID_VALUE, "bad conv geometry");
+        if(d->in[i] > 16384 || d->pad_left[i] >= 16384 || (long)(d->filter[i] - 1) * d->dilation[i] >= 16384)
+            return fail(CKX_UNSUPPORTED, "spatial extents above 16384 are not addressed");
+        // conv_util.cpp:103-114
+        const int o = (d->in[i] + d->pad_left[i] + d->pad_right[i] - ((d->filter[i] - 1) * d->dilation[i] + 1)) /
+                          d->stride[i] + 1;
+        if(o != d->out[i])
+            return fail(CKX_UNSUPPORTED, "output spatial lengths do not match the conv geometry");
+        in_px *= d->in[i], out_px *= d->out[i], taps *= d->filter[i];
+        if(in_px >= (1l << 31) || out_px >= (1l << 31) || taps >= (1l << 31))
+            return fail(CKX_UNSUPPORTED, "tensors of 2 GiB or more are not addressed");
+    }
+    if(((long)d->C * es) % 16)
+        return fail(CKX_UNSUPPORTED, "C must be a multiple of 16 bytes");
+    // (device_convnd_fwd_xdl_nhwc_kyxc_nhwk.hpp:883-890 refuses tensors above 2 GB as well)
+    if(in_px * d->C * es >= (1l << 31) || (long)d->K * taps * d->C * es >= (1l << 31) ||
+       out_px * d->K * es >= (1l << 31) || taps * d->C >= (1l << 31))
+        return fail(CKX_UNSUPPORTED, "tensors of 2 GiB or more are not addressed");
+    return CKX_OK;
+}
+
+long convnd_workspace_bytes(int op, const ckx_convnd_desc* d, int instance)
+{
+    ckx_conv2d_desc d2;
+    bool is2d;
+    if(check_convnd(op, d, CKX_EPI_PASSTHROUGH, instance, d2, is2d) != CKX_OK)
+        return 0;
+    if(is2d)
+        return conv_workspace_bytes(op, &d2, instance);
+    const int es = op == CKX_OP_CONV2D_FWD_I8 ? 1 : 2;
+    const long M = (long)d->N * d->out[0] * d->out[1] * d->out[2];
+    if(M <= 0 || d->K <= 0)
+        return 0;
+    const Plan pl = make_plan((int)M, d->K, d->filter[0] * d->filter[1] * d->filter[2] * d->C * es, instance, 1l << 60);
+    return pl.ksplit > 1 ? (long)pl.ksplit * M * d->K * 4 : 0;
+}
+
+int run_convnd(int op, const void* in, const void* wei, void* out, const ckx_convnd_desc* d, int epi, float sg,
+               float sr, int instance, void* ws, long ws_bytes, void* stream)
+{
+    ckx_conv2d_desc d2;
+    bool is2d;
+    int st = check_convnd(op, d, epi, instance, d2, is2d);
+    if(st != CKX_OK)
+        return st;
+    if(is2d)
+        return run_conv(op, in, wei, out, &d2, epi, sg, sr, instance, ws, ws_bytes, stream);
+    const int es = op == CKX_OP_CONV2D_FWD_I8 ? 1 : 2;
+    const int M = d->N * d->out[0] * d->out[1] * d->out[2], N = d->K;
+    const int K = d->filter[0] * d->filter[1] * d->filter[2] * d->C;
+    if(M == 0 || N == 0)
+        return CKX_OK;
+    if(!in || !wei || !out)
+        return fail(CKX_INVALID_VALUE, "null operand pointer");
+    if((reinterpret_cast<uintptr_t>(in) | reinterpret_cast<uintptr_t>(wei)) & 15)
+        return fail(CKX_UNSUPPORTED, "input and weight must be 16-byte aligned");
+    if(ws && (reinterpret_cast<uintptr_t>(ws) & 15))
+        return fail(CKX_INVALID_VALUE, "workspace must be 16-byte aligned");
+    const Plan pl         = make_plan(M, N, K * es, instance, ws ? ws_bytes : 0);
+    const TileInstance& t = kTiles[pl.tile];
+    ckx::GemmArgs g;
+    std::memset(&g, 0, sizeof(g));
+    g.a = in, g.b = wei, g.c = out;
+    g.M = M, g.N = N, g.K = K;
+    g.lda = 0, g.ldb = K, g.ldc = N;
+    g.a_bytes    = (uint32_t)((long)d->N * d->in[0] * d->in[1] * d->in[2] * d->C * es);
+    g.b_bytes    = (uint32_t)((long)N * K * es);
+    g.tiles_m    = (M + t.bm - 1) / t.bm;
+    g.tiles_n    = (N + t.bn - 1) / t.bn;
+    g.epi        = epi;
+    g.scale_gemm = sg;
+    g.scale_relu = sr;
+    g.nt_store   = es == 1 && (long)M * N * es >= stream_output_bytes();
+    g.cv.Di = d->in[0], g.cv.Hi = d->in[1], g.cv.Wi = d->in[2], g.cv.C = d->C;
+    g.cv.sD = d->stride[0], g.cv.sH = d->stride[1], g.cv.sW = d->stride[2];
+    g.cv.dD = d->dilation[0], g.cv.dH = d->dilation[1], g.cv.dW = d->dilation[2];
+    g.cv.pF = d->pad_left[0], g.cv.pT = d->pad_left[1], g.cv.pL = d->pad_left[2];
+    g.cv.div_dhowo = make_magic((uint32_t)(d->out[0] * d->out[1] * d->out[2]));
+    g.cv.div_howo  = make_magic((uint32_t)(d->out[1] * d->out[2]));
+    g.cv.div_wo    = make_magic((uint32_t)d->out[2]);
+    g.cv.div_yxc   = make_magic((uint32_t)(d->filter[1] * d->filter[2] * d->C));
+    g.cv.div_xc    = make_magic((uint32_t)(d->filter[2] * d->C));
+    g.cv.div_c     = make_magic((uint32_t)d->C);
+    g.ksplit = pl.ksplit;
+    g.nk_per = pl.nk_per;
+    g.ws     = ws;
+    const tile_launch_fn launch = ckx::conv3d_tile(es == 1 ? ckx::DT_I8 : ckx::DT_F16, pl.tile);
+    if(!launch)
+        return fail(CKX_UNSUPPORTED, "no kernel variant for this instance");
+    hipError_t e = launch(g, g.tiles_m * g.tiles_n * g.ksplit, (hipStream_t)stream);
+    if(e == hipSuccess && g.ksplit > 1)
+        e = es == 1 ? launch_reduce<ckx::DT_I8>(g, (hipStream_t)stream) : launch_reduce<ckx::DT_F16>(g, (hipStream_t)stream);
+    if(e != hipSuccess)
+        return hip_fail(e, t.name);
+    return CKX_OK;
+}
+
 } // namespace
 
 extern "C" {
@@ -863,6 +1017,26 @@ int ckx_conv2d_fwd_f16(const void* in, const void* wei, void* out, const ckx_con
 {
     return run_conv(CKX_OP_CONV2D_FWD_F16, in, wei, out, desc, CKX_EPI_PASSTHROUGH, 1.0f, 1.0f, instance,
                     workspace, workspace_bytes, stream);
+}
+
+int ckx_convnd_fwd_is_supported(int op, const ckx_convnd_desc* desc, int epilogue, int instance)
+{
+    ckx_conv2d_desc d2;
+    bool is2d;
+    return check_convnd(op, desc, epilogue, instance, d2, is2d);
+}
+
+int64_t ckx_convnd_fwd_workspace_bytes(int op, const ckx_convnd_desc* desc, int instance)
+{
+    return convnd_workspace_bytes(op, desc, instance);
+}
+
+int ckx_convnd_fwd(int op, const void* in, const void* wei, void* out, const ckx_convnd_desc* desc, int epilogue,
+                   float scale_gemm, float scale_relu, int instance, void* workspace, int64_t workspace_bytes,
+                   void* stream)
+{
+    return run_convnd(op, in, wei, out, desc, epilogue, scale_gemm, scale_relu, instance, workspace, workspace_bytes,
+                      stream);
 }
 
 int ckx_batched_gemm_gemm_f16_is_supported(int32_t M, int32_t N, int32_t K, int32_t O, int32_t batch,

@@ -97,6 +97,11 @@ struct ConvGeom
     MagicDiv div_wo;   // Wo
     MagicDiv div_xc;   // X*C
     MagicDiv div_c;    // C
+    // three spatial dimensions (device_convnd_fwd_xdl_nhwc_kyxc_nhwk.hpp, NumDimSpatial == 3):
+    //   row m -> (n, do, ho, wo), k -> (z, y, x, c); depth extent, stride, dilation, front padding
+    int Di, sD, dD, pF;
+    MagicDiv div_dhowo; // Do*Ho*Wo
+    MagicDiv div_yxc;   // Y*X*C
 };
 
 struct GemmArgs
@@ -391,7 +396,7 @@ __device__ __forceinline__ void store_row16_f16_fused(_Float16* crow, int n0, in
 // D loads of that epilogue leave the compiler with "some global load may be outstanding" at the top of
 // the K loop, which it answers with s_waitcnt vmcnt(0) in every iteration -- also for launches that
 // never run that epilogue -- and that wait holds the loop until the prefetched K tile has landed.
-template <int DT, int BM, int BN, int WM, int WN, int BKB, int NST, bool IM2COL, bool TA = false, bool TB = false,
+template <int DT, int BM, int BN, int WM, int WN, int BKB, int NST, int IM2COL, bool TA = false, bool TB = false,
           bool FUSED = false>
 struct GemmTile
 {
@@ -417,7 +422,7 @@ struct GemmTile
     static_assert(WTM % 16 == 0 && WTN % 64 == 0, "wave tile must be 16k x 64k");
     static_assert((BM * CPR) % NT == 0 && (BN * CPR) % NT == 0, "tile rows must split over the waves");
 
-    static_assert(!(IM2COL && (TA || TB)), "the im2col view is K-contiguous");
+    static_assert(IM2COL >= 0 && IM2COL <= 2 && !(IM2COL != 0 && (TA || TB)), "the im2col view (1: two spatial dimensions, 2: three) is K-contiguous");
     static_assert(!FUSED || (DT == DT_F16 && !TA && !TB), "D-operand epilogues: fp16, K-contiguous operands");
     static_assert((!TA || (BM >= 64 && BM * ES <= 1024)) && (!TB || (BN >= 64 && BN * ES <= 1024)),
                   "a K-major tile row is 64..1024 bytes");
@@ -477,6 +482,7 @@ struct GemmTile
         static_assert(RPI == 8, "one chunk position per thread");
         uint32_t a_off[NLA];  // dense: byte offset of (row, chunk) at K tile 0, or kOutOfRange
         uint32_t a_hw0[NLA]; // im2col: top-left input coordinate of the row's window, (hi0 << 16) | (wi0 & 0xffff)
+        int a_d0[IM2COL == 2 ? NLA : 1]; // three spatial dimensions: front input depth of the row's window
         uint32_t b_off[NLB];
         const uint32_t kb = ((uint32_t)(lane % CPR) ^ (uint32_t)((lane / CPR) & 7)) << 4; // chunk byte offset in a K tile
         // K-major operands: k row (within a K tile) of this thread's slot 0; slot j is j * NW * rows-per-load further
@@ -506,7 +512,7 @@ struct GemmTile
                 const uint32_t r  = (uint32_t)((j * NW + wave) * RPI + lane / CPR);
                 const uint32_t gm = (uint32_t)tm * BM + r;
                 const bool ok     = live && gm < (uint32_t)p.M;
-                if constexpr(!IM2COL)
+                if constexpr(IM2COL == 0)
                 {
                     a_off[j] = ok ? a_batch + gm * (uint32_t)p.lda * ES + kb : kOutOfRange;
                     a_hw0[j] = 0;
@@ -515,22 +521,39 @@ struct GemmTile
                 {
                     if(ok)
                     {
-                        const uint32_t n   = magic_div(gm, p.cv.div_howo);
-                        const uint32_t rem = gm - n * p.cv.div_howo.d;
+                        uint32_t img = 0, rem = gm; // img: 2-D image index n, or n * Di + front depth
+                        int d0 = 0;
+                        if constexpr(IM2COL == 2)
+                        {
+                            const uint32_t n  = magic_div(gm, p.cv.div_dhowo);
+                            const uint32_t r3 = gm - n * p.cv.div_dhowo.d;
+                            const uint32_t od = magic_div(r3, p.cv.div_howo);
+                            rem               = r3 - od * p.cv.div_howo.d;
+                            d0                = (int)od * p.cv.sD - p.cv.pF;
+                            img               = (uint32_t)((int)(n * (uint32_t)p.cv.Di) + d0);
+                            a_d0[j]           = d0;
+                        }
+                        else
+                        {
+                            img = magic_div(gm, p.cv.div_howo);
+                            rem = gm - img * p.cv.div_howo.d;
+                        }
                         const uint32_t ho  = magic_div(rem, p.cv.div_wo);
                         const uint32_t wo  = rem - ho * p.cv.div_wo.d;
                         const int hi0      = (int)ho * p.cv.sH - p.cv.pT;
                         const int wi0      = (int)wo * p.cv.sW - p.cv.pL;
                         a_hw0[j]           = ((uint32_t)hi0 << 16) | ((uint32_t)wi0 & 0xffffu);
-                        // byte offset of the window's top-left pixel; may be "negative" (wraps), the
+                        // byte offset of the window's top-left (front) pixel; may be "negative" (wraps), the
                         // sum with a valid tap's offset is always inside the tensor
-                        a_off[j] = (uint32_t)(((int)(n * (uint32_t)p.cv.Hi) + hi0) * p.cv.Wi + wi0) *
+                        a_off[j] = (uint32_t)(((int)(img * (uint32_t)p.cv.Hi) + hi0) * p.cv.Wi + wi0) *
                                    (uint32_t)(p.cv.C * ES);
                     }
                     else
                     {
                         a_hw0[j] = 0xC000C000u; // (-16384, -16384): every tap out of range
                         a_off[j] = 0;
+                        if constexpr(IM2COL == 2)
+                            a_d0[j] = 0;
                     }
                 }
             }
@@ -565,7 +588,8 @@ struct GemmTile
             uint32_t k_oob;   // top bit set for chunks past K: OR-ed into the offset (arithmetic on
                               // purpose: a select feeding the loads becomes divergent branches)
             int tap_dh, tap_dw; // im2col: decoded ONCE per thread and K tile, every slot of a thread
-            uint32_t tap_off;   // sits at the same chunk position
+            int tap_dd;         // sits at the same chunk position
+            uint32_t tap_off;
             bool tap_ok;
         };
         auto load_ctx = [&](int kt, int stage) {
@@ -577,19 +601,26 @@ struct GemmTile
             c.k0a   = TA ? (uint32_t)kt * KE * (uint32_t)p.lda * ES : 0u;
             c.k0b   = TB ? (uint32_t)kt * KE * (uint32_t)p.ldb * ES : 0u;
             c.klim  = p.K - kt * KE;
-            c.tap_dh = c.tap_dw = 0;
-            c.tap_off           = 0;
+            c.tap_dh = c.tap_dw = c.tap_dd = 0;
+            c.tap_off                      = 0;
             c.tap_ok            = true;
-            if constexpr(IM2COL)
+            if constexpr(IM2COL != 0)
             {
                 const uint32_t ke  = (c.k0 + kb) / ES; // element index along GEMM-K
-                const uint32_t y   = magic_div(ke, p.cv.div_xc);
-                const uint32_t rem = ke - y * p.cv.div_xc.d;
+                uint32_t kyx = ke;
+                if constexpr(IM2COL == 2)
+                {
+                    const uint32_t z = magic_div(ke, p.cv.div_yxc);
+                    kyx              = ke - z * p.cv.div_yxc.d;
+                    c.tap_dd         = (int)z * p.cv.dD;
+                }
+                const uint32_t y   = magic_div(kyx, p.cv.div_xc);
+                const uint32_t rem = kyx - y * p.cv.div_xc.d;
                 const uint32_t x   = magic_div(rem, p.cv.div_c);
                 const uint32_t cc  = rem - x * p.cv.div_c.d;
                 c.tap_dh           = (int)y * p.cv.dH;
                 c.tap_dw           = (int)x * p.cv.dW;
-                c.tap_off          = ((uint32_t)(c.tap_dh * p.cv.Wi + c.tap_dw) * (uint32_t)p.cv.C + cc) * ES;
+                c.tap_off          = ((uint32_t)((c.tap_dd * p.cv.Hi + c.tap_dh) * p.cv.Wi + c.tap_dw) * (uint32_t)p.cv.C + cc) * ES;
                 c.tap_ok           = ke < (uint32_t)p.K;
             }
             return c;
@@ -601,13 +632,15 @@ struct GemmTile
                 uint32_t voff;
                 if constexpr(TA)
                     voff = (a_off[j] + c.k0a) | (~(uint32_t)((int)(trow_a + j * NW * (1024 / (BM * ES))) - c.klim) & kOutOfRange);
-                else if constexpr(!IM2COL)
+                else if constexpr(IM2COL == 0)
                     voff = (a_off[j] + c.k0) | c.k_oob;
                 else
                 {
                     const int hi0 = (int)a_hw0[j] >> 16, wi0 = (int)(a_hw0[j] << 16) >> 16;
-                    const bool ok = c.tap_ok && (uint32_t)(hi0 + c.tap_dh) < (uint32_t)p.cv.Hi &&
-                                    (uint32_t)(wi0 + c.tap_dw) < (uint32_t)p.cv.Wi;
+                    bool ok = c.tap_ok && (uint32_t)(hi0 + c.tap_dh) < (uint32_t)p.cv.Hi &&
+                              (uint32_t)(wi0 + c.tap_dw) < (uint32_t)p.cv.Wi;
+                    if constexpr(IM2COL == 2)
+                        ok = ok && (uint32_t)(a_d0[j] + c.tap_dd) < (uint32_t)p.cv.Di;
                     voff = (a_off[j] + c.tap_off) | (ok ? 0u : kOutOfRange);
                 }
                 __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_a, (lds_ptr_t)(c.sa + (j * NW + wave) * 1024), 16,
@@ -1132,7 +1165,7 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(const GemmArgs p)
     }
 }
 
-template <int DT, int BM, int BN, int WM, int WN, int BKB, int NST, bool IM2COL, bool TA = false, bool TB = false,
+template <int DT, int BM, int BN, int WM, int WN, int BKB, int NST, int IM2COL, bool TA = false, bool TB = false,
           bool FUSED = false>
 __global__ __launch_bounds__(WM* WN * 64) void gemm_tile_kernel(const GemmArgs p)
 {

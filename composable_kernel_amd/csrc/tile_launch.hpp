@@ -40,7 +40,7 @@ inline int num_cus()
 
 // Persistent launch: at most (workgroups that fit a CU) x (CUs) workgroups, a multiple of 8 so
 // that workgroup b always lands on XCD b % 8 together with the tiles b, b + grid, ...
-template <int DT, int BM, int BN, int WM, int WN, int BKB, int NST, bool IM2COL, bool TA = false, bool TB = false,
+template <int DT, int BM, int BN, int WM, int WN, int BKB, int NST, int IM2COL, bool TA = false, bool TB = false,
           bool FUSED = false>
 hipError_t launch_tile(const GemmArgs& a, int tiles, hipStream_t s)
 {
@@ -68,5 +68,8 @@ hipError_t launch_tile(const GemmArgs& a, int tiles, hipStream_t s)
 // (DT_*), A K-major (a_kmajor: column-major "km") and / or B K-major (b_kmajor: row-major "kn");
 // null when that tile shape has no such variant (fewer than 64 rows)
 tile_launch_fn layout_tile(int dt, int tile, bool a_kmajor, bool b_kmajor);
+
+// conv forward with three spatial dimensions (conv3d.hip): launcher of tile instance `tile` for DT_I8 / DT_F16
+tile_launch_fn conv3d_tile(int dt, int tile);
 
 } // namespace ckx

@@ -407,6 +407,55 @@ class DeviceConv2dFwdF16(_DeviceConvFwd):
                                              a.p_workspace_ or 0, a.workspace_bytes_, C.c_void_p(stream or 0))
 
 
+class _DeviceConvNdFwd(BaseOperator):
+    """DeviceConvFwd<InOp, WeiOp, OutOp> as implemented by DeviceConvNDFwdXdl_Input_N_Hi_Wi_C_Weight_K_Y_X_C_
+    Output_N_Ho_Wo_K<..., NumDimSpatial> (device_convnd_fwd_xdl_nhwc_kyxc_nhwk.hpp:76-1046): NWC / NHWC / NDHWC
+    input, KXC / KYXC / KZYXC weight, NWK / NHWK / NDHWK output; every vector has NumDimSpatial entries."""
+
+    def __init__(self, NumDimSpatial=2, instance=capi.INSTANCE_AUTO):
+        super().__init__(instance)
+        if NumDimSpatial not in (1, 2, 3):
+            raise ValueError("NumDimSpatial is 1, 2 or 3")
+        self.NumDimSpatial = NumDimSpatial
+
+    def MakeArgumentPointer(self, p_in, p_wei, p_out, N, K, C_, input_spatial_lengths,
+                            filter_spatial_lengths, output_spatial_lengths, conv_filter_strides,
+                            conv_filter_dilations, input_left_pads, input_right_pads, in_element_op=None,
+                            wei_element_op=None, out_element_op=None):
+        if len(input_spatial_lengths) != self.NumDimSpatial:
+            raise ValueError(f"this operator has NumDimSpatial == {self.NumDimSpatial}")
+        d = capi.ConvNdDesc.make(N, K, C_, input_spatial_lengths, filter_spatial_lengths, output_spatial_lengths,
+                                 conv_filter_strides, conv_filter_dilations, input_left_pads, input_right_pads)
+        return _ConvArgument(p_in, p_wei, p_out, d, out_element_op or PassThrough())
+
+    def _supported(self, a):
+        return capi.lib().ckx_convnd_fwd_is_supported(self.op_family, C.byref(a.desc), a.out_op.epilogue, self.instance)
+
+    def GetWorkSpaceSize(self, a):
+        return int(capi.lib().ckx_convnd_fwd_workspace_bytes(self.op_family, C.byref(a.desc), self.instance))
+
+    def _launch(self, a, stream):
+        sg = getattr(a.out_op, "scale_gemm", 1.0)
+        sr = getattr(a.out_op, "scale_relu", 1.0)
+        return capi.lib().ckx_convnd_fwd(self.op_family, a.p_in, a.p_wei, a.p_out, C.byref(a.desc), a.out_op.epilogue,
+                                         sg, sr, self.instance, a.p_workspace_ or 0, a.workspace_bytes_,
+                                         C.c_void_p(stream or 0))
+
+
+    @classmethod
+    def GetInstances(cls, NumDimSpatial=2):
+        """ConvolutionFwdInstances<T, T, T>::Get<NumDimSpatial>() (library/include/ck/library/utility/conv_util.hpp:288-397)"""
+        return [cls(NumDimSpatial, i) for i in range(capi.lib().ckx_num_instances(cls.op_family))]
+
+
+class DeviceConvNdFwdInt8(_DeviceConvNdFwd):
+    op_family = capi.OP_CONV2D_FWD_I8
+
+
+class DeviceConvNdFwdF16(_DeviceConvNdFwd):
+    op_family = capi.OP_CONV2D_FWD_F16
+
+
 class DeviceConv2dFwdBiasActivationF16(_DeviceConvFwd):
     """DeviceConvFwdBiasActivation<InOp, WeiOp, AddRelu> and DeviceConvFwdBiasActivationAdd<..., AddReluAdd>
     (device_conv_fwd_bias_activation.hpp:18-41, device_conv_fwd_bias_activation_add.hpp): p_bias is a

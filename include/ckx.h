@@ -229,6 +229,30 @@ int ckx_conv2d_fwd_bias_activation_f16(const void* p_in, const void* p_wei, void
                                        const void* p_resi, const ckx_conv2d_desc* desc, int out_op, int instance,
                                        void* p_workspace, int64_t workspace_bytes, void* stream);
 
+/* ---- conv forward with 1, 2 or 3 spatial dimensions: NWC / NHWC / NDHWC input, KXC / KYXC / KZYXC
+ * weight, NWK / NHWK / NDHWK output --------------------------------------------------------------
+ * Replaces DeviceConvFwd<PassThrough, PassThrough, OutOp>::MakeArgumentPointer + Run as implemented by
+ * DeviceConvNDFwdXdl_Input_N_Hi_Wi_C_Weight_K_Y_X_C_Output_N_Ho_Wo_K<..., NumDimSpatial>
+ * (device_convnd_fwd_xdl_nhwc_kyxc_nhwk.hpp:76-1046; the instances conv_util.hpp:288-397 hands out for
+ * Get<1>(), Get<2>(), Get<3>()). The vectors of the reference interface arrive as arrays whose first
+ * `ndim` entries are used, slowest dimension first ((D,) (H,) W). op is CKX_OP_CONV2D_FWD_I8 or _F16 (the
+ * data type; the families and their instance lists are shared by every dimensionality), epilogue one of
+ * PassThrough / requant for int8, PassThrough for fp16. One and two dimensions (and three with an
+ * unconvolved depth axis) run as the 2-D problem; three convolved dimensions take the tile instances. */
+typedef struct ckx_convnd_desc
+{
+    int32_t ndim;
+    int32_t N, K, C;
+    int32_t in[3], filter[3], out[3];
+    int32_t stride[3], dilation[3], pad_left[3], pad_right[3];
+} ckx_convnd_desc;
+
+int ckx_convnd_fwd_is_supported(int op, const ckx_convnd_desc* desc, int epilogue, int instance);
+int64_t ckx_convnd_fwd_workspace_bytes(int op, const ckx_convnd_desc* desc, int instance);
+int ckx_convnd_fwd(int op, const void* p_in, const void* p_wei, void* p_out, const ckx_convnd_desc* desc,
+                   int epilogue, float scale_gemm, float scale_relu, int instance, void* p_workspace,
+                   int64_t workspace_bytes, void* stream);
+
 /* ---- batched fused GEMM-GEMM, fp16:  C[g] = half( half(A[g]*B0[g]) * B1[g] ) --
  * The reference snapshot has no such operator; the surface is upstream's
  * DeviceBatchedGemmGemm::MakeArgumentPointer (device_batched_gemm_gemm.hpp:15-56 of

@@ -8,6 +8,8 @@
 //       library/include/ck/library/reference_tensor_operation/cpu/reference_gemm.hpp:57-88
 //   cko_conv2d_fwd_{f32,f16,i8}      ReferenceConvFwd (NumDimSpatial == 2 branch)
 //       library/include/ck/library/reference_tensor_operation/cpu/reference_conv_fwd.hpp:132-185
+//   cko_conv3d_fwd_{f32,f16,i8}      ReferenceConvFwd, NumDimSpatial == 3 (:186-248); with unit extents
+//       also the 1-D branch (:92-131)
 //   cko_batched_gemm_f16             ReferenceBatchedGemm::Invoker::Run
 //       library/include/ck/library/reference_tensor_operation/cpu/reference_batched_gemm.hpp:56-88
 //   cko_batched_gemm_gemm_f16        two chained ReferenceBatchedGemm with an
@@ -483,6 +485,93 @@ void cko_conv2d_fwd_i8(const int8_t* in, const int8_t* wei, int8_t* out, int N, 
     conv2d_fwd(
         N, K, C, Hi, Wi, Y, X, Ho, Wo, sH, sW, dH, dW, pH, pW, nthreads,
         [=](std::size_t o) { return (float)in[o]; }, [=](std::size_t o) { return (float)wei[o]; },
+        [=](std::size_t o, float acc) { out[o] = float_to_i8_trunc_wrap(ep(acc)); });
+}
+
+} // extern "C"
+
+namespace {
+
+// Forward convolution with three spatial dimensions, NDHWC / KZYXC / NDHWK memory, fp32 accumulation
+// in the loop order c -> z -> y -> x (reference_conv_fwd.hpp:186-248). With D = Z = 1 the loop is the
+// 2-D one (:132-185), with D = H = Z = Y = 1 the 1-D one (:92-131): same taps, same order.
+template <typename LoadIn, typename LoadWei, typename StoreOut>
+void conv3d_fwd(int N, int K, int C, const int* in_len, const int* filt, const int* out_len, const int* stride,
+                const int* dil, const int* pad, int nthreads, LoadIn in_at, LoadWei wei_at, StoreOut store)
+{
+    const int Di = in_len[0], Hi = in_len[1], Wi = in_len[2], Z = filt[0], Y = filt[1], X = filt[2];
+    const int Do = out_len[0], Ho = out_len[1], Wo = out_len[2];
+    parallel_for((std::size_t)N * K * Do * Ho * Wo, nthreads, [&](std::size_t i0, std::size_t i1) {
+        for(std::size_t i = i0; i < i1; ++i)
+        {
+            std::size_t r = i;
+            const int wo  = (int)(r % (std::size_t)Wo);
+            r /= (std::size_t)Wo;
+            const int ho = (int)(r % (std::size_t)Ho);
+            r /= (std::size_t)Ho;
+            const int od = (int)(r % (std::size_t)Do);
+            r /= (std::size_t)Do;
+            const int k = (int)(r % (std::size_t)K);
+            const int n = (int)(r / (std::size_t)K);
+            float acc   = 0;
+            for(int c = 0; c < C; ++c)
+                for(int z = 0; z < Z; ++z)
+                {
+                    const long di = (long)od * stride[0] + (long)z * dil[0] - pad[0];
+                    for(int y = 0; y < Y; ++y)
+                    {
+                        const long hi = (long)ho * stride[1] + (long)y * dil[1] - pad[1];
+                        for(int x = 0; x < X; ++x)
+                        {
+                            const long wi = (long)wo * stride[2] + (long)x * dil[2] - pad[2];
+                            if(di >= 0 && di < Di && hi >= 0 && hi < Hi && wi >= 0 && wi < Wi)
+                            {
+                                const float v_in =
+                                    in_at(((((std::size_t)n * Di + di) * Hi + hi) * Wi + wi) * C + c);
+                                const float v_wei =
+                                    wei_at(((((std::size_t)k * Z + z) * Y + y) * X + x) * C + c);
+                                acc += v_in * v_wei;
+                            }
+                        }
+                    }
+                }
+            store(((((std::size_t)n * Do + od) * Ho + ho) * Wo + wo) * K + k, acc);
+        }
+    });
+}
+
+} // namespace
+
+extern "C" {
+
+// in_len / filt / out_len / stride / dil / pad: three entries each, (D, H, W) order
+void cko_conv3d_fwd_f32(const float* in, const float* wei, float* out, int N, int K, int C, const int* in_len,
+                        const int* filt, const int* out_len, const int* stride, const int* dil, const int* pad,
+                        int nthreads)
+{
+    conv3d_fwd(
+        N, K, C, in_len, filt, out_len, stride, dil, pad, nthreads, [=](std::size_t o) { return in[o]; },
+        [=](std::size_t o) { return wei[o]; }, [=](std::size_t o, float acc) { out[o] = acc; });
+}
+
+void cko_conv3d_fwd_f16(const uint16_t* in, const uint16_t* wei, uint16_t* out, int N, int K, int C,
+                        const int* in_len, const int* filt, const int* out_len, const int* stride, const int* dil,
+                        const int* pad, int nthreads)
+{
+    conv3d_fwd(
+        N, K, C, in_len, filt, out_len, stride, dil, pad, nthreads,
+        [=](std::size_t o) { return half_to_float(in[o]); }, [=](std::size_t o) { return half_to_float(wei[o]); },
+        [=](std::size_t o, float acc) { out[o] = float_to_half(acc); });
+}
+
+void cko_conv3d_fwd_i8(const int8_t* in, const int8_t* wei, int8_t* out, int N, int K, int C, const int* in_len,
+                       const int* filt, const int* out_len, const int* stride, const int* dil, const int* pad,
+                       int epi_kind, float scale_gemm, float scale_relu, int nthreads)
+{
+    Epilogue ep{epi_kind, scale_gemm, scale_relu};
+    conv3d_fwd(
+        N, K, C, in_len, filt, out_len, stride, dil, pad, nthreads, [=](std::size_t o) { return (float)in[o]; },
+        [=](std::size_t o) { return (float)wei[o]; },
         [=](std::size_t o, float acc) { out[o] = float_to_i8_trunc_wrap(ep(acc)); });
 }
 

@@ -90,6 +90,43 @@ def im2col(inp_nhwc, Y, X, strides, dilations, pads, right_pads=None):
     return cols.reshape(N * Ho * Wo, Y * X * C), Ho, Wo
 
 
+def im2col_nd(inp, filt, strides, dilations, pads, right_pads=None):
+    """[N, (D,) (H,) W, C] -> [N * prod(out), prod(filt) * C], taps slowest-dimension first, c fastest."""
+    nd = inp.ndim - 2
+    if right_pads is None:
+        right_pads = pads
+    lead = 3 - nd
+    x = inp.reshape(inp.shape[0], *([1] * lead), *inp.shape[1:])
+    f = [1] * lead + list(filt)
+    s = [1] * lead + list(strides)
+    d = [1] * lead + list(dilations)
+    pl = [0] * lead + list(pads)
+    pr = [0] * lead + list(right_pads)
+    N, Cc = x.shape[0], x.shape[-1]
+    o = [(x.shape[1 + i] + pl[i] + pr[i] - ((f[i] - 1) * d[i] + 1)) // s[i] + 1 for i in range(3)]
+    p = np.zeros((N, *[x.shape[1 + i] + pl[i] + pr[i] for i in range(3)], Cc), inp.dtype)
+    p[:, pl[0]:pl[0] + x.shape[1], pl[1]:pl[1] + x.shape[2], pl[2]:pl[2] + x.shape[3], :] = x
+    cols = np.empty((N, *o, *f, Cc), inp.dtype)
+    for z in range(f[0]):
+        for y in range(f[1]):
+            for xx in range(f[2]):
+                cols[:, :, :, :, z, y, xx, :] = p[:, z * d[0]:z * d[0] + (o[0] - 1) * s[0] + 1:s[0],
+                                                  y * d[1]:y * d[1] + (o[1] - 1) * s[1] + 1:s[1],
+                                                  xx * d[2]:xx * d[2] + (o[2] - 1) * s[2] + 1:s[2], :]
+    return cols.reshape(N * o[0] * o[1] * o[2], f[0] * f[1] * f[2] * Cc), o[lead:]
+
+
+def convnd_fwd(inp, wei, strides, dilations, pads, right_pads=None, epi=EPI_PASSTHROUGH, scale_gemm=1.0,
+               scale_relu=1.0):
+    """N-d forward conv through im2col + BLAS: int8 exact (with the requant epilogues), fp16 in BLAS order."""
+    K = wei.shape[0]
+    cols, o = im2col_nd(inp, wei.shape[1:-1], strides, dilations, pads, right_pads)
+    w = wei.reshape(K, -1).T
+    if inp.dtype == np.int8:
+        return epilogue_i8(gemm_i8_acc(cols, w), epi, scale_gemm, scale_relu).reshape(inp.shape[0], *o, K)
+    return (cols.astype(np.float32) @ w.astype(np.float32)).astype(np.float16).reshape(inp.shape[0], *o, K)
+
+
 def conv2d_fwd_i8(inp_nhwc, wei_kyxc, strides=(1, 1), dilations=(1, 1), pads=(0, 0), right_pads=None,
                   epi=EPI_PASSTHROUGH, scale_gemm=1.0, scale_relu=1.0):
     N = inp_nhwc.shape[0]

@@ -179,6 +179,40 @@ def conv2d_fwd(inp_nhwc, wei_kyxc, strides=(1, 1), dilations=(1, 1), pads=(0, 0)
     return out
 
 
+def convnd_fwd(inp, wei, strides, dilations, pads, right_pads=None, epi=EPI_PASSTHROUGH, scale_gemm=1.0,
+               scale_relu=1.0, nthreads=0):
+    """Forward convolution with 1, 2 or 3 spatial dimensions: N(D)(H)WC input, K(Z)(Y)XC weights ->
+    N(D)(H)WK output; dtype float32 / float16 / int8. Missing leading dimensions have extent 1."""
+    inp = np.ascontiguousarray(inp)
+    wei = np.ascontiguousarray(wei)
+    nd = inp.ndim - 2
+    assert nd in (1, 2, 3) and wei.ndim == inp.ndim and len(strides) == len(dilations) == len(pads) == nd
+    if right_pads is None:
+        right_pads = pads
+    lead = 3 - nd
+    in_len = [1] * lead + list(inp.shape[1:-1])
+    filt = [1] * lead + list(wei.shape[1:-1])
+    st = [1] * lead + list(strides)
+    dl = [1] * lead + list(dilations)
+    pl = [0] * lead + list(pads)
+    pr = [0] * lead + list(right_pads)
+    out_len = [conv_out_len(in_len[i], filt[i], st[i], dl[i], pl[i], pr[i]) for i in range(3)]
+    N, Cc, K = inp.shape[0], inp.shape[-1], wei.shape[0]
+    assert wei.shape[-1] == Cc
+    out = np.empty((N, *out_len[lead:], K), inp.dtype)
+    arr = lambda v: (C.c_int * 3)(*[int(x) for x in v])
+    args = [_p(inp), _p(wei), _p(out), N, K, Cc, arr(in_len), arr(filt), arr(out_len), arr(st), arr(dl), arr(pl)]
+    if inp.dtype == np.float32:
+        lib().cko_conv3d_fwd_f32(*args, int(nthreads))
+    elif inp.dtype == np.float16:
+        lib().cko_conv3d_fwd_f16(*args, int(nthreads))
+    elif inp.dtype == np.int8:
+        lib().cko_conv3d_fwd_i8(*args, int(epi), C.c_float(scale_gemm), C.c_float(scale_relu), int(nthreads))
+    else:
+        raise TypeError(inp.dtype)
+    return out
+
+
 def conv2d_fwd_bias_relu_f16(inp_nhwc, wei_kyxc, bias_k, resi_nhwk=None, strides=(1, 1), dilations=(1, 1),
                              pads=(0, 0), right_pads=None, nthreads=0):
     """conv + bias + ReLU (+ residual), fp16 tensors, fp32 through the functor, one rounding."""

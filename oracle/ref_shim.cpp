@@ -115,6 +115,57 @@ void run_conv(const T* in, const T* wei, T* out, int N, int K, int C, int Hi, in
     std::memcpy(out, to.mData.data(), to.mData.size() * sizeof(T));
 }
 
+// NumDimSpatial = ND: tensors addressed logically N,C,(D,)(H,)W with the channels-last strides of
+// conv_util.hpp:195-236 (NWC / NHWC / NDHWC and the matching weight / output layouts)
+template <typename T, int ND>
+void run_convnd(const T* in, const T* wei, T* out, int N, int K, int C, const int* in_len, const int* filt,
+                const int* out_len, const int* stride, const int* dil, const int* pad)
+{
+    using sz = std::size_t;
+    auto desc = [](sz n, sz c, const int* len) {
+        std::vector<sz> lens{n, c}, strides(2 + ND);
+        sz px = 1;
+        for(int i = 0; i < ND; ++i)
+        {
+            lens.push_back((sz)len[i]);
+            px *= (sz)len[i];
+        }
+        strides[0] = c * px;
+        strides[1] = 1;
+        sz run     = c;
+        for(int i = ND - 1; i >= 0; --i)
+        {
+            strides[2 + i] = run;
+            run *= (sz)len[i];
+        }
+        return std::make_pair(lens, strides);
+    };
+    auto di = desc((sz)N, (sz)C, in_len), dw = desc((sz)K, (sz)C, filt), dq = desc((sz)N, (sz)K, out_len);
+    auto ti = make_tensor<T>(di.first, di.second, in);
+    auto tw = make_tensor<T>(dw.first, dw.second, wei);
+    auto to = make_tensor<T>(dq.first, dq.second, (const T*)nullptr);
+    using Ref =
+        ck::tensor_operation::host::ReferenceConvFwd<T, T, T, PassThrough, PassThrough, PassThrough, ND>;
+    Ref ref;
+    auto inv = ref.MakeInvoker();
+    std::vector<ck::index_t> st(stride, stride + ND), dl(dil, dil + ND), pd(pad, pad + ND);
+    auto arg = ref.MakeArgument(ti, tw, to, st, dl, pd, pd, PassThrough{}, PassThrough{}, PassThrough{});
+    inv.Run(arg);
+    std::memcpy(out, to.mData.data(), to.mData.size() * sizeof(T));
+}
+
+template <typename T>
+void run_convnd_dispatch(int ndim, const T* in, const T* wei, T* out, int N, int K, int C, const int* in_len,
+                         const int* filt, const int* out_len, const int* stride, const int* dil, const int* pad)
+{
+    if(ndim == 1)
+        run_convnd<T, 1>(in, wei, out, N, K, C, in_len, filt, out_len, stride, dil, pad);
+    else if(ndim == 2)
+        run_convnd<T, 2>(in, wei, out, N, K, C, in_len, filt, out_len, stride, dil, pad);
+    else
+        run_convnd<T, 3>(in, wei, out, N, K, C, in_len, filt, out_len, stride, dil, pad);
+}
+
 } // namespace
 
 extern "C" {
@@ -173,6 +224,30 @@ void ckref_conv2d_fwd_i8(const int8_t* in, const int8_t* wei, int8_t* out, int N
                          int pW)
 {
     run_conv<int8_t>(in, wei, out, N, K, C, Hi, Wi, Y, X, Ho, Wo, sH, sW, dH, dW, pH, pW);
+}
+
+// ndim spatial dimensions, the first ndim entries of every array are used (slowest dimension first); symmetric pads
+void ckref_convnd_fwd_f32(int ndim, const float* in, const float* wei, float* out, int N, int K, int C,
+                          const int* in_len, const int* filt, const int* out_len, const int* stride, const int* dil,
+                          const int* pad)
+{
+    run_convnd_dispatch<float>(ndim, in, wei, out, N, K, C, in_len, filt, out_len, stride, dil, pad);
+}
+
+void ckref_convnd_fwd_f16(int ndim, const uint16_t* in, const uint16_t* wei, uint16_t* out, int N, int K, int C,
+                          const int* in_len, const int* filt, const int* out_len, const int* stride, const int* dil,
+                          const int* pad)
+{
+    using H = ck::half_t;
+    run_convnd_dispatch<H>(ndim, (const H*)in, (const H*)wei, (H*)out, N, K, C, in_len, filt, out_len, stride, dil,
+                           pad);
+}
+
+void ckref_convnd_fwd_i8(int ndim, const int8_t* in, const int8_t* wei, int8_t* out, int N, int K, int C,
+                         const int* in_len, const int* filt, const int* out_len, const int* stride, const int* dil,
+                         const int* pad)
+{
+    run_convnd_dispatch<int8_t>(ndim, in, wei, out, N, K, C, in_len, filt, out_len, stride, dil, pad);
 }
 
 void ckref_batched_gemm_f16(const uint16_t* a, const uint16_t* b, uint16_t* c, int G, int M, int N,

@@ -94,6 +94,23 @@ class _Ref:
            dilations[0], dilations[1], pads[0], pads[1])
         return out
 
+    def convnd_fwd(self, inp, wei, strides, dilations, pads):
+        """1, 2 or 3 spatial dimensions, channels-last tensors, symmetric pads."""
+        inp = np.ascontiguousarray(inp)
+        wei = np.ascontiguousarray(wei)
+        nd = inp.ndim - 2
+        in_len, filt = list(inp.shape[1:-1]), list(wei.shape[1:-1])
+        out_len = [self.conv_out_len(in_len[i], filt[i], strides[i], dilations[i], pads[i], pads[i]) for i in range(nd)]
+        N, Cc, K = inp.shape[0], inp.shape[-1], wei.shape[0]
+        out = np.zeros((N, *out_len, K), inp.dtype)
+        fn = {np.dtype(np.float32): self.lib.ckref_convnd_fwd_f32,
+              np.dtype(np.float16): self.lib.ckref_convnd_fwd_f16,
+              np.dtype(np.int8): self.lib.ckref_convnd_fwd_i8}[inp.dtype]
+        arr = lambda v: (C.c_int * 3)(*([int(x) for x in v] + [0] * (3 - nd)))
+        fn(nd, _p(inp), _p(wei), _p(out), N, K, Cc, arr(in_len), arr(filt), arr(out_len), arr(strides),
+           arr(dilations), arr(pads))
+        return out
+
     def conv2d_fwd_bias_relu_f16(self, inp_nhwc, wei_kyxc, bias_k, resi_nhwk=None, strides=(1, 1),
                                  dilations=(1, 1), pads=(0, 0)):
         inp = np.ascontiguousarray(inp_nhwc, np.float16)

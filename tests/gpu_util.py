@@ -82,6 +82,34 @@ def conv2d_fwd(inp_nhwc, wei_kyxc, strides, dilations, pads, out_op=None, instan
     return do.cpu().numpy()
 
 
+def convnd_fwd(inp, wei, strides, dilations, pads, out_op=None, instance=capi.INSTANCE_AUTO, right_pads=None,
+               workspace=False):
+    """Channels-last tensors with 1, 2 or 3 spatial dimensions through DeviceConvNdFwd*."""
+    nd = inp.ndim - 2
+    N, C, K = inp.shape[0], inp.shape[-1], wei.shape[0]
+    in_len, filt = list(inp.shape[1:-1]), list(wei.shape[1:-1])
+    right_pads = right_pads or pads
+    out_len = [(in_len[i] + pads[i] + right_pads[i] - ((filt[i] - 1) * dilations[i] + 1)) // strides[i] + 1
+               for i in range(nd)]
+    di, dw = dev(inp), dev(wei)
+    if inp.dtype == np.int8:
+        do = torch.full((N, *out_len, K), 77, dtype=torch.int8, device="cuda")
+        op = ck.DeviceConvNdFwdInt8(nd, instance)
+    else:
+        do = torch.full((N, *out_len, K), float("nan"), dtype=torch.float16, device="cuda")
+        op = ck.DeviceConvNdFwdF16(nd, instance)
+    arg = op.MakeArgumentPointer(di, dw, do, N, K, C, in_len, filt, out_len, list(strides), list(dilations),
+                                 list(pads), list(right_pads), None, None, out_op)
+    assert op.IsSupportedArgument(arg), capi.last_error()
+    if workspace:
+        need = op.GetWorkSpaceSize(arg)
+        ws = torch.full((max(need, 16),), 0x7F, dtype=torch.uint8, device="cuda")
+        op.SetWorkSpacePointer(arg, ws)
+    op.MakeInvokerPointer().Run(arg, ck.StreamConfig(stream()))
+    torch.cuda.synchronize()
+    return do.cpu().numpy()
+
+
 def gemm_gemm_f16(a_gmk, b0_gnk, b1_gno):
     G, M, K = a_gmk.shape
     N = b0_gnk.shape[1]

@@ -311,6 +311,77 @@ def test_conv2d_lit_fast_ref_agree(dtype):
                                           out.view(np.uint8))
 
 
+GOLD_ND = json.load(open(os.path.join(HERE, "golden", "reference_convnd_fwd_vectors.json")))
+
+
+def _monotonic_fill(n, start, step):
+    """FillMonotonicSeq (library/include/ck/library/utility/fill.hpp:66-80): x[i+1] = x[i] + step in fp32."""
+    out = np.empty(n, np.float32)
+    v = np.float32(start)
+    for i in range(n):
+        out[i] = v
+        v = np.float32(v + np.float32(step))
+    return out
+
+
+@pytest.mark.parametrize("case", GOLD_ND["cases"], ids=lambda c: c["name"])
+def test_convnd_reference_golden_vectors(case):
+    """The 1-D (NWC) and 3-D (NCDHW) outputs the reference's own ReferenceConvFwd test holds
+    (test/reference_conv_fwd/reference_conv_fwd.cpp:156-392), with that test's check_err tolerances."""
+    N, K, C = case["N"], case["K"], case["C"]
+    sp, filt = case["input"], case["filter"]
+    x = _monotonic_fill(N * C * int(np.prod(sp)), *case["fill_start_step"])
+    if case["layout"] == "channels_first":
+        inp = np.moveaxis(x.reshape(N, C, *sp), 1, -1)
+    else:
+        inp = x.reshape(N, *sp, C)
+    wei = np.full((K, *filt, C), 0.5, np.float32)
+    out = lit.convnd_fwd(inp, wei, case["strides"], case["dilations"], case["left_pads"], case["right_pads"])
+    assert list(out.shape) == [N, *case["out_dims_nk_spatial"][2:], K]
+    got = (np.moveaxis(out, -1, 1) if case["layout"] == "channels_first" else out).ravel()
+    exp = np.array(case["expected"], np.float32)
+    assert got.shape == exp.shape
+    assert (np.abs(got.astype(np.float64) - exp) <= case["atol"] + case["rtol"] * np.abs(exp)).all()
+    # BLAS / im2col form (another summation order, result rounded to fp16)
+    np.testing.assert_allclose(
+        fast.convnd_fwd(inp, wei, case["strides"], case["dilations"], case["left_pads"],
+                        case["right_pads"]).astype(np.float32), out, rtol=2e-3, atol=1e-3)
+    if REF is not None:
+        np.testing.assert_array_equal(
+            REF.convnd_fwd(inp, wei, case["strides"], case["dilations"], case["left_pads"]), out)
+
+
+@pytest.mark.parametrize("dtype", [np.float16, np.int8])
+def test_convnd_lit_fast_ref_agree(dtype):
+    """One and three spatial dimensions: literal restatement, im2col + BLAS form and the compiled reference."""
+    rng = np.random.default_rng(11)
+    for (shape_in, shape_w, s, d, p) in [((2, 9, 8), (5, 3, 8), (2,), (2,), (1,)),
+                                         ((3, 11, 16), (4, 1, 16), (1,), (1,), (0,)),
+                                         ((2, 5, 7, 6, 8), (5, 2, 3, 2, 8), (1, 2, 1), (2, 1, 2), (1, 1, 0)),
+                                         ((1, 4, 4, 4, 16), (3, 3, 3, 3, 16), (1, 1, 1), (1, 1, 1), (1, 1, 1)),
+                                         ((2, 3, 5, 4, 8), (6, 1, 1, 1, 8), (2, 2, 2), (1, 1, 1), (0, 0, 0))]:
+        if dtype == np.int8:
+            inp, wei = _rand_i8(rng, shape_in), _rand_i8(rng, shape_w)
+        else:
+            inp = rng.uniform(-1, 1, shape_in).astype(np.float16)
+            wei = rng.uniform(-1, 1, shape_w).astype(np.float16)
+        out = lit.convnd_fwd(inp, wei, s, d, p)
+        if dtype == np.int8:
+            np.testing.assert_array_equal(fast.convnd_fwd(inp, wei, s, d, p), out)
+            o2 = lit.convnd_fwd(inp, wei, s, d, p, epi=lit.EPI_REQUANT_RND, scale_gemm=0.5, scale_relu=0.3)
+            np.testing.assert_array_equal(
+                fast.convnd_fwd(inp, wei, s, d, p, epi=lit.EPI_REQUANT_RND, scale_gemm=0.5, scale_relu=0.3), o2)
+        else:
+            bad, _ = lit.check_err_f16(fast.convnd_fwd(inp, wei, s, d, p), out, 1e-3, 1e-3)
+            assert bad == 0
+        if REF is not None:
+            np.testing.assert_array_equal(REF.convnd_fwd(inp, wei, s, d, p).view(np.uint8), out.view(np.uint8))
+    # two dimensions through the N-d entry are the 2-D routine
+    inp, wei = _rand_i8(rng, (2, 6, 7, 8)), _rand_i8(rng, (4, 3, 2, 8))
+    np.testing.assert_array_equal(lit.convnd_fwd(inp, wei, (1, 2), (2, 1), (1, 1)),
+                                  lit.conv2d_fwd(inp, wei, (1, 2), (2, 1), (1, 1)))
+
+
 def test_conv2d_int8_passthrough_wraps_modulo_256():
     # the reference's int8 conv keeps the low byte of an out-of-range sum
     inp = np.full((1, 4, 4, 16), 5, np.int8)
