@@ -47,6 +47,16 @@ def _conv_workload(name, dtype, C, K, f, HW, st, pd, N=256, fused=None):
                 fused=fused)
 
 
+def _conv3d_workload(name, dtype, C, K, f, DHW, st, pd, N, dil=1):
+    """Three spatial dimensions, NDHWC / KZYXC / NDHWK, cubic extents."""
+    Do = (DHW + 2 * pd - ((f - 1) * dil + 1)) // st + 1
+    es = 1 if dtype == "i8" else 2
+    ops = 2.0 * N * K * Do ** 3 * C * f ** 3
+    byts = (N * DHW ** 3 * C + K * f ** 3 * C + N * Do ** 3 * K) * es
+    return dict(name=name, kind="conv", ndim=3, dtype=dtype, N=N, C=C, K=K, f=f, HW=DHW, st=st, pd=pd, dil=dil, ops=ops,
+                bytes=byts, fused=None)
+
+
 def _gemm_workload(name, dtype, M, N, K, values=5, scales=(0.5, 0.03), fused=None, batch=1, layout="mk_nk"):
     """fused: None or "bias_relu" (fp16: E = AddRelu(half(A*B), bias row)); batch > 1: strided batched GEMM;
     layout: how A ("mk" row-major / "km" column-major) and B ("nk" column-major / "kn" row-major) are stored."""
@@ -74,6 +84,10 @@ for w in (
     + [_gemm_workload("fp16_gemm_bias_relu_4096", "f16", 4096, 4096, 4096, fused="bias_relu"),
        _conv_workload("conv_f16_c64_k64_3x3_56_bias_relu_add", "f16", 64, 64, 3, 56, 1, 1, fused="bias_relu_add"),
        _conv_workload("conv_f16_c256_k512_1x1_56_s2_bias_relu", "f16", 256, 512, 1, 56, 2, 0, fused="bias_relu")]
+    # three spatial dimensions: the reference's device-test default (conv3d_fwd.cpp:76-77) and a larger 3x3x3 layer
+    + [_conv3d_workload("conv3d_f16_n4_c64_k256_3x3x3_28_s2_d2", "f16", 64, 256, 3, 28, 2, 2, 4, dil=2),
+       _conv3d_workload("conv3d_f16_n16_c64_k64_3x3x3_32", "f16", 64, 64, 3, 32, 1, 1, 16),
+       _conv3d_workload("conv3d_i8_n16_c64_k64_3x3x3_32", "i8", 64, 64, 3, 32, 1, 1, 16)]
     + [dict(name="gemm_gemm_f16_b64_512x64x512x64", kind="gemm_gemm", dtype="f16", G=64, M=512, N=512, K=64, O=64,
             ops=2.0 * 64 * 512 * 512 * 64 * 2, bytes=4 * 64 * 512 * 64 * 2),
        # the same shapes with a softmax between the GEMMs (attention): 64 heads of 512 x 512 scores, and a long one
@@ -144,18 +158,19 @@ def make_launcher(w, instance=-1, rotate=1):
             more_args.append(make(b2))
     elif w["kind"] == "conv":
         N, C, K, f, HW, st, pd = (w[k] for k in ("N", "C", "K", "f", "HW", "st", "pd"))
-        Ho = (HW + 2 * pd - f) // st + 1
+        nd, dil = w.get("ndim", 2), w.get("dil", 1)
+        Ho = (HW + 2 * pd - ((f - 1) * dil + 1)) // st + 1
         if w["dtype"] == "i8":
-            i, wt = dev(uniform_int8((N, HW, HW, C), -5, 5, 3)), dev(uniform_int8((K, f, f, C), -5, 5, 4))
-            c = torch.empty((N, Ho, Ho, K), dtype=torch.int8, device="cuda")
-            op = ck.DeviceConv2dFwdInt8(instance)
+            i, wt = dev(uniform_int8((N, *[HW] * nd, C), -5, 5, 3)), dev(uniform_int8((K, *[f] * nd, C), -5, 5, 4))
+            c = torch.empty((N, *[Ho] * nd, K), dtype=torch.int8, device="cuda")
+            op = ck.DeviceConv2dFwdInt8(instance) if nd == 2 else ck.DeviceConvNdFwdInt8(nd, instance)
             cop = ck.RequantReluRequant(0.01, 0.5, rounded=True)
         else:
-            i, wt = dev(uniform_f16((N, HW, HW, C), -1, 1, 3)), dev(uniform_f16((K, f, f, C), -1, 1, 4))
-            c = torch.empty((N, Ho, Ho, K), dtype=torch.float16, device="cuda")
-            op = ck.DeviceConv2dFwdF16(instance)
+            i, wt = dev(uniform_f16((N, *[HW] * nd, C), -1, 1, 3)), dev(uniform_f16((K, *[f] * nd, C), -1, 1, 4))
+            c = torch.empty((N, *[Ho] * nd, K), dtype=torch.float16, device="cuda")
+            op = ck.DeviceConv2dFwdF16(instance) if nd == 2 else ck.DeviceConvNdFwdF16(nd, instance)
             cop = ck.PassThrough()
-        geom = (N, K, C, [HW, HW], [f, f], [Ho, Ho], [st, st], [1, 1], [pd, pd], [pd, pd], None, None)
+        geom = (N, K, C, [HW] * nd, [f] * nd, [Ho] * nd, [st] * nd, [dil] * nd, [pd] * nd, [pd] * nd, None, None)
         if w.get("fused"):
             op = ck.DeviceConv2dFwdBiasActivationF16(instance)
             bias = dev(uniform_f16((K,), -1, 1, 7))

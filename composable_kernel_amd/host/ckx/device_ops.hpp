@@ -629,6 +629,106 @@ struct DeviceConv2dFwdMfma_Input_N_Hi_Wi_C_Weight_K_Y_X_C_Output_N_Ho_Wo_K
     int instance_;
 };
 
+// ------------------------------------------------------------------ conv fwd, 1 / 2 / 3 spatial dimensions
+// DeviceConvNDFwdXdl_Input_N_Hi_Wi_C_Weight_K_Y_X_C_Output_N_Ho_Wo_K<..., NumDimSpatial>
+// (include/ck/tensor_operation/gpu/device/device_convnd_fwd_xdl_nhwc_kyxc_nhwk.hpp:76-1046): NWC / NHWC / NDHWC
+// input, KXC / KYXC / KZYXC weight, NWK / NHWK / NDHWK output; every vector has NumDimSpatial entries.
+template <typename InDataType, typename WeiDataType, typename OutDataType, typename InElementwiseOperation,
+          typename WeiElementwiseOperation, typename OutElementwiseOperation, int NumDimSpatial>
+struct DeviceConvNDFwdMfma_Input_N_Hi_Wi_C_Weight_K_Y_X_C_Output_N_Ho_Wo_K
+    : public DeviceConvFwd<InElementwiseOperation, WeiElementwiseOperation, OutElementwiseOperation>
+{
+    static_assert(std::is_same_v<InDataType, WeiDataType> && std::is_same_v<InDataType, OutDataType>,
+                  "input, weight and output share one data type (int8_t or half_t)");
+    static_assert(NumDimSpatial >= 1 && NumDimSpatial <= 3, "1, 2 or 3 spatial dimensions");
+    static constexpr bool is_i8 = detail::DTypeOf<InDataType>::is_i8;
+    using Epi                   = ckx::EpilogueOf<OutElementwiseOperation>;
+    static constexpr int op_code = is_i8 ? CKX_OP_CONV2D_FWD_I8 : CKX_OP_CONV2D_FWD_F16;
+
+    struct Argument : public BaseArgument
+    {
+        const void* p_in;
+        const void* p_wei;
+        void* p_out;
+        ckx_convnd_desc desc;
+        bool dims_ok;
+        OutElementwiseOperation out_element_op;
+        Argument(const void* in, const void* wei, void* out, index_t N, index_t K, index_t C,
+                 const std::vector<index_t>& isp, const std::vector<index_t>& fsp, const std::vector<index_t>& osp,
+                 const std::vector<index_t>& st, const std::vector<index_t>& dl, const std::vector<index_t>& lp,
+                 const std::vector<index_t>& rp, OutElementwiseOperation oop)
+            : p_in(in), p_wei(wei), p_out(out), desc{}, out_element_op(oop)
+        {
+            constexpr std::size_t nd = NumDimSpatial;
+            dims_ok = isp.size() == nd && fsp.size() == nd && osp.size() == nd && st.size() == nd && dl.size() == nd &&
+                      lp.size() == nd && rp.size() == nd;
+            desc.ndim = NumDimSpatial, desc.N = N, desc.K = K, desc.C = C;
+            for(std::size_t i = 0; dims_ok && i < nd; ++i)
+            {
+                desc.in[i] = isp[i], desc.filter[i] = fsp[i], desc.out[i] = osp[i], desc.stride[i] = st[i];
+                desc.dilation[i] = dl[i], desc.pad_left[i] = lp[i], desc.pad_right[i] = rp[i];
+            }
+        }
+    };
+    static int Supported(const Argument& a, int inst)
+    {
+        if(!a.dims_ok)
+            return CKX_UNSUPPORTED;
+        return ckx_convnd_fwd_is_supported(op_code, &a.desc, Epi::kind, inst);
+    }
+    static int Launch(const Argument& a, int inst, void* stream)
+    {
+        const int64_t ws_bytes = a.p_workspace_ ? ckx_convnd_fwd_workspace_bytes(op_code, &a.desc, inst) : 0;
+        return ckx_convnd_fwd(op_code, a.p_in, a.p_wei, a.p_out, &a.desc, Epi::kind, Epi::scale_gemm(a.out_element_op),
+                              Epi::scale_relu(a.out_element_op), inst, a.p_workspace_, ws_bytes, stream);
+    }
+    size_t GetWorkSpaceSize(const BaseArgument* p) const override
+    {
+        const auto* a = dynamic_cast<const Argument*>(p);
+        return a && a->dims_ok ? (size_t)ckx_convnd_fwd_workspace_bytes(op_code, &a->desc, instance_) : 0;
+    }
+    using Invoker = detail::InvokerT<Argument, &Supported, &Launch>;
+
+    explicit DeviceConvNDFwdMfma_Input_N_Hi_Wi_C_Weight_K_Y_X_C_Output_N_Ho_Wo_K(int instance = CKX_INSTANCE_AUTO)
+        : instance_(instance)
+    {
+    }
+    static Argument MakeArgument(const InDataType* p_in, const WeiDataType* p_wei, OutDataType* p_out, index_t N,
+                                 index_t K, index_t C, std::vector<index_t> isp, std::vector<index_t> fsp,
+                                 std::vector<index_t> osp, std::vector<index_t> st, std::vector<index_t> dl,
+                                 std::vector<index_t> lp, std::vector<index_t> rp, InElementwiseOperation,
+                                 WeiElementwiseOperation, OutElementwiseOperation oop)
+    {
+        return Argument{p_in, p_wei, p_out, N, K, C, isp, fsp, osp, st, dl, lp, rp, oop};
+    }
+    Invoker MakeInvoker() const { return Invoker{instance_}; }
+    bool IsSupportedArgument(const Argument& a) const { return Supported(a, instance_) == CKX_OK; }
+    bool IsSupportedArgument(const BaseArgument* p) override
+    {
+        const auto* a = dynamic_cast<const Argument*>(p);
+        return a && IsSupportedArgument(*a);
+    }
+    std::unique_ptr<BaseArgument>
+    MakeArgumentPointer(const void* p_in, const void* p_wei, void* p_out, index_t N, index_t K, index_t C,
+                        std::vector<index_t> isp, std::vector<index_t> fsp, std::vector<index_t> osp,
+                        std::vector<index_t> st, std::vector<index_t> dl, std::vector<index_t> lp,
+                        std::vector<index_t> rp, InElementwiseOperation, WeiElementwiseOperation,
+                        OutElementwiseOperation oop) override
+    {
+        return std::make_unique<Argument>(p_in, p_wei, p_out, N, K, C, isp, fsp, osp, st, dl, lp, rp, oop);
+    }
+    std::unique_ptr<BaseInvoker> MakeInvokerPointer() override { return std::make_unique<Invoker>(instance_); }
+    std::string GetTypeString() const override
+    {
+        const std::string nd = "DeviceConv" + std::to_string(NumDimSpatial) + "dFwd";
+        if(instance_ == CKX_INSTANCE_AUTO)
+            return nd + (is_i8 ? "_i8_channels_last<auto>" : "_f16_channels_last<auto>");
+        const char* n = ckx_instance_name(op_code, instance_);
+        return nd + ":" + (n ? n : "?");
+    }
+    int instance_;
+};
+
 // ------------------------------------------------------------------ strided batched GEMM
 // One launch for all batches: the persistent workgroups walk the C tiles of every batch.
 template <typename ALayout, typename BLayout, typename CLayout, typename ADataType, typename BDataType,
@@ -1210,6 +1310,18 @@ std::vector<std::unique_ptr<DeviceConvFwd<InOp, WeiOp, OutOp>>> GetConv2dFwdInst
         v.push_back(std::make_unique<
                     DeviceConv2dFwdMfma_Input_N_Hi_Wi_C_Weight_K_Y_X_C_Output_N_Ho_Wo_K<T, T, T, InOp, WeiOp, OutOp>>(
             i));
+    return v;
+}
+
+// ConvolutionFwdInstances<T,T,T>::Get<NumDimSpatial>() (conv_util.hpp:288-397)
+template <int NumDimSpatial, typename T, typename InOp, typename WeiOp, typename OutOp>
+std::vector<std::unique_ptr<DeviceConvFwd<InOp, WeiOp, OutOp>>> GetConvNdFwdInstances()
+{
+    std::vector<std::unique_ptr<DeviceConvFwd<InOp, WeiOp, OutOp>>> v;
+    const int n = ckx_num_instances(detail::DTypeOf<T>::is_i8 ? CKX_OP_CONV2D_FWD_I8 : CKX_OP_CONV2D_FWD_F16);
+    for(int i = 0; i < n; ++i)
+        v.push_back(std::make_unique<DeviceConvNDFwdMfma_Input_N_Hi_Wi_C_Weight_K_Y_X_C_Output_N_Ho_Wo_K<
+                        T, T, T, InOp, WeiOp, OutOp, NumDimSpatial>>(i));
     return v;
 }
 

@@ -6,6 +6,8 @@
 //                     M N K StrideA StrideB StrideC [epilogue 0|1|2] [scale_gemm] [scale_relu] [nrepeat]
 //   ckx_profiler conv2d_fwd <dtype 1|3> <verify> <init> <log> <time>
 //                     N K C Y X Hi Wi Sy Sx Dy Dx LeftPy LeftPx RightPy RightPx [epilogue sg sr] [nrepeat]
+//   ckx_profiler convnd_fwd <dtype 1|3> <layout 1> <verify> <init> <log> <nrepeat> <NDim 1|2|3>
+//                     N K C <filter> <input> <strides> <dilations> <left pads> <right pads>   (NDim values each)
 //   ckx_profiler batched_gemm_gemm <verify> <init> <log> <time> M N K O Batch [nrepeat]
 //   ckx_profiler batched_gemm_softmax_gemm <verify> <init> <log> <time> M N K O Batch [scale] [mask 0|1] [nrepeat]
 //   ckx_profiler conv_fwd_bias_relu | conv_fwd_bias_relu_add <dtype 1> <verify> <init> <log> <time>
@@ -331,6 +333,85 @@ int profile_conv(int argc, char* argv[])
     return 1;
 }
 
+// conv forward with NDim spatial dimensions, channels-last tensors
+// (profiler/src/profile_convnd_fwd.cpp:81-115: N, K, C, then filter / input / strides / dilations / left pads /
+// right pads, NDim values each)
+template <int NDim, typename T, typename OutOp>
+int profile_convnd_t(bool verify, int init, bool time_kernel, const int* p, OutOp oop, int nrepeat)
+{
+    const int N = p[0], K = p[1], C = p[2];
+    std::vector<index_t> filt(p + 3, p + 3 + NDim), in_len(p + 3 + NDim, p + 3 + 2 * NDim),
+        st(p + 3 + 2 * NDim, p + 3 + 3 * NDim), dl(p + 3 + 3 * NDim, p + 3 + 4 * NDim),
+        lp(p + 3 + 4 * NDim, p + 3 + 5 * NDim), rp(p + 3 + 5 * NDim, p + 3 + 6 * NDim), out_len(NDim);
+    std::size_t in_px = N, out_px = N, taps = 1;
+    for(int i = 0; i < NDim; ++i)
+    {
+        // conv_util.cpp:103-114
+        out_len[i] = (in_len[i] + lp[i] + rp[i] - ((filt[i] - 1) * dl[i] + 1)) / st[i] + 1;
+        in_px *= in_len[i], out_px *= out_len[i] > 0 ? out_len[i] : 0, taps *= filt[i];
+    }
+    auto ops = device::instance::GetConvNdFwdInstances<NDim, T, Pass, Pass, OutOp>();
+    using Op = device::DeviceConvFwd<Pass, Pass, OutOp>;
+    std::vector<T> in(in_px * C), wei((std::size_t)K * taps * C);
+    fill(in, init, 0xC0FFEE + 2, true);
+    fill(wei, init, 0xC0FFEE + 3, true);
+    const std::size_t out_elems = out_px * K;
+    ckx::DeviceMem di(in.size() * sizeof(T)), dw(wei.size() * sizeof(T)), dout(out_elems * sizeof(T));
+    di.ToDevice(in.data());
+    dw.ToDevice(wei.data());
+    std::cout << NDim << " spatial dimensions; N " << N << " K " << K << " C " << C << "; output pixels per image "
+              << out_px / (N ? N : 1) << std::endl;
+    const double flop  = 2.0 * (double)out_px * K * C * (double)taps; // conv_util.cpp:22-39
+    const double bytes = sizeof(T) * ((double)in.size() + (double)wei.size() + (double)out_elems);
+    return run_family<T>(
+        ops,
+        [&](Op& op) {
+            return op.MakeArgumentPointer(di.GetDeviceBuffer(), dw.GetDeviceBuffer(), dout.GetDeviceBuffer(), N, K, C,
+                                          in_len, filt, out_len, st, dl, lp, rp, Pass{}, Pass{}, oop);
+        },
+        dout, out_elems, flop, bytes, verify, time_kernel, nrepeat);
+}
+
+template <int NDim>
+int profile_convnd_dim(int dtype, bool verify, int init, bool time_kernel, const int* p, int nrepeat)
+{
+    if(dtype == 1)
+        return profile_convnd_t<NDim, half_t>(verify, init, time_kernel, p, Pass{}, nrepeat);
+    if(dtype == 3)
+        return profile_convnd_t<NDim, int8_t>(verify, init, time_kernel, p, Pass{}, nrepeat);
+    std::cout << "this data_type is not implemented" << std::endl;
+    return 1;
+}
+
+int profile_convnd(int argc, char* argv[])
+{
+    const int ndim = argc > 8 ? std::atoi(argv[8]) : 0;
+    if(ndim < 1 || ndim > 3 || argc != 9 + 3 + 6 * ndim)
+    {
+        std::printf("arg1: tensor operation (convnd_fwd)\narg2: data type (1: fp16; 3: int8)\n"
+                    "arg3: data layout (1: channels last)\narg4: verification\narg5: initialization\n"
+                    "arg6: print tensor value\narg7: run kernel # of times\narg8: N spatial dimensions (1, 2, 3)\n"
+                    "then N, K, C, <filter>, <input>, <strides>, <dilations>, <left pads>, <right pads>\n");
+        return 1;
+    }
+    if(std::atoi(argv[3]) != 1)
+    {
+        std::cout << "this data layout is not implemented" << std::endl;
+        return 1;
+    }
+    const int dtype = std::atoi(argv[2]), init = std::atoi(argv[5]), nrep = std::atoi(argv[7]);
+    const bool verify = std::atoi(argv[4]);
+    int p[3 + 18];
+    for(int i = 0; i < 3 + 6 * ndim; ++i)
+        p[i] = std::atoi(argv[9 + i]);
+    const bool time_kernel = nrep > 0;
+    if(ndim == 1)
+        return profile_convnd_dim<1>(dtype, verify, init, time_kernel, p, nrep > 0 ? nrep : 1);
+    if(ndim == 2)
+        return profile_convnd_dim<2>(dtype, verify, init, time_kernel, p, nrep > 0 ? nrep : 1);
+    return profile_convnd_dim<3>(dtype, verify, init, time_kernel, p, nrep > 0 ? nrep : 1);
+}
+
 template <typename T>
 int profile_gemm_splitk_t(bool verify, int init, bool time_kernel, int M, int N, int K, int sa, int sb, int sc,
                           int kbatch, int nrepeat)
@@ -654,6 +735,8 @@ int main(int argc, char* argv[])
             return profile_gemm_gemm(argc, argv);
         if(argc >= 2 && std::strcmp(argv[1], "batched_gemm_softmax_gemm") == 0)
             return profile_gemm_softmax_gemm(argc, argv);
+        if(argc >= 2 && std::strcmp(argv[1], "convnd_fwd") == 0)
+            return profile_convnd(argc, argv);
         if(argc >= 2 && std::strcmp(argv[1], "conv_fwd_bias_relu") == 0)
             return profile_conv_bias_relu(argc, argv, false);
         if(argc >= 2 && std::strcmp(argv[1], "conv_fwd_bias_relu_add") == 0)
@@ -668,6 +751,7 @@ int main(int argc, char* argv[])
                     "                        conv2d_fwd: NHWC/KYXC/NHWK forward convolution\n"
                     "                        batched_gemm_gemm: batched fused GEMM+GEMM\n"
                     "                        batched_gemm_softmax_gemm: batched fused GEMM+Softmax+GEMM\n"
+                    "                        convnd_fwd: forward convolution, 1 / 2 / 3 spatial dimensions, channels last\n"
                     "                        conv_fwd_bias_relu: ForwardConvolution+Bias+ReLU\n"
                     "                        conv_fwd_bias_relu_add: ForwardConvolution+Bias+ReLU+Add\n"
                     "                        batched_gemm: Batched GEMM\n"

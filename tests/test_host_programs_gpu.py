@@ -64,6 +64,24 @@ def test_profiler_conv2d_fwd_int8(tmp_path):
     np.testing.assert_array_equal(c, want)
 
 
+@pytest.mark.parametrize("ndim", [1, 3])
+def test_profiler_convnd_fwd_int8(tmp_path, ndim):
+    """profile_convnd_fwd's argument order (profiler/src/profile_convnd_fwd.cpp:81-115): data type, layout, verify,
+    init, log, repeats, NDim, then N K C <filter> <input> <strides> <dilations> <left pads> <right pads>."""
+    if ndim == 1:
+        filt, inp_len, st, dl, pd = [3], [40], [2], [2], [2]
+    else:
+        filt, inp_len, st, dl, pd = [3, 3, 3], [7, 9, 8], [2, 1, 2], [1, 2, 1], [1, 2, 1]
+    N, K, C = 3, 64, 32
+    out, dump = _run("ckx_profiler", ["convnd_fwd", 3, 1, 1, 1, 0, 3, ndim, N, K, C] + filt + inp_len + st + dl + pd + pd,
+                     "CKX_PROFILER_DUMP", tmp_path)
+    assert "Best Perf:" in out and "Error" not in out
+    inp = uniform_int8((N, *inp_len, C), -5, 5, SEED + 2)
+    wei = uniform_int8((K, *filt, C), -5, 5, SEED + 3)
+    want = lit.convnd_fwd(inp, wei, st, dl, pd)
+    np.testing.assert_array_equal(np.fromfile(dump, np.int8).reshape(want.shape), want)
+
+
 def test_profiler_batched_gemm_gemm(tmp_path):
     M, N, K, O, G = 256, 384, 64, 64, 3
     out, dump = _run("ckx_profiler", ["batched_gemm_gemm", 1, 1, 0, 1, M, N, K, O, G], "CKX_PROFILER_DUMP", tmp_path)
