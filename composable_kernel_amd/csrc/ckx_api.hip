@@ -480,9 +480,12 @@ bool conv_pointwise_applicable(int op, const ckx_conv2d_desc* d, int epi)
            d->Wo >= 1;
 }
 // ... and the ones it is chosen for: enough pixels for every workgroup to amortise loading its weight slice
+// (measured crossover against the best tile instance, C = 256, K = 512 / 1024: fp16 between 25 K and 50 K pixels
+// per 512-channel block, int8 at about 12 K)
 bool conv_pointwise_preferred(int op, const ckx_conv2d_desc* d, int epi)
 {
-    return conv_pointwise_applicable(op, d, epi) && (long)d->N * d->Ho * d->Wo * (d->K / 512) >= 64 * 1024;
+    const long px = (long)d->N * d->Ho * d->Wo * (d->K / 512);
+    return conv_pointwise_applicable(op, d, epi) && px >= (op == CKX_OP_CONV2D_FWD_I8 ? 16 * 1024 : 40 * 1024);
 }
 
 template <int DT, bool FUSED>
