@@ -303,3 +303,35 @@ def test_conv2d_pointwise_instance_refuses_other_shapes():
         assert L.ckx_conv2d_fwd_is_supported(capi.OP_CONV2D_FWD_F16, C.byref(d), 0, -1) == capi.OK
     # the residual functor stays with the tile kernel
     assert L.ckx_conv2d_fwd_is_supported(capi.OP_CONV2D_FWD_F16, C.byref(ok), capi.EPI_ADD_RELU_ADD, pw) == capi.UNSUPPORTED
+
+
+@pytest.mark.parametrize("shape", ["patch", "pointwise"])
+def test_conv2d_specialists_fall_back_on_unaligned_output(shape):
+    """The input-patch and pointwise kernels store whole 16-byte vectors: an output that starts 2 bytes into a buffer
+    is not theirs. The automatic choice must run such a problem on a tile instance (element stores), the explicit
+    instance must refuse it."""
+    import torch
+    import gpu_util
+    if shape == "patch":
+        inp, wei, s, p = uniform_f16((2, 8, 56, 64), -1, 1, 1030), uniform_f16((64, 3, 3, 64), -1, 1, 1031), (1, 1), (1, 1)
+    else:
+        inp, wei, s, p = uniform_f16((40, 56, 56, 256), -1, 1, 1032), uniform_f16((512, 1, 1, 256), -1, 1, 1033), (2, 2), (0, 0)
+    N, Hi, Wi, Cc = inp.shape
+    K, Y, X, _ = wei.shape
+    Ho, Wo = (Hi + 2 * p[0] - Y) // s[0] + 1, (Wi + 2 * p[1] - X) // s[1] + 1
+    di, dw = gpu_util.dev(inp), gpu_util.dev(wei)
+    buf = torch.full((N * Ho * Wo * K + 8,), float("nan"), dtype=torch.float16, device="cuda")
+    out = buf[1:1 + N * Ho * Wo * K]
+    geom = (N, K, Cc, [Hi, Wi], [Y, X], [Ho, Wo], list(s), [1, 1], list(p), list(p), None, None, None)
+    op = ck.DeviceConv2dFwdF16()
+    arg = op.MakeArgumentPointer(di, dw, out.data_ptr(), *geom)
+    assert op.IsSupportedArgument(arg), capi.last_error()
+    op.MakeInvokerPointer().Run(arg, ck.StreamConfig(gpu_util.stream()))
+    torch.cuda.synchronize()
+    host = buf.cpu().numpy()
+    assert np.isnan(host[0]) and np.isnan(host[1 + N * Ho * Wo * K:]).all()
+    _f16_close(host[1:1 + N * Ho * Wo * K].reshape(N, Ho, Wo, K), fast.conv2d_fwd_f16(inp, wei, s, (1, 1), p))
+    special = ck.DeviceConv2dFwdF16(gpu_util.conv_instance(capi.OP_CONV2D_FWD_F16, "Patch" if shape == "patch" else "Pointwise"))
+    arg = special.MakeArgumentPointer(di, dw, out.data_ptr(), *geom)
+    with pytest.raises(RuntimeError):
+        special.MakeInvokerPointer().Run(arg, ck.StreamConfig(gpu_util.stream()))
