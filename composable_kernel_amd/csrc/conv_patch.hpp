@@ -19,7 +19,8 @@
 //    (y rows, x pixels): the same 128-byte rows, another base address. A lane keeps one
 //    precomputed byte offset per (M tile, x) and one per (M tile, y): a fragment address is one add.
 //  * 16-byte chunks are swizzled by the patch COLUMN (fp16: chunk ^ (col & 7); int8, 4 chunks per pixel:
-//    chunk ^ ((col >> 2) & 3)), so the 16 pixels of a fragment read spread over all banks.
+//    chunk ^ (bit 0 and bit 2 of col)), so the 16 lanes the LDS serves in one cycle of a fragment read land on
+//    different banks.
 //  * 2 x 2 waves: a wave multiplies 16 * MTW pixels x 32 output channels; D^T = B_frag x A_frag with
 //    the weight rows permuted in LDS so that a lane ends up with 8 consecutive channels of one
 //    pixel: one 16-byte store, no trip through LDS.
@@ -81,7 +82,10 @@ struct ConvPatch
     static_assert(LDS <= 160 * 1024, "ring + weights fit the LDS");
     using acc_t = typename std::conditional<DT == DT_I8, i32x4, f32x4>::type;
     // swizzle key of a pixel column / weight row: the 16 rows of a fragment read must land on distinct banks
-    __device__ static __forceinline__ uint32_t key(uint32_t r) { return CPP == 8 ? (r & 7u) : ((r >> 2) & 3u); }
+    // (a ds_read_b128 is served in four cycles; the 16 lanes of a cycle are those with equal (lane bit 5, parity of
+    // lane bits 2..4). For 64-byte pixels the first choice, (r >> 2) & 3, left two-way conflicts under that grouping:
+    // SQ_LDS_BANK_CONFLICT was half of SQ_LDS_IDX_ACTIVE)
+    __device__ static __forceinline__ uint32_t key(uint32_t r) { return CPP == 8 ? (r & 7u) : ((r & 1u) | ((r >> 1) & 2u)); }
 
     __device__ static __forceinline__ void run(const ConvPatchArgs& p, uint8_t* smem)
     {
@@ -174,7 +178,8 @@ struct ConvPatch
             asm volatile("" ::: "memory");
         };
 
-        uint32_t roff[MTW][Y]; // ring byte offset of (M tile's output row + y) for the current band
+        uint32_t roff[MTW][Y];   // ring byte offset of (M tile's output row + y) for the current band
+        uint32_t roff_n[MTW][Y]; // ... for the next band: worked out one value per MFMA group, in the MFMAs' shadow
         i32x4 af[2][MTW], bf[2][NBT];
         const int nbands = (p.Ho + TH - 1) / TH;
         for(int n = (int)blockIdx.x; n < p.N; n += (int)gridDim.x)
@@ -244,6 +249,8 @@ struct ConvPatch
                 // the first groups and finished two groups early] [one direct load of the next band's
                 // rows] [the 2 MFMAs of one M tile]. With one wave per SIMD nothing else hides the
                 // issue slots of the reads, so they go between the MFMAs.
+                const uint32_t j1mod = (uint32_t)((j0 + TH) % RING); // first ring row of the next band
+                static_assert(KSP * TAPS >= Y, "one k-step per filter row for the next band's ring offsets");
                 constexpr int NR = MTW + NBT, RG = MTW > 2 ? MTW - 2 : MTW;
                 constexpr int NS = KSP * TAPS;           // k-steps of a band
                 constexpr int NBLK = TH * BPR / 4;       // direct loads per wave for the next band's rows
@@ -266,6 +273,13 @@ struct ConvPatch
                             const int k = wave + 4 * s;
                             load_block(n, j0 + NEED_ROWS + TH * (AHEAD - 1) + k / BPR, k % BPR);
                         }
+                        // ring offsets of the next band's rows, one (M tile, y) per group of the first Y k-steps
+                        if(s < Y)
+                        {
+                            uint32_t sl  = j1mod + rout[g] + (uint32_t)s;
+                            sl           = sl >= (uint32_t)RING ? sl - RING : sl;
+                            roff_n[g][s] = sl * (PITCH * PXB);
+                        }
                         mfma_pair(s, g);
                         __builtin_amdgcn_sched_barrier(0);
                     }
@@ -281,16 +295,11 @@ struct ConvPatch
                 barrier();
                 if(b + 1 < nbands)
                 {
-                    const int j1 = j0 + TH;
 #pragma unroll
                     for(int t = 0; t < MTW; ++t)
 #pragma unroll
                         for(int y = 0; y < Y; ++y)
-                        {
-                            uint32_t sl = (uint32_t)(j1 % RING) + rout[t] + (uint32_t)y;
-                            sl          = sl >= (uint32_t)RING ? sl - RING : sl;
-                            roff[t][y]  = sl * (PITCH * PXB);
-                        }
+                            roff[t][y] = roff_n[t][y];
 #pragma unroll
                     for(int r = 0; r < MTW + NBT; ++r)
                         read_one(0, r);

@@ -77,8 +77,24 @@ struct GemmGemmCfg
     static constexpr int BNC  = 128; // columns of the intermediate per step
     static constexpr int KP   = KS * 32;
     static constexpr int OP   = OG * 64;
-    static constexpr int AST  = KP * 2 + 16;  // padded LDS row strides (bytes): 16 rows hit 16 bank groups
-    static constexpr int B1ST = BNC * 2 + 16;
+    // LDS rows are unpadded and their 16-byte chunks XOR-swizzled with bits of the row index (ab_key / b1_key).
+    // A ds_read_b128 is served in four cycles of 16 lanes each, and the lanes of a cycle are those with equal
+    // (lane bit 5, parity of lane bits 2..4) -- measured with random bank-balanced address patterns, which that
+    // partition predicts exactly; row padding (16 bytes) left every fragment read of this kernel with two- to
+    // four-way bank conflicts under it (SQ_LDS_BANK_CONFLICT = half of SQ_LDS_IDX_ACTIVE). The keys make the 16
+    // lanes of every cycle of every fragment read land on 16 different 16-byte bank groups.
+    static constexpr int AST  = KP * 2;  // LDS row strides (bytes)
+    static constexpr int B1ST = BNC * 2;
+    // chunk position of chunk c of staged row r of A / B0: c ^ ab_key(r); of row o of the transposed B1: c ^ b1_key(o)
+    __device__ static __forceinline__ uint32_t ab_key(uint32_t r)
+    {
+        // (KP / 8 chunks per row: 4, 8 or 16 -- the key stays inside the row)
+        return (((r >> 3) & 1u) << 1) | (KP >= 64 ? ((r >> 1) & 1u) << 2 : 0u) | (KP == 128 ? (r & 1u) << 3 : 0u);
+    }
+    __device__ static __forceinline__ uint32_t b1_key(uint32_t o)
+    {
+        return (((o >> 4) & 1u) << 1) | (((o >> 1) & 1u) << 2) | ((o & 1u) << 3);
+    }
     static constexpr int A_BYTES   = BM * AST;
     static constexpr int B0_BYTES  = BNC * AST;
     static constexpr int B1T_BYTES = OP * B1ST;
@@ -165,7 +181,7 @@ __global__ __launch_bounds__(NW * 64)
         {
             const int idx = tid + NT * i;
             const int row = idx / KCH, ch = idx - row * KCH;
-            *reinterpret_cast<i32x4*>(sB0 + row * Cfg::AST + ch * 16) = rb0[i];
+            *reinterpret_cast<i32x4*>(sB0 + row * Cfg::AST + ((uint32_t)ch ^ Cfg::ab_key((uint32_t)row)) * 16) = rb0[i];
         }
 #pragma unroll
         for(int i = 0; i < NB1; ++i)
@@ -175,7 +191,8 @@ __global__ __launch_bounds__(NW * 64)
             const f16x8 v = __builtin_bit_cast(f16x8, rb1[i]);
 #pragma unroll
             for(int e = 0; e < 8; ++e) // transpose: B1T[o][n]
-                *reinterpret_cast<_Float16*>(sB1T + (ch * 8 + e) * Cfg::B1ST + row * 2) = v[e];
+                *reinterpret_cast<_Float16*>(sB1T + (ch * 8 + e) * Cfg::B1ST +
+                                             (((uint32_t)row >> 3) ^ Cfg::b1_key((uint32_t)(ch * 8 + e))) * 16 + (row & 7) * 2) = v[e];
         }
     };
 
@@ -189,7 +206,7 @@ __global__ __launch_bounds__(NW * 64)
         i32x4 v = zero4;
         if(m < p.M && k < p.K)
             v = *reinterpret_cast<const i32x4*>(A + (int64_t)m * p.sa + k);
-        *reinterpret_cast<i32x4*>(sA + row * Cfg::AST + ch * 16) = v;
+        *reinterpret_cast<i32x4*>(sA + row * Cfg::AST + ((uint32_t)ch ^ Cfg::ab_key((uint32_t)row)) * 16) = v;
     }
     __syncthreads();
     f16x8 af[MT][KS];
@@ -197,8 +214,10 @@ __global__ __launch_bounds__(NW * 64)
     for(int mt = 0; mt < MT; ++mt)
 #pragma unroll
         for(int ks = 0; ks < KS; ++ks)
-            af[mt][ks] = *reinterpret_cast<const f16x8*>(sA + (wave * 16 * MT + mt * 16 + fr) * Cfg::AST +
-                                                         (ks * 4 + q) * 16);
+        {
+            const uint32_t arow = (uint32_t)(wave * 16 * MT + mt * 16 + fr);
+            af[mt][ks] = *reinterpret_cast<const f16x8*>(sA + arow * Cfg::AST + ((uint32_t)(ks * 4 + q) ^ Cfg::ab_key(arow)) * 16);
+        }
 
     f32x4 acc1[MT][OG * 4];
 #pragma unroll
@@ -252,7 +271,7 @@ __global__ __launch_bounds__(NW * 64)
             {
                 const int row = 32 * (t >> 1) + 8 * (fr >> 2) + 4 * (t & 1) + (fr & 3);
                 const f16x8 b0f =
-                    *reinterpret_cast<const f16x8*>(sB0 + row * Cfg::AST + (ks * 4 + q) * 16);
+                    *reinterpret_cast<const f16x8*>(sB0 + row * Cfg::AST + ((uint32_t)(ks * 4 + q) ^ Cfg::ab_key((uint32_t)row)) * 16);
 #pragma unroll
                 for(int mt = 0; mt < MT; ++mt)
                     s[mt][t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(b0f, af[mt][ks], s[mt][t], 0, 0, 0);
@@ -337,7 +356,7 @@ __global__ __launch_bounds__(NW * 64)
             {
                 const int o = 64 * (ot >> 2) + 16 * (fr >> 2) + 4 * (ot & 3) + (fr & 3);
                 const f16x8 b1f =
-                    *reinterpret_cast<const f16x8*>(sB1T + o * Cfg::B1ST + (32 * pr + 8 * q) * 2);
+                    *reinterpret_cast<const f16x8*>(sB1T + o * Cfg::B1ST + ((uint32_t)(4 * pr + q) ^ Cfg::b1_key((uint32_t)o)) * 16);
 #pragma unroll
                 for(int mt = 0; mt < MT; ++mt)
                     acc1[mt][ot] =
