@@ -17,7 +17,7 @@ typedef hipError_t (*tile_launch_fn)(const GemmArgs&, int grid, hipStream_t);
 // The position in this list is the instance index of the C ABI.
 #define CKX_FOR_EACH_TILE(X)     \
     X(256, 256, 2, 4, 2, 1.00f)  \
-    X(256, 128, 4, 2, 2, 0.84f)  \
+    X(256, 128, 4, 2, 3, 0.84f)  \
     X(128, 128, 2, 2, 2, 0.70f)  \
     X(128, 64, 4, 1, 2, 0.68f)   \
     X(64, 64, 4, 1, 2, 0.55f)    \
