@@ -196,6 +196,47 @@ __global__ __launch_bounds__(NW * 64)
         }
     };
 
+    // the same for the second register set of the two-step prefetch (unused, and gone, where PF == 1)
+    i32x4 rb0b[NB0], rb1b[NB1];
+    auto load_into = [&](int n0, i32x4(&r0)[NB0], i32x4(&r1)[NB1]) {
+#pragma unroll
+        for(int i = 0; i < NB0; ++i)
+        {
+            const int idx = tid + NT * i;
+            const int row = idx / KCH, ch = idx - row * KCH;
+            const int n = n0 + row, k = ch * 8;
+            r0[i] = (n < p.N && k < p.K) ? *reinterpret_cast<const i32x4*>(B0 + (int64_t)n * p.sb0 + k) : zero4;
+        }
+#pragma unroll
+        for(int i = 0; i < NB1; ++i)
+        {
+            const int idx = tid + NT * i;
+            const int ch = idx / Cfg::BNC, row = idx - ch * Cfg::BNC;
+            const int n = n0 + row, o = ch * 8;
+            r1[i] = (n < p.N && o < p.O) ? *reinterpret_cast<const i32x4*>(B1 + (int64_t)n * p.sb1 + o) : zero4;
+        }
+    };
+    auto store_from = [&](const i32x4(&r0)[NB0], const i32x4(&r1)[NB1]) {
+#pragma unroll
+        for(int i = 0; i < NB0; ++i)
+        {
+            const int idx = tid + NT * i;
+            const int row = idx / KCH, ch = idx - row * KCH;
+            *reinterpret_cast<i32x4*>(sB0 + row * Cfg::AST + ((uint32_t)ch ^ Cfg::ab_key((uint32_t)row)) * 16) = r0[i];
+        }
+#pragma unroll
+        for(int i = 0; i < NB1; ++i)
+        {
+            const int idx = tid + NT * i;
+            const int ch = idx / Cfg::BNC, row = idx - ch * Cfg::BNC;
+            const f16x8 v = __builtin_bit_cast(f16x8, r1[i]);
+#pragma unroll
+            for(int e = 0; e < 8; ++e)
+                *reinterpret_cast<_Float16*>(sB1T + (ch * 8 + e) * Cfg::B1ST +
+                                             (((uint32_t)row >> 3) ^ Cfg::b1_key((uint32_t)(ch * 8 + e))) * 16 + (row & 7) * 2) = v[e];
+        }
+    };
+
     load_step(0);
 
     // ---- A slab -> LDS -> registers (kept for the whole kernel) -----------------------
@@ -249,119 +290,51 @@ __global__ __launch_bounds__(NW * 64)
     // with the upper-triangle mask, columns past the slab's last row are masked for every row of it
     const int n_end = (SOFTMAX && p.mask_upper && m0 + Cfg::BM < p.N) ? m0 + Cfg::BM : p.N;
 
-    for(int n0 = 0; n0 < n_end; n0 += Cfg::BNC)
+    // ---- main loop over the steps ---------------------------------------------------------------------------
+    // A step's MFMAs take well under a microsecond, a load out of HBM longer: with one step of register prefetch
+    // every step of a short problem (N = 512: four steps) ends waiting for its successor's slices. Where the
+    // registers allow, the slices of TWO steps are in flight (PF == 2: a second register set, the loop unrolled by
+    // two). The softmax variants and the largest plain one have no room (they would spill) and keep one.
+    constexpr int PF = (SOFTMAX || (KS == 4 && OG == 2 && MT == 2) || (MT == 2 && NW == 4)) ? 1 : 2;
+    if constexpr(PF == 1)
     {
-        __syncthreads(); // everyone is done reading the previous step from LDS
-        store_step();
-        __syncthreads();
-        if(n0 + Cfg::BNC < n_end)
-            load_step(n0 + Cfg::BNC); // in flight while this step is multiplied
-
-        // ---- gemm0: S^T tiles, 8 tiles of 16 columns, pairs share a 32-column span -----
-        f32x4 s[MT][8];
-#pragma unroll
-        for(int mt = 0; mt < MT; ++mt)
-#pragma unroll
-            for(int t = 0; t < 8; ++t)
-                s[mt][t] = f32x4{0, 0, 0, 0};
-#pragma unroll
-        for(int ks = 0; ks < KS; ++ks)
-#pragma unroll
-            for(int t = 0; t < 8; ++t)
-            {
-                const int row = 32 * (t >> 1) + 8 * (fr >> 2) + 4 * (t & 1) + (fr & 3);
-                const f16x8 b0f =
-                    *reinterpret_cast<const f16x8*>(sB0 + row * Cfg::AST + ((uint32_t)(ks * 4 + q) ^ Cfg::ab_key((uint32_t)row)) * 16);
-#pragma unroll
-                for(int mt = 0; mt < MT; ++mt)
-                    s[mt][t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(b0f, af[mt][ks], s[mt][t], 0, 0, 0);
-            }
-
-        if constexpr(SOFTMAX)
+        for(int n0 = 0; n0 < n_end; n0 += Cfg::BNC)
         {
-            // s[mt][t][j] is the score of row m0 + wave*16*MT + 16*mt + fr, column n0 + 32*(t/2) + 8q + 4*(t%2) + j.
-            // The running maximum is kept as x = score * |scale| * log2(e), so that exp(score - max) is one
-            // fused multiply-add and one v_exp_f32 (a negative scale has been moved into A's sign above, which
-            // lets the maximum be taken over the raw scores).
-            // Does this step hold masked columns for any row of this wave? (wave-uniform: the plain path
-            // skips the per-element compare and select)
-            const int wave_m0    = m0 + wave * 16 * MT;
-            const bool step_mask = n0 + Cfg::BNC > p.N || (p.mask_upper && n0 + Cfg::BNC > wave_m0 + 1);
-#pragma unroll
-            for(int mt = 0; mt < MT; ++mt)
+            __syncthreads(); // everyone is done reading the previous step from LDS
+            store_step();
+            __syncthreads();
+            if(n0 + Cfg::BNC < n_end)
+                load_step(n0 + Cfg::BNC); // in flight while this step is multiplied
+#include "gemm_gemm_step.inc"
+        }
+    }
+    else
+    {
+        // step i lives in register set i % 2 until it goes to LDS
+        if(Cfg::BNC < n_end)
+            load_into(Cfg::BNC, rb0b, rb1b);
+        for(int nb = 0; nb < n_end; nb += 2 * Cfg::BNC)
+        {
             {
-                const int m     = wave_m0 + mt * 16 + fr;
-                const int n_lim = (p.mask_upper && m + 1 < p.N) ? m + 1 : p.N; // columns >= n_lim are masked
-                if(step_mask)
-                {
-#pragma unroll
-                    for(int t = 0; t < 8; ++t)
-#pragma unroll
-                        for(int j = 0; j < 4; ++j)
-                        {
-                            const int n = n0 + 32 * (t >> 1) + 8 * q + 4 * (t & 1) + j;
-                            s[mt][t][j] = n < n_lim ? s[mt][t][j] : ninf;
-                        }
-                }
-                float mx = ninf;
-#pragma unroll
-                for(int t = 0; t < 8; ++t)
-                    mx = __builtin_fmaxf(__builtin_fmaxf(mx, __builtin_fmaxf(s[mt][t][0], s[mt][t][1])),
-                                         __builtin_fmaxf(s[mt][t][2], s[mt][t][3]));
-                mx = quad_rows_max(mx);
-                // (c2 > 0: the maximum commutes with the scaling, and -inf stays -inf)
-                const float m_new  = __builtin_fmaxf(row_max[mt], mx * c2);
-                const float m_safe = m_new == ninf ? 0.0f : m_new; // a row with nothing unmasked yet: every p is 0
-                const float corr   = __builtin_amdgcn_exp2f(row_max[mt] - m_safe);
-                row_max[mt]        = m_new;
-                float part = 0.0f;
-#pragma unroll
-                for(int t = 0; t < 8; ++t)
-#pragma unroll
-                    for(int j = 0; j < 4; ++j)
-                    {
-                        const float e = __builtin_amdgcn_exp2f(__builtin_fmaf(s[mt][t][j], c2, -m_safe));
-                        s[mt][t][j]   = e;
-                        part += e;
-                    }
-                row_sum[mt] = row_sum[mt] * corr + part;
-                // (wave-uniform skip: once the running maxima have settled, corr is 1 in every lane)
-                if(__builtin_amdgcn_ballot_w64(corr != 1.0f) != 0)
-                {
-#pragma unroll
-                    for(int ot = 0; ot < OG * 4; ++ot)
-                        acc1[mt][ot] = acc1[mt][ot] * corr;
-                }
+                const int n0 = nb;
+                __syncthreads();
+                store_from(rb0, rb1);
+                __syncthreads();
+                if(n0 + 2 * Cfg::BNC < n_end)
+                    load_into(n0 + 2 * Cfg::BNC, rb0, rb1);
+#include "gemm_gemm_step.inc"
+            }
+            if(nb + Cfg::BNC < n_end)
+            {
+                const int n0 = nb + Cfg::BNC;
+                __syncthreads();
+                store_from(rb0b, rb1b);
+                __syncthreads();
+                if(n0 + 2 * Cfg::BNC < n_end)
+                    load_into(n0 + 2 * Cfg::BNC, rb0b, rb1b);
+#include "gemm_gemm_step.inc"
             }
         }
-
-        // ---- fp32 -> fp16 (RNE): the pair (2*pr, 2*pr+1) is the gemm1 operand for 32 n ----
-        f16x8 sf[MT][4];
-#pragma unroll
-        for(int mt = 0; mt < MT; ++mt)
-#pragma unroll
-            for(int pr = 0; pr < 4; ++pr)
-#pragma unroll
-                for(int j = 0; j < 4; ++j)
-                {
-                    sf[mt][pr][j]     = (_Float16)s[mt][2 * pr][j];
-                    sf[mt][pr][4 + j] = (_Float16)s[mt][2 * pr + 1][j];
-                }
-
-        // ---- gemm1: C^T tiles ------------------------------------------------------------
-#pragma unroll
-        for(int pr = 0; pr < 4; ++pr)
-#pragma unroll
-            for(int ot = 0; ot < OG * 4; ++ot)
-            {
-                const int o = 64 * (ot >> 2) + 16 * (fr >> 2) + 4 * (ot & 3) + (fr & 3);
-                const f16x8 b1f =
-                    *reinterpret_cast<const f16x8*>(sB1T + o * Cfg::B1ST + ((uint32_t)(4 * pr + q) ^ Cfg::b1_key((uint32_t)o)) * 16);
-#pragma unroll
-                for(int mt = 0; mt < MT; ++mt)
-                    acc1[mt][ot] =
-                        __builtin_amdgcn_mfma_f32_16x16x32_f16(b1f, sf[mt][pr], acc1[mt][ot], 0, 0, 0);
-            }
     }
 
     const bool vec_ok = ((reinterpret_cast<uintptr_t>(C) | ((uintptr_t)p.sc * 2)) & 15u) == 0;
@@ -473,7 +446,9 @@ inline hipError_t gemm_gemm_launch(const void* a, const void* b0, const void* b1
         // softmax: many short waves overlap one wave's exponentials with another's MFMAs (8 x 16 rows: 13.4 vs
         // 14.8 us at batch 64, 512 x 512 scores); over a long N the 32-row waves of the register-capped variant
         // read B0 / B1 fragments half as often per row and win (434 vs 581 us at 4096 x 4096)
-        instance = !softmax ? 0 : (K <= 64 && O <= 64 && N >= 1024) ? 0 : 2;
+        // plain: the 8-wave instance, the one with two steps of prefetch (8.6 against 10.2 us on G 64, 512 x 64 x 512 x 64,
+        // ahead on every shape measured); softmax: 32 rows per wave for long rows of small heads, else 8 waves
+        instance = !softmax ? 2 : (K <= 64 && O <= 64 && N >= 1024) ? 0 : 2;
     if(softmax)
         return instance == 0 ? gemm_gemm_launch_mt<2, 4, true>(g, s)
                : instance == 1 ? gemm_gemm_launch_mt<1, 4, true>(g, s)
