@@ -295,7 +295,7 @@ __global__ __launch_bounds__(NW * 64)
     // every step of a short problem (N = 512: four steps) ends waiting for its successor's slices. Where the
     // registers allow, the slices of TWO steps are in flight (PF == 2: a second register set, the loop unrolled by
     // two). The softmax variants and the largest plain one have no room (they would spill) and keep one.
-    constexpr int PF = (SOFTMAX || (KS == 4 && OG == 2 && MT == 2) || (MT == 2 && NW == 4)) ? 1 : 2;
+    constexpr int PF = ((MT == 2 && NW == 4) || (SOFTMAX && (NW != 8 || (KS == 4 && OG == 2)))) ? 1 : 2;
     if constexpr(PF == 1)
     {
         for(int n0 = 0; n0 < n_end; n0 += Cfg::BNC)
