@@ -185,9 +185,12 @@ struct ConvPatch
         for(int n = (int)blockIdx.x; n < p.N; n += (int)gridDim.x)
         {
             // rows of the first band (every wave has passed the barrier that ended the previous image)
+            // and of the AHEAD - 1 bands after it; only the first band's have to land before the MFMAs start (a wave
+            // issues its blocks in ascending order and loads retire in order)
+            static_assert((NEED_ROWS * BPR) % 4 == 0 && (TH * BPR) % 4 == 0, "the same number of blocks for every wave");
             for(int k = wave; k < (NEED_ROWS + TH * (AHEAD - 1)) * BPR; k += 4)
                 load_block(n, k / BPR, k % BPR);
-            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+            asm volatile("s_waitcnt vmcnt(%0)" ::"n"((AHEAD - 1) * TH * BPR / 4) : "memory");
             barrier();
 
             for(int b = 0; b < nbands; ++b)
