@@ -112,3 +112,48 @@ def test_random_conv(kind, seed):
     else:
         bad, max_err = lit.check_err_f16(out, fast.convnd_fwd(inp, wei, st, dil, pad, rpad), 1e-2, 1e-2)
         assert bad == 0, f"{desc}: {bad} outside tolerance, max err {max_err}"
+
+
+@pytest.mark.parametrize("seed", range(80))
+def test_random_gemm_gemm(seed):
+    """Fused GEMM-GEMM and GEMM-softmax-GEMM: random batch / row / column counts (ragged slabs and steps, one to
+    many 128-column steps), K and O at every multiple of 8 up to 128, padded strides, scale sign, mask, instance."""
+    import torch
+    import gpu_util
+    rng = np.random.default_rng(11000 + seed)
+    G, M, N = int(rng.integers(1, 5)), int(rng.integers(1, 300)), int(rng.integers(1, 700))
+    K, O = 8 * int(rng.integers(1, 17)), 8 * int(rng.integers(1, 17))
+    softmax = bool(rng.integers(0, 2))
+    mask = softmax and bool(rng.integers(0, 2))
+    scale = float(rng.choice([1.0, -0.7, 0.25])) / np.sqrt(K) if softmax else 1.0
+    instance = int(rng.integers(-1, capi.lib().ckx_num_instances(capi.OP_BATCHED_GEMM_GEMM)))
+    pad = [8 * int(rng.integers(0, 3)) for _ in range(4)]
+    lim = 1.0 if softmax else 0.5
+    a, b0, b1 = (rng.uniform(-lim, lim, s).astype(np.float16) for s in ((G, M, K), (G, N, K), (G, N, O)))
+
+    def padded(x, p):
+        out = np.zeros(x.shape[:2] + (x.shape[2] + p,), np.float16)
+        out[..., :x.shape[2]] = x
+        return out
+
+    ha, hb0, hb1 = padded(a, pad[0]), padded(b0, pad[1]), padded(b1, pad[2])
+    da, db0, db1 = (torch.from_numpy(x.view(np.int16)).cuda() for x in (ha, hb0, hb1))
+    dc = torch.full((G, M, O + pad[3]), 0x7E00, dtype=torch.int16, device="cuda")
+    dims = (M, N, K, O, G, K + pad[0], K + pad[1], O + pad[2], O + pad[3], M * (K + pad[0]), N * (K + pad[1]),
+            N * (O + pad[2]), M * (O + pad[3]))
+    if softmax:
+        op = ck.DeviceBatchedGemmSoftmaxGemmF16(instance, MaskOutUpperTriangle=mask)
+        arg = op.MakeArgumentPointer(da, db0, db1, dc, *dims, None, None, ck.Scale(scale))
+        ref = lit.batched_gemm_softmax_gemm_f16(a, b0.transpose(0, 2, 1), b1, scale, mask)
+    else:
+        op = ck.DeviceBatchedGemmGemmF16(instance)
+        arg = op.MakeArgumentPointer(da, db0, db1, dc, *dims)
+        ref = lit.batched_gemm_gemm_f16(a, b0.transpose(0, 2, 1), b1)
+    desc = f"G{G} M{M} N{N} K{K} O{O} softmax{softmax} mask{mask} scale{scale:.3f} inst{instance} pad{pad}"
+    assert op.IsSupportedArgument(arg), desc + ": " + capi.last_error().decode()
+    op.MakeInvokerPointer().Run(arg, ck.StreamConfig(gpu_util.stream()))
+    torch.cuda.synchronize()
+    out = dc.cpu().numpy().view(np.float16)
+    assert np.all(out[..., O:].view(np.uint16) == 0x7E00), desc + ": wrote outside the C rows"
+    bad, max_err = lit.check_err_f16(np.ascontiguousarray(out[..., :O]), ref, 1e-2, 1e-2)
+    assert bad == 0, f"{desc}: {bad} outside tolerance, max err {max_err}"
