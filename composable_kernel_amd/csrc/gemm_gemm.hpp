@@ -57,14 +57,39 @@ __device__ __forceinline__ float quad_rows_sum(float x)
     const uint32_t b0 = b[0], b1 = b[1];
     return __builtin_bit_cast(float, b0) + __builtin_bit_cast(float, b1);
 }
+// Maxima of scores as bare v_max_f32 / v_max3_f32. In front of every fmaxf operand that it cannot prove to be a quiet
+// number (an MFMA result, a lane swap) the compiler puts a canonicalising v_max_f32 x, x, x, which doubled the
+// instructions of the running maximum. (A NaN score makes its row of the output NaN through the exponentials
+// whatever the maximum is.) The compiler does not see what an asm statement reads, so it cannot keep the distance
+// that the hardware asks for between an MFMA and a VALU read of its result: mfma_results_settle() goes between.
+__device__ __forceinline__ float max2_valu(float a, float b)
+{
+    float d;
+    asm("v_max_f32 %0, %1, %2" : "=v"(d) : "v"(a), "v"(b));
+    return d;
+}
+__device__ __forceinline__ float max3_valu(float a, float b, float c)
+{
+    float d;
+    asm("v_max3_f32 %0, %1, %2, %3" : "=v"(d) : "v"(a), "v"(b), "v"(c));
+    return d;
+}
+// 24 wait states after the MFMAs issued so far, and nothing scheduled across: more than the longest
+// MFMA-write-to-VALU-read distance of the architecture (passes + 3 wait states for the 16-pass instructions).
+__device__ __forceinline__ void mfma_results_settle()
+{
+    __builtin_amdgcn_sched_barrier(0);
+    asm volatile("s_nop 15\n\ts_nop 7");
+    __builtin_amdgcn_sched_barrier(0);
+}
 __device__ __forceinline__ float quad_rows_max(float x)
 {
     auto a = __builtin_amdgcn_permlane16_swap(__builtin_bit_cast(uint32_t, x), __builtin_bit_cast(uint32_t, x), false, false);
     const uint32_t a0 = a[0], a1 = a[1];
-    x      = __builtin_fmaxf(__builtin_bit_cast(float, a0), __builtin_bit_cast(float, a1));
+    x      = max2_valu(__builtin_bit_cast(float, a0), __builtin_bit_cast(float, a1));
     auto b = __builtin_amdgcn_permlane32_swap(__builtin_bit_cast(uint32_t, x), __builtin_bit_cast(uint32_t, x), false, false);
     const uint32_t b0 = b[0], b1 = b[1];
-    return __builtin_fmaxf(__builtin_bit_cast(float, b0), __builtin_bit_cast(float, b1));
+    return max2_valu(__builtin_bit_cast(float, b0), __builtin_bit_cast(float, b1));
 }
 
 // KS  k-steps of gemm0 (K padded to 32*KS), OG  64-column groups of the output (O padded to 64*OG),
