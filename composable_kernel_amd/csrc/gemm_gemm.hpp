@@ -48,6 +48,9 @@ struct GemmGemmArgs
 };
 
 // maximum / sum over the four lanes l, l^16, l^32, l^48 (every one of them gets the result)
+typedef short s16x4_t __attribute__((__vector_size__(4 * sizeof(short))));
+typedef __attribute__((address_space(3))) s16x4_t lds_s16x4;
+
 __device__ __forceinline__ float quad_rows_sum(float x)
 {
     auto a = __builtin_amdgcn_permlane16_swap(__builtin_bit_cast(uint32_t, x), __builtin_bit_cast(uint32_t, x), false, false);
@@ -108,21 +111,29 @@ struct GemmGemmCfg
     // partition predicts exactly; row padding (16 bytes) left every fragment read of this kernel with two- to
     // four-way bank conflicts under it (SQ_LDS_BANK_CONFLICT = half of SQ_LDS_IDX_ACTIVE). The keys make the 16
     // lanes of every cycle of every fragment read land on 16 different 16-byte bank groups.
-    static constexpr int AST  = KP * 2;  // LDS row strides (bytes)
-    static constexpr int B1ST = BNC * 2;
-    // chunk position of chunk c of staged row r of A / B0: c ^ ab_key(r); of row o of the transposed B1: c ^ b1_key(o)
+    static constexpr int AST  = KP * 2; // LDS row stride of A / B0 (bytes)
+    // chunk position of chunk c of staged row r of A / B0: c ^ ab_key(r)
     __device__ static __forceinline__ uint32_t ab_key(uint32_t r)
     {
         // (KP / 8 chunks per row: 4, 8 or 16 -- the key stays inside the row)
         return (((r >> 3) & 1u) << 1) | (KP >= 64 ? ((r >> 1) & 1u) << 2 : 0u) | (KP == 128 ? (r & 1u) << 3 : 0u);
     }
-    __device__ static __forceinline__ uint32_t b1_key(uint32_t o)
+    // The B1 slice of a step stays as it is in memory, [n][o] (row stride B1RS bytes), and the gemm1 operand -- for
+    // one o, eight consecutive n -- comes out of it through the transposing read ds_read_b64_tr_b16: within 16 lanes,
+    // lane 4e + j points at four consecutive o of row n + e, and lane i receives element i of the 16 so addressed
+    // in each of the four rows. (Transposing on the way in took 32 two-byte LDS writes per thread and step.)
+    // b1_key(n): XOR mask on the byte offset inside row n, so that the 32 lanes of a half wave (rows n + e and
+    // n + 8 + e, four 8-byte pieces each) touch 32 different 8-byte bank pairs: with 128-byte rows the parity of n
+    // already selects the bank half and bits 1 and 3 of n move the piece (bits 3, 4 of the offset); 256-byte rows
+    // all start at bank 0, and bit 0 of n swaps the two 128-byte halves as well.
+    static constexpr int B1RS = OP * 2;
+    __device__ static __forceinline__ uint32_t b1_key(uint32_t n)
     {
-        return (((o >> 4) & 1u) << 1) | (((o >> 1) & 1u) << 2) | ((o & 1u) << 3);
+        return (((n >> 1) & 1u) << 3) | (((n >> 3) & 1u) << 4) | (OG == 2 ? (n & 1u) << 7 : 0u);
     }
     static constexpr int A_BYTES   = BM * AST;
     static constexpr int B0_BYTES  = BNC * AST;
-    static constexpr int B1T_BYTES = OP * B1ST;
+    static constexpr int B1T_BYTES = BNC * B1RS;
     static constexpr int LDS       = A_BYTES + B0_BYTES + B1T_BYTES;
     static constexpr int KCH = KP / 8; // 16-byte chunks per staged row of A / B0
     static constexpr int OCH = OP / 8;
@@ -191,11 +202,8 @@ __global__ __launch_bounds__(NW * 64)
 #pragma unroll
         for(int i = 0; i < NB1; ++i)
         {
-            // consecutive lanes take consecutive rows n: the transposed 2-byte LDS writes below
-            // then land in consecutive addresses (no bank conflicts); the 16-byte pieces of one
-            // 128-byte line are picked up by the same thread group across i and hit in L1
             const int idx = tid + NT * i;
-            const int ch = idx / Cfg::BNC, row = idx - ch * Cfg::BNC;
+            const int row = idx / OCH, ch = idx - row * OCH;
             const int n = n0 + row, o = ch * 8;
             rb1[i] = (n < p.N && o < p.O) ? *reinterpret_cast<const i32x4*>(B1 + (int64_t)n * p.sb1 + o) : zero4;
         }
@@ -212,12 +220,12 @@ __global__ __launch_bounds__(NW * 64)
         for(int i = 0; i < NB1; ++i)
         {
             const int idx = tid + NT * i;
-            const int ch = idx / Cfg::BNC, row = idx - ch * Cfg::BNC;
-            const f16x8 v = __builtin_bit_cast(f16x8, rb1[i]);
-#pragma unroll
-            for(int e = 0; e < 8; ++e) // transpose: B1T[o][n]
-                *reinterpret_cast<_Float16*>(sB1T + (ch * 8 + e) * Cfg::B1ST +
-                                             (((uint32_t)row >> 3) ^ Cfg::b1_key((uint32_t)(ch * 8 + e))) * 16 + (row & 7) * 2) = v[e];
+            const int row = idx / OCH, ch = idx - row * OCH;
+            // (two 8-byte halves: the key may swap them)
+            uint8_t* dst = sB1T + row * Cfg::B1RS;
+            const uint32_t off = (uint32_t)(ch * 16) ^ Cfg::b1_key((uint32_t)row);
+            *reinterpret_cast<i32x2*>(dst + off)       = i32x2{rb1[i][0], rb1[i][1]};
+            *reinterpret_cast<i32x2*>(dst + (off ^ 8)) = i32x2{rb1[i][2], rb1[i][3]};
         }
     };
 
@@ -236,7 +244,7 @@ __global__ __launch_bounds__(NW * 64)
         for(int i = 0; i < NB1; ++i)
         {
             const int idx = tid + NT * i;
-            const int ch = idx / Cfg::BNC, row = idx - ch * Cfg::BNC;
+            const int row = idx / OCH, ch = idx - row * OCH;
             const int n = n0 + row, o = ch * 8;
             r1[i] = (n < p.N && o < p.O) ? *reinterpret_cast<const i32x4*>(B1 + (int64_t)n * p.sb1 + o) : zero4;
         }
@@ -253,12 +261,11 @@ __global__ __launch_bounds__(NW * 64)
         for(int i = 0; i < NB1; ++i)
         {
             const int idx = tid + NT * i;
-            const int ch = idx / Cfg::BNC, row = idx - ch * Cfg::BNC;
-            const f16x8 v = __builtin_bit_cast(f16x8, r1[i]);
-#pragma unroll
-            for(int e = 0; e < 8; ++e)
-                *reinterpret_cast<_Float16*>(sB1T + (ch * 8 + e) * Cfg::B1ST +
-                                             (((uint32_t)row >> 3) ^ Cfg::b1_key((uint32_t)(ch * 8 + e))) * 16 + (row & 7) * 2) = v[e];
+            const int row = idx / OCH, ch = idx - row * OCH;
+            uint8_t* dst = sB1T + row * Cfg::B1RS;
+            const uint32_t off = (uint32_t)(ch * 16) ^ Cfg::b1_key((uint32_t)row);
+            *reinterpret_cast<i32x2*>(dst + off)       = i32x2{r1[i][0], r1[i][1]};
+            *reinterpret_cast<i32x2*>(dst + (off ^ 8)) = i32x2{r1[i][2], r1[i][3]};
         }
     };
 
@@ -284,6 +291,10 @@ __global__ __launch_bounds__(NW * 64)
             const uint32_t arow = (uint32_t)(wave * 16 * MT + mt * 16 + fr);
             af[mt][ks] = *reinterpret_cast<const f16x8*>(sA + arow * Cfg::AST + ((uint32_t)(ks * 4 + q) ^ Cfg::ab_key(arow)) * 16);
         }
+
+    // byte offset inside the B1 slice that this lane addresses in the transposing reads of gemm1
+    const uint32_t b1_lane =
+        (uint32_t)(8 * q + (fr >> 2)) * Cfg::B1RS + ((uint32_t)(32 * (fr & 3)) ^ Cfg::b1_key((uint32_t)(8 * q + (fr >> 2))));
 
     f32x4 acc1[MT][OG * 4];
 #pragma unroll
