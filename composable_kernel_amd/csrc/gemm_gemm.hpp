@@ -479,12 +479,12 @@ inline hipError_t gemm_gemm_launch(const void* a, const void* b0, const void* b1
     g.slabs = 0;
     g.scale = scale, g.mask_upper = mask_upper;
     if(instance < 0)
-        // softmax: many short waves overlap one wave's exponentials with another's MFMAs (8 x 16 rows: 13.4 vs
-        // 14.8 us at batch 64, 512 x 512 scores); over a long N the 32-row waves of the register-capped variant
-        // read B0 / B1 fragments half as often per row and win (434 vs 581 us at 4096 x 4096)
-        // plain: the 8-wave instance, the one with two steps of prefetch (8.6 against 10.2 us on G 64, 512 x 64 x 512 x 64,
-        // ahead on every shape measured); softmax: 32 rows per wave for long rows of small heads, else 8 waves
-        instance = !softmax ? 2 : (K <= 64 && O <= 64 && N >= 1024) ? 0 : 2;
+        // Many short waves (8 x 16 rows, the instance with two steps of prefetch where registers allow) are ahead on
+        // short problems: G 64, 512 x 64 x 512 x 64 plain 8.5 against 10.1 us, with softmax 10.9 against 13.0. Over a
+        // long N with small heads the 32-row waves read the B0 / B1 fragments half as often per row and win: G 64,
+        // 4096 x 64 x 4096 x 64 plain 267 against 302 us, softmax 367 against 433 (2048: 76 / 85 and 102 / 115; at
+        // N = 1024 the plain pair ties, softmax 31.3 / 34.0).
+        instance = (K <= 64 && O <= 64 && N >= (softmax ? 1024 : 2048)) ? 0 : 2;
     if(softmax)
         return instance == 0 ? gemm_gemm_launch_mt<2, 4, true>(g, s)
                : instance == 1 ? gemm_gemm_launch_mt<1, 4, true>(g, s)
