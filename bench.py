@@ -57,12 +57,12 @@ def _conv3d_workload(name, dtype, C, K, f, DHW, st, pd, N, dil=1):
                 bytes=byts, fused=None)
 
 
-def _gemm_workload(name, dtype, M, N, K, values=5, scales=(0.5, 0.03), fused=None, batch=1, layout="mk_nk"):
+def _gemm_workload(name, dtype, M, N, K, values=5, scales=(0.5, 0.03), fused=None, batch=1, layout="mk_nk", init="uniform"):
     """fused: None or "bias_relu" (fp16: E = AddRelu(half(A*B), bias row)); batch > 1: strided batched GEMM;
     layout: how A ("mk" row-major / "km" column-major) and B ("nk" column-major / "kn" row-major) are stored."""
     es = 1 if dtype == "i8" else 2
     return dict(name=name, kind="gemm", dtype=dtype, M=M, N=N, K=K, values=values, scales=scales, batch=batch,
-                layout=layout,
+                layout=layout, init=init,
                 ops=2.0 * M * N * K * batch, bytes=(M * K + N * K + M * N + (N if fused else 0)) * es * batch,
                 fused=fused)
 
@@ -82,6 +82,7 @@ for w in (
     + [_gemm_workload(f"fp16_gemm_4096_{lay}", "f16", 4096, 4096, 4096, layout=lay) for lay in ("km_kn", "km_nk", "mk_kn")]
     + [_gemm_workload(f"int8_requant_gemm_4096_{lay}", "i8", 4096, 4096, 4096, layout=lay) for lay in ("km_kn", "km_nk", "mk_kn")]
     + [_gemm_workload("fp16_gemm_bias_relu_4096", "f16", 4096, 4096, 4096, fused="bias_relu"),
+       _gemm_workload("fp16_gemm_4096_integer_init", "f16", 4096, 4096, 4096, init="integer"),
        _conv_workload("conv_f16_c64_k64_3x3_56_bias_relu_add", "f16", 64, 64, 3, 56, 1, 1, fused="bias_relu_add"),
        _conv_workload("conv_f16_c256_k512_1x1_56_s2_bias_relu", "f16", 256, 512, 1, 56, 2, 0, fused="bias_relu")]
     # three spatial dimensions: the reference's device-test default (conv3d_fwd.cpp:76-77) and a larger 3x3x3 layer
@@ -127,7 +128,12 @@ def make_launcher(w, instance=-1, rotate=1):
             op = ck.DeviceGemmInt8(instance, **lay)
             cop = ck.RequantReluRequant(w["scales"][0], w["scales"][1], rounded=True)
         else:
-            a, b = dev(uniform_f16(a_shape, -1, 1, 1)), dev(uniform_f16(b_shape, -1, 1, 2))
+            if w.get("init") == "integer":
+                # the reference profiler's initialisation 1 (its published runs): integers in [-5, 5]
+                a = dev(uniform_int8(a_shape, -5, 5, 1).astype(np.float16))
+                b = dev(uniform_int8(b_shape, -5, 5, 2).astype(np.float16))
+            else:
+                a, b = dev(uniform_f16(a_shape, -1, 1, 1)), dev(uniform_f16(b_shape, -1, 1, 2))
             c = torch.empty((M, N), dtype=torch.float16, device="cuda")
             op = ck.DeviceGemmF16(instance, **lay)
             cop = ck.PassThrough()
