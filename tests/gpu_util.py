@@ -110,13 +110,13 @@ def convnd_fwd(inp, wei, strides, dilations, pads, out_op=None, instance=capi.IN
     return do.cpu().numpy()
 
 
-def gemm_gemm_f16(a_gmk, b0_gnk, b1_gno):
+def gemm_gemm_f16(a_gmk, b0_gnk, b1_gno, instance=capi.INSTANCE_AUTO):
     G, M, K = a_gmk.shape
     N = b0_gnk.shape[1]
     O = b1_gno.shape[2]
     da, db0, db1 = dev(a_gmk), dev(b0_gnk), dev(b1_gno)
     dc = torch.full((G, M, O), float("nan"), dtype=torch.float16, device="cuda")
-    op = ck.DeviceBatchedGemmGemmF16()
+    op = ck.DeviceBatchedGemmGemmF16(instance)
     arg = op.MakeArgumentPointer(da, db0, db1, dc, M, N, K, O, G, K, K, O, O, M * K, N * K, N * O, M * O)
     assert op.IsSupportedArgument(arg), capi.last_error()
     op.MakeInvokerPointer().Run(arg, ck.StreamConfig(stream()))

@@ -127,6 +127,24 @@ def test_conv2d_config4_resnet50_layers(layer, dtype):
         _f16_close(out[:1], lit.conv2d_fwd(inp[:1], wei, s, d, p))
 
 
+@pytest.mark.parametrize("layer", RESNET)
+def test_conv2d_fp16_resnet50_layers_integer_operands_bit_exact(layer):
+    """Integers in [-3, 3] (the reference profiler's integer initialisation, narrowed so that the largest sum,
+    9 * 9 * 512, stays inside fp16): fp32 accumulation is exact in any order, so the fp16 output of the input-patch,
+    pointwise and tile kernels must equal the rounded exact sums bit for bit -- no tolerance to hide a wrong tap,
+    channel or pixel behind. Full N = 256 launch, every image checked."""
+    import gpu_util
+    C, K, f, HW, st, pd = layer
+    N = 256
+    s, d, p = (st, st), (1, 1), (pd, pd)
+    inp = uniform_int8((N, HW, HW, C), -3, 3, 510 + C).astype(np.float16)
+    wei = uniform_int8((K, f, f, C), -3, 3, 610 + K).astype(np.float16)
+    out = gpu_util.conv2d_fwd(inp, wei, s, d, p)
+    for n0 in range(0, N, 32):
+        # (the BLAS form is exact here too: integers below 2^24 in fp32)
+        np.testing.assert_array_equal(out[n0:n0 + 32], fast.conv2d_fwd_f16(inp[n0:n0 + 32], wei, s, d, p))
+
+
 def test_conv2d_unsupported_arguments_are_refused():
     import torch
     d = torch.zeros(1 << 16, dtype=torch.int8, device="cuda")

@@ -6,7 +6,8 @@ import numpy as np
 import pytest
 
 import composable_kernel_amd as ck
-from composable_kernel_amd.host_tensor import uniform_f16
+from composable_kernel_amd import capi
+from composable_kernel_amd.host_tensor import uniform_f16, uniform_int8
 from oracle import fast, lit
 
 pytestmark = pytest.mark.gpu
@@ -56,6 +57,23 @@ def test_gemm_gemm_config5():
     perm = np.random.default_rng(3).permutation(G)
     out2 = gpu_util.gemm_gemm_f16(a[perm], b0_gnk[perm], b1[perm])
     np.testing.assert_array_equal(out2.view(np.uint16), out[perm].view(np.uint16))
+
+
+@pytest.mark.parametrize("instance", [capi.INSTANCE_AUTO, 0, 1, 2])
+def test_gemm_gemm_config5_integer_operands_bit_exact(instance):
+    """Benchmark configuration 5's shape on integers in [-3, 3]: the intermediate (|sum| <= 9 * 64) is exact in fp32
+    and in its fp16 rounding, the output sums (|sum| <= 576 * 3 * 512 < 2^24) are exact in fp32 in any order, so the
+    fp16 output must equal the rounded exact product bit for bit."""
+    import gpu_util
+    G, M, N, K, O = 64, 512, 512, 64, 64
+    a = uniform_int8((G, M, K), -3, 3, 920).astype(np.float32)
+    b0_gnk = uniform_int8((G, N, K), -3, 3, 921).astype(np.float32)
+    b1 = uniform_int8((G, N, O), -3, 3, 922).astype(np.float32)
+    exact = np.matmul(np.matmul(a, b0_gnk.transpose(0, 2, 1)), b1)
+    assert np.abs(exact).max() < 60000
+    out = gpu_util.gemm_gemm_f16(a.astype(np.float16), b0_gnk.astype(np.float16), b1.astype(np.float16),
+                                 instance=instance)
+    np.testing.assert_array_equal(out, exact.astype(np.float16))
 
 
 def test_gemm_gemm_unsupported():

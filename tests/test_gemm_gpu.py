@@ -179,6 +179,21 @@ def test_fp16_gemm_config2_4096_cubed_within_tolerance():
     print("fp16 4096^3: elements outside the reference's 1e-3/1e-3 on sampled rows:", bad_strict)
 
 
+def test_fp16_gemm_4096_cubed_integer_operands_bit_exact():
+    """The reference profiler's initialisation 1 (integers in [-5, 5]) at the metric shape: every partial sum is an
+    integer below 2^24 in magnitude (|sum| <= 25 * 4096), so fp32 accumulation is exact in any order and the fp16
+    output must equal the rounded exact product bit for bit -- a full-size check that no tolerance can hide an
+    indexing mistake behind."""
+    import gpu_util
+    M = N = K = 4096
+    a = uniform_int8((M, K), -5, 5, 61).astype(np.float32)
+    b_nk = uniform_int8((N, K), -5, 5, 62).astype(np.float32)
+    exact = a @ b_nk.T                      # exact: integers below 2^24 in fp32
+    assert np.abs(exact).max() < 60000      # inside fp16's range
+    out = gpu_util.gemm_f16(a.astype(np.float16), b_nk.astype(np.float16))
+    np.testing.assert_array_equal(out, exact.astype(np.float16))
+
+
 def test_int8_gemm_4096_cubed_bit_exact():
     """Metric shape: full output against the exact fp32-BLAS form, sampled rows against the
     literal oracle."""

@@ -212,3 +212,17 @@ def test_batched_gemm_layouts(layout):
     for g in range(G):
         bad, max_err = lit.check_err_f16(out[g], refs[g], 1e-2, 1e-2)
         assert bad == 0, f"batch {g}: {bad} outside tolerance, max err {max_err}"
+
+
+@pytest.mark.parametrize("layout", sorted(LAYOUTS))
+def test_fp16_layouts_integer_operands_bit_exact_2048(layout):
+    """Integers in [-5, 5]: fp32 accumulation is exact in any order (|sum| <= 25 * 2048 < 2^24), so the fp16 output of
+    the transposing-read paths must equal the rounded exact product bit for bit."""
+    M = N = K = 2048
+    al, bl = LAYOUTS[layout]
+    a_mk = uniform_int8((M, K), -5, 5, 71).astype(np.float32)
+    b_kn = uniform_int8((K, N), -5, 5, 72).astype(np.float32)
+    a_st = (a_mk.T if al is ck.ColumnMajor else a_mk).astype(np.float16)
+    b_st = (b_kn if bl is ck.RowMajor else b_kn.T).astype(np.float16)
+    out = _run("f16", layout, np.ascontiguousarray(a_st), np.ascontiguousarray(b_st), M, N, K)
+    np.testing.assert_array_equal(out, (a_mk @ b_kn).astype(np.float16))
