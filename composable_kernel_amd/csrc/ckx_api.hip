@@ -165,6 +165,11 @@ Plan make_plan(int M, int N, int kbytes, int only_tile, long workspace_bytes, in
             const double floor_us = nst > 2 ? 0.36 : 0.42;
             iter_us        = iter_us < floor_us ? floor_us : iter_us;
             double us      = rounds * (iter_us * nk_per + 6.0 / per_cu + 2.0);
+            // a single, partly filled round of one four-stage workgroup per CU: measured fixed cost ~4 us, not 8 (M = 64,
+            // N = 11008, K = 4096 int8 on the four-stage 64 x 64 tile: 14.4 us = 3.8 + 0.33 per K tile; the 8 sent
+            // such problems to one-wave tiles at 20 us)
+            if(rounds == 1 && per_cu == 1 && nst > 2 && sp == 1)
+                us -= 4.0;
             if(sp > 1)
             {
                 // second launch + slice write/read (measured ~2 TB/s effective), and a split has to
@@ -186,9 +191,12 @@ Plan make_plan(int M, int N, int kbytes, int only_tile, long workspace_bytes, in
        ((long)M + N) * kbytes + (long)M * N <= (8l << 20))
     {
         const long t64 = (long)((M + 63) / 64) * ((N + 63) / 64);
+        // (and the two-stage instance also where the estimate picks its four-stage twin: 64 x 2048 x 2048 7.9 against
+        // 8.6 us -- the deeper pipeline pays when the operands stream from HBM, not out of L2)
+        const bool twin = kTiles[best.tile].bm == 64 && kTiles[best.tile].bn == 64 && kTiles[best.tile].lds > 2 * 128 * 128;
         for(int i = 0; i < kNumTiles; ++i)
-            if(kTiles[i].bm == 64 && kTiles[i].bn == 64 && kTiles[i].lds == 2 * 128 * 128 && t64 > 128 && t64 <= 256 &&
-               kTiles[best.tile].bm * kTiles[best.tile].bn < 64 * 64)
+            if(kTiles[i].bm == 64 && kTiles[i].bn == 64 && kTiles[i].lds == 2 * 128 * 128 &&
+               (twin || (t64 > 128 && t64 <= 256 && kTiles[best.tile].bm * kTiles[best.tile].bn < 64 * 64)))
                 best.tile = i;
     }
     return best;
