@@ -479,12 +479,19 @@ inline hipError_t gemm_gemm_launch(const void* a, const void* b0, const void* b1
     g.slabs = 0;
     g.scale = scale, g.mask_upper = mask_upper;
     if(instance < 0)
+    {
         // Many short waves (8 x 16 rows, the instance with two steps of prefetch where registers allow) are ahead on
         // short problems: G 64, 512 x 64 x 512 x 64 plain 8.5 against 10.1 us, with softmax 10.9 against 13.0. Over a
         // long N with small heads the 32-row waves read the B0 / B1 fragments half as often per row and win: G 64,
         // 4096 x 64 x 4096 x 64 plain 267 against 302 us, softmax 367 against 433 (2048: 76 / 85 and 102 / 115; at
-        // N = 1024 the plain pair ties, softmax 31.3 / 34.0).
-        instance = (K <= 64 && O <= 64 && N >= (softmax ? 1024 : 2048)) ? 0 : 2;
+        // N = 1024 plain 23.5 / 26.2, softmax 31.3 / 34.0).
+        // That needs workgroups to spare (two of them share a CU): below 256 slabs of 128 rows the 8-wave instance
+        // stays ahead with softmax (G 8, 2048 x 64 x 2048 x 64: 30.1 against 37.2 us), and without it, up to 128
+        // slabs of small heads, the 64-row instance, which doubles the workgroups (20.6 against 25.4 us).
+        const long slabs128 = (long)batch * ((M + 127) / 128);
+        const bool small_heads = K <= 64 && O <= 64;
+        instance = (!softmax && small_heads && slabs128 <= 128) ? 1 : (small_heads && N >= 1024 && slabs128 >= 256) ? 0 : 2;
+    }
     if(softmax)
         return instance == 0 ? gemm_gemm_launch_mt<2, 4, true>(g, s)
                : instance == 1 ? gemm_gemm_launch_mt<1, 4, true>(g, s)
