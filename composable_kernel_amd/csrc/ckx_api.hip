@@ -470,6 +470,13 @@ bool conv_patch_applicable(int op, const ckx_conv2d_desc* d, int epi)
            d->Wo == 56 && d->Ho >= 1 && d->N >= 1 && d->pad_left <= 2 && d->pad_top <= 2;
 }
 
+// ... and the ones it is chosen for: a workgroup owns whole images, so a small batch leaves CUs idle (N = 32: 54 us
+// against 18 us on the 256 x 64 tile instance, whose time grows with N: the curves cross near N = 100)
+bool conv_patch_preferred(int op, const ckx_conv2d_desc* d, int epi)
+{
+    return conv_patch_applicable(op, d, epi) && d->N >= 112;
+}
+
 // ---------------------------------------------------------- weight-stationary pointwise conv kernel
 const char* const kPointwiseName = "MI355X_Mfma16_Pointwise<1x1, C 256/512 bytes, K 512 per workgroup, 8 waves>";
 constexpr int kConvPatchInstance = kNumTiles, kConvPointwiseInstance = kNumTiles + 1, kNumConvInsts = kNumTiles + 2;
@@ -565,7 +572,7 @@ long conv_workspace_bytes(int op, const ckx_conv2d_desc* d, int instance)
         return 0;
     if(instance == kConvPatchInstance || instance == kConvPointwiseInstance ||
        (instance == CKX_INSTANCE_AUTO &&
-        (conv_patch_applicable(op, d, CKX_EPI_PASSTHROUGH) || conv_pointwise_preferred(op, d, CKX_EPI_PASSTHROUGH))))
+        (conv_patch_preferred(op, d, CKX_EPI_PASSTHROUGH) || conv_pointwise_preferred(op, d, CKX_EPI_PASSTHROUGH))))
         return 0;
     const Plan pl = make_plan((int)M, d->K, d->Y * d->X * d->C * es, instance, 1l << 60);
     return pl.ksplit > 1 ? (long)pl.ksplit * M * d->K * 4 : 0;
@@ -591,7 +598,7 @@ int run_conv(int op, const void* in, const void* wei, void* out, const ckx_conv2
         return fail(CKX_INVALID_VALUE, "workspace must be 16-byte aligned");
     const bool patch_aligned = !((reinterpret_cast<uintptr_t>(out) | reinterpret_cast<uintptr_t>(dops.d0) |
                                   (epi == CKX_EPI_ADD_RELU_ADD ? reinterpret_cast<uintptr_t>(dops.d1) : 0)) & 15);
-    if(instance == kConvPatchInstance || (instance == CKX_INSTANCE_AUTO && conv_patch_applicable(op, d, epi) && patch_aligned))
+    if(instance == kConvPatchInstance || (instance == CKX_INSTANCE_AUTO && conv_patch_preferred(op, d, epi) && patch_aligned))
     {
         if(!patch_aligned)
             return fail(CKX_UNSUPPORTED, "the input-patch instance needs 16-byte aligned output, bias and residual");
