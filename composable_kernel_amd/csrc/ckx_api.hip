@@ -130,7 +130,10 @@ int splitk_runs(int kbytes, int k_batch)
 
 // k_batch > 0: the caller fixed the number of K runs (DeviceGemmSplitK's KBatch)
 // kmajor: a K-major operand (A column-major / B row-major) -- only the tiles of 64 rows and more
-Plan make_plan(int M, int N, int kbytes, int only_tile, long workspace_bytes, int k_batch = 0, bool kmajor = false)
+// conv: A is gathered (im2col): the 8-wave 256 x 64 tile measures ahead of the 128 x 64 one there by 10 - 17 %
+// (ResNet-like layers at N = 32 and 256), which the GEMM-calibrated figures did not say
+Plan make_plan(int M, int N, int kbytes, int only_tile, long workspace_bytes, int k_batch = 0, bool kmajor = false,
+               bool conv = false)
 {
     Plan best;
     double best_us  = 1e30;
@@ -160,7 +163,8 @@ Plan make_plan(int M, int N, int kbytes, int only_tile, long workspace_bytes, in
             const long rounds = (units + 256l * per_cu - 1) / (256l * per_cu);
             // one K-tile iteration costs its MFMA time, but never less than the barrier + load
             // latency of the two-stage pipeline (~0.42 us measured on small tiles)
-            double iter_us = per_cu * (t.bm * t.bn / 65536.0) / t.eff * 1.1;
+            const double eff = conv && t.bm == 256 && t.bn == 64 ? t.eff * 1.1 : t.eff;
+            double iter_us   = per_cu * (t.bm * t.bn / 65536.0) / eff * 1.1;
             const int nst  = t.lds / ((t.bm + t.bn) * 128);
             const double floor_us = nst > 2 ? 0.36 : 0.42;
             iter_us        = iter_us < floor_us ? floor_us : iter_us;
@@ -168,7 +172,7 @@ Plan make_plan(int M, int N, int kbytes, int only_tile, long workspace_bytes, in
             // a single, partly filled round of one four-stage workgroup per CU: measured fixed cost ~4 us, not 8 (M = 64,
             // N = 11008, K = 4096 int8 on the four-stage 64 x 64 tile: 14.4 us = 3.8 + 0.33 per K tile; the 8 sent
             // such problems to one-wave tiles at 20 us)
-            if(rounds == 1 && per_cu == 1 && nst > 2 && sp == 1)
+            if(rounds == 1 && per_cu == 1 && sp == 1 && (nst > 2 || (conv && t.threads == 512)))
                 us -= 4.0;
             if(sp > 1)
             {
@@ -574,7 +578,7 @@ long conv_workspace_bytes(int op, const ckx_conv2d_desc* d, int instance)
        (instance == CKX_INSTANCE_AUTO &&
         (conv_patch_preferred(op, d, CKX_EPI_PASSTHROUGH) || conv_pointwise_preferred(op, d, CKX_EPI_PASSTHROUGH))))
         return 0;
-    const Plan pl = make_plan((int)M, d->K, d->Y * d->X * d->C * es, instance, 1l << 60);
+    const Plan pl = make_plan((int)M, d->K, d->Y * d->X * d->C * es, instance, 1l << 60, 0, false, true);
     return pl.ksplit > 1 ? (long)pl.ksplit * M * d->K * 4 : 0;
 }
 
@@ -640,7 +644,7 @@ int run_conv(int op, const void* in, const void* wei, void* out, const ckx_conv2
                                                   (hipStream_t)stream);
         return e == hipSuccess ? CKX_OK : hip_fail(e, kPointwiseName);
     }
-    const Plan pl = make_plan(M, N, K * es, instance, ws ? ws_bytes : 0);
+    const Plan pl = make_plan(M, N, K * es, instance, ws ? ws_bytes : 0, 0, false, true);
     const TileInstance& t = kTiles[pl.tile];
     ckx::GemmArgs g;
     std::memset(&g, 0, sizeof(g));
@@ -768,7 +772,7 @@ long convnd_workspace_bytes(int op, const ckx_convnd_desc* d, int instance)
     const long M = (long)d->N * d->out[0] * d->out[1] * d->out[2];
     if(M <= 0 || d->K <= 0)
         return 0;
-    const Plan pl = make_plan((int)M, d->K, d->filter[0] * d->filter[1] * d->filter[2] * d->C * es, instance, 1l << 60);
+    const Plan pl = make_plan((int)M, d->K, d->filter[0] * d->filter[1] * d->filter[2] * d->C * es, instance, 1l << 60, 0, false, true);
     return pl.ksplit > 1 ? (long)pl.ksplit * M * d->K * 4 : 0;
 }
 
@@ -793,7 +797,7 @@ int run_convnd(int op, const void* in, const void* wei, void* out, const ckx_con
         return fail(CKX_UNSUPPORTED, "input and weight must be 16-byte aligned");
     if(ws && (reinterpret_cast<uintptr_t>(ws) & 15))
         return fail(CKX_INVALID_VALUE, "workspace must be 16-byte aligned");
-    const Plan pl         = make_plan(M, N, K * es, instance, ws ? ws_bytes : 0);
+    const Plan pl         = make_plan(M, N, K * es, instance, ws ? ws_bytes : 0, 0, false, true);
     const TileInstance& t = kTiles[pl.tile];
     ckx::GemmArgs g;
     std::memset(&g, 0, sizeof(g));
