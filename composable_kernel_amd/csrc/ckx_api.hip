@@ -388,18 +388,22 @@ int run_gemm(int dt, const void* a, const void* b, void* c, int M, int N, int K,
     const int es = dt == ckx::DT_I8 ? 1 : 2;
     int ti = instance;
     Plan pl;
-    // 33..64 rows: the tile kernel wins when its C tiles (or C tiles x K runs) fill the machine
+    // 33..64 rows: the tile kernel wins when its C tiles fill the machine, or C tiles x K runs over a long K
+    // (64 x 4096 x 11008: 20 against 27 us; at K = 4096 the 64-row skinny instance is ahead, 11.8 against 13.0 us)
     const bool tile64 = kmajor || (M > 32 && M <= 64 &&
                                    ((N + 63) / 64 >= 160 ||
-                                    (ws && !(reinterpret_cast<uintptr_t>(ws) & 15) &&
+                                    (ws && !(reinterpret_cast<uintptr_t>(ws) & 15) && (long)K * es >= 8192 &&
                                      make_plan(M, N, K * es, -1, ws_bytes).ksplit > 1)));
     if(instance == CKX_INSTANCE_AUTO && M <= 64 && !tile64 && k_batch == 0 && batch == 1)
     {
         // (the skinny kernels read both operands K-contiguous: other layouts always take the tile kernel)
         // A handful of rows against a big weight matrix is an HBM-streaming problem. Wider
         // workgroups (32 / 64 columns) re-read A from L2 less often, as long as enough workgroups
-        // remain to keep every CU pulling on HBM; up to 8 rows A is too small to matter.
-        const int wide = M <= 8 ? 0 : (N + 63) / 64 >= 160 ? 2 : (N + 31) / 32 >= 160 ? 1 : 0;
+        // remain to keep every CU pulling on HBM; up to 4 rows A is too small to matter unless the columns are many.
+        // (measured: 8 x 11008 x 4096 11.5 against 12.4 us on the 64-column instance, 1 x 11008 x 4096 11.0 against
+        // 10.6; 1 and 8 x 16384 x 1024 5.5 against 8.7 / 9.4 us)
+        const int n64  = (N + 63) / 64;
+        const int wide = M <= 4 ? (n64 >= 256 ? 2 : 0) : n64 >= 160 ? 2 : (M > 8 && (N + 31) / 32 >= 160) ? 1 : 0;
         ti = kNumTiles + (M <= 16 ? (wide == 2 ? 4 : wide == 1 ? 5 : 0) : M <= 32 ? (wide == 2 ? 6 : wide == 1 ? 7 : 1) : 2);
     }
     else if(instance < kNumTiles)
