@@ -166,7 +166,7 @@ Plan make_plan(int M, int N, int kbytes, int only_tile, long workspace_bytes, in
             const double eff = conv && t.bm == 256 && t.bn == 64 ? t.eff * 1.1 : t.eff;
             double iter_us   = per_cu * (t.bm * t.bn / 65536.0) / eff * 1.1;
             const int nst  = t.lds / ((t.bm + t.bn) * 128);
-            const double floor_us = nst > 2 ? 0.36 : 0.42;
+            const double floor_us = nst > 2 ? 0.30 : 0.42; // (four stages: 0.33 measured over 32 K tiles, 0.26 over 64)
             iter_us        = iter_us < floor_us ? floor_us : iter_us;
             double us      = rounds * (iter_us * nk_per + 6.0 / per_cu + 2.0);
             // a single, partly filled round of one four-stage workgroup per CU: measured fixed cost ~4 us, not 8 (M = 64,
@@ -323,7 +323,9 @@ int check_gemm_shape(int dt, int M, int N, int K, int sa, int sb, int sc, int al
 long gemm_workspace_bytes(int dt, int M, int N, int K, int instance)
 {
     const int es = dt == ckx::DT_I8 ? 1 : 2;
-    if(M <= 0 || N <= 0 || (instance == CKX_INSTANCE_AUTO && M <= 32) || instance >= kNumTiles)
+    // (up to 32 rows go to the skinny kernels, which take none -- except few columns under a long K: see run_gemm)
+    const bool few_cols = M >= 8 && (N + 15) / 16 < (M > 16 ? 257 : 128) && (long)K * es >= 16384;
+    if(M <= 0 || N <= 0 || (instance == CKX_INSTANCE_AUTO && M <= 32 && !few_cols) || instance >= kNumTiles)
         return 0;
     const Plan pl = make_plan(M, N, K * es, instance, 1l << 60);
     return pl.ksplit > 1 ? (long)pl.ksplit * M * N * 4 : 0;
@@ -394,7 +396,12 @@ int run_gemm(int dt, const void* a, const void* b, void* c, int M, int N, int K,
                                    ((N + 63) / 64 >= 160 ||
                                     (ws && !(reinterpret_cast<uintptr_t>(ws) & 15) && (long)K * es >= 8192 &&
                                      make_plan(M, N, K * es, -1, ws_bytes).ksplit > 1)));
-    if(instance == CKX_INSTANCE_AUTO && M <= 64 && !tile64 && k_batch == 0 && batch == 1)
+    // few columns and a long K: the skinny kernels have N / 16 workgroups with all of K each, the tile kernel can cut K
+    // over the CUs (fp16 32 x 1024 x 8192: 12.4 against 23.3 us, 16 rows 12.1 against 16.2, 8 rows 11.7 against 13.4)
+    // (17 rows and more: up to 4096 columns -- fp16 32 x 4096 x 11008 24.6 against 31.9 us)
+    const bool few_cols = !kmajor && M >= 8 && M <= 64 && (N + 15) / 16 < (M > 16 ? 257 : 128) && (long)K * es >= 16384 && ws &&
+                          !(reinterpret_cast<uintptr_t>(ws) & 15) && make_plan(M, N, K * es, -1, ws_bytes).ksplit > 1;
+    if(instance == CKX_INSTANCE_AUTO && M <= 64 && !tile64 && !few_cols && k_batch == 0 && batch == 1)
     {
         // (the skinny kernels read both operands K-contiguous: other layouts always take the tile kernel)
         // A handful of rows against a big weight matrix is an HBM-streaming problem. Wider
