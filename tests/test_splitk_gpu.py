@@ -123,7 +123,11 @@ def test_conv2d_split_k(force_split, dtype):
 
 
 @pytest.mark.parametrize("shape", [(8, 10300, 256), (9, 10300, 256), (16, 5200, 192), (16, 1000, 320), (17, 10300, 128),
-                                   (32, 5200, 256), (33, 10300, 128), (48, 700, 4096), (64, 10304, 192), (65, 700, 2048)])
+                                   (32, 5200, 256), (33, 10300, 128), (48, 700, 4096), (64, 10304, 192), (65, 700, 2048),
+                                   # few columns under a long K (tile kernel with a K split when the workspace is there),
+                                   # many columns under up to 4 rows (wide skinny instance), 33..64 rows at K = 4096
+                                   (8, 1024, 8192), (16, 528, 16384), (32, 2048, 8192), (24, 4096, 8208), (4, 16384, 1024),
+                                   (1, 16400, 512), (48, 4096, 4096), (64, 2048, 8192)])
 def test_auto_instance_few_rows_routing_bit_exact(shape):
     """Automatic choice for few-row problems: narrow / wide skinny instances up to 32 rows, skinny or
     tile kernel (with a K split when the workspace is there) up to 64 rows. Every route must give
