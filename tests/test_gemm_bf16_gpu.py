@@ -73,6 +73,18 @@ def test_bf16_gemm_full_size_and_split_k(monkeypatch):
     _close(_gemm(a, b_nk, workspace=True), ref)
 
 
+def test_bf16_gemm_4096_cubed_integer_operands_bit_exact():
+    """Integers in [-5, 5] at the metric shape: fp32 accumulation is exact in any order (|sum| <= 25 * 4096 < 2^24), so
+    the bf16 output must be the round-to-nearest-even of the exact product, bit for bit."""
+    from composable_kernel_amd.host_tensor import uniform_int8
+    M = N = K = 4096
+    a = uniform_int8((M, K), -5, 5, 41).astype(np.float32)
+    b_nk = uniform_int8((N, K), -5, 5, 42).astype(np.float32)
+    exact = a @ b_nk.T
+    out = _gemm(fast.f32_to_bf16(a), fast.f32_to_bf16(b_nk))
+    np.testing.assert_array_equal(out, fast.f32_to_bf16(exact))
+
+
 def test_bf16_gemm_has_no_fused_epilogue():
     op = ck.DeviceGemmBF16()
     arg = op.MakeArgumentPointer(0, 0, 0, 64, 64, 64, 64, 64, 64, None, None, ck.RequantReluRequant(1, 1))
