@@ -9,13 +9,20 @@ metric (TFLOP/s and fraction of the dense fp16 MFMA peak) is quoted; the int8 ha
 (4096^3 requant GEMM, TOP/s) and every other config are measured too and attached under "also".
 Prints ONE JSON line on stdout.
 
-Timing: W untimed launches, then exactly K launches between two events recorded on the launch
-stream (torch's current stream, whose handle is what the C ABI receives), bracketed by device
-synchronisation; wall-clock over the same region gives ms_per_step. The K launches are replayed
-from a HIP graph captured from the same C-ABI calls, so that the GPU runs them back to back
-even for kernels shorter than a Python call (--no-graph launches eagerly). The defaults
-(K = 1000, W = 300) are long enough for the part to reach its operating clocks: the first few
-milliseconds after idle run several hundred MHz lower.
+Timing: a clock-settling phase, W untimed launches, then exactly K launches between two events
+recorded on the launch stream (torch's current stream, whose handle is what the C ABI receives),
+bracketed by device synchronisation; wall-clock over the same region gives ms_per_step. The K
+launches are replayed from a HIP graph captured from the same C-ABI calls, so that the GPU runs
+them back to back even for kernels shorter than a Python call (--no-graph launches eagerly).
+
+Clock settling: a GPU that was idle runs its first launches several hundred MHz below its
+operating point and takes tens of milliseconds of load to leave that state, so a short run
+(--steps 20 --warmup 5) would time the ramp, not the kernel. Before the W warm-up launches the
+same kernel is therefore replayed, untimed, in blocks until the mean launch time of a block stops
+changing (and at least --settle-ms of load have passed); the line discloses it ("settle_launches",
+"settle_ms") and also carries the figure WITHOUT it under "from_idle": 1 warm-up + 10 timed
+launches from the idle GPU, the reference's own timing protocol
+(include/ck/device_utility/kernel_launch.hpp:20-62).
 """
 import argparse
 import json
@@ -33,6 +40,8 @@ HBM_PEAK_GBS = 8000.0
 # Bytes crossing the L2 <-> fabric boundary per launch, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
 # scaled by a 256 MiB copy in the same run (profiles/gemm_tile_fp16_int8_4096_hbm_traffic.md).
 MEASURED_TRAFFIC = {"fp16_gemm_4096": 2.350e8, "int8_requant_gemm_4096": 1.178e8}
+TRAFFIC_SOURCE = ("cited, not measured in this run: profiles/gemm_tile_fp16_int8_4096_hbm_traffic.md "
+                  "(rocprofv3 --pmc FETCH_SIZE, then WRITE_SIZE, each scaled by a 256 MiB copy in the same run)")
 
 
 def _conv_workload(name, dtype, C, K, f, HW, st, pd, N=256, fused=None):
@@ -224,26 +233,76 @@ def make_launcher(w, instance=-1, rotate=1):
     return launch
 
 
-def time_workload(w, steps, warmup, instance=-1, use_graph=True, rotate=1):
-    """W untimed launches, then exactly K timed ones. The K launches are replayed from a HIP
-    graph (captured once from the same C-ABI calls) so that kernels run back to back on the GPU
-    even when one kernel is shorter than a Python call; use_graph=False launches eagerly."""
+def _figures(w, ev_ms):
+    tput = w["ops"] / (ev_ms * 1e-3) / 1e12
+    gbs = w["bytes"] / (ev_ms * 1e-3) / 1e9
+    compute_frac = tput / PEAK[w["dtype"]]
+    hbm_frac = gbs / HBM_PEAK_GBS
+    return dict(tput=tput, gbs=gbs, mfma_frac=compute_frac, hbm_frac=hbm_frac,
+                bound="mfma" if compute_frac >= hbm_frac else "hbm")
+
+
+def time_workload(w, steps, warmup, instance=-1, use_graph=True, rotate=1, settle_ms=300.0, from_idle=False):
+    """[from_idle: 1 + 10 eager launches first], clock settling, W untimed launches, then exactly K timed
+    ones. The K launches are replayed from a HIP graph (captured once from the same C-ABI calls) so that
+    kernels run back to back on the GPU even when one kernel is shorter than a Python call;
+    use_graph=False launches eagerly."""
     import torch
     launch = make_launcher(w, instance, rotate)
-    for _ in range(warmup):
-        launch()
     torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    idle = None
+    if from_idle:
+        # the reference's protocol (kernel_launch.hpp:20-62): one warm-up launch, a device
+        # synchronisation, ten launches between two events, the mean
+        launch()
+        torch.cuda.synchronize()
+        e0.record()
+        for _ in range(10):
+            launch()
+        e1.record()
+        torch.cuda.synchronize()
+        idle = e0.elapsed_time(e1) / 10
     # launches per captured graph: a divisor of K that walks the rotation a whole number of times
     cands = [d for d in range(1, min(steps, 50) + 1) if steps % d == 0 and d % rotate == 0]
     per_graph = max(cands) if cands else rotate
     graph = None
     if use_graph:
+        launch()   # (the library's one-time function attributes are set outside the capture)
+        torch.cuda.synchronize()
         graph = torch.cuda.CUDAGraph()
         with torch.cuda.graph(graph):
             for _ in range(per_graph):
                 launch()
-        graph.replay()   # one untimed replay
-    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+
+    def chunk():
+        if graph is not None:
+            graph.replay()
+        else:
+            for _ in range(per_graph):
+                launch()
+
+    # ---- clock settling: blocks of launches until a block's mean time stops moving ----------
+    settle_launches, settle_total, blocks = 0, 0.0, []
+    if settle_ms > 0:
+        est = None
+        while settle_total < 4000.0:
+            n_chunks = 4 if est is None else max(4, min(400, int(25.0 / max(est * per_graph, 1e-3))))  # ~25 ms blocks
+            e0.record()
+            for _ in range(n_chunks):
+                chunk()
+            e1.record()
+            torch.cuda.synchronize()
+            ms = e0.elapsed_time(e1)
+            est = ms / (n_chunks * per_graph)
+            settle_launches += n_chunks * per_graph
+            settle_total += ms
+            blocks.append(est)
+            if settle_total >= settle_ms and len(blocks) >= 3 and abs(blocks[-1] - blocks[-2]) <= 0.01 * blocks[-2] \
+                    and abs(blocks[-1] - blocks[-3]) <= 0.015 * blocks[-3]:
+                break
+    for _ in range(warmup):
+        launch()
     torch.cuda.synchronize()
     t0 = time.perf_counter()
     e0.record()
@@ -257,21 +316,45 @@ def time_workload(w, steps, warmup, instance=-1, use_graph=True, rotate=1):
     torch.cuda.synchronize()
     wall_ms = (time.perf_counter() - t0) * 1e3 / steps
     ev_ms = e0.elapsed_time(e1) / steps
-    tput = w["ops"] / (ev_ms * 1e-3) / 1e12
-    gbs = w["bytes"] / (ev_ms * 1e-3) / 1e9
-    compute_frac = tput / PEAK[w["dtype"]]
-    hbm_frac = gbs / HBM_PEAK_GBS
-    bound = "mfma" if compute_frac >= hbm_frac else "hbm"
-    return dict(workload=w["name"], dtype=w["dtype"], ms=ev_ms, wall_ms=wall_ms, tput=tput, gbs=gbs,
-                mfma_frac=compute_frac, hbm_frac=hbm_frac, bound=bound)
+    out = dict(workload=w["name"], dtype=w["dtype"], ms=ev_ms, wall_ms=wall_ms, settle_launches=settle_launches,
+               settle_ms=settle_total, settle_blocks_us=[round(b * 1e3, 1) for b in blocks], **_figures(w, ev_ms))
+    if idle is not None:
+        out["from_idle_ms"] = idle
+    return out
 
 
-def cpu_baseline(w, target_seconds=12.0):
-    """The oracle's literal ReferenceGemm restatement on a bounded row sample of the same
-    workload, on the host cores of this box."""
+def _cpu_model():
+    try:
+        with open("/proc/cpuinfo") as f:
+            for line in f:
+                if line.startswith("model name"):
+                    return line.split(":", 1)[1].strip()
+    except OSError:
+        pass
+    return "unknown"
+
+
+def cpu_threads():
+    """Threads of the CPU leg: the cores this process may run on -- its affinity mask, and where the host
+    is shared (a GPU box grants each GPU's job a share of the cores and says so in OMP_NUM_THREADS) that share.
+    The reference's host operators use std::thread::hardware_concurrency() threads (reference_gemm.hpp:83-85,
+    host_tensor.hpp:174-193), which is the same number on a host that is one's own."""
+    try:
+        n = len(os.sched_getaffinity(0))
+    except AttributeError:
+        n = os.cpu_count() or 1
+    share = os.environ.get("OMP_NUM_THREADS", "")
+    if share.isdigit() and int(share) > 0:
+        n = min(n, int(share))
+    return max(1, n)
+
+
+def cpu_baseline(w, threads=None, budget_seconds=30.0):
+    """The oracle's literal ReferenceGemm restatement on the host cores of this box: the WHOLE problem when a
+    probe says it fits the time budget, else a bounded row sample of it (stated in "sample")."""
     from oracle import lit
     from composable_kernel_amd.host_tensor import uniform_f16, uniform_int8
-    threads = max(1, min(16, os.cpu_count() or 1))
+    threads = threads or cpu_threads()
     N, K = w["N"], w["K"]
     if w["dtype"] == "f16":
         b = uniform_f16((N, K), -1, 1, 2)
@@ -281,19 +364,21 @@ def cpu_baseline(w, target_seconds=12.0):
         b = uniform_int8((N, K), -5, 5, 2)
         mk = lambda m: uniform_int8((m, K), -5, 5, 1)
         run = lambda a: lit.gemm_i8(a, b.T, lit.EPI_REQUANT_RND, 0.5, 0.03, nthreads=threads)
-    m0 = 2 * threads
+    m0 = min(w["M"], 2 * threads)
     t0 = time.perf_counter()
     run(mk(m0))
     dt = max(time.perf_counter() - t0, 1e-4)
-    rows = int(min(w["M"], max(m0, m0 * target_seconds / dt)))
+    rows = int(min(w["M"], max(m0, m0 * budget_seconds / dt)))
     a = mk(rows)
     t0 = time.perf_counter()
     run(a)
     dt = time.perf_counter() - t0
     unit = "TFLOP/s" if w["dtype"] == "f16" else "TOP/s"
+    what = "the whole" if rows == w["M"] else f"{rows} of {w['M']} rows of the same"
     return {"value": 2.0 * rows * N * K / dt / 1e12, "unit": unit, "cores": threads, "kind": "port",
-            "sample": f"{rows} of {w['M']} rows of the same {w['M']}x{N}x{K} problem, literal ReferenceGemm "
-                      f"restatement (oracle/ck_oracle.cpp), {dt:.1f} s"}
+            "host_cores": os.cpu_count(), "cpu_model": _cpu_model(),
+            "sample": f"{what} {w['M']}x{N}x{K} problem, literal ReferenceGemm restatement "
+                      f"(oracle/ck_oracle.cpp), {threads} threads, {dt:.1f} s"}
 
 
 def main():
@@ -305,7 +390,10 @@ def main():
     ap.add_argument("--instance", type=int, default=-1)
     ap.add_argument("--all", action="store_true", help="also time every other config (reported under 'also')")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--cpu-threads", type=int, default=0, help="threads of the CPU baseline (default: this job's share of the host)")
     ap.add_argument("--no-graph", action="store_true", help="launch eagerly instead of replaying a HIP graph")
+    ap.add_argument("--settle-ms", type=float, default=300.0,
+                    help="least duration of the untimed clock-settling phase before the warm-up launches (0: none)")
     ap.add_argument("--copy-probe", action="store_true",
                     help="also run one 256 MiB device-to-device copy (a kernel of known traffic, used to "
                          "scale the FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run)")
@@ -328,7 +416,8 @@ def main():
         dst.copy_(src)
         torch.cuda.synchronize()
     w = WORKLOADS[args.workload]
-    r = time_workload(w, args.steps, args.warmup, args.instance, not args.no_graph)
+    r = time_workload(w, args.steps, args.warmup, args.instance, not args.no_graph, settle_ms=args.settle_ms,
+                      from_idle=True)
     also = []
     extra = ["int8_requant_gemm_4096"] if args.workload == "fp16_gemm_4096" else []
     if args.all:
@@ -336,39 +425,51 @@ def main():
     for n in extra:
         wl = WORKLOADS[n]
         k_steps, k_warm = max(16, args.steps // 2), max(3, args.warmup // 2)
-        x = time_workload(wl, k_steps, k_warm, -1, not args.no_graph)
+        x = time_workload(wl, k_steps, k_warm, -1, not args.no_graph, settle_ms=args.settle_ms / 2)
         row = {"workload": n, "dtype": x["dtype"], "ms": round(x["ms"], 5),
                "value": round(x["tput"], 2), "unit": "TOP/s" if x["dtype"] == "i8" else "TFLOP/s",
                "GB/s": round(x["gbs"], 1), "bound": x["bound"],
-               "frac_of_bound": round(max(x["mfma_frac"], x["hbm_frac"]), 4)}
+               "frac_of_bound": round(max(x["mfma_frac"], x["hbm_frac"]), 4),
+               "settle_launches": x["settle_launches"], "settle_ms": round(x["settle_ms"], 1)}
         if wl["kind"] == "gemm" and x["bound"] == "hbm" and wl["bytes"] < 128e6:
             # the weight matrix fits the Infinity Cache: also time it cold, 8 copies in turn
-            cold = time_workload(wl, k_steps - k_steps % 8, k_warm, -1, not args.no_graph, rotate=8)
+            cold = time_workload(wl, k_steps - k_steps % 8, k_warm, -1, not args.no_graph, rotate=8,
+                                 settle_ms=args.settle_ms / 2)
             row.update({"cold_ms": round(cold["ms"], 5), "cold_GB/s": round(cold["gbs"], 1),
                         "cold_frac_of_bound": round(cold["hbm_frac"], 4)})
         also.append(row)
 
-    unit = "TFLOP/s" if w["dtype"] == "f16" else "TOP/s"
+    unit = "TOP/s" if w["dtype"] == "i8" else "TFLOP/s"
+    traffic = MEASURED_TRAFFIC.get(w["name"]) if args.instance < 0 else None
     if r["bound"] == "mfma":
         roof = {"bound": "mfma", "achieved": round(r["tput"], 2), "peak": PEAK[w["dtype"]], "unit": unit,
-                "frac": round(r["mfma_frac"], 4), "traffic": MEASURED_TRAFFIC.get(w["name"])}
+                "frac": round(r["mfma_frac"], 4), "traffic": traffic}
     else:
         roof = {"bound": "hbm", "achieved": round(r["gbs"], 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                "frac": round(r["hbm_frac"], 4), "traffic": MEASURED_TRAFFIC.get(w["name"])}
+                "frac": round(r["hbm_frac"], 4), "traffic": traffic}
+    roof["traffic_source"] = TRAFFIC_SOURCE if traffic is not None else None
+    idle = _figures(w, r["from_idle_ms"])
     line = {
         "metric": "int8 TOPS & fp16 TFLOPS at 4096^3 on 1 MI355X; % of dtype MFMA peak",
         "value": round(r["tput"], 2), "unit": unit, "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(r["wall_ms"], 5), "higher_is_better": True, "scaling": "weak",
-        "vs_baseline": None, "dtype": "f16" if w["dtype"] == "f16" else "i8", "data": "synthetic",
+        "vs_baseline": None, "dtype": w["dtype"], "data": "synthetic",
         "config": {"workload": w["name"], "layout": "A row-major, B column-major, C row-major",
-                   "accumulate": "fp32" if w["dtype"] == "f16" else "int32",
+                   "accumulate": "int32" if w["dtype"] == "i8" else "fp32",
                    "ops_per_step": w["ops"], "algorithmic_bytes_per_step": w["bytes"]},
         "roofline": roof,
         "kernel_ms": round(r["ms"], 5),
+        # untimed launches of the same kernel before the warm-up launches, until the GPU has left its idle clocks
+        "settle_launches": r["settle_launches"], "settle_ms": round(r["settle_ms"], 1),
+        "settle_blocks_us": r["settle_blocks_us"][:12],
+        "from_idle": {"protocol": "1 warm-up + 10 timed launches from the idle GPU, no settling "
+                                  "(the reference's launch_and_time_kernel)",
+                      "kernel_ms": round(r["from_idle_ms"], 5), "value": round(idle["tput"], 2), "unit": unit,
+                      "frac": round(max(idle["mfma_frac"], idle["hbm_frac"]), 4)},
         "also": also,
     }
     if not args.no_cpu:
-        line["cpu_baseline"] = cpu_baseline(w)
+        line["cpu_baseline"] = cpu_baseline(w, args.cpu_threads or None)
     print(json.dumps(line))
 
 
