@@ -18,6 +18,7 @@ EPI_ADD_RELU, EPI_ADD_RELU_ADD, EPI_CSHUFFLE_ADD_RELU = 3, 4, 5
 (OP_GEMM_I8, OP_GEMM_F16, OP_CONV2D_FWD_I8, OP_CONV2D_FWD_F16, OP_BATCHED_GEMM_GEMM, OP_GEMM_SPLITK, OP_GEMM_BF16,
  OP_BATCHED_GEMM_SOFTMAX_GEMM) = range(8)
 INSTANCE_AUTO = -1
+STATIC_WORKSPACE_BYTES = 32 * 1024 * 1024   # CKX_STATIC_WORKSPACE_BYTES
 
 # every symbol include/ckx.h declares
 SYMBOLS = [
@@ -26,7 +27,7 @@ SYMBOLS = [
     "ckx_gemm_f16_is_supported", "ckx_gemm_f16", "ckx_gemm_f16_workspace_bytes",
     "ckx_gemm_bf16_is_supported", "ckx_gemm_bf16", "ckx_gemm_bf16_workspace_bytes",
     "ckx_batched_gemm_is_supported", "ckx_batched_gemm_i8", "ckx_batched_gemm_f16",
-    "ckx_gemm_splitk_workspace_bytes", "ckx_gemm_i8_splitk", "ckx_gemm_f16_splitk",
+    "ckx_gemm_splitk_workspace_bytes", "ckx_gemm_i8_splitk", "ckx_gemm_f16_splitk", "ckx_gemm_i8_splitk_noalloc",
     "ckx_gemm_f16_multiple_d_is_supported", "ckx_gemm_f16_multiple_d", "ckx_conv2d_fwd_bias_activation_f16",
     "ckx_conv2d_fwd_is_supported", "ckx_conv2d_fwd_i8", "ckx_conv2d_fwd_f16", "ckx_conv2d_fwd_workspace_bytes",
     "ckx_convnd_fwd_is_supported", "ckx_convnd_fwd", "ckx_convnd_fwd_workspace_bytes",
@@ -106,6 +107,7 @@ def lib():
     L.ckx_gemm_splitk_workspace_bytes.argtypes = [C.c_int, i32, i32, i32, i32]
     L.ckx_gemm_i8_splitk.argtypes = [vp, vp, vp] + shape + [C.c_int, f32, f32, C.c_int, i32, vp, i64, vp]
     L.ckx_gemm_f16_splitk.argtypes = [vp, vp, vp] + shape + [C.c_int, i32, vp, i64, vp]
+    L.ckx_gemm_i8_splitk_noalloc.argtypes = [vp, vp, vp] + shape + [C.c_int, f32, f32, C.c_int, i32, vp]
     md = [i32] * 8 + [C.c_int] * 3
     L.ckx_gemm_f16_multiple_d_is_supported.argtypes = md + [C.c_int, C.c_int]
     L.ckx_gemm_f16_multiple_d.argtypes = [vp] * 5 + md + [C.c_int, C.c_int, vp, i64, vp]

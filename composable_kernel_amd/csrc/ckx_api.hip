@@ -17,6 +17,12 @@
 #include "conv_pointwise.hpp"
 #include "gemm_skinny.hpp"
 
+// Workspace of ckx_gemm_i8_splitk_noalloc: device memory that belongs to the library, one copy per GPU,
+// held from the time the code object is loaded on that GPU until the process ends. In host code the name
+// below is only a handle for hipGetSymbolAddress -- it is not a device address; kernels get the pointer
+// that static_workspace() returns.
+static __device__ __align__(256) unsigned char scratch[CKX_STATIC_WORKSPACE_BYTES];
+
 namespace {
 
 thread_local std::string g_last_error;
@@ -30,6 +36,32 @@ int fail(int code, const std::string& msg)
 int hip_fail(hipError_t e, const char* what)
 {
     return fail(CKX_HIP_ERROR, std::string(what) + ": " + hipGetErrorString(e));
+}
+
+// Device address of `scratch` on the current GPU, looked up once per device (every GPU has its own copy of
+// the array at its own address). No allocation: hipGetSymbolAddress only resolves the loaded symbol.
+int static_workspace(void** out)
+{
+    constexpr int kMaxDevices = 64;
+    static std::mutex mu;
+    static void* ptrs[kMaxDevices] = {};
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if(e != hipSuccess)
+        return hip_fail(e, "hipGetDevice");
+    if(dev < 0 || dev >= kMaxDevices)
+        return fail(CKX_UNSUPPORTED, "device ordinal beyond the static workspace table");
+    std::lock_guard<std::mutex> lock(mu);
+    if(!ptrs[dev])
+    {
+        void* p = nullptr;
+        e       = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        if(e != hipSuccess || !p)
+            return hip_fail(e, "hipGetSymbolAddress(static workspace)");
+        ptrs[dev] = p;
+    }
+    *out = ptrs[dev];
+    return CKX_OK;
 }
 
 // int8 outputs at least this large are stored non-temporally (measured on the N256 C256->K512
@@ -938,6 +970,25 @@ int ckx_gemm_i8_splitk(const void* a, const void* b, void* c, int32_t M, int32_t
         return fail(CKX_INVALID_VALUE, "KBatch must be at least 1");
     return run_gemm(ckx::DT_I8, a, b, c, M, N, K, sa, sb, sc, al, bl, cl, epilogue, scale_gemm, scale_relu,
                     instance, workspace, workspace_bytes, stream, DOperands{}, k_batch);
+}
+
+int ckx_gemm_i8_splitk_noalloc(const void* a, const void* b, void* c, int32_t M, int32_t N, int32_t K, int32_t sa,
+                               int32_t sb, int32_t sc, int al, int bl, int cl, int epilogue, float scale_gemm,
+                               float scale_relu, int instance, int32_t k_batch, void* stream)
+{
+    if(k_batch < 1)
+        return fail(CKX_INVALID_VALUE, "KBatch must be at least 1");
+    const int64_t need = ckx_gemm_splitk_workspace_bytes(CKX_OP_GEMM_I8, M, N, K, k_batch);
+    if(need > (int64_t)CKX_STATIC_WORKSPACE_BYTES)
+        return fail(CKX_UNSUPPORTED, "this split needs " + std::to_string(need) +
+                                         " bytes of workspace, the library's static workspace holds " +
+                                         std::to_string((long)CKX_STATIC_WORKSPACE_BYTES) +
+                                         ": use ckx_gemm_i8_splitk with a workspace of the caller's");
+    void* ws = nullptr;
+    if(int st = static_workspace(&ws))
+        return st;
+    return run_gemm(ckx::DT_I8, a, b, c, M, N, K, sa, sb, sc, al, bl, cl, epilogue, scale_gemm, scale_relu,
+                    instance, ws, (long)CKX_STATIC_WORKSPACE_BYTES, stream, DOperands{}, k_batch);
 }
 
 int ckx_gemm_f16_splitk(const void* a, const void* b, void* c, int32_t M, int32_t N, int32_t K, int32_t sa,

@@ -178,6 +178,23 @@ int ckx_gemm_f16_splitk(const void* p_a, const void* p_b, void* p_c, int32_t M, 
                         int c_layout, int instance, int32_t k_batch, void* p_workspace, int64_t workspace_bytes,
                         void* stream);
 
+/* ---- int8 split-K GEMM for callers that cannot allocate ----------------------
+ * No counterpart in the reference. For callers that cannot call hipMalloc (code under HIP graph capture,
+ * tight serving loops, harnesses that forbid it): ckx_gemm_i8_splitk with the workspace taken from a
+ * static device array of the library instead of an argument -- CKX_STATIC_WORKSPACE_BYTES per GPU, held
+ * from the load of the library's code object on that GPU until the process ends. The call allocates and
+ * frees nothing and synchronises nothing. A split that needs more than CKX_STATIC_WORKSPACE_BYTES
+ * (ckx_gemm_splitk_workspace_bytes(CKX_OP_GEMM_I8, M, N, K, k_batch)) is refused with CKX_UNSUPPORTED.
+ * Every call on one GPU uses the same array: calls that may run at the same time on one GPU (different
+ * streams, or graphs replayed concurrently) race on it and must be serialised by the caller. The array needs no
+ * initialisation (every slice element that is read was written by the same call). The first call on a GPU
+ * looks the array's address up (hipGetSymbolAddress): make it outside a stream capture. */
+#define CKX_STATIC_WORKSPACE_BYTES (32 * 1024 * 1024)
+int ckx_gemm_i8_splitk_noalloc(const void* p_a, const void* p_b, void* p_c, int32_t M, int32_t N, int32_t K,
+                               int32_t stride_a, int32_t stride_b, int32_t stride_c, int a_layout, int b_layout,
+                               int c_layout, int epilogue, float scale_gemm, float scale_relu, int instance,
+                               int32_t k_batch, void* stream);
+
 /* ---- fp16 GEMM with fused D operands:  E = cde_op(A * B, D0 [, D1]) ----------
  * Replaces DeviceGemmMultipleD<..., Tuple<half_t[, half_t]>, half_t, PassThrough, PassThrough, CDEOp>
  * ::MakeArgumentPointer + Run (device_gemm_multiple_d.hpp:14-55) for cde_op in
