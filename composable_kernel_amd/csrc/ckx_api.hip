@@ -16,6 +16,7 @@
 #include "conv_patch.hpp"
 #include "conv_pointwise.hpp"
 #include "gemm_skinny.hpp"
+#include "gemm_generic.hpp"
 
 // Workspace of ckx_gemm_i8_splitk_noalloc: device memory that belongs to the library, one copy per GPU,
 // held from the time the code object is loaded on that GPU until the process ends. In host code the name
@@ -271,7 +272,11 @@ const SkinnyInstance kSkinny[] = {
     CKX_SKINNY(2, 8, 2, 2),
 };
 constexpr int kNumSkinny    = sizeof(kSkinny) / sizeof(kSkinny[0]);
-constexpr int kNumGemmInsts = kNumTiles + kNumSkinny;
+// the element-granular instance (gemm_generic.hpp) closes every GEMM and conv instance list: any extent, leading
+// dimension, channel count and base address, all four GEMM layouts, every epilogue of the data type
+constexpr int kGenericGemmInstance = kNumTiles + kNumSkinny;
+constexpr int kNumGemmInsts        = kNumTiles + kNumSkinny + 1;
+const char* const kGenericName     = "MI355X_Mfma16_Generic<64, 64, one k-step, waves 2x2, element-wise loads>";
 
 const char* family_prefix(int op)
 {
@@ -316,6 +321,15 @@ int check_d_operands(int epi, int N, const DOperands& d)
     return CKX_OK;
 }
 
+// Problems outside the vectorised instances' reach: a contiguous extent or a leading dimension of A or B that is not
+// a whole 16-byte vector (the reference's KPadding / MNKPadding territory), D-operand epilogues on K-major operands
+bool gemm_needs_generic(int dt, int M, int N, int K, int sa, int sb, bool ta, bool tb, int epi)
+{
+    const int es = dt == ckx::DT_I8 ? 1 : 2;
+    return ((long)(ta ? M : K) * es) % 16 || ((long)(tb ? N : K) * es) % 16 || ((long)sa * es) % 16 ||
+           ((long)sb * es) % 16 || ((ta || tb) && epi >= CKX_EPI_ADD_RELU);
+}
+
 int check_gemm_shape(int dt, int M, int N, int K, int sa, int sb, int sc, int al, int bl, int cl, int epi,
                      int instance)
 {
@@ -324,7 +338,7 @@ int check_gemm_shape(int dt, int M, int N, int K, int sa, int sb, int sc, int al
         return fail(CKX_INVALID_VALUE, "negative GEMM dimension");
     if(instance != CKX_INSTANCE_AUTO && (instance < 0 || instance >= kNumGemmInsts))
         return fail(CKX_INVALID_VALUE, "no such instance");
-    if(instance >= kNumTiles && M > kSkinny[instance - kNumTiles].max_m)
+    if(instance >= kNumTiles && instance < kGenericGemmInstance && M > kSkinny[instance - kNumTiles].max_m)
         return fail(CKX_UNSUPPORTED, "this skinny instance covers fewer rows than M");
     if(epi < CKX_EPI_PASSTHROUGH || epi > CKX_EPI_CSHUFFLE_ADD_RELU)
         return fail(CKX_INVALID_VALUE, "unknown epilogue");
@@ -336,15 +350,17 @@ int check_gemm_shape(int dt, int M, int N, int K, int sa, int sb, int sc, int al
         return fail(CKX_UNSUPPORTED, "C is row-major in every instance (as in the reference's instance lists)");
     // K-major operands: A column-major (element (m,k) at k*sa + m), B row-major ((k,n) at k*sb + n)
     const bool ta = al == CKX_COL_MAJOR, tb = bl == CKX_ROW_MAJOR;
-    if((ta || tb) && epi >= CKX_EPI_ADD_RELU)
-        return fail(CKX_UNSUPPORTED, "the D-operand epilogues are built for A row-major, B column-major");
-    if((ta || tb) && instance != CKX_INSTANCE_AUTO && !ckx::layout_tile(dt, instance, ta, tb))
+    // what only the element-granular instance takes (AUTO sends it there)
+    const bool fast = instance != CKX_INSTANCE_AUTO && instance != kGenericGemmInstance;
+    if(fast && (ta || tb) && epi >= CKX_EPI_ADD_RELU)
+        return fail(CKX_UNSUPPORTED, "the D-operand epilogues of this instance are built for A row-major, B column-major");
+    if(fast && (ta || tb) && !ckx::layout_tile(dt, instance, ta, tb))
         return fail(CKX_UNSUPPORTED, "this instance has no variant for a K-major operand (tiles of 64 rows and more do)");
     if(sa < (ta ? M : K) || sb < (tb ? N : K) || sc < N)
         return fail(CKX_UNSUPPORTED, "stride smaller than the contiguous extent");
-    if(((long)(ta ? M : K) * es) % 16 || ((long)(tb ? N : K) * es) % 16 || ((long)sa * es) % 16 ||
-       ((long)sb * es) % 16)
-        return fail(CKX_UNSUPPORTED, "the contiguous extents of A and B and their strides must be multiples of 16 bytes");
+    if(fast && gemm_needs_generic(dt, M, N, K, sa, sb, ta, tb, epi))
+        return fail(CKX_UNSUPPORTED, "the contiguous extents of A and B and their strides must be multiples of 16 bytes "
+                                     "for this instance (the element-wise instance and AUTO take any)");
     if((long)(ta ? K : M) * sa * es >= (1l << 31) || (long)(tb ? K : N) * sb * es >= (1l << 31) ||
        (long)M * sc * es >= (1l << 31))
         return fail(CKX_UNSUPPORTED, "operands of 2 GiB or more are not addressed");
@@ -357,7 +373,8 @@ long gemm_workspace_bytes(int dt, int M, int N, int K, int instance)
     const int es = dt == ckx::DT_I8 ? 1 : 2;
     // (up to 32 rows go to the skinny kernels, which take none -- except few columns under a long K: see run_gemm)
     const bool few_cols = M >= 8 && (N + 15) / 16 < (M > 16 ? 257 : 128) && (long)K * es >= 16384;
-    if(M <= 0 || N <= 0 || (instance == CKX_INSTANCE_AUTO && M <= 32 && !few_cols) || instance >= kNumTiles)
+    if(M <= 0 || N <= 0 || (instance == CKX_INSTANCE_AUTO && M <= 32 && !few_cols) || instance >= kNumTiles ||
+       ((long)K * es) % 16)
         return 0;
     const Plan pl = make_plan(M, N, K * es, instance, 1l << 60);
     return pl.ksplit > 1 ? (long)pl.ksplit * M * N * 4 : 0;
@@ -378,12 +395,17 @@ int check_batch(int dt, int M, int N, int K, int sa, int sb, int sc, bool ta, bo
     if(batch > 1)
     {
         const int es = dt == ckx::DT_I8 ? 1 : 2;
-        if(instance >= kNumTiles)
-            return fail(CKX_UNSUPPORTED, "batched GEMM runs on the tile instances");
+        if(instance >= kNumTiles && instance != kGenericGemmInstance)
+            return fail(CKX_UNSUPPORTED, "batched GEMM runs on the tile instances and the element-wise instance");
         if(epi >= CKX_EPI_ADD_RELU || k_batch > 1)
             return fail(CKX_UNSUPPORTED, "batched GEMM has neither D operands nor a K split");
-        if(bsa < 0 || bsb < 0 || bsc < 0 || (bsa * es) % 16 || (bsb * es) % 16)
-            return fail(CKX_UNSUPPORTED, "batch strides of A and B must be non-negative multiples of 16 bytes");
+        if(bsa < 0 || bsb < 0 || bsc < 0)
+            return fail(CKX_UNSUPPORTED, "batch strides must be non-negative");
+        if(instance != CKX_INSTANCE_AUTO && instance != kGenericGemmInstance && ((bsa * es) % 16 || (bsb * es) % 16))
+            return fail(CKX_UNSUPPORTED, "batch strides of A and B must be multiples of 16 bytes for this instance");
+        if(batch > 65535 && (instance == kGenericGemmInstance || (bsa * es) % 16 || (bsb * es) % 16 ||
+                             gemm_needs_generic(dt, M, N, K, sa, sb, ta, tb, epi)))
+            return fail(CKX_UNSUPPORTED, "the element-wise instance takes at most 65535 batches");
         if(bsc < (long)(M - 1) * sc + N && M > 0 && N > 0)
             return fail(CKX_UNSUPPORTED, "C batches overlap");
         const long ea = operand_extent(batch, bsa, ta ? K : M, ta ? M : K, sa, es);
@@ -404,7 +426,7 @@ int run_gemm(int dt, const void* a, const void* b, void* c, int M, int N, int K,
         return st;
     if(k_batch < 0 || k_batch > 8)
         return fail(CKX_UNSUPPORTED, "KBatch must be 1..8");
-    if(k_batch > 0 && instance >= kNumTiles)
+    if(k_batch > 0 && instance >= kNumTiles && instance != kGenericGemmInstance)
         return fail(CKX_UNSUPPORTED, "the skinny instances split K over their waves, not over runs");
     const bool ta = al == CKX_COL_MAJOR, tb = bl == CKX_ROW_MAJOR, kmajor = ta || tb;
     if((st = check_batch(dt, M, N, K, sa, sb, sc, ta, tb, epi, instance, k_batch, batch, bsa, bsb, bsc)) != CKX_OK)
@@ -417,9 +439,35 @@ int run_gemm(int dt, const void* a, const void* b, void* c, int M, int N, int K,
         return CKX_OK;
     if(!a || !b || !c)
         return fail(CKX_INVALID_VALUE, "null operand pointer");
-    if((reinterpret_cast<uintptr_t>(a) | reinterpret_cast<uintptr_t>(b)) & 15)
-        return fail(CKX_UNSUPPORTED, "A and B must be 16-byte aligned");
     const int es = dt == ckx::DT_I8 ? 1 : 2;
+    const bool misaligned = ((reinterpret_cast<uintptr_t>(a) | reinterpret_cast<uintptr_t>(b)) & 15) != 0 ||
+                            (batch > 1 && ((bsa * es) % 16 || (bsb * es) % 16));
+    if(instance == kGenericGemmInstance ||
+       (instance == CKX_INSTANCE_AUTO && (misaligned || gemm_needs_generic(dt, M, N, K, sa, sb, ta, tb, epi))))
+    {
+        // element-granular instance: one pass over K whatever KBatch says (the result does not depend on the split)
+        if((reinterpret_cast<uintptr_t>(a) | reinterpret_cast<uintptr_t>(b) | reinterpret_cast<uintptr_t>(c) |
+            reinterpret_cast<uintptr_t>(dops.d0) | reinterpret_cast<uintptr_t>(dops.d1)) & (es - 1))
+            return fail(CKX_UNSUPPORTED, "operands must be aligned to their element size");
+        ckx::GemmArgs g;
+        std::memset(&g, 0, sizeof(g));
+        g.a = a, g.b = b, g.c = c;
+        g.M = M, g.N = N, g.K = K;
+        g.lda = sa, g.ldb = sb, g.ldc = sc;
+        g.batch = batch, g.bsa = bsa, g.bsb = bsb, g.bsc = bsc;
+        g.epi = epi, g.scale_gemm = sg, g.scale_relu = sr;
+        g.d0 = dops.d0, g.d1 = epi == CKX_EPI_ADD_RELU_ADD ? dops.d1 : nullptr;
+        g.ldd0 = dops.ldd0, g.ldd1 = dops.ldd1;
+        g.ksplit  = 1;
+        g.tiles_m = (M + 63) / 64, g.tiles_n = (N + 63) / 64;
+        ckx::GenericLayout lay{};
+        lay.a_sm = ta ? 1 : sa, lay.a_sk = ta ? sa : 1;
+        lay.b_sn = tb ? 1 : sb, lay.b_sk = tb ? sb : 1;
+        hipError_t e = ckx::launch_generic(dt, 0, g, lay, (hipStream_t)stream);
+        return e == hipSuccess ? CKX_OK : hip_fail(e, kGenericName);
+    }
+    if(misaligned)
+        return fail(CKX_UNSUPPORTED, "A and B (and their batch strides) must be 16-byte aligned for this instance");
     int ti = instance;
     Plan pl;
     // 33..64 rows: the tile kernel wins when its C tiles fill the machine, or C tiles x K runs over a long K
@@ -526,7 +574,8 @@ bool conv_patch_preferred(int op, const ckx_conv2d_desc* d, int epi)
 
 // ---------------------------------------------------------- weight-stationary pointwise conv kernel
 const char* const kPointwiseName = "MI355X_Mfma16_Pointwise<1x1, C 256/512 bytes, K 512 per workgroup, 8 waves>";
-constexpr int kConvPatchInstance = kNumTiles, kConvPointwiseInstance = kNumTiles + 1, kNumConvInsts = kNumTiles + 2;
+constexpr int kConvPatchInstance = kNumTiles, kConvPointwiseInstance = kNumTiles + 1, kConvGenericInstance = kNumTiles + 2,
+              kNumConvInsts = kNumTiles + 3;
 
 // shapes the pointwise kernel covers: 1x1 filters without padding, a pixel of 256 or 512 bytes, output channels in
 // whole blocks of 512
@@ -584,10 +633,13 @@ int check_conv(int op, const ckx_conv2d_desc* d, int epi, int instance)
        d->Ho < 0 || d->Wo < 0 || d->stride_h <= 0 || d->stride_w <= 0 || d->dilation_h <= 0 ||
        d->dilation_w <= 0 || d->pad_top < 0 || d->pad_left < 0 || d->pad_bottom < 0 || d->pad_right < 0)
         return fail(CKX_INVALID_VALUE, "bad conv geometry");
-    // window coordinates are kept as signed 16-bit pairs in the kernel
+    // window coordinates are kept as signed 16-bit pairs in the kernel: neither a window origin (ho * stride - pad,
+    // lowest -pad, highest (Ho - 1) * stride - pad) nor origin + tap offset may leave [-32768, 32767]
     if(d->Hi > 16384 || d->Wi > 16384 || d->pad_top >= 16384 || d->pad_left >= 16384 ||
-       (long)(d->Y - 1) * d->dilation_h >= 16384 || (long)(d->X - 1) * d->dilation_w >= 16384)
-        return fail(CKX_UNSUPPORTED, "spatial extents above 16384 are not addressed");
+       (long)(d->Y - 1) * d->dilation_h >= 16384 || (long)(d->X - 1) * d->dilation_w >= 16384 ||
+       (long)(d->Ho - 1) * d->stride_h - d->pad_top + (long)(d->Y - 1) * d->dilation_h >= 32768 ||
+       (long)(d->Wo - 1) * d->stride_w - d->pad_left + (long)(d->X - 1) * d->dilation_w >= 32768)
+        return fail(CKX_UNSUPPORTED, "spatial extents above 16384 (window coordinates above 32767) are not addressed");
     // the output extent has to be what the geometry implies (conv_util.cpp:103-114)
     const int ho = (d->Hi + d->pad_top + d->pad_bottom - ((d->Y - 1) * d->dilation_h + 1)) / d->stride_h + 1;
     const int wo = (d->Wi + d->pad_left + d->pad_right - ((d->X - 1) * d->dilation_w + 1)) / d->stride_w + 1;
@@ -595,8 +647,9 @@ int check_conv(int op, const ckx_conv2d_desc* d, int epi, int instance)
         return fail(CKX_UNSUPPORTED, "output spatial lengths do not match the conv geometry");
     // a 16-byte vector along c must not cross a filter tap
     // (device_conv2d_fwd_xdl_nhwc_kyxc_nhwk.hpp:595-601)
-    if(((long)d->C * es) % 16)
-        return fail(CKX_UNSUPPORTED, "C must be a multiple of 16 bytes");
+    // (ConvolutionForwardSpecialization::OddC is the element-wise instance; AUTO sends such layers there)
+    if(((long)d->C * es) % 16 && instance != CKX_INSTANCE_AUTO && instance != kConvGenericInstance)
+        return fail(CKX_UNSUPPORTED, "C must be a multiple of 16 bytes for this instance (the element-wise instance and AUTO take any)");
     const long in_b  = (long)d->N * d->Hi * d->Wi * d->C * es;
     const long wei_b = (long)d->K * d->Y * d->X * d->C * es;
     const long out_b = (long)d->N * d->Ho * d->Wo * d->K * es;
@@ -617,7 +670,8 @@ long conv_workspace_bytes(int op, const ckx_conv2d_desc* d, int instance)
     const long M = (long)d->N * d->Ho * d->Wo;
     if(M <= 0 || d->K <= 0)
         return 0;
-    if(instance == kConvPatchInstance || instance == kConvPointwiseInstance ||
+    if(instance == kConvPatchInstance || instance == kConvPointwiseInstance || instance == kConvGenericInstance ||
+       ((long)d->C * es) % 16 ||
        (instance == CKX_INSTANCE_AUTO &&
         (conv_patch_preferred(op, d, CKX_EPI_PASSTHROUGH) || conv_pointwise_preferred(op, d, CKX_EPI_PASSTHROUGH))))
         return 0;
@@ -639,8 +693,37 @@ int run_conv(int op, const void* in, const void* wei, void* out, const ckx_conv2
         return CKX_OK;
     if(!in || !wei || !out)
         return fail(CKX_INVALID_VALUE, "null operand pointer");
-    if((reinterpret_cast<uintptr_t>(in) | reinterpret_cast<uintptr_t>(wei)) & 15)
-        return fail(CKX_UNSUPPORTED, "input and weight must be 16-byte aligned");
+    const bool misaligned = ((reinterpret_cast<uintptr_t>(in) | reinterpret_cast<uintptr_t>(wei)) & 15) != 0;
+    if(instance == kConvGenericInstance || (instance == CKX_INSTANCE_AUTO && (misaligned || ((long)d->C * es) % 16)))
+    {
+        if((reinterpret_cast<uintptr_t>(in) | reinterpret_cast<uintptr_t>(wei) | reinterpret_cast<uintptr_t>(out) |
+            reinterpret_cast<uintptr_t>(dops.d0) | reinterpret_cast<uintptr_t>(dops.d1)) & (es - 1))
+            return fail(CKX_UNSUPPORTED, "operands must be aligned to their element size");
+        ckx::GemmArgs g;
+        std::memset(&g, 0, sizeof(g));
+        g.a = in, g.b = wei, g.c = out;
+        g.M = M, g.N = N, g.K = K;
+        g.ldb = K, g.ldc = N;
+        g.epi = epi, g.scale_gemm = sg, g.scale_relu = sr;
+        g.d0 = dops.d0, g.d1 = epi == CKX_EPI_ADD_RELU_ADD ? dops.d1 : nullptr;
+        g.ldd0 = dops.ldd0, g.ldd1 = dops.ldd1;
+        g.ksplit  = 1;
+        g.tiles_m = (M + 63) / 64, g.tiles_n = (N + 63) / 64;
+        g.cv.Hi = d->Hi, g.cv.Wi = d->Wi, g.cv.C = d->C;
+        g.cv.sH = d->stride_h, g.cv.sW = d->stride_w, g.cv.dH = d->dilation_h, g.cv.dW = d->dilation_w;
+        g.cv.pT = d->pad_top, g.cv.pL = d->pad_left;
+        g.cv.div_howo = make_magic((uint32_t)(d->Ho * d->Wo));
+        g.cv.div_wo   = make_magic((uint32_t)d->Wo);
+        g.cv.div_xc   = make_magic((uint32_t)(d->X * d->C));
+        g.cv.div_c    = make_magic((uint32_t)d->C);
+        ckx::GenericLayout lay{};
+        lay.b_sn = K, lay.b_sk = 1;
+        lay.X = d->X, lay.Y = d->Y;
+        hipError_t e = ckx::launch_generic(es == 1 ? ckx::DT_I8 : ckx::DT_F16, 1, g, lay, (hipStream_t)stream);
+        return e == hipSuccess ? CKX_OK : hip_fail(e, kGenericName);
+    }
+    if(misaligned)
+        return fail(CKX_UNSUPPORTED, "input and weight must be 16-byte aligned for this instance");
     if(ws && (reinterpret_cast<uintptr_t>(ws) & 15))
         return fail(CKX_INVALID_VALUE, "workspace must be 16-byte aligned");
     const bool patch_aligned = !((reinterpret_cast<uintptr_t>(out) | reinterpret_cast<uintptr_t>(dops.d0) |
@@ -771,7 +854,7 @@ int check_convnd(int op, const ckx_convnd_desc* d, int epi, int instance, ckx_co
     const int es = op == CKX_OP_CONV2D_FWD_I8 ? 1 : 2;
     if(instance != CKX_INSTANCE_AUTO && (instance < 0 || instance >= kNumConvInsts))
         return fail(CKX_INVALID_VALUE, "no such instance");
-    if(instance >= kNumTiles)
+    if(instance >= kNumTiles && instance != kConvGenericInstance)
         return fail(CKX_UNSUPPORTED, "the input-patch and pointwise instances cover two spatial dimensions");
     if(epi < CKX_EPI_PASSTHROUGH || epi > CKX_EPI_REQUANT_RND || !epilogue_fits_dtype(es, epi))
         return fail(CKX_INVALID_VALUE, "epilogue not available for this operator");
@@ -783,8 +866,9 @@ int check_convnd(int op, const ckx_convnd_desc* d, int epi, int instance, ckx_co
         if(d->in[i] <= 0 || d->filter[i] <= 0 || d->out[i] < 0 || d->stride[i] <= 0 || d->dilation[i] <= 0 ||
            d->pad_left[i] < 0 || d->pad_right[i] < 0)
             return fail(CKX_INVALID_VALUE, "bad conv geometry");
-        if(d->in[i] > 16384 || d->pad_left[i] >= 16384 || (long)(d->filter[i] - 1) * d->dilation[i] >= 16384)
-            return fail(CKX_UNSUPPORTED, "spatial extents above 16384 are not addressed");
+        if(d->in[i] > 16384 || d->pad_left[i] >= 16384 || (long)(d->filter[i] - 1) * d->dilation[i] >= 16384 ||
+           (long)(d->out[i] - 1) * d->stride[i] - d->pad_left[i] + (long)(d->filter[i] - 1) * d->dilation[i] >= 32768)
+            return fail(CKX_UNSUPPORTED, "spatial extents above 16384 (window coordinates above 32767) are not addressed");
         // conv_util.cpp:103-114
         const int o = (d->in[i] + d->pad_left[i] + d->pad_right[i] - ((d->filter[i] - 1) * d->dilation[i] + 1)) /
                           d->stride[i] + 1;
@@ -794,8 +878,8 @@ int check_convnd(int op, const ckx_convnd_desc* d, int epi, int instance, ckx_co
         if(in_px >= (1l << 31) || out_px >= (1l << 31) || taps >= (1l << 31))
             return fail(CKX_UNSUPPORTED, "tensors of 2 GiB or more are not addressed");
     }
-    if(((long)d->C * es) % 16)
-        return fail(CKX_UNSUPPORTED, "C must be a multiple of 16 bytes");
+    if(((long)d->C * es) % 16 && instance != CKX_INSTANCE_AUTO && instance != kConvGenericInstance)
+        return fail(CKX_UNSUPPORTED, "C must be a multiple of 16 bytes for this instance (the element-wise instance and AUTO take any)");
     // (device_convnd_fwd_xdl_nhwc_kyxc_nhwk.hpp:883-890 refuses tensors above 2 GB as well)
     if(in_px * d->C * es >= (1l << 31) || (long)d->K * taps * d->C * es >= (1l << 31) ||
        out_px * d->K * es >= (1l << 31) || taps * d->C >= (1l << 31))
@@ -813,7 +897,7 @@ long convnd_workspace_bytes(int op, const ckx_convnd_desc* d, int instance)
         return conv_workspace_bytes(op, &d2, instance);
     const int es = op == CKX_OP_CONV2D_FWD_I8 ? 1 : 2;
     const long M = (long)d->N * d->out[0] * d->out[1] * d->out[2];
-    if(M <= 0 || d->K <= 0)
+    if(M <= 0 || d->K <= 0 || instance == kConvGenericInstance || ((long)d->C * es) % 16)
         return 0;
     const Plan pl = make_plan((int)M, d->K, d->filter[0] * d->filter[1] * d->filter[2] * d->C * es, instance, 1l << 60, 0, false, true);
     return pl.ksplit > 1 ? (long)pl.ksplit * M * d->K * 4 : 0;
@@ -836,11 +920,16 @@ int run_convnd(int op, const void* in, const void* wei, void* out, const ckx_con
         return CKX_OK;
     if(!in || !wei || !out)
         return fail(CKX_INVALID_VALUE, "null operand pointer");
-    if((reinterpret_cast<uintptr_t>(in) | reinterpret_cast<uintptr_t>(wei)) & 15)
-        return fail(CKX_UNSUPPORTED, "input and weight must be 16-byte aligned");
+    const bool misaligned = ((reinterpret_cast<uintptr_t>(in) | reinterpret_cast<uintptr_t>(wei)) & 15) != 0;
+    const bool generic =
+        instance == kConvGenericInstance || (instance == CKX_INSTANCE_AUTO && (misaligned || ((long)d->C * es) % 16));
+    if(misaligned && !generic)
+        return fail(CKX_UNSUPPORTED, "input and weight must be 16-byte aligned for this instance");
+    if(generic && ((reinterpret_cast<uintptr_t>(in) | reinterpret_cast<uintptr_t>(wei) | reinterpret_cast<uintptr_t>(out)) & (es - 1)))
+        return fail(CKX_UNSUPPORTED, "operands must be aligned to their element size");
     if(ws && (reinterpret_cast<uintptr_t>(ws) & 15))
         return fail(CKX_INVALID_VALUE, "workspace must be 16-byte aligned");
-    const Plan pl         = make_plan(M, N, K * es, instance, ws ? ws_bytes : 0, 0, false, true);
+    const Plan pl         = generic ? Plan{} : make_plan(M, N, K * es, instance, ws ? ws_bytes : 0, 0, false, true);
     const TileInstance& t = kTiles[pl.tile];
     ckx::GemmArgs g;
     std::memset(&g, 0, sizeof(g));
@@ -868,6 +957,16 @@ int run_convnd(int op, const void* in, const void* wei, void* out, const ckx_con
     g.ksplit = pl.ksplit;
     g.nk_per = pl.nk_per;
     g.ws     = ws;
+    if(generic)
+    {
+        g.tiles_m = (M + 63) / 64, g.tiles_n = (N + 63) / 64;
+        g.ksplit  = 1;
+        ckx::GenericLayout lay{};
+        lay.b_sn = K, lay.b_sk = 1;
+        lay.X = d->filter[2], lay.Y = d->filter[1];
+        hipError_t e = ckx::launch_generic(es == 1 ? ckx::DT_I8 : ckx::DT_F16, 2, g, lay, (hipStream_t)stream);
+        return e == hipSuccess ? CKX_OK : hip_fail(e, kGenericName);
+    }
     const tile_launch_fn launch = ckx::conv3d_tile(es == 1 ? ckx::DT_I8 : ckx::DT_F16, pl.tile);
     if(!launch)
         return fail(CKX_UNSUPPORTED, "no kernel variant for this instance");
@@ -893,7 +992,7 @@ int ckx_num_instances(int op)
     if(op == CKX_OP_GEMM_SPLITK)
         return kNumTiles;
     if(op == CKX_OP_CONV2D_FWD_F16 || op == CKX_OP_CONV2D_FWD_I8)
-        return kNumConvInsts; // + the input-patch and the pointwise kernel
+        return kNumConvInsts; // + the input-patch, the pointwise and the element-wise kernel
     if(op == CKX_OP_BATCHED_GEMM_GEMM || op == CKX_OP_BATCHED_GEMM_SOFTMAX_GEMM)
         return ckx::kNumGemmGemmInstances;
     return 0;
@@ -909,8 +1008,10 @@ const char* ckx_instance_name(int op, int instance)
         (op == CKX_OP_BATCHED_GEMM_GEMM || op == CKX_OP_BATCHED_GEMM_SOFTMAX_GEMM
              ? ckx::gemm_gemm_instance_name(instance)
          : (op == CKX_OP_CONV2D_FWD_F16 || op == CKX_OP_CONV2D_FWD_I8) && instance >= kNumTiles
-             ? (instance == kConvPatchInstance ? kPatchName : kPointwiseName)
-             : instance >= kNumTiles ? kSkinny[instance - kNumTiles].name : kTiles[instance].name) +
+             ? (instance == kConvPatchInstance ? kPatchName : instance == kConvPointwiseInstance ? kPointwiseName : kGenericName)
+             : instance == kGenericGemmInstance ? kGenericName
+             : instance >= kNumTiles            ? kSkinny[instance - kNumTiles].name
+                                                : kTiles[instance].name) +
         ">";
     return s.c_str();
 }

@@ -101,9 +101,14 @@ const char* ckx_instance_name(int op, int instance);
  *   b_layout CKX_COL_MAJOR  "nk": B(k,n) at n*stride_b + k      CKX_ROW_MAJOR "kn": at k*stride_b + n
  *   c_layout CKX_ROW_MAJOR only (as in the reference's instance lists
  *   device_gemm_xdl_*_{mk_kn,mk_nk,km_kn,km_nk}_mn_instance.cpp).
- * The contiguous extent of A and of B and both strides must be whole 16-byte vectors. mk_nk runs on
- * every instance; a K-major operand (km / kn) on the tile instances of 64 rows and more (others report
- * CKX_UNSUPPORTED), with the PassThrough / requant epilogues. This holds for every ckx_gemm_* and
+ * The vectorised instances (tile and skinny) need the contiguous extent of A and of B, both strides and both
+ * base addresses to be whole 16-byte vectors, and report CKX_UNSUPPORTED otherwise -- the reference's
+ * GemmSpecialization::Default instances (gemm_specialization.hpp:10-20). mk_nk runs on every instance; a
+ * K-major operand (km / kn) on the tile instances of 64 rows and more, with the PassThrough / requant
+ * epilogues. The LAST instance of every GEMM family is element-granular (any K, M, N, strides and base
+ * addresses, all four layouts, every epilogue of the data type: the reference's KPadding / MNKPadding
+ * instances, device_gemm_xdl_cshuffle.hpp:99-184) and CKX_INSTANCE_AUTO sends there exactly the problems
+ * the vectorised instances refuse, so AUTO supports every shape. This holds for every ckx_gemm_* and
  * ckx_batched_gemm_* entry point below. */
 int ckx_gemm_i8_is_supported(int32_t M, int32_t N, int32_t K, int32_t stride_a, int32_t stride_b,
                              int32_t stride_c, int a_layout, int b_layout, int c_layout, int epilogue,
@@ -145,8 +150,9 @@ int64_t ckx_gemm_bf16_workspace_bytes(int32_t M, int32_t N, int32_t K, int insta
  * Batch, ...) + Run (device_batched_gemm.hpp:24-45; batch offsets as ComputePtrOffsetOfStridedBatch,
  * device_batched_gemm_xdl.hpp:256-285). Batch strides are in elements. The batches share one launch:
  * the persistent workgroups walk the C tiles of all batches. Shapes as for ckx_gemm_*_is_supported on a
- * tile instance (or AUTO); additionally the A / B batch strides must be multiples of 16 bytes, the C
- * batches must not overlap, and the whole A, B, C extents stay below 2 GiB. */
+ * tile instance, the element-granular instance or AUTO; the C batches must not overlap and the whole A, B, C
+ * extents stay below 2 GiB. On the tile instances the A / B batch strides must be multiples of 16 bytes; AUTO
+ * sends other strides (up to 65535 batches) to the element-granular instance. */
 int ckx_batched_gemm_is_supported(int op, int32_t M, int32_t N, int32_t K, int32_t stride_a, int32_t stride_b,
                                   int32_t stride_c, int64_t batch_stride_a, int64_t batch_stride_b,
                                   int64_t batch_stride_c, int32_t batch, int a_layout, int b_layout, int c_layout,
@@ -216,7 +222,13 @@ int ckx_gemm_f16_multiple_d(const void* p_a, const void* p_b, const void* p_d0, 
  * (device_conv2d_fwd_xdl_nhwc_kyxc_nhwk.hpp:57-720).
  * The vectors of the reference interface are passed as scalars in (H, W) order:
  * in_spatial = {Hi, Wi}, filter = {Y, X}, out_spatial = {Ho, Wo}, strides = {sH, sW},
- * dilations = {dH, dW}, left pads = {pad_top, pad_left}, right pads = {pad_bottom, pad_right}. */
+ * dilations = {dH, dW}, left pads = {pad_top, pad_left}, right pads = {pad_bottom, pad_right}.
+ * The vectorised instances need C to fill whole 16-byte vectors (C % 16 for int8, C % 8 for fp16; the
+ * reference: C % SrcScalarPerVector, device_conv2d_fwd_xdl_nhwc_kyxc_nhwk.hpp:595-601) and 16-byte aligned
+ * input and weight addresses. The LAST instance of both conv families is element-granular -- any C, the
+ * reference's ConvolutionForwardSpecialization::OddC instances (convolution_forward_specialization.hpp:13-19)
+ * -- for one, two and three spatial dimensions and every epilogue; CKX_INSTANCE_AUTO sends it the layers the
+ * vectorised instances refuse. */
 typedef struct ckx_conv2d_desc
 {
     int32_t N, K, C;

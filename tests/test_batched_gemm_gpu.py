@@ -81,6 +81,9 @@ def test_batched_gemm_argument_checks():
     ok = lambda *x: L.ckx_batched_gemm_is_supported(*x)
     assert ok(capi.OP_GEMM_F16, 64, 64, 64, 64, 64, 64, 4096, 4096, 4096, 4, 0, 1, 0, 0, -1) == capi.OK
     assert ok(capi.OP_GEMM_F16, 64, 64, 64, 64, 64, 64, 4096, 4096, 100, 4, 0, 1, 0, 0, -1) == capi.UNSUPPORTED   # C overlap
-    assert ok(capi.OP_GEMM_F16, 64, 64, 64, 64, 64, 64, 4100, 4096, 4096, 4, 0, 1, 0, 0, -1) == capi.UNSUPPORTED  # A stride
+    # a batch stride of A that is not a whole 16-byte vector: the element-wise instance (and AUTO through it) only
+    assert ok(capi.OP_GEMM_F16, 64, 64, 64, 64, 64, 64, 4100, 4096, 4096, 4, 0, 1, 0, 0, 0) == capi.UNSUPPORTED
+    assert ok(capi.OP_GEMM_F16, 64, 64, 64, 64, 64, 64, 4100, 4096, 4096, 4, 0, 1, 0, 0, -1) == capi.OK
+    assert ok(capi.OP_GEMM_F16, 64, 64, 64, 64, 64, 64, -8, 4096, 4096, 4, 0, 1, 0, 0, -1) == capi.UNSUPPORTED
     assert ok(capi.OP_GEMM_I8, 64, 64, 64, 64, 64, 64, 4096, 4096, 4096, -1, 0, 1, 0, 0, -1) == capi.INVALID_VALUE
     assert ok(capi.OP_GEMM_I8, 16, 64, 64, 64, 64, 64, 4096, 4096, 4096, 4, 0, 1, 0, 0, 9) == capi.UNSUPPORTED     # skinny

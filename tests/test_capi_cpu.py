@@ -43,9 +43,8 @@ def test_gemm_argument_validation_is_pure_host_logic():
     ok = op.MakeArgumentPointer(0, 0, 0, 1024, 1024, 1024, 1024, 1024, 1024, None, None,
                                 ck.RequantReluRequant(0.5, 0.03, rounded=True))
     assert op.IsSupportedArgument(ok)
-    # K not a multiple of 16 bytes; stride below K; column-major C; >= 2 GiB operand
+    # stride below K; column-major C; >= 2 GiB operand
     for bad in [
-        op.MakeArgumentPointer(0, 0, 0, 64, 64, 100, 100, 100, 64),
         op.MakeArgumentPointer(0, 0, 0, 64, 64, 128, 64, 128, 64),
         op.MakeArgumentPointer(0, 0, 0, 1 << 16, 64, 1 << 15, 1 << 15, 1 << 15, 64),
     ]:
@@ -55,12 +54,20 @@ def test_gemm_argument_validation_is_pure_host_logic():
     assert not ck.DeviceGemmInt8(instance=999).IsSupportedArgument(ok)
     f16 = ck.DeviceGemmF16()
     assert f16.IsSupportedArgument(f16.MakeArgumentPointer(0, 0, 0, 4096, 4096, 4096, 4096, 4096, 4096))
-    assert not f16.IsSupportedArgument(f16.MakeArgumentPointer(0, 0, 0, 64, 64, 60, 60, 60, 64))
+    # K not a multiple of 16 bytes (the reference's KPadding / MNKPadding instances): the vectorised instances
+    # refuse, the element-wise instance -- the last of the list -- and the automatic choice accept
+    last = capi.lib().ckx_num_instances(capi.OP_GEMM_I8) - 1
+    assert b"Generic" in capi.lib().ckx_instance_name(capi.OP_GEMM_I8, last)
+    for cls, (M, N, K) in ((ck.DeviceGemmInt8, (64, 64, 100)), (ck.DeviceGemmF16, (64, 64, 60))):
+        assert cls().IsSupportedArgument(cls().MakeArgumentPointer(0, 0, 0, M, N, K, K, K, N))
+        assert cls(last).IsSupportedArgument(cls(last).MakeArgumentPointer(0, 0, 0, M, N, K, K, K, N))
+        for inst in range(last):
+            assert not cls(inst).IsSupportedArgument(cls(inst).MakeArgumentPointer(0, 0, 0, 16, N, K, K, K, N))
     # a functor the fp16 operator does not fuse
     assert not f16.IsSupportedArgument(
         f16.MakeArgumentPointer(0, 0, 0, 64, 64, 64, 64, 64, 64, None, None, ck.RequantReluRequant(1, 1)))
     with pytest.raises(RuntimeError):
-        op.MakeInvokerPointer().Run(op.MakeArgumentPointer(0, 0, 0, 64, 64, 100, 100, 100, 64))
+        op.MakeInvokerPointer().Run(op.MakeArgumentPointer(0, 0, 0, 64, 64, 128, 64, 128, 64))
 
 
 def test_conv_argument_validation():
@@ -68,7 +75,11 @@ def test_conv_argument_validation():
     mk = lambda C_, osp: op.MakeArgumentPointer(0, 0, 0, 256, 64, C_, [56, 56], [3, 3], osp, [1, 1], [1, 1],
                                                 [1, 1], [1, 1])
     assert op.IsSupportedArgument(mk(64, [56, 56]))
-    assert not op.IsSupportedArgument(mk(3, [56, 56]))      # C*2 bytes not a multiple of 16
+    # C * 2 bytes not a multiple of 16 (ConvolutionForwardSpecialization::OddC): element-wise instance and AUTO only
+    assert op.IsSupportedArgument(mk(3, [56, 56]))
+    n = capi.lib().ckx_num_instances(capi.OP_CONV2D_FWD_F16)
+    assert ck.DeviceConv2dFwdF16(n - 1).IsSupportedArgument(mk(3, [56, 56]))
+    assert not any(ck.DeviceConv2dFwdF16(i).IsSupportedArgument(mk(3, [56, 56])) for i in range(n - 1))
     assert not op.IsSupportedArgument(mk(64, [55, 56]))     # output size does not follow from the geometry
     with pytest.raises(ValueError):
         op.MakeArgumentPointer(0, 0, 0, 1, 1, 8, [8], [3], [6], [1], [1], [0], [0])   # only 2-D is built

@@ -73,15 +73,17 @@ def test_conv2d_reference_golden_vectors_fp16():
         N, K, C = case["N"], case["K"], case["C"]
         Hi, Wi = case["input"]
         Y, X = case["filter"]
-        # C = 2 in the reference case; the kernel needs 16-byte channel vectors, so the two
-        # channels are embedded in 8 (zeros elsewhere), which leaves every sum unchanged.
-        inp = np.zeros((N, Hi, Wi, 8), np.float16)
-        inp[..., :C] = np.arange(N * Hi * Wi * C, dtype=np.float32).reshape(N, Hi, Wi, C)
-        wei = np.zeros((K, Y, X, 8), np.float16)
-        wei[..., :C] = 0.5
-        out = gpu_util.conv2d_fwd(inp, wei, case["strides"], case["dilations"], case["left_pads"],
-                                  right_pads=case["right_pads"])
-        np.testing.assert_array_equal(out.ravel(), np.array(case["expected"], np.float32).astype(np.float16))
+        # C = 2 as in the reference case (4-byte pixels: the element-wise instance), and the same two channels
+        # embedded in 8 (zeros elsewhere leave every sum unchanged: the vectorised instances)
+        want = np.array(case["expected"], np.float32).astype(np.float16)
+        for cpad in (C, 8):
+            inp = np.zeros((N, Hi, Wi, cpad), np.float16)
+            inp[..., :C] = np.arange(N * Hi * Wi * C, dtype=np.float32).reshape(N, Hi, Wi, C)
+            wei = np.zeros((K, Y, X, cpad), np.float16)
+            wei[..., :C] = 0.5
+            out = gpu_util.conv2d_fwd(inp, wei, case["strides"], case["dilations"], case["left_pads"],
+                                      right_pads=case["right_pads"])
+            np.testing.assert_array_equal(out.ravel(), want)
 
 
 RESNET = [
@@ -149,11 +151,13 @@ def test_conv2d_unsupported_arguments_are_refused():
     import torch
     d = torch.zeros(1 << 16, dtype=torch.int8, device="cuda")
     op = ck.DeviceConv2dFwdInt8()
-    # C = 3 (the reference's OddC case) is not a whole 16-byte vector
-    arg = op.MakeArgumentPointer(d, d, d, 1, 8, 3, [8, 8], [3, 3], [6, 6], [1, 1], [1, 1], [0, 0], [0, 0])
-    assert not op.IsSupportedArgument(arg)
+    # C = 3 (the reference's OddC case) is not a whole 16-byte vector: the vectorised instances refuse it
+    fast_op = ck.DeviceConv2dFwdInt8(0)
+    arg = fast_op.MakeArgumentPointer(d, d, d, 1, 8, 3, [8, 8], [3, 3], [6, 6], [1, 1], [1, 1], [0, 0], [0, 0])
+    assert not fast_op.IsSupportedArgument(arg)
     with pytest.raises(RuntimeError):
-        op.MakeInvokerPointer().Run(arg)
+        fast_op.MakeInvokerPointer().Run(arg)
+    assert op.IsSupportedArgument(op.MakeArgumentPointer(d, d, d, 1, 8, 3, [8, 8], [3, 3], [6, 6], [1, 1], [1, 1], [0, 0], [0, 0]))
     # output size inconsistent with the geometry
     arg = op.MakeArgumentPointer(d, d, d, 1, 8, 16, [8, 8], [3, 3], [7, 6], [1, 1], [1, 1], [0, 0], [0, 0])
     assert not op.IsSupportedArgument(arg)

@@ -73,18 +73,20 @@ GOLD_ND = json.load(open(os.path.join(HERE, "golden", "reference_convnd_fwd_vect
 @pytest.mark.parametrize("case", [c for c in GOLD_ND["cases"] if c["fill_start_step"] == [0.0, 1.0]],
                          ids=lambda c: c["name"])
 def test_convnd_reference_golden_vectors_fp16(case):
-    """The reference's 1-D golden cases with integer inputs: exactly representable in fp16, C padded to a whole
-    16-byte vector with zero channels (which add nothing)."""
+    """The reference's golden cases with integer inputs: exactly representable in fp16. Run with the case's own
+    channel count (C = 2: the element-wise instance) and with C padded to a whole 16-byte vector by zero channels,
+    which add nothing (the vectorised instances)."""
     import gpu_util
     N, K, Cc = case["N"], case["K"], case["C"]
     sp, filt = case["input"], case["filter"]
-    inp = np.zeros((N, *sp, 8), np.float16)
-    inp[..., :Cc] = np.arange(N * int(np.prod(sp)) * Cc, dtype=np.float32).reshape(N, *sp, Cc)
-    wei = np.zeros((K, *filt, 8), np.float16)
-    wei[..., :Cc] = 0.5
-    out = gpu_util.convnd_fwd(inp, wei, case["strides"], case["dilations"], case["left_pads"],
-                              right_pads=case["right_pads"])
-    np.testing.assert_array_equal(out.ravel().astype(np.float32), np.array(case["expected"], np.float32))
+    for cpad in (Cc, 8):
+        inp = np.zeros((N, *sp, cpad), np.float16)
+        inp[..., :Cc] = np.arange(N * int(np.prod(sp)) * Cc, dtype=np.float32).reshape(N, *sp, Cc)
+        wei = np.zeros((K, *filt, cpad), np.float16)
+        wei[..., :Cc] = 0.5
+        out = gpu_util.convnd_fwd(inp, wei, case["strides"], case["dilations"], case["left_pads"],
+                                  right_pads=case["right_pads"])
+        np.testing.assert_array_equal(out.ravel().astype(np.float32), np.array(case["expected"], np.float32))
 
 
 @pytest.mark.parametrize("dtype", ["i8", "f16"])
@@ -134,7 +136,9 @@ def test_convnd_unsupported_arguments_are_refused():
     bad = mk(2, 16, 16, [6, 6, 6], [3, 3, 3], [4, 5, 4], one, one, [0, 0, 0], [0, 0, 0])
     assert L.ckx_convnd_fwd_is_supported(capi.OP_CONV2D_FWD_F16, C.byref(bad), 0, -1) == capi.UNSUPPORTED
     n = L.ckx_num_instances(capi.OP_CONV2D_FWD_F16)
-    assert L.ckx_convnd_fwd_is_supported(capi.OP_CONV2D_FWD_F16, C.byref(ok), 0, n - 1) == capi.UNSUPPORTED
+    assert L.ckx_convnd_fwd_is_supported(capi.OP_CONV2D_FWD_F16, C.byref(ok), 0, n - 1) == capi.OK           # element-wise
+    assert L.ckx_convnd_fwd_is_supported(capi.OP_CONV2D_FWD_F16, C.byref(ok), 0, n - 2) == capi.UNSUPPORTED  # pointwise
+    assert L.ckx_convnd_fwd_is_supported(capi.OP_CONV2D_FWD_F16, C.byref(ok), 0, n - 3) == capi.UNSUPPORTED  # input patch
     assert L.ckx_convnd_fwd_is_supported(capi.OP_CONV2D_FWD_F16, C.byref(ok), 0, n) == capi.INVALID_VALUE
     four = capi.ConvNdDesc(4, 1, 16, 16)
     assert L.ckx_convnd_fwd_is_supported(capi.OP_CONV2D_FWD_F16, C.byref(four), 0, -1) == capi.INVALID_VALUE

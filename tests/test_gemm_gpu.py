@@ -16,7 +16,7 @@ from oracle import fast, lit
 
 pytestmark = pytest.mark.gpu
 
-N_INSTANCES = 17        # tile instances followed by the skinny (few-row) instances
+N_INSTANCES = 18        # tile instances, the skinny (few-row) instances, the element-wise (padding) instance
 SKINNY_MAX_M = {9: 16, 10: 32, 11: 64, 12: 16, 13: 16, 14: 16, 15: 32, 16: 32}
 RTOL = ATOL = 1e-2
 
@@ -124,11 +124,17 @@ def test_int8_gemm_unsupported_arguments_are_refused():
     import torch
     op = ck.DeviceGemmInt8()
     d = torch.zeros(1 << 16, dtype=torch.int8, device="cuda")
-    # K not a multiple of 16 bytes
-    arg = op.MakeArgumentPointer(d, d, d, 64, 64, 100, 100, 100, 64)
-    assert not op.IsSupportedArgument(arg)
-    with pytest.raises(RuntimeError):
-        op.MakeInvokerPointer().Run(arg)
+    # K not a multiple of 16 bytes: the vectorised instances refuse (as the reference's Default-specialisation
+    # instances do), the element-wise instance and the automatic choice take it (its KPadding instances)
+    for instance in range(N_INSTANCES - 1):
+        fast = ck.DeviceGemmInt8(instance)
+        arg = fast.MakeArgumentPointer(d, d, d, 16, 64, 100, 100, 100, 64)
+        assert not fast.IsSupportedArgument(arg)
+        with pytest.raises(RuntimeError):
+            fast.MakeInvokerPointer().Run(arg)
+    assert op.IsSupportedArgument(op.MakeArgumentPointer(d, d, d, 64, 64, 100, 100, 100, 64))
+    # a leading dimension below the row length
+    assert not op.IsSupportedArgument(op.MakeArgumentPointer(d, d, d, 64, 64, 100, 99, 100, 64))
     # column-major C is not built (nor is it in the reference's instance lists)
     op2 = ck.DeviceGemmInt8(CLayout=ck.ColumnMajor)
     assert not op2.IsSupportedArgument(op2.MakeArgumentPointer(d, d, d, 64, 64, 64, 64, 64, 64))

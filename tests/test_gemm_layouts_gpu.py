@@ -177,13 +177,16 @@ def test_layouts_refused_arguments(layout):
     for instance in (5, 6, n_tiles, n_tiles + 4):          # tiles of 32 / 16 rows, skinny instances
         _run("i8", layout, a_st, b_st, M, N, K, instance, expect_unsupported=True)
     al, bl = LAYOUTS[layout]
-    # contiguous extent of the K-major operand not a whole 16-byte vector
+    # contiguous extent of the K-major operand not a whole 16-byte vector: refused by the vectorised tile instances,
+    # taken by the element-wise instance and by the automatic choice; a stride below the extent by nobody
     lib = capi.lib()
     if al is ck.ColumnMajor:
-        assert lib.ckx_gemm_f16_is_supported(60, 64, 64, 64, 64, 64, al.code, bl.code, ck.RowMajor.code, -1) == capi.UNSUPPORTED
+        assert lib.ckx_gemm_f16_is_supported(60, 64, 64, 64, 64, 64, al.code, bl.code, ck.RowMajor.code, 0) == capi.UNSUPPORTED
+        assert lib.ckx_gemm_f16_is_supported(60, 64, 64, 64, 64, 64, al.code, bl.code, ck.RowMajor.code, -1) == capi.OK
         assert lib.ckx_gemm_f16_is_supported(64, 64, 64, 60, 64, 64, al.code, bl.code, ck.RowMajor.code, -1) == capi.UNSUPPORTED
     if bl is ck.RowMajor:
-        assert lib.ckx_gemm_i8_is_supported(64, 72, 64, 64, 80, 72, al.code, bl.code, ck.RowMajor.code, 0, -1) == capi.UNSUPPORTED
+        assert lib.ckx_gemm_i8_is_supported(64, 72, 64, 64, 80, 72, al.code, bl.code, ck.RowMajor.code, 0, 0) == capi.UNSUPPORTED
+        assert lib.ckx_gemm_i8_is_supported(64, 72, 64, 64, 80, 72, al.code, bl.code, ck.RowMajor.code, 0, -1) == capi.OK
     # column-major C is in none of the reference's instance lists either
     assert lib.ckx_gemm_f16_is_supported(64, 64, 64, 64, 64, 64, al.code, bl.code, ck.ColumnMajor.code, -1) == capi.UNSUPPORTED
 

@@ -94,12 +94,22 @@ def test_profiler_batched_gemm_gemm(tmp_path):
     assert bad == 0, max_err
 
 
-def test_profiler_reports_unsupported_problems():
+def test_profiler_reports_unsupported_problems(tmp_path):
+    """K = 100 is not a whole 16-byte vector: every vectorised instance says it does not support the problem (as the
+    reference's profiler prints, profile_gemm_impl.hpp:205-208), the element-wise instance runs it; a leading
+    dimension below K is supported by no instance and the profiler fails."""
+    M, N, K = 64, 64, 100
+    out, dump = _run("ckx_profiler", ["gemm", 3, 1, 1, 1, 0, 0, M, N, K, -1, -1, -1], "CKX_PROFILER_DUMP", tmp_path)
+    assert out.count("does not support this problem") == 17      # the tile and skinny instances; the last one runs
+    c = np.fromfile(dump, np.int8).reshape(M, N)
+    a = uniform_int8((M, K), -5, 5, SEED)
+    b_nk = uniform_int8((N, K), -5, 5, SEED + 1)
+    np.testing.assert_array_equal(c, lit.gemm_i8(a, b_nk.T))
     path = os.path.join(BIN, "ckx_profiler")
-    r = subprocess.run([path, "gemm", "3", "1", "0", "1", "0", "0", "64", "64", "100", "-1", "-1", "-1"],
+    r = subprocess.run([path, "gemm", "3", "1", "0", "1", "0", "0", "64", "64", "100", "50", "-1", "-1"],
                        stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=120)
     assert r.returncode == 1
-    assert "does not support this problem" in r.stdout
+    assert "does not support this problem" in r.stdout and "no instance supports this problem" in r.stdout
 
 
 def test_example_gemm_requant_relu_requant_int8(tmp_path):
