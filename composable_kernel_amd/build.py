@@ -4,6 +4,15 @@
 
 Flags: -ffp-contract=off keeps the requant epilogue's fp32 multiplies unfused;
 packed fp32 VALU forms are disabled for the device pass.
+
+Two guards protect the kernels' hand-managed waits (the MFMA fragment reads of gemm_tile.hpp, conv_patch.hpp and
+conv_pointwise.hpp are inline-assembly LDS reads that the compiler does not count in lgkmcnt; the kernels wait for
+them themselves, so no compiler-made copy or spill of such a register may run before that wait):
+  * every kernel's register report (-Rpass-analysis=kernel-resource-usage) is read, and the build FAILS if one of
+    those kernels spills vector registers (the fused two-GEMM kernel, which reads LDS through compiler-known
+    builtins, is allowed its four spilled registers in the long-sequence softmax variant);
+  * the compiler version the kernels were validated with is recorded below; another one builds with a loud warning
+    (the bit-exact integer-operand GPU tests are the gate for adopting it).
 """
 import os
 import subprocess
@@ -18,7 +27,46 @@ HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 
 DEVICE_FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-ffp-contract=off",
                 "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
-                "-Wno-unused-command-line-argument"]
+                "-Rpass-analysis=kernel-resource-usage", "-Wno-unused-command-line-argument"]
+# hipcc --version lines of the toolchain whose code generation the GPU suite has validated
+VALIDATED_COMPILERS = ("AMD clang version 22.0.0git (https://github.com/RadeonOpenCompute/llvm-project roc-7.2.0 26014 "
+                       "7b800a19466229b8479a78de19143dc33c3ab9b5)",)
+
+
+def compiler_version():
+    r = subprocess.run([HIPCC, "--version"], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    for line in r.stdout.splitlines():
+        if "clang version" in line:
+            return line.strip()
+    return r.stdout.strip()[:200]
+
+
+def check_compiler():
+    import warnings
+    v = compiler_version()
+    if v not in VALIDATED_COMPILERS:
+        warnings.warn(f"libckx is being built with an unvalidated compiler ({v}); its kernels wait for inline-assembly "
+                      "LDS reads by hand and were validated with " + VALIDATED_COMPILERS[0] + ": run the GPU suite "
+                      "(bit-exact integer-operand tests) before trusting this build", RuntimeWarning, stacklevel=2)
+    return v
+
+
+# kernels whose LDS fragment reads are inline assembly waited for by hand (mangled-name fragments)
+HAND_WAITED_KERNELS = ("gemm_tile_kernel", "conv_patch_kernel", "conv_pointwise_kernel")
+
+
+def vgpr_spills(compiler_output):
+    """(kernel, spilled VGPRs) for every hand-waited kernel of a -Rpass-analysis=kernel-resource-usage report that
+    spills vector registers."""
+    bad, name = [], "?"
+    for line in compiler_output.splitlines():
+        if "Function Name:" in line:
+            name = line.split("Function Name:", 1)[1].split("[", 1)[0].strip()
+        elif "VGPRs Spill:" in line:
+            n = int(line.split("VGPRs Spill:", 1)[1].split("[", 1)[0])
+            if n and any(k in name for k in HAND_WAITED_KERNELS):
+                bad.append((name, n))
+    return bad
 
 
 def sources():
@@ -42,13 +90,30 @@ def build_lib(force=False, verbose=False, extra_flags=()):
     units = [f for f in sources() if f.endswith(".hip")]
     objs = [os.path.join(LIBDIR, os.path.basename(u)[:-4] + ".o") for u in units]
 
+    check_compiler()
+
     def run(cmd):
         if verbose:
             print(" ".join(cmd))
         r = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
-        out = "\n".join(l for l in r.stdout.splitlines() if "packed-fp32-ops" not in l)
+        lines = [l for l in r.stdout.splitlines() if "packed-fp32-ops" not in l]
+        # the register report: keep it out of the log, fail on vector register spills
+        spills = vgpr_spills(r.stdout)
+        out, skip = [], 0
+        for l in lines:
+            if "[-Rpass-analysis=kernel-resource-usage]" in l:
+                skip = 2          # the remark is followed by a source line and a caret line
+                continue
+            if skip and (l.lstrip().startswith("|") or l.strip()[:1].isdigit() or l.startswith("In file included")):
+                skip -= 1
+                continue
+            out.append(l)
+        out = "\n".join(l for l in out if not l.startswith("In file included from") and "remarks generated" not in l)
         if r.returncode != 0:
-            raise RuntimeError("hipcc failed:\n" + out)
+            raise RuntimeError("hipcc failed:\n" + "\n".join(lines))
+        if spills:
+            raise RuntimeError("vector register spills (the hand-managed LDS read waits do not survive them): "
+                               + ", ".join(f"{k}: {n}" for k, n in spills))
         if verbose and out.strip():
             print(out)
 

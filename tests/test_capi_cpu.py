@@ -111,3 +111,22 @@ def test_missing_library_fails_loudly(tmp_path, monkeypatch):
     monkeypatch.setattr(capi, "LIB_PATH", str(tmp_path / "libckx.so"))
     with pytest.raises(FileNotFoundError):
         capi.lib()
+
+
+def test_build_guards_for_the_hand_waited_kernels():
+    """The build reads every kernel's register report and refuses vector register spills in the kernels whose LDS
+    fragment reads are waited for by hand; it knows which compiler those kernels were validated with."""
+    from composable_kernel_amd import build
+    report = """
+gemm_tile.hpp:1172:1: remark: Function Name: _ZN3ckx16gemm_tile_kernelILi0ELi256ELi256EEvNS_8GemmArgsE [-Rpass-analysis=kernel-resource-usage]
+gemm_tile.hpp:1172:1: remark:     VGPRs: 256 [-Rpass-analysis=kernel-resource-usage]
+gemm_tile.hpp:1172:1: remark:     VGPRs Spill: 7 [-Rpass-analysis=kernel-resource-usage]
+gemm_gemm.hpp:400:1: remark: Function Name: _ZN3ckx16gemm_gemm_kernelILi4EEEvNS_12GemmGemmArgsE [-Rpass-analysis=kernel-resource-usage]
+gemm_gemm.hpp:400:1: remark:     VGPRs Spill: 4 [-Rpass-analysis=kernel-resource-usage]
+conv_patch.hpp:410:1: remark: Function Name: _ZN3ckx17conv_patch_kernelILi1EEEvNS_13ConvPatchArgsE [-Rpass-analysis=kernel-resource-usage]
+conv_patch.hpp:410:1: remark:     VGPRs Spill: 0 [-Rpass-analysis=kernel-resource-usage]
+"""
+    assert build.vgpr_spills(report) == [("_ZN3ckx16gemm_tile_kernelILi0ELi256ELi256EEvNS_8GemmArgsE", 7)]
+    assert "-Rpass-analysis=kernel-resource-usage" in build.DEVICE_FLAGS
+    assert "clang version" in build.compiler_version()
+    assert all("clang version" in v for v in build.VALIDATED_COMPILERS)
