@@ -33,6 +33,7 @@ SYMBOLS = [
     "ckx_convnd_fwd_is_supported", "ckx_convnd_fwd", "ckx_convnd_fwd_workspace_bytes",
     "ckx_batched_gemm_gemm_f16_is_supported", "ckx_batched_gemm_gemm_f16", "ckx_time_launches",
     "ckx_batched_gemm_softmax_gemm_f16_is_supported", "ckx_batched_gemm_softmax_gemm_f16",
+    "ckx_gemm_plan", "ckx_conv2d_fwd_plan", "ckx_set_forced_k_runs",
 ]
 
 
@@ -130,6 +131,10 @@ def lib():
     L.ckx_batched_gemm_softmax_gemm_f16_is_supported.argtypes = gsg
     L.ckx_batched_gemm_softmax_gemm_f16.argtypes = [vp] * 4 + gsg + [vp]
     L.ckx_time_launches.argtypes = [LAUNCH_FN, vp, C.c_int, C.c_int, vp, C.POINTER(C.c_float)]
+    ip = C.POINTER(C.c_int)
+    L.ckx_gemm_plan.argtypes = [C.c_int] + shape + [C.c_int, i32, i64, ip, ip]
+    L.ckx_conv2d_fwd_plan.argtypes = [C.c_int, dp, C.c_int, i64, ip, ip]
+    L.ckx_set_forced_k_runs.argtypes = [C.c_int]
     _lib = L
     return L
 
@@ -149,3 +154,21 @@ def time_launches(fn, n_warmup, n_repeat, stream):
     cb = LAUNCH_FN(lambda _u: int(fn()))
     check(lib().ckx_time_launches(cb, None, int(n_warmup), int(n_repeat), C.c_void_p(stream or 0), C.byref(ms)))
     return float(ms.value)
+
+
+def gemm_plan(op, M, N, K, sa=None, sb=None, sc=None, a_layout=ROW_MAJOR, b_layout=COL_MAJOR, epilogue=EPI_PASSTHROUGH,
+              batch=1, workspace_bytes=0, instance=INSTANCE_AUTO):
+    """(instance, K runs) a launch of this GEMM would use (ckx_gemm_plan); strides default to the dense ones."""
+    sa = sa if sa is not None else (K if a_layout == ROW_MAJOR else M)
+    sb = sb if sb is not None else (K if b_layout == COL_MAJOR else N)
+    sc = sc if sc is not None else N
+    inst, runs = C.c_int(instance), C.c_int(0)
+    check(lib().ckx_gemm_plan(op, M, N, K, sa, sb, sc, a_layout, b_layout, ROW_MAJOR, epilogue, batch, int(workspace_bytes),
+                              C.byref(inst), C.byref(runs)))
+    return inst.value, runs.value
+
+
+def conv2d_fwd_plan(op, desc, epilogue=EPI_PASSTHROUGH, workspace_bytes=0, instance=INSTANCE_AUTO):
+    inst, runs = C.c_int(instance), C.c_int(0)
+    check(lib().ckx_conv2d_fwd_plan(op, C.byref(desc), epilogue, int(workspace_bytes), C.byref(inst), C.byref(runs)))
+    return inst.value, runs.value

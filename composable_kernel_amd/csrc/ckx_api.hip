@@ -6,6 +6,7 @@
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
+#include <atomic>
 #include <mutex>
 #include <string>
 
@@ -138,11 +139,20 @@ struct Plan
     int nk_per = 0;
 };
 
+// CKX_KSPLIT=n forces n K runs where the problem allows it (tuning / test knob). The environment is read on the first
+// call only; ckx_set_forced_k_runs() changes the value afterwards (tests force several splits in one process).
+std::atomic<int> g_force_ksplit{-1};
 int force_ksplit()
 {
-    // CKX_KSPLIT=n forces n K runs where the problem allows it (tuning / test knob); read per call
-    const char* e = std::getenv("CKX_KSPLIT");
-    return e ? std::atoi(e) : 0;
+    int v = g_force_ksplit.load(std::memory_order_relaxed);
+    if(v < 0)
+    {
+        const char* e = std::getenv("CKX_KSPLIT");
+        v             = e ? std::atoi(e) : 0;
+        v             = v < 0 ? 0 : v;
+        g_force_ksplit.store(v, std::memory_order_relaxed);
+    }
+    return v;
 }
 
 // Choice by a small cost model (microseconds on a 256-CU part): work units (C tile x K run) are
@@ -165,11 +175,12 @@ int splitk_runs(int kbytes, int k_batch)
 // kmajor: a K-major operand (A column-major / B row-major) -- only the tiles of 64 rows and more
 // conv: A is gathered (im2col): the 8-wave 256 x 64 tile measures ahead of the 128 x 64 one there by 10 - 17 %
 // (ResNet-like layers at N = 32 and 256), which the GEMM-calibrated figures did not say
-Plan make_plan(int M, int N, int kbytes, int only_tile, long workspace_bytes, int k_batch = 0, bool kmajor = false,
+Plan make_plan(long M, int N, int kbytes, int only_tile, long workspace_bytes, int k_batch = 0, bool kmajor = false,
                bool conv = false)
 {
     Plan best;
     double best_us  = 1e30;
+    const long cus  = num_cus(); // (the time constants below were measured on a 256-CU part)
     const int nk    = (kbytes + 127) / 128 > 0 ? (kbytes + 127) / 128 : 1;
     const int force = k_batch > 0 ? splitk_runs(kbytes, k_batch) : force_ksplit();
     for(int i = 0; i < kNumTiles; ++i)
@@ -192,8 +203,8 @@ Plan make_plan(int M, int N, int kbytes, int only_tile, long workspace_bytes, in
             int per_cu       = 160 * 1024 / t.lds;
             per_cu           = per_cu > 2048 / t.threads ? 2048 / t.threads : per_cu;
             per_cu           = per_cu > 4 ? 4 : per_cu;
-            per_cu           = (long)per_cu * 256 > units ? (int)((units + 255) / 256) : per_cu;
-            const long rounds = (units + 256l * per_cu - 1) / (256l * per_cu);
+            per_cu           = per_cu * cus > units ? (int)((units + cus - 1) / cus) : per_cu;
+            const long rounds = (units + cus * per_cu - 1) / (cus * per_cu);
             // one K-tile iteration costs its MFMA time, but never less than the barrier + load
             // latency of the two-stage pipeline (~0.42 us measured on small tiles)
             const double eff = conv && t.bm == 256 && t.bn == 64 ? t.eff * 1.1 : t.eff;
@@ -416,6 +427,52 @@ int check_batch(int dt, int M, int N, int K, int sa, int sb, int sc, bool ta, bo
     return CKX_OK;
 }
 
+// The instance (index into the GEMM family list) and K runs a launch of a vector-aligned problem uses: the automatic
+// choice for instance == CKX_INSTANCE_AUTO, else the given instance with its own K split. Pure host logic, shared by the
+// launcher and ckx_gemm_plan(). workspace_bytes: usable workspace (0: none, or unaligned).
+struct GemmChoice
+{
+    int instance;
+    int ksplit;
+    int nk_per;
+};
+
+GemmChoice choose_gemm(int dt, int M, int N, int K, bool kmajor, int instance, long workspace_bytes, int k_batch, int batch)
+{
+    const int es = dt == ckx::DT_I8 ? 1 : 2;
+    const int nk = ((long)K * es + 127) / 128 > 0 ? (int)(((long)K * es + 127) / 128) : 1;
+    if(instance >= kNumTiles)
+        return GemmChoice{instance, 1, nk};
+    const bool ws = workspace_bytes > 0;
+    // 33..64 rows: the tile kernel wins when its C tiles fill the machine, or C tiles x K runs over a long K
+    // (64 x 4096 x 11008: 20 against 27 us; at K = 4096 the 64-row skinny instance is ahead, 11.8 against 13.0 us)
+    const bool tile64 = kmajor || (M > 32 && M <= 64 &&
+                                   ((N + 63) / 64 >= 160 ||
+                                    (ws && (long)K * es >= 8192 && make_plan(M, N, K * es, -1, workspace_bytes).ksplit > 1)));
+    // few columns and a long K: the skinny kernels have N / 16 workgroups with all of K each, the tile kernel can cut K
+    // over the CUs (fp16 32 x 1024 x 8192: 12.4 against 23.3 us, 16 rows 12.1 against 16.2, 8 rows 11.7 against 13.4)
+    // (17 rows and more: up to 4096 columns -- fp16 32 x 4096 x 11008 24.6 against 31.9 us)
+    const bool few_cols = !kmajor && M >= 8 && M <= 64 && (N + 15) / 16 < (M > 16 ? 257 : 128) && (long)K * es >= 16384 &&
+                          ws && make_plan(M, N, K * es, -1, workspace_bytes).ksplit > 1;
+    if(instance == CKX_INSTANCE_AUTO && M <= 64 && !tile64 && !few_cols && k_batch == 0 && batch == 1)
+    {
+        // (the skinny kernels read both operands K-contiguous: other layouts always take the tile kernel)
+        // A handful of rows against a big weight matrix is an HBM-streaming problem. Wider
+        // workgroups (32 / 64 columns) re-read A from L2 less often, as long as enough workgroups
+        // remain to keep every CU pulling on HBM; up to 4 rows A is too small to matter unless the columns are many.
+        // (measured: 8 x 11008 x 4096 11.5 against 12.4 us on the 64-column instance, 1 x 11008 x 4096 11.0 against
+        // 10.6; 1 and 8 x 16384 x 1024 5.5 against 8.7 / 9.4 us)
+        const int n64  = (N + 63) / 64;
+        const int wide = M <= 4 ? (n64 >= 256 ? 2 : 0) : n64 >= 160 ? 2 : (M > 8 && (N + 31) / 32 >= 160) ? 1 : 0;
+        const int ti   = kNumTiles + (M <= 16 ? (wide == 2 ? 4 : wide == 1 ? 5 : 0) : M <= 32 ? (wide == 2 ? 6 : wide == 1 ? 7 : 1) : 2);
+        return GemmChoice{ti, 1, nk};
+    }
+    // a batch multiplies the C tiles: plan for a problem with that many rows, without a K split
+    const Plan pl = batch > 1 ? make_plan((long)M * (batch < 64 ? batch : 64), N, K * es, instance, 0, 1, kmajor)
+                              : make_plan(M, N, K * es, instance, workspace_bytes, k_batch, kmajor);
+    return GemmChoice{pl.tile, pl.ksplit, pl.nk_per};
+}
+
 int run_gemm(int dt, const void* a, const void* b, void* c, int M, int N, int K, int sa, int sb, int sc,
              int al, int bl, int cl, int epi, float sg, float sr, int instance, void* ws, long ws_bytes,
              void* stream, const DOperands& dops = DOperands{}, int k_batch = 0, int batch = 1, long bsa = 0,
@@ -468,43 +525,19 @@ int run_gemm(int dt, const void* a, const void* b, void* c, int M, int N, int K,
     }
     if(misaligned)
         return fail(CKX_UNSUPPORTED, "A and B (and their batch strides) must be 16-byte aligned for this instance");
-    int ti = instance;
-    Plan pl;
-    // 33..64 rows: the tile kernel wins when its C tiles fill the machine, or C tiles x K runs over a long K
-    // (64 x 4096 x 11008: 20 against 27 us; at K = 4096 the 64-row skinny instance is ahead, 11.8 against 13.0 us)
-    const bool tile64 = kmajor || (M > 32 && M <= 64 &&
-                                   ((N + 63) / 64 >= 160 ||
-                                    (ws && !(reinterpret_cast<uintptr_t>(ws) & 15) && (long)K * es >= 8192 &&
-                                     make_plan(M, N, K * es, -1, ws_bytes).ksplit > 1)));
-    // few columns and a long K: the skinny kernels have N / 16 workgroups with all of K each, the tile kernel can cut K
-    // over the CUs (fp16 32 x 1024 x 8192: 12.4 against 23.3 us, 16 rows 12.1 against 16.2, 8 rows 11.7 against 13.4)
-    // (17 rows and more: up to 4096 columns -- fp16 32 x 4096 x 11008 24.6 against 31.9 us)
-    const bool few_cols = !kmajor && M >= 8 && M <= 64 && (N + 15) / 16 < (M > 16 ? 257 : 128) && (long)K * es >= 16384 && ws &&
-                          !(reinterpret_cast<uintptr_t>(ws) & 15) && make_plan(M, N, K * es, -1, ws_bytes).ksplit > 1;
-    if(instance == CKX_INSTANCE_AUTO && M <= 64 && !tile64 && !few_cols && k_batch == 0 && batch == 1)
+    const bool ws_ok    = ws && !(reinterpret_cast<uintptr_t>(ws) & 15);
+    const GemmChoice ch = choose_gemm(dt, M, N, K, kmajor, instance, ws_ok ? ws_bytes : 0, k_batch, batch);
+    const int ti        = ch.instance;
+    if(ti < kNumTiles)
     {
-        // (the skinny kernels read both operands K-contiguous: other layouts always take the tile kernel)
-        // A handful of rows against a big weight matrix is an HBM-streaming problem. Wider
-        // workgroups (32 / 64 columns) re-read A from L2 less often, as long as enough workgroups
-        // remain to keep every CU pulling on HBM; up to 4 rows A is too small to matter unless the columns are many.
-        // (measured: 8 x 11008 x 4096 11.5 against 12.4 us on the 64-column instance, 1 x 11008 x 4096 11.0 against
-        // 10.6; 1 and 8 x 16384 x 1024 5.5 against 8.7 / 9.4 us)
-        const int n64  = (N + 63) / 64;
-        const int wide = M <= 4 ? (n64 >= 256 ? 2 : 0) : n64 >= 160 ? 2 : (M > 8 && (N + 31) / 32 >= 160) ? 1 : 0;
-        ti = kNumTiles + (M <= 16 ? (wide == 2 ? 4 : wide == 1 ? 5 : 0) : M <= 32 ? (wide == 2 ? 6 : wide == 1 ? 7 : 1) : 2);
-    }
-    else if(instance < kNumTiles)
-    {
-        if(ws && (reinterpret_cast<uintptr_t>(ws) & 15))
+        if(ws && !ws_ok)
             return fail(CKX_INVALID_VALUE, "workspace must be 16-byte aligned");
         if(k_batch > 1 && splitk_runs(K * es, k_batch) > 1 &&
            (!ws || ws_bytes < (long)splitk_runs(K * es, k_batch) * M * N * 4))
             return fail(CKX_INVALID_VALUE, "KBatch > 1 needs a workspace of ckx_gemm_splitk_workspace_bytes()");
-        // a batch multiplies the C tiles: plan for a problem with that many rows, without a K split
-        pl = batch > 1 ? make_plan(M * (batch < 64 ? batch : 64), N, K * es, instance, 0, 1, kmajor)
-                       : make_plan(M, N, K * es, instance, ws ? ws_bytes : 0, k_batch, kmajor);
-        ti = pl.tile;
     }
+    Plan pl;
+    pl.tile = ch.instance < kNumTiles ? ch.instance : 0, pl.ksplit = ch.ksplit, pl.nk_per = ch.nk_per;
     ckx::GemmArgs g;
     std::memset(&g, 0, sizeof(g));
     g.a = a, g.b = b, g.c = c;
@@ -1033,6 +1066,63 @@ int ckx_gemm_i8(const void* a, const void* b, void* c, int32_t M, int32_t N, int
 {
     return run_gemm(ckx::DT_I8, a, b, c, M, N, K, sa, sb, sc, al, bl, cl, epilogue, scale_gemm, scale_relu,
                     instance, workspace, workspace_bytes, stream);
+}
+
+int ckx_set_forced_k_runs(int k_runs)
+{
+    const int before = force_ksplit();
+    g_force_ksplit.store(k_runs < 0 ? 0 : k_runs, std::memory_order_relaxed);
+    return before;
+}
+
+int ckx_gemm_plan(int op, int32_t M, int32_t N, int32_t K, int32_t sa, int32_t sb, int32_t sc, int al, int bl, int cl,
+                  int epilogue, int32_t batch, int64_t workspace_bytes, int* instance, int* k_runs)
+{
+    if(op != CKX_OP_GEMM_I8 && op != CKX_OP_GEMM_F16 && op != CKX_OP_GEMM_BF16)
+        return fail(CKX_INVALID_VALUE, "not a GEMM operator family");
+    if(!instance || !k_runs || batch < 1)
+        return fail(CKX_INVALID_VALUE, "bad plan query");
+    const int dt = op == CKX_OP_GEMM_I8 ? ckx::DT_I8 : op == CKX_OP_GEMM_BF16 ? ckx::DT_BF16 : ckx::DT_F16;
+    int st       = check_gemm_shape(dt, M, N, K, sa, sb, sc, al, bl, cl, epilogue, *instance);
+    if(st != CKX_OK)
+        return st;
+    const bool ta = al == CKX_COL_MAJOR, tb = bl == CKX_ROW_MAJOR;
+    if(*instance == kGenericGemmInstance ||
+       (*instance == CKX_INSTANCE_AUTO && gemm_needs_generic(dt, M, N, K, sa, sb, ta, tb, epilogue)))
+    {
+        *instance = kGenericGemmInstance, *k_runs = 1;
+        return CKX_OK;
+    }
+    const GemmChoice ch = choose_gemm(dt, M, N, K, ta || tb, *instance, workspace_bytes > 0 ? workspace_bytes : 0, 0, batch);
+    *instance = ch.instance, *k_runs = ch.ksplit;
+    return CKX_OK;
+}
+
+int ckx_conv2d_fwd_plan(int op, const ckx_conv2d_desc* d, int epilogue, int64_t workspace_bytes, int* instance, int* k_runs)
+{
+    if(!instance || !k_runs)
+        return fail(CKX_INVALID_VALUE, "bad plan query");
+    int st = check_conv(op, d, epilogue, *instance);
+    if(st != CKX_OK)
+        return st;
+    const int es = op == CKX_OP_CONV2D_FWD_I8 ? 1 : 2;
+    *k_runs      = 1;
+    if(*instance == CKX_INSTANCE_AUTO)
+    {
+        if(((long)d->C * es) % 16)
+            *instance = kConvGenericInstance;
+        else if(conv_patch_preferred(op, d, epilogue))
+            *instance = kConvPatchInstance;
+        else if(conv_pointwise_preferred(op, d, epilogue))
+            *instance = kConvPointwiseInstance;
+    }
+    if(*instance == CKX_INSTANCE_AUTO || *instance < kNumTiles)
+    {
+        const Plan pl = make_plan((long)d->N * d->Ho * d->Wo, d->K, d->Y * d->X * d->C * es, *instance,
+                                  workspace_bytes > 0 ? workspace_bytes : 0, 0, false, true);
+        *instance = pl.tile, *k_runs = pl.ksplit;
+    }
+    return CKX_OK;
 }
 
 int ckx_gemm_f16_is_supported(int32_t M, int32_t N, int32_t K, int32_t sa, int32_t sb, int32_t sc, int al,

@@ -258,6 +258,63 @@ __device__ __forceinline__ int pack4_low_bytes(int b0, int b1, int b2, int b3)
     return (int)__builtin_amdgcn_perm(hi, lo, 0x05040100u);
 }
 
+// ---- the rounded requant epilogue through a 256-byte table ---------------------------------------------------
+// y = sat8(rint(sR * relu(sat8(rint(sG * acc))))) has an integer in [0, 127] in the middle: r = clamp(rint(sG * acc),
+// 0, 127). Everything after r is a function of 128 values, tabulated once per workgroup WITH THE SAME fp32 operations
+// (requant_tail), and r itself comes out of one instruction: v_cvt_pk_u8_f32 rounds to nearest even and saturates to
+// [0, 255] (entries 128 .. 255 of the table repeat entry 127), and it ORs the byte into a third operand -- the
+// 256-byte-aligned LDS address of the table -- so that its result IS the address of the table entry. Per value: int ->
+// float, multiply, convert-and-address, one LDS byte read; the eight VALU operations of requant_rnd become three.
+// Bit-identical to requant_rnd for finite scales (the exhaustive accumulator sweep of the GPU tests drives both).
+__device__ __forceinline__ int requant_tail(int r_index, float sr)
+{
+    const float r = (float)(r_index < 127 ? r_index : 127);
+    float u       = __builtin_rintf(sr * r);
+    u             = __builtin_amdgcn_fmed3f(u, -128.0f, 127.0f);
+    return (int)u;
+}
+// fills the table at LDS byte address lut_lds (256-byte aligned); the caller provides the barrier before the first use
+__device__ __forceinline__ void requant_lut_fill(uint8_t* lut, float sr, int tid, int nthreads)
+{
+    for(int i = tid; i < 256; i += nthreads)
+        lut[i] = (uint8_t)requant_tail(i, sr);
+}
+__device__ __forceinline__ int lds_read_u8(uint32_t addr)
+{
+    int v;
+    asm volatile("ds_read_u8 %0, %1" : "=v"(v) : "v"(addr));
+    return v;
+}
+// 16 consecutive int8 outputs of one row, rounded requant through the table (the reads are inline assembly, waited for
+// here: see lds_read_b128)
+__device__ __forceinline__ void store_row16_i8_lut(int8_t* crow, int n0, int N, bool vec_ok, const i32x4 (&v)[4], float sg,
+                                                   uint32_t lut_lds, bool nt)
+{
+    int b[16];
+#pragma unroll
+    for(int t = 0; t < 4; ++t)
+#pragma unroll
+        for(int j = 0; j < 4; ++j)
+            b[t * 4 + j] = lds_read_u8(__builtin_amdgcn_cvt_pk_u8_f32(sg * (float)v[t][j], 0u, lut_lds));
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    __builtin_amdgcn_sched_barrier(0);
+    if(vec_ok && n0 + 16 <= N)
+    {
+        i32x4 pk;
+#pragma unroll
+        for(int w = 0; w < 4; ++w)
+            pk[w] = pack4_low_bytes(b[4 * w], b[4 * w + 1], b[4 * w + 2], b[4 * w + 3]);
+        store_vec(reinterpret_cast<i32x4*>(crow + n0), pk, nt);
+    }
+    else
+    {
+#pragma unroll
+        for(int e = 0; e < 16; ++e)
+            if(n0 + e < N)
+                crow[n0 + e] = (int8_t)b[e];
+    }
+}
+
 // 16 consecutive int8 outputs of one row
 template <int EPI>
 __device__ __forceinline__ void store_row16_i8(int8_t* crow, int n0, int N, bool vec_ok, const i32x4 (&v)[4],
@@ -414,7 +471,8 @@ struct GemmTile
     static constexpr int A_TILE  = BM * BKB;
     static constexpr int B_TILE  = BN * BKB;
     static constexpr int STAGE   = A_TILE + B_TILE;
-    static constexpr int LDS     = NST * STAGE;
+    static constexpr int LUT     = DT == DT_I8 ? 256 : 0; // table of the rounded requant epilogue, after the stages
+    static constexpr int LDS     = NST * STAGE + LUT;
     static constexpr int NLA     = BM * CPR / NT; // 16-byte loads per thread and K tile, A
     static constexpr int NLB     = BN * CPR / NT;
     static constexpr int LPT     = NLA + NLB;
@@ -475,6 +533,12 @@ struct GemmTile
 
         const __amdgpu_buffer_rsrc_t rsrc_a = make_rsrc(p.a, p.a_bytes);
         const __amdgpu_buffer_rsrc_t rsrc_b = make_rsrc(p.b, p.b_bytes);
+        if constexpr(DT == DT_I8)
+        {
+            // (visible to every wave after the prologue's barrier, long before the first epilogue)
+            if(p.epi == EPI_REQUANT_RND && p.ksplit == 1)
+                requant_lut_fill(smem + NST * STAGE, p.scale_relu, tid, NT);
+        }
 
         // ---- per-thread load slots -------------------------------------------------
         // slot j of this thread fills LDS row (j*NW + wave)*RPI + lane/CPR, chunk position lane%CPR
@@ -854,7 +918,8 @@ struct GemmTile
                             const i32x4 v[4] = {acc[i][g * 4], acc[i][g * 4 + 1], acc[i][g * 4 + 2],
                                                 acc[i][g * 4 + 3]};
                             if(p.epi == EPI_REQUANT_RND)
-                                store_row16_i8<EPI_REQUANT_RND>(crow, n0, p.N, vec_ok, v, p.scale_gemm, p.scale_relu, nt);
+                                store_row16_i8_lut(crow, n0, p.N, vec_ok, v, p.scale_gemm,
+                                                   (uint32_t)(uintptr_t)(lds_ptr_t)smem + (uint32_t)(NST * STAGE), nt);
                             else if(p.epi == EPI_REQUANT_CK)
                                 store_row16_i8<EPI_REQUANT_CK>(crow, n0, p.N, vec_ok, v, p.scale_gemm, p.scale_relu, nt);
                             else

@@ -325,6 +325,22 @@ int ckx_batched_gemm_softmax_gemm_f16(const void* p_a, const void* p_b0, const v
                                       int64_t batch_stride_c, float acc0_scale, int mask_out_upper_triangle,
                                       int instance, void* stream);
 
+/* ---- what a launch would use (pure host) ---------------------------------------
+ * No counterpart in the reference, whose callers time every instance themselves (profile_gemm_impl.hpp:133-209):
+ * the instance and the number of K runs that ckx_gemm_* / ckx_batched_gemm_* (op = CKX_OP_GEMM_I8 / _F16 / _BF16) or
+ * ckx_conv2d_fwd_* would use for this problem with `workspace_bytes` of 16-byte aligned workspace (0: none).
+ * *instance is in / out: CKX_INSTANCE_AUTO asks for the automatic choice, an instance index for that instance's K
+ * split. Operand addresses are taken to be 16-byte aligned (a launch sends misaligned ones to the element-granular
+ * instance). The automatic choice is a cost model; tests/golden/planner_audit.json holds what it was measured against. */
+int ckx_gemm_plan(int op, int32_t M, int32_t N, int32_t K, int32_t stride_a, int32_t stride_b, int32_t stride_c,
+                  int a_layout, int b_layout, int c_layout, int epilogue, int32_t batch, int64_t workspace_bytes,
+                  int* instance, int* k_runs);
+int ckx_conv2d_fwd_plan(int op, const ckx_conv2d_desc* desc, int epilogue, int64_t workspace_bytes, int* instance,
+                        int* k_runs);
+/* Tuning / test knob: force `k_runs` K runs (0: automatic) wherever a problem and its workspace allow the split;
+ * returns the value in force before. The initial value is the environment variable CKX_KSPLIT, read once. */
+int ckx_set_forced_k_runs(int k_runs);
+
 /* ---- timing helper --------------------------------------------------------
  * launch_and_time_kernel (include/ck/device_utility/kernel_launch.hpp:13-74):
  * `fn(user)` is called n_warmup times untimed, then n_repeat times between two

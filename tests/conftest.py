@@ -27,3 +27,14 @@ def pytest_collection_modifyitems(config, items):
     for item in items:
         if "gpu" in item.keywords:
             item.add_marker(skip)
+
+
+@pytest.fixture
+def force_k_runs():
+    """force_k_runs(n): every launch that can cuts K into n runs (the library's tuning knob); reset afterwards."""
+    from composable_kernel_amd import capi
+
+    def _set(n):
+        capi.lib().ckx_set_forced_k_runs(int(n or 0))
+    yield _set
+    capi.lib().ckx_set_forced_k_runs(0)

@@ -1,0 +1,142 @@
+#!/usr/bin/env python3
+"""Measures what the launch planner is audited against (run on the MI355X; writes planner_audit.json beside itself).
+
+    python tests/golden/make_planner_audit.py [--quick]
+
+For every problem of a grid (int8 requant and fp16 GEMMs, A row-major, B column-major, LLM-like and square shapes
+from 1 to 4096 rows; the ResNet-like conv layers of the benchmark) every instance that supports the problem is
+timed with the workspace its own plan asks for: settled clocks, 200 launches replayed from a HIP graph, HIP events.
+The file keeps microseconds per instance and the K runs the instance's plan used, so that the CPU test
+tests/test_planner.py can hold the automatic choice (ckx_gemm_plan / ckx_conv2d_fwd_plan, pure host logic) against
+the best measured instance without a GPU.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+ROOT = os.path.dirname(os.path.dirname(HERE))
+sys.path.insert(0, ROOT)
+
+GEMM_NK = [(11008, 4096), (4096, 11008), (4096, 4096), (2048, 2048), (1024, 1024), (1024, 8192), (16384, 1024)]
+GEMM_M = [1, 8, 16, 32, 48, 64, 128, 256, 512, 1024, 4096]
+# (C, K, filter, HW, stride, pad) at N = 32 and 256: the benchmark's three layers and four more ResNet-50 shapes
+CONV = [(64, 64, 3, 56, 1, 1), (256, 512, 1, 56, 2, 0), (512, 512, 3, 7, 1, 1), (128, 128, 3, 28, 1, 1),
+        (256, 256, 3, 14, 1, 1), (64, 256, 1, 56, 1, 0), (1024, 2048, 1, 14, 2, 0)]
+
+
+def time_launch(launch, steps=200, settle_ms=20.0):
+    import torch
+    launch()
+    torch.cuda.synchronize()
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g):
+        for _ in range(20):
+            launch()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    while (time.perf_counter() - t0) * 1e3 < settle_ms:
+        g.replay()
+    torch.cuda.synchronize()
+    e0.record()
+    for _ in range(steps // 20):
+        g.replay()
+    e1.record()
+    torch.cuda.synchronize()
+    return e0.elapsed_time(e1) / steps * 1e3
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--quick", action="store_true", help="a fifth of the grid (smoke run of this script)")
+    args = ap.parse_args()
+    import torch
+    import composable_kernel_amd as ck
+    from composable_kernel_amd import capi
+    L = capi.lib()
+    stream = lambda: torch.cuda.current_stream().cuda_stream
+    out = {"device": torch.cuda.get_device_name(0), "library": L.ckx_version().decode(),
+           "auto": "the automatic choice [instance, K runs] of the library that was measured, with 256 MiB of workspace on offer",
+           "protocol": "per instance: clocks settled, 200 graph-replayed launches, HIP events, microseconds",
+           "gemm": [], "conv": []}
+    n_inst = L.ckx_num_instances(capi.OP_GEMM_I8)
+    ws = torch.empty(256 << 20, dtype=torch.uint8, device="cuda")
+    grid = [(kind, M, N, K) for kind in ("i8", "f16") for (N, K) in GEMM_NK for M in GEMM_M]
+    if args.quick:
+        grid = grid[::5]
+    for kind, M, N, K in grid:
+        tdt = torch.int8 if kind == "i8" else torch.float16
+        mk = (lambda s: torch.randint(-8, 9, s, dtype=torch.int8, device="cuda")) if kind == "i8" else \
+             (lambda s: (torch.rand(s, device="cuda") * 2 - 1).to(torch.float16))
+        a, b, c = mk((M, K)), mk((N, K)), torch.empty((M, N), dtype=tdt, device="cuda")
+        cls = ck.DeviceGemmInt8 if kind == "i8" else ck.DeviceGemmF16
+        c_op = ck.RequantReluRequant(0.02, 0.4, rounded=True) if kind == "i8" else None
+        opf = capi.OP_GEMM_I8 if kind == "i8" else capi.OP_GEMM_F16
+        epi = capi.EPI_REQUANT_RND if kind == "i8" else capi.EPI_PASSTHROUGH
+        row = {"op": kind, "M": M, "N": N, "K": K, "us": {}, "k_runs": {}}
+        for inst in range(n_inst - 1):        # (the element-wise instance is never the choice for an aligned problem)
+            op = cls(inst)
+            arg = op.MakeArgumentPointer(a, b, c, M, N, K, K, K, N, None, None, c_op)
+            if not op.IsSupportedArgument(arg):
+                continue
+            need = op.GetWorkSpaceSize(arg)
+            if need > ws.numel():
+                continue
+            op.SetWorkSpacePointer(arg, ws, need)
+            _, runs = capi.gemm_plan(opf, M, N, K, epilogue=epi, workspace_bytes=need, instance=inst)
+
+            def launch(op=op, arg=arg):
+                st = op._launch(arg, stream())
+                assert st == 0, capi.last_error()
+            row["us"][str(inst)] = round(time_launch(launch), 2)
+            row["k_runs"][str(inst)] = runs
+        row["auto"] = list(capi.gemm_plan(opf, M, N, K, epilogue=epi, workspace_bytes=ws.numel()))
+        out["gemm"].append(row)
+        print(row, flush=True)
+    n_conv = L.ckx_num_instances(capi.OP_CONV2D_FWD_I8)
+    cgrid = [(kind, n, *layer) for kind in ("i8", "f16") for n in (32, 256) for layer in CONV]
+    if args.quick:
+        cgrid = cgrid[::5]
+    for kind, Nb, C_, K, f, HW, st_, pd in cgrid:
+        Ho = (HW + 2 * pd - f) // st_ + 1
+        tdt = torch.int8 if kind == "i8" else torch.float16
+        mk = (lambda s: torch.randint(-5, 6, s, dtype=torch.int8, device="cuda")) if kind == "i8" else \
+             (lambda s: (torch.rand(s, device="cuda") * 2 - 1).to(torch.float16))
+        x, w, y = mk((Nb, HW, HW, C_)), mk((K, f, f, C_)), torch.empty((Nb, Ho, Ho, K), dtype=tdt, device="cuda")
+        cls = ck.DeviceConv2dFwdInt8 if kind == "i8" else ck.DeviceConv2dFwdF16
+        c_op = ck.RequantReluRequant(0.01, 0.5, rounded=True) if kind == "i8" else None
+        opf = capi.OP_CONV2D_FWD_I8 if kind == "i8" else capi.OP_CONV2D_FWD_F16
+        epi = capi.EPI_REQUANT_RND if kind == "i8" else capi.EPI_PASSTHROUGH
+        desc = capi.Conv2dDesc(Nb, K, C_, HW, HW, f, f, Ho, Ho, st_, st_, 1, 1, pd, pd, pd, pd)
+        row = {"op": kind, "N": Nb, "C": C_, "K": K, "filter": f, "HW": HW, "stride": st_, "pad": pd, "us": {}, "k_runs": {}}
+        for inst in range(n_conv - 1):
+            op = cls(inst)
+            arg = op.MakeArgumentPointer(x, w, y, Nb, K, C_, [HW, HW], [f, f], [Ho, Ho], [st_, st_], [1, 1], [pd, pd], [pd, pd],
+                                         None, None, c_op)
+            if not op.IsSupportedArgument(arg):
+                continue
+            need = op.GetWorkSpaceSize(arg)
+            if need > ws.numel():
+                continue
+            op.SetWorkSpacePointer(arg, ws, need)
+            _, runs = capi.conv2d_fwd_plan(opf, desc, epi, need, inst)
+
+            def launch(op=op, arg=arg):
+                st = op._launch(arg, stream())
+                assert st == 0, capi.last_error()
+            row["us"][str(inst)] = round(time_launch(launch), 2)
+            row["k_runs"][str(inst)] = runs
+        row["auto"] = list(capi.conv2d_fwd_plan(opf, desc, epi, ws.numel()))
+        out["conv"].append(row)
+        print(row, flush=True)
+    path = os.path.join(ROOT, "gpurun_out", "planner_audit.json") if os.path.isdir(os.path.join(ROOT, "gpurun_out")) \
+        else os.path.join(HERE, "planner_audit.json")
+    with open(path, "w") as f:
+        json.dump(out, f, indent=0, separators=(",", ":"))
+    print("wrote", path)
+
+
+if __name__ == "__main__":
+    main()

@@ -104,7 +104,7 @@ def test_conv2d_bias_relu_golden_vectors_exact(case):
     np.testing.assert_array_equal(_conv(inp, wei, bias, resi, *args), (want - 3.0).astype(np.float16))
 
 
-def test_conv2d_bias_relu_resnet_layer_and_split_k(monkeypatch):
+def test_conv2d_bias_relu_resnet_layer_and_split_k(force_k_runs):
     """ResNet-50 3x3 layer on a reduced batch against the im2col/BLAS form, also with the K loop
     cut into runs (the second pass applies the functor)."""
     inp = uniform_f16((4, 14, 14, 256), -1, 1, 31)
@@ -113,7 +113,7 @@ def test_conv2d_bias_relu_resnet_layer_and_split_k(monkeypatch):
     resi = uniform_f16((4, 14, 14, 256), -2, 2, 34)
     ref = fast.conv2d_fwd_bias_relu_f16(inp, wei, bias, resi, (1, 1), (1, 1), (1, 1))
     _close(_conv(inp, wei, bias, resi, (1, 1), (1, 1), (1, 1)), ref)
-    monkeypatch.setenv("CKX_KSPLIT", "3")
+    force_k_runs(3)
     _close(_conv(inp, wei, bias, resi, (1, 1), (1, 1), (1, 1), workspace=True), ref)
     _close(_conv(inp, wei, bias, None, (1, 1), (1, 1), (1, 1), instance=2, workspace=True),
            fast.conv2d_fwd_bias_relu_f16(inp, wei, bias, None, (1, 1), (1, 1), (1, 1)))

@@ -64,12 +64,12 @@ def test_bf16_gemm_exact_small_integers_and_tie():
     assert np.all(fast.bf16_to_f32(_gemm(a, b_nk)) == 192.0)
 
 
-def test_bf16_gemm_full_size_and_split_k(monkeypatch):
+def test_bf16_gemm_full_size_and_split_k(force_k_runs):
     a = uniform_bf16((1024, 2048), -1, 1, 31)
     b_nk = uniform_bf16((768, 2048), -1, 1, 32)
     ref = fast.gemm_bf16(a, b_nk.T)
     _close(_gemm(a, b_nk), ref)
-    monkeypatch.setenv("CKX_KSPLIT", "4")
+    force_k_runs(4)
     _close(_gemm(a, b_nk, workspace=True), ref)
 
 

@@ -150,12 +150,12 @@ def test_layouts_position_sensitive_operands(layout):
 
 @pytest.mark.parametrize("layout", sorted(LAYOUTS))
 @pytest.mark.parametrize("kind", ["i8", "f16", "bf16"])
-def test_layouts_large_problem_and_split_k(kind, layout, monkeypatch):
+def test_layouts_large_problem_and_split_k(kind, layout, force_k_runs):
     M, N, K = 1024, 768, 2048
     a_st, b_st, a_mk, b_kn = _operands(kind, layout, M, N, K, 1300)
     c_op = ck.RequantReluRequant(0.002, 0.9, rounded=True) if kind == "i8" else None
     _check(kind, _run(kind, layout, a_st, b_st, M, N, K, c_op=c_op), a_mk, b_kn, c_op, big=True)
-    monkeypatch.setenv("CKX_KSPLIT", "4")
+    force_k_runs(4)
     _check(kind, _run(kind, layout, a_st, b_st, M, N, K, c_op=c_op, workspace=True), a_mk, b_kn, c_op, big=True)
 
 

@@ -1,0 +1,85 @@
+"""The launch planner against measurements (CPU test: ckx_gemm_plan / ckx_conv2d_fwd_plan are pure host logic).
+
+tests/golden/planner_audit.json holds, for a grid of GEMM and conv problems, the microseconds every supporting
+instance took on an MI355X with the K split of its own plan (tests/golden/make_planner_audit.py wrote it). The
+automatic choice must (1) be the choice the measured library made, problem by problem -- a known-answer table: a
+changed constant of the cost model that moves any choice fails here, and the remedy is to measure again -- and (2)
+stay close to the best measured instance: within 10 % on five problems out of six, within 45 % on every one (what
+the model achieved when the table was measured: mean regret 4 %; timings of kernels of ten microseconds carry
+several per cent of noise themselves). The reference has no such choice to compare with: its callers time every
+instance themselves (profiler/include/profile_gemm_impl.hpp:133-209)."""
+import json
+import os
+
+import pytest
+
+from composable_kernel_amd import capi
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+with open(os.path.join(HERE, "golden", "planner_audit.json")) as f:
+    AUDIT = json.load(f)
+
+WORKSPACE = 256 << 20     # what the measurements had at their disposal
+CLOSE, FAR = 1.10, 1.45
+
+
+def _gemm_choice(row):
+    op = capi.OP_GEMM_I8 if row["op"] == "i8" else capi.OP_GEMM_F16
+    epi = capi.EPI_REQUANT_RND if row["op"] == "i8" else capi.EPI_PASSTHROUGH
+    return capi.gemm_plan(op, row["M"], row["N"], row["K"], epilogue=epi, workspace_bytes=WORKSPACE)
+
+
+def _conv_choice(row):
+    op = capi.OP_CONV2D_FWD_I8 if row["op"] == "i8" else capi.OP_CONV2D_FWD_F16
+    epi = capi.EPI_REQUANT_RND if row["op"] == "i8" else capi.EPI_PASSTHROUGH
+    ho = (row["HW"] + 2 * row["pad"] - row["filter"]) // row["stride"] + 1
+    d = capi.Conv2dDesc(row["N"], row["K"], row["C"], row["HW"], row["HW"], row["filter"], row["filter"], ho, ho,
+                        row["stride"], row["stride"], 1, 1, row["pad"], row["pad"], row["pad"], row["pad"])
+    return capi.conv2d_fwd_plan(op, d, epi, WORKSPACE)
+
+
+def _ratios(rows, choose):
+    out = []
+    for row in rows:
+        inst, runs = choose(row)
+        key = str(inst)
+        label = {k: v for k, v in row.items() if k not in ("us", "k_runs")}
+        assert [inst, runs] == row["auto"], \
+            f"{label}: the planner now picks instance {inst} x {runs} K runs, the measured library picked {row['auto']}: " \
+            "measure again (tests/golden/make_planner_audit.py)"
+        assert key in row["us"], f"{label}: the planner picks instance {inst}, which the audit never measured"
+        assert row["k_runs"][key] == runs, \
+            f"{label}: instance {inst} was measured with {row['k_runs'][key]} K runs, the planner now asks for {runs}"
+        out.append((row["us"][key] / min(row["us"].values()), label, inst, runs))
+    return out
+
+
+@pytest.mark.parametrize("family", ["gemm", "conv"])
+def test_automatic_choice_is_close_to_the_best_measured_instance(family):
+    ratios = _ratios(AUDIT[family], _gemm_choice if family == "gemm" else _conv_choice)
+    assert len(ratios) >= (100 if family == "gemm" else 20)
+    worst = max(ratios, key=lambda r: r[0])
+    assert worst[0] <= FAR, f"{worst[1]}: instance {worst[2]} x {worst[3]} K runs is {worst[0]:.2f} x the best measured"
+    behind = [r for r in ratios if r[0] > CLOSE]
+    assert len(behind) <= len(ratios) // 6, \
+        f"{len(behind)} of {len(ratios)} problems more than {CLOSE:.2f} x behind the best instance: " + \
+        "; ".join(f"{r[1]} -> {r[2]} x {r[3]} ({r[0]:.2f})" for r in behind[:8])
+
+
+def test_plan_queries_validate_like_the_launchers():
+    import ctypes as C
+    L = capi.lib()
+    inst, runs = C.c_int(-1), C.c_int(0)
+    assert L.ckx_gemm_plan(capi.OP_GEMM_I8, 64, 64, 128, 64, 128, 64, 0, 1, 0, 0, 1, 0, C.byref(inst), C.byref(runs)) == capi.UNSUPPORTED
+    assert L.ckx_gemm_plan(99, 64, 64, 128, 128, 128, 64, 0, 1, 0, 0, 1, 0, C.byref(inst), C.byref(runs)) == capi.INVALID_VALUE
+    # a K that is not a whole vector: the element-wise instance, one pass
+    n = L.ckx_num_instances(capi.OP_GEMM_I8)
+    assert capi.gemm_plan(capi.OP_GEMM_I8, 64, 64, 100) == (n - 1, 1)
+    # no workspace: never more than one K run
+    assert capi.gemm_plan(capi.OP_GEMM_I8, 128, 4096, 11008, workspace_bytes=0)[1] == 1
+    # the forced-runs knob changes the plan and reports what was in force before
+    assert L.ckx_set_forced_k_runs(3) == 0
+    try:
+        assert capi.gemm_plan(capi.OP_GEMM_I8, 256, 256, 4096, workspace_bytes=WORKSPACE)[1] == 3
+    finally:
+        assert L.ckx_set_forced_k_runs(0) == 3

@@ -1,6 +1,6 @@
 """GPU parity of the split-K plans (C tiles cut into K runs, raw accumulators in a caller
 workspace, second pass sums the runs and applies the epilogue). The run count is chosen by the
-library; CKX_KSPLIT forces it here so that small problems exercise every path. int8 stays
+library; ckx_set_forced_k_runs forces it here so that small problems exercise every path. int8 stays
 bit-exact for any split (int32 partial sums); fp16 slices are added in a fixed order."""
 import os
 
@@ -18,12 +18,9 @@ pytestmark = pytest.mark.gpu
 @pytest.fixture
 def force_split():
     def _set(n):
-        if n:
-            os.environ["CKX_KSPLIT"] = str(n)
-        else:
-            os.environ.pop("CKX_KSPLIT", None)
+        capi.lib().ckx_set_forced_k_runs(int(n or 0))
     yield _set
-    os.environ.pop("CKX_KSPLIT", None)
+    capi.lib().ckx_set_forced_k_runs(0)
 
 
 def _run_gemm(op, a, b_nk, c_dtype, c_op=None):
