@@ -73,7 +73,8 @@ struct ConvPatch
     static constexpr int TAPS   = Y * X;
     static constexpr int RING_BYTES = RING * PITCH * PXB;
     static constexpr int WEI_BYTES  = TAPS * KO * PXB;
-    static constexpr int LDS        = RING_BYTES + WEI_BYTES;
+    static constexpr int LUT        = DT == DT_I8 ? 256 : 0; // table of the rounded requant epilogue, behind the weights
+    static constexpr int LDS        = RING_BYTES + WEI_BYTES + LUT;
     static constexpr int NT         = 256;
     static constexpr int NEED_ROWS  = TH + Y - 1;   // input rows of one band
     static_assert(Y >= 1 && Y <= 3 && X >= 1 && X <= 3 && MTW >= 1 && MTW <= 7, "covered shapes");
@@ -98,6 +99,12 @@ struct ConvPatch
 
         const __amdgpu_buffer_rsrc_t rsrc_in  = make_rsrc(p.in, p.in_bytes);
         const __amdgpu_buffer_rsrc_t rsrc_wei = make_rsrc(p.wei, p.wei_bytes);
+
+        if constexpr(DT == DT_I8)
+        {
+            if(p.epi == EPI_REQUANT_RND)
+                requant_lut_fill(smem + RING_BYTES + WEI_BYTES, p.scale_relu, (int)threadIdx.x, 256);
+        }
 
         // ---- weights: LDS row tap*64 + r holds output channel w_row_to_ch(r), swizzled by r & 7
         {
@@ -338,12 +345,28 @@ struct ConvPatch
                             if(TH * b + (int)rout[t] < p.Ho)
                             {
                                 int o[NBT];
+                                if constexpr(EPI == EPI_REQUANT_RND)
+                                {
+                                    i32x4 v[NBT];
 #pragma unroll
-                                for(int j = 0; j < NBT; ++j)
-                                    o[j] = pack4_low_bytes(epilogue_i8<EPI>(acc[t][j][0], p.scale_gemm, p.scale_relu),
-                                                           epilogue_i8<EPI>(acc[t][j][1], p.scale_gemm, p.scale_relu),
-                                                           epilogue_i8<EPI>(acc[t][j][2], p.scale_gemm, p.scale_relu),
-                                                           epilogue_i8<EPI>(acc[t][j][3], p.scale_gemm, p.scale_relu));
+                                    for(int j = 0; j < NBT; ++j)
+                                        v[j] = acc[t][j];
+                                    int bb[4 * NBT];
+                                    requant_lut<NBT>(v, p.scale_gemm,
+                                                     (uint32_t)(uintptr_t)(lds_ptr_t)smem + (uint32_t)(RING_BYTES + WEI_BYTES), bb);
+#pragma unroll
+                                    for(int j = 0; j < NBT; ++j)
+                                        o[j] = pack4_low_bytes(bb[4 * j], bb[4 * j + 1], bb[4 * j + 2], bb[4 * j + 3]);
+                                }
+                                else
+                                {
+#pragma unroll
+                                    for(int j = 0; j < NBT; ++j)
+                                        o[j] = pack4_low_bytes(epilogue_i8<EPI>(acc[t][j][0], p.scale_gemm, p.scale_relu),
+                                                               epilogue_i8<EPI>(acc[t][j][1], p.scale_gemm, p.scale_relu),
+                                                               epilogue_i8<EPI>(acc[t][j][2], p.scale_gemm, p.scale_relu),
+                                                               epilogue_i8<EPI>(acc[t][j][3], p.scale_gemm, p.scale_relu));
+                                }
                                 if constexpr(NBT == 4)
                                     *reinterpret_cast<i32x4*>(out_band + ooff[t]) = i32x4{o[0], o[1], o[2], o[3]};
                                 else

@@ -58,7 +58,8 @@ struct ConvPointwise
     static constexpr int MB   = 16 * MT; // pixels per band
     static constexpr int SLOT = MB * RB;
     static constexpr int D    = 9;       // ring slots; D - 2 bands are in flight ahead of the one being multiplied
-    static constexpr int LDS  = D * SLOT;
+    static constexpr int LUT  = DT == DT_I8 ? 256 : 0; // table of the rounded requant epilogue, behind the ring
+    static constexpr int LDS  = D * SLOT + LUT;
     static constexpr int NW   = 8;
     static constexpr int NT   = 64 * NW;
     static constexpr int LPW  = SLOT / 1024 / NW; // direct loads per wave and band
@@ -76,6 +77,12 @@ struct ConvPointwise
         const uint32_t frow = (uint32_t)(lane & 15), fq = (uint32_t)(lane >> 4);
         const uint32_t smem_lds = (uint32_t)(uintptr_t)(lds_ptr_t)smem;
         const __amdgpu_buffer_rsrc_t rsrc_in = make_rsrc(p.in, p.in_bytes);
+        if constexpr(DT == DT_I8)
+        {
+            // table of the rounded requant epilogue (visible after the first band's barrier)
+            if(p.epi == EPI_REQUANT_RND)
+                requant_lut_fill(smem + D * SLOT, p.scale_relu, (int)threadIdx.x, 512);
+        }
 
         // ---- the wave's weight slice. A lane ends up with MFMA rows 4q..4q+3 of each of the four tiles (q = lane / 16);
         // which channel sits in which MFMA row is free, and chosen so that a lane's values are whole 16-byte runs of
@@ -224,12 +231,24 @@ struct ConvPointwise
                         if constexpr(DT == DT_I8)
                         {
                             i32x4 pk;
+                            if constexpr(EPI == EPI_REQUANT_RND)
+                            {
+                                const i32x4 v[4] = {acc[t & 1][0], acc[t & 1][1], acc[t & 1][2], acc[t & 1][3]};
+                                int b[16];
+                                requant_lut<4>(v, p.scale_gemm, smem_lds + (uint32_t)(D * SLOT), b);
 #pragma unroll
-                            for(int tn = 0; tn < 4; ++tn)
-                                pk[tn] = pack4_low_bytes(epilogue_i8<EPI>(acc[t & 1][tn][0], p.scale_gemm, p.scale_relu),
-                                                         epilogue_i8<EPI>(acc[t & 1][tn][1], p.scale_gemm, p.scale_relu),
-                                                         epilogue_i8<EPI>(acc[t & 1][tn][2], p.scale_gemm, p.scale_relu),
-                                                         epilogue_i8<EPI>(acc[t & 1][tn][3], p.scale_gemm, p.scale_relu));
+                                for(int tn = 0; tn < 4; ++tn)
+                                    pk[tn] = pack4_low_bytes(b[4 * tn], b[4 * tn + 1], b[4 * tn + 2], b[4 * tn + 3]);
+                            }
+                            else
+                            {
+#pragma unroll
+                                for(int tn = 0; tn < 4; ++tn)
+                                    pk[tn] = pack4_low_bytes(epilogue_i8<EPI>(acc[t & 1][tn][0], p.scale_gemm, p.scale_relu),
+                                                             epilogue_i8<EPI>(acc[t & 1][tn][1], p.scale_gemm, p.scale_relu),
+                                                             epilogue_i8<EPI>(acc[t & 1][tn][2], p.scale_gemm, p.scale_relu),
+                                                             epilogue_i8<EPI>(acc[t & 1][tn][3], p.scale_gemm, p.scale_relu));
+                            }
                             store_vec(reinterpret_cast<i32x4*>(reinterpret_cast<int8_t*>(p.out) + (size_t)m * p.Kout + n0), pk, nt);
                         }
                         else

@@ -278,6 +278,7 @@ __device__ __forceinline__ void requant_lut_fill(uint8_t* lut, float sr, int tid
 {
     for(int i = tid; i < 256; i += nthreads)
         lut[i] = (uint8_t)requant_tail(i, sr);
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); // written before this wave reaches the barrier
 }
 __device__ __forceinline__ int lds_read_u8(uint32_t addr)
 {
@@ -285,19 +286,25 @@ __device__ __forceinline__ int lds_read_u8(uint32_t addr)
     asm volatile("ds_read_u8 %0, %1" : "=v"(v) : "v"(addr));
     return v;
 }
-// 16 consecutive int8 outputs of one row, rounded requant through the table (the reads are inline assembly, waited for
-// here: see lds_read_b128)
-__device__ __forceinline__ void store_row16_i8_lut(int8_t* crow, int n0, int N, bool vec_ok, const i32x4 (&v)[4], float sg,
-                                                   uint32_t lut_lds, bool nt)
+// 4 * NQ accumulators -> their 4 * NQ requantised bytes b[], through the table (the reads are inline assembly, waited
+// for here: see lds_read_b128; LDS reads return in order, so whatever else the wave has in flight is complete too)
+template <int NQ>
+__device__ __forceinline__ void requant_lut(const i32x4 (&v)[NQ], float sg, uint32_t lut_lds, int (&b)[4 * NQ])
 {
-    int b[16];
 #pragma unroll
-    for(int t = 0; t < 4; ++t)
+    for(int t = 0; t < NQ; ++t)
 #pragma unroll
         for(int j = 0; j < 4; ++j)
             b[t * 4 + j] = lds_read_u8(__builtin_amdgcn_cvt_pk_u8_f32(sg * (float)v[t][j], 0u, lut_lds));
     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
     __builtin_amdgcn_sched_barrier(0);
+}
+// 16 consecutive int8 outputs of one row, rounded requant through the table
+__device__ __forceinline__ void store_row16_i8_lut(int8_t* crow, int n0, int N, bool vec_ok, const i32x4 (&v)[4], float sg,
+                                                   uint32_t lut_lds, bool nt)
+{
+    int b[16];
+    requant_lut<4>(v, sg, lut_lds, b);
     if(vec_ok && n0 + 16 <= N)
     {
         i32x4 pk;
