@@ -3,8 +3,13 @@ oracle -- ReferenceBatchedGemm with element_wise::Scale, the upper-triangle mask
 (reference_softmax.hpp:56-117) and a second ReferenceBatchedGemm, the chain upstream's
 batched_gemm_scale_softmax_gemm example verifies with. The fused operator is absent from the reference
 snapshot; the oracle chain is pinned bit for bit against those reference pieces in tests/test_oracle.py.
-Tolerance rtol = atol = 1e-2 (the kernel rounds the probabilities to fp16 before the division by the row
-sum, the reference after it); exact where the mathematics makes it exact."""
+This row is TOLERANCE-ONLY, by construction: rtol = atol = 1e-2. The kernel rounds the unnormalised
+probabilities exp(s - max) to fp16 (they are the A operand of the second MFMA GEMM) and divides the fp32
+result by the row sum afterwards; the reference divides first and rounds the normalised probabilities. The two
+round different numbers, so outputs differ by a few fp16 units in the last place of the probabilities (relative
+2^-11 each, accumulated over n): a comparison at 1e-3 fails on a share of the elements for this reason alone,
+and no reordering inside the kernel can make the row bit-exact without giving up the fused second GEMM.
+What the mathematics fixes exactly is still checked exactly (uniform rows, one-hot rows, the masked first row)."""
 import numpy as np
 import pytest
 
