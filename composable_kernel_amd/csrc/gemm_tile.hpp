@@ -484,7 +484,11 @@ struct GemmTile
     static constexpr int A_TILE  = BM * BKB;
     static constexpr int B_TILE  = BN * BKB;
     static constexpr int STAGE   = A_TILE + B_TILE;
-    static constexpr int LUT     = DT == DT_I8 ? 256 : 0; // table of the rounded requant epilogue, after the stages
+    // table of the rounded requant epilogue, after the stages -- unless its 256 bytes would cost a co-resident
+    // workgroup (two 256 x 64 workgroups fill the 160 KB exactly: that instance keeps the arithmetic epilogue)
+    static constexpr int LDS_CU  = 160 * 1024;
+    static constexpr bool USE_LUT = DT == DT_I8 && LDS_CU / (NST * STAGE) == LDS_CU / (NST * STAGE + 256);
+    static constexpr int LUT     = USE_LUT ? 256 : 0;
     static constexpr int LDS     = NST * STAGE + LUT;
     static constexpr int NLA     = BM * CPR / NT; // 16-byte loads per thread and K tile, A
     static constexpr int NLB     = BN * CPR / NT;
@@ -546,7 +550,7 @@ struct GemmTile
 
         const __amdgpu_buffer_rsrc_t rsrc_a = make_rsrc(p.a, p.a_bytes);
         const __amdgpu_buffer_rsrc_t rsrc_b = make_rsrc(p.b, p.b_bytes);
-        if constexpr(DT == DT_I8)
+        if constexpr(USE_LUT)
         {
             // (visible to every wave after the prologue's barrier, long before the first epilogue)
             if(p.epi == EPI_REQUANT_RND && p.ksplit == 1)
@@ -929,9 +933,11 @@ struct GemmTile
                             int8_t* crow = reinterpret_cast<int8_t*>(c_batch) + (size_t)m * p.ldc;
                             const i32x4 v[4] = {acc[i][g * 4], acc[i][g * 4 + 1], acc[i][g * 4 + 2],
                                                 acc[i][g * 4 + 3]};
-                            if(p.epi == EPI_REQUANT_RND)
+                            if(p.epi == EPI_REQUANT_RND && USE_LUT)
                                 store_row16_i8_lut(crow, n0, p.N, vec_ok, v, p.scale_gemm,
                                                    (uint32_t)(uintptr_t)(lds_ptr_t)smem + (uint32_t)(NST * STAGE), nt);
+                            else if(p.epi == EPI_REQUANT_RND)
+                                store_row16_i8<EPI_REQUANT_RND>(crow, n0, p.N, vec_ok, v, p.scale_gemm, p.scale_relu, nt);
                             else if(p.epi == EPI_REQUANT_CK)
                                 store_row16_i8<EPI_REQUANT_CK>(crow, n0, p.N, vec_ok, v, p.scale_gemm, p.scale_relu, nt);
                             else
