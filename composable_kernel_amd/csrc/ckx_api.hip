@@ -313,17 +313,31 @@ struct DOperands
     int ldd0 = 0, ldd1 = 0;
 };
 
+// the fp16 add / ReLU functors with fp16 D operands; the int8 functors with a per-column fp32 scale row as D0
+bool f16_fused(int epi) { return epi >= CKX_EPI_ADD_RELU && epi <= CKX_EPI_CSHUFFLE_ADD_RELU; }
+bool per_column_scale(int epi) { return epi == CKX_EPI_MUL2_CLAMP || epi == CKX_EPI_RELU_MUL2_CLAMP; }
+
 bool epilogue_fits_dtype(int es, int epi)
 {
     if(es == 1)
-        return epi >= CKX_EPI_PASSTHROUGH && epi <= CKX_EPI_REQUANT_RND;
-    return epi == CKX_EPI_PASSTHROUGH || (epi >= CKX_EPI_ADD_RELU && epi <= CKX_EPI_CSHUFFLE_ADD_RELU);
+        return (epi >= CKX_EPI_PASSTHROUGH && epi <= CKX_EPI_REQUANT_RND) || per_column_scale(epi);
+    return epi == CKX_EPI_PASSTHROUGH || f16_fused(epi);
 }
 
 int check_d_operands(int epi, int N, const DOperands& d)
 {
     if(epi < CKX_EPI_ADD_RELU)
         return CKX_OK;
+    if(per_column_scale(epi))
+    {
+        if(!d.d0)
+            return fail(CKX_INVALID_VALUE, "null D operand pointer");
+        if(d.ldd0 != 0)
+            return fail(CKX_UNSUPPORTED, "the requant scales are one row of N floats: D0 stride 0 (broadcast over the rows)");
+        if(reinterpret_cast<uintptr_t>(d.d0) & 3)
+            return fail(CKX_UNSUPPORTED, "operands must be aligned to their element size");
+        return CKX_OK;
+    }
     if(!d.d0 || (epi == CKX_EPI_ADD_RELU_ADD && !d.d1))
         return fail(CKX_INVALID_VALUE, "null D operand pointer");
     if((d.ldd0 != 0 && d.ldd0 < N) || (epi == CKX_EPI_ADD_RELU_ADD && d.ldd1 != 0 && d.ldd1 < N) || d.ldd0 < 0 ||
@@ -338,7 +352,7 @@ bool gemm_needs_generic(int dt, int M, int N, int K, int sa, int sb, bool ta, bo
 {
     const int es = dt == ckx::DT_I8 ? 1 : 2;
     return ((long)(ta ? M : K) * es) % 16 || ((long)(tb ? N : K) * es) % 16 || ((long)sa * es) % 16 ||
-           ((long)sb * es) % 16 || ((ta || tb) && epi >= CKX_EPI_ADD_RELU);
+           ((long)sb * es) % 16 || ((ta || tb) && f16_fused(epi));
 }
 
 int check_gemm_shape(int dt, int M, int N, int K, int sa, int sb, int sc, int al, int bl, int cl, int epi,
@@ -351,7 +365,7 @@ int check_gemm_shape(int dt, int M, int N, int K, int sa, int sb, int sc, int al
         return fail(CKX_INVALID_VALUE, "no such instance");
     if(instance >= kNumTiles && instance < kGenericGemmInstance && M > kSkinny[instance - kNumTiles].max_m)
         return fail(CKX_UNSUPPORTED, "this skinny instance covers fewer rows than M");
-    if(epi < CKX_EPI_PASSTHROUGH || epi > CKX_EPI_CSHUFFLE_ADD_RELU)
+    if(epi < CKX_EPI_PASSTHROUGH || epi > CKX_EPI_RELU_MUL2_CLAMP)
         return fail(CKX_INVALID_VALUE, "unknown epilogue");
     if(!epilogue_fits_dtype(es, epi) || (dt == ckx::DT_BF16 && epi != CKX_EPI_PASSTHROUGH))
         return fail(CKX_UNSUPPORTED, "epilogue not available for this dtype");
@@ -363,7 +377,7 @@ int check_gemm_shape(int dt, int M, int N, int K, int sa, int sb, int sc, int al
     const bool ta = al == CKX_COL_MAJOR, tb = bl == CKX_ROW_MAJOR;
     // what only the element-granular instance takes (AUTO sends it there)
     const bool fast = instance != CKX_INSTANCE_AUTO && instance != kGenericGemmInstance;
-    if(fast && (ta || tb) && epi >= CKX_EPI_ADD_RELU)
+    if(fast && (ta || tb) && f16_fused(epi))
         return fail(CKX_UNSUPPORTED, "the D-operand epilogues of this instance are built for A row-major, B column-major");
     if(fast && (ta || tb) && !ckx::layout_tile(dt, instance, ta, tb))
         return fail(CKX_UNSUPPORTED, "this instance has no variant for a K-major operand (tiles of 64 rows and more do)");
@@ -504,7 +518,7 @@ int run_gemm(int dt, const void* a, const void* b, void* c, int M, int N, int K,
     {
         // element-granular instance: one pass over K whatever KBatch says (the result does not depend on the split)
         if((reinterpret_cast<uintptr_t>(a) | reinterpret_cast<uintptr_t>(b) | reinterpret_cast<uintptr_t>(c) |
-            reinterpret_cast<uintptr_t>(dops.d0) | reinterpret_cast<uintptr_t>(dops.d1)) & (es - 1))
+            (f16_fused(epi) ? reinterpret_cast<uintptr_t>(dops.d0) | reinterpret_cast<uintptr_t>(dops.d1) : 0)) & (es - 1))
             return fail(CKX_UNSUPPORTED, "operands must be aligned to their element size");
         ckx::GemmArgs g;
         std::memset(&g, 0, sizeof(g));
@@ -566,7 +580,7 @@ int run_gemm(int dt, const void* a, const void* b, void* c, int M, int N, int K,
     g.ksplit     = pl.ksplit;
     g.nk_per     = pl.nk_per;
     g.ws         = ws;
-    const bool fused            = epi >= CKX_EPI_ADD_RELU && g.ksplit == 1; // (after a K split the second pass applies it)
+    const bool fused            = f16_fused(epi) && g.ksplit == 1; // (after a K split the second pass applies it)
     const tile_launch_fn launch = kmajor               ? ckx::layout_tile(dt, ti, ta, tb)
                                   : dt == ckx::DT_I8   ? t.dense_i8
                                   : dt == ckx::DT_BF16 ? t.dense_bf16
@@ -659,7 +673,7 @@ int check_conv(int op, const ckx_conv2d_desc* d, int epi, int instance)
     const int es = op == CKX_OP_CONV2D_FWD_I8 ? 1 : 2;
     if(instance != CKX_INSTANCE_AUTO && (instance < 0 || instance >= kNumConvInsts))
         return fail(CKX_INVALID_VALUE, "no such instance");
-    if(epi < CKX_EPI_PASSTHROUGH || epi > CKX_EPI_CSHUFFLE_ADD_RELU || !epilogue_fits_dtype(es, epi) ||
+    if(epi < CKX_EPI_PASSTHROUGH || epi > CKX_EPI_RELU_MUL2_CLAMP || !epilogue_fits_dtype(es, epi) ||
        epi == CKX_EPI_CSHUFFLE_ADD_RELU)
         return fail(CKX_INVALID_VALUE, "epilogue not available for this operator");
     if(d->N < 0 || d->K < 0 || d->C < 0 || d->Hi <= 0 || d->Wi <= 0 || d->Y <= 0 || d->X <= 0 ||
@@ -730,7 +744,7 @@ int run_conv(int op, const void* in, const void* wei, void* out, const ckx_conv2
     if(instance == kConvGenericInstance || (instance == CKX_INSTANCE_AUTO && (misaligned || ((long)d->C * es) % 16)))
     {
         if((reinterpret_cast<uintptr_t>(in) | reinterpret_cast<uintptr_t>(wei) | reinterpret_cast<uintptr_t>(out) |
-            reinterpret_cast<uintptr_t>(dops.d0) | reinterpret_cast<uintptr_t>(dops.d1)) & (es - 1))
+            (f16_fused(epi) ? reinterpret_cast<uintptr_t>(dops.d0) | reinterpret_cast<uintptr_t>(dops.d1) : 0)) & (es - 1))
             return fail(CKX_UNSUPPORTED, "operands must be aligned to their element size");
         ckx::GemmArgs g;
         std::memset(&g, 0, sizeof(g));
@@ -830,7 +844,7 @@ int run_conv(int op, const void* in, const void* wei, void* out, const ckx_conv2
     g.ksplit = pl.ksplit;
     g.nk_per = pl.nk_per;
     g.ws     = ws;
-    const bool fused = epi >= CKX_EPI_ADD_RELU && g.ksplit == 1;
+    const bool fused = f16_fused(epi) && g.ksplit == 1;
     hipError_t e     = (es == 1 ? t.conv_i8 : fused ? t.conv_f16_fused : t.conv_f16)(g, g.tiles_m * g.tiles_n * g.ksplit,
                                                                                  (hipStream_t)stream);
     if(e == hipSuccess && g.ksplit > 1)
@@ -1052,6 +1066,8 @@ const char* ckx_instance_name(int op, int instance)
 int ckx_gemm_i8_is_supported(int32_t M, int32_t N, int32_t K, int32_t sa, int32_t sb, int32_t sc, int al,
                              int bl, int cl, int epilogue, int instance)
 {
+    if(per_column_scale(epilogue))
+        return fail(CKX_UNSUPPORTED, "epilogues with a scale row as D operand go through ckx_gemm_i8_multiple_d");
     return check_gemm_shape(ckx::DT_I8, M, N, K, sa, sb, sc, al, bl, cl, epilogue, instance);
 }
 
@@ -1263,6 +1279,44 @@ int ckx_gemm_f16_multiple_d(const void* a, const void* b, const void* d0, const 
     DOperands d;
     d.d0 = d0, d.d1 = d1, d.ldd0 = sd0, d.ldd1 = sd1;
     return run_gemm(ckx::DT_F16, a, b, e, M, N, K, sa, sb, se, al, bl, el, cde_op, 1.0f, 1.0f, instance, workspace,
+                    workspace_bytes, stream, d);
+}
+
+int ckx_gemm_i8_multiple_d_is_supported(int32_t M, int32_t N, int32_t K, int32_t sa, int32_t sb, int32_t sd0,
+                                        int32_t se, int al, int bl, int el, int cde_op, int instance)
+{
+    if(!per_column_scale(cde_op))
+        return fail(CKX_INVALID_VALUE, "not a CDE element-wise operation of the int8 family");
+    int st = check_gemm_shape(ckx::DT_I8, M, N, K, sa, sb, se, al, bl, el, cde_op, instance);
+    if(st != CKX_OK)
+        return st;
+    static const float probe = 0.0f; // only the stride is under test here
+    DOperands d;
+    d.d0 = &probe, d.ldd0 = sd0;
+    return check_d_operands(cde_op, N, d);
+}
+
+int ckx_gemm_i8_multiple_d(const void* a, const void* b, const void* d0, void* e, int32_t M, int32_t N, int32_t K,
+                           int32_t sa, int32_t sb, int32_t sd0, int32_t se, int al, int bl, int el, int cde_op,
+                           int instance, void* workspace, int64_t workspace_bytes, void* stream)
+{
+    if(!per_column_scale(cde_op))
+        return fail(CKX_INVALID_VALUE, "not a CDE element-wise operation of the int8 family");
+    DOperands d;
+    d.d0 = d0, d.ldd0 = sd0;
+    return run_gemm(ckx::DT_I8, a, b, e, M, N, K, sa, sb, se, al, bl, el, cde_op, 1.0f, 1.0f, instance, workspace,
+                    workspace_bytes, stream, d);
+}
+
+int ckx_conv2d_fwd_i8_multiple_d(const void* in, const void* wei, const void* scale, void* out,
+                                 const ckx_conv2d_desc* desc, int out_op, int instance, void* workspace,
+                                 int64_t workspace_bytes, void* stream)
+{
+    if(!per_column_scale(out_op))
+        return fail(CKX_INVALID_VALUE, "not a per-channel requant output operation");
+    DOperands d;
+    d.d0 = scale, d.ldd0 = 0;
+    return run_conv(CKX_OP_CONV2D_FWD_I8, in, wei, out, desc, out_op, 1.0f, 1.0f, instance, workspace,
                     workspace_bytes, stream, d);
 }
 

@@ -207,9 +207,11 @@ __global__ __launch_bounds__(256) void gemm_generic_kernel(const GemmArgs p, con
                 if constexpr(DT == DT_I8)
                 {
                     const int v = acc[i][t][j];
-                    const int o = p.epi == EPI_REQUANT_RND  ? requant_rnd(v, p.scale_gemm, p.scale_relu)
-                                  : p.epi == EPI_REQUANT_CK ? requant_ck(v, p.scale_gemm, p.scale_relu)
-                                                            : v;
+                    const int o = epi_per_column_scale(p.epi)
+                                      ? mul2_clamp(v, reinterpret_cast<const float*>(p.d0)[n], p.epi == EPI_RELU_MUL2_CLAMP)
+                                  : p.epi == EPI_REQUANT_RND ? requant_rnd(v, p.scale_gemm, p.scale_relu)
+                                  : p.epi == EPI_REQUANT_CK  ? requant_ck(v, p.scale_gemm, p.scale_relu)
+                                                             : v;
                     reinterpret_cast<int8_t*>(p.c)[ci] = (int8_t)o;
                 }
                 else if constexpr(DT == DT_BF16)

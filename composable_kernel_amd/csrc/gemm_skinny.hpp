@@ -135,11 +135,21 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(const GemmArgs p)
         if constexpr(DT == DT_I8)
         {
             int b[4];
+            if(epi_per_column_scale(p.epi))
+            {
+                const float* sc = reinterpret_cast<const float*>(p.d0);
 #pragma unroll
-            for(int j = 0; j < 4; ++j)
-                b[j] = p.epi == EPI_REQUANT_RND  ? requant_rnd(s[j], p.scale_gemm, p.scale_relu)
-                       : p.epi == EPI_REQUANT_CK ? requant_ck(s[j], p.scale_gemm, p.scale_relu)
-                                                 : s[j];
+                for(int j = 0; j < 4; ++j)
+                    b[j] = nn + j < p.N ? mul2_clamp(s[j], sc[nn + j], p.epi == EPI_RELU_MUL2_CLAMP) : 0;
+            }
+            else
+            {
+#pragma unroll
+                for(int j = 0; j < 4; ++j)
+                    b[j] = p.epi == EPI_REQUANT_RND  ? requant_rnd(s[j], p.scale_gemm, p.scale_relu)
+                           : p.epi == EPI_REQUANT_CK ? requant_ck(s[j], p.scale_gemm, p.scale_relu)
+                                                     : s[j];
+            }
             int8_t* crow = reinterpret_cast<int8_t*>(p.c) + (size_t)m * p.ldc + nn;
             if(nn + 4 <= p.N && ((reinterpret_cast<uintptr_t>(crow)) & 3u) == 0)
                 *reinterpret_cast<int*>(crow) = pack4_low_bytes(b[0], b[1], b[2], b[3]);

@@ -56,8 +56,13 @@ enum
     // fp16 outputs with extra "D" operands (bias row / residual tensor), all arithmetic in fp32:
     EPI_ADD_RELU          = 3, // e = half(relu(acc + d0))
     EPI_ADD_RELU_ADD      = 4, // e = half(relu(acc + d0) + d1)
-    EPI_CSHUFFLE_ADD_RELU = 5  // e = relu(half(half(acc) + d0)): C rounded to fp16 before the functor
+    EPI_CSHUFFLE_ADD_RELU = 5, // e = relu(half(half(acc) + d0)): C rounded to fp16 before the functor
+    // int8 outputs with a per-column fp32 requant scale as the "D" operand (d0 = scale[N]): upstream's
+    // element_wise::Activation_Mul2_Clamp<PassThrough / Relu>, e = int8(clamp(scale[n] * act(float(acc)), -128, 127))
+    EPI_MUL2_CLAMP      = 6,
+    EPI_RELU_MUL2_CLAMP = 7
 };
+__host__ __device__ constexpr bool epi_per_column_scale(int epi) { return epi == EPI_MUL2_CLAMP || epi == EPI_RELU_MUL2_CLAMP; }
 
 // C tile stores: plain, or streaming (non-temporal) when the output is too large to be worth
 // keeping in L2: dirty lines of a streamed output otherwise queue up behind the write-back
@@ -245,6 +250,15 @@ __device__ __forceinline__ int requant_rnd(int acc, float sg, float sr)
     return (int)u;
 }
 
+// Activation_Mul2_Clamp: the activation runs on the converted accumulator (ReLU of an integer-valued float is the
+// float of max(acc, 0)), one fp32 multiply by the column's scale, clamp, truncation toward zero (type_convert<int8_t>)
+__device__ __forceinline__ int mul2_clamp(int acc, float scale, bool relu)
+{
+    const float x = (float)(relu && acc < 0 ? 0 : acc);
+    const float y = __builtin_amdgcn_fmed3f(scale * x, -128.0f, 127.0f);
+    return (int)y;
+}
+
 template <int EPI>
 __device__ __forceinline__ int epilogue_i8(int acc, float sg, float sr)
 {
@@ -354,6 +368,41 @@ __device__ __forceinline__ void store_row16_i8(int8_t* crow, int n0, int N, bool
             if(n0 + e < N)
                 crow[n0 + e] = (int8_t)b[e];
     }
+}
+
+// 16 consecutive int8 outputs of one row under per-column scales sc[0..15] (columns n0 .. n0 + 15)
+__device__ __forceinline__ void store_row16_i8_cols(int8_t* crow, int n0, int N, bool vec_ok, const i32x4 (&v)[4],
+                                                    const float (&sc)[16], bool relu, bool nt = false)
+{
+    int b[16];
+#pragma unroll
+    for(int t = 0; t < 4; ++t)
+#pragma unroll
+        for(int j = 0; j < 4; ++j)
+            b[t * 4 + j] = mul2_clamp(v[t][j], sc[t * 4 + j], relu);
+    if(vec_ok && n0 + 16 <= N)
+    {
+        i32x4 pk;
+#pragma unroll
+        for(int w = 0; w < 4; ++w)
+            pk[w] = pack4_low_bytes(b[4 * w], b[4 * w + 1], b[4 * w + 2], b[4 * w + 3]);
+        store_vec(reinterpret_cast<i32x4*>(crow + n0), pk, nt);
+    }
+    else
+    {
+#pragma unroll
+        for(int e = 0; e < 16; ++e)
+            if(n0 + e < N)
+                crow[n0 + e] = (int8_t)b[e];
+    }
+}
+
+// the 16 scales of columns n0 .. n0 + 15 (zeros past N: a bounds-checked buffer read, no alignment beyond a float's)
+__device__ __forceinline__ void load_col_scales(const __amdgpu_buffer_rsrc_t& rs, int n0, float (&sc)[16])
+{
+#pragma unroll
+    for(int e = 0; e < 16; ++e)
+        sc[e] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(rs, (n0 + e) * 4, 0, 0));
 }
 
 // The fused add epilogues of the fp16 path (element-wise functors AddRelu / AddReluAdd of
@@ -900,6 +949,39 @@ struct GemmTile
             acc_t* slice = reinterpret_cast<acc_t*>(reinterpret_cast<uint8_t*>(p.ws) +
                                                     (size_t)(unit / ntiles_all) * p.M * p.N * 4);
             uint8_t* c_batch = reinterpret_cast<uint8_t*>(p.c) + (size_t)bi * p.bsc * ES;
+            // Per-column requant scales: a loop nest of its own, column group outermost, so that the 16 scales of the
+            // lane's columns are fetched once per group and before that group's stores (a load issued after a store
+            // waits for it) and only 16 registers hold them.
+            if constexpr(DT == DT_I8)
+            {
+                if(epi_per_column_scale(p.epi) && p.ksplit == 1)
+                {
+                    const __amdgpu_buffer_rsrc_t rs = make_rsrc(p.d0, (uint32_t)p.N * 4u);
+                    const bool relu                 = p.epi == EPI_RELU_MUL2_CLAMP;
+#pragma unroll
+                    for(int g = 0; g < NG; ++g)
+                    {
+                        const int n0 = tn * BN + wn * WTN + 64 * g + 16 * (lane >> 4);
+                        float sc[16];
+                        load_col_scales(rs, n0, sc);
+#pragma unroll
+                        for(int i = 0; i < MT; ++i)
+                        {
+                            const int m = tm * BM + wm * WTM + 16 * i + (lane & 15);
+                            if(m < p.M && n0 < p.N)
+                            {
+                                const i32x4 v[4] = {acc[i][g * 4], acc[i][g * 4 + 1], acc[i][g * 4 + 2], acc[i][g * 4 + 3]};
+                                store_row16_i8_cols(reinterpret_cast<int8_t*>(c_batch) + (size_t)m * p.ldc, n0, p.N, vec_ok,
+                                                    v, sc, relu, nt);
+                            }
+#pragma unroll
+                            for(int t = 0; t < 4; ++t)
+                                acc[i][g * 4 + t] = acc_t{0, 0, 0, 0};
+                        }
+                    }
+                    return;
+                }
+            }
 #pragma unroll
             for(int i = 0; i < MT; ++i)
             {
@@ -1223,7 +1305,13 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(const GemmArgs p)
     if constexpr(DT == DT_I8)
     {
         int8_t* crow = reinterpret_cast<int8_t*>(p.c) + (size_t)m * p.ldc;
-        if(p.epi == EPI_REQUANT_RND)
+        if(epi_per_column_scale(p.epi))
+        {
+            float sc[16];
+            load_col_scales(make_rsrc(p.d0, (uint32_t)p.N * 4u), n0, sc);
+            store_row16_i8_cols(crow, n0, p.N, vec_ok, v, sc, p.epi == EPI_RELU_MUL2_CLAMP);
+        }
+        else if(p.epi == EPI_REQUANT_RND)
             store_row16_i8<EPI_REQUANT_RND>(crow, n0, p.N, vec_ok, v, p.scale_gemm, p.scale_relu);
         else if(p.epi == EPI_REQUANT_CK)
             store_row16_i8<EPI_REQUANT_CK>(crow, n0, p.N, vec_ok, v, p.scale_gemm, p.scale_relu);

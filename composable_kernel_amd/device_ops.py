@@ -63,6 +63,25 @@ class AddReluAdd:
     cde_epilogue = capi.EPI_ADD_RELU_ADD
 
 
+class Relu:
+    """element_wise::Relu (unary_element_wise_operation.hpp): y = x > 0 ? x : 0"""
+
+
+class ActivationMul2Clamp:
+    """element_wise::Activation_Mul2_Clamp<Activation> of upstream Composable Kernel
+    (ck/tensor_operation/gpu/element/quantization_operation.hpp as shipped with ROCm; newer than the reference
+    snapshot): y = int8(clamp(requant_scale * activation(float(x)), -128, 127)) with one requant scale per output
+    column / output channel, passed as the D operand. Activation is PassThrough or Relu."""
+
+    def __init__(self, activation=None):
+        activation = activation or PassThrough()
+        if not isinstance(activation, (PassThrough, Relu)):
+            raise TypeError("activation not built")
+        self.activation = activation
+        self.epilogue = self.cde_epilogue = (capi.EPI_RELU_MUL2_CLAMP if isinstance(activation, Relu)
+                                             else capi.EPI_MUL2_CLAMP)
+
+
 class RowMajor:
     code = capi.ROW_MAJOR
 
@@ -358,6 +377,43 @@ class DeviceGemmMultipleDF16(BaseOperator):
             a.workspace_bytes_, C.c_void_p(stream or 0))
 
 
+class DeviceGemmMultipleDInt8(BaseOperator):
+    """DeviceGemmMultipleD<ALayout, BLayout, Row, int8_t, int8_t, Tuple<float>, int8_t, PassThrough, PassThrough,
+    Activation_Mul2_Clamp<Act>> (device_gemm_multiple_d.hpp:14-55): E = cde_op(A*B, D0) with D0 one row of N fp32
+    requant scales (stride 0: broadcast over the rows), the per-channel int8 requantisation."""
+    op_family = capi.OP_GEMM_I8
+
+    def __init__(self, instance=capi.INSTANCE_AUTO, ALayout=RowMajor, BLayout=ColumnMajor, DELayout=RowMajor):
+        super().__init__(instance)
+        self.layouts = (ALayout.code, BLayout.code, DELayout.code)
+
+    def MakeArgumentPointer(self, p_a, p_b, p_ds, p_e, M, N, K, StrideA, StrideB, StrideDs, StrideE,
+                            a_element_op=None, b_element_op=None, cde_element_op=None):
+        if len(p_ds) != 1 or len(StrideDs) != 1:
+            raise ValueError("one D tensor: the row of requant scales")
+        if not isinstance(cde_element_op, ActivationMul2Clamp):
+            raise TypeError("CDE element-wise operation not built")
+        a = _GemmArgument(p_a, p_b, p_e, M, N, K, StrideA, StrideB, StrideE, a_element_op or PassThrough(),
+                          b_element_op or PassThrough(), cde_element_op, self.layouts)
+        a.p_ds = [_ptr(p_ds[0])]
+        a.StrideDs = [int(StrideDs[0])]
+        return a
+
+    def _supported(self, a):
+        return capi.lib().ckx_gemm_i8_multiple_d_is_supported(
+            a.M, a.N, a.K, a.StrideA, a.StrideB, a.StrideDs[0], a.StrideC, *self.layouts, a.c_op.cde_epilogue,
+            self.instance)
+
+    def GetWorkSpaceSize(self, a):
+        return int(capi.lib().ckx_gemm_i8_workspace_bytes(a.M, a.N, a.K, self.instance))
+
+    def _launch(self, a, stream):
+        return capi.lib().ckx_gemm_i8_multiple_d(
+            a.p_a, a.p_b, a.p_ds[0], a.p_c, a.M, a.N, a.K, a.StrideA, a.StrideB, a.StrideDs[0], a.StrideC,
+            *self.layouts, a.c_op.cde_epilogue, self.instance, a.p_workspace_ or 0, a.workspace_bytes_,
+            C.c_void_p(stream or 0))
+
+
 # -------------------------------------------------------------------- conv
 class _ConvArgument(BaseArgument):
     def __init__(self, p_in, p_wei, p_out, desc, out_op):
@@ -397,6 +453,25 @@ class DeviceConv2dFwdInt8(_DeviceConvFwd):
         return capi.lib().ckx_conv2d_fwd_i8(a.p_in, a.p_wei, a.p_out, C.byref(a.desc), a.out_op.epilogue,
                                             a.out_op.scale_gemm, a.out_op.scale_relu, self.instance,
                                             a.p_workspace_ or 0, a.workspace_bytes_, C.c_void_p(stream or 0))
+
+
+class DeviceConv2dFwdMultipleDInt8(_DeviceConvFwd):
+    """2-D conv forward, int8, with one fp32 requant scale per output channel as the D operand and
+    Activation_Mul2_Clamp<Act> as the output operation (upstream's per-channel conv quantisation; the
+    DeviceConvFwd argument list of device_conv_fwd.hpp:18-39 with the scale pointer after p_out)."""
+    op_family = capi.OP_CONV2D_FWD_I8
+
+    def MakeArgumentPointer(self, p_in, p_wei, p_out, p_scale, *rest):
+        if not isinstance(rest[-1], ActivationMul2Clamp):
+            raise TypeError("output operation not built")
+        a = super().MakeArgumentPointer(p_in, p_wei, p_out, *rest)
+        a.p_scale = _ptr(p_scale)
+        return a
+
+    def _launch(self, a, stream):
+        return capi.lib().ckx_conv2d_fwd_i8_multiple_d(a.p_in, a.p_wei, a.p_scale, a.p_out, C.byref(a.desc),
+                                                       a.out_op.epilogue, self.instance, a.p_workspace_ or 0,
+                                                       a.workspace_bytes_, C.c_void_p(stream or 0))
 
 
 class DeviceConv2dFwdF16(_DeviceConvFwd):

@@ -139,6 +139,35 @@ struct AddReluAdd
     }
 };
 
+// y = x > 0 ? x : 0 (unary_element_wise_operation.hpp, Relu)
+struct Relu
+{
+    template <typename T>
+    void operator()(T& y, const T& x) const
+    {
+        y = x > T(0) ? x : T(0);
+    }
+};
+
+// Per-channel requantisation of an int32 accumulator: upstream Composable Kernel's Activation_Mul2_Clamp<Activation>
+// (ck/tensor_operation/gpu/element/quantization_operation.hpp as shipped with ROCm; newer than the reference
+// snapshot). requantScale is the D operand: one fp32 value per output column / output channel.
+//   y = float(x); y = activation(y); y = clamp(requantScale * y, -128, 127); e = int8(y)  (toward zero)
+template <typename Activation>
+struct Activation_Mul2_Clamp
+{
+    Activation_Mul2_Clamp(Activation activationOp = {}) : activationOp_(activationOp) {}
+    void operator()(int8_t& y, const int32_t& x, const float& requantScale) const
+    {
+        float f = static_cast<float>(x);
+        activationOp_(f, f);
+        f = requantScale * f;
+        f = f < -128.f ? -128.f : f > 127.f ? 127.f : f;
+        y = static_cast<int8_t>(f);
+    }
+    Activation activationOp_;
+};
+
 } // namespace element_wise
 } // namespace tensor_operation
 
@@ -961,6 +990,80 @@ struct DeviceGemmMultipleDMfma
         const std::string base = instance_ == CKX_INSTANCE_AUTO ? std::string("DeviceGemm_f16_f16_f16_mk_nk_mn<auto>")
                                                                 : std::string(ckx_instance_name(CKX_OP_GEMM_F16, instance_));
         return base + (is_add_relu ? " + AddRelu" : " + AddReluAdd");
+    }
+    int instance_;
+};
+
+// ------------------------------------------------ int8 GEMM with one requant scale per output column
+// DeviceGemmMultipleD<..., int8_t, int8_t, Tuple<float>, int8_t, PassThrough, PassThrough,
+// Activation_Mul2_Clamp<Activation>> (device_gemm_multiple_d.hpp:14-55): D0 is a row of N floats, stride 0.
+template <typename ALayout, typename BLayout, typename DELayout, typename Activation>
+struct DeviceGemmMultipleDInt8Mfma
+    : public DeviceGemmMultipleD<ALayout, BLayout, DELayout, int8_t, int8_t, Tuple<float>, int8_t,
+                                 element_wise::PassThrough, element_wise::PassThrough,
+                                 element_wise::Activation_Mul2_Clamp<Activation>>
+{
+    static constexpr bool is_relu = std::is_same_v<Activation, element_wise::Relu>;
+    static_assert(is_relu || std::is_same_v<Activation, element_wise::PassThrough>, "built activations: PassThrough, Relu");
+    static constexpr int cde_code = is_relu ? CKX_EPI_RELU_MUL2_CLAMP : CKX_EPI_MUL2_CLAMP;
+    using Pass                    = element_wise::PassThrough;
+    using CDEOp                   = element_wise::Activation_Mul2_Clamp<Activation>;
+
+    struct Argument : public BaseArgument
+    {
+        const void *p_a, *p_b, *p_d0;
+        void* p_e;
+        index_t M, N, K, StrideA, StrideB, StrideD0, StrideE;
+    };
+    static int Supported(const Argument& a, int inst)
+    {
+        return ckx_gemm_i8_multiple_d_is_supported(a.M, a.N, a.K, a.StrideA, a.StrideB, a.StrideD0, a.StrideE,
+                                                   ALayout::code, BLayout::code, DELayout::code, cde_code, inst);
+    }
+    static int Launch(const Argument& a, int inst, void* stream)
+    {
+        const int64_t ws_bytes = a.p_workspace_ ? ckx_gemm_i8_workspace_bytes(a.M, a.N, a.K, inst) : 0;
+        return ckx_gemm_i8_multiple_d(a.p_a, a.p_b, a.p_d0, a.p_e, a.M, a.N, a.K, a.StrideA, a.StrideB, a.StrideD0,
+                                      a.StrideE, ALayout::code, BLayout::code, DELayout::code, cde_code, inst,
+                                      a.p_workspace_, ws_bytes, stream);
+    }
+    using Invoker = detail::InvokerT<Argument, &Supported, &Launch>;
+
+    explicit DeviceGemmMultipleDInt8Mfma(int instance = CKX_INSTANCE_AUTO) : instance_(instance) {}
+    static Argument MakeArgument(const void* p_a, const void* p_b, std::array<const void*, 1> p_ds, void* p_e,
+                                 index_t M, index_t N, index_t K, index_t StrideA, index_t StrideB,
+                                 std::array<index_t, 1> StrideDs, index_t StrideE, Pass = {}, Pass = {}, CDEOp = {})
+    {
+        Argument a;
+        a.p_a = p_a, a.p_b = p_b, a.p_d0 = p_ds[0], a.p_e = p_e;
+        a.M = M, a.N = N, a.K = K, a.StrideA = StrideA, a.StrideB = StrideB, a.StrideD0 = StrideDs[0], a.StrideE = StrideE;
+        return a;
+    }
+    Invoker MakeInvoker() const { return Invoker{instance_}; }
+    bool IsSupportedArgument(const Argument& a) const { return Supported(a, instance_) == CKX_OK; }
+    bool IsSupportedArgument(const BaseArgument* p) override
+    {
+        const auto* a = dynamic_cast<const Argument*>(p);
+        return a && IsSupportedArgument(*a);
+    }
+    size_t GetWorkSpaceSize(const BaseArgument* p) const override
+    {
+        const auto* a = dynamic_cast<const Argument*>(p);
+        return a ? (size_t)ckx_gemm_i8_workspace_bytes(a->M, a->N, a->K, instance_) : 0;
+    }
+    std::unique_ptr<BaseArgument>
+    MakeArgumentPointer(const void* p_a, const void* p_b, std::array<const void*, 1> p_ds, void* p_e, index_t M,
+                        index_t N, index_t K, index_t StrideA, index_t StrideB, std::array<index_t, 1> StrideDs,
+                        index_t StrideE, Pass, Pass, CDEOp) override
+    {
+        return std::make_unique<Argument>(MakeArgument(p_a, p_b, p_ds, p_e, M, N, K, StrideA, StrideB, StrideDs, StrideE));
+    }
+    std::unique_ptr<BaseInvoker> MakeInvokerPointer() override { return std::make_unique<Invoker>(instance_); }
+    std::string GetTypeString() const override
+    {
+        const std::string base = instance_ == CKX_INSTANCE_AUTO ? std::string("DeviceGemm_i8_i8_i8_mk_nk_mn<auto>")
+                                                                : std::string(ckx_instance_name(CKX_OP_GEMM_I8, instance_));
+        return base + (is_relu ? " + Relu_Mul2_Clamp" : " + Mul2_Clamp");
     }
     int instance_;
 };

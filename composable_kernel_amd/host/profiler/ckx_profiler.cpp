@@ -624,6 +624,58 @@ int profile_gemm_bias_relu(int argc, char* argv[])
         de, (std::size_t)M * se, flop, bytes, verify, time_kernel, nrepeat);
 }
 
+// gemm_perchannel_quant <verify> <init> <log> <time> M N K StrideA StrideB StrideE [activation: 0 PassThrough, 1 Relu] [nrepeat]
+// int8 A[m,k] * B[n,k] with one fp32 requant scale per output column (the D operand) and Activation_Mul2_Clamp
+template <typename Act>
+int profile_gemm_perchannel_quant_t(bool verify, int init, bool time_kernel, int M, int N, int K, int sa, int sb, int se,
+                                    int nrepeat)
+{
+    using T        = int8_t;
+    using CDE      = element_wise::Activation_Mul2_Clamp<Act>;
+    using DeviceOp = device::DeviceGemmMultipleD<Row, Col, Row, T, T, ck::Tuple<float>, T, Pass, Pass, CDE>;
+    std::vector<std::unique_ptr<DeviceOp>> ops;
+    for(int i = 0; i < ckx_num_instances(CKX_OP_GEMM_I8); ++i)
+        ops.push_back(std::make_unique<device::DeviceGemmMultipleDInt8Mfma<Row, Col, Row, Act>>(i));
+    std::vector<T> a((std::size_t)M * sa), b((std::size_t)N * sb);
+    fill(a, init, 0xC0FFEE, false);
+    fill(b, init, 0xC0FFEE + 1, false);
+    std::vector<float> scale((std::size_t)N);
+    for(int n = 0; n < N; ++n) // a different, exactly representable scale per column, both signs
+        scale[n] = (float)((n * 37) % 61 - 20) / 256.0f;
+    ckx::DeviceMem da(a.size()), db(b.size()), dd(scale.size() * sizeof(float)), de((std::size_t)M * se);
+    da.ToDevice(a.data());
+    db.ToDevice(b.data());
+    dd.ToDevice(scale.data());
+    const double flop = 2.0 * M * N * K, bytes = (double)M * K + (double)K * N + (double)M * N + 4.0 * N;
+    return run_family<T>(
+        ops,
+        [&](DeviceOp& op) {
+            return op.MakeArgumentPointer(da.GetDeviceBuffer(), db.GetDeviceBuffer(), {dd.GetDeviceBuffer()},
+                                          de.GetDeviceBuffer(), M, N, K, sa, sb, {0}, se, Pass{}, Pass{}, CDE{});
+        },
+        de, (std::size_t)M * se, flop, bytes, verify, time_kernel, nrepeat);
+}
+
+int profile_gemm_perchannel_quant(int argc, char* argv[])
+{
+    if(argc < 9)
+    {
+        std::printf("arg1: tensor operation (gemm_perchannel_quant)\narg2: verification\narg3: initialization\n"
+                    "arg4: print tensor value\narg5: time kernel\narg6 to 11: M, N, K, StrideA, StrideB, StrideE\n"
+                    "arg12: activation (0: PassThrough; 1: Relu)\narg13: nrepeat\n");
+        return 1;
+    }
+    const bool verify = std::atoi(argv[2]), time_kernel = std::atoi(argv[5]);
+    const int init = std::atoi(argv[3]);
+    const int M = std::atoi(argv[6]), N = std::atoi(argv[7]), K = std::atoi(argv[8]);
+    int sa = argc > 9 ? std::atoi(argv[9]) : -1, sb = argc > 10 ? std::atoi(argv[10]) : -1,
+        se = argc > 11 ? std::atoi(argv[11]) : -1;
+    sa = sa < 0 ? K : sa, sb = sb < 0 ? K : sb, se = se < 0 ? N : se;
+    const int act = argc > 12 ? std::atoi(argv[12]) : 1, nrepeat = argc > 13 ? std::atoi(argv[13]) : 10;
+    return act ? profile_gemm_perchannel_quant_t<element_wise::Relu>(verify, init, time_kernel, M, N, K, sa, sb, se, nrepeat)
+               : profile_gemm_perchannel_quant_t<Pass>(verify, init, time_kernel, M, N, K, sa, sb, se, nrepeat);
+}
+
 int profile_gemm_gemm(int argc, char* argv[])
 {
     if(argc < 11)
@@ -745,6 +797,8 @@ int main(int argc, char* argv[])
             return profile_batched_gemm(argc, argv);
         if(argc >= 2 && std::strcmp(argv[1], "gemm_splitk") == 0)
             return profile_gemm_splitk(argc, argv);
+        if(argc >= 2 && std::strcmp(argv[1], "gemm_perchannel_quant") == 0)
+            return profile_gemm_perchannel_quant(argc, argv);
         if(argc >= 2 && std::strcmp(argv[1], "gemm_bias_relu") == 0)
             return profile_gemm_bias_relu(argc, argv);
         std::printf("arg1: tensor operation (gemm: GEMM\n"

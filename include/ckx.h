@@ -61,7 +61,18 @@ enum
      *                     fp16 (example/03_gemm_bias_relu/gemm_bias_relu_xdl_fp16.cpp:31-40,251-275) */
     CKX_EPI_ADD_RELU          = 3,
     CKX_EPI_ADD_RELU_ADD      = 4,
-    CKX_EPI_CSHUFFLE_ADD_RELU = 5
+    CKX_EPI_CSHUFFLE_ADD_RELU = 5,
+    /* int8 outputs with ONE ROW OF N fp32 REQUANT SCALES as the "D" operand (per output column of a GEMM, per output
+     * channel of a conv): upstream Composable Kernel's element_wise::Activation_Mul2_Clamp<Activation>
+     * (ck/tensor_operation/gpu/element/quantization_operation.hpp as shipped with ROCm; the operator is newer than
+     * the reference snapshot, whose DeviceGemmMultipleD interface, device_gemm_multiple_d.hpp:14-55, it plugs into):
+     *   y = float(acc); y = act(y); y = clamp(scale[n] * y, -128, 127); e = int8(y)   (truncation toward zero)
+     *  MUL2_CLAMP       act = PassThrough
+     *  RELU_MUL2_CLAMP  act = Relu
+     * One fp32 multiply on the exactly converted accumulator (|acc| < 2^24; larger ones round to nearest even on both
+     * sides); scales are finite by contract. */
+    CKX_EPI_MUL2_CLAMP      = 6,
+    CKX_EPI_RELU_MUL2_CLAMP = 7
 };
 
 /* Operator families, for the instance queries below. */
@@ -215,6 +226,20 @@ int ckx_gemm_f16_multiple_d(const void* p_a, const void* p_b, const void* p_d0, 
                             int32_t stride_d1, int32_t stride_e, int a_layout, int b_layout, int e_layout,
                             int cde_op, int instance, void* p_workspace, int64_t workspace_bytes, void* stream);
 
+/* ---- int8 GEMM with per-column requant scales:  E = cde_op(A * B, D0), D0 = scale[N] (fp32) ----------
+ * Replaces DeviceGemmMultipleD<..., int8_t, int8_t, Tuple<float>, int8_t, PassThrough, PassThrough,
+ * Activation_Mul2_Clamp<Act>>::MakeArgumentPointer + Run (device_gemm_multiple_d.hpp:14-55) for cde_op in
+ * CKX_EPI_MUL2_CLAMP / CKX_EPI_RELU_MUL2_CLAMP. D0 is one contiguous row of N floats, broadcast over the rows
+ * (stride_d0 must be 0, as a per-channel scale is passed upstream). Every instance of the int8 GEMM family takes it
+ * (tile, skinny, element-wise; K runs through the workspace; all four operand layouts); batches do not. */
+int ckx_gemm_i8_multiple_d_is_supported(int32_t M, int32_t N, int32_t K, int32_t stride_a, int32_t stride_b,
+                                        int32_t stride_d0, int32_t stride_e, int a_layout, int b_layout, int e_layout,
+                                        int cde_op, int instance);
+int ckx_gemm_i8_multiple_d(const void* p_a, const void* p_b, const void* p_d0, void* p_e, int32_t M, int32_t N,
+                           int32_t K, int32_t stride_a, int32_t stride_b, int32_t stride_d0, int32_t stride_e,
+                           int a_layout, int b_layout, int e_layout, int cde_op, int instance, void* p_workspace,
+                           int64_t workspace_bytes, void* stream);
+
 /* ---- conv2d forward, NHWC input / KYXC weight / NHWK output, implicit GEMM --
  * Replaces DeviceConvFwd<PassThrough, PassThrough, OutOp>::MakeArgumentPointer + Run
  * (device_conv_fwd.hpp:18-39) as implemented by
@@ -257,6 +282,15 @@ int64_t ckx_conv2d_fwd_workspace_bytes(int op, const ckx_conv2d_desc* desc, int 
 int ckx_conv2d_fwd_bias_activation_f16(const void* p_in, const void* p_wei, void* p_out, const void* p_bias,
                                        const void* p_resi, const ckx_conv2d_desc* desc, int out_op, int instance,
                                        void* p_workspace, int64_t workspace_bytes, void* stream);
+
+/* conv2d forward, int8, with one fp32 requant scale per OUTPUT CHANNEL (p_scale: K contiguous floats): out_op is
+ * CKX_EPI_MUL2_CLAMP or CKX_EPI_RELU_MUL2_CLAMP (upstream's per-channel quantisation of a conv: the same functor as
+ * the CDE operation of its multiple-D conv operators). Runs on the tile instances and the element-wise instance
+ * (the patch-window and pointwise specialists have no such epilogue); supported geometries are those of
+ * ckx_conv2d_fwd_is_supported(CKX_OP_CONV2D_FWD_I8, desc, out_op, instance). */
+int ckx_conv2d_fwd_i8_multiple_d(const void* p_in, const void* p_wei, const void* p_scale, void* p_out,
+                                 const ckx_conv2d_desc* desc, int out_op, int instance, void* p_workspace,
+                                 int64_t workspace_bytes, void* stream);
 
 /* ---- conv forward with 1, 2 or 3 spatial dimensions: NWC / NHWC / NDHWC input, KXC / KYXC / KZYXC
  * weight, NWK / NHWK / NDHWK output --------------------------------------------------------------

@@ -26,6 +26,9 @@
 //   epilogue functors                RequantReluRequant
 //       example/14_gemm_xdl_requant_relu_requant/gemm_xdl_requant_relu_requant_int8.cpp:21-39
 //       PassThrough include/ck/tensor_operation/gpu/element/unary_element_wise_operation.hpp:13-25
+//   per-channel requant functor      Activation_Mul2_Clamp<PassThrough / Relu> of upstream Composable Kernel
+//       (ck/tensor_operation/gpu/element/quantization_operation.hpp as shipped with ROCm; NOT in the reference
+//       snapshot: PARITY UNPINNED by reference vectors; pinned by closed forms and brute force in tests/test_oracle.py)
 //   type_convert                     include/ck/utility/data_type.hpp:934-938
 //   work split over threads          ParallelTensorFunctor
 //       library/include/ck/library/host_tensor/host_tensor.hpp:143-194
@@ -220,6 +223,20 @@ int8_t cko_epilogue_i8(int32_t acc, int kind, float scale_gemm, float scale_relu
     if(kind == EPI_PASSTHROUGH)
         return (int8_t)(uint8_t)(acc & 0xFF);
     return float_to_i8_trunc_wrap(ep((float)acc));
+}
+
+// Activation_Mul2_Clamp<Activation>::operator()(int8_t& y, const int32_t& x, const float& requantScale):
+//   y_fp32 = type_convert<float>(x); activation(y_fp32, y_fp32); y_fp32 = clamp(requantScale * y_fp32, -128, 127);
+//   y = type_convert<int8_t>(y_fp32)   -- Relu: y = x > 0 ? x : 0 (unary_element_wise_operation.hpp); clamp is
+//   min(max(x, lo), hi) (include/ck/utility/math.hpp); the conversion truncates toward zero (data_type.hpp:934-938)
+int8_t cko_mul2_clamp(int32_t acc, float requant_scale, int relu)
+{
+    float y = static_cast<float>(acc);
+    if(relu)
+        y = y > 0 ? y : 0;
+    y = requant_scale * y;
+    y = std::min(std::max(y, -128.f), 127.f);
+    return static_cast<int8_t>(y);
 }
 
 // int8 GEMM. A is logical [M,K] with strides (sa_m, sa_k), B logical [K,N] with

@@ -36,6 +36,18 @@ def epilogue_i8(acc_i32, epi, scale_gemm=1.0, scale_relu=1.0):
     return y.astype(np.int32).astype(np.int8)  # truncation toward zero; in range after the clamp
 
 
+def epilogue_i8_mul2_clamp(acc_i32, scales, relu):
+    """Activation_Mul2_Clamp over a [.., N] accumulator array with N scales (numpy float32 ufuncs, one rounding each)."""
+    x = np.asarray(acc_i32).astype(np.float32)
+    if relu:
+        x = np.where(x > 0, x, np.float32(0))
+    y = np.asarray(scales, np.float32) * x
+    lo, hi = np.float32(-128), np.float32(127)
+    y = np.minimum(np.maximum(y, lo), hi)
+    assert y.dtype == np.float32
+    return y.astype(np.int32).astype(np.int8)
+
+
 def gemm_i8_acc(a_mk, b_kn):
     a = np.asarray(a_mk)
     b = np.asarray(b_kn)
@@ -134,6 +146,19 @@ def conv2d_fwd_i8(inp_nhwc, wei_kyxc, strides=(1, 1), dilations=(1, 1), pads=(0,
     cols, Ho, Wo = im2col(inp_nhwc, Y, X, strides, dilations, pads, right_pads)
     acc = gemm_i8_acc(cols, wei_kyxc.reshape(K, Y * X * C).T)
     return epilogue_i8(acc, epi, scale_gemm, scale_relu).reshape(N, Ho, Wo, K)
+
+
+def gemm_i8_mul2_clamp(a_mk, b_kn, scales, relu):
+    return epilogue_i8_mul2_clamp(gemm_i8_acc(a_mk, b_kn), scales, relu)
+
+
+def conv2d_fwd_i8_mul2_clamp(inp_nhwc, wei_kyxc, scales_k, relu, strides=(1, 1), dilations=(1, 1), pads=(0, 0),
+                             right_pads=None):
+    N = inp_nhwc.shape[0]
+    K, Y, X, C = wei_kyxc.shape
+    cols, Ho, Wo = im2col(inp_nhwc, Y, X, strides, dilations, pads, right_pads)
+    acc = gemm_i8_acc(cols, wei_kyxc.reshape(K, Y * X * C).T)
+    return epilogue_i8_mul2_clamp(acc, scales_k, relu).reshape(N, Ho, Wo, K)
 
 
 def conv2d_fwd_f16(inp_nhwc, wei_kyxc, strides=(1, 1), dilations=(1, 1), pads=(0, 0), right_pads=None):

@@ -35,6 +35,8 @@ def lib():
         _lib.cko_float_to_half.argtypes = [C.c_float]
         _lib.cko_epilogue_i8.restype = C.c_int8
         _lib.cko_epilogue_i8.argtypes = [C.c_int32, C.c_int, C.c_float, C.c_float]
+        _lib.cko_mul2_clamp.restype = C.c_int8
+        _lib.cko_mul2_clamp.argtypes = [C.c_int32, C.c_float, C.c_int]
         _lib.cko_conv_out_len.restype = C.c_int
         _lib.cko_magic_division_divide.restype = C.c_uint32
         _lib.cko_magic_division_divide.argtypes = [C.c_uint32, C.c_uint32, C.c_uint32]
@@ -247,6 +249,21 @@ def gemm_f16_add_relu(a_mk, b_kn, d_mn, nthreads=0):
 
 def epilogue_i8(acc, epi, scale_gemm, scale_relu):
     return int(lib().cko_epilogue_i8(int(acc), int(epi), C.c_float(scale_gemm), C.c_float(scale_relu)))
+
+
+def mul2_clamp(acc, requant_scale, relu):
+    """Activation_Mul2_Clamp<PassThrough / Relu> on one accumulator (upstream functor, literal restatement)."""
+    return int(lib().cko_mul2_clamp(int(acc), C.c_float(requant_scale), int(bool(relu))))
+
+
+def gemm_i8_mul2_clamp(a_mk, b_kn, scales_n, relu, nthreads=0):
+    """int8 GEMM with int32 accumulation and one requant scale per output column, element by element."""
+    acc = gemm_i8_acc(a_mk, b_kn, nthreads)
+    out = np.empty(acc.shape, np.int8)
+    for m in range(acc.shape[0]):
+        for n in range(acc.shape[1]):
+            out[m, n] = mul2_clamp(acc[m, n], scales_n[n], relu)
+    return out
 
 
 def magic_params(d):

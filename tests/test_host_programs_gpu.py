@@ -156,6 +156,22 @@ def test_profiler_gemm_bias_relu(tmp_path):
     assert bad == 0, max_err
 
 
+@pytest.mark.parametrize("act", [0, 1])
+def test_profiler_gemm_perchannel_quant(tmp_path, act):
+    """C++ DeviceGemmMultipleD<int8, ..., Tuple<float>, int8, Activation_Mul2_Clamp<Act>> over every instance: all
+    agree with the first, the best one matches the oracle bit for bit (init 1: int8 in [-5, 5]; the profiler's scale
+    of column n is ((37 n) mod 61 - 20) / 256)."""
+    M, N, K = 200, 320, 512
+    out, dump = _run("ckx_profiler", ["gemm_perchannel_quant", 1, 1, 0, 1, M, N, K, -1, -1, -1, act], "CKX_PROFILER_DUMP",
+                     tmp_path)
+    assert "Best Perf:" in out and "Error" not in out and "Mul2_Clamp" in out
+    e = np.fromfile(dump, np.int8).reshape(M, N)
+    a = uniform_int8((M, K), -5, 5, SEED)
+    b_nk = uniform_int8((N, K), -5, 5, SEED + 1)
+    scale = (((np.arange(N) * 37) % 61 - 20) / 256.0).astype(np.float32)
+    np.testing.assert_array_equal(e, fast.gemm_i8_mul2_clamp(a, b_nk.T, scale, bool(act)))
+
+
 def test_profiler_gemm_splitk_int8(tmp_path):
     """profile_gemm_splitk's argument list (KBatch = arg14); PassThrough int8 output keeps the low byte."""
     M, N, K = 128, 512, 4096

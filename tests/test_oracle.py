@@ -133,6 +133,59 @@ def test_epilogue_scalar_against_exact_arithmetic(epi, sg, sr):
                                   np.array([lit.epilogue_i8(a, epi, sg, sr) for a in accs], np.int8))
 
 
+def _mul2_clamp_exact(acc, scale, relu):
+    """Independent derivation of Activation_Mul2_Clamp: exact fp32 product through float64 (as above), ordinary
+    min / max, truncation toward zero."""
+    x = np.float32(acc)
+    if relu and x < 0:
+        x = np.float32(0)
+    y = np.float32(np.float64(np.float32(scale)) * np.float64(x))
+    return int(min(max(float(y), -128.0), 127.0))
+
+
+@pytest.mark.parametrize("relu", [False, True])
+@pytest.mark.parametrize("scale", [0.03, -0.03, 0.4, 1.0, 2.0 ** -20, 37.5, 0.0, -1.0])
+def test_mul2_clamp_scalar_against_exact_arithmetic(scale, relu):
+    """The per-channel functor (upstream's Activation_Mul2_Clamp; absent from the reference snapshot, so no reference
+    vectors: parity unpinned by the reference, pinned by what follows)."""
+    rng = np.random.default_rng(4)
+    accs = list(range(-5000, 5000)) + [int(v) for v in rng.integers(-2 ** 24, 2 ** 24, 4000)] + \
+        [2 ** 24, -(2 ** 24), 2 ** 24 + 1, 2 ** 31 - 1, -(2 ** 31)]       # beyond 2^24 the conversion itself rounds
+    for acc in accs:
+        assert lit.mul2_clamp(acc, scale, relu) == _mul2_clamp_exact(acc, scale, relu), (acc, scale, relu)
+    arr = np.array(accs, np.int32)
+    np.testing.assert_array_equal(fast.epilogue_i8_mul2_clamp(arr, np.float32(scale), relu),
+                                  np.array([lit.mul2_clamp(a, scale, relu) for a in accs], np.int8))
+
+
+def test_mul2_clamp_closed_forms():
+    # the Relu form with requant scale s IS the reference's RequantReluRequant(1, s), literal form (example 14):
+    # both are trunc(clamp(s * relu(float(acc)))) -- and that functor is pinned against the reference itself
+    for s in (0.03, 0.4, 1.0, 2.5, 0.0078125):
+        for acc in list(range(-300, 6000, 7)) + [10 ** 6, -10 ** 6]:
+            assert lit.mul2_clamp(acc, s, True) == lit.epilogue_i8(acc, lit.EPI_REQUANT_CK, 1.0, s)
+    # dyadic scales: the product is exact, the result is integer arithmetic -- truncation TOWARD ZERO on both sides
+    for k in (1, 3, 100, 255):
+        for acc in range(-2000, 2000):
+            q = acc * k                      # value * 256
+            want = max(-128, min(127, -((-q) // 256) if q < 0 else q // 256))
+            assert lit.mul2_clamp(acc, k / 256.0, False) == want
+    # clamp is asymmetric, a negative scale flips the sign after the ReLU, zero scale gives zero
+    assert lit.mul2_clamp(10 ** 6, 1.0, False) == 127 and lit.mul2_clamp(-10 ** 6, 1.0, False) == -128
+    assert lit.mul2_clamp(100, -0.5, True) == -50 and lit.mul2_clamp(-100, -0.5, True) == 0
+    assert lit.mul2_clamp(-100, -0.5, False) == 50 and lit.mul2_clamp(12345, 0.0, False) == 0
+    # per column: column n of the GEMM form uses scale n only
+    a = np.arange(-20, 20, dtype=np.int8).reshape(5, 8)
+    b = (np.arange(24, dtype=np.int8).reshape(8, 3) - 11)
+    s = np.array([0.5, -0.25, 3.0], np.float32)
+    acc = a.astype(np.int64) @ b.astype(np.int64)
+    for relu in (False, True):
+        out = lit.gemm_i8_mul2_clamp(a, b, s, relu)
+        np.testing.assert_array_equal(out, fast.gemm_i8_mul2_clamp(a, b, s, relu))
+        for n in range(3):
+            assert [int(v) for v in out[:, n]] == [_mul2_clamp_exact(int(v), s[n], relu) for v in acc[:, n]]
+
+
 def test_epilogue_special_cases():
     R, Cc = lit.EPI_REQUANT_RND, lit.EPI_REQUANT_CK
     # ties go to even with scale 0.5
