@@ -114,6 +114,7 @@ struct TileInstance
     float eff; // measured MFMA throughput of this tile shape relative to the 256x256 one
     tile_launch_fn dense_i8, dense_f16, conv_i8, conv_f16, dense_bf16;
     tile_launch_fn dense_f16_fused, conv_f16_fused; // fp16 with the add / ReLU epilogues and D operands
+    tile_launch_fn dense_i8_fused, conv_i8_fused;   // int8 with the per-column requant scales as D operand
 };
 
 #define CKX_TILE(BM, BN, WM, WN, NST, EFF)                                                         \
@@ -125,7 +126,9 @@ struct TileInstance
             &launch_tile<ckx::DT_F16, BM, BN, WM, WN, 128, NST, true>,                                \
             &launch_tile<ckx::DT_BF16, BM, BN, WM, WN, 128, NST, false>,                              \
             &launch_tile<ckx::DT_F16, BM, BN, WM, WN, 128, NST, false, false, false, true>,           \
-            &launch_tile<ckx::DT_F16, BM, BN, WM, WN, 128, NST, true, false, false, true>             \
+            &launch_tile<ckx::DT_F16, BM, BN, WM, WN, 128, NST, true, false, false, true>,            \
+            &launch_tile<ckx::DT_I8, BM, BN, WM, WN, 128, NST, false, false, false, true>,            \
+            &launch_tile<ckx::DT_I8, BM, BN, WM, WN, 128, NST, true, false, false, true>              \
     },
 
 const TileInstance kTiles[] = {CKX_FOR_EACH_TILE(CKX_TILE)};
@@ -352,7 +355,7 @@ bool gemm_needs_generic(int dt, int M, int N, int K, int sa, int sb, bool ta, bo
 {
     const int es = dt == ckx::DT_I8 ? 1 : 2;
     return ((long)(ta ? M : K) * es) % 16 || ((long)(tb ? N : K) * es) % 16 || ((long)sa * es) % 16 ||
-           ((long)sb * es) % 16 || ((ta || tb) && f16_fused(epi));
+           ((long)sb * es) % 16 || ((ta || tb) && (f16_fused(epi) || per_column_scale(epi)));
 }
 
 int check_gemm_shape(int dt, int M, int N, int K, int sa, int sb, int sc, int al, int bl, int cl, int epi,
@@ -377,7 +380,7 @@ int check_gemm_shape(int dt, int M, int N, int K, int sa, int sb, int sc, int al
     const bool ta = al == CKX_COL_MAJOR, tb = bl == CKX_ROW_MAJOR;
     // what only the element-granular instance takes (AUTO sends it there)
     const bool fast = instance != CKX_INSTANCE_AUTO && instance != kGenericGemmInstance;
-    if(fast && (ta || tb) && f16_fused(epi))
+    if(fast && (ta || tb) && (f16_fused(epi) || per_column_scale(epi)))
         return fail(CKX_UNSUPPORTED, "the D-operand epilogues of this instance are built for A row-major, B column-major");
     if(fast && (ta || tb) && !ckx::layout_tile(dt, instance, ta, tb))
         return fail(CKX_UNSUPPORTED, "this instance has no variant for a K-major operand (tiles of 64 rows and more do)");
@@ -582,7 +585,7 @@ int run_gemm(int dt, const void* a, const void* b, void* c, int M, int N, int K,
     g.ws         = ws;
     const bool fused            = f16_fused(epi) && g.ksplit == 1; // (after a K split the second pass applies it)
     const tile_launch_fn launch = kmajor               ? ckx::layout_tile(dt, ti, ta, tb)
-                                  : dt == ckx::DT_I8   ? t.dense_i8
+                                  : dt == ckx::DT_I8   ? (per_column_scale(epi) && g.ksplit == 1 ? t.dense_i8_fused : t.dense_i8)
                                   : dt == ckx::DT_BF16 ? t.dense_bf16
                                   : fused              ? t.dense_f16_fused
                                                        : t.dense_f16;
@@ -845,7 +848,9 @@ int run_conv(int op, const void* in, const void* wei, void* out, const ckx_conv2
     g.nk_per = pl.nk_per;
     g.ws     = ws;
     const bool fused = f16_fused(epi) && g.ksplit == 1;
-    hipError_t e     = (es == 1 ? t.conv_i8 : fused ? t.conv_f16_fused : t.conv_f16)(g, g.tiles_m * g.tiles_n * g.ksplit,
+    hipError_t e     = (es == 1  ? (per_column_scale(epi) && g.ksplit == 1 ? t.conv_i8_fused : t.conv_i8)
+                        : fused ? t.conv_f16_fused
+                                : t.conv_f16)(g, g.tiles_m * g.tiles_n * g.ksplit,
                                                                                  (hipStream_t)stream);
     if(e == hipSuccess && g.ksplit > 1)
         e = es == 1 ? launch_reduce<ckx::DT_I8>(g, (hipStream_t)stream)

@@ -548,7 +548,8 @@ struct GemmTile
     static_assert((BM * CPR) % NT == 0 && (BN * CPR) % NT == 0, "tile rows must split over the waves");
 
     static_assert(IM2COL >= 0 && IM2COL <= 2 && !(IM2COL != 0 && (TA || TB)), "the im2col view (1: two spatial dimensions, 2: three) is K-contiguous");
-    static_assert(!FUSED || (DT == DT_F16 && !TA && !TB), "D-operand epilogues: fp16, K-contiguous operands");
+    static_assert(!FUSED || ((DT == DT_F16 || DT == DT_I8) && !TA && !TB),
+                  "D-operand epilogues (fp16: add / ReLU functors; int8: per-column requant scales): K-contiguous operands");
     static_assert((!TA || (BM >= 64 && BM * ES <= 1024)) && (!TB || (BN >= 64 && BN * ES <= 1024)),
                   "a K-major tile row is 64..1024 bytes");
     static constexpr int KE = BKB / ES; // k rows of a K tile
@@ -949,10 +950,11 @@ struct GemmTile
             acc_t* slice = reinterpret_cast<acc_t*>(reinterpret_cast<uint8_t*>(p.ws) +
                                                     (size_t)(unit / ntiles_all) * p.M * p.N * 4);
             uint8_t* c_batch = reinterpret_cast<uint8_t*>(p.c) + (size_t)bi * p.bsc * ES;
-            // Per-column requant scales: a loop nest of its own, column group outermost, so that the 16 scales of the
-            // lane's columns are fetched once per group and before that group's stores (a load issued after a store
-            // waits for it) and only 16 registers hold them.
-            if constexpr(DT == DT_I8)
+            // Per-column requant scales (the FUSED variant of the int8 kernel: compiled into the plain one it cost the
+            // im2col instances ten more spilled SGPRs and 7 - 10 % on the conv and LLM shapes): a loop nest of its own,
+            // column group outermost, so that the 16 scales of the lane's columns are fetched once per group and before
+            // that group's stores (a load issued after a store waits for it) and only 16 registers hold them.
+            if constexpr(DT == DT_I8 && FUSED)
             {
                 if(epi_per_column_scale(p.epi) && p.ksplit == 1)
                 {
@@ -1230,7 +1232,7 @@ struct GemmTile
             {
                 if constexpr(TB)
                     transpose_acc();
-                if constexpr(FUSED)
+                if constexpr(FUSED && DT == DT_F16)
                 {
                     if(p.epi == EPI_PASSTHROUGH || p.ksplit > 1)
                         epilogue(unit);
