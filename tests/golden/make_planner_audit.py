@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Measures what the launch planner is audited against (run on the MI355X; writes planner_audit.json beside itself).
 
-    python tests/golden/make_planner_audit.py [--quick]
+    python tests/golden/make_planner_audit.py [--quick] [--out PATH]
 
 For every problem of a grid (int8 requant and fp16 GEMMs, A row-major, B column-major, LLM-like and square shapes
 from 1 to 4096 rows; the ResNet-like conv layers of the benchmark) every instance that supports the problem is
@@ -51,6 +51,7 @@ def time_launch(launch, steps=200, settle_ms=20.0):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--quick", action="store_true", help="a fifth of the grid (smoke run of this script)")
+    ap.add_argument("--out", default=None, help="where to write the table (default: planner_audit.json beside this script)")
     args = ap.parse_args()
     import torch
     import composable_kernel_amd as ck
@@ -131,8 +132,7 @@ def main():
         row["auto"] = list(capi.conv2d_fwd_plan(opf, desc, epi, ws.numel()))
         out["conv"].append(row)
         print(row, flush=True)
-    path = os.path.join(ROOT, "gpurun_out", "planner_audit.json") if os.path.isdir(os.path.join(ROOT, "gpurun_out")) \
-        else os.path.join(HERE, "planner_audit.json")
+    path = args.out or os.path.join(HERE, "planner_audit.json")
     with open(path, "w") as f:
         json.dump(out, f, indent=0, separators=(",", ":"))
     print("wrote", path)
