@@ -609,7 +609,8 @@ bool conv_patch_applicable(int op, const ckx_conv2d_desc* d, int epi)
 {
     const bool epi_ok = op == CKX_OP_CONV2D_FWD_F16
                             ? (epi == CKX_EPI_PASSTHROUGH || epi == CKX_EPI_ADD_RELU || epi == CKX_EPI_ADD_RELU_ADD)
-                            : (epi == CKX_EPI_PASSTHROUGH || epi == CKX_EPI_REQUANT_CK || epi == CKX_EPI_REQUANT_RND);
+                            : (epi == CKX_EPI_PASSTHROUGH || epi == CKX_EPI_REQUANT_CK || epi == CKX_EPI_REQUANT_RND ||
+                               per_column_scale(epi));
     return (op == CKX_OP_CONV2D_FWD_F16 || op == CKX_OP_CONV2D_FWD_I8) && epi_ok && d->C == 64 && d->K == 64 && d->Y == 3 &&
            d->X == 3 && d->stride_h == 1 && d->stride_w == 1 && d->dilation_h == 1 && d->dilation_w == 1 &&
            d->Wo == 56 && d->Ho >= 1 && d->N >= 1 && d->pad_left <= 2 && d->pad_top <= 2;
@@ -634,7 +635,10 @@ bool conv_pointwise_applicable(int op, const ckx_conv2d_desc* d, int epi)
     const int es      = op == CKX_OP_CONV2D_FWD_I8 ? 1 : 2;
     const bool epi_ok = op == CKX_OP_CONV2D_FWD_F16
                             ? (epi == CKX_EPI_PASSTHROUGH || epi == CKX_EPI_ADD_RELU)
-                            : (epi == CKX_EPI_PASSTHROUGH || epi == CKX_EPI_REQUANT_CK || epi == CKX_EPI_REQUANT_RND);
+                            : (epi == CKX_EPI_PASSTHROUGH || epi == CKX_EPI_REQUANT_CK || epi == CKX_EPI_REQUANT_RND ||
+                               per_column_scale(epi));
+    if(per_column_scale(epi) && d->C * es != 256) // (no registers for the scales beside the weights of a 512-byte pixel)
+        return false;
     return (op == CKX_OP_CONV2D_FWD_F16 || op == CKX_OP_CONV2D_FWD_I8) && epi_ok && d->Y == 1 && d->X == 1 &&
            d->pad_top == 0 && d->pad_left == 0 && d->pad_bottom == 0 && d->pad_right == 0 &&
            (d->C * es == 256 || d->C * es == 512) && d->K >= 512 && d->K % 512 == 0 && d->N >= 1 && d->Ho >= 1 &&
@@ -793,7 +797,8 @@ int run_conv(int op, const void* in, const void* wei, void* out, const ckx_conv2
         a.epi    = epi;
         a.bias = dops.d0, a.resi = epi == CKX_EPI_ADD_RELU_ADD ? dops.d1 : nullptr;
         a.scale_gemm = sg, a.scale_relu = sr;
-        hipError_t e = es == 1                     ? launch_conv_patch<ckx::DT_I8, false>(a, (hipStream_t)stream)
+        hipError_t e = es == 1 && per_column_scale(epi) ? launch_conv_patch<ckx::DT_I8, true>(a, (hipStream_t)stream)
+                       : es == 1                     ? launch_conv_patch<ckx::DT_I8, false>(a, (hipStream_t)stream)
                        : epi == CKX_EPI_PASSTHROUGH ? launch_conv_patch<ckx::DT_F16, false>(a, (hipStream_t)stream)
                                                     : launch_conv_patch<ckx::DT_F16, true>(a, (hipStream_t)stream);
         return e == hipSuccess ? CKX_OK : hip_fail(e, kPatchName);
@@ -816,7 +821,8 @@ int run_conv(int op, const void* in, const void* wei, void* out, const ckx_conv2
         a.epi = epi, a.bias = dops.d0;
         a.scale_gemm = sg, a.scale_relu = sr;
         a.nt_store   = (long)M * N * es >= stream_output_bytes();
-        hipError_t e = ckx::launch_conv_pointwise(es == 1 ? ckx::DT_I8 : ckx::DT_F16, d->C * es, epi == CKX_EPI_ADD_RELU, a,
+        hipError_t e = ckx::launch_conv_pointwise(es == 1 ? ckx::DT_I8 : ckx::DT_F16, d->C * es,
+                                                  epi == CKX_EPI_ADD_RELU || per_column_scale(epi), a,
                                                   (hipStream_t)stream);
         return e == hipSuccess ? CKX_OK : hip_fail(e, kPointwiseName);
     }

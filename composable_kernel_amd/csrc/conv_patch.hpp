@@ -39,8 +39,9 @@ struct ConvPatchArgs
     int N, Hi, Wi, Ho, Wo;
     int pT, pL;
     MagicDiv div_wo;
-    int epi; // fp16: EPI_PASSTHROUGH, EPI_ADD_RELU, EPI_ADD_RELU_ADD; int8: EPI_PASSTHROUGH, EPI_REQUANT_CK, EPI_REQUANT_RND
-    const void* bias; // [64] fp16
+    int epi; // fp16: EPI_PASSTHROUGH, EPI_ADD_RELU, EPI_ADD_RELU_ADD; int8: EPI_PASSTHROUGH, EPI_REQUANT_CK, EPI_REQUANT_RND,
+             // EPI_MUL2_CLAMP / EPI_RELU_MUL2_CLAMP (one requant scale per output channel)
+    const void* bias; // [64]: fp16 bias (fp16 kernels), fp32 requant scales (the int8 per-channel variant)
     const void* resi; // NHWK fp16
     float scale_gemm, scale_relu; // int8 requant epilogues
 };
@@ -78,7 +79,8 @@ struct ConvPatch
     static constexpr int NT         = 256;
     static constexpr int NEED_ROWS  = TH + Y - 1;   // input rows of one band
     static_assert(Y >= 1 && Y <= 3 && X >= 1 && X <= 3 && MTW >= 1 && MTW <= 7, "covered shapes");
-    static_assert(DT == DT_F16 || (DT == DT_I8 && !FUSED), "fp16 (optionally with the add / ReLU epilogues) or int8");
+    static_assert(DT == DT_F16 || DT == DT_I8, "fp16 (FUSED: the add / ReLU epilogues) or int8 (FUSED: per-channel requant)");
+    static constexpr bool F16FUSED = FUSED && DT == DT_F16, I8PERCH = FUSED && DT == DT_I8;
     static_assert((WMW == 2 || WMW == 4) && (NBT == 2 || DT == DT_I8), "wave arrangements built");
     static_assert(LDS <= 160 * 1024, "ring + weights fit the LDS");
     using acc_t = typename std::conditional<DT == DT_I8, i32x4, f32x4>::type;
@@ -144,14 +146,22 @@ struct ConvPatch
             }
         }
         // fused add / ReLU epilogues: the lane's 8 bias values once, its residual values band by band
-        const bool has_resi = FUSED && p.epi == EPI_ADD_RELU_ADD;
+        const bool has_resi = F16FUSED && p.epi == EPI_ADD_RELU_ADD;
         f16x8 bias8 = {0, 0, 0, 0, 0, 0, 0, 0};
-        if constexpr(FUSED)
+        if constexpr(F16FUSED)
             bias8 = *reinterpret_cast<const f16x8*>(reinterpret_cast<const _Float16*>(p.bias) + CPW * wn + 4 * NBT * (int)fq);
-        f16x8 resi8[FUSED ? MTW : 1];
+        f16x8 resi8[F16FUSED ? MTW : 1];
 #pragma unroll
-        for(int t = 0; t < (FUSED ? MTW : 1); ++t)
+        for(int t = 0; t < (F16FUSED ? MTW : 1); ++t)
             resi8[t] = f16x8{0, 0, 0, 0, 0, 0, 0, 0};
+        // int8, per-channel requant: the scales of the lane's 4 * NBT consecutive channels, for the life of the workgroup
+        float chsc[I8PERCH ? 4 * NBT : 1];
+        if constexpr(I8PERCH)
+        {
+#pragma unroll
+            for(int e = 0; e < 4 * NBT; ++e)
+                chsc[e] = reinterpret_cast<const float*>(p.bias)[CPW * wn + 4 * NBT * (int)fq + e];
+        }
 
         uint32_t boff[NBT]; // weight fragment of n-tile j, k-step 0, tap 0
 #pragma unroll
@@ -245,7 +255,7 @@ struct ConvPatch
                 }
                 // residual values of this band: plain loads, issued before the band's direct loads and
                 // waited for with them (a load issued after the stores would have to wait for those)
-                if constexpr(FUSED)
+                if constexpr(F16FUSED)
                   if(has_resi)
                 {
                     const uint8_t* resi_band = reinterpret_cast<const uint8_t*>(p.resi) +
@@ -253,7 +263,7 @@ struct ConvPatch
 #pragma unroll
                     for(int t = 0; t < MTW; ++t)
                         if(TH * b + (int)rout[t] < p.Ho)
-                            resi8[FUSED ? t : 0] = *reinterpret_cast<const f16x8*>(resi_band + ooff[t]);
+                            resi8[F16FUSED ? t : 0] = *reinterpret_cast<const f16x8*>(resi_band + ooff[t]);
                 }
                 // One k-step = MTW groups pinned in source order: [reads of the NEXT k-step, spread over
                 // the first groups and finished two groups early] [one direct load of the next band's
@@ -345,7 +355,18 @@ struct ConvPatch
                             if(TH * b + (int)rout[t] < p.Ho)
                             {
                                 int o[NBT];
-                                if constexpr(EPI == EPI_REQUANT_RND)
+                                if constexpr(EPI == EPI_MUL2_CLAMP || EPI == EPI_RELU_MUL2_CLAMP)
+                                {
+                                    constexpr bool relu = EPI == EPI_RELU_MUL2_CLAMP;
+                                    constexpr int NS    = I8PERCH ? 4 * NBT : 1;
+#pragma unroll
+                                    for(int j = 0; j < NBT; ++j)
+                                        o[j] = pack4_low_bytes(mul2_clamp(acc[t][j][0], chsc[(4 * j) % NS], relu),
+                                                               mul2_clamp(acc[t][j][1], chsc[(4 * j + 1) % NS], relu),
+                                                               mul2_clamp(acc[t][j][2], chsc[(4 * j + 2) % NS], relu),
+                                                               mul2_clamp(acc[t][j][3], chsc[(4 * j + 3) % NS], relu));
+                                }
+                                else if constexpr(EPI == EPI_REQUANT_RND)
                                 {
                                     i32x4 v[NBT];
 #pragma unroll
@@ -377,7 +398,14 @@ struct ConvPatch
                                 acc[t][j] = acc_t{0, 0, 0, 0};
                         }
                     };
-                    if(p.epi == EPI_REQUANT_RND)
+                    if constexpr(I8PERCH)
+                    {
+                        if(p.epi == EPI_RELU_MUL2_CLAMP)
+                            store_band(std::integral_constant<int, EPI_RELU_MUL2_CLAMP>{});
+                        else
+                            store_band(std::integral_constant<int, EPI_MUL2_CLAMP>{});
+                    }
+                    else if(p.epi == EPI_REQUANT_RND)
                         store_band(std::integral_constant<int, EPI_REQUANT_RND>{});
                     else if(p.epi == EPI_REQUANT_CK)
                         store_band(std::integral_constant<int, EPI_REQUANT_CK>{});

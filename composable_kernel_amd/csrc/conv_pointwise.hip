@@ -34,6 +34,10 @@ hipError_t launch_pw(const ConvPointwiseArgs& a, hipStream_t s)
 
 hipError_t launch_conv_pointwise(int dt, int pixel_bytes, bool fused, const ConvPointwiseArgs& a, hipStream_t s)
 {
+    // one requant scale per output channel: 16 more registers per lane, which the 512-byte-pixel kernel (128 weight
+    // registers) does not have -- the caller sends those layers to the tile instances
+    if(dt == DT_I8 && fused)
+        return pixel_bytes == 256 ? launch_pw<DT_I8, 4, true>(a, s) : hipErrorInvalidValue;
     if(dt == DT_I8)
         return pixel_bytes == 256 ? launch_pw<DT_I8, 4, false>(a, s) : launch_pw<DT_I8, 8, false>(a, s);
     if(pixel_bytes == 256)

@@ -41,14 +41,16 @@ struct ConvPointwiseArgs
     int Kout; // output channels
     int Hi, Wi, Wo, HoWo, sH, sW;
     MagicDiv div_howo, div_wo;
-    int epi; // fp16: EPI_PASSTHROUGH, EPI_ADD_RELU (bias row); int8: EPI_PASSTHROUGH, EPI_REQUANT_CK, EPI_REQUANT_RND
-    const void* bias; // [Kout] fp16
+    int epi; // fp16: EPI_PASSTHROUGH, EPI_ADD_RELU (bias row); int8: EPI_PASSTHROUGH, EPI_REQUANT_CK, EPI_REQUANT_RND,
+             // EPI_MUL2_CLAMP / EPI_RELU_MUL2_CLAMP (one requant scale per output channel)
+    const void* bias; // [Kout]: fp16 bias (fp16 kernels), fp32 requant scales (the int8 per-channel variant)
     float scale_gemm, scale_relu;
     int nt_store; // stream the output past L2 (outputs too large to be re-read from cache)
 };
 
 // KS: MFMA k-steps per pixel (C * element size / 64 bytes); MT: 16-pixel tiles per band;
-// FUSED (fp16): the bias + ReLU epilogue is compiled in
+// FUSED: fp16 -- the bias + ReLU epilogue is compiled in; int8 -- the per-channel requant epilogue
+// (Activation_Mul2_Clamp) INSTEAD of the per-tensor ones
 template <int DT, int KS, int MT, bool FUSED>
 struct ConvPointwise
 {
@@ -65,7 +67,7 @@ struct ConvPointwise
     static constexpr int LPW  = SLOT / 1024 / NW; // direct loads per wave and band
     static constexpr int NWG  = 64 * NW;          // output channels per workgroup
     static_assert(KS == 4 || KS == 8, "pixels of 256 or 512 bytes");
-    static_assert(DT == DT_F16 || (DT == DT_I8 && !FUSED), "fp16 (optionally bias + ReLU) or int8");
+    static_assert(DT == DT_F16 || DT == DT_I8, "fp16 (optionally bias + ReLU) or int8 (per-tensor or per-channel requant)");
     static_assert(SLOT % (1024 * NW) == 0 && LPW >= 1 && LPW <= KS, "every wave issues the same number of loads");
     static_assert(LDS <= 160 * 1024 && (D - 3) * LPW < 64, "ring fits the LDS, vmcnt is a 6-bit counter");
     using acc_t = typename std::conditional<DT == DT_I8, i32x4, f32x4>::type;
@@ -105,7 +107,14 @@ struct ConvPointwise
         // pixel), fp16 two runs of 8, at n0 and n0 + 32 (each store instruction again 64 contiguous bytes per pixel)
         const int n0 = n_wave + (ES == 1 ? 16 : 8) * (int)fq;
         f16x8 bias_lo = {0, 0, 0, 0, 0, 0, 0, 0}, bias_hi = bias_lo;
-        if constexpr(FUSED)
+        float chsc[DT == DT_I8 && FUSED ? 16 : 1]; // the requant scales of the lane's 16 channels
+        if constexpr(DT == DT_I8 && FUSED)
+        {
+#pragma unroll
+            for(int e = 0; e < 16; ++e)
+                chsc[e] = reinterpret_cast<const float*>(p.bias)[n0 + e];
+        }
+        else if constexpr(FUSED)
         {
             bias_lo = *reinterpret_cast<const f16x8*>(reinterpret_cast<const _Float16*>(p.bias) + n0);
             bias_hi = *reinterpret_cast<const f16x8*>(reinterpret_cast<const _Float16*>(p.bias) + n0 + 32);
@@ -231,7 +240,17 @@ struct ConvPointwise
                         if constexpr(DT == DT_I8)
                         {
                             i32x4 pk;
-                            if constexpr(EPI == EPI_REQUANT_RND)
+                            if constexpr(EPI == EPI_MUL2_CLAMP || EPI == EPI_RELU_MUL2_CLAMP)
+                            {
+#pragma unroll
+                                for(int tn = 0; tn < 4; ++tn)
+                                    pk[tn] = pack4_low_bytes(
+                                        mul2_clamp(acc[t & 1][tn][0], chsc[(4 * tn) % (FUSED ? 16 : 1)], EPI == EPI_RELU_MUL2_CLAMP),
+                                        mul2_clamp(acc[t & 1][tn][1], chsc[(4 * tn + 1) % (FUSED ? 16 : 1)], EPI == EPI_RELU_MUL2_CLAMP),
+                                        mul2_clamp(acc[t & 1][tn][2], chsc[(4 * tn + 2) % (FUSED ? 16 : 1)], EPI == EPI_RELU_MUL2_CLAMP),
+                                        mul2_clamp(acc[t & 1][tn][3], chsc[(4 * tn + 3) % (FUSED ? 16 : 1)], EPI == EPI_RELU_MUL2_CLAMP));
+                            }
+                            else if constexpr(EPI == EPI_REQUANT_RND)
                             {
                                 const i32x4 v[4] = {acc[t & 1][0], acc[t & 1][1], acc[t & 1][2], acc[t & 1][3]};
                                 int b[16];
@@ -280,7 +299,14 @@ struct ConvPointwise
                 ld_slot = ld_slot + 1 == D ? 0 : ld_slot + 1;
             }
         };
-        if constexpr(DT == DT_I8)
+        if constexpr(DT == DT_I8 && FUSED)
+        {
+            if(p.epi == EPI_RELU_MUL2_CLAMP)
+                run_bands(std::integral_constant<int, EPI_RELU_MUL2_CLAMP>{});
+            else
+                run_bands(std::integral_constant<int, EPI_MUL2_CLAMP>{});
+        }
+        else if constexpr(DT == DT_I8)
         {
             if(p.epi == EPI_REQUANT_RND)
                 run_bands(std::integral_constant<int, EPI_REQUANT_RND>{});

@@ -7,7 +7,8 @@ DeviceGemmMultipleD interface (device_gemm_multiple_d.hpp:14-55); the reference 
 there are no reference vectors: the oracle's restatement is pinned in tests/test_oracle.py (against the reference's
 RequantReluRequant, which the Relu form equals at scaleGemm = 1, against exact dyadic arithmetic and brute force),
 and the same identities are checked on the GPU here. Every instance of the int8 GEMM family takes the functor
-(tile, skinny, element-wise), with and without a K split; batches and the conv specialists do not.
+(tile, skinny, element-wise), with and without a K split, and so do the conv specialists (patch-window kernel;
+pointwise kernel for 256-byte pixels); batches do not.
 """
 import ctypes as C
 
@@ -189,13 +190,50 @@ def test_conv2d_per_output_channel(layer):
         np.testing.assert_array_equal(out, fast.conv2d_fwd_i8_mul2_clamp(x, w, s, act == "relu", (st, st), (1, 1), (pd, pd)))
 
 
-def test_conv_specialists_refuse_the_functor():
+@pytest.mark.parametrize("act", list(ACTS))
+def test_conv_specialists_take_the_functor(act):
+    """the patch-window kernel (3x3, C = K = 64, Wo = 56) and the pointwise kernel (1x1, 256-byte pixels) with one
+    scale per output channel, forced and as the automatic choice; 512-byte pixels stay on the tile instances"""
     import gpu_util
-    x = uniform_int8((2, 56, 56, 64), -5, 5, 91)
+    patch = gpu_util.conv_instance(capi.OP_CONV2D_FWD_I8, "Patch")
+    point = gpu_util.conv_instance(capi.OP_CONV2D_FWD_I8, "Pointwise")
+    relu = act == "relu"
+    x = uniform_int8((5, 56, 56, 64), -5, 5, 91)
     w = uniform_int8((64, 3, 3, 64), -5, 5, 92)
     s = scales_for(64, 93)
-    patch = gpu_util.conv_instance(capi.OP_CONV2D_FWD_I8, "Patch")
-    assert _conv(x, w, s, "relu", (1, 1), (1, 1), instance=patch, allow_unsupported=True) is None
+    want = fast.conv2d_fwd_i8_mul2_clamp(x, w, s, relu, (1, 1), (1, 1), (1, 1))
+    np.testing.assert_array_equal(_conv(x, w, s, act, (1, 1), (1, 1), instance=patch), want)
+    x = uniform_int8((3, 28, 28, 256), -5, 5, 94)
+    w = uniform_int8((512, 1, 1, 256), -5, 5, 95)
+    s = scales_for(512, 96)
+    want = fast.conv2d_fwd_i8_mul2_clamp(x, w, s, relu, (2, 2), (1, 1), (0, 0))
+    np.testing.assert_array_equal(_conv(x, w, s, act, (2, 2), (0, 0), instance=point), want)
+    x = uniform_int8((2, 14, 14, 512), -5, 5, 97)
+    w = uniform_int8((512, 1, 1, 512), -5, 5, 98)
+    assert _conv(x, w, s, act, (1, 1), (0, 0), instance=point, allow_unsupported=True) is None
+    np.testing.assert_array_equal(_conv(x, w, s, act, (1, 1), (0, 0)),
+                                  fast.conv2d_fwd_i8_mul2_clamp(x, w, s, relu, (1, 1), (1, 1), (0, 0)))
+
+
+def test_conv_automatic_choice_reaches_the_specialists():
+    """batches large enough for the planner to prefer them (N >= 112 for the patch kernel, 16 K pixels for pointwise)"""
+    x = uniform_int8((112, 56, 56, 64), -5, 5, 101)
+    w = uniform_int8((64, 3, 3, 64), -5, 5, 102)
+    s = scales_for(64, 103)
+    d = capi.Conv2dDesc(112, 64, 64, 56, 56, 3, 3, 56, 56, 1, 1, 1, 1, 1, 1, 1, 1)
+    import gpu_util
+    assert capi.conv2d_fwd_plan(capi.OP_CONV2D_FWD_I8, d, capi.EPI_RELU_MUL2_CLAMP, 0)[0] == \
+        gpu_util.conv_instance(capi.OP_CONV2D_FWD_I8, "Patch")
+    np.testing.assert_array_equal(_conv(x, w, s, "relu", (1, 1), (1, 1)),
+                                  fast.conv2d_fwd_i8_mul2_clamp(x, w, s, True, (1, 1), (1, 1), (1, 1)))
+    x = uniform_int8((32, 56, 56, 256), -5, 5, 104)
+    w = uniform_int8((512, 1, 1, 256), -5, 5, 105)
+    s = scales_for(512, 106)
+    d = capi.Conv2dDesc(32, 512, 256, 56, 56, 1, 1, 28, 28, 2, 2, 1, 1, 0, 0, 0, 0)
+    assert capi.conv2d_fwd_plan(capi.OP_CONV2D_FWD_I8, d, capi.EPI_MUL2_CLAMP, 0)[0] == \
+        gpu_util.conv_instance(capi.OP_CONV2D_FWD_I8, "Pointwise")
+    np.testing.assert_array_equal(_conv(x, w, s, "passthrough", (2, 2), (0, 0)),
+                                  fast.conv2d_fwd_i8_mul2_clamp(x, w, s, False, (2, 2), (1, 1), (0, 0)))
 
 
 def test_refused_arguments():
