@@ -215,6 +215,14 @@ Plan make_plan(long M, int N, int kbytes, int only_tile, long workspace_bytes, i
             const int nst  = t.lds / ((t.bm + t.bn) * 128);
             const double floor_us = nst > 2 ? 0.30 : 0.42; // (four stages: 0.33 measured over 32 K tiles, 0.26 over 64)
             iter_us        = iter_us < floor_us ? floor_us : iter_us;
+            // three and more co-resident workgroups pull their K tiles through ONE CU's load path: 105 GB/s out of L2
+            // with every CU busy (measured with a streaming probe), 85 in a kernel that also computes. Without this term
+            // 128 x 64 tiles at three per CU were rated 43 us on fp16 512 x 11008 x 4096 and took 60 (256 x 128: 48).
+            if(per_cu >= 3)
+            {
+                const double load_us = per_cu * (double)(t.bm + t.bn) * 128.0 / 85.0e3;
+                iter_us              = iter_us < load_us ? load_us : iter_us;
+            }
             double us      = rounds * (iter_us * nk_per + 6.0 / per_cu + 2.0);
             // a single, partly filled round of one four-stage workgroup per CU: measured fixed cost ~4 us, not 8 (M = 64,
             // N = 11008, K = 4096 int8 on the four-stage 64 x 64 tile: 14.4 us = 3.8 + 0.33 per K tile; the 8 sent
@@ -227,7 +235,7 @@ Plan make_plan(long M, int N, int kbytes, int only_tile, long workspace_bytes, i
                 // promise a clear win: the single-pass estimate is the better calibrated one
                 us += 3.0 + (sp + 0.25) * M * (double)N * 4 / 2.0e6;
                 if(force <= 0)
-                    us *= 1.25;
+                    us *= 1.5;
             }
             if(us < best_us)
                 best_us = us, best.tile = i, best.ksplit = sp, best.nk_per = nk_per;
@@ -399,9 +407,9 @@ int check_gemm_shape(int dt, int M, int N, int K, int sa, int sb, int sc, int al
 long gemm_workspace_bytes(int dt, int M, int N, int K, int instance)
 {
     const int es = dt == ckx::DT_I8 ? 1 : 2;
-    // (up to 32 rows go to the skinny kernels, which take none -- except few columns under a long K: see run_gemm)
+    // (up to 16 rows go to the skinny kernels, which take none -- except few columns under a long K: see run_gemm)
     const bool few_cols = M >= 8 && (N + 15) / 16 < (M > 16 ? 257 : 128) && (long)K * es >= 16384;
-    if(M <= 0 || N <= 0 || (instance == CKX_INSTANCE_AUTO && M <= 32 && !few_cols) || instance >= kNumTiles ||
+    if(M <= 0 || N <= 0 || (instance == CKX_INSTANCE_AUTO && M <= 16 && !few_cols) || instance >= kNumTiles ||
        ((long)K * es) % 16)
         return 0;
     const Plan pl = make_plan(M, N, K * es, instance, 1l << 60);
@@ -461,9 +469,11 @@ GemmChoice choose_gemm(int dt, int M, int N, int K, bool kmajor, int instance, l
     if(instance >= kNumTiles)
         return GemmChoice{instance, 1, nk};
     const bool ws = workspace_bytes > 0;
-    // 33..64 rows: the tile kernel wins when its C tiles fill the machine, or C tiles x K runs over a long K
+    // 17..64 rows: the tile kernel wins when its C tiles fill the machine, or C tiles x K runs over a long K
+    // (17..32 rows since the re-measured audit: fp16 32 x 11008 x 4096 18.3 us on the four-stage 64 x 64 tile against
+    // 25.4 on the widest skinny instance, int8 13.8 against 14.3)
     // (64 x 4096 x 11008: 20 against 27 us; at K = 4096 the 64-row skinny instance is ahead, 11.8 against 13.0 us)
-    const bool tile64 = kmajor || (M > 32 && M <= 64 &&
+    const bool tile64 = kmajor || (M > 16 && M <= 64 &&
                                    ((N + 63) / 64 >= 160 ||
                                     (ws && (long)K * es >= 8192 && make_plan(M, N, K * es, -1, workspace_bytes).ksplit > 1)));
     // few columns and a long K: the skinny kernels have N / 16 workgroups with all of K each, the tile kernel can cut K

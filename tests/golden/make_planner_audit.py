@@ -5,7 +5,8 @@
 
 For every problem of a grid (int8 requant and fp16 GEMMs, A row-major, B column-major, LLM-like and square shapes
 from 1 to 4096 rows; the ResNet-like conv layers of the benchmark) every instance that supports the problem is
-timed with the workspace its own plan asks for: settled clocks, 200 launches replayed from a HIP graph, HIP events.
+timed with the workspace its own plan asks for: graph-replayed launches in 8 ms blocks until two blocks agree within
+3 %, then the least of three more blocks (HIP events).
 The file keeps microseconds per instance and the K runs the instance's plan used, so that the CPU test
 tests/test_planner.py can hold the automatic choice (ckx_gemm_plan / ckx_conv2d_fwd_plan, pure host logic) against
 the best measured instance without a GPU.
@@ -27,7 +28,10 @@ CONV = [(64, 64, 3, 56, 1, 1), (256, 512, 1, 56, 2, 0), (512, 512, 3, 7, 1, 1), 
         (256, 256, 3, 14, 1, 1), (64, 256, 1, 56, 1, 0), (1024, 2048, 1, 14, 2, 0)]
 
 
-def time_launch(launch, steps=200, settle_ms=20.0):
+def time_launch(launch, block_ms=8.0, max_settle_ms=400.0):
+    """microseconds per launch: launches replayed from a HIP graph in blocks of about block_ms; blocks run until two in
+    a row agree within 3 % (the clock governor has settled on this kernel: a light kernel is clocked down, and a
+    cold one is clocked low), then the least of three more blocks counts."""
     import torch
     launch()
     torch.cuda.synchronize()
@@ -36,21 +40,32 @@ def time_launch(launch, steps=200, settle_ms=20.0):
         for _ in range(20):
             launch()
     e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    t0 = time.perf_counter()
-    while (time.perf_counter() - t0) * 1e3 < settle_ms:
-        g.replay()
-    torch.cuda.synchronize()
-    e0.record()
-    for _ in range(steps // 20):
-        g.replay()
-    e1.record()
-    torch.cuda.synchronize()
-    return e0.elapsed_time(e1) / steps * 1e3
+
+    def block(replays):
+        e0.record()
+        for _ in range(replays):
+            g.replay()
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) / (20 * replays) * 1e3
+
+    us = block(2)
+    replays = max(2, int(block_ms * 1e3 / (20 * us)))
+    t0, prev = time.perf_counter(), block(replays)
+    while (time.perf_counter() - t0) * 1e3 < max_settle_ms:
+        cur = block(replays)
+        if abs(cur - prev) <= 0.03 * prev:
+            break
+        prev = cur
+    return min(block(replays) for _ in range(3))
 
 
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--quick", action="store_true", help="a fifth of the grid (smoke run of this script)")
+    ap.add_argument("--only", default="i8,f16,conv",
+                    help="comma-separated parts to measure: i8 (int8 GEMM rows), f16 (fp16 GEMM rows), conv; parts "
+                         "measured in separate runs are merged by hand (same keys)")
     ap.add_argument("--out", default=None, help="where to write the table (default: planner_audit.json beside this script)")
     args = ap.parse_args()
     import torch
@@ -60,11 +75,12 @@ def main():
     stream = lambda: torch.cuda.current_stream().cuda_stream
     out = {"device": torch.cuda.get_device_name(0), "library": L.ckx_version().decode(),
            "auto": "the automatic choice [instance, K runs] of the library that was measured, with 256 MiB of workspace on offer",
-           "protocol": "per instance: clocks settled, 200 graph-replayed launches, HIP events, microseconds",
+           "protocol": "per instance: graph-replayed launches in 8 ms blocks until two agree within 3 %, then the least of three more blocks, HIP events, microseconds",
            "gemm": [], "conv": []}
     n_inst = L.ckx_num_instances(capi.OP_GEMM_I8)
     ws = torch.empty(256 << 20, dtype=torch.uint8, device="cuda")
-    grid = [(kind, M, N, K) for kind in ("i8", "f16") for (N, K) in GEMM_NK for M in GEMM_M]
+    only = set(args.only.split(","))
+    grid = [(kind, M, N, K) for kind in ("i8", "f16") if kind in only for (N, K) in GEMM_NK for M in GEMM_M]
     if args.quick:
         grid = grid[::5]
     for kind, M, N, K in grid:
@@ -97,7 +113,7 @@ def main():
         out["gemm"].append(row)
         print(row, flush=True)
     n_conv = L.ckx_num_instances(capi.OP_CONV2D_FWD_I8)
-    cgrid = [(kind, n, *layer) for kind in ("i8", "f16") for n in (32, 256) for layer in CONV]
+    cgrid = [(kind, n, *layer) for kind in ("i8", "f16") for n in (32, 256) for layer in CONV] if "conv" in only else []
     if args.quick:
         cgrid = cgrid[::5]
     for kind, Nb, C_, K, f, HW, st_, pd in cgrid:
