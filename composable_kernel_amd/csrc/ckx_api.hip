@@ -473,7 +473,10 @@ GemmChoice choose_gemm(int dt, int M, int N, int K, bool kmajor, int instance, l
     // (17..32 rows since the re-measured audit: fp16 32 x 11008 x 4096 18.3 us on the four-stage 64 x 64 tile against
     // 25.4 on the widest skinny instance, int8 13.8 against 14.3)
     // (64 x 4096 x 11008: 20 against 27 us; at K = 4096 the 64-row skinny instance is ahead, 11.8 against 13.0 us)
-    const bool tile64 = kmajor || (M > 16 && M <= 64 &&
+    // (fp16, 8..16 rows, many columns and a long K: HBM streaming either way, and the skinny kernels' A re-reads out of
+    // L2 show -- 16 x 11008 x 4096 fp16: 21.6 us against 18.2 on the four-stage tile; int8 stays: 12.2 against 13.8)
+    const bool f16_long = es == 2 && M >= 8 && M <= 64 && (long)K * es >= 8192 && (N + 63) / 64 >= 160;
+    const bool tile64 = kmajor || f16_long || (M > 16 && M <= 64 &&
                                    ((N + 63) / 64 >= 160 ||
                                     (ws && (long)K * es >= 8192 && make_plan(M, N, K * es, -1, workspace_bytes).ksplit > 1)));
     // few columns and a long K: the skinny kernels have N / 16 workgroups with all of K each, the tile kernel can cut K
