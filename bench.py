@@ -375,10 +375,35 @@ def cpu_baseline(w, threads=None, budget_seconds=30.0):
     dt = time.perf_counter() - t0
     unit = "TFLOP/s" if w["dtype"] == "f16" else "TOP/s"
     what = "the whole" if rows == w["M"] else f"{rows} of {w['M']} rows of the same"
-    return {"value": 2.0 * rows * N * K / dt / 1e12, "unit": unit, "cores": threads, "kind": "port",
+    port = {"value": 2.0 * rows * N * K / dt / 1e12, "unit": unit, "cores": threads, "kind": "port",
             "host_cores": os.cpu_count(), "cpu_model": _cpu_model(),
             "sample": f"{what} {w['M']}x{N}x{K} problem, literal ReferenceGemm restatement "
                       f"(oracle/ck_oracle.cpp), {threads} threads, {dt:.1f} s"}
+    # The reference's OWN host operator (ReferenceGemm compiled in place from the reference tree into oracle/_ref,
+    # where that build exists): slower than the restatement (tensor accessors through descriptors), so a row sample
+    # sized for about ten seconds. It starts std::thread::hardware_concurrency() threads whatever the job may use.
+    import oracle
+    ref = oracle.load_ref()
+    if ref is None:
+        return port
+    ref_run = (lambda a: ref.gemm_f16(a, b.T)) if w["dtype"] == "f16" else \
+              (lambda a: ref.gemm_i8_requant(a, b.T, lit.EPI_REQUANT_RND, 0.5, 0.03))
+    m0 = min(w["M"], 64)
+    t0 = time.perf_counter()
+    ref_run(mk(m0))
+    dt0 = max(time.perf_counter() - t0, 1e-4)
+    rrows = int(min(w["M"], max(m0, m0 * 10.0 / dt0)))
+    a = mk(rrows)
+    t0 = time.perf_counter()
+    ref_run(a)
+    rdt = time.perf_counter() - t0
+    what = "the whole" if rrows == w["M"] else f"{rrows} of {w['M']} rows of the same"
+    return {"value": 2.0 * rrows * N * K / rdt / 1e12, "unit": unit, "cores": min(threads, os.cpu_count() or threads),
+            "kind": "reference", "reference_threads": os.cpu_count(), "host_cores": os.cpu_count(),
+            "cpu_model": _cpu_model(),
+            "sample": f"{what} {w['M']}x{N}x{K} problem, the reference's ReferenceGemm host operator compiled in place "
+                      f"(oracle/_ref), {rdt:.1f} s; it starts one thread per host CPU, this job may use {threads}",
+            "port": port}
 
 
 def main():
