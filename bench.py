@@ -67,12 +67,15 @@ def _conv3d_workload(name, dtype, C, K, f, DHW, st, pd, N, dil=1):
 
 
 def _gemm_workload(name, dtype, M, N, K, values=5, scales=(0.5, 0.03), fused=None, batch=1, layout="mk_nk", init="uniform"):
-    """fused: None or "bias_relu" (fp16: E = AddRelu(half(A*B), bias row)); batch > 1: strided batched GEMM;
+    """fused: None, "bias_relu" (fp16: E = AddRelu(half(A*B), bias row)), "bilinear" (E = alpha * A*B + beta * D, D a
+    full [M,N] tensor, example 02) or "add_add_fastgelu" (E = fast_gelu(A*B + bias row + D1), example 04);
+    batch > 1: strided batched GEMM;
     layout: how A ("mk" row-major / "km" column-major) and B ("nk" column-major / "kn" row-major) are stored."""
     es = 1 if dtype == "i8" else 2
+    d_elems = {None: 0, "bias_relu": N, "bilinear": M * N, "add_add_fastgelu": N + M * N}[fused]
     return dict(name=name, kind="gemm", dtype=dtype, M=M, N=N, K=K, values=values, scales=scales, batch=batch,
                 layout=layout, init=init,
-                ops=2.0 * M * N * K * batch, bytes=(M * K + N * K + M * N + (N if fused else 0)) * es * batch,
+                ops=2.0 * M * N * K * batch, bytes=(M * K + N * K + M * N + d_elems) * es * batch,
                 fused=fused)
 
 
@@ -91,6 +94,8 @@ for w in (
     + [_gemm_workload(f"fp16_gemm_4096_{lay}", "f16", 4096, 4096, 4096, layout=lay) for lay in ("km_kn", "km_nk", "mk_kn")]
     + [_gemm_workload(f"int8_requant_gemm_4096_{lay}", "i8", 4096, 4096, 4096, layout=lay) for lay in ("km_kn", "km_nk", "mk_kn")]
     + [_gemm_workload("fp16_gemm_bias_relu_4096", "f16", 4096, 4096, 4096, fused="bias_relu"),
+       _gemm_workload("fp16_gemm_bilinear_4096", "f16", 4096, 4096, 4096, fused="bilinear"),
+       _gemm_workload("fp16_gemm_add_add_fastgelu_4096", "f16", 4096, 4096, 4096, fused="add_add_fastgelu"),
        _gemm_workload("fp16_gemm_4096_integer_init", "f16", 4096, 4096, 4096, init="integer"),
        _conv_workload("conv_f16_c64_k64_3x3_56_bias_relu_add", "f16", 64, 64, 3, 56, 1, 1, fused="bias_relu_add"),
        _conv_workload("conv_f16_c256_k512_1x1_56_s2_bias_relu", "f16", 256, 512, 1, 56, 2, 0, fused="bias_relu")]
@@ -163,6 +168,15 @@ def make_launcher(w, instance=-1, rotate=1):
             bias = dev(uniform_f16((N,), -1, 1, 9))
             op = ck.DeviceGemmMultipleDF16(instance)
             make = lambda bb: op.MakeArgumentPointer(a, bb, [bias], c, M, N, K, K, K, [0], N, None, None, ck.AddRelu())
+        elif w.get("fused") in ("bilinear", "add_add_fastgelu"):
+            bias, full = dev(uniform_f16((N,), -1, 1, 9)), dev(uniform_f16((M, N), -1, 1, 10))
+            op = ck.DeviceGemmMultipleDF16(instance)
+            if w["fused"] == "bilinear":
+                make = lambda bb: op.MakeArgumentPointer(a, bb, [full], c, M, N, K, K, K, [N], N, None, None,
+                                                         ck.Bilinear(0.5, 1.5))
+            else:
+                make = lambda bb: op.MakeArgumentPointer(a, bb, [bias, full], c, M, N, K, K, K, [0, N], N, None, None,
+                                                         ck.AddAddFastGelu())
         else:
             make = lambda bb: op.MakeArgumentPointer(a, bb, c, M, N, K, sa, sb, N, None, None, cop)
         arg = make(b)

@@ -8,7 +8,7 @@
 """
 from . import capi, device_ops, host_tensor  # noqa: F401
 from .device_ops import (  # noqa: F401
-    PassThrough, Scale, RequantReluRequant, AddRelu, AddReluAdd, Relu, ActivationMul2Clamp, RowMajor, ColumnMajor, StreamConfig,
+    PassThrough, Scale, RequantReluRequant, AddRelu, AddReluAdd, Bilinear, AddAddFastGelu, Relu, ActivationMul2Clamp, RowMajor, ColumnMajor, StreamConfig,
     DeviceGemmInt8, DeviceGemmF16, DeviceGemmBF16, DeviceGemmSplitKInt8, DeviceGemmSplitKF16, DeviceBatchedGemmInt8, DeviceBatchedGemmF16, DeviceGemmMultipleDF16, DeviceGemmMultipleDInt8,
     DeviceConv2dFwdInt8, DeviceConv2dFwdMultipleDInt8, DeviceConv2dFwdF16,
     DeviceConvNdFwdInt8, DeviceConvNdFwdF16,

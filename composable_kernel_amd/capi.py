@@ -16,6 +16,7 @@ ROW_MAJOR, COL_MAJOR = 0, 1
 EPI_PASSTHROUGH, EPI_REQUANT_CK, EPI_REQUANT_RND = 0, 1, 2
 EPI_ADD_RELU, EPI_ADD_RELU_ADD, EPI_CSHUFFLE_ADD_RELU = 3, 4, 5
 EPI_MUL2_CLAMP, EPI_RELU_MUL2_CLAMP = 6, 7   # int8, one fp32 requant scale per output column as the D operand
+EPI_BILINEAR, EPI_ADD_ADD_FASTGELU = 8, 9    # fp16 GEMM: alpha * acc + beta * d0; fast_gelu(acc + d0 + d1)
 (OP_GEMM_I8, OP_GEMM_F16, OP_CONV2D_FWD_I8, OP_CONV2D_FWD_F16, OP_BATCHED_GEMM_GEMM, OP_GEMM_SPLITK, OP_GEMM_BF16,
  OP_BATCHED_GEMM_SOFTMAX_GEMM) = range(8)
 INSTANCE_AUTO = -1
@@ -29,7 +30,7 @@ SYMBOLS = [
     "ckx_gemm_bf16_is_supported", "ckx_gemm_bf16", "ckx_gemm_bf16_workspace_bytes",
     "ckx_batched_gemm_is_supported", "ckx_batched_gemm_i8", "ckx_batched_gemm_f16",
     "ckx_gemm_splitk_workspace_bytes", "ckx_gemm_i8_splitk", "ckx_gemm_f16_splitk", "ckx_gemm_i8_splitk_noalloc",
-    "ckx_gemm_f16_multiple_d_is_supported", "ckx_gemm_f16_multiple_d", "ckx_conv2d_fwd_bias_activation_f16",
+    "ckx_gemm_f16_multiple_d_is_supported", "ckx_gemm_f16_multiple_d", "ckx_gemm_f16_bilinear", "ckx_conv2d_fwd_bias_activation_f16",
     "ckx_gemm_i8_multiple_d_is_supported", "ckx_gemm_i8_multiple_d", "ckx_conv2d_fwd_i8_multiple_d",
     "ckx_conv2d_fwd_is_supported", "ckx_conv2d_fwd_i8", "ckx_conv2d_fwd_f16", "ckx_conv2d_fwd_workspace_bytes",
     "ckx_convnd_fwd_is_supported", "ckx_convnd_fwd", "ckx_convnd_fwd_workspace_bytes",
@@ -115,6 +116,7 @@ def lib():
     L.ckx_gemm_f16_multiple_d_is_supported.argtypes = md + [C.c_int, C.c_int]
     L.ckx_gemm_f16_multiple_d.argtypes = [vp] * 5 + md + [C.c_int, C.c_int, vp, i64, vp]
     mdi = [i32] * 7 + [C.c_int] * 3
+    L.ckx_gemm_f16_bilinear.argtypes = [vp] * 4 + mdi + [C.c_float, C.c_float, C.c_int, vp, i64, vp]
     L.ckx_gemm_i8_multiple_d_is_supported.argtypes = mdi + [C.c_int, C.c_int]
     L.ckx_gemm_i8_multiple_d.argtypes = [vp] * 4 + mdi + [C.c_int, C.c_int, vp, i64, vp]
     dp = C.POINTER(Conv2dDesc)

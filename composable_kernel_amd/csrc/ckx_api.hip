@@ -325,7 +325,14 @@ struct DOperands
 };
 
 // the fp16 add / ReLU functors with fp16 D operands; the int8 functors with a per-column fp32 scale row as D0
-bool f16_fused(int epi) { return epi >= CKX_EPI_ADD_RELU && epi <= CKX_EPI_CSHUFFLE_ADD_RELU; }
+bool f16_fused(int epi)
+{
+    return (epi >= CKX_EPI_ADD_RELU && epi <= CKX_EPI_CSHUFFLE_ADD_RELU) || epi == CKX_EPI_BILINEAR ||
+           epi == CKX_EPI_ADD_ADD_FASTGELU;
+}
+bool uses_d1(int epi) { return epi == CKX_EPI_ADD_RELU_ADD || epi == CKX_EPI_ADD_ADD_FASTGELU; }
+// the CDE operations of ckx_gemm_f16_multiple_d (the bilinear one has its scalars and its own entry point)
+bool f16_cde_op(int epi) { return f16_fused(epi) && epi != CKX_EPI_BILINEAR; }
 bool per_column_scale(int epi) { return epi == CKX_EPI_MUL2_CLAMP || epi == CKX_EPI_RELU_MUL2_CLAMP; }
 
 bool epilogue_fits_dtype(int es, int epi)
@@ -349,9 +356,9 @@ int check_d_operands(int epi, int N, const DOperands& d)
             return fail(CKX_UNSUPPORTED, "operands must be aligned to their element size");
         return CKX_OK;
     }
-    if(!d.d0 || (epi == CKX_EPI_ADD_RELU_ADD && !d.d1))
+    if(!d.d0 || (uses_d1(epi) && !d.d1))
         return fail(CKX_INVALID_VALUE, "null D operand pointer");
-    if((d.ldd0 != 0 && d.ldd0 < N) || (epi == CKX_EPI_ADD_RELU_ADD && d.ldd1 != 0 && d.ldd1 < N) || d.ldd0 < 0 ||
+    if((d.ldd0 != 0 && d.ldd0 < N) || (uses_d1(epi) && d.ldd1 != 0 && d.ldd1 < N) || d.ldd0 < 0 ||
        d.ldd1 < 0)
         return fail(CKX_UNSUPPORTED, "D stride must be 0 (broadcast row) or at least N");
     return CKX_OK;
@@ -376,7 +383,7 @@ int check_gemm_shape(int dt, int M, int N, int K, int sa, int sb, int sc, int al
         return fail(CKX_INVALID_VALUE, "no such instance");
     if(instance >= kNumTiles && instance < kGenericGemmInstance && M > kSkinny[instance - kNumTiles].max_m)
         return fail(CKX_UNSUPPORTED, "this skinny instance covers fewer rows than M");
-    if(epi < CKX_EPI_PASSTHROUGH || epi > CKX_EPI_RELU_MUL2_CLAMP)
+    if(epi < CKX_EPI_PASSTHROUGH || epi > CKX_EPI_ADD_ADD_FASTGELU)
         return fail(CKX_INVALID_VALUE, "unknown epilogue");
     if(!epilogue_fits_dtype(es, epi) || (dt == ckx::DT_BF16 && epi != CKX_EPI_PASSTHROUGH))
         return fail(CKX_UNSUPPORTED, "epilogue not available for this dtype");
@@ -543,7 +550,7 @@ int run_gemm(int dt, const void* a, const void* b, void* c, int M, int N, int K,
         g.lda = sa, g.ldb = sb, g.ldc = sc;
         g.batch = batch, g.bsa = bsa, g.bsb = bsb, g.bsc = bsc;
         g.epi = epi, g.scale_gemm = sg, g.scale_relu = sr;
-        g.d0 = dops.d0, g.d1 = epi == CKX_EPI_ADD_RELU_ADD ? dops.d1 : nullptr;
+        g.d0 = dops.d0, g.d1 = uses_d1(epi) ? dops.d1 : nullptr;
         g.ldd0 = dops.ldd0, g.ldd1 = dops.ldd1;
         g.ksplit  = 1;
         g.tiles_m = (M + 63) / 64, g.tiles_n = (N + 63) / 64;
@@ -580,7 +587,7 @@ int run_gemm(int dt, const void* a, const void* b, void* c, int M, int N, int K,
     g.scale_gemm = sg;
     g.scale_relu = sr;
     g.nt_store   = es == 1 && (long)M * N * es >= stream_output_bytes();
-    g.d0 = dops.d0, g.d1 = epi == CKX_EPI_ADD_RELU_ADD ? dops.d1 : nullptr;
+    g.d0 = dops.d0, g.d1 = uses_d1(epi) ? dops.d1 : nullptr;
     g.ldd0 = dops.ldd0, g.ldd1 = dops.ldd1;
     g.ksplit     = 1;
     if(ti >= kNumTiles)
@@ -772,7 +779,7 @@ int run_conv(int op, const void* in, const void* wei, void* out, const ckx_conv2
         g.M = M, g.N = N, g.K = K;
         g.ldb = K, g.ldc = N;
         g.epi = epi, g.scale_gemm = sg, g.scale_relu = sr;
-        g.d0 = dops.d0, g.d1 = epi == CKX_EPI_ADD_RELU_ADD ? dops.d1 : nullptr;
+        g.d0 = dops.d0, g.d1 = uses_d1(epi) ? dops.d1 : nullptr;
         g.ldd0 = dops.ldd0, g.ldd1 = dops.ldd1;
         g.ksplit  = 1;
         g.tiles_m = (M + 63) / 64, g.tiles_n = (N + 63) / 64;
@@ -854,7 +861,7 @@ int run_conv(int op, const void* in, const void* wei, void* out, const ckx_conv2
     g.scale_gemm = sg;
     g.scale_relu = sr;
     g.nt_store   = es == 1 && (long)M * N * es >= stream_output_bytes();
-    g.d0 = dops.d0, g.d1 = epi == CKX_EPI_ADD_RELU_ADD ? dops.d1 : nullptr;
+    g.d0 = dops.d0, g.d1 = uses_d1(epi) ? dops.d1 : nullptr;
     g.ldd0 = dops.ldd0, g.ldd1 = dops.ldd1;
     g.cv.Hi = d->Hi, g.cv.Wi = d->Wi, g.cv.C = d->C;
     g.cv.sH = d->stride_h, g.cv.sW = d->stride_w, g.cv.dH = d->dilation_h, g.cv.dW = d->dilation_w;
@@ -1282,7 +1289,7 @@ int ckx_batched_gemm_f16(const void* a, const void* b, void* c, int32_t M, int32
 int ckx_gemm_f16_multiple_d_is_supported(int32_t M, int32_t N, int32_t K, int32_t sa, int32_t sb, int32_t sd0,
                                          int32_t sd1, int32_t se, int al, int bl, int el, int cde_op, int instance)
 {
-    if(cde_op < CKX_EPI_ADD_RELU || cde_op > CKX_EPI_CSHUFFLE_ADD_RELU)
+    if(!f16_fused(cde_op))
         return fail(CKX_INVALID_VALUE, "not a CDE element-wise operation");
     int st = check_gemm_shape(ckx::DT_F16, M, N, K, sa, sb, se, al, bl, el, cde_op, instance);
     if(st != CKX_OK)
@@ -1298,12 +1305,22 @@ int ckx_gemm_f16_multiple_d(const void* a, const void* b, const void* d0, const 
                             int al, int bl, int el, int cde_op, int instance, void* workspace,
                             int64_t workspace_bytes, void* stream)
 {
-    if(cde_op < CKX_EPI_ADD_RELU || cde_op > CKX_EPI_CSHUFFLE_ADD_RELU)
+    if(!f16_cde_op(cde_op))
         return fail(CKX_INVALID_VALUE, "not a CDE element-wise operation");
     DOperands d;
     d.d0 = d0, d.d1 = d1, d.ldd0 = sd0, d.ldd1 = sd1;
     return run_gemm(ckx::DT_F16, a, b, e, M, N, K, sa, sb, se, al, bl, el, cde_op, 1.0f, 1.0f, instance, workspace,
                     workspace_bytes, stream, d);
+}
+
+int ckx_gemm_f16_bilinear(const void* a, const void* b, const void* d0, void* e, int32_t M, int32_t N, int32_t K,
+                          int32_t sa, int32_t sb, int32_t sd, int32_t se, int al, int bl, int el, float alpha,
+                          float beta, int instance, void* workspace, int64_t workspace_bytes, void* stream)
+{
+    DOperands d;
+    d.d0 = d0, d.ldd0 = sd;
+    return run_gemm(ckx::DT_F16, a, b, e, M, N, K, sa, sb, se, al, bl, el, CKX_EPI_BILINEAR, alpha, beta, instance,
+                    workspace, workspace_bytes, stream, d);
 }
 
 int ckx_gemm_i8_multiple_d_is_supported(int32_t M, int32_t N, int32_t K, int32_t sa, int32_t sb, int32_t sd0,

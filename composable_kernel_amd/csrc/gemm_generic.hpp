@@ -221,7 +221,8 @@ __global__ __launch_bounds__(256) void gemm_generic_kernel(const GemmArgs p, con
                     float v = acc[i][t][j];
                     if(p.epi != EPI_PASSTHROUGH)
                         v = epi_f16_value(p.epi, v, (float)d0p[m * p.ldd0 + n],
-                                          p.epi == EPI_ADD_RELU_ADD ? (float)d1p[m * p.ldd1 + n] : 0.0f);
+                                          epi_has_d1(p.epi) ? (float)d1p[m * p.ldd1 + n] : 0.0f, p.scale_gemm,
+                                          p.scale_relu);
                     reinterpret_cast<_Float16*>(p.c)[ci] = (_Float16)v;
                 }
             }

@@ -180,8 +180,8 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(const GemmArgs p)
                 {
                     float val = s[j];
                     if(p.epi != EPI_PASSTHROUGH)
-                        val = epi_f16_value(p.epi, val, (float)d0row[j],
-                                            p.epi == EPI_ADD_RELU_ADD ? (float)d1row[j] : 0.0f);
+                        val = epi_f16_value(p.epi, val, (float)d0row[j], epi_has_d1(p.epi) ? (float)d1row[j] : 0.0f,
+                                            p.scale_gemm, p.scale_relu);
                     crow[j] = (_Float16)val;
                 }
         }

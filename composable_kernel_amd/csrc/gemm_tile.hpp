@@ -60,9 +60,14 @@ enum
     // int8 outputs with a per-column fp32 requant scale as the "D" operand (d0 = scale[N]): upstream's
     // element_wise::Activation_Mul2_Clamp<PassThrough / Relu>, e = int8(clamp(scale[n] * act(float(acc)), -128, 127))
     EPI_MUL2_CLAMP      = 6,
-    EPI_RELU_MUL2_CLAMP = 7
+    EPI_RELU_MUL2_CLAMP = 7,
+    // fp16 outputs again (GEMM only; the two scalars travel in scale_gemm / scale_relu):
+    EPI_BILINEAR         = 8, // e = half(alpha * acc + beta * d0)
+    EPI_ADD_ADD_FASTGELU = 9  // e = half(fast_gelu(acc + d0 + d1))
 };
 __host__ __device__ constexpr bool epi_per_column_scale(int epi) { return epi == EPI_MUL2_CLAMP || epi == EPI_RELU_MUL2_CLAMP; }
+// fp16 epilogues that read a second D tensor
+__host__ __device__ constexpr bool epi_has_d1(int epi) { return epi == EPI_ADD_RELU_ADD || epi == EPI_ADD_ADD_FASTGELU; }
 
 // C tile stores: plain, or streaming (non-temporal) when the output is too large to be worth
 // keeping in L2: dirty lines of a streamed output otherwise queue up behind the write-back
@@ -409,8 +414,24 @@ __device__ __forceinline__ void load_col_scales(const __amdgpu_buffer_rsrc_t& rs
 // include/ck/tensor_operation/gpu/element/{binary_,}element_wise_operation.hpp as the host
 // references apply them: reference_conv_fwd_bias_activation[_add].hpp on the fp32 accumulator,
 // example/03_gemm_bias_relu on the accumulator already rounded to fp16).
-__device__ __forceinline__ float epi_f16_value(int mode, float acc, float d0, float d1)
+// EXT = false leaves the scaled / GELU modes out of the generated code (callers that have already branched on them).
+// fast_gelu(x) = x / (1 + exp(-2x(0.035677 x^2 + 0.797885))), the closed form of the reference's
+// 0.5 + 0.5 * (2 / (1 + emu) - 1) (element_wise_operation.hpp:127-133); x -> -inf gives exp -> +inf and -0.
+template <bool EXT = true>
+__device__ __forceinline__ float epi_f16_value(int mode, float acc, float d0, float d1, float alpha = 1.0f,
+                                               float beta = 1.0f)
 {
+    if constexpr(EXT)
+    {
+        if(mode == EPI_BILINEAR)
+            return alpha * acc + beta * d0;
+        if(mode == EPI_ADD_ADD_FASTGELU)
+        {
+            const float x = acc + d0 + d1;
+            const float u = 2.0f * x * (0.035677f * x * x + 0.797885f);
+            return x / (1.0f + __expf(-u));
+        }
+    }
     if(mode == EPI_CSHUFFLE_ADD_RELU)
     {
         const float x = (float)(_Float16)((float)(_Float16)acc + d0);
@@ -425,7 +446,7 @@ __device__ __forceinline__ float epi_f16_value(int mode, float acc, float d0, fl
 // row's D values (d1row may be null)
 __device__ __forceinline__ void store_row16_f16_fused(_Float16* crow, int n0, int N, bool vec_ok, f32x4 (&v)[4],
                                                       int mode, const _Float16* d0row, const _Float16* d1row,
-                                                      bool dvec_ok, bool nt);
+                                                      bool dvec_ok, bool nt, float alpha, float beta);
 
 // T = _Float16 or __bf16
 template <typename T>
@@ -460,9 +481,9 @@ __device__ __forceinline__ void store_row16_f16(T* crow, int n0, int N, bool vec
 
 __device__ __forceinline__ void store_row16_f16_fused(_Float16* crow, int n0, int N, bool vec_ok, f32x4 (&v)[4],
                                                       int mode, const _Float16* d0row, const _Float16* d1row,
-                                                      bool dvec_ok, bool nt)
+                                                      bool dvec_ok, bool nt, float alpha, float beta)
 {
-    const bool has_d1 = mode == EPI_ADD_RELU_ADD;
+    const bool has_d1 = epi_has_d1(mode);
     if(dvec_ok && n0 + 16 <= N)
     {
         const f16x8 z   = {0, 0, 0, 0, 0, 0, 0, 0};
@@ -477,7 +498,7 @@ __device__ __forceinline__ void store_row16_f16_fused(_Float16* crow, int n0, in
             {
                 const int e = t * 4 + j;
                 v[t][j]     = epi_f16_value(mode, v[t][j], (float)(e < 8 ? b_lo[e] : b_hi[e - 8]),
-                                            (float)(e < 8 ? r_lo[e] : r_hi[e - 8]));
+                                            (float)(e < 8 ? r_lo[e] : r_hi[e - 8]), alpha, beta);
             }
     }
     else
@@ -489,7 +510,7 @@ __device__ __forceinline__ void store_row16_f16_fused(_Float16* crow, int n0, in
             {
                 const int n = n0 + t * 4 + j;
                 if(n < N)
-                    v[t][j] = epi_f16_value(mode, v[t][j], (float)d0row[n], has_d1 ? (float)d1row[n] : 0.0f);
+                    v[t][j] = epi_f16_value(mode, v[t][j], (float)d0row[n], has_d1 ? (float)d1row[n] : 0.0f, alpha, beta);
             }
     }
     store_row16_f16(crow, n0, N, vec_ok, v, nt);
@@ -1052,10 +1073,14 @@ struct GemmTile
         // a bias row once for the whole tile, per-row tensors (residual) chunk by chunk.
         // (which tensors are per-row is a compile-time property of each variant: registers are only
         // set aside for what is fetched)
-        auto epilogue_fused = [&](int unit, auto chunk_rows, auto d0_row_tensor, auto with_d1) {
+        // (so is the functor family: EXT = false builds the add / ReLU modes alone, EXT = true the scaled and GELU ones)
+        auto epilogue_fused = [&](int unit, auto chunk_rows, auto d0_row_tensor, auto with_d1, auto extended) {
             constexpr int CH          = decltype(chunk_rows)::value < MT ? decltype(chunk_rows)::value : MT;
             constexpr bool d0_per_row = decltype(d0_row_tensor)::value;
             constexpr bool has_d1     = decltype(with_d1)::value;
+            constexpr bool EXT        = decltype(extended)::value;
+            // (with a second D tensor the only extended mode is the GELU one, without it the bilinear one)
+            const int mode = !EXT ? p.epi : has_d1 ? (int)EPI_ADD_ADD_FASTGELU : (int)EPI_BILINEAR;
             int tm, tn, bi; // (the fused epilogues are never combined with a batch)
             tile_of_block(unit % ntiles, p.tiles_m, p.tiles_n, 1, bi, tm, tn);
             const _Float16* d0 = reinterpret_cast<const _Float16*>(p.d0);
@@ -1131,7 +1156,7 @@ struct GemmTile
                                     const float x = d0_per_row ? (float)(e < 8 ? x_lo[cx][g][e & 7] : x_hi[cx][g][e & 7])
                                                                : (float)(e < 8 ? b_lo[g][e & 7] : b_hi[g][e & 7]);
                                     const float y = has_d1 ? (float)(e < 8 ? y_lo[cy][g][e & 7] : y_hi[cy][g][e & 7]) : 0.0f;
-                                    v[t][j]       = epi_f16_value(p.epi, acc[i][g * 4 + t][j], x, y);
+                                    v[t][j] = epi_f16_value<EXT>(mode, acc[i][g * 4 + t][j], x, y, p.scale_gemm, p.scale_relu);
                                 }
                             _Float16* crow = reinterpret_cast<_Float16*>(p.c) + (size_t)m * p.ldc;
                             store_row16_f16(crow, col0(g), p.N, vec_ok, v, nt);
@@ -1241,15 +1266,27 @@ struct GemmTile
                         using std::integral_constant;
                         using std::false_type;
                         using std::true_type;
-                        const bool d0_rows = p.ldd0 != 0, resi = p.epi == EPI_ADD_RELU_ADD;
-                        if(!d0_rows && !resi)
-                            epilogue_fused(unit, integral_constant<int, MT>{}, false_type{}, false_type{});
-                        else if(!d0_rows)
-                            epilogue_fused(unit, integral_constant<int, 2>{}, false_type{}, true_type{});
-                        else if(!resi)
-                            epilogue_fused(unit, integral_constant<int, 2>{}, true_type{}, false_type{});
+                        const bool d0_rows = p.ldd0 != 0, resi = epi_has_d1(p.epi);
+                        auto by_operands = [&](auto extended) {
+                            if(!d0_rows && !resi)
+                                epilogue_fused(unit, integral_constant<int, MT>{}, false_type{}, false_type{}, extended);
+                            else if(!d0_rows)
+                                epilogue_fused(unit, integral_constant<int, 2>{}, false_type{}, true_type{}, extended);
+                            else if(!resi)
+                                epilogue_fused(unit, integral_constant<int, 2>{}, true_type{}, false_type{}, extended);
+                            else
+                                epilogue_fused(unit, integral_constant<int, 1>{}, true_type{}, true_type{}, extended);
+                        };
+                        // (the conv operators take the add / ReLU functors only)
+                        if constexpr(IM2COL == 0)
+                        {
+                            if(p.epi >= EPI_BILINEAR)
+                                by_operands(true_type{});
+                            else
+                                by_operands(false_type{});
+                        }
                         else
-                            epilogue_fused(unit, integral_constant<int, 1>{}, true_type{}, true_type{});
+                            by_operands(false_type{});
                     }
                 }
                 else
@@ -1334,7 +1371,7 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(const GemmArgs p)
             store_row16_f16_fused(crow, n0, p.N, vec_ok, v, p.epi,
                                   reinterpret_cast<const _Float16*>(p.d0) + (size_t)m * p.ldd0,
                                   p.d1 ? reinterpret_cast<const _Float16*>(p.d1) + (size_t)m * p.ldd1 : nullptr,
-                                  dvec_ok, false);
+                                  dvec_ok, false, p.scale_gemm, p.scale_relu);
         }
     }
 }

@@ -63,6 +63,22 @@ class AddReluAdd:
     cde_epilogue = capi.EPI_ADD_RELU_ADD
 
 
+class Bilinear:
+    """element_wise::Bilinear (binary_element_wise_operation.hpp:93-116): y = half(alpha * x0 + beta * float(x1)) with
+    x0 the fp32 accumulator (example/02_gemm_bilinear/gemm_bilinear_xdl_fp16.cpp:18-36 is the same functor)."""
+    cde_epilogue = capi.EPI_BILINEAR
+
+    def __init__(self, alpha, beta):
+        self.alpha_ = float(alpha)
+        self.beta_ = float(beta)
+
+
+class AddAddFastGelu:
+    """element_wise::AddAddFastGelu (element_wise_operation.hpp:113-140): e = half(fast_gelu(c + d0 + d1)) on the fp32
+    accumulator c, fast_gelu(x) = x * (0.5 + 0.5 * (2 / (1 + exp(-u)) - 1)), u = 2x(0.035677 x^2 + 0.797885)."""
+    cde_epilogue = capi.EPI_ADD_ADD_FASTGELU
+
+
 class Relu:
     """element_wise::Relu (unary_element_wise_operation.hpp): y = x > 0 ? x : 0"""
 
@@ -354,8 +370,10 @@ class DeviceGemmMultipleDF16(BaseOperator):
                             a_element_op=None, b_element_op=None, cde_element_op=None):
         if not 1 <= len(p_ds) <= 2 or len(StrideDs) != len(p_ds):
             raise ValueError("one or two D tensors")
-        if not isinstance(cde_element_op, (AddRelu, AddReluAdd)):
+        if not isinstance(cde_element_op, (AddRelu, AddReluAdd, Bilinear, AddAddFastGelu)):
             raise TypeError("CDE element-wise operation not built")
+        if len(p_ds) != (2 if isinstance(cde_element_op, (AddReluAdd, AddAddFastGelu)) else 1):
+            raise ValueError("number of D tensors does not match the CDE element-wise operation")
         a = _GemmArgument(p_a, p_b, p_e, M, N, K, StrideA, StrideB, StrideE, a_element_op or PassThrough(),
                           b_element_op or PassThrough(), cde_element_op, self.layouts)
         a.p_ds = [_ptr(p) for p in p_ds] + [0] * (2 - len(p_ds))
@@ -371,6 +389,11 @@ class DeviceGemmMultipleDF16(BaseOperator):
         return int(capi.lib().ckx_gemm_f16_workspace_bytes(a.M, a.N, a.K, self.instance))
 
     def _launch(self, a, stream):
+        if isinstance(a.c_op, Bilinear):
+            return capi.lib().ckx_gemm_f16_bilinear(
+                a.p_a, a.p_b, a.p_ds[0], a.p_c, a.M, a.N, a.K, a.StrideA, a.StrideB, a.StrideDs[0], a.StrideC,
+                *self.layouts, a.c_op.alpha_, a.c_op.beta_, self.instance, a.p_workspace_ or 0, a.workspace_bytes_,
+                C.c_void_p(stream or 0))
         return capi.lib().ckx_gemm_f16_multiple_d(
             a.p_a, a.p_b, a.p_ds[0], a.p_ds[1], a.p_c, a.M, a.N, a.K, a.StrideA, a.StrideB, a.StrideDs[0],
             a.StrideDs[1], a.StrideC, *self.layouts, a.c_op.cde_epilogue, self.instance, a.p_workspace_ or 0,

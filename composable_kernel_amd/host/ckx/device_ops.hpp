@@ -139,6 +139,41 @@ struct AddReluAdd
     }
 };
 
+// y = alpha * x0 + beta * x1 in fp32, x0 the fp32 accumulator (binary_element_wise_operation.hpp:93-116)
+struct Bilinear
+{
+    Bilinear(float alpha = 1.f, float beta = 1.f) : alpha_(alpha), beta_(beta) {}
+    template <typename Y, typename X0, typename X1>
+    void operator()(Y& y, const X0& x0, const X1& x1) const
+    {
+        y = static_cast<Y>(alpha_ * static_cast<float>(x0) + beta_ * static_cast<float>(x1));
+    }
+    float alpha_, beta_;
+};
+
+// y = x * cdf, the logistic form of the tanh GELU approximation (unary_element_wise_operation.hpp:121-135)
+struct FastGelu
+{
+    void operator()(float& y, const float& x) const
+    {
+        const float u   = 2.f * x * (0.035677f * x * x + 0.797885f);
+        const float emu = std::exp(-u);
+        y               = x * (0.5f + 0.5f * (2.f / (1.f + emu) - 1.f));
+    }
+};
+
+// e = fast_gelu(c + d0 + d1) on the fp32 accumulator c (element_wise_operation.hpp:113-140)
+struct AddAddFastGelu
+{
+    template <typename E, typename C, typename D0, typename D1>
+    void operator()(E& e, const C& c, const D0& d0, const D1& d1) const
+    {
+        float y;
+        FastGelu{}(y, static_cast<float>(c) + static_cast<float>(d0) + static_cast<float>(d1));
+        e = static_cast<E>(y);
+    }
+};
+
 // y = x > 0 ? x : 0 (unary_element_wise_operation.hpp, Relu)
 struct Relu
 {
@@ -914,8 +949,9 @@ struct DeviceGemmSplitKMfma : public DeviceGemmSplitK<ALayout, BLayout, CLayout,
 };
 
 // ------------------------------------------------ GEMM with fused D operands (fp16)
-// CDE operation: AddRelu (one D: E = relu(half(C) + D0), example 03) or AddReluAdd (two Ds:
-// E = relu(C + D0) + D1 in fp32). A D stride of 0 broadcasts one row (a bias vector).
+// CDE operation: AddRelu (one D: E = relu(half(C) + D0), example 03), AddReluAdd (two Ds: E = relu(C + D0) + D1 in
+// fp32), Bilinear (one D: E = alpha * C + beta * D0, example 02) or AddAddFastGelu (two Ds: E = fast_gelu(C + D0 + D1),
+// example 04). A D stride of 0 broadcasts one row (a bias vector).
 template <typename ALayout, typename BLayout, typename DELayout, typename DsDataType,
           typename CDEElementwiseOperation>
 struct DeviceGemmMultipleDMfma
@@ -924,10 +960,15 @@ struct DeviceGemmMultipleDMfma
 {
     static constexpr index_t NumDTensor = DsDataType::Size();
     static constexpr bool is_add_relu   = std::is_same_v<CDEElementwiseOperation, element_wise::AddRelu>;
-    static_assert((is_add_relu && NumDTensor == 1) ||
-                      (std::is_same_v<CDEElementwiseOperation, element_wise::AddReluAdd> && NumDTensor == 2),
-                  "built CDE operations: AddRelu with one D tensor, AddReluAdd with two");
-    static constexpr int cde_code = is_add_relu ? CKX_EPI_CSHUFFLE_ADD_RELU : CKX_EPI_ADD_RELU_ADD;
+    static constexpr bool is_bilinear   = std::is_same_v<CDEElementwiseOperation, element_wise::Bilinear>;
+    static constexpr bool is_gelu       = std::is_same_v<CDEElementwiseOperation, element_wise::AddAddFastGelu>;
+    static_assert(((is_add_relu || is_bilinear) && NumDTensor == 1) ||
+                      ((std::is_same_v<CDEElementwiseOperation, element_wise::AddReluAdd> || is_gelu) && NumDTensor == 2),
+                  "built CDE operations: AddRelu and Bilinear with one D tensor, AddReluAdd and AddAddFastGelu with two");
+    static constexpr int cde_code = is_add_relu   ? CKX_EPI_CSHUFFLE_ADD_RELU
+                                    : is_bilinear ? CKX_EPI_BILINEAR
+                                    : is_gelu     ? CKX_EPI_ADD_ADD_FASTGELU
+                                                  : CKX_EPI_ADD_RELU_ADD;
     using Pass                    = element_wise::PassThrough;
 
     struct Argument : public BaseArgument
@@ -935,6 +976,7 @@ struct DeviceGemmMultipleDMfma
         const void *p_a, *p_b, *p_d0, *p_d1;
         void* p_e;
         index_t M, N, K, StrideA, StrideB, StrideD0, StrideD1, StrideE;
+        CDEElementwiseOperation cde_element_op_;
     };
     static int Supported(const Argument& a, int inst)
     {
@@ -945,9 +987,15 @@ struct DeviceGemmMultipleDMfma
     static int Launch(const Argument& a, int inst, void* stream)
     {
         const int64_t ws_bytes = a.p_workspace_ ? ckx_gemm_f16_workspace_bytes(a.M, a.N, a.K, inst) : 0;
-        return ckx_gemm_f16_multiple_d(a.p_a, a.p_b, a.p_d0, a.p_d1, a.p_e, a.M, a.N, a.K, a.StrideA, a.StrideB,
-                                       a.StrideD0, a.StrideD1, a.StrideE, ALayout::code, BLayout::code,
-                                       DELayout::code, cde_code, inst, a.p_workspace_, ws_bytes, stream);
+        if constexpr(is_bilinear)
+            return ckx_gemm_f16_bilinear(a.p_a, a.p_b, a.p_d0, a.p_e, a.M, a.N, a.K, a.StrideA, a.StrideB, a.StrideD0,
+                                         a.StrideE, ALayout::code, BLayout::code, DELayout::code,
+                                         a.cde_element_op_.alpha_, a.cde_element_op_.beta_, inst, a.p_workspace_,
+                                         ws_bytes, stream);
+        else
+            return ckx_gemm_f16_multiple_d(a.p_a, a.p_b, a.p_d0, a.p_d1, a.p_e, a.M, a.N, a.K, a.StrideA, a.StrideB,
+                                           a.StrideD0, a.StrideD1, a.StrideE, ALayout::code, BLayout::code,
+                                           DELayout::code, cde_code, inst, a.p_workspace_, ws_bytes, stream);
     }
     using Invoker = detail::InvokerT<Argument, &Supported, &Launch>;
 
@@ -955,9 +1003,10 @@ struct DeviceGemmMultipleDMfma
     static Argument MakeArgument(const void* p_a, const void* p_b, std::array<const void*, NumDTensor> p_ds,
                                  void* p_e, index_t M, index_t N, index_t K, index_t StrideA, index_t StrideB,
                                  std::array<index_t, NumDTensor> StrideDs, index_t StrideE, Pass = {}, Pass = {},
-                                 CDEElementwiseOperation = {})
+                                 CDEElementwiseOperation cde_element_op = {})
     {
         Argument a;
+        a.cde_element_op_ = cde_element_op;
         a.p_a = p_a, a.p_b = p_b, a.p_e = p_e;
         a.p_d0 = p_ds[0], a.StrideD0 = StrideDs[0];
         a.p_d1 = NumDTensor > 1 ? p_ds[NumDTensor - 1] : nullptr, a.StrideD1 = NumDTensor > 1 ? StrideDs[NumDTensor - 1] : 0;
@@ -980,16 +1029,17 @@ struct DeviceGemmMultipleDMfma
     MakeArgumentPointer(const void* p_a, const void* p_b, std::array<const void*, NumDTensor> p_ds, void* p_e,
                         index_t M, index_t N, index_t K, index_t StrideA, index_t StrideB,
                         std::array<index_t, NumDTensor> StrideDs, index_t StrideE, Pass, Pass,
-                        CDEElementwiseOperation) override
+                        CDEElementwiseOperation cde_element_op) override
     {
-        return std::make_unique<Argument>(MakeArgument(p_a, p_b, p_ds, p_e, M, N, K, StrideA, StrideB, StrideDs, StrideE));
+        return std::make_unique<Argument>(MakeArgument(p_a, p_b, p_ds, p_e, M, N, K, StrideA, StrideB, StrideDs, StrideE,
+                                                       Pass{}, Pass{}, cde_element_op));
     }
     std::unique_ptr<BaseInvoker> MakeInvokerPointer() override { return std::make_unique<Invoker>(instance_); }
     std::string GetTypeString() const override
     {
         const std::string base = instance_ == CKX_INSTANCE_AUTO ? std::string("DeviceGemm_f16_f16_f16_mk_nk_mn<auto>")
                                                                 : std::string(ckx_instance_name(CKX_OP_GEMM_F16, instance_));
-        return base + (is_add_relu ? " + AddRelu" : " + AddReluAdd");
+        return base + (is_add_relu ? " + AddRelu" : is_bilinear ? " + Bilinear" : is_gelu ? " + AddAddFastGelu" : " + AddReluAdd");
     }
     int instance_;
 };

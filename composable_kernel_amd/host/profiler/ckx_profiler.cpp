@@ -19,6 +19,10 @@
 //                     BatchCount [nrepeat]   (profiler/src/profile_batched_gemm.cpp; dense batch strides)
 //   ckx_profiler gemm_bias_relu <verify> <init> <log> <time> M N K StrideA StrideB StrideE [nrepeat]
 //                     (example/03_gemm_bias_relu: E = AddRelu(half(A*B), bias row), fp16)
+//   ckx_profiler gemm_bilinear <dtype 1> <layout 0..3> <verify> <init> <log> <time> M N K StrideA StrideB StrideD StrideE
+//                     alpha beta [nrepeat]   (profiler/src/profile_gemm_bilinear.cpp:28-66)
+//   ckx_profiler gemm_add_add_fastgelu <dtype 1> <layout 0..3> <verify> <init> <log> <time> M N K StrideA StrideB
+//                     StrideD0 StrideD1 StrideE [nrepeat]   (profiler/src/profile_gemm_add_add_fastgelu.cpp:29-62)
 //
 // Every instance of the family is run (DeviceOperationInstanceFactory), one "Perf:" line each
 // and a final "Best Perf:" line, in the reference's format (profile_gemm_impl.hpp:176-177,
@@ -676,6 +680,111 @@ int profile_gemm_perchannel_quant(int argc, char* argv[])
                : profile_gemm_perchannel_quant_t<Pass>(verify, init, time_kernel, M, N, K, sa, sb, se, nrepeat);
 }
 
+// E = cde(A * B, D0[, D1]) for the fp16 CDE operations with the reference's own profiler commands: Bilinear (one D
+// tensor) and AddAddFastGelu (two). A D stride of 0 broadcasts one row; a negative stride stands for the dense default.
+template <typename CDE, int NumD, typename AL, typename BL>
+int profile_gemm_cde_l(bool verify, int init, bool time_kernel, int M, int N, int K, int sa, int sb, int sd0, int sd1,
+                       int se, CDE cde, int nrepeat)
+{
+    using T        = half_t;
+    using Ds       = std::conditional_t<NumD == 1, ck::Tuple<T>, ck::Tuple<T, T>>;
+    using DeviceOp = device::DeviceGemmMultipleD<AL, BL, Row, T, T, Ds, T, Pass, Pass, CDE>;
+    auto ops       = device::instance::DeviceOperationInstanceFactory<DeviceOp>::GetInstances();
+    constexpr bool a_row = std::is_same_v<AL, Row>, b_row = std::is_same_v<BL, Row>;
+    sa = sa < 0 ? (a_row ? K : M) : sa, sb = sb < 0 ? (b_row ? N : K) : sb, se = se < 0 ? N : se;
+    sd0 = sd0 < 0 ? N : sd0, sd1 = sd1 < 0 ? N : sd1;
+    std::vector<T> a((std::size_t)(a_row ? M : K) * sa), b((std::size_t)(b_row ? K : N) * sb);
+    std::vector<T> d0(sd0 ? (std::size_t)M * sd0 : (std::size_t)N), d1(sd1 ? (std::size_t)M * sd1 : (std::size_t)N);
+    fill(a, init, 0xC0FFEE, false);
+    fill(b, init, 0xC0FFEE + 1, false);
+    fill(d0, init, 0xC0FFEE + 9, false);
+    fill(d1, init, 0xC0FFEE + 10, false);
+    ckx::DeviceMem da(a.size() * sizeof(T)), db(b.size() * sizeof(T)), dd0(d0.size() * sizeof(T)),
+        dd1(d1.size() * sizeof(T)), de((std::size_t)M * se * sizeof(T));
+    da.ToDevice(a.data());
+    db.ToDevice(b.data());
+    dd0.ToDevice(d0.data());
+    dd1.ToDevice(d1.data());
+    const double flop  = 2.0 * M * N * K;
+    const double bytes = sizeof(T) * ((double)M * K + (double)K * N + (double)M * N + (sd0 ? (double)M * N : (double)N) +
+                                      (NumD > 1 ? (sd1 ? (double)M * N : (double)N) : 0.0));
+    return run_family<T>(
+        ops,
+        [&](DeviceOp& op) {
+            if constexpr(NumD == 1)
+                return op.MakeArgumentPointer(da.GetDeviceBuffer(), db.GetDeviceBuffer(), {dd0.GetDeviceBuffer()},
+                                              de.GetDeviceBuffer(), M, N, K, sa, sb, {sd0}, se, Pass{}, Pass{}, cde);
+            else
+                return op.MakeArgumentPointer(da.GetDeviceBuffer(), db.GetDeviceBuffer(),
+                                              {dd0.GetDeviceBuffer(), dd1.GetDeviceBuffer()}, de.GetDeviceBuffer(), M, N,
+                                              K, sa, sb, {sd0, sd1}, se, Pass{}, Pass{}, cde);
+        },
+        de, (std::size_t)M * se, flop, bytes, verify, time_kernel, nrepeat);
+}
+
+template <typename CDE, int NumD>
+int profile_gemm_cde(int layout, bool verify, int init, bool time_kernel, int M, int N, int K, int sa, int sb, int sd0,
+                     int sd1, int se, CDE cde, int nrepeat)
+{
+    switch(layout)
+    {
+    case MK_KN_MN: return profile_gemm_cde_l<CDE, NumD, Row, Row>(verify, init, time_kernel, M, N, K, sa, sb, sd0, sd1, se, cde, nrepeat);
+    case MK_NK_MN: return profile_gemm_cde_l<CDE, NumD, Row, Col>(verify, init, time_kernel, M, N, K, sa, sb, sd0, sd1, se, cde, nrepeat);
+    case KM_KN_MN: return profile_gemm_cde_l<CDE, NumD, Col, Row>(verify, init, time_kernel, M, N, K, sa, sb, sd0, sd1, se, cde, nrepeat);
+    case KM_NK_MN: return profile_gemm_cde_l<CDE, NumD, Col, Col>(verify, init, time_kernel, M, N, K, sa, sb, sd0, sd1, se, cde, nrepeat);
+    }
+    std::printf("unknown matrix layout\n");
+    return 1;
+}
+
+int profile_gemm_bilinear(int argc, char* argv[])
+{
+    if(argc < 17 || std::atoi(argv[2]) != 1)
+    {
+        std::printf("arg1: tensor operation (gemm_bilinear: GEMM+Bilinear)\narg2: data type (1: fp16)\n"
+                    "arg3: matrix layout (0: E[m, n] = alpha * A[m, k] * B[k, n] + beta * D[m, n];\n"
+                    "                     1: E[m, n] = alpha * A[m, k] * B[n, k] + beta * D[m, n];\n"
+                    "                     2: E[m, n] = alpha * A[k, m] * B[k, n] + beta * D[m, n];\n"
+                    "                     3: E[m, n] = alpha * A[k, m] * B[n, k] + beta * D[m, n])\n"
+                    "arg4: verification (0: no; 1: yes)\narg5: initialization (0: no init; 1: integer value; 2: decimal value)\n"
+                    "arg6: print tensor value (0: no; 1: yes)\narg7: time kernel (0=no, 1=yes)\n"
+                    "arg8 to 14: M, N, K, StrideA, StrideB, StrideD, StrideE\narg15 to 16: alpha, beta\narg17: nrepeat\n");
+        return 1;
+    }
+    const int layout = std::atoi(argv[3]), init = std::atoi(argv[5]);
+    const bool verify = std::atoi(argv[4]), time_kernel = std::atoi(argv[7]);
+    const int M = std::atoi(argv[8]), N = std::atoi(argv[9]), K = std::atoi(argv[10]);
+    const int sa = std::atoi(argv[11]), sb = std::atoi(argv[12]), sd = std::atoi(argv[13]), se = std::atoi(argv[14]);
+    const float alpha = (float)std::atof(argv[15]), beta = (float)std::atof(argv[16]);
+    const int nrepeat = argc > 17 ? std::atoi(argv[17]) : 10;
+    return profile_gemm_cde<element_wise::Bilinear, 1>(layout, verify, init, time_kernel, M, N, K, sa, sb, sd, 0, se,
+                                                       element_wise::Bilinear{alpha, beta}, nrepeat);
+}
+
+int profile_gemm_add_add_fastgelu(int argc, char* argv[])
+{
+    if(argc < 16 || std::atoi(argv[2]) != 1)
+    {
+        std::printf("arg1: tensor operation (gemm_add_add_fastgelu: GEMM+Add+Add+FastGeLU)\narg2: data type (1: fp16)\n"
+                    "arg3: matrix layout (0: E[m, n] = FastGeLU(A[m, k] * B[k, n] + D0[m, n] + D1[m, n]);\n"
+                    "                     1: E[m, n] = FastGeLU(A[m, k] * B[n, k] + D0[m, n] + D1[m, n]);\n"
+                    "                     2: E[m, n] = FastGeLU(A[k, m] * B[k, n] + D0[m, n] + D1[m, n]);\n"
+                    "                     3: E[m, n] = FastGeLU(A[k, m] * B[n, k] + D0[m, n] + D1[m, n]))\n"
+                    "arg4: verification (0: no; 1: yes)\narg5: initialization (0: no init; 1: integer value; 2: decimal value)\n"
+                    "arg6: print tensor value (0: no; 1: yes)\narg7: time kernel (0=no, 1=yes)\n"
+                    "arg8 to 15: M, N, K, StrideA, StrideB, StrideD0, StrideD1, StrideE\narg16: nrepeat\n");
+        return 1;
+    }
+    const int layout = std::atoi(argv[3]), init = std::atoi(argv[5]);
+    const bool verify = std::atoi(argv[4]), time_kernel = std::atoi(argv[7]);
+    const int M = std::atoi(argv[8]), N = std::atoi(argv[9]), K = std::atoi(argv[10]);
+    const int sa = std::atoi(argv[11]), sb = std::atoi(argv[12]), sd0 = std::atoi(argv[13]), sd1 = std::atoi(argv[14]),
+              se = std::atoi(argv[15]);
+    const int nrepeat = argc > 16 ? std::atoi(argv[16]) : 10;
+    return profile_gemm_cde<element_wise::AddAddFastGelu, 2>(layout, verify, init, time_kernel, M, N, K, sa, sb, sd0,
+                                                             sd1, se, element_wise::AddAddFastGelu{}, nrepeat);
+}
+
 int profile_gemm_gemm(int argc, char* argv[])
 {
     if(argc < 11)
@@ -801,6 +910,10 @@ int main(int argc, char* argv[])
             return profile_gemm_perchannel_quant(argc, argv);
         if(argc >= 2 && std::strcmp(argv[1], "gemm_bias_relu") == 0)
             return profile_gemm_bias_relu(argc, argv);
+        if(argc >= 2 && std::strcmp(argv[1], "gemm_bilinear") == 0)
+            return profile_gemm_bilinear(argc, argv);
+        if(argc >= 2 && std::strcmp(argv[1], "gemm_add_add_fastgelu") == 0)
+            return profile_gemm_add_add_fastgelu(argc, argv);
         std::printf("arg1: tensor operation (gemm: GEMM\n"
                     "                        conv2d_fwd: NHWC/KYXC/NHWK forward convolution\n"
                     "                        batched_gemm_gemm: batched fused GEMM+GEMM\n"

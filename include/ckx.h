@@ -72,7 +72,17 @@ enum
      * One fp32 multiply on the exactly converted accumulator (|acc| < 2^24; larger ones round to nearest even on both
      * sides); scales are finite by contract. */
     CKX_EPI_MUL2_CLAMP      = 6,
-    CKX_EPI_RELU_MUL2_CLAMP = 7
+    CKX_EPI_RELU_MUL2_CLAMP = 7,
+    /* fp16 GEMM outputs, fp32 arithmetic on the fp32 accumulator, one rounding at the store:
+     *  BILINEAR          e = half(alpha * acc + beta * d0)        element_wise::Bilinear
+     *                    (binary_element_wise_operation.hpp:93-116; example/02_gemm_bilinear/gemm_bilinear_xdl_fp16.cpp:
+     *                    18-36,290-297); alpha and beta are arguments of ckx_gemm_f16_bilinear
+     *  ADD_ADD_FASTGELU  e = half(fast_gelu(acc + d0 + d1))       element_wise::AddAddFastGelu
+     *                    (element_wise_operation.hpp:113-140; example/04_gemm_add_add_fastgelu), with
+     *                    fast_gelu(x) = x * (0.5 + 0.5 * (2 / (1 + exp(-u)) - 1)), u = 2x(0.035677 x^2 + 0.797885),
+     *                    evaluated as x / (1 + exp(-u)) */
+    CKX_EPI_BILINEAR         = 8,
+    CKX_EPI_ADD_ADD_FASTGELU = 9
 };
 
 /* Operator families, for the instance queries below. */
@@ -215,9 +225,9 @@ int ckx_gemm_i8_splitk_noalloc(const void* p_a, const void* p_b, void* p_c, int3
 /* ---- fp16 GEMM with fused D operands:  E = cde_op(A * B, D0 [, D1]) ----------
  * Replaces DeviceGemmMultipleD<..., Tuple<half_t[, half_t]>, half_t, PassThrough, PassThrough, CDEOp>
  * ::MakeArgumentPointer + Run (device_gemm_multiple_d.hpp:14-55) for cde_op in
- * CKX_EPI_ADD_RELU / _ADD_RELU_ADD / _CSHUFFLE_ADD_RELU. D0, D1 are [M,N] row-major fp16 with row
- * strides stride_d0 / stride_d1 in elements; stride 0 broadcasts one row (a bias vector), as
- * example 03 does. p_d1 is ignored unless cde_op uses it. */
+ * CKX_EPI_ADD_RELU / _ADD_RELU_ADD / _CSHUFFLE_ADD_RELU / _ADD_ADD_FASTGELU (and, for the query, _BILINEAR). D0, D1 are
+ * [M,N] row-major fp16 with row strides stride_d0 / stride_d1 in elements; stride 0 broadcasts one row (a bias
+ * vector), as examples 03 and 04 do. p_d1 is ignored unless cde_op uses it. */
 int ckx_gemm_f16_multiple_d_is_supported(int32_t M, int32_t N, int32_t K, int32_t stride_a, int32_t stride_b,
                                          int32_t stride_d0, int32_t stride_d1, int32_t stride_e, int a_layout,
                                          int b_layout, int e_layout, int cde_op, int instance);
@@ -225,6 +235,15 @@ int ckx_gemm_f16_multiple_d(const void* p_a, const void* p_b, const void* p_d0, 
                             int32_t M, int32_t N, int32_t K, int32_t stride_a, int32_t stride_b, int32_t stride_d0,
                             int32_t stride_d1, int32_t stride_e, int a_layout, int b_layout, int e_layout,
                             int cde_op, int instance, void* p_workspace, int64_t workspace_bytes, void* stream);
+
+/* E = half(alpha * (A * B) + beta * D): DeviceGemmMultipleD<..., Tuple<half_t>, half_t, PassThrough, PassThrough,
+ * Bilinear> (device_gemm_multiple_d.hpp:14-55 with binary_element_wise_operation.hpp:93-116), the operator behind
+ * the reference's "gemm_bilinear" instances and profiler command (profiler/include/profile_gemm_bilinear_impl.hpp).
+ * Arguments as ckx_gemm_f16_multiple_d with one D tensor; query with cde_op = CKX_EPI_BILINEAR. */
+int ckx_gemm_f16_bilinear(const void* p_a, const void* p_b, const void* p_d, void* p_e, int32_t M, int32_t N,
+                          int32_t K, int32_t stride_a, int32_t stride_b, int32_t stride_d, int32_t stride_e,
+                          int a_layout, int b_layout, int e_layout, float alpha, float beta, int instance,
+                          void* p_workspace, int64_t workspace_bytes, void* stream);
 
 /* ---- int8 GEMM with per-column requant scales:  E = cde_op(A * B, D0), D0 = scale[N] (fp32) ----------
  * Replaces DeviceGemmMultipleD<..., int8_t, int8_t, Tuple<float>, int8_t, PassThrough, PassThrough,

@@ -635,6 +635,57 @@ void cko_gemm_f16_add_relu(const uint16_t* a, const uint16_t* b, const uint16_t*
     });
 }
 
+// fp16 GEMM + Bilinear the way example 02 verifies it: ReferenceGemm into an fp32 C (CShuffleDataType is float
+// there), then e = half(alpha * c + beta * float(d)) -- ONE rounding, of the fp32 result
+// (example/02_gemm_bilinear/gemm_bilinear_xdl_fp16.cpp:18-36,271-297; element_wise::Bilinear,
+// binary_element_wise_operation.hpp:93-116, is the same expression). d is [M,N] with element strides.
+void cko_gemm_f16_bilinear(const uint16_t* a, const uint16_t* b, const uint16_t* d, uint16_t* e, int M, int N,
+                           int K, int64_t sa_m, int64_t sa_k, int64_t sb_k, int64_t sb_n, int64_t sd_m,
+                           int64_t sd_n, int64_t se_m, int64_t se_n, float alpha, float beta, int nthreads)
+{
+    parallel_for((std::size_t)M * (std::size_t)N, nthreads, [&](std::size_t i0, std::size_t i1) {
+        for(std::size_t i = i0; i < i1; ++i)
+        {
+            const std::size_t m = i / (std::size_t)N, n = i % (std::size_t)N;
+            float acc           = 0;
+            for(int k = 0; k < K; ++k)
+                acc += half_to_float(a[m * sa_m + k * sa_k]) * half_to_float(b[k * sb_k + n * sb_n]);
+            e[m * se_m + n * se_n] = float_to_half(alpha * acc + beta * half_to_float(d[m * sd_m + n * sd_n]));
+        }
+    });
+}
+
+// element_wise::FastGelu / the lambda inside AddAddFastGelu, in fp32 as written
+// (unary_element_wise_operation.hpp:121-135, element_wise_operation.hpp:127-133)
+float cko_fast_gelu(float x)
+{
+    const float u   = 2.0f * x * (0.035677f * x * x + 0.797885f);
+    const float emu = std::exp(-u);
+    const float cdf = 0.5f + 0.5f * (2.0f / (1.0f + emu) - 1.0f);
+    return x * cdf;
+}
+
+// fp16 GEMM + AddAddFastGelu the way example 04 verifies it: ReferenceGemm into an fp32 C, then
+// e = half(fast_gelu(c + float(d0) + float(d1))) (example/04_gemm_add_add_fastgelu/gemm_add_add_fastgelu_xdl_fp16.cpp:
+// 213-241; element_wise_operation.hpp:113-140). d0, d1 are [M,N] with element strides (a row stride of 0 broadcasts).
+void cko_gemm_f16_add_add_fastgelu(const uint16_t* a, const uint16_t* b, const uint16_t* d0, const uint16_t* d1,
+                                   uint16_t* e, int M, int N, int K, int64_t sa_m, int64_t sa_k, int64_t sb_k,
+                                   int64_t sb_n, int64_t sd0_m, int64_t sd0_n, int64_t sd1_m, int64_t sd1_n,
+                                   int64_t se_m, int64_t se_n, int nthreads)
+{
+    parallel_for((std::size_t)M * (std::size_t)N, nthreads, [&](std::size_t i0, std::size_t i1) {
+        for(std::size_t i = i0; i < i1; ++i)
+        {
+            const std::size_t m = i / (std::size_t)N, n = i % (std::size_t)N;
+            float acc           = 0;
+            for(int k = 0; k < K; ++k)
+                acc += half_to_float(a[m * sa_m + k * sa_k]) * half_to_float(b[k * sb_k + n * sb_n]);
+            const float x = acc + half_to_float(d0[m * sd0_m + n * sd0_n]) + half_to_float(d1[m * sd1_m + n * sd1_n]);
+            e[m * se_m + n * se_n] = float_to_half(cko_fast_gelu(x));
+        }
+    });
+}
+
 // ---- magic-number division (dividend < 2^31, divisor >= 1) ----
 void cko_magic_division_params(uint32_t divisor, uint32_t* multiplier, uint32_t* shift)
 {

@@ -189,6 +189,27 @@ def gemm_f16_add_relu(a_mk, b_kn, d_mn):
     return np.maximum(x, np.float16(0))
 
 
+def gemm_f16_bilinear(a_mk, b_kn, d_mn, alpha, beta):
+    """half(alpha * (A*B) + beta * D) on the fp32 product (fp32 BLAS sums: within tolerance of the literal form)."""
+    acc = np.asarray(a_mk, np.float32) @ np.asarray(b_kn, np.float32)
+    return (np.float32(alpha) * acc + np.float32(beta) * np.asarray(d_mn, np.float32)).astype(np.float16)
+
+
+def fast_gelu(x):
+    """element_wise::FastGelu in fp32 on an array, written as the reference writes it."""
+    x = np.asarray(x, np.float32)
+    with np.errstate(over="ignore"):
+        u = np.float32(2) * x * (np.float32(0.035677) * x * x + np.float32(0.797885))
+        emu = np.exp(-u)
+        cdf = np.float32(0.5) + np.float32(0.5) * (np.float32(2) / (np.float32(1) + emu) - np.float32(1))
+    return x * cdf
+
+
+def gemm_f16_add_add_fastgelu(a_mk, b_kn, d0_mn, d1_mn):
+    acc = np.asarray(a_mk, np.float32) @ np.asarray(b_kn, np.float32)
+    return fast_gelu(acc + np.asarray(d0_mn, np.float32) + np.asarray(d1_mn, np.float32)).astype(np.float16)
+
+
 def batched_gemm_gemm_f16(a_gmk, b0_gkn, b1_gno):
     s = np.matmul(np.asarray(a_gmk, np.float32), np.asarray(b0_gkn, np.float32)).astype(np.float16)
     return np.matmul(s.astype(np.float32), np.asarray(b1_gno, np.float32)).astype(np.float16)

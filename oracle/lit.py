@@ -37,6 +37,8 @@ def lib():
         _lib.cko_epilogue_i8.argtypes = [C.c_int32, C.c_int, C.c_float, C.c_float]
         _lib.cko_mul2_clamp.restype = C.c_int8
         _lib.cko_mul2_clamp.argtypes = [C.c_int32, C.c_float, C.c_int]
+        _lib.cko_fast_gelu.restype = C.c_float
+        _lib.cko_fast_gelu.argtypes = [C.c_float]
         _lib.cko_conv_out_len.restype = C.c_int
         _lib.cko_magic_division_divide.restype = C.c_uint32
         _lib.cko_magic_division_divide.argtypes = [C.c_uint32, C.c_uint32, C.c_uint32]
@@ -244,6 +246,36 @@ def gemm_f16_add_relu(a_mk, b_kn, d_mn, nthreads=0):
     e = np.empty((M, N), np.float16)
     lib().cko_gemm_f16_add_relu(_p(a_mk), _p(b_kn), _p(d), _p(e), M, N, K, *_i64(*_estrides(a_mk)),
                                 *_i64(*_estrides(b_kn)), *_i64(*_estrides(d)), *_i64(N, 1), int(nthreads))
+    return e
+
+
+def gemm_f16_bilinear(a_mk, b_kn, d_mn, alpha, beta, nthreads=0):
+    """E = half(alpha * (A*B) + beta * D) as example 02 verifies it: one rounding, of the fp32 result."""
+    M, K = a_mk.shape
+    _, N = b_kn.shape
+    d = np.broadcast_to(d_mn, (M, N))
+    e = np.empty((M, N), np.float16)
+    lib().cko_gemm_f16_bilinear(_p(a_mk), _p(b_kn), _p(d), _p(e), M, N, K, *_i64(*_estrides(a_mk)),
+                                *_i64(*_estrides(b_kn)), *_i64(*_estrides(d)), *_i64(N, 1), C.c_float(alpha),
+                                C.c_float(beta), int(nthreads))
+    return e
+
+
+def fast_gelu(x):
+    """element_wise::FastGelu on one float, as written in the reference."""
+    return float(lib().cko_fast_gelu(float(x)))
+
+
+def gemm_f16_add_add_fastgelu(a_mk, b_kn, d0_mn, d1_mn, nthreads=0):
+    """E = half(fast_gelu(A*B + D0 + D1)) as example 04 verifies it; D0 / D1 may be broadcast views."""
+    M, K = a_mk.shape
+    _, N = b_kn.shape
+    d0 = np.broadcast_to(d0_mn, (M, N))
+    d1 = np.broadcast_to(d1_mn, (M, N))
+    e = np.empty((M, N), np.float16)
+    lib().cko_gemm_f16_add_add_fastgelu(_p(a_mk), _p(b_kn), _p(d0), _p(d1), _p(e), M, N, K, *_i64(*_estrides(a_mk)),
+                                        *_i64(*_estrides(b_kn)), *_i64(*_estrides(d0)), *_i64(*_estrides(d1)),
+                                        *_i64(N, 1), int(nthreads))
     return e
 
 

@@ -394,6 +394,64 @@ void ckref_gemm_f16_add_relu(const uint16_t* a, const uint16_t* b, const uint16_
         }
 }
 
+// example 02's verification: ReferenceGemm<half,half,float,float,...> then the reference's own Bilinear functor
+// (binary_element_wise_operation.hpp:93-116) on (half_t&, const float&, const half_t&)
+void ckref_gemm_f16_bilinear(const uint16_t* a, const uint16_t* b, const uint16_t* d, uint16_t* e, int M, int N,
+                             int K, long sa_m, long sa_k, long sb_k, long sb_n, long sd_m, long sd_n, float alpha,
+                             float beta)
+{
+    using T  = ck::half_t;
+    using sz = std::size_t;
+    auto ta  = make_tensor<T>({(sz)M, (sz)K}, {(sz)sa_m, (sz)sa_k}, reinterpret_cast<const T*>(a));
+    auto tb  = make_tensor<T>({(sz)K, (sz)N}, {(sz)sb_k, (sz)sb_n}, reinterpret_cast<const T*>(b));
+    auto tc  = make_tensor<float>({(sz)M, (sz)N}, {(sz)N, 1}, (const float*)nullptr);
+    using Ref =
+        ck::tensor_operation::host::ReferenceGemm<T, T, float, float, PassThrough, PassThrough, PassThrough>;
+    Ref ref;
+    auto inv = ref.MakeInvoker();
+    auto arg = ref.MakeArgument(ta, tb, tc, PassThrough{}, PassThrough{}, PassThrough{});
+    inv.Run(arg);
+    const T* dd = reinterpret_cast<const T*>(d);
+    T* ee       = reinterpret_cast<T*>(e);
+    ck::tensor_operation::element_wise::Bilinear op{alpha, beta};
+    for(int m = 0; m < M; ++m)
+        for(int n = 0; n < N; ++n)
+            op(ee[(sz)m * N + n], tc(m, n), dd[(sz)m * sd_m + (sz)n * sd_n]);
+}
+
+// example 04's verification: ReferenceGemm into fp32, then the reference's own AddAddFastGelu functor
+// (element_wise_operation.hpp:113-140) on (half_t&, const float&, const half_t&, const half_t&)
+void ckref_gemm_f16_add_add_fastgelu(const uint16_t* a, const uint16_t* b, const uint16_t* d0, const uint16_t* d1,
+                                     uint16_t* e, int M, int N, int K, long sa_m, long sa_k, long sb_k, long sb_n,
+                                     long sd0_m, long sd0_n, long sd1_m, long sd1_n)
+{
+    using T  = ck::half_t;
+    using sz = std::size_t;
+    auto ta  = make_tensor<T>({(sz)M, (sz)K}, {(sz)sa_m, (sz)sa_k}, reinterpret_cast<const T*>(a));
+    auto tb  = make_tensor<T>({(sz)K, (sz)N}, {(sz)sb_k, (sz)sb_n}, reinterpret_cast<const T*>(b));
+    auto tc  = make_tensor<float>({(sz)M, (sz)N}, {(sz)N, 1}, (const float*)nullptr);
+    using Ref =
+        ck::tensor_operation::host::ReferenceGemm<T, T, float, float, PassThrough, PassThrough, PassThrough>;
+    Ref ref;
+    auto inv = ref.MakeInvoker();
+    auto arg = ref.MakeArgument(ta, tb, tc, PassThrough{}, PassThrough{}, PassThrough{});
+    inv.Run(arg);
+    const T* p0 = reinterpret_cast<const T*>(d0);
+    const T* p1 = reinterpret_cast<const T*>(d1);
+    T* ee       = reinterpret_cast<T*>(e);
+    ck::tensor_operation::element_wise::AddAddFastGelu op;
+    for(int m = 0; m < M; ++m)
+        for(int n = 0; n < N; ++n)
+            op(ee[(sz)m * N + n], tc(m, n), p0[(sz)m * sd0_m + (sz)n * sd0_n], p1[(sz)m * sd1_m + (sz)n * sd1_n]);
+}
+
+float ckref_fast_gelu(float x)
+{
+    float y;
+    ck::tensor_operation::element_wise::FastGelu{}(y, x);
+    return y;
+}
+
 int ckref_conv_out_len(int in_len, int filter_len, int stride, int dilation, int pad_left, int pad_right)
 {
     ck::utils::conv::ConvParams p;

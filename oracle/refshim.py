@@ -135,6 +135,29 @@ class _Ref:
         self.lib.ckref_gemm_f16_add_relu(_p(a_mk), _p(b_kn), _p(d), _p(e), M, N, K, *_es(a_mk), *_es(b_kn), *_es(d))
         return e
 
+    def gemm_f16_bilinear(self, a_mk, b_kn, d_mn, alpha, beta):
+        M, K = a_mk.shape
+        _, N = b_kn.shape
+        d = np.broadcast_to(d_mn, (M, N))
+        e = np.zeros((M, N), np.float16)
+        self.lib.ckref_gemm_f16_bilinear(_p(a_mk), _p(b_kn), _p(d), _p(e), M, N, K, *_es(a_mk), *_es(b_kn), *_es(d),
+                                         C.c_float(alpha), C.c_float(beta))
+        return e
+
+    def gemm_f16_add_add_fastgelu(self, a_mk, b_kn, d0_mn, d1_mn):
+        M, K = a_mk.shape
+        _, N = b_kn.shape
+        d0 = np.broadcast_to(d0_mn, (M, N))
+        d1 = np.broadcast_to(d1_mn, (M, N))
+        e = np.zeros((M, N), np.float16)
+        self.lib.ckref_gemm_f16_add_add_fastgelu(_p(a_mk), _p(b_kn), _p(d0), _p(d1), _p(e), M, N, K, *_es(a_mk),
+                                                 *_es(b_kn), *_es(d0), *_es(d1))
+        return e
+
+    def fast_gelu(self, x):
+        self.lib.ckref_fast_gelu.restype = C.c_float
+        return float(self.lib.ckref_fast_gelu(C.c_float(x)))
+
     def gemm_bf16(self, a_mk, b_kn):
         M, K = a_mk.shape
         _, N = b_kn.shape

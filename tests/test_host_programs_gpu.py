@@ -156,6 +156,38 @@ def test_profiler_gemm_bias_relu(tmp_path):
     assert bad == 0, max_err
 
 
+@pytest.mark.parametrize("layout", [1, 2])
+def test_profiler_gemm_bilinear(tmp_path, layout):
+    """profile_gemm_bilinear's argument list (alpha, beta = arg15, 16) over every instance of the C++
+    DeviceGemmMultipleD<..., Tuple<half_t>, half_t, ..., Bilinear>; layout 2 stores A as [K, M] and B as [K, N]."""
+    M, N, K = 320, 256, 512
+    out, dump = _run("ckx_profiler", ["gemm_bilinear", 1, layout, 1, 2, 0, 1, M, N, K, -1, -1, -1, -1, 0.5, -1.25],
+                     "CKX_PROFILER_DUMP", tmp_path)
+    assert "Best Perf:" in out and "Error" not in out and "Bilinear" in out
+    e = np.fromfile(dump, np.float16).reshape(M, N)
+    a_st = uniform_f16((M, K) if layout == 1 else (K, M), -1, 1, SEED)
+    b_st = uniform_f16((N, K) if layout == 1 else (K, N), -1, 1, SEED + 1)
+    d = uniform_f16((M, N), -1, 1, SEED + 9)
+    a_mk, b_kn = (a_st, b_st.T) if layout == 1 else (a_st.T, b_st)
+    bad, max_err = lit.check_err_f16(e, fast.gemm_f16_bilinear(a_mk, b_kn, d, 0.5, -1.25), 1e-2, 1e-2)
+    assert bad == 0, max_err
+
+
+def test_profiler_gemm_add_add_fastgelu(tmp_path):
+    """profile_gemm_add_add_fastgelu's argument list with example 04's strides: D0 a bias row (StrideD0 = 0), D1 dense."""
+    M, N, K = 320, 256, 512
+    out, dump = _run("ckx_profiler", ["gemm_add_add_fastgelu", 1, 1, 1, 2, 0, 1, M, N, K, -1, -1, 0, -1, -1],
+                     "CKX_PROFILER_DUMP", tmp_path)
+    assert "Best Perf:" in out and "Error" not in out and "AddAddFastGelu" in out
+    e = np.fromfile(dump, np.float16).reshape(M, N)
+    a = uniform_f16((M, K), -1, 1, SEED)
+    b_nk = uniform_f16((N, K), -1, 1, SEED + 1)
+    d0 = uniform_f16((N,), -1, 1, SEED + 9)
+    d1 = uniform_f16((M, N), -1, 1, SEED + 10)
+    bad, max_err = lit.check_err_f16(e, fast.gemm_f16_add_add_fastgelu(a, b_nk.T, d0[None, :], d1), 1e-2, 1e-2)
+    assert bad == 0, max_err
+
+
 @pytest.mark.parametrize("act", [0, 1])
 def test_profiler_gemm_perchannel_quant(tmp_path, act):
     """C++ DeviceGemmMultipleD<int8, ..., Tuple<float>, int8, Activation_Mul2_Clamp<Act>> over every instance: all

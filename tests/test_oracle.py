@@ -531,6 +531,78 @@ def test_gemm_add_relu_random_lit_ref_bit_exact_and_full_d():
             np.testing.assert_array_equal(REF.gemm_f16_add_relu(a, b, d), e)
 
 
+# ------------------------------------------------------------------- Bilinear / AddAddFastGelu
+def test_gemm_bilinear_rounds_once_and_reduces_to_its_parts():
+    """alpha * acc + beta * d is rounded ONCE: K = 2049 ones give acc = 2049; + 1 = 2050 is a fp16 value (rounding C
+    first would store 2048). alpha = 1, beta = 0 is the plain GEMM; alpha = 0, beta = 1 returns D bit for bit;
+    small integers are exact. The reference's own functor agrees bit for bit."""
+    a = np.ones((3, 2049), np.float16)
+    b = np.ones((2049, 4), np.float16)
+    d = np.array([1.0, -1.0, -4096.0, 0.5], np.float16)[None, :]
+    e = lit.gemm_f16_bilinear(a, b, d, 1.0, 1.0)
+    np.testing.assert_array_equal(e, np.broadcast_to(np.array([2050, 2048, -2047, 2050], np.float16), (3, 4)))
+    np.testing.assert_array_equal(lit.gemm_f16_bilinear(a, b, d, 2.0, -3.0),
+                                  np.broadcast_to(np.array([4095, 4100, 16384, 4096], np.float16), (3, 4)))
+    rng = np.random.default_rng(21)
+    a = rng.uniform(-1, 1, (19, 72)).astype(np.float16)
+    b = np.asfortranarray(rng.uniform(-1, 1, (72, 13)).astype(np.float16))
+    d = rng.uniform(-3, 3, (19, 13)).astype(np.float16)
+    np.testing.assert_array_equal(lit.gemm_f16_bilinear(a, b, d, 1.0, 0.0), lit.gemm_f16(a, b))
+    np.testing.assert_array_equal(lit.gemm_f16_bilinear(a, b, d, 0.0, 1.0), d)
+    e = lit.gemm_f16_bilinear(a, b, d, 0.75, -1.5)
+    assert lit.check_err_f16(fast.gemm_f16_bilinear(a, b, d, 0.75, -1.5), e, 1e-3, 1e-3)[0] == 0
+    # swapped scalars or operands change the result
+    assert (lit.gemm_f16_bilinear(a, b, d, -1.5, 0.75) != e).mean() > 0.9
+    if REF is not None:
+        np.testing.assert_array_equal(REF.gemm_f16_bilinear(a, b, d, 0.75, -1.5), e)
+        np.testing.assert_array_equal(REF.gemm_f16_bilinear(a, b, d[:1], 0.75, -1.5),
+                                      lit.gemm_f16_bilinear(a, b, d[:1], 0.75, -1.5))
+
+
+def test_fast_gelu_against_the_tanh_form_and_its_limits():
+    """fast_gelu(x) = 0.5 x (1 + tanh(sqrt(2/pi) (x + 0.044715 x^3))) with the constants rounded to six digits
+    (0.035677 = 0.044715 * 0.797885): checked against the tanh form in float64, at 0, and far out on both sides,
+    where it is x and -0 / 0 (no NaN from the overflowing exponential)."""
+    xs = np.concatenate([np.linspace(-12, 12, 481), [1e-3, -1e-3, 30.0, -30.0, 65504.0, -65504.0]])
+    for x in xs:
+        want = 0.5 * x * (1.0 + np.tanh(np.sqrt(2.0 / np.pi) * (x + 0.044715 * x ** 3)))
+        got = lit.fast_gelu(x)
+        assert np.isfinite(got)
+        assert abs(got - want) <= 2e-6 * max(1.0, abs(x)), (x, got, want)
+    assert lit.fast_gelu(0.0) == 0.0
+    assert lit.fast_gelu(40.0) == 40.0 and lit.fast_gelu(-40.0) == 0.0
+    assert lit.fast_gelu(-0.5) < 0 < lit.fast_gelu(0.5)
+    np.testing.assert_allclose(fast.fast_gelu(xs.astype(np.float32)), [lit.fast_gelu(x) for x in xs],
+                               rtol=2e-6, atol=1e-7)
+    if REF is not None:
+        for x in xs:
+            assert abs(REF.fast_gelu(x) - lit.fast_gelu(x)) <= 1e-6 * max(1.0, abs(x))
+
+
+def test_gemm_add_add_fastgelu_lit_fast_ref():
+    """example 04's layout: D0 a bias row (stride 0), D1 a full tensor. The literal form against the reference's own
+    functor (bit-exact up to the exp of the C library in use: at most one fp16 ulp on a handful of elements) and the
+    BLAS form; with A = 0 it is fast_gelu(d0 + d1) element by element; D0 and D1 are interchangeable."""
+    rng = np.random.default_rng(22)
+    a = rng.uniform(-1, 1, (21, 64)).astype(np.float16)
+    b = np.asfortranarray(rng.uniform(-1, 1, (64, 18)).astype(np.float16))
+    d0 = rng.uniform(-3, 3, (1, 18)).astype(np.float16)
+    d1 = rng.uniform(-2, 2, (21, 18)).astype(np.float16)
+    e = lit.gemm_f16_add_add_fastgelu(a, b, d0, d1)
+    assert (e < 0).any() and (e > 1).any()
+    assert lit.check_err_f16(fast.gemm_f16_add_add_fastgelu(a, b, d0, d1), e, 1e-3, 1e-3)[0] == 0
+    z = lit.gemm_f16_add_add_fastgelu(np.zeros_like(a), b, d0, d1)
+    s = np.broadcast_to(d0, d1.shape).astype(np.float32) + d1.astype(np.float32)
+    want = np.array([lit.fast_gelu(v) for v in s.ravel()], np.float32).astype(np.float16).reshape(s.shape)
+    np.testing.assert_array_equal(z, want)
+    d0_full = np.ascontiguousarray(np.broadcast_to(d0, d1.shape))
+    np.testing.assert_array_equal(lit.gemm_f16_add_add_fastgelu(a, b, d1, d0_full), e)
+    if REF is not None:
+        r = REF.gemm_f16_add_add_fastgelu(a, b, d0, d1)
+        ulp = np.abs(r.view(np.int16).astype(np.int32) - e.view(np.int16).astype(np.int32))
+        assert ulp.max() <= 1 and (ulp != 0).mean() < 0.02
+
+
 # ------------------------------------------------------------------------------- bfloat16
 def test_bf16_conversion_is_round_to_nearest_even_like_torch_and_the_reference():
     """type_convert<bhalf_t, float> (data_type.hpp:953-993): checked against torch's bfloat16 cast (an
