@@ -36,7 +36,7 @@ SYMBOLS = [
     "ckx_convnd_fwd_is_supported", "ckx_convnd_fwd", "ckx_convnd_fwd_workspace_bytes",
     "ckx_batched_gemm_gemm_f16_is_supported", "ckx_batched_gemm_gemm_f16", "ckx_time_launches",
     "ckx_batched_gemm_softmax_gemm_f16_is_supported", "ckx_batched_gemm_softmax_gemm_f16",
-    "ckx_gemm_plan", "ckx_conv2d_fwd_plan", "ckx_set_forced_k_runs",
+    "ckx_gemm_plan", "ckx_conv2d_fwd_plan", "ckx_set_forced_k_runs", "ckx_set_big_tile_waves",
 ]
 
 
@@ -143,6 +143,7 @@ def lib():
     L.ckx_gemm_plan.argtypes = [C.c_int] + shape + [C.c_int, i32, i64, ip, ip]
     L.ckx_conv2d_fwd_plan.argtypes = [C.c_int, dp, C.c_int, i64, ip, ip]
     L.ckx_set_forced_k_runs.argtypes = [C.c_int]
+    L.ckx_set_big_tile_waves.argtypes = [C.c_int]
     _lib = L
     return L
 

@@ -142,6 +142,36 @@ struct Plan
     int nk_per = 0;
 };
 
+// Which body runs the 256 x 256 tile instance on a dense K-contiguous GEMM with a plain epilogue: 0 chooses (below), 4 / 8
+// force the four-wave / eight-wave kernel wherever the four-wave one applies (tuning / test knob; CKX_BIG_TILE_WAVES in
+// the environment is read on the first call only).
+std::atomic<int> g_big_tile_waves{-1};
+int big_tile_waves()
+{
+    int v = g_big_tile_waves.load(std::memory_order_relaxed);
+    if(v < 0)
+    {
+        const char* e = std::getenv("CKX_BIG_TILE_WAVES");
+        v             = e ? std::atoi(e) : 0;
+        v             = (v == 4 || v == 8) ? v : 0;
+        g_big_tile_waves.store(v, std::memory_order_relaxed);
+    }
+    return v;
+}
+// The four-wave body (one wave per SIMD, 128 x 128 wave tiles) has the faster K loop -- 18.0 against 18.9 cycles per
+// MFMA -- and the higher fixed cost (a lane zeroes, converts and stores twice as many accumulators with nothing to
+// overlap them; the int8 epilogues feel it most): measured faster from 16 K tiles on for fp16 / bf16 and from 32 on
+// for int8, and for int8 only while every CU gets at most one tile (the eight-wave body prefetches across tiles).
+bool four_wave_body_pays(int dt, int K, int tiles)
+{
+    const int waves = big_tile_waves();
+    if(waves)
+        return waves == 4;
+    const int es = dt == ckx::DT_I8 ? 1 : 2;
+    const long nk = ((long)K * es + 127) / 128;
+    return dt == ckx::DT_I8 ? (nk >= 32 && tiles <= ckx::num_cus()) : nk >= 16;
+}
+
 // CKX_KSPLIT=n forces n K runs where the problem allows it (tuning / test knob). The environment is read on the first
 // call only; ckx_set_forced_k_runs() changes the value afterwards (tests force several splits in one process).
 std::atomic<int> g_force_ksplit{-1};
@@ -604,7 +634,10 @@ int run_gemm(int dt, const void* a, const void* b, void* c, int M, int N, int K,
     g.nk_per     = pl.nk_per;
     g.ws         = ws;
     const bool fused            = f16_fused(epi) && g.ksplit == 1; // (after a K split the second pass applies it)
-    const tile_launch_fn launch = kmajor               ? ckx::layout_tile(dt, ti, ta, tb)
+    const bool w4 = ti == 0 && !kmajor && batch == 1 && g.ksplit == 1 && epi <= CKX_EPI_REQUANT_RND &&
+                    four_wave_body_pays(dt, K, g.tiles_m * g.tiles_n);
+    const tile_launch_fn launch = w4                   ? ckx::w4_tile(dt)
+                                  : kmajor             ? ckx::layout_tile(dt, ti, ta, tb)
                                   : dt == ckx::DT_I8   ? (per_column_scale(epi) && g.ksplit == 1 ? t.dense_i8_fused : t.dense_i8)
                                   : dt == ckx::DT_BF16 ? t.dense_bf16
                                   : fused              ? t.dense_f16_fused
@@ -1113,6 +1146,13 @@ int ckx_gemm_i8(const void* a, const void* b, void* c, int32_t M, int32_t N, int
 {
     return run_gemm(ckx::DT_I8, a, b, c, M, N, K, sa, sb, sc, al, bl, cl, epilogue, scale_gemm, scale_relu,
                     instance, workspace, workspace_bytes, stream);
+}
+
+int ckx_set_big_tile_waves(int waves)
+{
+    const int before = big_tile_waves();
+    g_big_tile_waves.store((waves == 4 || waves == 8) ? waves : 0, std::memory_order_relaxed);
+    return before;
 }
 
 int ckx_set_forced_k_runs(int k_runs)

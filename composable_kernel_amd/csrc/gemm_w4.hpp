@@ -1,0 +1,322 @@
+// 256 x 256 C tile computed by FOUR waves -- one per SIMD, wave tile 128 x 128 -- for dense K-contiguous GEMMs
+// (A row-major, B column-major) whose tiles give every CU one round of work.
+//
+// Same data path as gemm_tile.hpp (128-byte K tiles, direct global->LDS loads with the XOR swizzle and the B row
+// permutation applied by the choice of each lane's global chunk, D^T = B_frag x A_frag, register epilogue, 16 contiguous
+// outputs per lane), a different division of labour:
+//  * one wave per SIMD. Two waves of one SIMD do not interleave evenly: the older one runs ahead, issues its direct
+//    loads early, the younger one issues its loads late and everybody waits for those at the next barrier. With a
+//    single wave per SIMD the loads of all four waves go out at the same point of the iteration. (An instruction-mix
+//    model of both loops with real operand traffic: 19.7 cycles per MFMA with two waves per SIMD, 17.8 with one.)
+//  * 128 x 128 wave tiles: 16 fragment reads per 64 MFMAs instead of 12 per 32.
+//  * the 256 accumulator registers of a lane live in AccVGPRs: the MFMAs are inline assembly with the accumulator
+//    tied ("+a"), which is what keeps the register allocator from shuffling them through VGPRs; the 128 VGPRs of the
+//    two fragment sets (register double buffer over the two k-steps of a K tile), the 16 load offsets and the
+//    addresses fit the architectural half.
+// The K loop is a loop of its own inside the loop over tiles (no prefetch across tiles): a workgroup normally has one.
+#pragma once
+
+#include "gemm_tile.hpp"
+
+namespace ckx {
+
+template <int DT>
+struct GemmW4
+{
+    static constexpr int BM = 256, BN = 256, BKB = 128, NW = 4, NT = NW * 64, NST = 2;
+    static constexpr int ES     = DT == DT_I8 ? 1 : 2;
+    static constexpr int A_TILE = BM * BKB, B_TILE = BN * BKB, STAGE = A_TILE + B_TILE;
+    static constexpr int LUT    = DT == DT_I8 ? 256 : 0;
+    static constexpr int LDS    = NST * STAGE + LUT;
+    static constexpr int MT = 8, NB = 8;  // A fragments (16 rows each) and B fragments (16 columns each) of a wave per k-step
+    static constexpr int NLA = 8, NLB = 8, LPT = NLA + NLB; // 16-byte direct loads per thread and K tile
+    static constexpr int NMH = MT * NB;   // MFMAs per half-iteration (one k-step)
+    using acc_t = typename std::conditional<DT == DT_I8, i32x4, f32x4>::type;
+
+    // (the accumulators of the last fragment row stay in VGPRs: with all 256 AccVGPRs tied the allocator has no
+    // register left to move one through and spills)
+    template <bool IN_VGPR>
+    __device__ static __forceinline__ void mfma(acc_t& c, const i32x4& b, const i32x4& a)
+    {
+        if constexpr(IN_VGPR)
+        {
+            if constexpr(DT == DT_I8)
+                asm volatile("v_mfma_i32_16x16x64_i8 %0, %1, %2, %0" : "+v"(c) : "v"(b), "v"(a));
+            else if constexpr(DT == DT_BF16)
+                asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+v"(c) : "v"(b), "v"(a));
+            else
+                asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+v"(c) : "v"(b), "v"(a));
+        }
+        else
+        {
+            if constexpr(DT == DT_I8)
+                asm volatile("v_mfma_i32_16x16x64_i8 %0, %1, %2, %0" : "+a"(c) : "v"(b), "v"(a));
+            else if constexpr(DT == DT_BF16)
+                asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+a"(c) : "v"(b), "v"(a));
+            else
+                asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+a"(c) : "v"(b), "v"(a));
+        }
+    }
+
+    // The four accumulator tuples of column group g of one fragment row, as VGPR values. Read out of the AccVGPRs by
+    // inline assembly, in program order, one group at a time: left to itself the compiler reads all 224 of them at the
+    // top of the epilogue and the allocator, short of 200 VGPRs there, spills fragment registers inside the K loop.
+    template <bool IN_VGPR>
+    __device__ static __forceinline__ void fetch_acc(std::integral_constant<bool, IN_VGPR>, const acc_t (&row)[NB], int g,
+                                                     acc_t (&v)[4])
+    {
+#pragma unroll
+        for(int t = 0; t < 4; ++t)
+        {
+            if constexpr(IN_VGPR)
+                v[t] = row[g * 4 + t];
+            else
+            {
+#pragma unroll
+                for(int j = 0; j < 4; ++j)
+                {
+                    decltype(row[0][0] + 0) x;
+                    asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(x) : "a"(row[g * 4 + t][j]));
+                    v[t][j] = x;
+                }
+            }
+        }
+    }
+
+    // 16 consecutive int8 outputs of one row from their (already requantised) values b[0..15]
+    __device__ static __forceinline__ void store_bytes16(int8_t* crow, int n0, int N, bool vec_ok, const int* b, bool nt)
+    {
+        if(vec_ok && n0 + 16 <= N)
+        {
+            i32x4 pk;
+#pragma unroll
+            for(int w = 0; w < 4; ++w)
+                pk[w] = pack4_low_bytes(b[4 * w], b[4 * w + 1], b[4 * w + 2], b[4 * w + 3]);
+            store_vec(reinterpret_cast<i32x4*>(crow + n0), pk, nt);
+        }
+        else
+        {
+#pragma unroll
+            for(int e = 0; e < 16; ++e)
+                if(n0 + e < N)
+                    crow[n0 + e] = (int8_t)b[e];
+        }
+    }
+
+    __device__ static __forceinline__ void run(const GemmArgs& p, uint8_t* smem)
+    {
+        const int tid  = threadIdx.x;
+        const int lane = tid & 63;
+        const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+        const int wm = wave >> 1, wn = wave & 1;
+        const int ntiles      = p.tiles_m * p.tiles_n;
+        const uint32_t kbytes = (uint32_t)p.K * ES;
+        const int nk_real     = (int)((kbytes + BKB - 1) / BKB);
+        const int nk          = nk_real > 0 ? nk_real : 1;
+
+        const __amdgpu_buffer_rsrc_t rsrc_a = make_rsrc(p.a, p.a_bytes);
+        const __amdgpu_buffer_rsrc_t rsrc_b = make_rsrc(p.b, p.b_bytes);
+        const uint32_t smem_lds             = (uint32_t)(uintptr_t)(lds_ptr_t)smem;
+        if constexpr(DT == DT_I8)
+        {
+            if(p.epi == EPI_REQUANT_RND) // (visible to every wave after the first barrier of the K loop)
+                requant_lut_fill(smem + NST * STAGE, p.scale_relu, tid, NT);
+        }
+
+        // slot j of a thread fills LDS row (j * NW + wave) * 8 + lane / 8, chunk position lane % 8 of the A (B) tile
+        // with chunk (lane % 8) ^ (row & 7) of that row
+        const uint32_t kb = ((uint32_t)(lane & 7) ^ (uint32_t)((lane >> 3) & 7)) << 4;
+        // fragment addresses relative to a stage: row = wave rows + 16 * fragment + lane % 16, chunk 4 * ks + lane / 16
+        const uint32_t frow = (uint32_t)(lane & 15), fq = (uint32_t)(lane >> 4);
+        auto frag_part      = [&](int row0, int ks) {
+            return (uint32_t)(row0 + (int)frow) * BKB + ((((uint32_t)ks * 4 + fq) ^ (frow & 7u)) << 4);
+        };
+        const uint32_t fa[2] = {frag_part(wm * 128, 0), frag_part(wm * 128, 1)};
+        const uint32_t fb[2] = {A_TILE + frag_part(wn * 128, 0), A_TILE + frag_part(wn * 128, 1)};
+
+        const bool vec_ok = ((reinterpret_cast<uintptr_t>(p.c) | ((uintptr_t)p.ldc * ES)) & 15u) == 0;
+        const bool nt     = p.nt_store != 0;
+
+        for(int unit = (int)blockIdx.x; unit < ntiles; unit += (int)gridDim.x)
+        {
+            int tm, tn, bi;
+            tile_of_block(unit, p.tiles_m, p.tiles_n, 1, bi, tm, tn);
+            uint32_t a_off[NLA], b_off[NLB];
+#pragma unroll
+            for(int j = 0; j < NLA; ++j)
+            {
+                const uint32_t r  = (uint32_t)((j * NW + wave) * 8 + (lane >> 3));
+                const uint32_t gm = (uint32_t)tm * BM + r;
+                const uint32_t gn = (uint32_t)tn * BN + b_row_to_col(r);
+                a_off[j]          = gm < (uint32_t)p.M ? gm * (uint32_t)p.lda * ES + kb : kOutOfRange;
+                b_off[j]          = gn < (uint32_t)p.N ? gn * (uint32_t)p.ldb * ES + kb : kOutOfRange;
+            }
+            // One direct load: slot < NLA an A row group, else a B row group, of the K tile at byte offset k0 into the
+            // stage at stage_off. k0 travels in the instruction's scalar offset, which the address uses and the range check
+            // does not: the per-lane offset alone decides between the row (in range) and zeros (row past M / N: top bit).
+            // MASKED adds the top bit for chunks past K and K tiles past the end -- two VALU instructions per load that
+            // the K tiles in the middle of the loop do without (a VALU instruction between the MFMAs of a SIMD's only
+            // wave costs about seven cycles of the matrix pipeline).
+            auto issue = [&](auto masked, int slot, uint32_t k0, uint32_t k_oob, uint32_t stage_off) {
+                constexpr bool MASKED = decltype(masked)::value;
+                if(slot < NLA)
+                    __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_a, (lds_ptr_t)(smem + stage_off + (slot * NW + wave) * 1024),
+                                                             16, MASKED ? (a_off[slot] | k_oob) : a_off[slot], (int)k0, 0, 0);
+                else
+                    __builtin_amdgcn_raw_ptr_buffer_load_lds(
+                        rsrc_b, (lds_ptr_t)(smem + stage_off + A_TILE + ((slot - NLA) * NW + wave) * 1024), 16,
+                        MASKED ? (b_off[slot - NLA] | k_oob) : b_off[slot - NLA], (int)k0, 0, 0);
+            };
+            auto k_oob_of = [&](int kt) { return ((uint32_t)kt * BKB + kb < kbytes && kt < nk) ? 0u : kOutOfRange; };
+
+            acc_t acc[MT][NB];
+#pragma unroll
+            for(int i = 0; i < MT; ++i)
+#pragma unroll
+                for(int t = 0; t < NB; ++t)
+                    acc[i][t] = acc_t{0, 0, 0, 0};
+
+            // The previous tile's fragment reads are complete (its loop ends with a wait) but other waves may still be
+            // reading: one barrier before the stages are refilled. Its C stores share the load counter and are not
+            // ordered against loads: drained here, so that the counted wait below sees loads only.
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+            __builtin_amdgcn_s_barrier();
+#pragma unroll
+            for(int st = 0; st < NST; ++st)
+            {
+                const uint32_t oob = k_oob_of(st);
+#pragma unroll
+                for(int s = 0; s < LPT; ++s)
+                    issue(std::true_type{}, s, (uint32_t)st * BKB, oob, (uint32_t)(st * STAGE));
+            }
+            asm volatile("s_waitcnt vmcnt(%0)" ::"n"(LPT) : "memory");
+            __builtin_amdgcn_s_barrier();
+            asm volatile("" ::: "memory");
+
+            i32x4 af0[MT], bf0[NB], af1[MT], bf1[NB];
+            // fragment r of k-step ks of the stage at LDS address stage_lds: the B fragments first, then the A fragments
+            auto read_one = [&](uint32_t stage_lds, auto ks_c, auto r_c, i32x4(&af)[MT], i32x4(&bf)[NB]) {
+                constexpr int KS = decltype(ks_c)::value, R = decltype(r_c)::value;
+                if constexpr(R < NB)
+                    bf[R] = lds_read_b128<R * 16 * BKB>(stage_lds + fb[KS]);
+                else
+                    af[R - NB] = lds_read_b128<(R - NB) * 16 * BKB>(stage_lds + fa[KS]);
+            };
+            static_for<MT + NB>([&](auto r_c) { read_one(smem_lds, std::integral_constant<int, 0>{}, r_c, af0, bf0); });
+
+            // One half of an iteration: the 64 MFMAs of one k-step; behind every third MFMA one fragment read of the next
+            // k-step (16 reads, done after three quarters of the half); with_loads: behind every fourth MFMA one direct
+            // load of the K tile after next into the stage whose fragments are all in registers.
+            auto half_step = [&](auto with_loads, auto masked, uint32_t k0, uint32_t k_oob, uint32_t load_stage_off,
+                                 const i32x4(&caf)[MT], const i32x4(&cbf)[NB], uint32_t nstage_lds, auto nks,
+                                 i32x4(&naf)[MT], i32x4(&nbf)[NB]) {
+                static_for<NMH>([&](auto m_c) {
+                    constexpr int m = decltype(m_c)::value;
+                    if constexpr(decltype(with_loads)::value && m % 4 == 0)
+                    {
+                        issue(masked, m / 4, k0, k_oob, load_stage_off);
+                        __builtin_amdgcn_sched_barrier(0);
+                    }
+                    mfma<m / NB == MT - 1>(acc[m / NB][m % NB], cbf[m % NB], caf[m / NB]);
+                    if constexpr(m % 3 == 2 && m / 3 < MT + NB)
+                        read_one(nstage_lds, nks, std::integral_constant<int, m / 3>{}, naf, nbf);
+                    if constexpr(m % 4 == 3)
+                        __builtin_amdgcn_sched_barrier(0);
+                });
+            };
+
+            int st_cur = 0;
+            auto iteration = [&](auto masked, int kt) {
+                asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+                __builtin_amdgcn_sched_barrier(0);
+                half_step(std::false_type{}, masked, 0u, 0u, 0u, af0, bf0, smem_lds + (uint32_t)(st_cur * STAGE),
+                          std::integral_constant<int, 1>{}, af1, bf1);
+                // K tile kt is in registers, K tile kt + 1 has landed (the loads of a wave retire in order)
+                asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+                __builtin_amdgcn_sched_barrier(0);
+                __builtin_amdgcn_s_barrier();
+                asm volatile("" ::: "memory");
+                half_step(std::true_type{}, masked, (uint32_t)(kt + 2) * BKB,
+                          decltype(masked)::value ? k_oob_of(kt + 2) : 0u, (uint32_t)(st_cur * STAGE), af1, bf1,
+                          smem_lds + (uint32_t)((st_cur ^ 1) * STAGE), std::integral_constant<int, 0>{}, af0, bf0);
+                st_cur ^= 1;
+            };
+            // iterations whose loads fetch a whole K tile, then the (at most three) whose loads need the mask
+            const int nk_whole = (int)(kbytes / BKB);
+            int kt             = 0;
+            for(; kt + 2 < nk_whole; ++kt)
+                iteration(std::false_type{}, kt);
+            for(; kt < nk; ++kt)
+                iteration(std::true_type{}, kt);
+            // the trailing fragment reads and (all-zero) loads; the MFMA results must have left the pipeline before the
+            // epilogue reads them (inline-assembly MFMAs are invisible to the compiler's hazard handling)
+            asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_nop 15\n\ts_nop 15" ::: "memory");
+            __builtin_amdgcn_sched_barrier(0);
+
+            // ---- epilogue: 16 consecutive columns of one row per lane, fragment row by fragment row
+            const uint32_t lut_lds = smem_lds + (uint32_t)(NST * STAGE);
+            static_for<MT>([&](auto i_c) {
+                constexpr int i = decltype(i_c)::value;
+                const int m     = tm * BM + wm * 128 + 16 * i + (lane & 15);
+                const int nb    = tn * BN + wn * 128 + 16 * (lane >> 4); // first column of group 0; group 1 is 64 further
+                if constexpr(DT == DT_I8)
+                {
+                    if(p.epi == EPI_REQUANT_RND)
+                    {
+                        // the 32 values of the lane's two column groups go through the table behind ONE wait: with a single
+                        // wave per SIMD nothing else hides the latency of the byte reads
+                        i32x4 v[8];
+                        acc_t lo[4], hi[4];
+                        fetch_acc(std::integral_constant<bool, (i == MT - 1)>{}, acc[i], 0, lo);
+                        fetch_acc(std::integral_constant<bool, (i == MT - 1)>{}, acc[i], 1, hi);
+#pragma unroll
+                        for(int t = 0; t < 4; ++t)
+                            v[t] = lo[t], v[4 + t] = hi[t];
+                        int b[32];
+                        requant_lut<8>(v, p.scale_gemm, lut_lds, b);
+                        if(m < p.M)
+                        {
+                            int8_t* crow = reinterpret_cast<int8_t*>(p.c) + (size_t)m * p.ldc;
+                            if(nb < p.N)
+                                store_bytes16(crow, nb, p.N, vec_ok, b, nt);
+                            if(nb + 64 < p.N)
+                                store_bytes16(crow, nb + 64, p.N, vec_ok, b + 16, nt);
+                        }
+                        return;
+                    }
+                }
+#pragma unroll
+                for(int g = 0; g < 2; ++g)
+                {
+                    const int n0 = nb + 64 * g;
+                    if(m < p.M && n0 < p.N)
+                    {
+                        acc_t v[4];
+                        fetch_acc(std::integral_constant<bool, (i == MT - 1)>{}, acc[i], g, v);
+                        if constexpr(DT == DT_I8)
+                        {
+                            int8_t* crow = reinterpret_cast<int8_t*>(p.c) + (size_t)m * p.ldc;
+                            if(p.epi == EPI_REQUANT_CK)
+                                store_row16_i8<EPI_REQUANT_CK>(crow, n0, p.N, vec_ok, v, p.scale_gemm, p.scale_relu, nt);
+                            else
+                                store_row16_i8<EPI_PASSTHROUGH>(crow, n0, p.N, vec_ok, v, p.scale_gemm, p.scale_relu, nt);
+                        }
+                        else if constexpr(DT == DT_BF16)
+                            store_row16_f16(reinterpret_cast<__bf16*>(p.c) + (size_t)m * p.ldc, n0, p.N, vec_ok, v, nt);
+                        else
+                            store_row16_f16(reinterpret_cast<_Float16*>(p.c) + (size_t)m * p.ldc, n0, p.N, vec_ok, v, nt);
+                    }
+                }
+            });
+        }
+    }
+};
+
+template <int DT>
+__global__ __launch_bounds__(256) void gemm_w4_kernel(const GemmArgs p)
+{
+    extern __shared__ __attribute__((aligned(1024))) uint8_t ckx_smem[];
+    GemmW4<DT>::run(p, ckx_smem);
+}
+
+} // namespace ckx

@@ -393,6 +393,11 @@ int ckx_conv2d_fwd_plan(int op, const ckx_conv2d_desc* desc, int epilogue, int64
 /* Tuning / test knob: force `k_runs` K runs (0: automatic) wherever a problem and its workspace allow the split;
  * returns the value in force before. The initial value is the environment variable CKX_KSPLIT, read once. */
 int ckx_set_forced_k_runs(int k_runs);
+/* Tuning / test knob: the 256 x 256 tile instance has two kernel bodies for dense K-contiguous GEMMs with a plain
+ * epilogue -- eight waves (two per SIMD) and four waves (one per SIMD, 128 x 128 wave tiles), bit-identical results.
+ * 4 or 8 forces one of them wherever both apply, 0 lets the library choose by problem size; returns the value in force
+ * before. The initial value is the environment variable CKX_BIG_TILE_WAVES, read once. */
+int ckx_set_big_tile_waves(int waves);
 
 /* ---- timing helper --------------------------------------------------------
  * launch_and_time_kernel (include/ck/device_utility/kernel_launch.hpp:13-74):

@@ -1,0 +1,136 @@
+"""The 256 x 256 tile instance has two kernel bodies for dense K-contiguous GEMMs with a plain epilogue: eight waves
+(two per SIMD, 128 x 64 wave tiles) and four waves (one per SIMD, 128 x 128 wave tiles, accumulators in AccVGPRs).
+ckx_set_big_tile_waves forces either; the library chooses by problem size otherwise. Here the four-wave body runs every
+kind of shape -- ragged M and N, K tails, K of one tile and less, more tiles than CUs, padded C rows -- through the C ABI
+against the CPU oracle (int8 bit-exact in all three epilogues, fp16 / bf16 at rtol = atol = 1e-2 and bit-exact on integer
+operands), and against the eight-wave body bit for bit: both add the K tiles in the same order.
+"""
+import numpy as np
+import pytest
+
+import composable_kernel_amd as ck
+from composable_kernel_amd import capi
+from composable_kernel_amd.host_tensor import uniform_bf16, uniform_f16, uniform_int8
+from oracle import fast, lit
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture
+def waves():
+    def _set(n):
+        capi.lib().ckx_set_big_tile_waves(int(n))
+    yield _set
+    capi.lib().ckx_set_big_tile_waves(0)
+
+
+def _gemm_bf16(a, b_nk, instance=0):
+    import torch
+    import gpu_util
+    M, K = a.shape
+    N = b_nk.shape[0]
+    da, db = torch.from_numpy(a.view(np.int16)).cuda(), torch.from_numpy(b_nk.view(np.int16)).cuda()
+    dc = torch.full((M, N), 0x7FC0, dtype=torch.int16, device="cuda")
+    op = ck.DeviceGemmBF16(instance)
+    arg = op.MakeArgumentPointer(da, db, dc, M, N, K, K, K, N)
+    assert op.IsSupportedArgument(arg), capi.last_error()
+    op.MakeInvokerPointer().Run(arg, ck.StreamConfig(gpu_util.stream()))
+    torch.cuda.synchronize()
+    return dc.cpu().numpy().view(np.uint16)
+
+
+SHAPES = [(256, 256, 128), (256, 256, 64), (512, 768, 1024), (300, 520, 208), (1, 16, 16), (255, 257, 4096),
+          (513, 80, 1040), (1024, 1024, 2064), (77, 1000, 144)]
+OPS = {"pass": (ck.PassThrough(), lit.EPI_PASSTHROUGH, 1.0, 1.0),
+       "ck": (ck.RequantReluRequant(0.02, 0.4), lit.EPI_REQUANT_CK, 0.02, 0.4),
+       "rnd": (ck.RequantReluRequant(0.5, 0.03, rounded=True), lit.EPI_REQUANT_RND, 0.5, 0.03)}
+
+
+@pytest.mark.parametrize("shape", SHAPES)
+@pytest.mark.parametrize("op", list(OPS))
+def test_int8_four_wave_body_bit_exact(waves, shape, op):
+    import gpu_util
+    M, N, K = shape
+    a = uniform_int8((M, K), -5, 5, 3100 + M)
+    b_nk = uniform_int8((N, K), -5, 5, 3101 + N)
+    c_op, epi, sg, sr = OPS[op]
+    waves(4)
+    out = gpu_util.gemm_i8(a, b_nk, c_op, 0, ldc=N + 16)
+    np.testing.assert_array_equal(out, fast.gemm_i8(a, b_nk.T, epi, sg, sr))
+    waves(8)
+    np.testing.assert_array_equal(gpu_util.gemm_i8(a, b_nk, c_op, 0, ldc=N + 16), out)
+
+
+@pytest.mark.parametrize("shape", SHAPES)
+def test_fp16_four_wave_body(waves, shape):
+    import gpu_util
+    M, N, K = shape
+    a = uniform_f16((M, K), -1, 1, 3200 + M)
+    b_nk = uniform_f16((N, K), -1, 1, 3201 + N)
+    waves(4)
+    out = gpu_util.gemm_f16(a, b_nk, 0)
+    bad, max_err = lit.check_err_f16(out, fast.gemm_f16(a, b_nk.T), 1e-2, 1e-2)
+    assert bad == 0, max_err
+    waves(8)
+    np.testing.assert_array_equal(gpu_util.gemm_f16(a, b_nk, 0).view(np.uint16), out.view(np.uint16))
+    # integer operands: every partial sum is exact, the result is the integer matrix product
+    ai = uniform_int8((M, K), -3, 3, 3202).astype(np.float16)
+    bi = uniform_int8((N, K), -3, 3, 3203).astype(np.float16)
+    waves(4)
+    want = (ai.astype(np.float32) @ bi.T.astype(np.float32)).astype(np.float16)
+    np.testing.assert_array_equal(gpu_util.gemm_f16(ai, bi, 0), want)
+
+
+@pytest.mark.parametrize("shape", [(256, 256, 128), (300, 520, 208), (513, 80, 1040), (255, 257, 4096)])
+def test_bf16_four_wave_body(waves, shape):
+    M, N, K = shape
+    a = uniform_bf16((M, K), -1, 1, 3300 + M)
+    b_nk = uniform_bf16((N, K), -1, 1, 3301 + N)
+    waves(4)
+    out = _gemm_bf16(a, b_nk)
+    o, r = fast.bf16_to_f32(out), fast.bf16_to_f32(lit.gemm_bf16(a, b_nk.T) if M * N * K < 3e7 else fast.gemm_bf16(a, b_nk.T))
+    assert np.all(np.isfinite(o)) and np.all(np.abs(o - r) <= 1e-2 + 1e-2 * np.abs(r))
+    waves(8)
+    np.testing.assert_array_equal(_gemm_bf16(a, b_nk), out)
+
+
+def test_more_tiles_than_cus_and_empty_k(waves):
+    """17 x 17 tiles of 256 x 256 (289 workgroups' worth on 256 CUs: some workgroups take a second tile, with the C
+    stores of the first still in flight), and K = 0 (C = epilogue(0))."""
+    import gpu_util
+    M = N = 4352
+    K = 256
+    a = uniform_int8((M, K), -5, 5, 3400)
+    b_nk = uniform_int8((N, K), -5, 5, 3401)
+    c_op, epi, sg, sr = OPS["rnd"]
+    waves(4)
+    np.testing.assert_array_equal(gpu_util.gemm_i8(a, b_nk, c_op, 0), fast.gemm_i8(a, b_nk.T, epi, sg, sr))
+    af = uniform_f16((M, 192), -1, 1, 3402)
+    bf = uniform_f16((N, 192), -1, 1, 3403)
+    bad, max_err = lit.check_err_f16(gpu_util.gemm_f16(af, bf, 0), fast.gemm_f16(af, bf.T), 1e-2, 1e-2)
+    assert bad == 0, max_err
+    import torch
+    d = torch.ones(1 << 12, dtype=torch.float16, device="cuda")          # never read: K = 0
+    c = torch.full((300, 260), float("nan"), dtype=torch.float16, device="cuda")
+    op = ck.DeviceGemmF16(0)
+    arg = op.MakeArgumentPointer(d, d, c, 300, 260, 0, 8, 8, 260)
+    assert op.IsSupportedArgument(arg), capi.last_error()
+    op.MakeInvokerPointer().Run(arg, ck.StreamConfig(gpu_util.stream()))
+    torch.cuda.synchronize()
+    assert not c.cpu().numpy().any()
+
+
+def test_automatic_choice_is_either_body_with_identical_results(waves):
+    """Long K: the four-wave body is what the library picks for fp16; short K: the eight-wave one. The results do not
+    depend on it."""
+    import gpu_util
+    for K in (128, 2048):
+        a = uniform_f16((512, K), -1, 1, 3500 + K)
+        b_nk = uniform_f16((512, K), -1, 1, 3501 + K)
+        waves(0)
+        auto = gpu_util.gemm_f16(a, b_nk, 0)
+        for w in (4, 8):
+            waves(w)
+            np.testing.assert_array_equal(gpu_util.gemm_f16(a, b_nk, 0).view(np.uint16), auto.view(np.uint16))
+    assert capi.lib().ckx_set_big_tile_waves(0) == 8
+    assert capi.lib().ckx_set_big_tile_waves(5) == 0 and capi.lib().ckx_set_big_tile_waves(0) == 0   # 5 is not a choice
