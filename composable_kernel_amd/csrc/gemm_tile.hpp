@@ -786,7 +786,7 @@ struct GemmTile
                 if constexpr(TA)
                     voff = (a_off[j] + c.k0a) | (~(uint32_t)((int)(trow_a + j * NW * (1024 / (BM * ES))) - c.klim) & kOutOfRange);
                 else if constexpr(IM2COL == 0)
-                    voff = (a_off[j] + c.k0) | c.k_oob;
+                    voff = a_off[j] | c.k_oob; // (the K tile's offset travels in the scalar offset: one VALU instruction less)
                 else
                 {
                     const int hi0 = (int)a_hw0[j] >> 16, wi0 = (int)(a_hw0[j] << 16) >> 16;
@@ -797,16 +797,16 @@ struct GemmTile
                     voff = (a_off[j] + c.tap_off) | (ok ? 0u : kOutOfRange);
                 }
                 __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_a, (lds_ptr_t)(c.sa + (j * NW + wave) * 1024), 16,
-                                                         voff, 0, 0, 0);
+                                                         voff, (!TA && IM2COL == 0) ? (int)c.k0 : 0, 0, 0);
             }
             else
             {
                 const int j         = slot - NLA;
                 const uint32_t voff =
                     TB ? (b_off[j] + c.k0b) | (~(uint32_t)((int)(trow_b + j * NW * (1024 / (BN * ES))) - c.klim) & kOutOfRange)
-                       : (b_off[j] + c.k0) | c.k_oob;
+                       : b_off[j] | c.k_oob;
                 __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_b, (lds_ptr_t)(c.sb + (j * NW + wave) * 1024), 16,
-                                                         voff, 0, 0, 0);
+                                                         voff, TB ? 0 : (int)c.k0, 0, 0);
             }
         };
         auto issue_loads = [&](int kt, int stage) {

@@ -83,6 +83,49 @@ struct GemmW4
         }
     }
 
+    // LDS row of the staged B tile -> column of the tile. int8: b_row_to_col, a lane ends with 16 consecutive columns
+    // (one 16-byte store, four lanes = 64 contiguous bytes of a row). 16-bit outputs: within a 64-column group, MFMA tile
+    // t, MFMA row j = 4q + jj holds column 32 * (t / 2) + 8 * q + 4 * (t % 2) + jj, so the lane in 16-lane row q ends with
+    // columns 8q .. 8q + 7 (tiles 0, 1) and 32 + 8q .. 32 + 8q + 7 (tiles 2, 3): each of its two 16-byte stores joins
+    // those of the three other lanes of the row into 64 contiguous bytes, where 16 consecutive columns per lane would
+    // interleave the two stores' 16-byte pieces.
+    __device__ static __forceinline__ uint32_t row_to_col(uint32_t r)
+    {
+        if constexpr(DT == DT_I8)
+            return b_row_to_col(r);
+        else
+        {
+            const uint32_t t = (r >> 4) & 3u, q = (r & 15u) >> 2, jj = r & 3u;
+            return (r & ~63u) | ((t >> 1) << 5) | (q << 3) | ((t & 1u) << 2) | jj;
+        }
+    }
+    // the lane's 16 outputs of one row and 64-column group (first column n64) as two runs of 8 consecutive 16-bit values
+    template <typename T>
+    __device__ static __forceinline__ void store_2x8(T* crow, int n64, int q, int N, bool vec_ok, const f32x4 (&v)[4], bool nt)
+    {
+        typedef T tx8 __attribute__((ext_vector_type(8)));
+#pragma unroll
+        for(int h = 0; h < 2; ++h)
+        {
+            const int n0 = n64 + 32 * h + 8 * q;
+            if(vec_ok && n0 + 8 <= N)
+            {
+                tx8 x;
+#pragma unroll
+                for(int j = 0; j < 4; ++j)
+                    x[j] = (T)v[2 * h][j], x[4 + j] = (T)v[2 * h + 1][j];
+                store_vec(reinterpret_cast<tx8*>(crow + n0), x, nt);
+            }
+            else
+            {
+#pragma unroll
+                for(int e = 0; e < 8; ++e)
+                    if(n0 + e < N)
+                        crow[n0 + e] = (T)v[2 * h + e / 4][e % 4];
+            }
+        }
+    }
+
     // 16 consecutive int8 outputs of one row from their (already requantised) values b[0..15]
     __device__ static __forceinline__ void store_bytes16(int8_t* crow, int n0, int N, bool vec_ok, const int* b, bool nt)
     {
@@ -147,7 +190,7 @@ struct GemmW4
             {
                 const uint32_t r  = (uint32_t)((j * NW + wave) * 8 + (lane >> 3));
                 const uint32_t gm = (uint32_t)tm * BM + r;
-                const uint32_t gn = (uint32_t)tn * BN + b_row_to_col(r);
+                const uint32_t gn = (uint32_t)tn * BN + row_to_col(r);
                 a_off[j]          = gm < (uint32_t)p.M ? gm * (uint32_t)p.lda * ES + kb : kOutOfRange;
                 b_off[j]          = gn < (uint32_t)p.N ? gn * (uint32_t)p.ldb * ES + kb : kOutOfRange;
             }
@@ -288,23 +331,32 @@ struct GemmW4
 #pragma unroll
                 for(int g = 0; g < 2; ++g)
                 {
-                    const int n0 = nb + 64 * g;
-                    if(m < p.M && n0 < p.N)
+                    if constexpr(DT == DT_I8)
                     {
-                        acc_t v[4];
-                        fetch_acc(std::integral_constant<bool, (i == MT - 1)>{}, acc[i], g, v);
-                        if constexpr(DT == DT_I8)
+                        const int n0 = nb + 64 * g;
+                        if(m < p.M && n0 < p.N)
                         {
+                            acc_t v[4];
+                            fetch_acc(std::integral_constant<bool, (i == MT - 1)>{}, acc[i], g, v);
                             int8_t* crow = reinterpret_cast<int8_t*>(p.c) + (size_t)m * p.ldc;
                             if(p.epi == EPI_REQUANT_CK)
                                 store_row16_i8<EPI_REQUANT_CK>(crow, n0, p.N, vec_ok, v, p.scale_gemm, p.scale_relu, nt);
                             else
                                 store_row16_i8<EPI_PASSTHROUGH>(crow, n0, p.N, vec_ok, v, p.scale_gemm, p.scale_relu, nt);
                         }
-                        else if constexpr(DT == DT_BF16)
-                            store_row16_f16(reinterpret_cast<__bf16*>(p.c) + (size_t)m * p.ldc, n0, p.N, vec_ok, v, nt);
-                        else
-                            store_row16_f16(reinterpret_cast<_Float16*>(p.c) + (size_t)m * p.ldc, n0, p.N, vec_ok, v, nt);
+                    }
+                    else
+                    {
+                        const int n64 = tn * BN + wn * 128 + 64 * g;
+                        if(m < p.M && n64 < p.N)
+                        {
+                            acc_t v[4];
+                            fetch_acc(std::integral_constant<bool, (i == MT - 1)>{}, acc[i], g, v);
+                            if constexpr(DT == DT_BF16)
+                                store_2x8(reinterpret_cast<__bf16*>(p.c) + (size_t)m * p.ldc, n64, lane >> 4, p.N, vec_ok, v, nt);
+                            else
+                                store_2x8(reinterpret_cast<_Float16*>(p.c) + (size_t)m * p.ldc, n64, lane >> 4, p.N, vec_ok, v, nt);
+                        }
                     }
                 }
             });
