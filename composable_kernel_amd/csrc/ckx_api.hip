@@ -159,17 +159,15 @@ int big_tile_waves()
     return v;
 }
 // The four-wave body (one wave per SIMD, 128 x 128 wave tiles) has the faster K loop -- 18.0 against 18.9 cycles per
-// MFMA -- and the higher fixed cost (a lane zeroes, converts and stores twice as many accumulators with nothing to
-// overlap them; the int8 epilogues feel it most): measured faster from 16 K tiles on for fp16 / bf16 and from 32 on
-// for int8, and for int8 only while every CU gets at most one tile (the eight-wave body prefetches across tiles).
-bool four_wave_body_pays(int dt, int K, int tiles)
+// MFMA -- and, for 16-bit outputs, the faster stores (64-byte runs): measured ahead at every K for fp16 / bf16. Its int8
+// epilogues have nothing to overlap their table reads with (one wave per SIMD): behind by 0.6 us at one K tile with the
+// rounded requant, ahead from eight K tiles on.
+bool four_wave_body_pays(int dt, int K)
 {
     const int waves = big_tile_waves();
     if(waves)
         return waves == 4;
-    const int es = dt == ckx::DT_I8 ? 1 : 2;
-    const long nk = ((long)K * es + 127) / 128;
-    return dt == ckx::DT_I8 ? (nk >= 32 && tiles <= ckx::num_cus()) : nk >= 16;
+    return dt != ckx::DT_I8 || ((long)K + 127) / 128 >= 8;
 }
 
 // CKX_KSPLIT=n forces n K runs where the problem allows it (tuning / test knob). The environment is read on the first
@@ -635,7 +633,7 @@ int run_gemm(int dt, const void* a, const void* b, void* c, int M, int N, int K,
     g.ws         = ws;
     const bool fused            = f16_fused(epi) && g.ksplit == 1; // (after a K split the second pass applies it)
     const bool w4 = ti == 0 && !kmajor && batch == 1 && g.ksplit == 1 && epi <= CKX_EPI_REQUANT_RND &&
-                    four_wave_body_pays(dt, K, g.tiles_m * g.tiles_n);
+                    four_wave_body_pays(dt, K);
     const tile_launch_fn launch = w4                   ? ckx::w4_tile(dt)
                                   : kmajor             ? ckx::layout_tile(dt, ti, ta, tb)
                                   : dt == ckx::DT_I8   ? (per_column_scale(epi) && g.ksplit == 1 ? t.dense_i8_fused : t.dense_i8)

@@ -35,27 +35,33 @@ struct GemmW4
 
     // (the accumulators of the last fragment row stay in VGPRs: with all 256 AccVGPRs tied the allocator has no
     // register left to move one through and spills)
-    template <bool IN_VGPR>
+    // FIRST: the accumulator starts at zero (the literal 0 as the addend) instead of being read -- the first k-step of
+    // a tile, which saves zeroing 256 registers per lane beforehand
+    template <bool IN_VGPR, bool FIRST>
     __device__ static __forceinline__ void mfma(acc_t& c, const i32x4& b, const i32x4& a)
     {
-        if constexpr(IN_VGPR)
+#define CKX_W4_MFMA(OP)                                                                        \
+    if constexpr(IN_VGPR && FIRST)                                                             \
+        asm volatile(OP " %0, %1, %2, 0" : "=v"(c) : "v"(b), "v"(a));                          \
+    else if constexpr(IN_VGPR)                                                                 \
+        asm volatile(OP " %0, %1, %2, %0" : "+v"(c) : "v"(b), "v"(a));                         \
+    else if constexpr(FIRST)                                                                   \
+        asm volatile(OP " %0, %1, %2, 0" : "=a"(c) : "v"(b), "v"(a));                          \
+    else                                                                                       \
+        asm volatile(OP " %0, %1, %2, %0" : "+a"(c) : "v"(b), "v"(a));
+        if constexpr(DT == DT_I8)
         {
-            if constexpr(DT == DT_I8)
-                asm volatile("v_mfma_i32_16x16x64_i8 %0, %1, %2, %0" : "+v"(c) : "v"(b), "v"(a));
-            else if constexpr(DT == DT_BF16)
-                asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+v"(c) : "v"(b), "v"(a));
-            else
-                asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+v"(c) : "v"(b), "v"(a));
+            CKX_W4_MFMA("v_mfma_i32_16x16x64_i8")
+        }
+        else if constexpr(DT == DT_BF16)
+        {
+            CKX_W4_MFMA("v_mfma_f32_16x16x32_bf16")
         }
         else
         {
-            if constexpr(DT == DT_I8)
-                asm volatile("v_mfma_i32_16x16x64_i8 %0, %1, %2, %0" : "+a"(c) : "v"(b), "v"(a));
-            else if constexpr(DT == DT_BF16)
-                asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+a"(c) : "v"(b), "v"(a));
-            else
-                asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+a"(c) : "v"(b), "v"(a));
+            CKX_W4_MFMA("v_mfma_f32_16x16x32_f16")
         }
+#undef CKX_W4_MFMA
     }
 
     // The four accumulator tuples of column group g of one fragment row, as VGPR values. Read out of the AccVGPRs by
@@ -212,12 +218,7 @@ struct GemmW4
             };
             auto k_oob_of = [&](int kt) { return ((uint32_t)kt * BKB + kb < kbytes && kt < nk) ? 0u : kOutOfRange; };
 
-            acc_t acc[MT][NB];
-#pragma unroll
-            for(int i = 0; i < MT; ++i)
-#pragma unroll
-                for(int t = 0; t < NB; ++t)
-                    acc[i][t] = acc_t{0, 0, 0, 0};
+            acc_t acc[MT][NB]; // (defined by the first k-step's MFMAs)
 
             // The previous tile's fragment reads are complete (its loop ends with a wait) but other waves may still be
             // reading: one barrier before the stages are refilled. Its C stores share the load counter and are not
@@ -250,7 +251,7 @@ struct GemmW4
             // One half of an iteration: the 64 MFMAs of one k-step; behind every third MFMA one fragment read of the next
             // k-step (16 reads, done after three quarters of the half); with_loads: behind every fourth MFMA one direct
             // load of the K tile after next into the stage whose fragments are all in registers.
-            auto half_step = [&](auto with_loads, auto masked, uint32_t k0, uint32_t k_oob, uint32_t load_stage_off,
+            auto half_step = [&](auto first, auto with_loads, auto masked, uint32_t k0, uint32_t k_oob, uint32_t load_stage_off,
                                  const i32x4(&caf)[MT], const i32x4(&cbf)[NB], uint32_t nstage_lds, auto nks,
                                  i32x4(&naf)[MT], i32x4(&nbf)[NB]) {
                 static_for<NMH>([&](auto m_c) {
@@ -260,7 +261,7 @@ struct GemmW4
                         issue(masked, m / 4, k0, k_oob, load_stage_off);
                         __builtin_amdgcn_sched_barrier(0);
                     }
-                    mfma<m / NB == MT - 1>(acc[m / NB][m % NB], cbf[m % NB], caf[m / NB]);
+                    mfma<m / NB == MT - 1, decltype(first)::value>(acc[m / NB][m % NB], cbf[m % NB], caf[m / NB]);
                     if constexpr(m % 3 == 2 && m / 3 < MT + NB)
                         read_one(nstage_lds, nks, std::integral_constant<int, m / 3>{}, naf, nbf);
                     if constexpr(m % 4 == 3)
@@ -269,28 +270,29 @@ struct GemmW4
             };
 
             int st_cur = 0;
-            auto iteration = [&](auto masked, int kt) {
+            auto iteration = [&](auto first, auto masked, int kt) {
                 asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
                 __builtin_amdgcn_sched_barrier(0);
-                half_step(std::false_type{}, masked, 0u, 0u, 0u, af0, bf0, smem_lds + (uint32_t)(st_cur * STAGE),
+                half_step(first, std::false_type{}, masked, 0u, 0u, 0u, af0, bf0, smem_lds + (uint32_t)(st_cur * STAGE),
                           std::integral_constant<int, 1>{}, af1, bf1);
                 // K tile kt is in registers, K tile kt + 1 has landed (the loads of a wave retire in order)
                 asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
                 __builtin_amdgcn_sched_barrier(0);
                 __builtin_amdgcn_s_barrier();
                 asm volatile("" ::: "memory");
-                half_step(std::true_type{}, masked, (uint32_t)(kt + 2) * BKB,
+                half_step(std::false_type{}, std::true_type{}, masked, (uint32_t)(kt + 2) * BKB,
                           decltype(masked)::value ? k_oob_of(kt + 2) : 0u, (uint32_t)(st_cur * STAGE), af1, bf1,
                           smem_lds + (uint32_t)((st_cur ^ 1) * STAGE), std::integral_constant<int, 0>{}, af0, bf0);
                 st_cur ^= 1;
             };
             // iterations whose loads fetch a whole K tile, then the (at most three) whose loads need the mask
             const int nk_whole = (int)(kbytes / BKB);
-            int kt             = 0;
+            iteration(std::true_type{}, std::true_type{}, 0);
+            int kt = 1;
             for(; kt + 2 < nk_whole; ++kt)
-                iteration(std::false_type{}, kt);
+                iteration(std::false_type{}, std::false_type{}, kt);
             for(; kt < nk; ++kt)
-                iteration(std::true_type{}, kt);
+                iteration(std::false_type{}, std::true_type{}, kt);
             // the trailing fragment reads and (all-zero) loads; the MFMA results must have left the pipeline before the
             // epilogue reads them (inline-assembly MFMAs are invisible to the compiler's hazard handling)
             asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_nop 15\n\ts_nop 15" ::: "memory");
