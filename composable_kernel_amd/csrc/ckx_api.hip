@@ -632,9 +632,10 @@ int run_gemm(int dt, const void* a, const void* b, void* c, int M, int N, int K,
     g.nk_per     = pl.nk_per;
     g.ws         = ws;
     const bool fused            = f16_fused(epi) && g.ksplit == 1; // (after a K split the second pass applies it)
-    const bool w4 = ti == 0 && !kmajor && batch == 1 && g.ksplit == 1 && epi <= CKX_EPI_REQUANT_RND &&
-                    four_wave_body_pays(dt, K);
-    const tile_launch_fn launch = w4                   ? ckx::w4_tile(dt)
+    // (the functors with a second D tensor stay on the eight-wave body: see the fused epilogue of gemm_w4.hpp)
+    const bool w4 = ti == 0 && !kmajor && batch == 1 && g.ksplit == 1 &&
+                    (epi <= CKX_EPI_REQUANT_RND || (f16_fused(epi) && !uses_d1(epi))) && four_wave_body_pays(dt, K);
+    const tile_launch_fn launch = w4                   ? ckx::w4_tile(dt, fused)
                                   : kmajor             ? ckx::layout_tile(dt, ti, ta, tb)
                                   : dt == ckx::DT_I8   ? (per_column_scale(epi) && g.ksplit == 1 ? t.dense_i8_fused : t.dense_i8)
                                   : dt == ckx::DT_BF16 ? t.dense_bf16

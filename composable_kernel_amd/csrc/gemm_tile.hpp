@@ -416,7 +416,8 @@ __device__ __forceinline__ void load_col_scales(const __amdgpu_buffer_rsrc_t& rs
 // example/03_gemm_bias_relu on the accumulator already rounded to fp16).
 // EXT = false leaves the scaled / GELU modes out of the generated code (callers that have already branched on them).
 // fast_gelu(x) = x / (1 + exp(-2x(0.035677 x^2 + 0.797885))), the closed form of the reference's
-// 0.5 + 0.5 * (2 / (1 + emu) - 1) (element_wise_operation.hpp:127-133); x -> -inf gives exp -> +inf and -0.
+// 0.5 + 0.5 * (2 / (1 + emu) - 1) (element_wise_operation.hpp:127-133), the quotient through v_rcp_f32;
+// x -> -inf gives exp -> +inf, a reciprocal of 0 and -0.
 template <bool EXT = true>
 __device__ __forceinline__ float epi_f16_value(int mode, float acc, float d0, float d1, float alpha = 1.0f,
                                                float beta = 1.0f)
@@ -429,7 +430,7 @@ __device__ __forceinline__ float epi_f16_value(int mode, float acc, float d0, fl
         {
             const float x = acc + d0 + d1;
             const float u = 2.0f * x * (0.035677f * x * x + 0.797885f);
-            return x / (1.0f + __expf(-u));
+            return x * __builtin_amdgcn_rcpf(1.0f + __expf(-u)); // (one ulp of fp32: far inside the fp16 result's rounding)
         }
     }
     if(mode == EPI_CSHUFFLE_ADD_RELU)

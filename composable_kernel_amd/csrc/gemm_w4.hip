@@ -7,15 +7,16 @@
 namespace ckx {
 namespace {
 
-template <int DT>
+template <int DT, bool FUSED = false>
 hipError_t launch_w4(const GemmArgs& a, int tiles, hipStream_t s)
 {
-    auto* kern = &gemm_w4_kernel<DT>;
+    using T    = GemmW4<DT, FUSED>;
+    auto* kern = &gemm_w4_kernel<DT, FUSED>;
     static std::once_flag once;
     static hipError_t attr_err = hipSuccess;
     std::call_once(once, [&] {
         attr_err = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                       GemmW4<DT>::LDS);
+                                       T::LDS);
     });
     if(attr_err != hipSuccess)
         return attr_err;
@@ -23,14 +24,16 @@ hipError_t launch_w4(const GemmArgs& a, int tiles, hipStream_t s)
     int grid = num_cus();
     grid -= grid % 8;
     grid = tiles < grid ? tiles : grid;
-    hipLaunchKernelGGL(kern, dim3(grid), dim3(GemmW4<DT>::NT), GemmW4<DT>::LDS, s, a);
+    hipLaunchKernelGGL(kern, dim3(grid), dim3(T::NT), T::LDS, s, a);
     return hipGetLastError();
 }
 
 } // namespace
 
-tile_launch_fn w4_tile(int dt)
+tile_launch_fn w4_tile(int dt, bool fused)
 {
+    if(fused)
+        return dt == DT_F16 ? &launch_w4<DT_F16, true> : nullptr;
     return dt == DT_I8 ? &launch_w4<DT_I8> : dt == DT_BF16 ? &launch_w4<DT_BF16> : &launch_w4<DT_F16>;
 }
 

@@ -20,9 +20,12 @@
 
 namespace ckx {
 
-template <int DT>
+// FUSED (fp16): the epilogues with D operands (add / ReLU functors, Bilinear, AddAddFastGelu) as a kernel of their own,
+// like the FUSED variants of the tile kernel.
+template <int DT, bool FUSED = false>
 struct GemmW4
 {
+    static_assert(!FUSED || DT == DT_F16, "D-operand epilogues: fp16");
     static constexpr int BM = 256, BN = 256, BKB = 128, NW = 4, NT = NW * 64, NST = 2;
     static constexpr int ES     = DT == DT_I8 ? 1 : 2;
     static constexpr int A_TILE = BM * BKB, B_TILE = BN * BKB, STAGE = A_TILE + B_TILE;
@@ -300,6 +303,101 @@ struct GemmW4
 
             // ---- epilogue: 16 consecutive columns of one row per lane, fragment row by fragment row
             const uint32_t lut_lds = smem_lds + (uint32_t)(NST * STAGE);
+            if constexpr(FUSED)
+            {
+                if(p.epi != EPI_PASSTHROUGH)
+                {
+                    // A load issued after a store waits for that store too, and this SIMD has no other wave to run
+                    // meanwhile: the D values of a whole chunk of fragment rows -- four with one D tensor, two with two (64
+                    // registers; eight and four spill) -- are requested before the chunk's first store; a bias row
+                    // (stride 0) once per tile. The functor is a compile-time constant of each copy of
+                    // the epilogue: a run-time switch per value costs hundreds of scalar branches per tile.
+                    const _Float16* d0  = reinterpret_cast<const _Float16*>(p.d0);
+                    const _Float16* d1  = reinterpret_cast<const _Float16*>(p.d1);
+                    const bool d0_rows  = p.ldd0 != 0;
+                    const bool dvec_ok  = ((reinterpret_cast<uintptr_t>(p.d0) | ((uintptr_t)p.ldd0 * ES) |
+                                           reinterpret_cast<uintptr_t>(p.d1) | ((uintptr_t)p.ldd1 * ES)) & 15u) == 0;
+                    const int q         = lane >> 4;
+                    const f16x8 zero8   = {0, 0, 0, 0, 0, 0, 0, 0};
+                    auto load8          = [&](const _Float16* row, int n0) {
+                        f16x8 x = zero8;
+                        if(dvec_ok && n0 + 8 <= p.N)
+                            x = *reinterpret_cast<const f16x8*>(row + n0);
+                        else
+                        {
+#pragma unroll
+                            for(int e = 0; e < 8; ++e)
+                                if(n0 + e < p.N)
+                                    x[e] = row[n0 + e];
+                        }
+                        return x;
+                    };
+                    auto col0 = [&](int g, int h) { return tn * BN + wn * 128 + 64 * g + 32 * h + 8 * q; };
+                    auto with_functor = [&](auto mode_c) {
+                        constexpr int MODE    = decltype(mode_c)::value;
+                        constexpr bool HAS_D1 = epi_has_d1(MODE);
+                        constexpr int CH      = HAS_D1 ? 2 : 4;
+                        f16x8 bias[2][2];
+#pragma unroll
+                        for(int g = 0; g < 2; ++g)
+#pragma unroll
+                            for(int h = 0; h < 2; ++h)
+                                bias[g][h] = (!d0_rows && col0(g, h) < p.N) ? load8(d0, col0(g, h)) : zero8;
+                        static_for<MT / CH>([&](auto chunk_c) {
+                            constexpr int i0 = decltype(chunk_c)::value * CH;
+                            f16x8 x[CH][2][2], y[HAS_D1 ? CH : 1][2][2];
+#pragma unroll
+                            for(int c = 0; c < CH; ++c)
+                            {
+                                const int m = tm * BM + wm * 128 + 16 * (i0 + c) + (lane & 15);
+#pragma unroll
+                                for(int g = 0; g < 2; ++g)
+#pragma unroll
+                                    for(int h = 0; h < 2; ++h)
+                                    {
+                                        const bool live = m < p.M && col0(g, h) < p.N;
+                                        x[c][g][h] = (live && d0_rows) ? load8(d0 + (size_t)m * p.ldd0, col0(g, h)) : bias[g][h];
+                                        if constexpr(HAS_D1)
+                                            y[c][g][h] = live ? load8(d1 + (size_t)m * p.ldd1, col0(g, h)) : zero8;
+                                    }
+                            }
+                            static_for<CH>([&](auto c_c) {
+                                constexpr int c = decltype(c_c)::value, i = i0 + c;
+                                const int m     = tm * BM + wm * 128 + 16 * i + (lane & 15);
+#pragma unroll
+                                for(int g = 0; g < 2; ++g)
+                                {
+                                    const int n64 = tn * BN + wn * 128 + 64 * g;
+                                    acc_t v[4];
+                                    fetch_acc(std::integral_constant<bool, (i == MT - 1)>{}, acc[i], g, v);
+#pragma unroll
+                                    for(int t = 0; t < 4; ++t)
+#pragma unroll
+                                        for(int j = 0; j < 4; ++j)
+                                        {
+                                            const int h = t >> 1, e = 4 * (t & 1) + j;
+                                            const float yv = HAS_D1 ? (float)y[HAS_D1 ? c : 0][g][h][e] : 0.0f;
+                                            v[t][j] = epi_f16_value<(MODE >= EPI_BILINEAR)>(MODE, v[t][j], (float)x[c][g][h][e], yv,
+                                                                                          p.scale_gemm, p.scale_relu);
+                                        }
+                                    if(m < p.M && n64 < p.N)
+                                        store_2x8(reinterpret_cast<_Float16*>(p.c) + (size_t)m * p.ldc, n64, q, p.N, vec_ok, v, nt);
+                                }
+                            });
+                        });
+                    };
+                    using std::integral_constant;
+                    // (the host sends the functors with a second D tensor to the eight-wave body: their chunks of two
+                    // fragment rows serialise four times per tile here -- AddAddFastGelu 125 against 116 us at 4096^3)
+                    if(p.epi == EPI_ADD_RELU)
+                        with_functor(integral_constant<int, EPI_ADD_RELU>{});
+                    else if(p.epi == EPI_CSHUFFLE_ADD_RELU)
+                        with_functor(integral_constant<int, EPI_CSHUFFLE_ADD_RELU>{});
+                    else
+                        with_functor(integral_constant<int, EPI_BILINEAR>{});
+                    continue;
+                }
+            }
             static_for<MT>([&](auto i_c) {
                 constexpr int i = decltype(i_c)::value;
                 const int m     = tm * BM + wm * 128 + 16 * i + (lane & 15);
@@ -366,11 +464,11 @@ struct GemmW4
     }
 };
 
-template <int DT>
+template <int DT, bool FUSED = false>
 __global__ __launch_bounds__(256) void gemm_w4_kernel(const GemmArgs p)
 {
     extern __shared__ __attribute__((aligned(1024))) uint8_t ckx_smem[];
-    GemmW4<DT>::run(p, ckx_smem);
+    GemmW4<DT, FUSED>::run(p, ckx_smem);
 }
 
 } // namespace ckx

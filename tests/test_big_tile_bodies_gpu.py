@@ -133,3 +133,49 @@ def test_automatic_choice_is_either_body_with_identical_results(waves):
             np.testing.assert_array_equal(gpu_util.gemm_f16(a, b_nk, 0).view(np.uint16), auto.view(np.uint16))
     assert capi.lib().ckx_set_big_tile_waves(0) == 8
     assert capi.lib().ckx_set_big_tile_waves(5) == 0 and capi.lib().ckx_set_big_tile_waves(0) == 0   # 5 is not a choice
+
+
+@pytest.mark.parametrize("shape", [(256, 256, 128), (300, 520, 208), (1024, 1024, 1040), (77, 1000, 144)])
+def test_fp16_d_operand_epilogues_on_both_bodies(waves, shape):
+    """AddRelu (C rounded first) and Bilinear run on either body, bit-identical; the functors with two D tensors
+    (AddReluAdd, AddAddFastGelu) stay on the eight-wave body whatever the knob says. All against the oracle; bias row
+    and full D tensors, padded strides."""
+    import torch
+    import gpu_util
+    M, N, K = shape
+    a = uniform_f16((M, K), -0.5, 0.5, 3600 + M)
+    b_nk = uniform_f16((N, K), -0.5, 0.5, 3601 + N)
+    row = uniform_f16((1, N), -2, 2, 3602)
+    full = uniform_f16((M, N + 8), -2, 2, 3603)
+    full2 = uniform_f16((M, N), -2, 2, 3604)
+    acc = a.astype(np.float32) @ b_nk.T.astype(np.float32)
+    cases = [
+        (ck.AddRelu(), [row], [0], fast.gemm_f16_add_relu(a, b_nk.T, row)),
+        (ck.AddRelu(), [full], [N + 8], fast.gemm_f16_add_relu(a, b_nk.T, full[:, :N])),
+        (ck.AddReluAdd(), [row, full], [0, N + 8],
+         (np.maximum(acc + row.astype(np.float32), 0) + full[:, :N].astype(np.float32)).astype(np.float16)),
+        (ck.AddReluAdd(), [full2, full], [N, N + 8],
+         (np.maximum(acc + full2.astype(np.float32), 0) + full[:, :N].astype(np.float32)).astype(np.float16)),
+        (ck.Bilinear(0.75, -1.5), [full], [N + 8], fast.gemm_f16_bilinear(a, b_nk.T, full[:, :N], 0.75, -1.5)),
+        (ck.Bilinear(2.0, 0.5), [row], [0], fast.gemm_f16_bilinear(a, b_nk.T, row, 2.0, 0.5)),
+        (ck.AddAddFastGelu(), [row, full], [0, N + 8], fast.gemm_f16_add_add_fastgelu(a, b_nk.T, row, full[:, :N])),
+        (ck.AddAddFastGelu(), [full, full2], [N + 8, N], fast.gemm_f16_add_add_fastgelu(a, b_nk.T, full[:, :N], full2)),
+    ]
+    da, db = gpu_util.dev(a), gpu_util.dev(b_nk)
+    for functor, ds, strides, want in cases:
+        outs = []
+        for w in (4, 8):
+            waves(w)
+            dds = [gpu_util.dev(d) for d in ds]
+            de = torch.full((M, N + 24), 77.0, dtype=torch.float16, device="cuda")
+            op = ck.DeviceGemmMultipleDF16(0)
+            arg = op.MakeArgumentPointer(da, db, dds, de, M, N, K, K, K, strides, N + 24, None, None, functor)
+            assert op.IsSupportedArgument(arg), capi.last_error()
+            op.MakeInvokerPointer().Run(arg, ck.StreamConfig(gpu_util.stream()))
+            torch.cuda.synchronize()
+            out = de.cpu().numpy()
+            assert np.all(out[:, N:] == 77.0)
+            outs.append(out[:, :N].copy())
+        bad, max_err = lit.check_err_f16(outs[0], want, 1e-2, 1e-2)
+        assert bad == 0, (type(functor).__name__, max_err)
+        np.testing.assert_array_equal(outs[0].view(np.uint16), outs[1].view(np.uint16))
