@@ -246,7 +246,9 @@ Plan make_plan(long M, int N, int kbytes, int only_tile, long workspace_bytes, i
             // three and more co-resident workgroups pull their K tiles through ONE CU's load path: 105 GB/s out of L2
             // with every CU busy (measured with a streaming probe), 85 in a kernel that also computes. Without this term
             // 128 x 64 tiles at three per CU were rated 43 us on fp16 512 x 11008 x 4096 and took 60 (256 x 128: 48).
-            if(per_cu >= 3)
+            // (GEMM launches only: an im2col A operand re-reads its pixels out of L1 / L2 tap after tap, and with the term
+            // the 3-D layer 4 x 28^3 x 64 -> 256, stride 2, went from the 64 x 64 tile, 24.7 us, to 256 x 64 at 35.9)
+            if(per_cu >= 3 && !conv)
             {
                 const double load_us = per_cu * (double)(t.bm + t.bn) * 128.0 / 85.0e3;
                 iter_us              = iter_us < load_us ? load_us : iter_us;
