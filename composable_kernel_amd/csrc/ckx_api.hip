@@ -635,7 +635,7 @@ int run_gemm(int dt, const void* a, const void* b, void* c, int M, int N, int K,
     g.ws         = ws;
     const bool fused            = f16_fused(epi) && g.ksplit == 1; // (after a K split the second pass applies it)
     // (the functors with a second D tensor stay on the eight-wave body: see the fused epilogue of gemm_w4.hpp)
-    const bool w4 = ti == 0 && !kmajor && batch == 1 && g.ksplit == 1 &&
+    const bool w4 = ti == 0 && !kmajor && g.ksplit == 1 &&
                     (epi <= CKX_EPI_REQUANT_RND || (f16_fused(epi) && !uses_d1(epi))) && four_wave_body_pays(dt, K);
     const tile_launch_fn launch = w4                   ? ckx::w4_tile(dt, fused)
                                   : kmajor             ? ckx::layout_tile(dt, ti, ta, tb)

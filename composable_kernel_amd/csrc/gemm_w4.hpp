@@ -1,5 +1,5 @@
 // 256 x 256 C tile computed by FOUR waves -- one per SIMD, wave tile 128 x 128 -- for dense K-contiguous GEMMs
-// (A row-major, B column-major) whose tiles give every CU one round of work.
+// (A row-major, B column-major, optionally a strided batch of them) whose tiles give every CU one round of work.
 //
 // Same data path as gemm_tile.hpp (128-byte K tiles, direct global->LDS loads with the XOR swizzle and the B row
 // permutation applied by the choice of each lane's global chunk, D^T = B_frag x A_frag, register epilogue, 16 contiguous
@@ -161,7 +161,8 @@ struct GemmW4
         const int lane = tid & 63;
         const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
         const int wm = wave >> 1, wn = wave & 1;
-        const int ntiles      = p.tiles_m * p.tiles_n;
+        const int nbatch      = p.batch > 0 ? p.batch : 1;
+        const int ntiles      = p.tiles_m * p.tiles_n * nbatch; // C tiles of all batches, dealt to the XCDs batch by batch
         const uint32_t kbytes = (uint32_t)p.K * ES;
         const int nk_real     = (int)((kbytes + BKB - 1) / BKB);
         const int nk          = nk_real > 0 ? nk_real : 1;
@@ -186,13 +187,16 @@ struct GemmW4
         const uint32_t fa[2] = {frag_part(wm * 128, 0), frag_part(wm * 128, 1)};
         const uint32_t fb[2] = {A_TILE + frag_part(wn * 128, 0), A_TILE + frag_part(wn * 128, 1)};
 
-        const bool vec_ok = ((reinterpret_cast<uintptr_t>(p.c) | ((uintptr_t)p.ldc * ES)) & 15u) == 0;
+        const bool vec_ok = ((reinterpret_cast<uintptr_t>(p.c) | ((uintptr_t)p.ldc * ES) |
+                              (nbatch > 1 ? (uintptr_t)p.bsc * ES : 0)) & 15u) == 0;
         const bool nt     = p.nt_store != 0;
 
         for(int unit = (int)blockIdx.x; unit < ntiles; unit += (int)gridDim.x)
         {
             int tm, tn, bi;
-            tile_of_block(unit, p.tiles_m, p.tiles_n, 1, bi, tm, tn);
+            tile_of_block(unit, p.tiles_m, p.tiles_n, nbatch, bi, tm, tn);
+            const uint32_t a_batch = (uint32_t)((long)bi * p.bsa * ES), b_batch = (uint32_t)((long)bi * p.bsb * ES);
+            uint8_t* const c_batch = reinterpret_cast<uint8_t*>(p.c) + (size_t)bi * p.bsc * ES;
             uint32_t a_off[NLA], b_off[NLB];
 #pragma unroll
             for(int j = 0; j < NLA; ++j)
@@ -200,8 +204,8 @@ struct GemmW4
                 const uint32_t r  = (uint32_t)((j * NW + wave) * 8 + (lane >> 3));
                 const uint32_t gm = (uint32_t)tm * BM + r;
                 const uint32_t gn = (uint32_t)tn * BN + row_to_col(r);
-                a_off[j]          = gm < (uint32_t)p.M ? gm * (uint32_t)p.lda * ES + kb : kOutOfRange;
-                b_off[j]          = gn < (uint32_t)p.N ? gn * (uint32_t)p.ldb * ES + kb : kOutOfRange;
+                a_off[j]          = gm < (uint32_t)p.M ? a_batch + gm * (uint32_t)p.lda * ES + kb : kOutOfRange;
+                b_off[j]          = gn < (uint32_t)p.N ? b_batch + gn * (uint32_t)p.ldb * ES + kb : kOutOfRange;
             }
             // One direct load: slot < NLA an A row group, else a B row group, of the K tile at byte offset k0 into the
             // stage at stage_off. k0 travels in the instruction's scalar offset, which the address uses and the range check
@@ -381,7 +385,7 @@ struct GemmW4
                                                                                           p.scale_gemm, p.scale_relu);
                                         }
                                     if(m < p.M && n64 < p.N)
-                                        store_2x8(reinterpret_cast<_Float16*>(p.c) + (size_t)m * p.ldc, n64, q, p.N, vec_ok, v, nt);
+                                        store_2x8(reinterpret_cast<_Float16*>(c_batch) + (size_t)m * p.ldc, n64, q, p.N, vec_ok, v, nt);
                                 }
                             });
                         });
@@ -419,7 +423,7 @@ struct GemmW4
                         requant_lut<8>(v, p.scale_gemm, lut_lds, b);
                         if(m < p.M)
                         {
-                            int8_t* crow = reinterpret_cast<int8_t*>(p.c) + (size_t)m * p.ldc;
+                            int8_t* crow = reinterpret_cast<int8_t*>(c_batch) + (size_t)m * p.ldc;
                             if(nb < p.N)
                                 store_bytes16(crow, nb, p.N, vec_ok, b, nt);
                             if(nb + 64 < p.N)
@@ -438,7 +442,7 @@ struct GemmW4
                         {
                             acc_t v[4];
                             fetch_acc(std::integral_constant<bool, (i == MT - 1)>{}, acc[i], g, v);
-                            int8_t* crow = reinterpret_cast<int8_t*>(p.c) + (size_t)m * p.ldc;
+                            int8_t* crow = reinterpret_cast<int8_t*>(c_batch) + (size_t)m * p.ldc;
                             if(p.epi == EPI_REQUANT_CK)
                                 store_row16_i8<EPI_REQUANT_CK>(crow, n0, p.N, vec_ok, v, p.scale_gemm, p.scale_relu, nt);
                             else
@@ -453,9 +457,9 @@ struct GemmW4
                             acc_t v[4];
                             fetch_acc(std::integral_constant<bool, (i == MT - 1)>{}, acc[i], g, v);
                             if constexpr(DT == DT_BF16)
-                                store_2x8(reinterpret_cast<__bf16*>(p.c) + (size_t)m * p.ldc, n64, lane >> 4, p.N, vec_ok, v, nt);
+                                store_2x8(reinterpret_cast<__bf16*>(c_batch) + (size_t)m * p.ldc, n64, lane >> 4, p.N, vec_ok, v, nt);
                             else
-                                store_2x8(reinterpret_cast<_Float16*>(p.c) + (size_t)m * p.ldc, n64, lane >> 4, p.N, vec_ok, v, nt);
+                                store_2x8(reinterpret_cast<_Float16*>(c_batch) + (size_t)m * p.ldc, n64, lane >> 4, p.N, vec_ok, v, nt);
                         }
                     }
                 }

@@ -69,7 +69,7 @@ hipError_t launch_tile(const GemmArgs& a, int tiles, hipStream_t s)
 // null when that tile shape has no such variant (fewer than 64 rows)
 tile_launch_fn layout_tile(int dt, int tile, bool a_kmajor, bool b_kmajor);
 
-// four-wave body of the 256 x 256 tile instance (gemm_w4.hip): dense K-contiguous GEMM, one K run, no batch; launcher for
+// four-wave body of the 256 x 256 tile instance (gemm_w4.hip): dense K-contiguous GEMM or strided batch, one K run; launcher for
 // element type dt (DT_*) with the plain epilogues (PassThrough and the two uniform requant modes) or, fused (fp16 only,
 // else null), with the D-operand epilogues
 tile_launch_fn w4_tile(int dt, bool fused);

@@ -179,3 +179,32 @@ def test_fp16_d_operand_epilogues_on_both_bodies(waves, shape):
         bad, max_err = lit.check_err_f16(outs[0], want, 1e-2, 1e-2)
         assert bad == 0, (type(functor).__name__, max_err)
         np.testing.assert_array_equal(outs[0].view(np.uint16), outs[1].view(np.uint16))
+
+
+@pytest.mark.parametrize("case", [(3, 256, 256, 128, (0, 0, 0), False), (3, 130, 200, 272, (16, 32, 8), False),
+                                  (5, 300, 72, 1040, (0, 0, 24), True), (20, 512, 256, 1024, (0, 0, 0), False)])
+def test_strided_batches_on_both_bodies(waves, case):
+    """DeviceBatchedGemm on tile instance 0: the tiles of all batches are one work list for either body (padded batch
+    strides, a B matrix shared by all batches, more tiles than CUs in the last case)."""
+    import torch
+    from test_batched_gemm_gpu import _run as run_batched
+    G, M, N, K, bs, share_b = case
+    a = uniform_int8((G, M, K), -8, 8, 3700 + M)
+    b = uniform_int8((G, N, K), -8, 8, 3701 + N)
+    if share_b:
+        b[:] = b[0]
+    c_op = ck.RequantReluRequant(0.02, 0.4, rounded=True)
+    af, bf = uniform_f16((G, M, K), -1, 1, 3702), uniform_f16((G, N, K), -1, 1, 3703)
+    if share_b:
+        bf[:] = bf[0]
+    outs = {}
+    for w in (4, 8):
+        waves(w)
+        outs[w] = (run_batched(ck.DeviceBatchedGemmInt8(0), a, b, torch.int8, bs, share_b, c_op),
+                   run_batched(ck.DeviceBatchedGemmF16(0), af, bf, torch.float16, bs, share_b))
+    for g in range(G):
+        np.testing.assert_array_equal(outs[4][0][g], fast.gemm_i8(a[g], b[g].T, lit.EPI_REQUANT_RND, 0.02, 0.4))
+        bad, max_err = lit.check_err_f16(outs[4][1][g], fast.gemm_f16(af[g], bf[g].T), 1e-2, 1e-2)
+        assert bad == 0, max_err
+    np.testing.assert_array_equal(outs[4][0], outs[8][0])
+    np.testing.assert_array_equal(outs[4][1].view(np.uint16), outs[8][1].view(np.uint16))
