@@ -38,9 +38,9 @@ sys.path.insert(0, ROOT)
 PEAK = {"f16": 2516.6, "bf16": 2516.6, "i8": 5033.2}   # dense MFMA TFLOP/s / TOP/s, 256 CUs x 2.4 GHz
 HBM_PEAK_GBS = 8000.0
 # Bytes crossing the L2 <-> fabric boundary per launch, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
-# scaled by a 256 MiB copy in the same run (profiles/gemm_tile_fp16_int8_4096_hbm_traffic.md).
-MEASURED_TRAFFIC = {"fp16_gemm_4096": 2.350e8, "int8_requant_gemm_4096": 1.178e8}
-TRAFFIC_SOURCE = ("cited, not measured in this run: profiles/gemm_tile_fp16_int8_4096_hbm_traffic.md "
+# scaled by a 256 MiB copy in the same run (profiles/gemm_w4_fp16_int8_4096_hbm_traffic.md).
+MEASURED_TRAFFIC = {"fp16_gemm_4096": 2.350e8, "int8_requant_gemm_4096": 1.180e8}
+TRAFFIC_SOURCE = ("cited, not measured in this run: profiles/gemm_w4_fp16_int8_4096_hbm_traffic.md "
                   "(rocprofv3 --pmc FETCH_SIZE, then WRITE_SIZE, each scaled by a 256 MiB copy in the same run)")
 
 
