@@ -159,15 +159,15 @@ int big_tile_waves()
     return v;
 }
 // The four-wave body (one wave per SIMD, 128 x 128 wave tiles) has the faster K loop -- 18.0 against 18.9 cycles per
-// MFMA -- and, for 16-bit outputs, the faster stores (64-byte runs): measured ahead at every K for fp16 / bf16. Its int8
-// epilogues have nothing to overlap their table reads with (one wave per SIMD): behind by 0.6 us at one K tile with the
-// rounded requant, ahead from eight K tiles on.
+// MFMA -- and, for 16-bit outputs, the faster stores (64-byte runs): measured ahead or level at every K for fp16 / bf16.
+// Its int8 epilogues have nothing to overlap their table reads with (one wave per SIMD) and it does not prefetch across
+// tiles: over the audited int8 problems it is 5 - 18 % behind at 8 K tiles, 2 % at 16, 3 - 6 % ahead from 32 on.
 bool four_wave_body_pays(int dt, int K)
 {
     const int waves = big_tile_waves();
     if(waves)
         return waves == 4;
-    return dt != ckx::DT_I8 || ((long)K + 127) / 128 >= 8;
+    return dt != ckx::DT_I8 || ((long)K + 127) / 128 >= 32;
 }
 
 // CKX_KSPLIT=n forces n K runs where the problem allows it (tuning / test knob). The environment is read on the first

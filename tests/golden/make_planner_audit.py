@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Measures what the launch planner is audited against (run on the MI355X; writes planner_audit.json beside itself).
 
-    python tests/golden/make_planner_audit.py [--quick] [--out PATH]
+    python tests/golden/make_planner_audit.py [--quick] [--out PATH] [--instances 0,3 --update]
 
 For every problem of a grid (int8 requant and fp16 GEMMs, A row-major, B column-major, LLM-like and square shapes
 from 1 to 4096 rows; the ResNet-like conv layers of the benchmark) every instance that supports the problem is
@@ -67,6 +67,12 @@ def main():
                     help="comma-separated parts to measure: i8 (int8 GEMM rows), f16 (fp16 GEMM rows), conv; parts "
                          "measured in separate runs are merged by hand (same keys)")
     ap.add_argument("--out", default=None, help="where to write the table (default: planner_audit.json beside this script)")
+    ap.add_argument("--instances", default=None,
+                    help="comma-separated GEMM instance indices: time only these columns (with --update, after a kernel "
+                         "behind an instance has changed)")
+    ap.add_argument("--update", action="store_true",
+                    help="start from the table beside this script: rows are matched by their problem, the measured columns "
+                         "and the automatic choice replace the old entries, everything else is kept")
     args = ap.parse_args()
     import torch
     import composable_kernel_amd as ck
@@ -78,6 +84,13 @@ def main():
            "protocol": "per instance: graph-replayed launches in 8 ms blocks until two agree within 3 %, then the least of three more blocks, HIP events, microseconds",
            "gemm": [], "conv": []}
     n_inst = L.ckx_num_instances(capi.OP_GEMM_I8)
+    columns = None if args.instances is None else {int(x) for x in args.instances.split(",")}
+    old = None
+    if args.update:
+        with open(os.path.join(HERE, "planner_audit.json")) as f:
+            old = json.load(f)
+        out["conv"] = old["conv"]
+        out["updated"] = "columns " + (args.instances or "all") + " of the GEMM rows re-measured with this library"
     ws = torch.empty(256 << 20, dtype=torch.uint8, device="cuda")
     only = set(args.only.split(","))
     grid = [(kind, M, N, K) for kind in ("i8", "f16") if kind in only for (N, K) in GEMM_NK for M in GEMM_M]
@@ -93,7 +106,13 @@ def main():
         opf = capi.OP_GEMM_I8 if kind == "i8" else capi.OP_GEMM_F16
         epi = capi.EPI_REQUANT_RND if kind == "i8" else capi.EPI_PASSTHROUGH
         row = {"op": kind, "M": M, "N": N, "K": K, "us": {}, "k_runs": {}}
+        if old is not None:
+            prev = [r for r in old["gemm"] if (r["op"], r["M"], r["N"], r["K"]) == (kind, M, N, K)]
+            if prev:
+                row["us"], row["k_runs"] = dict(prev[0]["us"]), dict(prev[0]["k_runs"])
         for inst in range(n_inst - 1):        # (the element-wise instance is never the choice for an aligned problem)
+            if columns is not None and inst not in columns:
+                continue
             op = cls(inst)
             arg = op.MakeArgumentPointer(a, b, c, M, N, K, K, K, N, None, None, c_op)
             if not op.IsSupportedArgument(arg):
@@ -112,8 +131,12 @@ def main():
         row["auto"] = list(capi.gemm_plan(opf, M, N, K, epilogue=epi, workspace_bytes=ws.numel()))
         out["gemm"].append(row)
         print(row, flush=True)
+    if old is not None:   # rows outside this run's grid are kept as they were, in the table's order
+        done = {(r["op"], r["M"], r["N"], r["K"]): r for r in out["gemm"]}
+        out["gemm"] = [done.get((r["op"], r["M"], r["N"], r["K"]), r) for r in old["gemm"]]
     n_conv = L.ckx_num_instances(capi.OP_CONV2D_FWD_I8)
-    cgrid = [(kind, n, *layer) for kind in ("i8", "f16") for n in (32, 256) for layer in CONV] if "conv" in only else []
+    cgrid = [(kind, n, *layer) for kind in ("i8", "f16") for n in (32, 256) for layer in CONV] \
+        if "conv" in only and not args.update else []
     if args.quick:
         cgrid = cgrid[::5]
     for kind, Nb, C_, K, f, HW, st_, pd in cgrid:
