@@ -268,7 +268,9 @@ struct GemmW4
                         issue(masked, m / 4, k0, k_oob, load_stage_off);
                         __builtin_amdgcn_sched_barrier(0);
                     }
-                    mfma<m / NB == MT - 1, decltype(first)::value>(acc[m / NB][m % NB], cbf[m % NB], caf[m / NB]);
+                    // (B fragments in snake order: across a change of the A fragment the other operand stays put)
+                    constexpr int fi = m / NB, ft = (fi & 1) ? NB - 1 - m % NB : m % NB;
+                    mfma<fi == MT - 1, decltype(first)::value>(acc[fi][ft], cbf[ft], caf[fi]);
                     if constexpr(m % 3 == 2 && m / 3 < MT + NB)
                         read_one(nstage_lds, nks, std::integral_constant<int, m / 3>{}, naf, nbf);
                     if constexpr(m % 4 == 3)
