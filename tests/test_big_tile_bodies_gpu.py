@@ -208,3 +208,33 @@ def test_strided_batches_on_both_bodies(waves, case):
         assert bad == 0, max_err
     np.testing.assert_array_equal(outs[4][0], outs[8][0])
     np.testing.assert_array_equal(outs[4][1].view(np.uint16), outs[8][1].view(np.uint16))
+
+
+def test_padded_operand_strides_on_both_bodies(waves):
+    """Leading dimensions larger than K (multiples of 16 bytes) and a padded C: the rows the kernels fetch are the
+    problem's, whatever lies between them."""
+    import torch
+    import gpu_util
+    M, N, K = 520, 300, 328
+    lda, ldb, ldc = K + 8, K + 24, N + 8
+    a = np.full((M, lda), np.float16(7.0))
+    b = np.full((N, ldb), np.float16(-9.0))
+    a[:, :K] = uniform_f16((M, K), -1, 1, 3800)
+    b[:, :K] = uniform_f16((N, K), -1, 1, 3801)
+    want = fast.gemm_f16(a[:, :K], b[:, :K].T)
+    outs = []
+    for w in (4, 8):
+        waves(w)
+        da, db = gpu_util.dev(a), gpu_util.dev(b)
+        dc = torch.full((M, ldc), 77.0, dtype=torch.float16, device="cuda")
+        op = ck.DeviceGemmF16(0)
+        arg = op.MakeArgumentPointer(da, db, dc, M, N, K, lda, ldb, ldc)
+        assert op.IsSupportedArgument(arg), capi.last_error()
+        op.MakeInvokerPointer().Run(arg, ck.StreamConfig(gpu_util.stream()))
+        torch.cuda.synchronize()
+        out = dc.cpu().numpy()
+        assert np.all(out[:, N:] == 77.0)
+        outs.append(out[:, :N].copy())
+    bad, max_err = lit.check_err_f16(outs[0], want, 1e-2, 1e-2)
+    assert bad == 0, max_err
+    np.testing.assert_array_equal(outs[0].view(np.uint16), outs[1].view(np.uint16))
