@@ -1,19 +1,24 @@
 // 256 x 256 C tile computed by FOUR waves -- one per SIMD, wave tile 128 x 128 -- for dense K-contiguous GEMMs
-// (A row-major, B column-major, optionally a strided batch of them) whose tiles give every CU one round of work.
+// (A row-major, B column-major, optionally a strided batch of them), one K run.
 //
 // Same data path as gemm_tile.hpp (128-byte K tiles, direct global->LDS loads with the XOR swizzle and the B row
-// permutation applied by the choice of each lane's global chunk, D^T = B_frag x A_frag, register epilogue, 16 contiguous
-// outputs per lane), a different division of labour:
+// permutation applied by the choice of each lane's global chunk, D^T = B_frag x A_frag, register epilogue), a different
+// division of labour:
 //  * one wave per SIMD. Two waves of one SIMD do not interleave evenly: the older one runs ahead, issues its direct
 //    loads early, the younger one issues its loads late and everybody waits for those at the next barrier. With a
 //    single wave per SIMD the loads of all four waves go out at the same point of the iteration. (An instruction-mix
 //    model of both loops with real operand traffic: 19.7 cycles per MFMA with two waves per SIMD, 17.8 with one.)
+//  * nothing but MFMAs, fragment reads and loads in the K loop: a VALU instruction between the MFMAs of a SIMD's only
+//    wave costs about seven cycles of the matrix pipeline (nothing else runs meanwhile), so the loads' offsets are fixed
+//    registers and the K tile's offset travels in the scalar offset.
 //  * 128 x 128 wave tiles: 16 fragment reads per 64 MFMAs instead of 12 per 32.
-//  * the 256 accumulator registers of a lane live in AccVGPRs: the MFMAs are inline assembly with the accumulator
-//    tied ("+a"), which is what keeps the register allocator from shuffling them through VGPRs; the 128 VGPRs of the
-//    two fragment sets (register double buffer over the two k-steps of a K tile), the 16 load offsets and the
-//    addresses fit the architectural half.
-// The K loop is a loop of its own inside the loop over tiles (no prefetch across tiles): a workgroup normally has one.
+//  * the accumulators live in AccVGPRs (224 of a lane's 256; the last fragment row's in VGPRs): the MFMAs are inline
+//    assembly with the accumulator tied ("+a"), which is what keeps the register allocator from shuffling them through
+//    VGPRs; the 128 VGPRs of the two fragment sets (register double buffer over the two k-steps of a K tile), the 16
+//    load offsets and the addresses fit the architectural half.
+//  * 16-bit outputs leave in 64-byte runs per row and store instruction (row_to_col).
+// The K loop is a loop of its own inside the loop over tiles, without prefetch across tiles: a workgroup normally has
+// one tile; the eight-wave tile kernel keeps the problems whose epilogues or operand layouts this one does not have.
 #pragma once
 
 #include "gemm_tile.hpp"
