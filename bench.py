@@ -37,6 +37,7 @@ sys.path.insert(0, ROOT)
 
 PEAK = {"f16": 2516.6, "bf16": 2516.6, "i8": 5033.2}   # dense MFMA TFLOP/s / TOP/s, 256 CUs x 2.4 GHz
 HBM_PEAK_GBS = 8000.0
+PEAK_CLOCK_MHZ = 2400.0   # the engine clock the published MFMA peaks are quoted at
 # Bytes crossing the L2 <-> fabric boundary per launch, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
 # scaled by a 256 MiB copy in the same run (profiles/gemm_w4_fp16_int8_4096_hbm_traffic.md).
 MEASURED_TRAFFIC = {"fp16_gemm_4096": 2.350e8, "int8_requant_gemm_4096": 1.180e8}
@@ -256,7 +257,34 @@ def _figures(w, ev_ms):
                 bound="mfma" if compute_frac >= hbm_frac else "hbm")
 
 
-def time_workload(w, steps, warmup, instance=-1, use_graph=True, rotate=1, settle_ms=300.0, from_idle=False):
+def _sclk_under_load(chunk, chunk_ms, busy_ms=1500.0):
+    """Engine clock (MHz) read with rocm-smi while the same launches keep replaying, after the timed region: about
+    busy_ms of work is queued, the clock is read up to three times, and a reading counts only if the queue was
+    still busy after it. Empty when rocm-smi is missing, slow or prints something else."""
+    import re
+    import subprocess
+    import torch
+    done = torch.cuda.Event()
+    for _ in range(max(1, int(busy_ms / max(chunk_ms, 1e-3)))):
+        chunk()
+    done.record()
+    seen = []
+    try:
+        for _ in range(3):
+            txt = subprocess.run(["rocm-smi", "--showclocks"], capture_output=True, text=True, timeout=5).stdout
+            m = re.search(r"sclk clock level[^\n]*\((\d+)Mhz\)", txt)
+            if done.query():
+                break
+            if m:
+                seen.append(int(m.group(1)))
+    except (OSError, subprocess.SubprocessError):
+        pass
+    torch.cuda.synchronize()
+    return seen
+
+
+def time_workload(w, steps, warmup, instance=-1, use_graph=True, rotate=1, settle_ms=300.0, from_idle=False,
+                  sample_clock=False):
     """[from_idle: 1 + 10 eager launches first], clock settling, W untimed launches, then exactly K timed
     ones. The K launches are replayed from a HIP graph (captured once from the same C-ABI calls) so that
     kernels run back to back on the GPU even when one kernel is shorter than a Python call;
@@ -332,6 +360,8 @@ def time_workload(w, steps, warmup, instance=-1, use_graph=True, rotate=1, settl
     ev_ms = e0.elapsed_time(e1) / steps
     out = dict(workload=w["name"], dtype=w["dtype"], ms=ev_ms, wall_ms=wall_ms, settle_launches=settle_launches,
                settle_ms=settle_total, settle_blocks_us=[round(b * 1e3, 1) for b in blocks], **_figures(w, ev_ms))
+    if sample_clock:
+        out["sclk_mhz"] = _sclk_under_load(chunk, ev_ms * per_graph)
     if idle is not None:
         out["from_idle_ms"] = idle
     return out
@@ -456,7 +486,7 @@ def main():
         torch.cuda.synchronize()
     w = WORKLOADS[args.workload]
     r = time_workload(w, args.steps, args.warmup, args.instance, not args.no_graph, settle_ms=args.settle_ms,
-                      from_idle=True)
+                      from_idle=True, sample_clock=True)
     also = []
     extra = ["int8_requant_gemm_4096"] if args.workload == "fp16_gemm_4096" else []
     if args.all:
@@ -487,6 +517,12 @@ def main():
         roof = {"bound": "hbm", "achieved": round(r["gbs"], 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                 "frac": round(r["hbm_frac"], 4), "traffic": traffic}
     roof["traffic_source"] = TRAFFIC_SOURCE if traffic is not None else None
+    if r.get("sclk_mhz") and r["bound"] == "mfma":
+        # the published peak is the rate at 2400 MHz; with toggling operands the power limit holds the engine
+        # clock below it, whatever the instruction stream
+        mhz = sum(r["sclk_mhz"]) / len(r["sclk_mhz"])
+        roof["sclk_mhz_under_load"] = r["sclk_mhz"]
+        roof["frac_of_peak_at_that_clock"] = round(r["mfma_frac"] * PEAK_CLOCK_MHZ / mhz, 4)
     idle = _figures(w, r["from_idle_ms"])
     line = {
         "metric": "int8 TOPS & fp16 TFLOPS at 4096^3 on 1 MI355X; % of dtype MFMA peak",
