@@ -161,13 +161,14 @@ int big_tile_waves()
 // The four-wave body (one wave per SIMD, 128 x 128 wave tiles) has the faster K loop -- 18.0 against 18.9 cycles per
 // MFMA -- and, for 16-bit outputs, the faster stores (64-byte runs): measured ahead or level at every K for fp16 / bf16.
 // Its int8 epilogues have nothing to overlap their table reads with (one wave per SIMD) and it does not prefetch across
-// tiles: over the audited int8 problems it is 5 - 18 % behind at 8 K tiles, 2 % at 16, 3 - 6 % ahead from 32 on.
-bool four_wave_body_pays(int dt, int K)
+// tiles: over the audited int8 problems it is 5 - 18 % behind at 8 K tiles, 2 % at 16, 3 - 6 % ahead from 32 on with one
+// tile per CU; with several tiles per CU level at 32 (4096 x 11008 x 4096: 1 % behind), level at 48, 1 - 3 % ahead at 64.
+bool four_wave_body_pays(int dt, int K, long tiles)
 {
     const int waves = big_tile_waves();
     if(waves)
         return waves == 4;
-    return dt != ckx::DT_I8 || ((long)K + 127) / 128 >= 32;
+    return dt != ckx::DT_I8 || ((long)K + 127) / 128 >= (tiles > num_cus() ? 48 : 32);
 }
 
 // CKX_KSPLIT=n forces n K runs where the problem allows it (tuning / test knob). The environment is read on the first
@@ -636,7 +637,7 @@ int run_gemm(int dt, const void* a, const void* b, void* c, int M, int N, int K,
     const bool fused            = f16_fused(epi) && g.ksplit == 1; // (after a K split the second pass applies it)
     // (the functors with a second D tensor stay on the eight-wave body: see the fused epilogue of gemm_w4.hpp)
     const bool w4 = ti == 0 && !kmajor && g.ksplit == 1 &&
-                    (epi <= CKX_EPI_REQUANT_RND || (f16_fused(epi) && !uses_d1(epi))) && four_wave_body_pays(dt, K);
+                    (epi <= CKX_EPI_REQUANT_RND || (f16_fused(epi) && !uses_d1(epi))) && four_wave_body_pays(dt, K, (long)g.tiles_m * g.tiles_n * (batch > 1 ? batch : 1));
     const tile_launch_fn launch = w4                   ? ckx::w4_tile(dt, fused)
                                   : kmajor             ? ckx::layout_tile(dt, ti, ta, tb)
                                   : dt == ckx::DT_I8   ? (per_column_scale(epi) && g.ksplit == 1 ? t.dense_i8_fused : t.dense_i8)
