@@ -238,3 +238,45 @@ def test_padded_operand_strides_on_both_bodies(waves):
     bad, max_err = lit.check_err_f16(outs[0], want, 1e-2, 1e-2)
     assert bad == 0, max_err
     np.testing.assert_array_equal(outs[0].view(np.uint16), outs[1].view(np.uint16))
+
+
+@pytest.mark.parametrize("seed", range(24))
+def test_seeded_random_problems_on_the_four_wave_body(waves, seed):
+    """Random extents, K tails of every 16-byte multiple, padded leading dimensions and C rows, forced onto the four-wave
+    body: int8 (rounded requant) bit-exact against the oracle, fp16 on small integers bit-exact
+    against the exact product (every partial sum is an integer below 2^24)."""
+    import torch
+    import gpu_util
+    rng = np.random.default_rng(4100 + seed)
+    M, N = int(rng.integers(1, 1100)), int(rng.integers(1, 1100))
+    if seed % 6 == 0:
+        M = int(rng.integers(2200, 4200))            # more tiles than the workgroups of a launch now and then
+    waves(4)
+    if seed % 2 == 0:
+        K = 16 * int(rng.integers(1, 160))
+        lda, ldb, ldc = K + 16 * int(rng.integers(0, 3)), K + 16 * int(rng.integers(0, 3)), N + int(rng.integers(0, 20))
+        a = rng.integers(-15, 16, (M, lda), dtype=np.int8)
+        b = rng.integers(-15, 16, (N, ldb), dtype=np.int8)
+        sg, sr = 0.02, 0.75
+        da, db = gpu_util.dev(a), gpu_util.dev(b)
+        dc = torch.full((M, ldc), 77, dtype=torch.int8, device="cuda")
+        op = ck.DeviceGemmInt8(0)
+        arg = op.MakeArgumentPointer(da, db, dc, M, N, K, lda, ldb, ldc, ck.PassThrough(), ck.PassThrough(),
+                                     ck.RequantReluRequant(sg, sr, rounded=True))
+        want = fast.gemm_i8(a[:, :K], b[:, :K].T, lit.EPI_REQUANT_RND, sg, sr)
+    else:
+        K = 8 * int(rng.integers(1, 200))
+        lda, ldb, ldc = K + 8 * int(rng.integers(0, 3)), K + 8 * int(rng.integers(0, 3)), N + int(rng.integers(0, 20))
+        a = rng.integers(-4, 5, (M, lda)).astype(np.float16)
+        b = rng.integers(-4, 5, (N, ldb)).astype(np.float16)
+        da, db = gpu_util.dev(a), gpu_util.dev(b)
+        dc = torch.full((M, ldc), 77.0, dtype=torch.float16, device="cuda")
+        op = ck.DeviceGemmF16(0)
+        arg = op.MakeArgumentPointer(da, db, dc, M, N, K, lda, ldb, ldc)
+        want = (a[:, :K].astype(np.int64) @ b[:, :K].astype(np.int64).T).astype(np.float32).astype(np.float16)
+    assert op.IsSupportedArgument(arg), capi.last_error()
+    op.MakeInvokerPointer().Run(arg, ck.StreamConfig(gpu_util.stream()))
+    torch.cuda.synchronize()
+    out = dc.cpu().numpy()
+    assert np.all(out[:, N:] == 77), "wrote outside the C rows"
+    np.testing.assert_array_equal(out[:, :N], want)
