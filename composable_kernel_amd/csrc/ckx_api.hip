@@ -636,7 +636,8 @@ int run_gemm(int dt, const void* a, const void* b, void* c, int M, int N, int K,
     g.ws         = ws;
     const bool fused            = f16_fused(epi) && g.ksplit == 1; // (after a K split the second pass applies it)
     // (the functors with a second D tensor stay on the eight-wave body: see the fused epilogue of gemm_w4.hpp)
-    const bool w4 = ti == 0 && !kmajor && g.ksplit == 1 &&
+    // (its buffer resources start 3 KB before the operands and are that much longer: see kImmBias in gemm_w4.hpp)
+    const bool w4 = ti == 0 && !kmajor && g.ksplit == 1 && g.a_bytes < (1u << 31) - 4096 && g.b_bytes < (1u << 31) - 4096 &&
                     (epi <= CKX_EPI_REQUANT_RND || (f16_fused(epi) && !uses_d1(epi))) && four_wave_body_pays(dt, K, (long)g.tiles_m * g.tiles_n * (batch > 1 ? batch : 1));
     const tile_launch_fn launch = w4                   ? ckx::w4_tile(dt, fused)
                                   : kmajor             ? ckx::layout_tile(dt, ti, ta, tb)

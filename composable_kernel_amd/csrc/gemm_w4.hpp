@@ -39,23 +39,81 @@ struct GemmW4
     static constexpr int MT = 8, NB = 8;  // A fragments (16 rows each) and B fragments (16 columns each) of a wave per k-step
     static constexpr int NLA = 8, NLB = 8, LPT = NLA + NLB; // 16-byte direct loads per thread and K tile
     static constexpr int NMH = MT * NB;   // MFMAs per half-iteration (one k-step)
+    // LDS: [A stage 0 | A stage 1 | B stage 0 | B stage 1 | requant table]. Both stages of an operand lie within the
+    // 16-bit offset field of a fragment read, so a lane's four read addresses (A / B x k-step) serve both stages.
+    static constexpr int A_AT(int st) { return st * A_TILE; }
+    static constexpr int B_AT(int st) { return NST * A_TILE + st * B_TILE; }
+    // A direct load's immediate offset moves its LDS address AND its global address. A wave's eight load slots of an
+    // operand are 1 KB apart in LDS, so one M0 value serves four loads (immediates 0 .. 3 KB); the per-lane global
+    // offsets carry kImmBias minus the immediate, and the buffer resources start kImmBias bytes before the operands.
+    static constexpr int kImmBias = 3072;
+    // M0 for load slot SLOT (and the three after it) of stage ST, relative to the wave's first slot in A stage 0; a
+    // stage that is only known at run time (ST < 0) is added to the base register instead (A_TILE == B_TILE)
+    static constexpr int m0_add(int slot, int st)
+    {
+        return (slot < NLA ? A_AT(st < 0 ? 0 : st) : B_AT(st < 0 ? 0 : st)) + ((slot % NLA) / 4) * 4096;
+    }
+    template <typename ST>
+    static constexpr int stage_ct(ST)
+    {
+        if constexpr(std::is_same<ST, int>::value)
+            return -1;
+        else
+            return ST::value;
+    }
+    template <typename ST>
+    __device__ static __forceinline__ uint32_t stage_rt(ST st)
+    {
+        if constexpr(std::is_same<ST, int>::value)
+            return (uint32_t)st * A_TILE;
+        else
+            return 0u;
+    }
+    // SPREAD: the B half of the K tile after next is requested during the FIRST half of an iteration (behind a
+    // second barrier, once every wave has the current tile's B fragments of k-step 1), the A half during the second:
+    // the CU's address unit sees eight loads per wave and half instead of sixteen in one.
+#ifndef CKX_W4_SPREAD
+#define CKX_W4_SPREAD 2
+#endif
+    static constexpr bool SPREAD = CKX_W4_SPREAD != 0;
+    // first half of a SPREAD iteration: a B read behind every H0_RB-th MFMA, wait + barrier behind MFMA H0_BAR, B loads
+    // behind MFMAs H0_L0 + i * H0_LS, A reads behind MFMAs H0_RA0 + i * H0_RAS
+    static constexpr int H0_RB  = CKX_W4_SPREAD == 2 ? 1 : 2;
+    static constexpr int H0_BAR = CKX_W4_SPREAD == 2 ? 13 : 23;
+    static constexpr int H0_L0 = H0_BAR + 1, H0_LS = CKX_W4_SPREAD == 2 ? 6 : 5;
+    static constexpr int H0_RA0 = H0_BAR + 3, H0_RAS = CKX_W4_SPREAD == 2 ? 5 : 4;
+    static_assert(H0_L0 + (NLB - 1) * H0_LS < MT * NB && H0_RA0 + (MT - 1) * H0_RAS < MT * NB - 4 && NB * H0_RB <= H0_BAR, "");
     using acc_t = typename std::conditional<DT == DT_I8, i32x4, f32x4>::type;
 
     // (the accumulators of the last fragment row stay in VGPRs: with all 256 AccVGPRs tied the allocator has no
     // register left to move one through and spills)
     // FIRST: the accumulator starts at zero (the literal 0 as the addend) instead of being read -- the first k-step of
     // a tile, which saves zeroing 256 registers per lane beforehand
-    template <bool IN_VGPR, bool FIRST>
-    __device__ static __forceinline__ void mfma(acc_t& c, const i32x4& b, const i32x4& a)
+    // M0ADD >= 0: the statement first writes M0 = m0_base + M0ADD for the direct loads that follow it (the MFMA is the
+    // instruction the hazard wants between an M0 write and the load that uses it; as statements of their own the
+    // compiler puts an s_nop in front of every such write).
+    template <bool IN_VGPR, bool FIRST, int M0ADD = -1>
+    __device__ static __forceinline__ void mfma(acc_t& c, const i32x4& b, const i32x4& a, uint32_t m0_base = 0)
     {
-#define CKX_W4_MFMA(OP)                                                                        \
-    if constexpr(IN_VGPR && FIRST)                                                             \
-        asm volatile(OP " %0, %1, %2, 0" : "=v"(c) : "v"(b), "v"(a));                          \
-    else if constexpr(IN_VGPR)                                                                 \
-        asm volatile(OP " %0, %1, %2, %0" : "+v"(c) : "v"(b), "v"(a));                         \
-    else if constexpr(FIRST)                                                                   \
-        asm volatile(OP " %0, %1, %2, 0" : "=a"(c) : "v"(b), "v"(a));                          \
-    else                                                                                       \
+#define CKX_W4_MFMA(OP)                                                                                           \
+    if constexpr(M0ADD >= 0)                                                                                      \
+    {                                                                                                             \
+        if constexpr(IN_VGPR && FIRST)                                                                            \
+            asm volatile("s_add_u32 m0, %3, %4\n\t" OP " %0, %1, %2, 0" : "=v"(c) : "v"(b), "v"(a), "s"(m0_base), "n"(M0ADD) : "scc"); \
+        else if constexpr(IN_VGPR)                                                                                \
+            asm volatile("s_add_u32 m0, %3, %4\n\t" OP " %0, %1, %2, %0" : "+v"(c) : "v"(b), "v"(a), "s"(m0_base), "n"(M0ADD) : "scc"); \
+        else if constexpr(FIRST)                                                                                  \
+            asm volatile("s_add_u32 m0, %3, %4\n\t" OP " %0, %1, %2, 0" : "=a"(c) : "v"(b), "v"(a), "s"(m0_base), "n"(M0ADD) : "scc"); \
+        else                                                                                                      \
+            asm volatile("s_add_u32 m0, %3, %4\n\t" OP " %0, %1, %2, %0" : "+a"(c) : "v"(b), "v"(a), "s"(m0_base), "n"(M0ADD) : "scc"); \
+    }                                                                                                             \
+    else if constexpr(IN_VGPR && FIRST)                                                                           \
+        asm volatile(OP " %0, %1, %2, 0" : "=v"(c) : "v"(b), "v"(a));                                             \
+    else if constexpr(IN_VGPR)                                                                                    \
+        asm volatile(OP " %0, %1, %2, %0" : "+v"(c) : "v"(b), "v"(a));                                            \
+    else if constexpr(FIRST)                                                                                      \
+        asm volatile(OP " %0, %1, %2, 0" : "=a"(c) : "v"(b), "v"(a));                                             \
+    else                                                                                                          \
         asm volatile(OP " %0, %1, %2, %0" : "+a"(c) : "v"(b), "v"(a));
         if constexpr(DT == DT_I8)
         {
@@ -172,25 +230,29 @@ struct GemmW4
         const int nk_real     = (int)((kbytes + BKB - 1) / BKB);
         const int nk          = nk_real > 0 ? nk_real : 1;
 
-        const __amdgpu_buffer_rsrc_t rsrc_a = make_rsrc(p.a, p.a_bytes);
-        const __amdgpu_buffer_rsrc_t rsrc_b = make_rsrc(p.b, p.b_bytes);
-        const uint32_t smem_lds             = (uint32_t)(uintptr_t)(lds_ptr_t)smem;
+        const __amdgpu_buffer_rsrc_t rsrc_a =
+            make_rsrc(reinterpret_cast<const uint8_t*>(p.a) - kImmBias, p.a_bytes + (uint32_t)kImmBias);
+        const __amdgpu_buffer_rsrc_t rsrc_b =
+            make_rsrc(reinterpret_cast<const uint8_t*>(p.b) - kImmBias, p.b_bytes + (uint32_t)kImmBias);
+        const uint32_t smem_lds = (uint32_t)(uintptr_t)(lds_ptr_t)smem;
         if constexpr(DT == DT_I8)
         {
             if(p.epi == EPI_REQUANT_RND) // (visible to every wave after the first barrier of the K loop)
                 requant_lut_fill(smem + NST * STAGE, p.scale_relu, tid, NT);
         }
 
-        // slot j of a thread fills LDS row (j * NW + wave) * 8 + lane / 8, chunk position lane % 8 of the A (B) tile
-        // with chunk (lane % 8) ^ (row & 7) of that row
+        // slot j of a wave fills LDS rows (wave * 8 + j) * 8 + lane / 8 of the A (B) tile, chunk position lane % 8 with
+        // chunk (lane % 8) ^ (row & 7) of that row
         const uint32_t kb = ((uint32_t)(lane & 7) ^ (uint32_t)((lane >> 3) & 7)) << 4;
-        // fragment addresses relative to a stage: row = wave rows + 16 * fragment + lane % 16, chunk 4 * ks + lane / 16
+        // LDS address of the wave's first load slot in A stage 0 (a scalar: M0 is this plus a constant)
+        const uint32_t m0_base = smem_lds + (uint32_t)wave * (NLA * 1024);
+        // fragment addresses: row = wave rows + 16 * fragment + lane % 16, chunk 4 * ks + lane / 16
         const uint32_t frow = (uint32_t)(lane & 15), fq = (uint32_t)(lane >> 4);
         auto frag_part      = [&](int row0, int ks) {
             return (uint32_t)(row0 + (int)frow) * BKB + ((((uint32_t)ks * 4 + fq) ^ (frow & 7u)) << 4);
         };
-        const uint32_t fa[2] = {frag_part(wm * 128, 0), frag_part(wm * 128, 1)};
-        const uint32_t fb[2] = {A_TILE + frag_part(wn * 128, 0), A_TILE + frag_part(wn * 128, 1)};
+        const uint32_t fa[2] = {smem_lds + frag_part(wm * 128, 0), smem_lds + frag_part(wm * 128, 1)};
+        const uint32_t fb[2] = {smem_lds + B_AT(0) + frag_part(wn * 128, 0), smem_lds + B_AT(0) + frag_part(wn * 128, 1)};
 
         const bool vec_ok = ((reinterpret_cast<uintptr_t>(p.c) | ((uintptr_t)p.ldc * ES) |
                               (nbatch > 1 ? (uintptr_t)p.bsc * ES : 0)) & 15u) == 0;
@@ -206,27 +268,29 @@ struct GemmW4
 #pragma unroll
             for(int j = 0; j < NLA; ++j)
             {
-                const uint32_t r  = (uint32_t)((j * NW + wave) * 8 + (lane >> 3));
-                const uint32_t gm = (uint32_t)tm * BM + r;
-                const uint32_t gn = (uint32_t)tn * BN + row_to_col(r);
-                a_off[j]          = gm < (uint32_t)p.M ? a_batch + gm * (uint32_t)p.lda * ES + kb : kOutOfRange;
-                b_off[j]          = gn < (uint32_t)p.N ? b_batch + gn * (uint32_t)p.ldb * ES + kb : kOutOfRange;
+                const uint32_t r    = (uint32_t)((wave * NLA + j) * 8 + (lane >> 3));
+                const uint32_t gm   = (uint32_t)tm * BM + r;
+                const uint32_t gn   = (uint32_t)tn * BN + row_to_col(r);
+                const uint32_t bias = kb + (uint32_t)(kImmBias - (j & 3) * 1024);
+                a_off[j]            = gm < (uint32_t)p.M ? a_batch + gm * (uint32_t)p.lda * ES + bias : kOutOfRange;
+                b_off[j]            = gn < (uint32_t)p.N ? b_batch + gn * (uint32_t)p.ldb * ES + bias : kOutOfRange;
             }
-            // One direct load: slot < NLA an A row group, else a B row group, of the K tile at byte offset k0 into the
-            // stage at stage_off. k0 travels in the instruction's scalar offset, which the address uses and the range check
-            // does not: the per-lane offset alone decides between the row (in range) and zeros (row past M / N: top bit).
-            // MASKED adds the top bit for chunks past K and K tiles past the end -- two VALU instructions per load that
-            // the K tiles in the middle of the loop do without (a VALU instruction between the MFMAs of a SIMD's only
-            // wave costs about seven cycles of the matrix pipeline).
-            auto issue = [&](auto masked, int slot, uint32_t k0, uint32_t k_oob, uint32_t stage_off) {
-                constexpr bool MASKED = decltype(masked)::value;
-                if(slot < NLA)
-                    __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_a, (lds_ptr_t)(smem + stage_off + (slot * NW + wave) * 1024),
-                                                             16, MASKED ? (a_off[slot] | k_oob) : a_off[slot], (int)k0, 0, 0);
-                else
-                    __builtin_amdgcn_raw_ptr_buffer_load_lds(
-                        rsrc_b, (lds_ptr_t)(smem + stage_off + A_TILE + ((slot - NLA) * NW + wave) * 1024), 16,
-                        MASKED ? (b_off[slot - NLA] | k_oob) : b_off[slot - NLA], (int)k0, 0, 0);
+            // One direct load, as inline assembly (the compiler's form writes M0 and a hazard nop before every load):
+            // slot < NLA an A row group, else a B row group, of the K tile at byte offset k0, into the stage M0 points
+            // into: M0 = m0_of(stage) + m0_add(slot) serves four consecutive slots, and is written by the statement of
+            // the MFMA in front of the first of them (or, in the prologue, by a statement of its own). k0 travels in the
+            // scalar offset, which the address uses and the range check does not: the per-lane offset alone decides
+            // between the row (in range) and zeros (row past M / N: top bit). MASKED adds the top bit for chunks past K
+            // and K tiles past the end -- a VALU instruction per load that the K tiles in the middle of the loop do
+            // without (a VALU instruction between the MFMAs of a SIMD's only wave costs about seven cycles of the matrix
+            // pipeline).
+            auto load_slot = [&](auto slot_c, auto masked, uint32_t k0, uint32_t k_oob) {
+                constexpr int SLOT = decltype(slot_c)::value, J = SLOT % NLA;
+                const uint32_t off  = SLOT < NLA ? a_off[J] : b_off[J];
+                const uint32_t voff = decltype(masked)::value ? (off | k_oob) : off;
+                const __amdgpu_buffer_rsrc_t rsrc = SLOT < NLA ? rsrc_a : rsrc_b;
+                asm volatile("buffer_load_dwordx4 %0, %1, %2 offen offset:%3 lds" ::"v"(voff), "s"(rsrc), "s"(k0),
+                             "n"((J % 4) * 1024));
             };
             auto k_oob_of = [&](int kt) { return ((uint32_t)kt * BKB + kb < kbytes && kt < nk) ? 0u : kOutOfRange; };
 
@@ -237,76 +301,128 @@ struct GemmW4
             // ordered against loads: drained here, so that the counted wait below sees loads only.
             asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
             __builtin_amdgcn_s_barrier();
-#pragma unroll
-            for(int st = 0; st < NST; ++st)
-            {
-                const uint32_t oob = k_oob_of(st);
-#pragma unroll
-                for(int s = 0; s < LPT; ++s)
-                    issue(std::true_type{}, s, (uint32_t)st * BKB, oob, (uint32_t)(st * STAGE));
-            }
+            static_for<NST>([&](auto st_c) {
+                const uint32_t oob = k_oob_of(decltype(st_c)::value);
+                static_for<LPT>([&](auto s_c) {
+                    if constexpr(decltype(s_c)::value % 4 == 0) // (one instruction between an M0 write and its load)
+                        asm volatile("s_add_u32 m0, %0, %1\n\ts_nop 0" ::"s"(m0_base),
+                                     "n"(m0_add(decltype(s_c)::value, decltype(st_c)::value))
+                                     : "scc");
+                    load_slot(s_c, std::true_type{}, (uint32_t)decltype(st_c)::value * BKB, oob);
+                });
+            });
             asm volatile("s_waitcnt vmcnt(%0)" ::"n"(LPT) : "memory");
             __builtin_amdgcn_s_barrier();
             asm volatile("" ::: "memory");
 
             i32x4 af0[MT], bf0[NB], af1[MT], bf1[NB];
-            // fragment r of k-step ks of the stage at LDS address stage_lds: the B fragments first, then the A fragments
-            auto read_one = [&](uint32_t stage_lds, auto ks_c, auto r_c, i32x4(&af)[MT], i32x4(&bf)[NB]) {
+            // fragment r of k-step KS of stage ST: the B fragments first, then the A fragments
+            auto read_one = [&](auto st, auto ks_c, auto r_c, i32x4(&af)[MT], i32x4(&bf)[NB]) {
                 constexpr int KS = decltype(ks_c)::value, R = decltype(r_c)::value;
-                if constexpr(R < NB)
-                    bf[R] = lds_read_b128<R * 16 * BKB>(stage_lds + fb[KS]);
+                if constexpr(std::is_same<decltype(st), int>::value)
+                {
+                    if constexpr(R < NB)
+                        bf[R] = lds_read_b128<R * 16 * BKB>(fb[KS] + (uint32_t)st * B_TILE);
+                    else
+                        af[R - NB] = lds_read_b128<(R - NB) * 16 * BKB>(fa[KS] + (uint32_t)st * A_TILE);
+                }
                 else
-                    af[R - NB] = lds_read_b128<(R - NB) * 16 * BKB>(stage_lds + fa[KS]);
+                {
+                    constexpr int ST = decltype(st)::value;
+                    if constexpr(R < NB)
+                        bf[R] = lds_read_b128<B_AT(ST) - B_AT(0) + R * 16 * BKB>(fb[KS]);
+                    else
+                        af[R - NB] = lds_read_b128<A_AT(ST) + (R - NB) * 16 * BKB>(fa[KS]);
+                }
             };
-            static_for<MT + NB>([&](auto r_c) { read_one(smem_lds, std::integral_constant<int, 0>{}, r_c, af0, bf0); });
+            static_for<MT + NB>([&](auto r_c) {
+                read_one(std::integral_constant<int, 0>{}, std::integral_constant<int, 0>{}, r_c, af0, bf0);
+            });
 
-            // One half of an iteration: the 64 MFMAs of one k-step; behind every third MFMA one fragment read of the next
-            // k-step (16 reads, done after three quarters of the half); with_loads: behind every fourth MFMA one direct
-            // load of the K tile after next into the stage whose fragments are all in registers.
-            auto half_step = [&](auto first, auto with_loads, auto masked, uint32_t k0, uint32_t k_oob, uint32_t load_stage_off,
-                                 const i32x4(&caf)[MT], const i32x4(&cbf)[NB], uint32_t nstage_lds, auto nks,
-                                 i32x4(&naf)[MT], i32x4(&nbf)[NB]) {
+            // One half of an iteration: the 64 MFMAs of one k-step on the fragments (caf, cbf); the 16 fragment reads of
+            // the next k-step (k-step NKS of stage NST_) into (naf, nbf); direct loads of the K tile after next into
+            // stage LST, whose fragments (of the operand being loaded) are all in registers by then.
+            //   plain: no loads in the first half; all 16 in the second, one behind every fourth MFMA; reads behind
+            //          every third MFMA (done after three quarters of the half);
+            //   SPREAD, first half: the B reads behind every second MFMA, wait + barrier behind MFMA 23, then the eight B
+            //          loads (one per five MFMAs) and the A reads; second half: the eight A loads, one per eight MFMAs.
+            auto half_step = [&](auto first, auto second_half, auto masked, uint32_t k0, uint32_t k_oob, auto lst_c,
+                                 const i32x4(&caf)[MT], const i32x4(&cbf)[NB], auto nst_c, auto nks, i32x4(&naf)[MT],
+                                 i32x4(&nbf)[NB]) {
+                constexpr bool H1 = decltype(second_half)::value;
                 static_for<NMH>([&](auto m_c) {
                     constexpr int m = decltype(m_c)::value;
-                    if constexpr(decltype(with_loads)::value && m % 4 == 0)
-                    {
-                        issue(masked, m / 4, k0, k_oob, load_stage_off);
-                        __builtin_amdgcn_sched_barrier(0);
-                    }
                     // (B fragments in snake order: across a change of the A fragment the other operand stays put)
                     constexpr int fi = m / NB, ft = (fi & 1) ? NB - 1 - m % NB : m % NB;
-                    mfma<fi == MT - 1, decltype(first)::value>(acc[fi][ft], cbf[ft], caf[fi]);
-                    if constexpr(m % 3 == 2 && m / 3 < MT + NB)
-                        read_one(nstage_lds, nks, std::integral_constant<int, m / 3>{}, naf, nbf);
+                    // which load slot, if any, goes out behind this MFMA
+                    constexpr int slot = !SPREAD ? ((H1 && m % 4 == 0) ? m / 4 : -1)
+                                         : H1    ? (m % 8 == 0 ? m / 8 : -1)
+                                                 : ((m >= H0_L0 && (m - H0_L0) % H0_LS == 0 && (m - H0_L0) / H0_LS < NLB)
+                                                        ? NLA + (m - H0_L0) / H0_LS
+                                                        : -1);
+                    constexpr int LST = stage_ct(decltype(lst_c){});
+                    if constexpr(slot >= 0 && slot % 4 == 0)
+                        mfma<fi == MT - 1, decltype(first)::value, m0_add(slot < 0 ? 0 : slot, LST)>(acc[fi][ft], cbf[ft], caf[fi],
+                                                                                                m0_base + stage_rt(lst_c));
+                    else
+                        mfma<fi == MT - 1, decltype(first)::value>(acc[fi][ft], cbf[ft], caf[fi]);
+                    if constexpr(slot >= 0)
+                        load_slot(std::integral_constant<int, (slot < 0 ? 0 : slot)>{}, masked, k0, k_oob);
+                    // which fragment read, if any, follows it
+                    constexpr int rd = (!SPREAD || H1) ? ((m % 3 == 2 && m / 3 < MT + NB) ? m / 3 : -1)
+                                       : m < NB * H0_RB ? ((m % H0_RB == H0_RB - 1) ? m / H0_RB : -1)
+                                                        : ((m >= H0_RA0 && (m - H0_RA0) % H0_RAS == 0 && (m - H0_RA0) / H0_RAS < MT)
+                                                               ? NB + (m - H0_RA0) / H0_RAS
+                                                               : -1);
+                    if constexpr(rd >= 0)
+                        read_one(nst_c, nks, std::integral_constant<int, rd>{}, naf, nbf);
+                    if constexpr(SPREAD && !H1 && m == H0_BAR)
+                    {
+                        // every wave holds the B fragments of both k-steps of this K tile: its B stage may be refilled
+                        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+                        __builtin_amdgcn_s_barrier();
+                        asm volatile("" ::: "memory");
+                    }
                     if constexpr(m % 4 == 3)
                         __builtin_amdgcn_sched_barrier(0);
                 });
             };
 
-            int st_cur = 0;
-            auto iteration = [&](auto first, auto masked, int kt) {
+            // K tile kt, staged in stage ST: k-step 0 out of (af0, bf0) while k-step 1 is read, then k-step 1 while
+            // k-step 0 of K tile kt + 1 (stage ST ^ 1) is read and K tile kt + 2 is requested into stage ST.
+            auto iteration = [&](auto st, auto other, auto first, auto masked, int kt) {
+                const uint32_t k0 = (uint32_t)(kt + 2) * BKB, k_oob = decltype(masked)::value ? k_oob_of(kt + 2) : 0u;
                 asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
                 __builtin_amdgcn_sched_barrier(0);
-                half_step(first, std::false_type{}, masked, 0u, 0u, 0u, af0, bf0, smem_lds + (uint32_t)(st_cur * STAGE),
-                          std::integral_constant<int, 1>{}, af1, bf1);
-                // K tile kt is in registers, K tile kt + 1 has landed (the loads of a wave retire in order)
-                asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+                half_step(first, std::false_type{}, masked, k0, k_oob, st, af0, bf0, st, std::integral_constant<int, 1>{},
+                          af1, bf1);
+                // K tile kt is in registers, K tile kt + 1 has landed (the loads of a wave retire in order; with SPREAD
+                // the B half of K tile kt + 2 may still be on its way)
+                if constexpr(SPREAD)
+                    asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" ::"n"(NLB) : "memory");
+                else
+                    asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
                 __builtin_amdgcn_sched_barrier(0);
                 __builtin_amdgcn_s_barrier();
                 asm volatile("" ::: "memory");
-                half_step(std::false_type{}, std::true_type{}, masked, (uint32_t)(kt + 2) * BKB,
-                          decltype(masked)::value ? k_oob_of(kt + 2) : 0u, (uint32_t)(st_cur * STAGE), af1, bf1,
-                          smem_lds + (uint32_t)((st_cur ^ 1) * STAGE), std::integral_constant<int, 0>{}, af0, bf0);
-                st_cur ^= 1;
+                half_step(std::false_type{}, std::true_type{}, masked, k0, k_oob, st, af1, bf1, other,
+                          std::integral_constant<int, 0>{}, af0, bf0);
             };
-            // iterations whose loads fetch a whole K tile, then the (at most three) whose loads need the mask
+            using st0 = std::integral_constant<int, 0>;
+            using st1 = std::integral_constant<int, 1>;
+            // K tile 0, then pairs of iterations whose loads fetch a whole K tile (two copies of the loop body: the
+            // stage is a compile-time constant of every address), then the (at most four) whose loads need the mask, with the
+            // stage as a scalar
             const int nk_whole = (int)(kbytes / BKB);
-            iteration(std::true_type{}, std::true_type{}, 0);
+            iteration(st0{}, st1{}, std::true_type{}, std::true_type{}, 0);
             int kt = 1;
-            for(; kt + 2 < nk_whole; ++kt)
-                iteration(std::false_type{}, std::false_type{}, kt);
+            for(; kt + 3 < nk_whole; kt += 2)
+            {
+                iteration(st1{}, st0{}, std::false_type{}, std::false_type{}, kt);
+                iteration(st0{}, st1{}, std::false_type{}, std::false_type{}, kt + 1);
+            }
             for(; kt < nk; ++kt)
-                iteration(std::false_type{}, std::true_type{}, kt);
+                iteration(kt & 1, (kt & 1) ^ 1, std::false_type{}, std::true_type{}, kt);
             // the trailing fragment reads and (all-zero) loads; the MFMA results must have left the pipeline before the
             // epilogue reads them (inline-assembly MFMAs are invisible to the compiler's hazard handling)
             asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_nop 15\n\ts_nop 15" ::: "memory");
