@@ -168,6 +168,9 @@ bool four_wave_body_pays(int dt, int K, long tiles)
     const int waves = big_tile_waves();
     if(waves)
         return waves == 4;
+    // (a single K tile: the four-wave body's plain epilogues run inside a last K tile of their own, all zeros here)
+    if((long)K * (dt == ckx::DT_I8 ? 1 : 2) <= 128)
+        return false;
     return dt != ckx::DT_I8 || ((long)K + 127) / 128 >= (tiles > num_cus() ? 48 : 32);
 }
 

@@ -7,11 +7,11 @@
 namespace ckx {
 namespace {
 
-template <int DT, bool FUSED = false>
+template <int DT, bool FUSED = false, int EPI = EPI_PASSTHROUGH>
 hipError_t launch_w4(const GemmArgs& a, int tiles, hipStream_t s)
 {
-    using T    = GemmW4<DT, FUSED>;
-    auto* kern = &gemm_w4_kernel<DT, FUSED>;
+    using T    = GemmW4<DT, FUSED, EPI>;
+    auto* kern = &gemm_w4_kernel<DT, FUSED, EPI>;
     static std::once_flag once;
     static hipError_t attr_err = hipSuccess;
     std::call_once(once, [&] {
@@ -28,13 +28,21 @@ hipError_t launch_w4(const GemmArgs& a, int tiles, hipStream_t s)
     return hipGetLastError();
 }
 
+// int8: one kernel per plain epilogue (the requant form is a compile-time constant of the kernel)
+hipError_t launch_w4_i8(const GemmArgs& a, int tiles, hipStream_t s)
+{
+    return a.epi == EPI_REQUANT_RND  ? launch_w4<DT_I8, false, EPI_REQUANT_RND>(a, tiles, s)
+           : a.epi == EPI_REQUANT_CK ? launch_w4<DT_I8, false, EPI_REQUANT_CK>(a, tiles, s)
+                                     : launch_w4<DT_I8, false, EPI_PASSTHROUGH>(a, tiles, s);
+}
+
 } // namespace
 
 tile_launch_fn w4_tile(int dt, bool fused)
 {
     if(fused)
         return dt == DT_F16 ? &launch_w4<DT_F16, true> : nullptr;
-    return dt == DT_I8 ? &launch_w4<DT_I8> : dt == DT_BF16 ? &launch_w4<DT_BF16> : &launch_w4<DT_F16>;
+    return dt == DT_I8 ? &launch_w4_i8 : dt == DT_BF16 ? &launch_w4<DT_BF16> : &launch_w4<DT_F16>;
 }
 
 } // namespace ckx

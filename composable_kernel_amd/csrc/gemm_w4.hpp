@@ -27,10 +27,13 @@ namespace ckx {
 
 // FUSED (fp16): the epilogues with D operands (add / ReLU functors, Bilinear, AddAddFastGelu) as a kernel of their own,
 // like the FUSED variants of the tile kernel.
-template <int DT, bool FUSED = false>
+// EPI (int8, plain epilogues): the requant form as a compile-time constant, so that the last K tile's loop, which stores
+// finished fragment rows between its MFMAs, carries no branch on it.
+template <int DT, bool FUSED = false, int EPI = EPI_PASSTHROUGH>
 struct GemmW4
 {
     static_assert(!FUSED || DT == DT_F16, "D-operand epilogues: fp16");
+    static_assert(EPI == EPI_PASSTHROUGH || (DT == DT_I8 && (EPI == EPI_REQUANT_CK || EPI == EPI_REQUANT_RND)), "");
     static constexpr int BM = 256, BN = 256, BKB = 128, NW = 4, NT = NW * 64, NST = 2;
     static constexpr int ES     = DT == DT_I8 ? 1 : 2;
     static constexpr int A_TILE = BM * BKB, B_TILE = BN * BKB, STAGE = A_TILE + B_TILE;
@@ -228,18 +231,17 @@ struct GemmW4
         const int ntiles      = p.tiles_m * p.tiles_n * nbatch; // C tiles of all batches, dealt to the XCDs batch by batch
         const uint32_t kbytes = (uint32_t)p.K * ES;
         const int nk_real     = (int)((kbytes + BKB - 1) / BKB);
-        const int nk          = nk_real > 0 ? nk_real : 1;
+        // (the plain epilogues run inside an iteration of their own, the last one: at least two K tiles, the second one
+        // all zeros if need be)
+        const int nk = nk_real > (FUSED ? 0 : 1) ? nk_real : (FUSED ? 1 : 2);
 
         const __amdgpu_buffer_rsrc_t rsrc_a =
             make_rsrc(reinterpret_cast<const uint8_t*>(p.a) - kImmBias, p.a_bytes + (uint32_t)kImmBias);
         const __amdgpu_buffer_rsrc_t rsrc_b =
             make_rsrc(reinterpret_cast<const uint8_t*>(p.b) - kImmBias, p.b_bytes + (uint32_t)kImmBias);
         const uint32_t smem_lds = (uint32_t)(uintptr_t)(lds_ptr_t)smem;
-        if constexpr(DT == DT_I8)
-        {
-            if(p.epi == EPI_REQUANT_RND) // (visible to every wave after the first barrier of the K loop)
-                requant_lut_fill(smem + NST * STAGE, p.scale_relu, tid, NT);
-        }
+        if constexpr(DT == DT_I8 && EPI == EPI_REQUANT_RND) // (visible to every wave after the first barrier of the K loop)
+            requant_lut_fill(smem + NST * STAGE, p.scale_relu, tid, NT);
 
         // slot j of a wave fills LDS rows (wave * 8 + j) * 8 + lane / 8 of the A (B) tile, chunk position lane % 8 with
         // chunk (lane % 8) ^ (row & 7) of that row
@@ -421,15 +423,89 @@ struct GemmW4
                 iteration(st1{}, st0{}, std::false_type{}, std::false_type{}, kt);
                 iteration(st0{}, st1{}, std::false_type{}, std::false_type{}, kt + 1);
             }
-            for(; kt < nk; ++kt)
+            for(; kt < nk - (FUSED ? 0 : 1); ++kt)
                 iteration(kt & 1, (kt & 1) ^ 1, std::false_type{}, std::true_type{}, kt);
-            // the trailing fragment reads and (all-zero) loads; the MFMA results must have left the pipeline before the
-            // epilogue reads them (inline-assembly MFMAs are invisible to the compiler's hazard handling)
-            asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_nop 15\n\ts_nop 15" ::: "memory");
-            __builtin_amdgcn_sched_barrier(0);
 
             // ---- epilogue: 16 consecutive columns of one row per lane, fragment row by fragment row
             const uint32_t lut_lds = smem_lds + (uint32_t)(NST * STAGE);
+            // fragment row i through the plain epilogue; G = 0 / 1: one 64-column group of it, G < 0: both
+            using both_groups = std::integral_constant<int, -1>;
+            auto store_row = [&](auto i_c, auto g_sel) {
+                constexpr int i = decltype(i_c)::value, G = decltype(g_sel)::value;
+                const int m     = tm * BM + wm * 128 + 16 * i + (lane & 15);
+                const int nb    = tn * BN + wn * 128 + 16 * (lane >> 4); // first column of group 0; group 1 is 64 further
+                using in_vgpr   = std::integral_constant<bool, (i == MT - 1)>;
+                if constexpr(DT == DT_I8 && EPI == EPI_REQUANT_RND)
+                {
+                    // the values go through the table behind ONE wait per call (both column groups where the caller
+                    // allows): with a single wave per SIMD nothing else hides the latency of the byte reads
+                    if constexpr(G < 0)
+                    {
+                        i32x4 v[8];
+                        acc_t lo[4], hi[4];
+                        fetch_acc(in_vgpr{}, acc[i], 0, lo);
+                        fetch_acc(in_vgpr{}, acc[i], 1, hi);
+#pragma unroll
+                        for(int t = 0; t < 4; ++t)
+                            v[t] = lo[t], v[4 + t] = hi[t];
+                        int b[32];
+                        requant_lut<8>(v, p.scale_gemm, lut_lds, b);
+                        if(m < p.M)
+                        {
+                            int8_t* crow = reinterpret_cast<int8_t*>(c_batch) + (size_t)m * p.ldc;
+                            if(nb < p.N)
+                                store_bytes16(crow, nb, p.N, vec_ok, b, nt);
+                            if(nb + 64 < p.N)
+                                store_bytes16(crow, nb + 64, p.N, vec_ok, b + 16, nt);
+                        }
+                    }
+                    else
+                    {
+                        acc_t v[4];
+                        fetch_acc(in_vgpr{}, acc[i], G, v);
+                        int b[16];
+                        requant_lut<4>(v, p.scale_gemm, lut_lds, b);
+                        if(m < p.M && nb + 64 * G < p.N)
+                            store_bytes16(reinterpret_cast<int8_t*>(c_batch) + (size_t)m * p.ldc, nb + 64 * G, p.N, vec_ok, b, nt);
+                    }
+                    return;
+                }
+#pragma unroll
+                for(int g = (G < 0 ? 0 : G); g < (G < 0 ? 2 : G + 1); ++g)
+                {
+                    if constexpr(DT == DT_I8)
+                    {
+                        const int n0 = nb + 64 * g;
+                        if(m < p.M && n0 < p.N)
+                        {
+                            acc_t v[4];
+                            fetch_acc(in_vgpr{}, acc[i], g, v);
+                            int8_t* crow = reinterpret_cast<int8_t*>(c_batch) + (size_t)m * p.ldc;
+                            store_row16_i8<EPI>(crow, n0, p.N, vec_ok, v, p.scale_gemm, p.scale_relu, nt);
+                        }
+                    }
+                    else
+                    {
+                        const int n64 = tn * BN + wn * 128 + 64 * g;
+                        if(m < p.M && n64 < p.N)
+                        {
+                            acc_t v[4];
+                            fetch_acc(in_vgpr{}, acc[i], g, v);
+                            if constexpr(DT == DT_BF16)
+                                store_2x8(reinterpret_cast<__bf16*>(c_batch) + (size_t)m * p.ldc, n64, lane >> 4, p.N, vec_ok, v, nt);
+                            else
+                                store_2x8(reinterpret_cast<_Float16*>(c_batch) + (size_t)m * p.ldc, n64, lane >> 4, p.N, vec_ok, v, nt);
+                        }
+                    }
+                }
+            };
+            if constexpr(FUSED)
+            {
+                // the trailing fragment reads and (all-zero) loads; the MFMA results must have left the pipeline before the
+                // epilogue reads them (inline-assembly MFMAs are invisible to the compiler's hazard handling)
+                asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_nop 15\n\ts_nop 15" ::: "memory");
+                __builtin_amdgcn_sched_barrier(0);
+            }
             if constexpr(FUSED)
             {
                 if(p.epi != EPI_PASSTHROUGH)
@@ -525,77 +601,78 @@ struct GemmW4
                     continue;
                 }
             }
-            static_for<MT>([&](auto i_c) {
-                constexpr int i = decltype(i_c)::value;
-                const int m     = tm * BM + wm * 128 + 16 * i + (lane & 15);
-                const int nb    = tn * BN + wn * 128 + 16 * (lane >> 4); // first column of group 0; group 1 is 64 further
-                if constexpr(DT == DT_I8)
-                {
-                    if(p.epi == EPI_REQUANT_RND)
-                    {
-                        // the 32 values of the lane's two column groups go through the table behind ONE wait: with a single
-                        // wave per SIMD nothing else hides the latency of the byte reads
-                        i32x4 v[8];
-                        acc_t lo[4], hi[4];
-                        fetch_acc(std::integral_constant<bool, (i == MT - 1)>{}, acc[i], 0, lo);
-                        fetch_acc(std::integral_constant<bool, (i == MT - 1)>{}, acc[i], 1, hi);
-#pragma unroll
-                        for(int t = 0; t < 4; ++t)
-                            v[t] = lo[t], v[4 + t] = hi[t];
-                        int b[32];
-                        requant_lut<8>(v, p.scale_gemm, lut_lds, b);
-                        if(m < p.M)
-                        {
-                            int8_t* crow = reinterpret_cast<int8_t*>(c_batch) + (size_t)m * p.ldc;
-                            if(nb < p.N)
-                                store_bytes16(crow, nb, p.N, vec_ok, b, nt);
-                            if(nb + 64 < p.N)
-                                store_bytes16(crow, nb + 64, p.N, vec_ok, b + 16, nt);
-                        }
-                        return;
-                    }
-                }
-#pragma unroll
-                for(int g = 0; g < 2; ++g)
-                {
-                    if constexpr(DT == DT_I8)
-                    {
-                        const int n0 = nb + 64 * g;
-                        if(m < p.M && n0 < p.N)
-                        {
-                            acc_t v[4];
-                            fetch_acc(std::integral_constant<bool, (i == MT - 1)>{}, acc[i], g, v);
-                            int8_t* crow = reinterpret_cast<int8_t*>(c_batch) + (size_t)m * p.ldc;
-                            if(p.epi == EPI_REQUANT_CK)
-                                store_row16_i8<EPI_REQUANT_CK>(crow, n0, p.N, vec_ok, v, p.scale_gemm, p.scale_relu, nt);
-                            else
-                                store_row16_i8<EPI_PASSTHROUGH>(crow, n0, p.N, vec_ok, v, p.scale_gemm, p.scale_relu, nt);
-                        }
-                    }
-                    else
-                    {
-                        const int n64 = tn * BN + wn * 128 + 64 * g;
-                        if(m < p.M && n64 < p.N)
-                        {
-                            acc_t v[4];
-                            fetch_acc(std::integral_constant<bool, (i == MT - 1)>{}, acc[i], g, v);
-                            if constexpr(DT == DT_BF16)
-                                store_2x8(reinterpret_cast<__bf16*>(c_batch) + (size_t)m * p.ldc, n64, lane >> 4, p.N, vec_ok, v, nt);
-                            else
-                                store_2x8(reinterpret_cast<_Float16*>(c_batch) + (size_t)m * p.ldc, n64, lane >> 4, p.N, vec_ok, v, nt);
-                        }
-                    }
-                }
-            });
+            if constexpr(FUSED)
+            {
+                // (PassThrough on the kernel with the D-operand epilogues)
+                static_for<MT>([&](auto i_c) { store_row(i_c, both_groups{}); });
+            }
+            else
+            {
+                // ---- the last K tile (in stage kt & 1, its k-step 0 fragments on their way into af0 / bf0) and the
+                // epilogue in one: fragment row by fragment row, both k-steps of a row back to back (every accumulator
+                // still takes k-step 0 before k-step 1: same sums), so that a row is final 16 MFMAs after the one before
+                // it and its conversion and stores run between the MFMAs of the rows behind it. The C tile's way to
+                // memory starts seven eighths of a K tile earlier than behind the whole loop. Nothing is loaded and
+                // nothing read ahead any more. Rows 0 and 1 take their k-step 0 first, while the k-step 1 fragments
+                // arrive.
+                const int st = kt & 1;
+                auto row_mfmas = [&](auto fi_c, auto ks_c, auto part_c) { // MFMAs 4 * part .. 4 * part + 3 of the row's k-step
+                    constexpr int fi = decltype(fi_c)::value, KS = decltype(ks_c)::value;
+                    static_for<4>([&](auto j_c) {
+                        constexpr int j  = 4 * decltype(part_c)::value + decltype(j_c)::value;
+                        constexpr int ft = ((fi + KS) & 1) ? NB - 1 - j : j;
+                        if constexpr(KS == 0)
+                            mfma<fi == MT - 1, false>(acc[fi][ft], bf0[ft], af0[fi]);
+                        else
+                            mfma<fi == MT - 1, false>(acc[fi][ft], bf1[ft], af1[fi]);
+                    });
+                };
+                using std::integral_constant;
+                asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+                __builtin_amdgcn_sched_barrier(0);
+                static_for<16>([&](auto m_c) {
+                    constexpr int m = decltype(m_c)::value, fi = m / 8, j = m % 8, ft = (fi & 1) ? NB - 1 - j : j;
+                    mfma<false, false>(acc[fi][ft], bf0[ft], af0[fi]);
+                    read_one(st, integral_constant<int, 1>{}, m_c, af1, bf1); // B fragments 0 .. 7, then A fragments 0 .. 7
+                });
+                // (LDS reads return in order: all but the last six, the A fragments of rows 2 .. 7)
+                asm volatile("s_waitcnt lgkmcnt(6)" ::: "memory");
+                __builtin_amdgcn_sched_barrier(0);
+                static_for<2>([&](auto fi_c) {
+                    row_mfmas(fi_c, integral_constant<int, 1>{}, integral_constant<int, 0>{});
+                    row_mfmas(fi_c, integral_constant<int, 1>{}, integral_constant<int, 1>{});
+                });
+                asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+                __builtin_amdgcn_sched_barrier(0);
+                // (a row stored here took its last MFMA at least twelve MFMAs ago: the results have left the pipeline;
+                // inline-assembly MFMAs are invisible to the compiler's hazard handling)
+                static_for<MT - 2>([&](auto r_c) {
+                    using fi_c = integral_constant<int, decltype(r_c)::value + 2>;
+                    row_mfmas(fi_c{}, integral_constant<int, 0>{}, integral_constant<int, 0>{});
+                    __builtin_amdgcn_sched_barrier(0);
+                    store_row(r_c, integral_constant<int, 0>{});
+                    __builtin_amdgcn_sched_barrier(0);
+                    row_mfmas(fi_c{}, integral_constant<int, 0>{}, integral_constant<int, 1>{});
+                    row_mfmas(fi_c{}, integral_constant<int, 1>{}, integral_constant<int, 0>{});
+                    __builtin_amdgcn_sched_barrier(0);
+                    store_row(r_c, integral_constant<int, 1>{});
+                    __builtin_amdgcn_sched_barrier(0);
+                    row_mfmas(fi_c{}, integral_constant<int, 1>{}, integral_constant<int, 1>{});
+                });
+                asm volatile("s_waitcnt vmcnt(0)\n\ts_nop 15\n\ts_nop 15" ::: "memory");
+                __builtin_amdgcn_sched_barrier(0);
+                store_row(integral_constant<int, MT - 2>{}, both_groups{});
+                store_row(integral_constant<int, MT - 1>{}, both_groups{});
+            }
         }
     }
 };
 
-template <int DT, bool FUSED = false>
+template <int DT, bool FUSED = false, int EPI = EPI_PASSTHROUGH>
 __global__ __launch_bounds__(256) void gemm_w4_kernel(const GemmArgs p)
 {
     extern __shared__ __attribute__((aligned(1024))) uint8_t ckx_smem[];
-    GemmW4<DT, FUSED>::run(p, ckx_smem);
+    GemmW4<DT, FUSED, EPI>::run(p, ckx_smem);
 }
 
 } // namespace ckx
