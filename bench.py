@@ -114,6 +114,30 @@ for w in (
 ):
     WORKLOADS[w["name"]] = w
 
+# The layers the reference's own whole-network script drives through ckProfiler at N = 256
+# (script/profile_resnet50.sh:24-46: the de-duplicated list, run as `conv_fwd`): (K, C, filter, H = W, stride, pad)
+RESNET50_LAYERS = [
+    (256, 1024, 1, 14, 1, 0), (512, 1024, 1, 14, 1, 0), (128, 128, 3, 28, 1, 1), (512, 128, 1, 28, 1, 0),
+    (128, 128, 3, 56, 2, 1), (512, 2048, 1, 7, 1, 0), (1024, 256, 1, 14, 1, 0), (256, 256, 3, 14, 1, 1),
+    (256, 256, 3, 28, 2, 1), (128, 256, 1, 56, 1, 0), (64, 256, 1, 56, 1, 0), (512, 512, 3, 14, 2, 1),
+    (128, 512, 1, 28, 1, 0), (256, 512, 1, 28, 1, 0), (2048, 512, 1, 7, 1, 0), (512, 512, 3, 7, 1, 1),
+    (256, 64, 1, 56, 1, 0), (64, 64, 1, 56, 1, 0), (64, 64, 3, 56, 1, 1), (64, 3, 7, 224, 2, 3)]
+# ... and the distinct (operation, layer) pairs of its fused run (:47-99): conv_fwd_bias_relu_add on these layers, on
+# top of conv_fwd_bias_relu on every layer above
+RESNET50_BIAS_RELU_ADD = [(256, 64, 1, 56, 1, 0), (512, 128, 1, 28, 1, 0), (1024, 256, 1, 14, 1, 0), (2048, 512, 1, 7, 1, 0)]
+
+
+def resnet50_workloads(N=256):
+    out = []
+    for (K, C, f, HW, st, pd) in RESNET50_LAYERS:
+        tag = f"c{C}_k{K}_{f}x{f}_{HW}" + (f"_s{st}" if st > 1 else "")
+        for dt in ("f16", "i8"):
+            out.append(_conv_workload(f"conv_{dt}_{tag}", dt, C, K, f, HW, st, pd, N))
+        out.append(_conv_workload(f"conv_f16_{tag}_bias_relu", "f16", C, K, f, HW, st, pd, N, fused="bias_relu"))
+        if (K, C, f, HW, st, pd) in RESNET50_BIAS_RELU_ADD:
+            out.append(_conv_workload(f"conv_f16_{tag}_bias_relu_add", "f16", C, K, f, HW, st, pd, N, fused="bias_relu_add"))
+    return out
+
 
 def make_launcher(w, instance=-1, rotate=1):
     """Allocates the workload's synthetic operands on the GPU, returns the launch function.
@@ -453,6 +477,119 @@ def cpu_baseline(w, threads=None, budget_seconds=30.0):
             "port": port}
 
 
+def cpu_baseline_row(w, seconds=2.0, threads=None):
+    """The reference's own host operator for this workload's family (compiled in place into oracle/_ref: ReferenceGemm,
+    ReferenceConvFwd, ReferenceBatchedGemm; the oracle's restatement where that build is absent), timed on a sample of
+    the same problem -- rows of A, images, or batches -- sized by a probe for about `seconds` of work."""
+    import oracle
+    from oracle import lit
+    from composable_kernel_amd.host_tensor import uniform_f16, uniform_int8
+    threads = threads or cpu_threads()
+    ref = oracle.load_ref()
+    kind = "reference" if ref is not None else "port"
+    dt = w["dtype"]
+    if w["kind"] == "gemm":
+        M, N, K, G = w["M"], w["N"], w["K"], w.get("batch", 1)
+        unit_name, total, per_unit = "rows", M * G, 2.0 * N * K
+        if dt == "i8":
+            b = uniform_int8((N, K), -w["values"], w["values"], 2)
+            mk = lambda m: uniform_int8((m, K), -w["values"], w["values"], 1)
+            sg, sr = w["scales"]
+            run = (lambda a: ref.gemm_i8_requant(a, b.T, lit.EPI_REQUANT_RND, sg, sr)) if ref is not None else \
+                  (lambda a: lit.gemm_i8(a, b.T, lit.EPI_REQUANT_RND, sg, sr, nthreads=threads))
+            what = "ReferenceGemm<int8> + RequantReluRequant"
+        elif dt == "bf16":
+            from composable_kernel_amd.host_tensor import uniform_bf16
+            b = uniform_bf16((N, K), -1, 1, 2)
+            mk = lambda m: uniform_bf16((m, K), -1, 1, 1)
+            run = (lambda a: ref.gemm_bf16(a, b.T)) if ref is not None else (lambda a: lit.gemm_bf16(a, b.T, nthreads=threads))
+            what = "ReferenceGemm<bhalf_t>"
+        else:
+            b = uniform_f16((N, K), -1, 1, 2)
+            mk = lambda m: uniform_f16((m, K), -1, 1, 1)
+            run = (lambda a: ref.gemm_f16(a, b.T)) if ref is not None else (lambda a: lit.gemm_f16(a, b.T, nthreads=threads))
+            what = "ReferenceGemm<half_t> (the D-operand functor of the fused variants left out)" if w.get("fused") \
+                else "ReferenceGemm<half_t>"
+        call = lambda n: run(mk(n))
+    elif w["kind"] == "conv":
+        C_, K, f, HW, st, pd, nd, dil = w["C"], w["K"], w["f"], w["HW"], w["st"], w["pd"], w.get("ndim", 2), w.get("dil", 1)
+        Ho = (HW + 2 * pd - ((f - 1) * dil + 1)) // st + 1
+        unit_name, total, per_unit = "images", w["N"], 2.0 * K * Ho ** nd * C_ * f ** nd
+        gen = (lambda shp, seed: uniform_int8(shp, -5, 5, seed)) if dt == "i8" else (lambda shp, seed: uniform_f16(shp, -1, 1, seed))
+        wt = gen((K, *[f] * nd, C_), 4)
+        if ref is not None:
+            run = lambda x: ref.convnd_fwd(x, wt, [st] * nd, [dil] * nd, [pd] * nd)
+        else:
+            run = lambda x: lit.convnd_fwd(x, wt, [st] * nd, [dil] * nd, [pd] * nd)
+        what = f"ReferenceConvFwd<{'int8' if dt == 'i8' else 'half_t'}, {nd} spatial dimensions>, PassThrough output functor"
+        call = lambda n: run(gen((n, *[HW] * nd, C_), 3))
+    else:
+        G, M, N, K, O = (w[k] for k in ("G", "M", "N", "K", "O"))
+        unit_name, total, per_unit = "batches", G, 2.0 * M * N * (K + O)
+        mk3 = lambda g: [uniform_f16(shp, -0.5, 0.5, 5 + j) for j, shp in enumerate([(g, M, K), (g, N, K), (g, N, O)])]
+        if w.get("softmax"):
+            fn = ref.batched_gemm_softmax_gemm_f16 if ref is not None else lit.batched_gemm_softmax_gemm_f16
+            run = lambda a, b0, b1: fn(a, b0.transpose(0, 2, 1), b1, K ** -0.5)
+            what = "ReferenceBatchedGemm -> ReferenceSoftmax -> ReferenceBatchedGemm"
+        elif ref is not None:
+            run = lambda a, b0, b1: ref.batched_gemm_f16(ref.batched_gemm_f16(a, b0.transpose(0, 2, 1)), b1)
+            what = "two chained ReferenceBatchedGemm<half_t> (fp16 intermediate)"
+        else:
+            run = lambda a, b0, b1: lit.batched_gemm_gemm_f16(a, b0.transpose(0, 2, 1), b1, nthreads=threads)
+            what = "two chained batched GEMMs (fp16 intermediate)"
+        call = lambda n: run(*mk3(n))
+    n0 = min(total, 1 if w["kind"] != "gemm" else 8)
+    t0 = time.perf_counter()
+    call(n0)
+    dt0 = max(time.perf_counter() - t0, 1e-4)
+    n = int(min(total, max(n0, n0 * seconds / dt0)))
+    if n > n0:
+        t0 = time.perf_counter()
+        call(n)
+        dt0 = time.perf_counter() - t0
+    return {"value": round(per_unit * n / dt0 / 1e12, 5), "unit": "TOP/s" if dt == "i8" else "TFLOP/s",
+            "cores": min(threads, os.cpu_count() or threads) if ref is not None else threads, "kind": kind,
+            "host_cores": os.cpu_count(),
+            "sample": f"{n} of {total} {unit_name} of the same problem, {what}"
+                      + (" compiled in place (oracle/_ref; it starts one thread per host CPU)" if ref is not None
+                         else " restated (oracle/ck_oracle.cpp)") + f", {dt0:.1f} s (input generation included)"}
+
+
+def resnet50_sweep(args):
+    """Every layer of the reference's ResNet-50 script through the automatic instance choice: microseconds, rate, the
+    fraction of the binding roofline (algorithmic flops against the MFMA peak or algorithmic bytes against HBM,
+    whichever is larger) and the instance that ran."""
+    from composable_kernel_amd import capi
+    L = capi.lib()
+    rows = []
+    steps, warm = max(16, min(args.steps, 200)), max(3, min(args.warmup, 20))
+    print(f"| layer (N = 256) | dtype | op | instance | us | T(FL)OP/s | GB/s | of roofline |\n|---|---|---|---|---|---|---|---|",
+          file=sys.stderr)
+    for w in resnet50_workloads():
+        x = time_workload(w, steps, warm, -1, not args.no_graph, settle_ms=min(args.settle_ms, 100.0))
+        op = capi.OP_CONV2D_FWD_I8 if w["dtype"] == "i8" else capi.OP_CONV2D_FWD_F16
+        Ho = (w["HW"] + 2 * w["pd"] - w["f"]) // w["st"] + 1
+        desc = capi.Conv2dDesc(w["N"], w["K"], w["C"], w["HW"], w["HW"], w["f"], w["f"], Ho, Ho, w["st"], w["st"], 1, 1,
+                               w["pd"], w["pd"], w["pd"], w["pd"])
+        epi = {None: capi.EPI_REQUANT_RND if w["dtype"] == "i8" else capi.EPI_PASSTHROUGH,
+               "bias_relu": capi.EPI_ADD_RELU, "bias_relu_add": capi.EPI_ADD_RELU_ADD}[w["fused"]]
+        inst, runs = capi.conv2d_fwd_plan(op, desc, epi, 1 << 30)
+        name = L.ckx_instance_name(op, inst).decode()
+        frac = max(x["mfma_frac"], x["hbm_frac"])
+        row = {"workload": w["name"], "dtype": w["dtype"], "op": "conv_fwd" + ("_" + w["fused"] if w["fused"] else ""),
+               "instance": name, "k_runs": runs, "us": round(x["ms"] * 1e3, 2), "value": round(x["tput"], 1),
+               "unit": "TOP/s" if w["dtype"] == "i8" else "TFLOP/s", "GB/s": round(x["gbs"], 1), "bound": x["bound"],
+               "frac_of_bound": round(frac, 4)}
+        if not args.no_cpu:
+            row["cpu_baseline"] = cpu_baseline_row(w, min(args.cpu_seconds, 1.0), args.cpu_threads or None)
+        rows.append(row)
+        geo = f"C{w['C']} K{w['K']} {w['f']}x{w['f']} {w['HW']}^2 s{w['st']} p{w['pd']}"
+        print(f"| {geo} | {w['dtype']} | {row['op']} | {name}{' x' + str(runs) + ' K runs' if runs > 1 else ''} | {row['us']} | "
+              f"{row['value']} | {row['GB/s']} | {frac:.2f} {x['bound']} |", file=sys.stderr, flush=True)
+    print(json.dumps({"metric": "ResNet-50 conv forward layers, N = 256 (script/profile_resnet50.sh of the reference)",
+                      "steps": steps, "warmup": warm, "rows": rows}))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -466,6 +603,13 @@ def main():
     ap.add_argument("--no-graph", action="store_true", help="launch eagerly instead of replaying a HIP graph")
     ap.add_argument("--settle-ms", type=float, default=300.0,
                     help="least duration of the untimed clock-settling phase before the warm-up launches (0: none)")
+    ap.add_argument("--cpu-seconds", type=float, default=2.0,
+                    help="CPU time spent on the reference host operator beside every row under 'also' (the headline "
+                         "workload's own CPU leg is sized separately)")
+    ap.add_argument("--resnet50", action="store_true",
+                    help="instead of the headline: the ResNet-50 layers of the reference's whole-network script "
+                         "(script/profile_resnet50.sh) at N = 256, fp16 and int8, plain and fused; one JSON line with a "
+                         "row per layer, a table on stderr")
     ap.add_argument("--copy-probe", action="store_true",
                     help="also run one 256 MiB device-to-device copy (a kernel of known traffic, used to "
                          "scale the FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run)")
@@ -487,6 +631,8 @@ def main():
         dst = torch.empty_like(src)
         dst.copy_(src)
         torch.cuda.synchronize()
+    if args.resnet50:
+        return resnet50_sweep(args)
     w = WORKLOADS[args.workload]
     r = time_workload(w, args.steps, args.warmup, args.instance, not args.no_graph, settle_ms=args.settle_ms,
                       from_idle=True, sample_clock=True)
@@ -509,6 +655,9 @@ def main():
                                  settle_ms=args.settle_ms / 2)
             row.update({"cold_ms": round(cold["ms"], 5), "cold_GB/s": round(cold["gbs"], 1),
                         "cold_frac_of_bound": round(cold["hbm_frac"], 4)})
+        if not args.no_cpu:
+            # the reference's host operator on a bounded sample of the same problem, in the same run
+            row["cpu_baseline"] = cpu_baseline_row(wl, args.cpu_seconds, args.cpu_threads or None)
         also.append(row)
 
     unit = "TOP/s" if w["dtype"] == "i8" else "TFLOP/s"

@@ -5,14 +5,18 @@
 Flags: -ffp-contract=off keeps the requant epilogue's fp32 multiplies unfused;
 packed fp32 VALU forms are disabled for the device pass.
 
-Two guards protect the kernels' hand-managed waits (the MFMA fragment reads of gemm_tile.hpp, conv_patch.hpp and
+Three guards protect the kernels' hand-managed waits (the MFMA fragment reads of gemm_tile.hpp, conv_patch.hpp and
 conv_pointwise.hpp are inline-assembly LDS reads that the compiler does not count in lgkmcnt; the kernels wait for
 them themselves, so no compiler-made copy or spill of such a register may run before that wait):
   * every kernel's register report (-Rpass-analysis=kernel-resource-usage) is read, and the build FAILS if one of
     those kernels spills vector registers (the fused two-GEMM kernel, which reads LDS through compiler-known
     builtins, is allowed its four spilled registers in the long-sequence softmax variant);
-  * the compiler version the kernels were validated with is recorded below; another one builds with a loud warning
-    (the bit-exact integer-operand GPU tests are the gate for adopting it).
+  * the four-wave GEMM body (gemm_w4.hpp) also issues its MFMAs and direct loads as inline assembly: its kernels must
+    use no scratch memory and exactly the AccVGPRs the source ties accumulators to (a compiler that moved an
+    accumulator or fragment through another register between the assembly and its wait would show up there);
+  * the compiler version the kernels were validated with is recorded below; another one FAILS the build unless
+    CKX_ALLOW_UNVALIDATED_COMPILER=1 is set (then it builds with a loud warning; the bit-exact integer-operand GPU
+    tests are the gate for adding a compiler to the list).
 """
 import os
 import subprocess
@@ -44,6 +48,10 @@ def compiler_version():
 def check_compiler():
     import warnings
     v = compiler_version()
+    if v not in VALIDATED_COMPILERS and os.environ.get("CKX_ALLOW_UNVALIDATED_COMPILER") != "1":
+        raise RuntimeError(f"libckx: hipcc is {v!r}; its hand-waited inline-assembly kernels were validated with "
+                           f"{VALIDATED_COMPILERS[0]!r}. Set CKX_ALLOW_UNVALIDATED_COMPILER=1 to build anyway, then run "
+                           "the GPU suite (bit-exact integer-operand tests) before trusting the build.")
     if v not in VALIDATED_COMPILERS:
         warnings.warn(f"libckx is being built with an unvalidated compiler ({v}); its kernels wait for inline-assembly "
                       "LDS reads by hand and were validated with " + VALIDATED_COMPILERS[0] + ": run the GPU suite "
@@ -66,6 +74,32 @@ def vgpr_spills(compiler_output):
             n = int(line.split("VGPRs Spill:", 1)[1].split("[", 1)[0])
             if n and any(k in name for k in HAND_WAITED_KERNELS):
                 bad.append((name, n))
+    return bad
+
+
+# gemm_w4_kernel: AccVGPRs a lane's accumulators are tied to (the last fragment row's live in VGPRs); the variants with
+# D operands may park a few more values there
+W4_AGPRS = 224
+W4_AGPRS_FUSED_MAX = 232
+
+
+def w4_register_faults(compiler_output):
+    """(kernel, what) for every gemm_w4_kernel of the resource-usage report that uses scratch memory or another number of
+    AccVGPRs than the source ties."""
+    bad, name = [], None
+    for line in compiler_output.splitlines():
+        if "Function Name:" in line:
+            name = line.split("Function Name:", 1)[1].split("[", 1)[0].strip()
+            name = name if "gemm_w4_kernel" in name else None
+        elif name and "ScratchSize [bytes/lane]:" in line:
+            n = int(line.split("ScratchSize [bytes/lane]:", 1)[1].split("[", 1)[0])
+            if n:
+                bad.append((name, f"{n} bytes of scratch per lane"))
+        elif name and "AGPRs:" in line:
+            n = int(line.split("AGPRs:", 1)[1].split("[", 1)[0])
+            fused = "ILi1ELb1E" in name      # <DT_F16, FUSED = true, ...>
+            if (n != W4_AGPRS and not fused) or (fused and not W4_AGPRS <= n <= W4_AGPRS_FUSED_MAX):
+                bad.append((name, f"{n} AccVGPRs"))
     return bad
 
 
@@ -99,6 +133,7 @@ def build_lib(force=False, verbose=False, extra_flags=()):
         lines = [l for l in r.stdout.splitlines() if "packed-fp32-ops" not in l]
         # the register report: keep it out of the log, fail on vector register spills
         spills = vgpr_spills(r.stdout)
+        w4_bad = w4_register_faults(r.stdout)
         out, skip = [], 0
         for l in lines:
             if "[-Rpass-analysis=kernel-resource-usage]" in l:
@@ -114,6 +149,9 @@ def build_lib(force=False, verbose=False, extra_flags=()):
         if spills:
             raise RuntimeError("vector register spills (the hand-managed LDS read waits do not survive them): "
                                + ", ".join(f"{k}: {n}" for k, n in spills))
+        if w4_bad:
+            raise RuntimeError("four-wave GEMM body: register allocation differs from what its inline assembly assumes: "
+                               + ", ".join(f"{k}: {what}" for k, what in w4_bad))
         if verbose and out.strip():
             print(out)
 

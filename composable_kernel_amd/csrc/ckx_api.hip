@@ -588,6 +588,9 @@ int run_gemm(int dt, const void* a, const void* b, void* c, int M, int N, int K,
         g.ldd0 = dops.ldd0, g.ldd1 = dops.ldd1;
         g.ksplit  = 1;
         g.tiles_m = (M + 63) / 64, g.tiles_n = (N + 63) / 64;
+        if(batch > 65535)
+            return fail(CKX_UNSUPPORTED, "the element-granular instance (operands that are not 16-byte aligned vectors) "
+                                         "takes at most 65535 batches per launch");
         ckx::GenericLayout lay{};
         lay.a_sm = ta ? 1 : sa, lay.a_sk = ta ? sa : 1;
         lay.b_sn = tb ? 1 : sb, lay.b_sk = tb ? sb : 1;
@@ -1262,6 +1265,13 @@ int ckx_gemm_i8_splitk_noalloc(const void* a, const void* b, void* c, int32_t M,
 {
     if(k_batch < 1)
         return fail(CKX_INVALID_VALUE, "KBatch must be at least 1");
+    // (argument errors and empty problems are answered before the GPU is touched)
+    if(int st = check_gemm_shape(ckx::DT_I8, M, N, K, sa, sb, sc, al, bl, cl, epilogue, instance))
+        return st;
+    if(k_batch > 8)
+        return fail(CKX_UNSUPPORTED, "KBatch must be 1..8");
+    if(M == 0 || N == 0)
+        return CKX_OK;
     const int64_t need = ckx_gemm_splitk_workspace_bytes(CKX_OP_GEMM_I8, M, N, K, k_batch);
     if(need > (int64_t)CKX_STATIC_WORKSPACE_BYTES)
         return fail(CKX_UNSUPPORTED, "this split needs " + std::to_string(need) +

@@ -417,7 +417,9 @@ __device__ __forceinline__ void load_col_scales(const __amdgpu_buffer_rsrc_t& rs
 // EXT = false leaves the scaled / GELU modes out of the generated code (callers that have already branched on them).
 // fast_gelu(x) = x / (1 + exp(-2x(0.035677 x^2 + 0.797885))), the closed form of the reference's
 // 0.5 + 0.5 * (2 / (1 + emu) - 1) (element_wise_operation.hpp:127-133), the quotient through v_rcp_f32;
-// x -> -inf gives exp -> +inf, a reciprocal of 0 and -0.
+// x -> -inf gives exp -> +inf, a reciprocal of 0 and -0. Not bit for bit the reference's functor: its form cancels to a
+// coarse or zero factor for x below about -5, where this one returns small negative values (a few fp16 subnormal
+// steps apart) -- parity with it is by tolerance (rtol = atol = 1e-2).
 template <bool EXT = true>
 __device__ __forceinline__ float epi_f16_value(int mode, float acc, float d0, float d1, float alpha = 1.0f,
                                                float beta = 1.0f)
@@ -430,7 +432,7 @@ __device__ __forceinline__ float epi_f16_value(int mode, float acc, float d0, fl
         {
             const float x = acc + d0 + d1;
             const float u = 2.0f * x * (0.035677f * x * x + 0.797885f);
-            return x * __builtin_amdgcn_rcpf(1.0f + __expf(-u)); // (one ulp of fp32: far inside the fp16 result's rounding)
+            return x * __builtin_amdgcn_rcpf(1.0f + __expf(-u)); // (v_rcp_f32: one ulp of fp32)
         }
     }
     if(mode == EPI_CSHUFFLE_ADD_RELU)

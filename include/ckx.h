@@ -227,7 +227,12 @@ int ckx_gemm_i8_splitk_noalloc(const void* p_a, const void* p_b, void* p_c, int3
  * ::MakeArgumentPointer + Run (device_gemm_multiple_d.hpp:14-55) for cde_op in
  * CKX_EPI_ADD_RELU / _ADD_RELU_ADD / _CSHUFFLE_ADD_RELU / _ADD_ADD_FASTGELU (and, for the query, _BILINEAR). D0, D1 are
  * [M,N] row-major fp16 with row strides stride_d0 / stride_d1 in elements; stride 0 broadcasts one row (a bias
- * vector), as examples 03 and 04 do. p_d1 is ignored unless cde_op uses it. */
+ * vector), as examples 03 and 04 do. p_d1 is ignored unless cde_op uses it. With a K-major operand (A column-major
+ * or B row-major) these run on CKX_INSTANCE_AUTO or the element-granular instance only; an explicit tile or skinny
+ * instance answers CKX_UNSUPPORTED. CKX_EPI_ADD_ADD_FASTGELU agrees with the reference's functor
+ * (element_wise_operation.hpp:113-140) within rtol = atol = 1e-2, not bit for bit: the device evaluates
+ * x / (1 + exp(-u)); the reference's 0.5 + 0.5 * (2 / (1 + exp(-u)) - 1) cancels to a coarse or zero factor for
+ * x below about -5, where the device returns small negative values (a few fp16 subnormal steps apart). */
 int ckx_gemm_f16_multiple_d_is_supported(int32_t M, int32_t N, int32_t K, int32_t stride_a, int32_t stride_b,
                                          int32_t stride_d0, int32_t stride_d1, int32_t stride_e, int a_layout,
                                          int b_layout, int e_layout, int cde_op, int instance);
@@ -250,7 +255,9 @@ int ckx_gemm_f16_bilinear(const void* p_a, const void* p_b, const void* p_d, voi
  * Activation_Mul2_Clamp<Act>>::MakeArgumentPointer + Run (device_gemm_multiple_d.hpp:14-55) for cde_op in
  * CKX_EPI_MUL2_CLAMP / CKX_EPI_RELU_MUL2_CLAMP. D0 is one contiguous row of N floats, broadcast over the rows
  * (stride_d0 must be 0, as a per-channel scale is passed upstream). Every instance of the int8 GEMM family takes it
- * (tile, skinny, element-wise; K runs through the workspace; all four operand layouts); batches do not. */
+ * (tile, skinny, element-wise; K runs through the workspace) with A row-major and B column-major; with a K-major
+ * operand (A column-major or B row-major) it runs on CKX_INSTANCE_AUTO or the element-granular instance only -- an
+ * explicit tile or skinny instance answers CKX_UNSUPPORTED. Batches do not take it. */
 int ckx_gemm_i8_multiple_d_is_supported(int32_t M, int32_t N, int32_t K, int32_t stride_a, int32_t stride_b,
                                         int32_t stride_d0, int32_t stride_e, int a_layout, int b_layout, int e_layout,
                                         int cde_op, int instance);

@@ -130,3 +130,30 @@ conv_patch.hpp:410:1: remark:     VGPRs Spill: 0 [-Rpass-analysis=kernel-resourc
     assert "-Rpass-analysis=kernel-resource-usage" in build.DEVICE_FLAGS
     assert "clang version" in build.compiler_version()
     assert all("clang version" in v for v in build.VALIDATED_COMPILERS)
+
+
+def test_d_operand_epilogues_with_k_major_operands_run_on_auto_or_the_element_granular_instance_only():
+    """The is_supported answers per instance and layout, as include/ckx.h states them: with A column-major or B
+    row-major the D-operand epilogues (per-column requant scales, the fp16 add / scale / GELU functors) are
+    supported by CKX_INSTANCE_AUTO and by the element-granular instance (the last of the family) and by no explicit
+    tile or skinny instance; with A row-major and B column-major every instance that takes the shape supports them."""
+    L = capi.lib()
+    M, N, K = 16, 256, 512   # (16 rows: within the reach of every skinny instance)
+    n_i8, n_f16 = L.ckx_num_instances(capi.OP_GEMM_I8), L.ckx_num_instances(capi.OP_GEMM_F16)
+    lay = {"mk_nk": (capi.ROW_MAJOR, capi.COL_MAJOR), "km_nk": (capi.COL_MAJOR, capi.COL_MAJOR),
+           "mk_kn": (capi.ROW_MAJOR, capi.ROW_MAJOR), "km_kn": (capi.COL_MAJOR, capi.ROW_MAJOR)}
+    for name, (al, bl) in lay.items():
+        sa, sb = (K if al == capi.ROW_MAJOR else M), (K if bl == capi.COL_MAJOR else N)
+        for inst in [capi.INSTANCE_AUTO] + list(range(n_i8)):
+            st = L.ckx_gemm_i8_multiple_d_is_supported(M, N, K, sa, sb, 0, N, al, bl, capi.ROW_MAJOR, capi.EPI_MUL2_CLAMP, inst)
+            if name == "mk_nk" or inst in (capi.INSTANCE_AUTO, n_i8 - 1):
+                assert st == capi.OK, (name, inst, capi.last_error())
+            else:
+                assert st == capi.UNSUPPORTED, (name, inst)
+        for inst in [capi.INSTANCE_AUTO] + list(range(n_f16)):
+            st = L.ckx_gemm_f16_multiple_d_is_supported(M, N, K, sa, sb, 0, N, N, al, bl, capi.ROW_MAJOR,
+                                                        capi.EPI_ADD_ADD_FASTGELU, inst)
+            if name == "mk_nk" or inst in (capi.INSTANCE_AUTO, n_f16 - 1):
+                assert st == capi.OK, (name, inst, capi.last_error())
+            else:
+                assert st == capi.UNSUPPORTED, (name, inst)

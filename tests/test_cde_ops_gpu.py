@@ -164,6 +164,29 @@ def test_fastgelu_limits_through_the_kernel(instance):
     assert out[0, 0] == 0 and out[0, 7] == np.float16(30000.0) and out[3, 0] == 0
 
 
+def test_fastgelu_negative_tail_is_pinned():
+    """Parity of AddAddFastGelu with the reference's functor is by tolerance, not bit for bit: the device evaluates
+    x / (1 + exp(-u)), the reference 0.5 + 0.5 * (2 / (1 + exp(-u)) - 1), whose cancellation makes the factor coarse or
+    exactly zero for x below about -5 where the device still returns small negative values. A = 0 turns the GEMM into
+    fast_gelu(d0 + d1): a sweep of the sum over [-12, 12] pins the deviation -- at most a few fp16 subnormal steps
+    (2^-24 each) in that tail, the suite's rtol = atol = 1e-2 everywhere."""
+    M, N, K = 64, 256, 64
+    a = np.zeros((M, K), np.float16)
+    b_kn = uniform_f16((K, N), -1, 1, 1250)
+    s = np.linspace(-12.0, 12.0, M * N, dtype=np.float32).reshape(M, N)
+    d0 = np.zeros((1, N), np.float16)
+    d1 = s.astype(np.float16)
+    out = _run(a, b_kn, [d0, d1], [0, N], ck.AddAddFastGelu(), capi.INSTANCE_AUTO).astype(np.float32)
+    x = d1.astype(np.float32)
+    want = fast.fast_gelu(x).astype(np.float16).astype(np.float32)
+    _close(out.astype(np.float16), want.astype(np.float16))
+    tail = x < -5.0
+    assert tail.any()
+    # in the tail both results are tiny: the device's within 8 fp16 subnormal steps of the reference's, and never positive
+    assert np.abs(out[tail] - want[tail]).max() <= 8 * 2.0 ** -24
+    assert (out[tail] <= 0).all()
+
+
 @pytest.mark.parametrize("runs", [2, 3])
 def test_k_runs_apply_the_functor_in_the_second_pass(force_k_runs, runs):
     M, N, K = 96, 136, 2048

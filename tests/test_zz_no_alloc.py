@@ -46,6 +46,40 @@ def test_noalloc_split_k_matches_the_workspace_entry_point_twice_in_a_row():
         np.testing.assert_array_equal(got, want)
 
 
+def test_noalloc_entry_point_allocates_no_device_memory():
+    """hipMemGetInfo before and after two calls (the first resolves the static array's address): the free figure
+    does not move. Operands and the output are allocated beforehand."""
+    import torch
+    import gpu_util
+    L = capi.lib()
+    M, N, K, kb = 136, 200, 2048, 4
+    da = gpu_util.dev(uniform_int8((M, K), -8, 8, 330))
+    db = gpu_util.dev(uniform_int8((N, K), -8, 8, 331))
+    dc = torch.zeros((M, N), dtype=torch.int8, device="cuda")
+    s = C.c_void_p(gpu_util.stream())
+    torch.cuda.synchronize()
+    free0, _ = torch.cuda.mem_get_info()
+    for _ in range(2):
+        capi.check(L.ckx_gemm_i8_splitk_noalloc(da.data_ptr(), db.data_ptr(), dc.data_ptr(), M, N, K, K, K, N, capi.ROW_MAJOR,
+                                                capi.COL_MAJOR, capi.ROW_MAJOR, capi.EPI_REQUANT_RND, SG, SR, capi.INSTANCE_AUTO,
+                                                kb, s))
+    torch.cuda.synchronize()
+    free1, _ = torch.cuda.mem_get_info()
+    assert free1 == free0
+
+
+def test_noalloc_argument_errors_are_answered_like_the_workspace_entry_point():
+    """Bad arguments and empty problems come back before any device work: the codes of ckx_gemm_i8_splitk."""
+    L = capi.lib()
+    s = C.c_void_p(0)
+    call = lambda M, N, K, bl, kb: L.ckx_gemm_i8_splitk_noalloc(0, 0, 0, M, N, K, K, K, N, capi.ROW_MAJOR, bl, capi.ROW_MAJOR,
+                                                            capi.EPI_REQUANT_RND, SG, SR, capi.INSTANCE_AUTO, kb, s)
+    assert call(64, 64, 1024, capi.COL_MAJOR, 9) == capi.UNSUPPORTED
+    assert call(64, 64, 1024, 7, 2) == capi.INVALID_VALUE
+    assert call(0, 64, 1024, capi.COL_MAJOR, 2) == capi.OK
+    assert call(64, 64, 1024, capi.COL_MAJOR, 0) == capi.INVALID_VALUE
+
+
 def test_noalloc_split_k_at_the_size_limit_and_beyond():
     import torch
     import gpu_util
