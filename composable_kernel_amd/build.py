@@ -60,7 +60,8 @@ def check_compiler():
 
 
 # kernels whose LDS fragment reads are inline assembly waited for by hand (mangled-name fragments)
-HAND_WAITED_KERNELS = ("gemm_tile_kernel", "gemm_w4_kernel", "conv_patch_kernel", "conv_pointwise_kernel")
+HAND_WAITED_KERNELS = ("gemm_tile_kernel", "gemm_w4_kernel", "gemm_astream_kernel", "conv_patch_kernel",
+                       "conv_pointwise_kernel")
 
 
 def vgpr_spills(compiler_output):

@@ -317,6 +317,15 @@ hipError_t launch_skinny(const ckx::GemmArgs& a, int grid, hipStream_t s)
             &launch_skinny<ckx::DT_BF16, MT, NW, KU, NT>                                                    \
     }
 
+// the weight-streaming instance for up to 128 rows (gemm_astream.hpp): A tiles of all rows in LDS, requested by loader
+// waves; B straight into the compute waves' registers; the whole K extent per workgroup
+#define CKX_ASTREAM(NT)                                                                                                \
+    {                                                                                                                  \
+        "MI355X_Mfma16_Stream<rows 8x16, cols " #NT "x16, 4 compute + 4 loader waves, A tiles in LDS, B in registers>", 128, NT * 16, \
+            ckx::astream_launcher(ckx::DT_I8, NT), ckx::astream_launcher(ckx::DT_F16, NT),                              \
+            ckx::astream_launcher(ckx::DT_BF16, NT)                                                                    \
+    }
+
 const SkinnyInstance kSkinny[] = {
     CKX_SKINNY(1, 8, 4, 1),
     CKX_SKINNY(2, 8, 4, 1),
@@ -326,7 +335,9 @@ const SkinnyInstance kSkinny[] = {
     CKX_SKINNY(1, 8, 2, 2),
     CKX_SKINNY(2, 8, 2, 4),
     CKX_SKINNY(2, 8, 2, 2),
+    CKX_ASTREAM(3),
 };
+constexpr int kAStream = 8; // (position in kSkinny)
 constexpr int kNumSkinny    = sizeof(kSkinny) / sizeof(kSkinny[0]);
 // the element-granular instance (gemm_generic.hpp) closes every GEMM and conv instance list: any extent, leading
 // dimension, channel count and base address, all four GEMM layouts, every epilogue of the data type
@@ -516,6 +527,16 @@ GemmChoice choose_gemm(int dt, int M, int N, int K, bool kmajor, int instance, l
     // (64 x 4096 x 11008: 20 against 27 us; at K = 4096 the 64-row skinny instance is ahead, 11.8 against 13.0 us)
     // (fp16, 8..16 rows, many columns and a long K: HBM streaming either way, and the skinny kernels' A re-reads out of
     // L2 show -- 16 x 11008 x 4096 fp16: 21.6 us against 18.2 on the four-stage tile; int8 stays: 12.2 against 13.8)
+    // 65 .. 128 rows against a weight matrix of 32 MB and more whose 48-column blocks fill most of the CUs in one round: the
+    // weight-streaming instance (A tiles of all rows through LDS by loader waves, B straight into registers, all of K per
+    // workgroup, one launch). 128 x 11008 x 4096 int8: 20.1 us against 23.3 with the weights coming out of HBM (eight
+    // copies used in turn), 17.2 against 16.5 us when they sit in the Infinity Cache -- weights of a model that does not
+    // fit that cache are the case that counts. (A longer K means more of A per byte of B through every CU: at K = 8192 the
+    // tile kernel with K runs is ahead, 25.0 against 32.9 us; fp16 doubles the bytes of K as well.)
+    const long stream_blocks = (N + 47) / 48;
+    if(instance == CKX_INSTANCE_AUTO && !kmajor && batch == 1 && k_batch == 0 && es == 1 && M > 64 && M <= 128 &&
+       (long)N * K * es >= (32l << 20) && (long)K * es <= 6144 && stream_blocks >= 160 && stream_blocks <= num_cus())
+        return GemmChoice{kNumTiles + kAStream, 1, nk};
     const bool f16_long = es == 2 && M >= 8 && M <= 64 && (long)K * es >= 8192 && (N + 63) / 64 >= 160;
     const bool tile64 = kmajor || f16_long || (M > 16 && M <= 64 &&
                                    ((N + 63) / 64 >= 160 ||

@@ -15,6 +15,69 @@
 
 namespace ckx {
 
+// Epilogue and store of one lane's four consecutive outputs (row m, columns nn .. nn + 3) of a summed 16 x 16
+// accumulator tile in the D^T = B_frag x A_frag lane layout: lane (m % 16, q) holds columns 4q .. 4q + 3.
+template <int DT, typename ACC>
+__device__ __forceinline__ void store_quad(const GemmArgs& p, const ACC& s, int m, int nn)
+{
+    // lane (m = lane%16, q): columns 4q .. 4q+3 of the tile's 16, row 16*mt + m
+    if(m >= p.M || nn >= p.N)
+        return;
+    if constexpr(DT == DT_I8)
+    {
+        int b[4];
+        if(epi_per_column_scale(p.epi))
+        {
+            const float* sc = reinterpret_cast<const float*>(p.d0);
+#pragma unroll
+            for(int j = 0; j < 4; ++j)
+                b[j] = nn + j < p.N ? mul2_clamp(s[j], sc[nn + j], p.epi == EPI_RELU_MUL2_CLAMP) : 0;
+        }
+        else
+        {
+#pragma unroll
+            for(int j = 0; j < 4; ++j)
+                b[j] = p.epi == EPI_REQUANT_RND  ? requant_rnd(s[j], p.scale_gemm, p.scale_relu)
+                       : p.epi == EPI_REQUANT_CK ? requant_ck(s[j], p.scale_gemm, p.scale_relu)
+                                                 : s[j];
+        }
+        int8_t* crow = reinterpret_cast<int8_t*>(p.c) + (size_t)m * p.ldc + nn;
+        if(nn + 4 <= p.N && ((reinterpret_cast<uintptr_t>(crow)) & 3u) == 0)
+            *reinterpret_cast<int*>(crow) = pack4_low_bytes(b[0], b[1], b[2], b[3]);
+        else
+        {
+#pragma unroll
+            for(int j = 0; j < 4; ++j)
+                if(nn + j < p.N)
+                    crow[j] = (int8_t)b[j];
+        }
+    }
+    else if constexpr(DT == DT_BF16)
+    {
+        __bf16* crow = reinterpret_cast<__bf16*>(p.c) + (size_t)m * p.ldc + nn;
+#pragma unroll
+        for(int j = 0; j < 4; ++j)
+            if(nn + j < p.N)
+                crow[j] = (__bf16)s[j];
+    }
+    else
+    {
+        _Float16* crow       = reinterpret_cast<_Float16*>(p.c) + (size_t)m * p.ldc + nn;
+        const _Float16* d0row = reinterpret_cast<const _Float16*>(p.d0) + (size_t)m * p.ldd0 + nn;
+        const _Float16* d1row = reinterpret_cast<const _Float16*>(p.d1) + (size_t)m * p.ldd1 + nn;
+#pragma unroll
+        for(int j = 0; j < 4; ++j)
+            if(nn + j < p.N)
+            {
+                float val = s[j];
+                if(p.epi != EPI_PASSTHROUGH)
+                    val = epi_f16_value(p.epi, val, (float)d0row[j], epi_has_d1(p.epi) ? (float)d1row[j] : 0.0f,
+                                        p.scale_gemm, p.scale_relu);
+                crow[j] = (_Float16)val;
+            }
+    }
+}
+
 template <int DT, int MT, int NW, int KU, int NT = 1>
 __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(const GemmArgs p)
 {
@@ -128,63 +191,7 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(const GemmArgs p)
             s[0] += v[0], s[1] += v[1], s[2] += v[2], s[3] += v[3];
         }
         // lane (m = lane%16, q): columns 4q .. 4q+3 of the tile's 16, row 16*mt + m
-        const int m  = 16 * mt + (int)r;
-        const int nn = n0 + 16 * nt + 4 * (int)q;
-        if(m >= p.M || nn >= p.N)
-            continue;
-        if constexpr(DT == DT_I8)
-        {
-            int b[4];
-            if(epi_per_column_scale(p.epi))
-            {
-                const float* sc = reinterpret_cast<const float*>(p.d0);
-#pragma unroll
-                for(int j = 0; j < 4; ++j)
-                    b[j] = nn + j < p.N ? mul2_clamp(s[j], sc[nn + j], p.epi == EPI_RELU_MUL2_CLAMP) : 0;
-            }
-            else
-            {
-#pragma unroll
-                for(int j = 0; j < 4; ++j)
-                    b[j] = p.epi == EPI_REQUANT_RND  ? requant_rnd(s[j], p.scale_gemm, p.scale_relu)
-                           : p.epi == EPI_REQUANT_CK ? requant_ck(s[j], p.scale_gemm, p.scale_relu)
-                                                     : s[j];
-            }
-            int8_t* crow = reinterpret_cast<int8_t*>(p.c) + (size_t)m * p.ldc + nn;
-            if(nn + 4 <= p.N && ((reinterpret_cast<uintptr_t>(crow)) & 3u) == 0)
-                *reinterpret_cast<int*>(crow) = pack4_low_bytes(b[0], b[1], b[2], b[3]);
-            else
-            {
-#pragma unroll
-                for(int j = 0; j < 4; ++j)
-                    if(nn + j < p.N)
-                        crow[j] = (int8_t)b[j];
-            }
-        }
-        else if constexpr(DT == DT_BF16)
-        {
-            __bf16* crow = reinterpret_cast<__bf16*>(p.c) + (size_t)m * p.ldc + nn;
-#pragma unroll
-            for(int j = 0; j < 4; ++j)
-                if(nn + j < p.N)
-                    crow[j] = (__bf16)s[j];
-        }
-        else
-        {
-            _Float16* crow       = reinterpret_cast<_Float16*>(p.c) + (size_t)m * p.ldc + nn;
-            const _Float16* d0row = reinterpret_cast<const _Float16*>(p.d0) + (size_t)m * p.ldd0 + nn;
-            const _Float16* d1row = reinterpret_cast<const _Float16*>(p.d1) + (size_t)m * p.ldd1 + nn;
-#pragma unroll
-            for(int j = 0; j < 4; ++j)
-                if(nn + j < p.N)
-                {
-                    float val = s[j];
-                    if(p.epi != EPI_PASSTHROUGH)
-                        val = epi_f16_value(p.epi, val, (float)d0row[j], epi_has_d1(p.epi) ? (float)d1row[j] : 0.0f,
-                                            p.scale_gemm, p.scale_relu);
-                    crow[j] = (_Float16)val;
-                }
-        }
+        store_quad<DT>(p, s, 16 * mt + (int)r, n0 + 16 * nt + 4 * (int)q);
     }
 }
 

@@ -74,6 +74,10 @@ tile_launch_fn layout_tile(int dt, int tile, bool a_kmajor, bool b_kmajor);
 // else null), with the D-operand epilogues
 tile_launch_fn w4_tile(int dt, bool fused);
 
+// weight-streaming GEMM for up to 128 rows (gemm_astream.hip): launcher for element type dt (DT_*) with 16 * nt output
+// columns per workgroup (nt = 3), grid = number of such column blocks
+tile_launch_fn astream_launcher(int dt, int nt);
+
 // conv forward with three spatial dimensions (conv3d.hip): launcher of tile instance `tile` for DT_I8 / DT_F16
 tile_launch_fn conv3d_tile(int dt, int tile);
 

@@ -16,8 +16,8 @@ from oracle import fast, lit
 
 pytestmark = pytest.mark.gpu
 
-N_INSTANCES = 18        # tile instances, the skinny (few-row) instances, the element-wise (padding) instance
-SKINNY_MAX_M = {9: 16, 10: 32, 11: 64, 12: 16, 13: 16, 14: 16, 15: 32, 16: 32}
+N_INSTANCES = 19        # tile instances, the skinny (few-row) and weight-streaming instances, the element-wise (padding) instance
+SKINNY_MAX_M = {9: 16, 10: 32, 11: 64, 12: 16, 13: 16, 14: 16, 15: 32, 16: 32, 17: 128}
 RTOL = ATOL = 1e-2
 
 EPILOGUES = {

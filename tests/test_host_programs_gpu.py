@@ -100,7 +100,7 @@ def test_profiler_reports_unsupported_problems(tmp_path):
     dimension below K is supported by no instance and the profiler fails."""
     M, N, K = 64, 64, 100
     out, dump = _run("ckx_profiler", ["gemm", 3, 1, 1, 1, 0, 0, M, N, K, -1, -1, -1], "CKX_PROFILER_DUMP", tmp_path)
-    assert out.count("does not support this problem") == 17      # the tile and skinny instances; the last one runs
+    assert out.count("does not support this problem") == 18      # the tile and skinny instances; the last one runs
     c = np.fromfile(dump, np.int8).reshape(M, N)
     a = uniform_int8((M, K), -5, 5, SEED)
     b_nk = uniform_int8((N, K), -5, 5, SEED + 1)

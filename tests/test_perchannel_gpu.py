@@ -22,8 +22,8 @@ from oracle import fast, lit
 
 pytestmark = pytest.mark.gpu
 
-N_INSTANCES = 18
-SKINNY_MAX_M = {9: 16, 10: 32, 11: 64, 12: 16, 13: 16, 14: 16, 15: 32, 16: 32}
+N_INSTANCES = 19
+SKINNY_MAX_M = {9: 16, 10: 32, 11: 64, 12: 16, 13: 16, 14: 16, 15: 32, 16: 32, 17: 128}
 ACTS = {"relu": ck.Relu, "passthrough": ck.PassThrough}
 
 
