@@ -16,6 +16,7 @@
 #include "gemm_gemm.hpp"
 #include "conv_patch.hpp"
 #include "conv_pointwise.hpp"
+#include "conv_stem.hpp"
 #include "gemm_skinny.hpp"
 #include "gemm_generic.hpp"
 
@@ -708,8 +709,25 @@ bool conv_patch_preferred(int op, const ckx_conv2d_desc* d, int epi)
 
 // ---------------------------------------------------------- weight-stationary pointwise conv kernel
 const char* const kPointwiseName = "MI355X_Mfma16_Pointwise<1x1, C 256/512 bytes, K 512 per workgroup, 8 waves>";
-constexpr int kConvPatchInstance = kNumTiles, kConvPointwiseInstance = kNumTiles + 1, kConvGenericInstance = kNumTiles + 2,
-              kNumConvInsts = kNumTiles + 3;
+constexpr int kConvPatchInstance = kNumTiles, kConvPointwiseInstance = kNumTiles + 1, kConvStemInstance = kNumTiles + 2,
+              kConvGenericInstance = kNumTiles + 3, kNumConvInsts = kNumTiles + 4;
+
+// ---------------------------------------------------------- stem conv kernel (three input channels)
+const char* const kStemName = "MI355X_Mfma16_Stem<7x7, stride 2, pad 3, C 3, K 64, pixels padded to 4 channels in LDS, 4 waves>";
+// the first layer of an image network: C = 3, 7 x 7, stride 2, padding 3 on every side, 64 output channels; the LDS holds
+// the 13 input rows of a band of four output rows
+bool conv_stem_applicable(int op, const ckx_conv2d_desc* d, int epi)
+{
+    const bool epi_ok = op == CKX_OP_CONV2D_FWD_F16 ? (epi == CKX_EPI_PASSTHROUGH || epi == CKX_EPI_ADD_RELU)
+                                                    : (epi == CKX_EPI_PASSTHROUGH || epi == CKX_EPI_REQUANT_CK ||
+                                                       epi == CKX_EPI_REQUANT_RND);
+    if(!((op == CKX_OP_CONV2D_FWD_F16 || op == CKX_OP_CONV2D_FWD_I8) && epi_ok && d->C == 3 && d->K == 64 && d->Y == 7 &&
+         d->X == 7 && d->stride_h == 2 && d->stride_w == 2 && d->dilation_h == 1 && d->dilation_w == 1 && d->pad_top == 3 &&
+         d->pad_left == 3 && d->pad_bottom == 3 && d->pad_right == 3 && d->N >= 1 && d->Ho >= 1 && d->Wo >= 1))
+        return false;
+    const int lds = op == CKX_OP_CONV2D_FWD_I8 ? ckx::ConvStem<ckx::DT_I8>::lds_bytes(d->Wo) : ckx::ConvStem<ckx::DT_F16>::lds_bytes(d->Wo);
+    return lds <= 160 * 1024;
+}
 
 // shapes the pointwise kernel covers: 1x1 filters without padding, a pixel of 256 or 512 bytes, output channels in
 // whole blocks of 512
@@ -785,7 +803,7 @@ int check_conv(int op, const ckx_conv2d_desc* d, int epi, int instance)
     // a 16-byte vector along c must not cross a filter tap
     // (device_conv2d_fwd_xdl_nhwc_kyxc_nhwk.hpp:595-601)
     // (ConvolutionForwardSpecialization::OddC is the element-wise instance; AUTO sends such layers there)
-    if(((long)d->C * es) % 16 && instance != CKX_INSTANCE_AUTO && instance != kConvGenericInstance)
+    if(((long)d->C * es) % 16 && instance != CKX_INSTANCE_AUTO && instance != kConvGenericInstance && instance != kConvStemInstance)
         return fail(CKX_UNSUPPORTED, "C must be a multiple of 16 bytes for this instance (the element-wise instance and AUTO take any)");
     const long in_b  = (long)d->N * d->Hi * d->Wi * d->C * es;
     const long wei_b = (long)d->K * d->Y * d->X * d->C * es;
@@ -795,6 +813,9 @@ int check_conv(int op, const ckx_conv2d_desc* d, int epi, int instance)
         return fail(CKX_UNSUPPORTED, "tensors of 2 GiB or more are not addressed");
     if(instance == kConvPatchInstance && !conv_patch_applicable(op, d, epi))
         return fail(CKX_UNSUPPORTED, "the input-patch instance covers 3x3 stride-1 layers with C = K = 64, Wo = 56");
+    if(instance == kConvStemInstance && !conv_stem_applicable(op, d, epi))
+        return fail(CKX_UNSUPPORTED, "the stem instance covers 7x7 stride-2 layers with C = 3, K = 64 and padding 3, PassThrough / "
+                                     "requant / bias + ReLU epilogues");
     if(instance == kConvPointwiseInstance && !conv_pointwise_applicable(op, d, epi))
         return fail(CKX_UNSUPPORTED, "the pointwise instance covers 1x1 layers without padding, C of 256 or 512 bytes, "
                                      "K a multiple of 512, PassThrough / requant / bias + ReLU epilogues");
@@ -808,7 +829,7 @@ long conv_workspace_bytes(int op, const ckx_conv2d_desc* d, int instance)
     if(M <= 0 || d->K <= 0)
         return 0;
     if(instance == kConvPatchInstance || instance == kConvPointwiseInstance || instance == kConvGenericInstance ||
-       ((long)d->C * es) % 16 ||
+       instance == kConvStemInstance || ((long)d->C * es) % 16 ||
        (instance == CKX_INSTANCE_AUTO &&
         (conv_patch_preferred(op, d, CKX_EPI_PASSTHROUGH) || conv_pointwise_preferred(op, d, CKX_EPI_PASSTHROUGH))))
         return 0;
@@ -831,6 +852,25 @@ int run_conv(int op, const void* in, const void* wei, void* out, const ckx_conv2
     if(!in || !wei || !out)
         return fail(CKX_INVALID_VALUE, "null operand pointer");
     const bool misaligned = ((reinterpret_cast<uintptr_t>(in) | reinterpret_cast<uintptr_t>(wei)) & 15) != 0;
+    // (the stem kernel reads its operands element by element: alignment to the element size is all it asks of them; a bias
+    // row means D0 stride 0)
+    const bool stem_ok = conv_stem_applicable(op, d, epi) && dops.ldd0 == 0 &&
+                         !((reinterpret_cast<uintptr_t>(in) | reinterpret_cast<uintptr_t>(wei) | reinterpret_cast<uintptr_t>(out) |
+                            reinterpret_cast<uintptr_t>(dops.d0)) & (es - 1));
+    if(instance == kConvStemInstance || (instance == CKX_INSTANCE_AUTO && stem_ok))
+    {
+        if(!stem_ok)
+            return fail(CKX_UNSUPPORTED, "the stem instance adds a bias row (D0 row stride 0) only and needs operands aligned to "
+                                         "their element size");
+        ckx::ConvStemArgs a;
+        std::memset(&a, 0, sizeof(a));
+        a.in = in, a.wei = wei, a.out = out, a.bias = dops.d0;
+        a.N = d->N, a.Hi = d->Hi, a.Wi = d->Wi, a.Ho = d->Ho, a.Wo = d->Wo;
+        a.epi = epi, a.scale_gemm = sg, a.scale_relu = sr;
+        a.nt_store   = es == 1 && (long)M * N * es >= stream_output_bytes();
+        hipError_t e = ckx::launch_conv_stem(es == 1 ? ckx::DT_I8 : ckx::DT_F16, a, (hipStream_t)stream);
+        return e == hipSuccess ? CKX_OK : hip_fail(e, kStemName);
+    }
     if(instance == kConvGenericInstance || (instance == CKX_INSTANCE_AUTO && (misaligned || ((long)d->C * es) % 16)))
     {
         if((reinterpret_cast<uintptr_t>(in) | reinterpret_cast<uintptr_t>(wei) | reinterpret_cast<uintptr_t>(out) |
@@ -1133,7 +1173,7 @@ int ckx_num_instances(int op)
     if(op == CKX_OP_GEMM_SPLITK)
         return kNumTiles;
     if(op == CKX_OP_CONV2D_FWD_F16 || op == CKX_OP_CONV2D_FWD_I8)
-        return kNumConvInsts; // + the input-patch, the pointwise and the element-wise kernel
+        return kNumConvInsts; // + the input-patch, the pointwise, the stem and the element-wise kernel
     if(op == CKX_OP_BATCHED_GEMM_GEMM || op == CKX_OP_BATCHED_GEMM_SOFTMAX_GEMM)
         return ckx::kNumGemmGemmInstances;
     return 0;
@@ -1149,7 +1189,8 @@ const char* ckx_instance_name(int op, int instance)
         (op == CKX_OP_BATCHED_GEMM_GEMM || op == CKX_OP_BATCHED_GEMM_SOFTMAX_GEMM
              ? ckx::gemm_gemm_instance_name(instance)
          : (op == CKX_OP_CONV2D_FWD_F16 || op == CKX_OP_CONV2D_FWD_I8) && instance >= kNumTiles
-             ? (instance == kConvPatchInstance ? kPatchName : instance == kConvPointwiseInstance ? kPointwiseName : kGenericName)
+             ? (instance == kConvPatchInstance ? kPatchName : instance == kConvPointwiseInstance ? kPointwiseName
+                : instance == kConvStemInstance ? kStemName : kGenericName)
              : instance == kGenericGemmInstance ? kGenericName
              : instance >= kNumTiles            ? kSkinny[instance - kNumTiles].name
                                                 : kTiles[instance].name) +
@@ -1226,7 +1267,9 @@ int ckx_conv2d_fwd_plan(int op, const ckx_conv2d_desc* d, int epilogue, int64_t 
     *k_runs      = 1;
     if(*instance == CKX_INSTANCE_AUTO)
     {
-        if(((long)d->C * es) % 16)
+        if(conv_stem_applicable(op, d, epilogue))
+            *instance = kConvStemInstance;
+        else if(((long)d->C * es) % 16)
             *instance = kConvGenericInstance;
         else if(conv_patch_preferred(op, d, epilogue))
             *instance = kConvPatchInstance;
