@@ -20,10 +20,10 @@ hipError_t launch_one(const ConvStemArgs& a, hipStream_t s)
     });
     if(attr_err != hipSuccess)
         return attr_err;
-    // bands of TH output rows, walked by at most two workgroups per CU (their registers hold the weights)
+    // bands of TH output rows, walked by two (fp16) or three (int8) workgroups per CU (their registers hold the weights)
     const long units = (long)a.N * ((a.Ho + T::TH - 1) / T::TH);
     int per_cu       = 160 * 1024 / lds;
-    per_cu           = per_cu > 2 ? 2 : per_cu;
+    per_cu           = per_cu > (DT == DT_I8 ? 3 : 2) ? (DT == DT_I8 ? 3 : 2) : per_cu;
     long grid        = (long)num_cus() * per_cu;
     grid             = units < grid ? units : grid;
     hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(T::NTHR), lds, s, a);

@@ -13,7 +13,11 @@
 //     channels permuted so that a lane ends with 16 consecutive channels of one pixel (four lanes = one whole pixel of
 //     64 channels: 128 / 64 contiguous bytes per pixel, 2 / 1 KB per MFMA tile);
 //   * several workgroups per CU overlap one's copy phase with another's MFMAs and stores.
-// Algorithmic traffic is the output (N x 112 x 112 x 64) by far: the layer is bound by HBM writes.
+// Algorithmic traffic is the output (N x 112 x 112 x 64) by far: the layer is bound by HBM writes. Measured at N = 256
+// (timing-only builds, fp16): 148 us; 86 without the input loads (the stores alone, at the write rate of the part);
+// 78 without the stores; 59 without either (MFMAs at 28 per 16 pixels, LDS, barriers). Reads issued into a memory system
+// that is saturated with writes come back late; a variant with a dedicated copy wave per workgroup and two band buffers
+// (no wave both loads and stores) measured the same for fp16 and worse for int8, and was not kept.
 #pragma once
 
 #include "gemm_tile.hpp"
@@ -47,7 +51,12 @@ struct ConvStem
 
     // bytes of an LDS row: windows of 8 padded pixels for every output pixel of the (padded) tile row
     __host__ __device__ static int slot_bytes(int Wo) { return ((Wo + 15) / 16 * 16) * S * PX + 8 * PX; }
-    __host__ __device__ static int lds_bytes(int Wo) { return ROWS * slot_bytes(Wo); }
+    // (the padded weight matrix passes through the same LDS first: 64 rows x 7 (8) filter rows x 32 elements)
+    __host__ __device__ static int lds_bytes(int Wo)
+    {
+        const int band = ROWS * slot_bytes(Wo), weights = KOUT * (DT == DT_I8 ? 8 : 7) * 32 * ES;
+        return band > weights ? band : weights;
+    }
 
     __device__ static __forceinline__ void run(const ConvStemArgs& p, uint8_t* smem)
     {
@@ -61,8 +70,25 @@ struct ConvStem
         const elem_t* in  = reinterpret_cast<const elem_t*>(p.in);
         const elem_t* wei = reinterpret_cast<const elem_t*>(p.wei);
 
-        // ---- the weights as B fragments: N tile t, k-step ks; lane (r, q) holds the 8 (16) K elements 8 q .. (16 q ..)
-        // of LDS-order row 16 t + r, which is output channel b_row_to_col(16 t + r)
+        // ---- the weights as B fragments. First the padded [64][KP] matrix in LDS, K order (y, x', c') with zeros at
+        // x' = 7, c' = 3 (and filter row 7 for int8), filled by all threads with consecutive addresses; then N tile t,
+        // k-step ks: lane (r, q) takes the 16 bytes at K element ks * KE + q * VE of LDS-order row 16 t + r, which is
+        // output channel b_row_to_col(16 t + r). (Fetched from global memory element by element under the validity
+        // test, a lane's 224 loads each took a round trip.)
+        constexpr int KP = (DT == DT_I8 ? 8 : 7) * 32, KE = DT == DT_I8 ? 64 : 32, VE = 16 / ES;
+        {
+            elem_t* wl = reinterpret_cast<elem_t*>(smem);
+#pragma unroll 8
+            for(int i = tid; i < KOUT * KP; i += NTHR)
+            {
+                const int n = i / KP, k = i - n * KP;
+                const int y = k >> 5, x = (k >> 2) & 7, c = k & 3;
+                const bool ok = y < Y && x < X && c < C;
+                const elem_t v = wei[((n * Y + (ok ? y : 0)) * X + (ok ? x : 0)) * C + (ok ? c : 0)];
+                wl[i]          = ok ? v : (elem_t)0;
+            }
+        }
+        __syncthreads();
         i32x4 bfr[4][NKS];
 #pragma unroll
         for(int t = 0; t < 4; ++t)
@@ -70,33 +96,9 @@ struct ConvStem
             const int n = (int)b_row_to_col((uint32_t)(16 * t) + r);
 #pragma unroll
             for(int ks = 0; ks < NKS; ++ks)
-            {
-                if constexpr(DT == DT_F16)
-                {
-                    f16x8 v;
-#pragma unroll
-                    for(int e = 0; e < 8; ++e)
-                    {
-                        const int j = 8 * (int)q + e, x = j >> 2, c = j & 3; // k' = 32 ks + j: filter row ks
-                        v[e]        = (x < X && c < C) ? wei[((n * Y + ks) * X + x) * C + c] : (_Float16)0;
-                    }
-                    bfr[t][ks] = __builtin_bit_cast(i32x4, v);
-                }
-                else
-                {
-                    typedef int8_t i8x16 __attribute__((ext_vector_type(16)));
-                    i8x16 v;
-                    const int y = 2 * ks + ((int)q >> 1); // k' = 64 ks + 16 q + e: filter rows 2 ks, 2 ks + 1
-#pragma unroll
-                    for(int e = 0; e < 16; ++e)
-                    {
-                        const int j = 16 * ((int)q & 1) + e, x = j >> 2, c = j & 3;
-                        v[e]        = (y < Y && x < X && c < C) ? wei[((n * Y + y) * X + x) * C + c] : (int8_t)0;
-                    }
-                    bfr[t][ks] = __builtin_bit_cast(i32x4, v);
-                }
-            }
+                bfr[t][ks] = *reinterpret_cast<const i32x4*>(smem + (n * KP + ks * KE + (int)q * VE) * ES);
         }
+        // (the band copy below starts behind a barrier)
         f32x4 bias[4];
 #pragma unroll
         for(int t = 0; t < 4; ++t)
@@ -112,30 +114,34 @@ struct ConvStem
         {
             const int n = unit / bands, ho0 = (unit - n * bands) * TH;
             const int hi0 = ho0 * S - PAD;
-            // ---- copy the band: padded pixel slot pp of LDS row rr <- input pixel (hi0 + rr, pp - PAD), zeros outside
+            // ---- copy the band: padded pixel slot pp of LDS row rr <- input pixel (hi0 + rr, pp - PAD), zeros outside.
+            // A thread takes one pixel column of all the band's rows: every load is requested before the first LDS write
+            // (row by row, each write behind its own load, the copy took ROWS memory round trips per band: 219 us for the
+            // layer against 157).
             const int npx = slot / PX;
             __syncthreads(); // (every wave is done with the previous band)
-            for(int i = tid; i < ROWS * npx; i += NTHR)
+            for(int pp = tid; pp < npx; pp += NTHR)
             {
-                const int rr = i / npx, pp = i - rr * npx;
-                const int hi = hi0 + rr, wi = pp - PAD;
-                const bool ok = hi >= 0 && hi < p.Hi && wi >= 0 && wi < p.Wi;
-                const elem_t* src = in + ((size_t)(n * p.Hi + (ok ? hi : 0)) * p.Wi + (ok ? wi : 0)) * C;
-                if constexpr(DT == DT_F16)
+                const int wi     = pp - PAD;
+                const bool wi_ok = wi >= 0 && wi < p.Wi;
+                struct __attribute__((packed, aligned(ES))) px3
                 {
-                    typedef _Float16 f16x4 __attribute__((ext_vector_type(4)));
-                    f16x4 v = {0, 0, 0, 0};
-                    if(ok)
-                        v[0] = src[0], v[1] = src[1], v[2] = src[2];
-                    *reinterpret_cast<f16x4*>(smem + rr * slot + pp * PX) = v;
+                    elem_t c[3];
+                };
+                px3 v[ROWS];
+#pragma unroll
+                for(int rr = 0; rr < ROWS; ++rr)
+                {
+                    const int hi  = hi0 + rr;
+                    const bool ok = wi_ok && hi >= 0 && hi < p.Hi;
+                    const px3* src = reinterpret_cast<const px3*>(in + ((size_t)(n * p.Hi + (ok ? hi : 0)) * p.Wi + (ok ? wi : 0)) * C);
+                    v[rr]          = ok ? *src : px3{{(elem_t)0, (elem_t)0, (elem_t)0}};
                 }
-                else
+#pragma unroll
+                for(int rr = 0; rr < ROWS; ++rr)
                 {
-                    typedef int8_t i8x4 __attribute__((ext_vector_type(4)));
-                    i8x4 v = {0, 0, 0, 0};
-                    if(ok)
-                        v[0] = src[0], v[1] = src[1], v[2] = src[2];
-                    *reinterpret_cast<i8x4*>(smem + rr * slot + pp * PX) = v;
+                    typedef elem_t ex4 __attribute__((ext_vector_type(4)));
+                    *reinterpret_cast<ex4*>(smem + rr * slot + pp * PX) = ex4{v[rr].c[0], v[rr].c[1], v[rr].c[2], (elem_t)0};
                 }
             }
             __syncthreads();
@@ -209,7 +215,7 @@ struct ConvStem
 };
 
 template <int DT>
-__global__ __launch_bounds__(256, 2) void conv_stem_kernel(const ConvStemArgs p)
+__global__ __launch_bounds__(256, DT == DT_I8 ? 3 : 2) void conv_stem_kernel(const ConvStemArgs p)
 {
     extern __shared__ __attribute__((aligned(16))) uint8_t ckx_smem[];
     ConvStem<DT>::run(p, ckx_smem);
