@@ -310,14 +310,35 @@ def _sclk_under_load(chunk, chunk_ms, busy_ms=1500.0):
     return seen
 
 
+def vendor_launcher(w):
+    """The vendor library's kernel for the same problem on operands of the same distribution, for the figure
+    beside the headline rows: torch.matmul (hipBLASLt) for fp16, torch._int_mm for int8 (int32 output: it does
+    not requantize, so it writes four times the C bytes of the int8 row)."""
+    import torch
+    from composable_kernel_amd.host_tensor import uniform_f16, uniform_int8
+    M, N, K = w["M"], w["N"], w["K"]
+    if w["dtype"] == "f16":
+        a = torch.from_numpy(uniform_f16((M, K), -1, 1, 1)).cuda()
+        bt = torch.from_numpy(uniform_f16((N, K), -1, 1, 2)).cuda().t()
+        c = torch.empty((M, N), dtype=torch.float16, device="cuda")
+        fn = lambda: torch.matmul(a, bt, out=c)
+    else:
+        a = torch.from_numpy(uniform_int8((M, K), -5, 5, 1)).cuda()
+        bt = torch.from_numpy(uniform_int8((N, K), -5, 5, 2)).cuda().t()
+        c = torch.empty((M, N), dtype=torch.int32, device="cuda")
+        fn = lambda: torch._int_mm(a, bt, out=c)
+    fn.keep = [a, bt, c]
+    return fn
+
+
 def time_workload(w, steps, warmup, instance=-1, use_graph=True, rotate=1, settle_ms=300.0, from_idle=False,
-                  sample_clock=False):
+                  sample_clock=False, launch=None):
     """[from_idle: 1 + 10 eager launches first], clock settling, W untimed launches, then exactly K timed
     ones. The K launches are replayed from a HIP graph (captured once from the same C-ABI calls) so that
     kernels run back to back on the GPU even when one kernel is shorter than a Python call;
     use_graph=False launches eagerly."""
     import torch
-    launch = make_launcher(w, instance, rotate)
+    launch = launch or make_launcher(w, instance, rotate)
     torch.cuda.synchronize()
     e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     idle = None
@@ -610,6 +631,13 @@ def main():
                     help="instead of the headline: the ResNet-50 layers of the reference's whole-network script "
                          "(script/profile_resnet50.sh) at N = 256, fp16 and int8, plain and fused; one JSON line with a "
                          "row per layer, a table on stderr")
+    ap.add_argument("--no-clock", action="store_true",
+                    help="do not read the engine clock after the timed region (the reading starts rocm-smi as a child "
+                         "process, which a counter-collecting profiler around this program does not allow; left out "
+                         "by itself when LD_PRELOAD names a profiler library)")
+    ap.add_argument("--vendor", action="store_true",
+                    help="also time the vendor library on the headline shapes with the same protocol, in the same "
+                         "process (torch.matmul for fp16, torch._int_mm for int8), reported under 'vendor'")
     ap.add_argument("--copy-probe", action="store_true",
                     help="also run one 256 MiB device-to-device copy (a kernel of known traffic, used to "
                          "scale the FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run)")
@@ -634,8 +662,9 @@ def main():
     if args.resnet50:
         return resnet50_sweep(args)
     w = WORKLOADS[args.workload]
+    profiled = "rocprof" in os.environ.get("LD_PRELOAD", "") or any(k.startswith("ROCPROF") for k in os.environ)
     r = time_workload(w, args.steps, args.warmup, args.instance, not args.no_graph, settle_ms=args.settle_ms,
-                      from_idle=True, sample_clock=True)
+                      from_idle=True, sample_clock=not (args.no_clock or profiled))
     also = []
     extra = ["int8_requant_gemm_4096"] if args.workload == "fp16_gemm_4096" else []
     if args.all:
@@ -695,6 +724,19 @@ def main():
                       "frac": round(max(idle["mfma_frac"], idle["hbm_frac"]), 4)},
         "also": also,
     }
+    if args.vendor:
+        line["vendor"] = []
+        for n in [args.workload] + [x for x in extra if x in ("fp16_gemm_4096", "int8_requant_gemm_4096")]:
+            wl = WORKLOADS[n]
+            if wl["kind"] != "gemm" or wl.get("G", 1) > 1 or wl.get("fused") or wl["dtype"] not in ("f16", "i8"):
+                continue
+            # ours again right before the vendor's, so that both see the same clock state of the same box
+            ours = time_workload(wl, args.steps, args.warmup, -1, not args.no_graph, settle_ms=args.settle_ms)
+            v = time_workload(wl, args.steps, args.warmup, -1, not args.no_graph, settle_ms=args.settle_ms,
+                              launch=vendor_launcher(wl))
+            line["vendor"].append({"workload": n, "call": "torch.matmul" if wl["dtype"] == "f16" else "torch._int_mm (int32 C)",
+                                   "vendor_ms": round(v["ms"], 5), "ours_ms": round(ours["ms"], 5),
+                                   "ours_over_vendor": round(ours["ms"] / v["ms"], 4)})
     if not args.no_cpu:
         line["cpu_baseline"] = cpu_baseline(w, args.cpu_threads or None)
     print(json.dumps(line))

@@ -104,6 +104,29 @@ def w4_register_faults(compiler_output):
     return bad
 
 
+# conv_patch_kernel: the AccVGPRs hold exactly the wave's 36 weight fragments
+PATCH_AGPRS = 144
+
+
+def patch_register_faults(compiler_output):
+    """(kernel, what) for every conv_patch_kernel of the resource-usage report that uses scratch memory or does not keep
+    its weights -- and nothing else -- in AccVGPRs."""
+    bad, name = [], None
+    for line in compiler_output.splitlines():
+        if "Function Name:" in line:
+            name = line.split("Function Name:", 1)[1].split("[", 1)[0].strip()
+            name = name if "conv_patch_kernel" in name else None
+        elif name and "ScratchSize [bytes/lane]:" in line:
+            n = int(line.split("ScratchSize [bytes/lane]:", 1)[1].split("[", 1)[0])
+            if n:
+                bad.append((name, f"{n} bytes of scratch per lane"))
+        elif name and "AGPRs:" in line:
+            n = int(line.split("AGPRs:", 1)[1].split("[", 1)[0])
+            if n != PATCH_AGPRS:
+                bad.append((name, f"{n} AccVGPRs"))
+    return bad
+
+
 def sources():
     return [os.path.join(CSRC, f) for f in sorted(os.listdir(CSRC))]
 
@@ -135,6 +158,7 @@ def build_lib(force=False, verbose=False, extra_flags=()):
         # the register report: keep it out of the log, fail on vector register spills
         spills = vgpr_spills(r.stdout)
         w4_bad = w4_register_faults(r.stdout)
+        patch_bad = patch_register_faults(r.stdout)
         out, skip = [], 0
         for l in lines:
             if "[-Rpass-analysis=kernel-resource-usage]" in l:
@@ -153,6 +177,9 @@ def build_lib(force=False, verbose=False, extra_flags=()):
         if w4_bad:
             raise RuntimeError("four-wave GEMM body: register allocation differs from what its inline assembly assumes: "
                                + ", ".join(f"{k}: {what}" for k, what in w4_bad))
+        if patch_bad:
+            raise RuntimeError("input-patch conv kernel: register allocation differs from what its inline assembly assumes: "
+                               + ", ".join(f"{k}: {what}" for k, what in patch_bad))
         if verbose and out.strip():
             print(out)
 

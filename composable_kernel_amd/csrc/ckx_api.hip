@@ -754,24 +754,6 @@ bool conv_pointwise_preferred(int op, const ckx_conv2d_desc* d, int epi)
     return conv_pointwise_applicable(op, d, epi) && px >= (op == CKX_OP_CONV2D_FWD_I8 ? 16 * 1024 : 40 * 1024);
 }
 
-template <int DT, bool FUSED>
-hipError_t launch_conv_patch(const ckx::ConvPatchArgs& a, hipStream_t s)
-{
-    using T    = ckx::ConvPatch<DT, 7, 3, 3, FUSED>;
-    auto* kern = &ckx::conv_patch_kernel<DT, 7, 3, 3, FUSED>;
-    static std::once_flag once;
-    static hipError_t attr_err = hipSuccess;
-    std::call_once(once, [&] {
-        attr_err = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, T::LDS);
-    });
-    if(attr_err != hipSuccess)
-        return attr_err;
-    const int grid = a.N < num_cus() ? a.N : num_cus();
-    hipLaunchKernelGGL(kern, dim3(grid), dim3(T::NT), T::LDS, s, a);
-    return hipGetLastError();
-}
-
 int check_conv(int op, const ckx_conv2d_desc* d, int epi, int instance)
 {
     if(!d)
@@ -914,16 +896,15 @@ int run_conv(int op, const void* in, const void* wei, void* out, const ckx_conv2
         a.in = in, a.wei = wei, a.out = out;
         a.in_bytes  = (uint32_t)((long)d->N * d->Hi * d->Wi * d->C * es);
         a.wei_bytes = (uint32_t)((long)N * K * es);
+        a.out_bytes = (uint32_t)((long)d->N * d->Ho * d->Wo * d->K * es);
         a.N = d->N, a.Hi = d->Hi, a.Wi = d->Wi, a.Ho = d->Ho, a.Wo = d->Wo;
         a.pT = d->pad_top, a.pL = d->pad_left;
         a.div_wo = make_magic((uint32_t)d->Wo);
         a.epi    = epi;
         a.bias = dops.d0, a.resi = epi == CKX_EPI_ADD_RELU_ADD ? dops.d1 : nullptr;
         a.scale_gemm = sg, a.scale_relu = sr;
-        hipError_t e = es == 1 && per_column_scale(epi) ? launch_conv_patch<ckx::DT_I8, true>(a, (hipStream_t)stream)
-                       : es == 1                     ? launch_conv_patch<ckx::DT_I8, false>(a, (hipStream_t)stream)
-                       : epi == CKX_EPI_PASSTHROUGH ? launch_conv_patch<ckx::DT_F16, false>(a, (hipStream_t)stream)
-                                                    : launch_conv_patch<ckx::DT_F16, true>(a, (hipStream_t)stream);
+        const bool fused = es == 1 ? per_column_scale(epi) : epi != CKX_EPI_PASSTHROUGH;
+        hipError_t e     = ckx::launch_conv_patch(es == 1 ? ckx::DT_I8 : ckx::DT_F16, fused, a, (hipStream_t)stream);
         return e == hipSuccess ? CKX_OK : hip_fail(e, kPatchName);
     }
     if(instance == kConvPointwiseInstance ||

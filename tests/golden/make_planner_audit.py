@@ -23,9 +23,14 @@ sys.path.insert(0, ROOT)
 
 GEMM_NK = [(11008, 4096), (4096, 11008), (4096, 4096), (2048, 2048), (1024, 1024), (1024, 8192), (16384, 1024)]
 GEMM_M = [1, 8, 16, 32, 48, 64, 128, 256, 512, 1024, 4096]
-# (C, K, filter, HW, stride, pad) at N = 32 and 256: the benchmark's three layers and four more ResNet-50 shapes
+# (C, K, filter, HW, stride, pad) at N = 32 and 256: the benchmark's three layers, one more strided pointwise layer and
+# the twenty distinct layers of the reference's whole-network run (script/profile_resnet50.sh:24-46)
 CONV = [(64, 64, 3, 56, 1, 1), (256, 512, 1, 56, 2, 0), (512, 512, 3, 7, 1, 1), (128, 128, 3, 28, 1, 1),
-        (256, 256, 3, 14, 1, 1), (64, 256, 1, 56, 1, 0), (1024, 2048, 1, 14, 2, 0)]
+        (256, 256, 3, 14, 1, 1), (64, 256, 1, 56, 1, 0), (1024, 2048, 1, 14, 2, 0),
+        (1024, 256, 1, 14, 1, 0), (1024, 512, 1, 14, 1, 0), (128, 512, 1, 28, 1, 0), (128, 128, 3, 56, 2, 1),
+        (2048, 512, 1, 7, 1, 0), (256, 1024, 1, 14, 1, 0), (256, 256, 3, 28, 2, 1), (256, 128, 1, 56, 1, 0),
+        (512, 512, 3, 14, 2, 1), (512, 128, 1, 28, 1, 0), (512, 256, 1, 28, 1, 0), (512, 2048, 1, 7, 1, 0),
+        (64, 64, 1, 56, 1, 0), (256, 64, 1, 56, 1, 0), (3, 64, 7, 224, 2, 3)]
 
 
 def time_launch(launch, block_ms=8.0, max_settle_ms=400.0):
@@ -93,6 +98,9 @@ def main():
         out["updated"] = "columns " + (args.instances or "all") + " of the GEMM rows re-measured with this library"
     ws = torch.empty(256 << 20, dtype=torch.uint8, device="cuda")
     only = set(args.only.split(","))
+    if not args.update and not only & {"i8", "f16"} and os.path.exists(os.path.join(HERE, "planner_audit.json")):
+        with open(os.path.join(HERE, "planner_audit.json")) as f:   # a conv-only run keeps the GEMM rows it finds
+            out["gemm"] = json.load(f)["gemm"]
     grid = [(kind, M, N, K) for kind in ("i8", "f16") if kind in only for (N, K) in GEMM_NK for M in GEMM_M]
     if args.quick:
         grid = grid[::5]

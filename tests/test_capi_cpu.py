@@ -127,6 +127,18 @@ conv_patch.hpp:410:1: remark: Function Name: _ZN3ckx17conv_patch_kernelILi1EEEvN
 conv_patch.hpp:410:1: remark:     VGPRs Spill: 0 [-Rpass-analysis=kernel-resource-usage]
 """
     assert build.vgpr_spills(report) == [("_ZN3ckx16gemm_tile_kernelILi0ELi256ELi256EEvNS_8GemmArgsE", 7)]
+    # the input-patch conv kernel keeps its weights, and nothing else, in AccVGPRs, and has no scratch
+    patch = """
+conv_patch.hpp:500:1: remark: Function Name: _ZN3ckx17conv_patch_kernelILi1ELi7ELb0EEEvNS_13ConvPatchArgsE [-Rpass-analysis=kernel-resource-usage]
+conv_patch.hpp:500:1: remark:     AGPRs: 144 [-Rpass-analysis=kernel-resource-usage]
+conv_patch.hpp:500:1: remark:     ScratchSize [bytes/lane]: 0 [-Rpass-analysis=kernel-resource-usage]
+conv_patch.hpp:500:1: remark: Function Name: _ZN3ckx17conv_patch_kernelILi0ELi7ELb0EEEvNS_13ConvPatchArgsE [-Rpass-analysis=kernel-resource-usage]
+conv_patch.hpp:500:1: remark:     AGPRs: 200 [-Rpass-analysis=kernel-resource-usage]
+conv_patch.hpp:500:1: remark:     ScratchSize [bytes/lane]: 16 [-Rpass-analysis=kernel-resource-usage]
+"""
+    assert build.patch_register_faults(patch) == [
+        ("_ZN3ckx17conv_patch_kernelILi0ELi7ELb0EEEvNS_13ConvPatchArgsE", "200 AccVGPRs"),
+        ("_ZN3ckx17conv_patch_kernelILi0ELi7ELb0EEEvNS_13ConvPatchArgsE", "16 bytes of scratch per lane")]
     assert "-Rpass-analysis=kernel-resource-usage" in build.DEVICE_FLAGS
     assert "clang version" in build.compiler_version()
     assert all("clang version" in v for v in build.VALIDATED_COMPILERS)
