@@ -633,8 +633,7 @@ def main():
                          "row per layer, a table on stderr")
     ap.add_argument("--no-clock", action="store_true",
                     help="do not read the engine clock after the timed region (the reading starts rocm-smi as a child "
-                         "process, which a counter-collecting profiler around this program does not allow; left out "
-                         "by itself when LD_PRELOAD names a profiler library)")
+                         "process, which a counter-collecting profiler around this program does not allow)")
     ap.add_argument("--vendor", action="store_true",
                     help="also time the vendor library on the headline shapes with the same protocol, in the same "
                          "process (torch.matmul for fp16, torch._int_mm for int8), reported under 'vendor'")
@@ -662,9 +661,8 @@ def main():
     if args.resnet50:
         return resnet50_sweep(args)
     w = WORKLOADS[args.workload]
-    profiled = "rocprof" in os.environ.get("LD_PRELOAD", "") or any(k.startswith("ROCPROF") for k in os.environ)
     r = time_workload(w, args.steps, args.warmup, args.instance, not args.no_graph, settle_ms=args.settle_ms,
-                      from_idle=True, sample_clock=not (args.no_clock or profiled))
+                      from_idle=True, sample_clock=not args.no_clock)
     also = []
     extra = ["int8_requant_gemm_4096"] if args.workload == "fp16_gemm_4096" else []
     if args.all:

@@ -209,10 +209,12 @@ int splitk_runs(int kbytes, int k_batch)
 
 // k_batch > 0: the caller fixed the number of K runs (DeviceGemmSplitK's KBatch)
 // kmajor: a K-major operand (A column-major / B row-major) -- only the tiles of 64 rows and more
-// conv: A is gathered (im2col): the 8-wave 256 x 64 tile measures ahead of the 128 x 64 one there by 10 - 17 %
-// (ResNet-like layers at N = 32 and 256), which the GEMM-calibrated figures did not say
+// conv: A is gathered (im2col); taps > 1: with several filter taps the 8-wave 256 x 64 tile measures ahead of the
+// 128 x 64 one by 10 - 17 % (ResNet-like layers at N = 32 and 256), which the GEMM-calibrated figures did not say; the
+// 1 x 1 layers of the same networks follow the GEMM figures (256 x 64 rated up sent C 256 -> K 128 at 56 x 56 to it, 20 %
+// behind the 256 x 128 tile)
 Plan make_plan(long M, int N, int kbytes, int only_tile, long workspace_bytes, int k_batch = 0, bool kmajor = false,
-               bool conv = false)
+               bool conv = false, int taps = 2)
 {
     Plan best;
     double best_us  = 1e30;
@@ -243,7 +245,7 @@ Plan make_plan(long M, int N, int kbytes, int only_tile, long workspace_bytes, i
             const long rounds = (units + cus * per_cu - 1) / (cus * per_cu);
             // one K-tile iteration costs its MFMA time, but never less than the barrier + load
             // latency of the two-stage pipeline (~0.42 us measured on small tiles)
-            const double eff = conv && t.bm == 256 && t.bn == 64 ? t.eff * 1.1 : t.eff;
+            const double eff = conv && taps > 1 && t.bm == 256 && t.bn == 64 ? t.eff * 1.1 : t.eff;
             double iter_us   = per_cu * (t.bm * t.bn / 65536.0) / eff * 1.1;
             const int nst  = t.lds / ((t.bm + t.bn) * 128);
             const double floor_us = nst > 2 ? 0.30 : 0.42; // (four stages: 0.33 measured over 32 K tiles, 0.26 over 64)
@@ -686,7 +688,7 @@ int run_gemm(int dt, const void* a, const void* b, void* c, int M, int N, int K,
 }
 
 // ---------------------------------------------------------- input-patch conv kernel
-const char* const kPatchName = "MI355X_Mfma16_Patch<rows x 56, 3x3, C 64, K 64, 4 waves>";
+const char* const kPatchName = "MI355X_Mfma16_Patch<rows x 56, 3x3, C 64, K 64, weights in AccVGPRs, 4 waves>";
 
 // shapes the input-patch kernel covers (one instantiation per data type: 3x3 taps, Wo = 56)
 bool conv_patch_applicable(int op, const ckx_conv2d_desc* d, int epi)
@@ -815,7 +817,7 @@ long conv_workspace_bytes(int op, const ckx_conv2d_desc* d, int instance)
        (instance == CKX_INSTANCE_AUTO &&
         (conv_patch_preferred(op, d, CKX_EPI_PASSTHROUGH) || conv_pointwise_preferred(op, d, CKX_EPI_PASSTHROUGH))))
         return 0;
-    const Plan pl = make_plan((int)M, d->K, d->Y * d->X * d->C * es, instance, 1l << 60, 0, false, true);
+    const Plan pl = make_plan((int)M, d->K, d->Y * d->X * d->C * es, instance, 1l << 60, 0, false, true, d->Y * d->X);
     return pl.ksplit > 1 ? (long)pl.ksplit * M * d->K * 4 : 0;
 }
 
@@ -930,7 +932,7 @@ int run_conv(int op, const void* in, const void* wei, void* out, const ckx_conv2
                                                   (hipStream_t)stream);
         return e == hipSuccess ? CKX_OK : hip_fail(e, kPointwiseName);
     }
-    const Plan pl = make_plan(M, N, K * es, instance, ws ? ws_bytes : 0, 0, false, true);
+    const Plan pl = make_plan(M, N, K * es, instance, ws ? ws_bytes : 0, 0, false, true, d->Y * d->X);
     const TileInstance& t = kTiles[pl.tile];
     ckx::GemmArgs g;
     std::memset(&g, 0, sizeof(g));
@@ -1260,7 +1262,7 @@ int ckx_conv2d_fwd_plan(int op, const ckx_conv2d_desc* d, int epilogue, int64_t 
     if(*instance == CKX_INSTANCE_AUTO || *instance < kNumTiles)
     {
         const Plan pl = make_plan((long)d->N * d->Ho * d->Wo, d->K, d->Y * d->X * d->C * es, *instance,
-                                  workspace_bytes > 0 ? workspace_bytes : 0, 0, false, true);
+                                  workspace_bytes > 0 ? workspace_bytes : 0, 0, false, true, d->Y * d->X);
         *instance = pl.tile, *k_runs = pl.ksplit;
     }
     return CKX_OK;
