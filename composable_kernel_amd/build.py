@@ -60,7 +60,7 @@ def check_compiler():
 
 
 # kernels whose LDS fragment reads are inline assembly waited for by hand (mangled-name fragments)
-HAND_WAITED_KERNELS = ("gemm_tile_kernel", "gemm_w4_kernel", "gemm_astream_kernel", "conv_patch_kernel",
+HAND_WAITED_KERNELS = ("gemm_tile_kernel", "gemm_w4_kernel", "gemm_astream_kernel", "conv_patch_kernel", "conv_patch_wide_kernel",
                        "conv_pointwise_kernel")
 
 
@@ -115,14 +115,16 @@ def patch_register_faults(compiler_output):
     for line in compiler_output.splitlines():
         if "Function Name:" in line:
             name = line.split("Function Name:", 1)[1].split("[", 1)[0].strip()
-            name = name if "conv_patch_kernel" in name else None
+            name = name if "conv_patch_kernel" in name or "conv_patch_wide_kernel" in name else None
         elif name and "ScratchSize [bytes/lane]:" in line:
             n = int(line.split("ScratchSize [bytes/lane]:", 1)[1].split("[", 1)[0])
             if n:
                 bad.append((name, f"{n} bytes of scratch per lane"))
         elif name and "AGPRs:" in line:
             n = int(line.split("AGPRs:", 1)[1].split("[", 1)[0])
-            if n != PATCH_AGPRS:
+            # (the 128-channel kernel: 32 of the 36 fp16 fragments, all 18 int8 ones)
+            want = PATCH_AGPRS if "conv_patch_kernel" in name else (72 if "kernelILi0E" in name else 128)
+            if n != want:
                 bad.append((name, f"{n} AccVGPRs"))
     return bad
 

@@ -15,6 +15,7 @@
 #include "tile_launch.hpp"
 #include "gemm_gemm.hpp"
 #include "conv_patch.hpp"
+#include "conv_patch_wide.hpp"
 #include "conv_pointwise.hpp"
 #include "conv_stem.hpp"
 #include "gemm_skinny.hpp"
@@ -688,11 +689,23 @@ int run_gemm(int dt, const void* a, const void* b, void* c, int M, int N, int K,
 }
 
 // ---------------------------------------------------------- input-patch conv kernel
-const char* const kPatchName = "MI355X_Mfma16_Patch<rows x 56, 3x3, C 64, K 64, weights in AccVGPRs, 4 waves>";
+const char* const kPatchName = "MI355X_Mfma16_Patch<3x3, C = K = 64 rows x 56 (4 waves) or C = K = 128 rows x 28 (8 waves), weights in AccVGPRs>";
 
-// shapes the input-patch kernel covers (one instantiation per data type: 3x3 taps, Wo = 56)
+// the second shape of the instance (conv_patch_wide.hpp): C = K = 128, Wo = 28; plain epilogues and fp16 bias + ReLU
+bool conv_patch_wide_applicable(int op, const ckx_conv2d_desc* d, int epi)
+{
+    const bool epi_ok = op == CKX_OP_CONV2D_FWD_F16 ? (epi == CKX_EPI_PASSTHROUGH || epi == CKX_EPI_ADD_RELU)
+                                                    : (epi == CKX_EPI_PASSTHROUGH || epi == CKX_EPI_REQUANT_CK || epi == CKX_EPI_REQUANT_RND);
+    return (op == CKX_OP_CONV2D_FWD_F16 || op == CKX_OP_CONV2D_FWD_I8) && epi_ok && d->C == 128 && d->K == 128 && d->Y == 3 &&
+           d->X == 3 && d->stride_h == 1 && d->stride_w == 1 && d->dilation_h == 1 && d->dilation_w == 1 &&
+           d->Wo == 28 && d->Ho >= 1 && d->N >= 1 && d->pad_left <= 2 && d->pad_top <= 2;
+}
+
+// shapes the input-patch kernels cover (one instantiation per data type and shape: 3x3 taps, Wo = 56 / 28)
 bool conv_patch_applicable(int op, const ckx_conv2d_desc* d, int epi)
 {
+    if(conv_patch_wide_applicable(op, d, epi))
+        return true;
     const bool epi_ok = op == CKX_OP_CONV2D_FWD_F16
                             ? (epi == CKX_EPI_PASSTHROUGH || epi == CKX_EPI_ADD_RELU || epi == CKX_EPI_ADD_RELU_ADD)
                             : (epi == CKX_EPI_PASSTHROUGH || epi == CKX_EPI_REQUANT_CK || epi == CKX_EPI_REQUANT_RND ||
@@ -796,7 +809,8 @@ int check_conv(int op, const ckx_conv2d_desc* d, int epi, int instance)
        (long)d->N * d->Ho * d->Wo >= (1l << 31))
         return fail(CKX_UNSUPPORTED, "tensors of 2 GiB or more are not addressed");
     if(instance == kConvPatchInstance && !conv_patch_applicable(op, d, epi))
-        return fail(CKX_UNSUPPORTED, "the input-patch instance covers 3x3 stride-1 layers with C = K = 64, Wo = 56");
+        return fail(CKX_UNSUPPORTED, "the input-patch instance covers 3x3 stride-1 layers with C = K = 64, Wo = 56 or C = K = 128, Wo = 28 "
+                                     "(the latter with PassThrough / requant / bias + ReLU epilogues)");
     if(instance == kConvStemInstance && !conv_stem_applicable(op, d, epi))
         return fail(CKX_UNSUPPORTED, "the stem instance covers 7x7 stride-2 layers with C = 3, K = 64 and padding 3, PassThrough / "
                                      "requant / bias + ReLU epilogues");
@@ -906,7 +920,8 @@ int run_conv(int op, const void* in, const void* wei, void* out, const ckx_conv2
         a.bias = dops.d0, a.resi = epi == CKX_EPI_ADD_RELU_ADD ? dops.d1 : nullptr;
         a.scale_gemm = sg, a.scale_relu = sr;
         const bool fused = es == 1 ? per_column_scale(epi) : epi != CKX_EPI_PASSTHROUGH;
-        hipError_t e     = ckx::launch_conv_patch(es == 1 ? ckx::DT_I8 : ckx::DT_F16, fused, a, (hipStream_t)stream);
+        hipError_t e     = d->C == 128 ? ckx::launch_conv_patch_wide(es == 1 ? ckx::DT_I8 : ckx::DT_F16, fused, a, (hipStream_t)stream)
+                                       : ckx::launch_conv_patch(es == 1 ? ckx::DT_I8 : ckx::DT_F16, fused, a, (hipStream_t)stream);
         return e == hipSuccess ? CKX_OK : hip_fail(e, kPatchName);
     }
     if(instance == kConvPointwiseInstance ||

@@ -245,6 +245,71 @@ def test_conv2d_int8_input_patch_kernel_full_range_and_many_images():
     np.testing.assert_array_equal(out, fast.conv2d_fwd_i8(inp, wei, (1, 1), (1, 1), (1, 1)))
 
 
+# (N, Hi, Wi, pads): C = K = 128, 3x3, stride 1, dilation 1, Wo = 28 -- the second shape of the input-patch instance
+# (ResNet-50 conv3_x: eight waves that share the pixels, weights in registers)
+PATCH_WIDE = [
+    (2, 9, 28, (1, 1)),       # partial last band (Ho = 9)
+    (1, 4, 28, (1, 1)),       # a single band
+    (3, 12, 30, (1, 0)),      # no horizontal padding
+    (2, 7, 26, (0, 2)),       # wide horizontal padding, none vertically (Ho = 5)
+    (1, 28, 28, (1, 1)),      # the ResNet-50 conv3_x layer, one image (seven bands: the ring wraps, its first rows are loaded twice)
+    (2, 70, 28, (1, 1)),      # eighteen bands: every ring position several times
+]
+
+
+@pytest.mark.parametrize("case", PATCH_WIDE)
+def test_conv2d_fp16_input_patch_kernel_128_channels(case):
+    """The 128-channel form of the input-patch instance against the literal oracle (sampled images for the tall case);
+    the tile kernel must agree on the same problem."""
+    import gpu_util
+    N, Hi, Wi, p = case
+    inp = uniform_f16((N, Hi, Wi, 128), -1, 1, 700 + Hi)
+    wei = uniform_f16((128, 3, 3, 128), -1, 1, 701 + Wi)
+    patch = gpu_util.conv_instance(capi.OP_CONV2D_FWD_F16, "Patch")
+    out = gpu_util.conv2d_fwd(inp, wei, (1, 1), (1, 1), p, instance=patch)
+    ref = fast.conv2d_fwd_f16(inp, wei, (1, 1), (1, 1), p) if Hi > 30 else lit.conv2d_fwd(inp, wei, (1, 1), (1, 1), p)
+    assert out.shape == ref.shape and out.shape[2] == 28
+    _f16_close(out, ref)
+    _f16_close(gpu_util.conv2d_fwd(inp, wei, (1, 1), (1, 1), p, instance=7), ref)
+
+
+@pytest.mark.parametrize("case", PATCH_WIDE)
+def test_conv2d_int8_input_patch_kernel_128_channels_bit_exact(case):
+    """... int8: PassThrough (low byte) and both requant epilogues, bit for bit."""
+    import gpu_util
+    N, Hi, Wi, p = case
+    inp = uniform_int8((N, Hi, Wi, 128), -5, 5, 750 + Hi)
+    wei = uniform_int8((128, 3, 3, 128), -5, 5, 751 + Wi)
+    patch = gpu_util.conv_instance(capi.OP_CONV2D_FWD_I8, "Patch")
+    out = gpu_util.conv2d_fwd(inp, wei, (1, 1), (1, 1), p, instance=patch)
+    np.testing.assert_array_equal(out, fast.conv2d_fwd_i8(inp, wei, (1, 1), (1, 1), p))
+    for rq, kind in ((ck.RequantReluRequant(0.02, 0.7, rounded=True), lit.EPI_REQUANT_RND),
+                     (ck.RequantReluRequant(0.015, 1.0), lit.EPI_REQUANT_CK)):
+        out = gpu_util.conv2d_fwd(inp, wei, (1, 1), (1, 1), p, out_op=rq, instance=patch)
+        ref = gpu_util.conv2d_fwd(inp, wei, (1, 1), (1, 1), p, out_op=rq, instance=7)
+        np.testing.assert_array_equal(out, ref)
+        if Hi <= 12:
+            np.testing.assert_array_equal(out, lit.conv2d_fwd(inp, wei, (1, 1), (1, 1), p, epi=kind, scale_gemm=rq.scale_gemm,
+                                                              scale_relu=rq.scale_relu))
+        assert out.max() > 0
+
+
+def test_conv2d_input_patch_kernel_128_channels_many_images_and_automatic_choice():
+    """More images than workgroups, through the automatic choice (which takes the instance from 112 images on); integer
+    fp16 operands make the fp32 sums exact, so the result must equal the rounded exact product."""
+    import gpu_util
+    inp = uniform_int8((300, 5, 28, 128), -3, 3, 97)
+    wei = uniform_int8((128, 3, 3, 128), -3, 3, 98)
+    d = capi.Conv2dDesc(300, 128, 128, 5, 28, 3, 3, 5, 28, 1, 1, 1, 1, 1, 1, 1, 1)
+    patch = gpu_util.conv_instance(capi.OP_CONV2D_FWD_I8, "Patch")
+    assert capi.conv2d_fwd_plan(capi.OP_CONV2D_FWD_I8, d, capi.EPI_PASSTHROUGH, 0)[0] == patch
+    np.testing.assert_array_equal(gpu_util.conv2d_fwd(inp, wei, (1, 1), (1, 1), (1, 1)),
+                                  fast.conv2d_fwd_i8(inp, wei, (1, 1), (1, 1), (1, 1)))
+    out = gpu_util.conv2d_fwd(inp.astype(np.float16), wei.astype(np.float16), (1, 1), (1, 1), (1, 1))
+    exact = fast.conv2d_fwd_f16(inp.astype(np.float16), wei.astype(np.float16), (1, 1), (1, 1), (1, 1))
+    np.testing.assert_array_equal(out, exact)
+
+
 # (N, C, K, Hi, Wi, strides): 1x1 filters, no padding, a pixel of 256 or 512 bytes, K in blocks of 512 -- the
 # weight-stationary pointwise kernel's shapes (the reference's Filter1x1Pad0 / Filter1x1Stride1Pad0 specialisations)
 POINTWISE_F16 = [

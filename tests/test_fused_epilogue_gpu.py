@@ -216,6 +216,27 @@ def test_conv2d_bias_relu_on_the_input_patch_kernel(shape, auto):
            lit.conv2d_fwd_bias_relu_f16(inp, wei, bias, resi, (1, 1), (1, 1), p))
 
 
+@pytest.mark.parametrize("shape", [(2, 9, 28, (1, 1)), (1, 28, 28, (1, 1)), (3, 6, 30, (0, 0))])
+def test_conv2d_bias_relu_on_the_input_patch_kernel_128_channels(shape):
+    """ResNet conv3_x shapes (C = K = 128, 3x3, Wo = 28) on the input-patch instance with bias + ReLU compiled in; the
+    residual form is not one of its epilogues (explicit instance refused, the automatic choice takes a tile instance)."""
+    N, Hi, Wi, p = shape
+    inp = uniform_f16((N, Hi, Wi, 128), -1, 1, 960 + Hi)
+    wei = uniform_f16((128, 3, 3, 128), -0.5, 0.5, 961)
+    bias = uniform_f16((128,), -2, 2, 962)
+    import gpu_util
+    inst = gpu_util.conv_instance(capi.OP_CONV2D_FWD_F16, "Patch")
+    ref = lit.conv2d_fwd_bias_relu_f16(inp, wei, bias, None, (1, 1), (1, 1), p)
+    out = _conv(inp, wei, bias, None, (1, 1), (1, 1), p, inst)
+    _close(out, ref)
+    assert (out == 0).any() and (out > 0).any()
+    resi = uniform_f16(ref.shape, -2, 2, 963)
+    with pytest.raises(AssertionError):
+        _conv(inp, wei, bias, resi, (1, 1), (1, 1), p, inst)
+    _close(_conv(inp, wei, bias, resi, (1, 1), (1, 1), p, capi.INSTANCE_AUTO),
+           lit.conv2d_fwd_bias_relu_f16(inp, wei, bias, resi, (1, 1), (1, 1), p))
+
+
 @pytest.mark.parametrize("shape", [(3, 256, 512, 7, 5, (1, 1)), (2, 128, 1024, 9, 9, (2, 2)), (40, 256, 512, 56, 56, (2, 2))])
 def test_conv2d_bias_relu_on_the_pointwise_kernel(shape):
     """1x1 layers on the weight-stationary kernel with the bias + ReLU functor compiled in (explicit instance for the
