@@ -7,19 +7,22 @@
 // (DeviceConv2dFwdXdl_Input_N_Hi_Wi_C_Weight_K_Y_X_C_Output_N_Ho_Wo_K, device_conv2d_fwd_xdl_nhwc_kyxc_nhwk.hpp:57-720)
 // for C = 128, K = 128, 3 x 3 taps, stride 1, dilation 1, Wo = 28.
 //
-//  * EIGHT waves, two per SIMD, and the OUTPUT CHANNELS are dealt to them: wave w owns channels 16 w .. 16 w + 15 of every
-//    pixel and keeps their 9 taps x 128 input channels as 36 (fp16) / 18 (int8) MFMA operand fragments in registers: 128
-//    (72) AccVGPRs and, fp16, the last tap's 16 in VGPRs beside 7 accumulator tiles, 7 pixel fragments and 21 read addresses
-//    (a wave has 128 + 128 registers).
-//  * All eight waves multiply the same pixels: a band of 4 output rows x 28 pixels = 7 M tiles, one MFMA per tile and
-//    k-step, one fragment read per MFMA -- the LDS pipe is as busy as the matrix cores (8 waves x 4 cycles per read against
-//    2 waves x 16 cycles per MFMA and SIMD), which is the ceiling of this arrangement.
+//  * FOUR waves, one per SIMD, multiply the SAME pixels and split the OUTPUT CHANNELS: wave w owns channels 32 w .. 32 w + 31
+//    and keeps their 9 taps x 128 input channels as 72 (fp16) / 36 (int8) MFMA operand fragments in registers -- fp16: 60 of
+//    them in 240 AccVGPRs and the last 12 in VGPRs (all 256 AccVGPRs would leave the allocator nothing to move a value
+//    through), int8: 144 AccVGPRs -- beside 14 accumulator tiles, 7 pixel fragments and 21 read addresses.
+//  * A band of 4 output rows x 28 pixels is 7 M tiles for every wave; a pixel fragment read feeds two MFMAs. That ratio is
+//    what decides the arrangement: a wave-wide ds_read_b128 occupies the CU's LDS pipe for 8 cycles, an MFMA a SIMD's
+//    matrix core for 16, so four waves at one read per two MFMAs keep the LDS pipe as busy as the matrix cores. EIGHT
+//    waves of 16 channels (NW_ = 8: 36 fragments per wave, 128 AccVGPRs + 16 VGPRs of the 128 + 128 a wave then has) read
+//    one fragment per MFMA: measured 60.0 against 50.2 us in fp16 and 33.0 against 29.1 in int8 at N = 256, and timing-only
+//    builds of that form took 54 us with a seventh of the MFMAs, 49 us with a seventh of the reads -- bound by the LDS.
 //  * A ring row is 4 (fp16) / 2 (int8) planes of 32 pixels x 64 bytes; the k-step, the tap row and the band's position in
 //    the ring are offsets, the tap column selects one of three per-lane registers; the ring never wraps inside a band
 //    (its first two rows exist twice); where the ring is longer than the 16-bit offset field (fp16) the one register set is
 //    moved by a constant between the bands that cross the middle -- 21 vector adds per band, outside the MFMA stream.
-//  * Direct loads: a row is 8 (fp16) / 4 (int8) wave-wide loads of 16 pixels of one plane; wave w always fetches the
-//    same plane and pixel half, so its lanes' column terms are one fixed register (int8: the waves take every other row).
+//  * Direct loads: a row is 8 (fp16) / 4 (int8) wave-wide loads of 16 pixels of one plane; a wave always fetches the same
+//    planes and pixel halves, so its lanes' column terms are fixed registers.
 #pragma once
 
 #include "conv_patch.hpp"
@@ -27,14 +30,15 @@
 namespace ckx {
 
 // FUSED: fp16 -- bias + ReLU (EPI_ADD_RELU)
-template <int DT, bool FUSED, int AHEAD_ = 2>
+template <int DT, bool FUSED, int NW_ = 4, int AHEAD_ = 2>
 struct ConvPatchWide
 {
     static constexpr int ES     = DT == DT_I8 ? 1 : 2;
     static constexpr int CIN = 128, KO = 128, Y = 3, X = 3, TAPS = 9;
     static constexpr int TH     = 4;                     // output rows per band
     static constexpr int WO     = 28, MTW = TH * WO / 16; // 7 M tiles per band, shared by all waves
-    static constexpr int NW     = 8, NT = NW * 64;
+    static constexpr int NW     = NW_, NT = NW * 64;      // 8 waves x 16 channels or 4 waves x 32
+    static constexpr int CPW    = KO / NW, NBT = CPW / 16; // channels and 16-channel weight tiles per wave
     static constexpr int AHEAD  = AHEAD_;
     static constexpr int PXB    = CIN * ES;              // bytes per pixel (256 / 128)
     static constexpr int KSP    = PXB / 64;              // MFMA k-steps per tap = planes of a ring row (4 / 2)
@@ -55,8 +59,9 @@ struct ConvPatchWide
     static constexpr int SPLIT  = MOVES ? TH * ((NPH + 1) / 2) : PERIOD;
     // a row's wave-wide loads, and the waves that share a row's loads / take alternate rows
     static constexpr int UPR    = KSP * (PITCH / 16);    // loads per row (8 / 4)
-    static constexpr int NGRP   = NW / UPR;              // wave groups taking rows in turn (1 / 2)
-    static_assert(NW % UPR == 0 && TH % NGRP == 0 && (Y - 1) % NGRP == 0, "rows dealt evenly to the wave groups");
+    static constexpr int NGRP   = NW > UPR ? NW / UPR : 1; // wave groups taking rows in turn
+    static constexpr int UPW    = UPR > NW ? UPR / NW : 1; // load units of a row per wave
+    static_assert((NW == 4 || NW == 8) && TH % NGRP == 0 && (Y - 1) % NGRP == 0 && NGRP * UPR == NW * UPW, "rows dealt evenly to the waves");
     static_assert(DT == DT_F16 || DT == DT_I8, "fp16 or int8");
     static_assert(!FUSED || DT == DT_F16, "fused epilogue: fp16 bias + ReLU");
     static_assert(LDS <= 160 * 1024, "the ring fits the LDS");
@@ -66,10 +71,10 @@ struct ConvPatchWide
     using acc_t = typename std::conditional<DT == DT_I8, i32x4, f32x4>::type;
     __device__ static __forceinline__ uint32_t key(uint32_t c) { return (c & 1u) | ((c >> 1) & 2u); }
 
-    // With two waves per SIMD the compiler grants a wave 128 VGPRs and 128 AccVGPRs: the fp16 weights are 144 registers, so
-    // the last tap's fragments (W_V) stay in VGPRs, where 97 registers are in use otherwise.
-    static constexpr int W_A_FRAGS = 128 / 4;   // weight fragments that fit the AccVGPRs
-    __host__ __device__ static constexpr bool w_in_vgpr(int tap, int ks) { return tap * KSP + ks >= W_A_FRAGS; }
+    // The fragments that do not fit the AccVGPRs (W_V) stay in VGPRs: four waves may use 240 of their 256 AccVGPRs; with
+    // two waves per SIMD (NW = 8) the compiler grants a wave 128 VGPRs and 128 AccVGPRs.
+    static constexpr int W_A_FRAGS = (NW == 8 ? 128 : 240) / 4;   // weight fragments kept in AccVGPRs
+    __host__ __device__ static constexpr bool w_in_vgpr(int tap, int ks, int j) { return (tap * KSP + ks) * NBT + j >= W_A_FRAGS; }
 
     // acc (+)= w x a: the weights out of AccVGPRs (W_V: VGPRs), pixels and accumulator in VGPRs; FIRST: the accumulator
     // starts at zero (the literal 0 as the addend)
@@ -114,21 +119,25 @@ struct ConvPatchWide
                 requant_lut_fill(smem + RING_BYTES, p.scale_relu, (int)threadIdx.x, NT);
         }
 
-        // ---- weights: fragment (tap, k-step) of this wave's 16 channels. MFMA row frow is output channel 16 w + frow, so
-        // the lane in 16-lane row fq ends with the four consecutive channels 16 w + 4 fq .. + 3 of its pixel. Each
-        // workgroup starts at another filter row (all of them read the same weights at the same time).
-        i32x4 wreg[TAPS][KSP];
+        // ---- weights: fragment (tap, k-step, channel tile j) of this wave. MFMA row frow = 4 q + i of tile j is output channel
+        // CPW w + 4 NBT q + 4 j + i, so the lane in 16-lane row fq ends with the 4 NBT consecutive channels from
+        // CPW w + 4 NBT fq on. Each workgroup starts at another filter row (all of them read the same weights at the same time).
+        i32x4 wreg[TAPS][KSP][NBT];
         auto load_weights = [&](auto y0_c) {
             static_for<Y>([&](auto yy_c) {
                 constexpr int y = (decltype(y0_c)::value + decltype(yy_c)::value) % Y;
-                const uint32_t ch = (uint32_t)(16 * wave) + frow;
 #pragma unroll
-                for(int x = 0; x < X; ++x)
+                for(int j = 0; j < NBT; ++j)
+                {
+                    const uint32_t ch = (uint32_t)(CPW * wave) + (uint32_t)(4 * NBT) * (frow >> 2) + 4u * j + (frow & 3u);
 #pragma unroll
-                    for(int ks = 0; ks < KSP; ++ks)
-                        wreg[y * X + x][ks] = __builtin_bit_cast(
-                            i32x4, __builtin_amdgcn_raw_buffer_load_b128(
-                                       rsrc_wei, (ch * TAPS + (uint32_t)(y * X + x)) * PXB + (uint32_t)ks * 64u + fq * 16u, 0, 0));
+                    for(int x = 0; x < X; ++x)
+#pragma unroll
+                        for(int ks = 0; ks < KSP; ++ks)
+                            wreg[y * X + x][ks][j] = __builtin_bit_cast(
+                                i32x4, __builtin_amdgcn_raw_buffer_load_b128(
+                                           rsrc_wei, (ch * TAPS + (uint32_t)(y * X + x)) * PXB + (uint32_t)ks * 64u + fq * 16u, 0, 0));
+                }
             });
         };
 
@@ -137,7 +146,7 @@ struct ConvPatchWide
         uint32_t rout = 0;    // output rows of the lane's pixels within the band, two bits per tile
         // byte offset of the lane's outputs of tile 0 relative to the band (a band's output rows are contiguous: tile t is
         // 16 t pixels further on, which travels in the scalar offset)
-        const uint32_t ooff0 = (frow * KO + (uint32_t)(16 * wave) + 4u * fq) * ES;
+        const uint32_t ooff0 = (frow * KO + (uint32_t)(CPW * wave) + (uint32_t)(4 * NBT) * fq) * ES;
 #pragma unroll
         for(int t = 0; t < MTW; ++t)
         {
@@ -153,38 +162,43 @@ struct ConvPatchWide
             }
         }
         static_assert(TH <= 4, "two bits per tile row");
-        float bias4[4] = {0.0f, 0.0f, 0.0f, 0.0f};
-        if constexpr(FUSED)
-        {
+        float bias4[4 * NBT];
 #pragma unroll
-            for(int i = 0; i < 4; ++i)
-                bias4[i] = (float)reinterpret_cast<const _Float16*>(p.bias)[16 * wave + 4 * (int)fq + i];
-        }
+        for(int i = 0; i < 4 * NBT; ++i)
+            bias4[i] = FUSED ? (float)reinterpret_cast<const _Float16*>(p.bias)[CPW * wave + 4 * NBT * (int)fq + i] : 0.0f;
 
         // ---- input rows -> ring. Wave w fetches load unit w % UPR (plane unit / 2, pixels 16 (unit % 2) .. + 15) of the rows
         // i = w / UPR, w / UPR + NGRP, ... : lane -> pixel 16 (unit % 2) + lane / 4, LDS chunk position lane % 4 <- global chunk
         // 4 plane + (position ^ key(pixel)). The row travels in the scalar offset; a row outside the image is fetched
         // through a buffer resource of zero bytes (zero fill).
-        const int unit = wave % UPR, grp = wave / UPR;
-        uint32_t gcol;
+        const int grp = wave / UPR; // (NW <= UPR: 0)
+        uint32_t gcol[UPW];
+        uint32_t dst_off[UPW];      // LDS offset of the wave's load units within a ring row
+#pragma unroll
+        for(int u = 0; u < UPW; ++u)
         {
+            const int unit = wave % UPR + NW * u; // (UPW > 1: the wave takes units w, w + NW, ...)
             const int cc = 16 * (unit % 2) + lane / 4, wi = cc - p.pL;
-            gcol = (uint32_t)wi < (uint32_t)p.Wi ? (uint32_t)wi * PXB + (uint32_t)(unit / 2) * 64u + ((((uint32_t)lane & 3u) ^ key((uint32_t)cc)) << 4)
-                                                 : kOutOfRange;
+            gcol[u]    = (uint32_t)wi < (uint32_t)p.Wi ? (uint32_t)wi * PXB + (uint32_t)(unit / 2) * 64u + ((((uint32_t)lane & 3u) ^ key((uint32_t)cc)) << 4)
+                                                       : kOutOfRange;
+            dst_off[u] = (uint32_t)((unit / 2) * PLANE + (unit % 2) * 1024);
         }
-        uint8_t* wave_dst = smem + (unit / 2) * PLANE + (unit % 2) * 1024;
-        // patch row j of image n (input row j - pT) into physical ring row slot
+        // patch row j of image n (input row j - pT) into physical ring row slot: the wave's UPW load units of it
         auto load_row = [&](int n, int j, int slot) {
             const int hi        = j - p.pT;
             const bool ok       = (uint32_t)hi < (uint32_t)p.Hi;
             const uint32_t soff = (uint32_t)((n * p.Hi + (ok ? hi : 0)) * p.Wi) * PXB;
-            __builtin_amdgcn_raw_ptr_buffer_load_lds(ok ? rsrc_in : rsrc_none, (lds_ptr_t)(wave_dst + slot * ROWB), 16, gcol, soff, 0, 0);
+#pragma unroll
+            for(int u = 0; u < UPW; ++u)
+                __builtin_amdgcn_raw_ptr_buffer_load_lds(ok ? rsrc_in : rsrc_none,
+                                                         (lds_ptr_t)(smem + __builtin_amdgcn_readfirstlane(dst_off[u]) + slot * ROWB), 16,
+                                                         gcol[u], soff, 0, 0);
         };
 
-        acc_t acc[MTW];
+        acc_t acc[MTW][NBT];
         // pixel fragments: a ring of NF register tuples over the band's NS * MTW (k-step, tile) pairs in order; the fragment NF
         // pairs ahead is requested into the tuple an MFMA has just read
-        constexpr int NF = DT == DT_I8 ? 5 : 3, NPAIR = NS * MTW; // (fp16: what the 128 VGPRs leave room for; int8: level from 3 to 7)
+        constexpr int NF = NW == 4 ? 7 : (DT == DT_I8 ? 5 : 3), NPAIR = NS * MTW; // (eight fp16 waves: what their 128 VGPRs leave room for)
         i32x4 af[NF];
 
         // fragment of M tile T for k-step S of the band at ring position PH (the registers stand SPLIT rows further on
@@ -204,37 +218,53 @@ struct ConvPatchWide
         // resource (a pixel row past Ho gets the out-of-range offset and is dropped)
         auto store_tile = [&](auto t_c, auto epi_c, int n, int bd) {
             constexpr int t = decltype(t_c)::value, EPI = decltype(epi_c)::value;
-            const acc_t v       = acc[t];
             const uint32_t soff = (uint32_t)((n * p.Ho + TH * bd) * p.Wo + 16 * t) * (KO * ES);
             const uint32_t voff = (int)((rout >> (2 * t)) & 3u) < p.Ho - TH * bd ? ooff0 : kOutOfRange;
             if constexpr(DT == DT_I8)
             {
-                int o;
+                int o[NBT];
                 if constexpr(EPI == EPI_REQUANT_RND)
                 {
-                    const i32x4 vv[1] = {v};
-                    int bb[4];
-                    requant_lut<1>(vv, p.scale_gemm, ring_lds + (uint32_t)RING_BYTES, bb);
-                    o = pack4_low_bytes(bb[0], bb[1], bb[2], bb[3]);
+                    i32x4 vv[NBT];
+#pragma unroll
+                    for(int j = 0; j < NBT; ++j)
+                        vv[j] = acc[t][j];
+                    int bb[4 * NBT];
+                    requant_lut<NBT>(vv, p.scale_gemm, ring_lds + (uint32_t)RING_BYTES, bb);
+#pragma unroll
+                    for(int j = 0; j < NBT; ++j)
+                        o[j] = pack4_low_bytes(bb[4 * j], bb[4 * j + 1], bb[4 * j + 2], bb[4 * j + 3]);
                 }
                 else
-                    o = pack4_low_bytes(epilogue_i8<EPI>(v[0], p.scale_gemm, p.scale_relu), epilogue_i8<EPI>(v[1], p.scale_gemm, p.scale_relu),
-                                        epilogue_i8<EPI>(v[2], p.scale_gemm, p.scale_relu), epilogue_i8<EPI>(v[3], p.scale_gemm, p.scale_relu));
-                __builtin_amdgcn_raw_buffer_store_b32(o, rsrc_out, voff, soff, 0);
+                {
+#pragma unroll
+                    for(int j = 0; j < NBT; ++j)
+                        o[j] = pack4_low_bytes(epilogue_i8<EPI>(acc[t][j][0], p.scale_gemm, p.scale_relu), epilogue_i8<EPI>(acc[t][j][1], p.scale_gemm, p.scale_relu),
+                                               epilogue_i8<EPI>(acc[t][j][2], p.scale_gemm, p.scale_relu), epilogue_i8<EPI>(acc[t][j][3], p.scale_gemm, p.scale_relu));
+                }
+                if constexpr(NBT == 2)
+                    __builtin_amdgcn_raw_buffer_store_b64(i32x2{o[0], o[NBT - 1]}, rsrc_out, voff, soff, 0);
+                else
+                    __builtin_amdgcn_raw_buffer_store_b32(o[0], rsrc_out, voff, soff, 0);
             }
             else
             {
-                typedef _Float16 f16x4 __attribute__((ext_vector_type(4)));
-                f16x4 o;
+                typedef _Float16 f16xn __attribute__((ext_vector_type(4 * NBT)));
+                f16xn o;
 #pragma unroll
-                for(int i = 0; i < 4; ++i)
-                {
-                    float x = v[i];
-                    if constexpr(EPI == EPI_ADD_RELU)
-                        x = __builtin_fmaxf(x + bias4[i], 0.0f);
-                    o[i] = (_Float16)x;
-                }
-                __builtin_amdgcn_raw_buffer_store_b64(__builtin_bit_cast(i32x2, o), rsrc_out, voff, soff, 0);
+                for(int j = 0; j < NBT; ++j)
+#pragma unroll
+                    for(int i = 0; i < 4; ++i)
+                    {
+                        float x = acc[t][j][i];
+                        if constexpr(EPI == EPI_ADD_RELU)
+                            x = __builtin_fmaxf(x + bias4[4 * j + i], 0.0f);
+                        o[4 * j + i] = (_Float16)x;
+                    }
+                if constexpr(NBT == 2)
+                    __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(i32x4, o), rsrc_out, voff, soff, 0);
+                else
+                    __builtin_amdgcn_raw_buffer_store_b64(__builtin_bit_cast(i32x2, o), rsrc_out, voff, soff, 0);
             }
         };
 
@@ -259,7 +289,10 @@ struct ConvPatchWide
                     constexpr int k = s * MTW + g;
                     asm volatile("s_waitcnt lgkmcnt(%0)" ::"n"(k + NF <= NPAIR ? NF - 1 : NPAIR - 1 - k) : "memory");
                     __builtin_amdgcn_sched_barrier(0);
-                    mfma<s == 0, w_in_vgpr(s / KSP, s % KSP)>(acc[g], wreg[s / KSP][s % KSP], af[k % NF]);
+                    static_for<NBT>([&](auto j_c) {
+                        constexpr int j = decltype(j_c)::value;
+                        mfma<s == 0, w_in_vgpr(s / KSP, s % KSP, j)>(acc[g][j], wreg[s / KSP][s % KSP][j], af[k % NF]);
+                    });
                     if constexpr(k + NF < NPAIR)
                         read_pair(ph_c, std::integral_constant<int, k + NF>{});
                     // direct loads of this wave's rows of band b + AHEAD, over the first five eighths of the band
@@ -288,7 +321,7 @@ struct ConvPatchWide
             // the next band's rows have landed (this wave's share): a wave's loads retire in order, the stores of the band
             // before are older still, and what may remain are the loads issued in this band body (AHEAD = 2)
             static_assert(AHEAD == 1 || AHEAD == 2, "the wait below counts this band's loads only");
-            asm volatile("s_waitcnt vmcnt(%0)" ::"n"((AHEAD - 1) * NLW) : "memory");
+            asm volatile("s_waitcnt vmcnt(%0)" ::"n"((AHEAD - 1) * NLW * UPW) : "memory");
             barrier();
             if constexpr(MOVES && (PHN == SPLIT || PHN == 0))
             {
@@ -320,11 +353,15 @@ struct ConvPatchWide
             // Only the first band's rows have to land before the MFMAs start: a wave's loads retire in order, and behind them
             // are the later bands' rows and, in the first image, the weights
             if(first)
-                asm volatile("s_waitcnt vmcnt(%0)" ::"n"((AHEAD - 1) * TH / NGRP + TAPS * KSP) : "memory");
+            {
+                // (the counter holds 63: with more loads behind, a few of the weights are waited for as well)
+                constexpr int behind = (AHEAD - 1) * TH / NGRP * UPW + TAPS * KSP * NBT;
+                asm volatile("s_waitcnt vmcnt(%0)" ::"n"(behind < 63 ? behind : 63) : "memory");
+            }
             else
             {
                 first_rows(n);
-                asm volatile("s_waitcnt vmcnt(%0)" ::"n"((AHEAD - 1) * TH / NGRP) : "memory");
+                asm volatile("s_waitcnt vmcnt(%0)" ::"n"((AHEAD - 1) * TH / NGRP * UPW) : "memory");
             }
             barrier();
             static_for<NF>([&](auto k_c) { read_pair(std::integral_constant<int, 0>{}, k_c); });
@@ -388,7 +425,7 @@ struct ConvPatchWide
 };
 
 template <int DT, bool FUSED>
-__global__ __launch_bounds__(512) void conv_patch_wide_kernel(const ConvPatchArgs p)
+__global__ __launch_bounds__((ConvPatchWide<DT, FUSED>::NT)) void conv_patch_wide_kernel(const ConvPatchArgs p)
 {
     extern __shared__ __attribute__((aligned(1024))) uint8_t ckx_patch_smem[];
     ConvPatchWide<DT, FUSED>::run(p, ckx_patch_smem);

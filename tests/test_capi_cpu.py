@@ -139,10 +139,10 @@ conv_patch.hpp:500:1: remark:     ScratchSize [bytes/lane]: 16 [-Rpass-analysis=
     assert build.patch_register_faults(patch) == [
         ("_ZN3ckx17conv_patch_kernelILi0ELi7ELb0EEEvNS_13ConvPatchArgsE", "200 AccVGPRs"),
         ("_ZN3ckx17conv_patch_kernelILi0ELi7ELb0EEEvNS_13ConvPatchArgsE", "16 bytes of scratch per lane")]
-    # ... and its 128-channel form: 32 of the 36 fp16 fragments (128 AccVGPRs), all 18 int8 ones (72)
+    # ... and its 128-channel form: 60 of the 72 fp16 fragments (240 AccVGPRs), all 36 int8 ones (144)
     wide = """
 conv_patch_wide.hpp:390:1: remark: Function Name: _ZN3ckx22conv_patch_wide_kernelILi1ELb0EEEvNS_13ConvPatchArgsE [-Rpass-analysis=kernel-resource-usage]
-conv_patch_wide.hpp:390:1: remark:     AGPRs: 128 [-Rpass-analysis=kernel-resource-usage]
+conv_patch_wide.hpp:390:1: remark:     AGPRs: 240 [-Rpass-analysis=kernel-resource-usage]
 conv_patch_wide.hpp:390:1: remark:     ScratchSize [bytes/lane]: 0 [-Rpass-analysis=kernel-resource-usage]
 conv_patch_wide.hpp:390:1: remark: Function Name: _ZN3ckx22conv_patch_wide_kernelILi0ELb0EEEvNS_13ConvPatchArgsE [-Rpass-analysis=kernel-resource-usage]
 conv_patch_wide.hpp:390:1: remark:     AGPRs: 128 [-Rpass-analysis=kernel-resource-usage]
