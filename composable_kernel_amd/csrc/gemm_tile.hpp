@@ -445,6 +445,30 @@ __device__ __forceinline__ float epi_f16_value(int mode, float acc, float d0, fl
     return mode == EPI_ADD_RELU_ADD ? b + d1 : b;
 }
 
+// How a copy of the fused epilogue knows its functor: FunctorIs<M> fixes it when the copy is compiled (nothing of the
+// other functors is left in it); FunctorOf<D1, EXT> fixes the operand count and the family only and reads the functor
+// from the arguments, one copy serving several.
+template <int M>
+struct FunctorIs
+{
+    static constexpr bool has_d1 = epi_has_d1(M), ext = M >= EPI_BILINEAR;
+    __device__ static constexpr int mode(const GemmArgs&) { return M; }
+};
+template <bool D1, bool EXT, bool CONV = false>
+struct FunctorOf
+{
+    static constexpr bool has_d1 = D1, ext = EXT;
+    // (with a second D tensor the only extended functor is the GELU one, without it the bilinear one)
+    __device__ static int mode(const GemmArgs& p)
+    {
+        // (and two of the plain functors take one D tensor, of which the conv operators use add + ReLU only)
+        return EXT ? (D1 ? (int)EPI_ADD_ADD_FASTGELU : (int)EPI_BILINEAR)
+               : D1 ? (int)EPI_ADD_RELU_ADD
+               : CONV ? (int)EPI_ADD_RELU
+                      : p.epi;
+    }
+};
+
 // 16 consecutive fp16 outputs of one row with D operands; d0row / d1row point at column 0 of the
 // row's D values (d1row may be null)
 __device__ __forceinline__ void store_row16_f16_fused(_Float16* crow, int n0, int N, bool vec_ok, f32x4 (&v)[4],
@@ -537,9 +561,9 @@ __device__ __forceinline__ void store_row16_f16_fused(_Float16* crow, int n0, in
 // the epilogue moves accumulators between the four 16-lane rows instead (transpose_acc).
 //
 // FUSED (fp16): the variant with the add / ReLU epilogues and their D operands. A kernel of its own: the
-// D loads of that epilogue leave the compiler with "some global load may be outstanding" at the top of
-// the K loop, which it answers with s_waitcnt vmcnt(0) in every iteration -- also for launches that
-// never run that epilogue -- and that wait holds the loop until the prefetched K tile has landed.
+// D values of that epilogue take registers (256 x 128: 171 VGPRs against 146; im2col 194 against 150) that
+// launches which never run it need not pay for. Its K loop is the plain one as long as the epilogue awaits
+// its D loads explicitly (see d_values_landed there).
 template <int DT, int BM, int BN, int WM, int WN, int BKB, int NST, int IM2COL, bool TA = false, bool TB = false,
           bool FUSED = false>
 struct GemmTile
@@ -1079,13 +1103,15 @@ struct GemmTile
         // (which tensors are per-row is a compile-time property of each variant: registers are only
         // set aside for what is fetched)
         // (so is the functor family: EXT = false builds the add / ReLU modes alone, EXT = true the scaled and GELU ones)
-        auto epilogue_fused = [&](int unit, auto chunk_rows, auto d0_row_tensor, auto with_d1, auto extended) {
+        // The functor is a compile-time constant of each copy: as a run-time value every output paid for both add / ReLU
+        // forms and the selects between them (bias + ReLU on a 200704 x 256 x 64 problem: 43.4 us against 29.3 plain).
+        auto epilogue_fused = [&](int unit, auto chunk_rows, auto d0_row_tensor, auto mode_c) {
             constexpr int CH          = decltype(chunk_rows)::value < MT ? decltype(chunk_rows)::value : MT;
             constexpr bool d0_per_row = decltype(d0_row_tensor)::value;
-            constexpr bool has_d1     = decltype(with_d1)::value;
-            constexpr bool EXT        = decltype(extended)::value;
-            // (with a second D tensor the only extended mode is the GELU one, without it the bilinear one)
-            const int mode = !EXT ? p.epi : has_d1 ? (int)EPI_ADD_ADD_FASTGELU : (int)EPI_BILINEAR;
+            using functor             = decltype(mode_c);
+            constexpr bool has_d1     = functor::has_d1;
+            constexpr bool EXT        = functor::ext;
+            const int mode            = functor::mode(p);
             int tm, tn, bi; // (the fused epilogues are never combined with a batch)
             tile_of_block(unit % ntiles, p.tiles_m, p.tiles_n, 1, bi, tm, tn);
             const _Float16* d0 = reinterpret_cast<const _Float16*>(p.d0);
@@ -1116,6 +1142,13 @@ struct GemmTile
                 if(!d0_per_row && col0(g) < p.N)
                     load16(d0, col0(g), b_lo[g], b_hi[g]);
             }
+            // The D values are awaited where every lane passes, right behind their loads (they are the youngest
+            // requests, so the first use would wait for as much). Left to the uses, which sit under the same conditions
+            // as the loads but not provably so, the compiler sees a path on which a load is still on its way when the
+            // K loop starts over, and guards that loop's fragment registers with a wait for all loads in every iteration.
+            auto d_values_landed = [] { __builtin_amdgcn_s_waitcnt(0x0F70); /* vmcnt(0), nothing else */ };
+            if constexpr(!d0_per_row)
+                d_values_landed();
 #pragma unroll
             for(int i0 = 0; i0 < MT; i0 += CH)
             {
@@ -1141,6 +1174,8 @@ struct GemmTile
                                 load16(d1 + (size_t)m * p.ldd1, col0(g), y_lo[c][g], y_hi[c][g]);
                         }
                     }
+                if constexpr(d0_per_row || has_d1)
+                    d_values_landed();
 #pragma unroll
                 for(int c = 0; c < CH; ++c)
 #pragma unroll
@@ -1271,27 +1306,54 @@ struct GemmTile
                         using std::integral_constant;
                         using std::false_type;
                         using std::true_type;
-                        const bool d0_rows = p.ldd0 != 0, resi = epi_has_d1(p.epi);
-                        auto by_operands = [&](auto extended) {
-                            if(!d0_rows && !resi)
-                                epilogue_fused(unit, integral_constant<int, MT>{}, false_type{}, false_type{}, extended);
-                            else if(!d0_rows)
-                                epilogue_fused(unit, integral_constant<int, 2>{}, false_type{}, true_type{}, extended);
-                            else if(!resi)
-                                epilogue_fused(unit, integral_constant<int, 2>{}, true_type{}, false_type{}, extended);
+                        const bool d0_rows = p.ldd0 != 0;
+                        // chunks of fragment rows whose D values are fetched together: all of them for a bias row alone,
+                        // two with one per-row tensor, one with two
+                        auto with_functor = [&](auto mode_c) {
+                            constexpr bool resi = decltype(mode_c)::has_d1;
+                            if(!d0_rows)
+                                epilogue_fused(unit, integral_constant<int, (resi ? 2 : MT)>{}, false_type{}, mode_c);
                             else
-                                epilogue_fused(unit, integral_constant<int, 1>{}, true_type{}, true_type{}, extended);
+                                epilogue_fused(unit, integral_constant<int, (resi ? 1 : 2)>{}, true_type{}, mode_c);
                         };
-                        // (the conv operators take the add / ReLU functors only)
-                        if constexpr(IM2COL == 0)
+                        if constexpr(BM * BN >= 256 * 256)
                         {
-                            if(p.epi >= EPI_BILINEAR)
-                                by_operands(true_type{});
+                            // (the instance that holds 128 accumulators per lane fills the register file already: with
+                            // a copy of the epilogue per functor it spills)
+                            auto by_operands = [&](auto extended) {
+                                constexpr bool EXT = decltype(extended)::value;
+                                if(epi_has_d1(p.epi))
+                                    with_functor(FunctorOf<true, EXT, IM2COL != 0>{});
+                                else if(!EXT && IM2COL == 0 && p.epi == EPI_ADD_RELU)
+                                    with_functor(FunctorOf<false, false, true>{});
+                                else
+                                    with_functor(FunctorOf<false, EXT, IM2COL != 0>{});
+                            };
+                            if(IM2COL == 0 && p.epi >= EPI_BILINEAR)
+                            {
+                                if constexpr(IM2COL == 0)
+                                    by_operands(true_type{});
+                            }
                             else
                                 by_operands(false_type{});
                         }
+                        else if(p.epi == EPI_ADD_RELU)
+                            with_functor(FunctorIs<EPI_ADD_RELU>{});
+                        else if(p.epi == EPI_ADD_RELU_ADD)
+                            with_functor(FunctorIs<EPI_ADD_RELU_ADD>{});
                         else
-                            by_operands(false_type{});
+                        {
+                            // (the conv operators take the two functors above only)
+                            if constexpr(IM2COL == 0)
+                            {
+                                if(p.epi == EPI_CSHUFFLE_ADD_RELU)
+                                    with_functor(FunctorIs<EPI_CSHUFFLE_ADD_RELU>{});
+                                else if(p.epi == EPI_BILINEAR)
+                                    with_functor(FunctorIs<EPI_BILINEAR>{});
+                                else
+                                    with_functor(FunctorIs<EPI_ADD_ADD_FASTGELU>{});
+                            }
+                        }
                     }
                 }
                 else
