@@ -214,8 +214,12 @@ int splitk_runs(int kbytes, int k_batch)
 // 128 x 64 one by 10 - 17 % (ResNet-like layers at N = 32 and 256), which the GEMM-calibrated figures did not say; the
 // 1 x 1 layers of the same networks follow the GEMM figures (256 x 64 rated up sent C 256 -> K 128 at 56 x 56 to it, 20 %
 // behind the 256 x 128 tile)
+// d_epilogue: a conv launch with D operands (bias / residual). On K loops of a few tiles the 128 x 128 instance -- two
+// co-resident workgroups of one wave per SIMD, each held at the epilogue's wait for its D values with nobody to cover
+// for it -- measured 30 - 100 % behind its plain self (C 256 -> K 128, 1x1, 56 x 56, N = 256: 169 us against 128; the
+// 256 x 128 instance 132 against 127), so it is left out there.
 Plan make_plan(long M, int N, int kbytes, int only_tile, long workspace_bytes, int k_batch = 0, bool kmajor = false,
-               bool conv = false, int taps = 2)
+               bool conv = false, int taps = 2, bool d_epilogue = false)
 {
     Plan best;
     double best_us  = 1e30;
@@ -228,6 +232,8 @@ Plan make_plan(long M, int N, int kbytes, int only_tile, long workspace_bytes, i
             continue;
         const TileInstance& t = kTiles[i];
         if(kmajor && t.bm < 64)
+            continue;
+        if(conv && d_epilogue && only_tile < 0 && t.bm == 128 && t.bn == 128 && nk <= 8)
             continue;
         const long tiles      = (long)((M + t.bm - 1) / t.bm) * ((N + t.bn - 1) / t.bn);
         for(int sp = 1; sp <= 8; ++sp)
@@ -689,7 +695,7 @@ int run_gemm(int dt, const void* a, const void* b, void* c, int M, int N, int K,
 }
 
 // ---------------------------------------------------------- input-patch conv kernel
-const char* const kPatchName = "MI355X_Mfma16_Patch<3x3, C = K = 64 rows x 56 (4 waves) or C = K = 128 rows x 28 (8 waves), weights in AccVGPRs>";
+const char* const kPatchName = "MI355X_Mfma16_Patch<3x3, C = K = 64 rows x 56 or C = K = 128 rows x 28, 4 waves, weights in AccVGPRs>";
 
 // the second shape of the instance (conv_patch_wide.hpp): C = K = 128, Wo = 28; plain epilogues and fp16 bias + ReLU
 bool conv_patch_wide_applicable(int op, const ckx_conv2d_desc* d, int epi)
@@ -947,7 +953,7 @@ int run_conv(int op, const void* in, const void* wei, void* out, const ckx_conv2
                                                   (hipStream_t)stream);
         return e == hipSuccess ? CKX_OK : hip_fail(e, kPointwiseName);
     }
-    const Plan pl = make_plan(M, N, K * es, instance, ws ? ws_bytes : 0, 0, false, true, d->Y * d->X);
+    const Plan pl = make_plan(M, N, K * es, instance, ws ? ws_bytes : 0, 0, false, true, d->Y * d->X, f16_fused(epi));
     const TileInstance& t = kTiles[pl.tile];
     ckx::GemmArgs g;
     std::memset(&g, 0, sizeof(g));
@@ -1277,7 +1283,8 @@ int ckx_conv2d_fwd_plan(int op, const ckx_conv2d_desc* d, int epilogue, int64_t 
     if(*instance == CKX_INSTANCE_AUTO || *instance < kNumTiles)
     {
         const Plan pl = make_plan((long)d->N * d->Ho * d->Wo, d->K, d->Y * d->X * d->C * es, *instance,
-                                  workspace_bytes > 0 ? workspace_bytes : 0, 0, false, true, d->Y * d->X);
+                                  workspace_bytes > 0 ? workspace_bytes : 0, 0, false, true, d->Y * d->X,
+                                  f16_fused(epilogue));
         *instance = pl.tile, *k_runs = pl.ksplit;
     }
     return CKX_OK;

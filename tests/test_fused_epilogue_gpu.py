@@ -68,7 +68,7 @@ def _conv(inp, wei, bias, resi, s, d, p, instance=capi.INSTANCE_AUTO, workspace=
 
 
 @pytest.mark.parametrize("case", CONV)
-@pytest.mark.parametrize("instance", [capi.INSTANCE_AUTO, 0, 3, 6, 8])
+@pytest.mark.parametrize("instance", [capi.INSTANCE_AUTO, 0, 1, 3, 6, 7, 8])
 def test_conv2d_bias_relu_and_residual(case, instance):
     N, C, K, Hi, Wi, Y, X, s, d, p = case
     inp = uniform_f16((N, Hi, Wi, C), -1, 1, 300 + C)
@@ -117,6 +117,23 @@ def test_conv2d_bias_relu_resnet_layer_and_split_k(force_k_runs):
     _close(_conv(inp, wei, bias, resi, (1, 1), (1, 1), (1, 1), workspace=True), ref)
     _close(_conv(inp, wei, bias, None, (1, 1), (1, 1), (1, 1), instance=2, workspace=True),
            fast.conv2d_fwd_bias_relu_f16(inp, wei, bias, None, (1, 1), (1, 1), (1, 1)))
+
+
+@pytest.mark.parametrize("instance", [1, 7])
+@pytest.mark.parametrize("filt", [1, 3])
+def test_conv2d_bias_relu_several_tiles_per_workgroup(instance, filt):
+    """The 256 x 128 and 256 x 64 instances on 588 row tiles: more than the persistent grid has workgroups, so most
+    of them finish a tile, hand the zeroed accumulators back to the K loop and finish another (these two instances
+    issue their matrix instructions outside the compiler's view and order that hand-over themselves). 3x3 with
+    padding and 1x1, bias + ReLU and the residual form."""
+    C, K, pad = (32, 128, 1) if filt == 3 else (64, 128, 0)
+    inp = uniform_f16((48, 56, 56, C), -1, 1, 71)
+    wei = uniform_f16((K, filt, filt, C), -0.3, 0.3, 72)
+    bias = uniform_f16((K,), -3, 3, 73)
+    resi = uniform_f16((48, 56, 56, K), -2, 2, 74)
+    args = ((1, 1), (1, 1), (pad, pad))
+    _close(_conv(inp, wei, bias, None, *args, instance=instance), fast.conv2d_fwd_bias_relu_f16(inp, wei, bias, None, *args))
+    _close(_conv(inp, wei, bias, resi, *args, instance=instance), fast.conv2d_fwd_bias_relu_f16(inp, wei, bias, resi, *args))
 
 
 def _gemm_md(a, b_nk, ds, strides, op_functor, instance=capi.INSTANCE_AUTO, lde=None):
