@@ -189,25 +189,37 @@ __global__ __launch_bounds__(NW * 64)
     const i32x4 zero4  = {0, 0, 0, 0};
 
     // ---- register prefetch of one step's B0 / B1 slices ------------------------------------
+    // Buffer loads: one resource per operand over the batch's rows, and per thread and load a byte offset that is fixed
+    // for the whole kernel (row inside the slice, 16-byte chunk; out of range for chunks past K / O) -- a step adds its
+    // first row, one addition per load, and rows past N read as zeros through the range check.
+    const __amdgpu_buffer_rsrc_t rsrc_b0 = make_rsrc(B0, p.N > 0 ? (uint32_t)(((int64_t)(p.N - 1) * p.sb0 + p.K) * 2) : 0u);
+    const __amdgpu_buffer_rsrc_t rsrc_b1 = make_rsrc(B1, p.N > 0 ? (uint32_t)(((int64_t)(p.N - 1) * p.sb1 + p.O) * 2) : 0u);
+    uint32_t vb0[NB0], vb1[NB1];
+#pragma unroll
+    for(int i = 0; i < NB0; ++i)
+    {
+        const int idx = tid + NT * i;
+        const int row = idx / KCH, ch = idx - row * KCH;
+        vb0[i]        = ch * 8 < p.K ? (uint32_t)row * (uint32_t)p.sb0 * 2u + (uint32_t)ch * 16u : kOutOfRange;
+    }
+#pragma unroll
+    for(int i = 0; i < NB1; ++i)
+    {
+        const int idx = tid + NT * i;
+        const int row = idx / OCH, ch = idx - row * OCH;
+        vb1[i]        = ch * 8 < p.O ? (uint32_t)row * (uint32_t)p.sb1 * 2u + (uint32_t)ch * 16u : kOutOfRange;
+    }
     i32x4 rb0[NB0], rb1[NB1];
-    auto load_step = [&](int n0) {
+    auto load_into = [&](int n0, i32x4(&r0)[NB0], i32x4(&r1)[NB1]) {
+        const uint32_t step0 = (uint32_t)n0 * (uint32_t)p.sb0 * 2u, step1 = (uint32_t)n0 * (uint32_t)p.sb1 * 2u;
 #pragma unroll
         for(int i = 0; i < NB0; ++i)
-        {
-            const int idx = tid + NT * i;
-            const int row = idx / KCH, ch = idx - row * KCH;
-            const int n = n0 + row, k = ch * 8;
-            rb0[i] = (n < p.N && k < p.K) ? *reinterpret_cast<const i32x4*>(B0 + (int64_t)n * p.sb0 + k) : zero4;
-        }
+            r0[i] = __builtin_bit_cast(i32x4, __builtin_amdgcn_raw_buffer_load_b128(rsrc_b0, vb0[i] + step0, 0, 0));
 #pragma unroll
         for(int i = 0; i < NB1; ++i)
-        {
-            const int idx = tid + NT * i;
-            const int row = idx / OCH, ch = idx - row * OCH;
-            const int n = n0 + row, o = ch * 8;
-            rb1[i] = (n < p.N && o < p.O) ? *reinterpret_cast<const i32x4*>(B1 + (int64_t)n * p.sb1 + o) : zero4;
-        }
+            r1[i] = __builtin_bit_cast(i32x4, __builtin_amdgcn_raw_buffer_load_b128(rsrc_b1, vb1[i] + step1, 0, 0));
     };
+    auto load_step = [&](int n0) { load_into(n0, rb0, rb1); };
     auto store_step = [&]() {
 #pragma unroll
         for(int i = 0; i < NB0; ++i)
@@ -231,24 +243,6 @@ __global__ __launch_bounds__(NW * 64)
 
     // the same for the second register set of the two-step prefetch (unused, and gone, where PF == 1)
     i32x4 rb0b[NB0], rb1b[NB1];
-    auto load_into = [&](int n0, i32x4(&r0)[NB0], i32x4(&r1)[NB1]) {
-#pragma unroll
-        for(int i = 0; i < NB0; ++i)
-        {
-            const int idx = tid + NT * i;
-            const int row = idx / KCH, ch = idx - row * KCH;
-            const int n = n0 + row, k = ch * 8;
-            r0[i] = (n < p.N && k < p.K) ? *reinterpret_cast<const i32x4*>(B0 + (int64_t)n * p.sb0 + k) : zero4;
-        }
-#pragma unroll
-        for(int i = 0; i < NB1; ++i)
-        {
-            const int idx = tid + NT * i;
-            const int row = idx / OCH, ch = idx - row * OCH;
-            const int n = n0 + row, o = ch * 8;
-            r1[i] = (n < p.N && o < p.O) ? *reinterpret_cast<const i32x4*>(B1 + (int64_t)n * p.sb1 + o) : zero4;
-        }
-    };
     auto store_from = [&](const i32x4(&r0)[NB0], const i32x4(&r1)[NB1]) {
 #pragma unroll
         for(int i = 0; i < NB0; ++i)
@@ -432,6 +426,9 @@ inline bool gemm_gemm_supported(int M, int N, int K, int O, int batch, int sa, i
         return why = "stride smaller than the contiguous extent", false;
     if((long)((M + 63) / 64) * batch >= (1l << 31))
         return why = "grid too large", false;
+    // (the slices of a batch are addressed through 32-bit buffer offsets)
+    if((long)N * sb0 * 2 >= (1l << 31) || (long)N * sb1 * 2 >= (1l << 31))
+        return why = "B0 / B1 of one batch must stay below 2 GiB", false;
     return true;
 }
 
