@@ -1044,6 +1044,9 @@ struct GemmTile
                         const int n0 = tn * BN + wn * WTN + 64 * g + 16 * (lane >> 4);
                         float sc[16];
                         load_col_scales(rs, n0, sc);
+                        // (awaited here, where every lane passes: the uses sit under a condition, and a load that the
+                        // compiler cannot prove consumed makes it wait for all loads in every K iteration)
+                        __builtin_amdgcn_s_waitcnt(0x0F70); // vmcnt(0)
 #pragma unroll
                         for(int i = 0; i < MT; ++i)
                         {
