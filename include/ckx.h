@@ -348,7 +348,9 @@ int ckx_convnd_fwd(int op, const void* p_in, const void* p_wei, void* p_out, con
  * later Composable Kernel releases), with the batch offsets of
  * kernel_batched_gemm_xdlops_v2r3 (device_batched_gemm_xdl.hpp:49-117).
  * Layout "gmk_gnk_gno_gmo": A [G,M,K] row-major, B0 column-major (memory [G,N,K]),
- * B1 [G,N,O] row-major, C [G,M,O] row-major. The [M,N] intermediate stays on chip. */
+ * B1 [G,N,O] row-major, C [G,M,O] row-major. The [M,N] intermediate stays on chip.
+ * Limits: K, O <= 128; K, O and the A / B0 / B1 strides multiples of 8 elements; B0 and B1 of ONE batch below 2 GiB each
+ * (N * stride * 2 bytes: the kernels address a batch's rows through 32-bit buffer offsets). */
 int ckx_batched_gemm_gemm_f16_is_supported(int32_t M, int32_t N, int32_t K, int32_t O, int32_t batch,
                                            int32_t stride_a, int32_t stride_b0, int32_t stride_b1,
                                            int32_t stride_c, int64_t batch_stride_a,

@@ -93,6 +93,12 @@ def test_gemm_gemm_argument_validation():
     assert op.IsSupportedArgument(mk(128, 128))
     assert not op.IsSupportedArgument(mk(256, 64))
     assert not op.IsSupportedArgument(mk(60, 64))
+    # B0 / B1 of one batch are addressed through 32-bit offsets: 70000 rows of 16384 elements are 2.3 GB
+    wide = lambda sb0, sb1: op.MakeArgumentPointer(0, 0, 0, 0, 128, 70000, 64, 64, 1, 64, sb0, sb1, 64, 0, 0, 0, 0)
+    assert op.IsSupportedArgument(wide(64, 64))
+    assert not op.IsSupportedArgument(wide(16384, 64))
+    assert not op.IsSupportedArgument(wide(64, 16384))
+    assert "2 GiB" in capi.last_error()
 
 
 def test_generators_are_counter_based_and_in_range():
