@@ -78,6 +78,22 @@ def vgpr_spills(compiler_output):
     return bad
 
 
+def scratch_users(compiler_output):
+    """(kernel, bytes per lane) for every hand-waited kernel of the resource-usage report that uses scratch memory at
+    all: spills, but also a per-lane array that the compiler could not keep in registers (the 3-D im2col kernels once
+    held their window offsets there: scratch loads in every K iteration, and the compiler's waits for them, which wait
+    for the prefetched K tiles as well)."""
+    bad, name = [], "?"
+    for line in compiler_output.splitlines():
+        if "Function Name:" in line:
+            name = line.split("Function Name:", 1)[1].split("[", 1)[0].strip()
+        elif "ScratchSize [bytes/lane]:" in line:
+            n = int(line.split("ScratchSize [bytes/lane]:", 1)[1].split("[", 1)[0])
+            if n and any(k in name for k in HAND_WAITED_KERNELS):
+                bad.append((name, n))
+    return bad
+
+
 # gemm_w4_kernel: AccVGPRs a lane's accumulators are tied to (the last fragment row's live in VGPRs); the variants with
 # D operands may park a few more values there
 W4_AGPRS = 224
@@ -159,6 +175,7 @@ def build_lib(force=False, verbose=False, extra_flags=()):
         lines = [l for l in r.stdout.splitlines() if "packed-fp32-ops" not in l]
         # the register report: keep it out of the log, fail on vector register spills
         spills = vgpr_spills(r.stdout)
+        scratch = scratch_users(r.stdout)
         w4_bad = w4_register_faults(r.stdout)
         patch_bad = patch_register_faults(r.stdout)
         out, skip = [], 0
@@ -176,6 +193,9 @@ def build_lib(force=False, verbose=False, extra_flags=()):
         if spills:
             raise RuntimeError("vector register spills (the hand-managed LDS read waits do not survive them): "
                                + ", ".join(f"{k}: {n}" for k, n in spills))
+        if scratch:
+            raise RuntimeError("scratch memory in a kernel whose loads are counted by hand: "
+                               + ", ".join(f"{k}: {n} bytes per lane" for k, n in scratch))
         if w4_bad:
             raise RuntimeError("four-wave GEMM body: register allocation differs from what its inline assembly assumes: "
                                + ", ".join(f"{k}: {what}" for k, what in w4_bad))

@@ -706,6 +706,12 @@ struct GemmTile
                 }
                 else
                 {
+                    // (cleared up here, not in the branch for rows past M: there it was the branch's last store, and the
+                    // compiler folded it with the other branch's last store, that of a_off[j], into ONE store through a
+                    // selected address -- which kept both arrays in scratch memory, with scratch loads and waits for all
+                    // loads in every K iteration of the 3-D kernels)
+                    if constexpr(IM2COL == 2)
+                        a_d0[j] = 0;
                     if(ok)
                     {
                         uint32_t img = 0, rem = gm; // img: 2-D image index n, or n * Di + front depth
@@ -739,8 +745,6 @@ struct GemmTile
                     {
                         a_hw0[j] = 0xC000C000u; // (-16384, -16384): every tap out of range
                         a_off[j] = 0;
-                        if constexpr(IM2COL == 2)
-                            a_d0[j] = 0;
                     }
                 }
             }

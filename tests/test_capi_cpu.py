@@ -133,6 +133,17 @@ conv_patch.hpp:410:1: remark: Function Name: _ZN3ckx17conv_patch_kernelILi1EEEvN
 conv_patch.hpp:410:1: remark:     VGPRs Spill: 0 [-Rpass-analysis=kernel-resource-usage]
 """
     assert build.vgpr_spills(report) == [("_ZN3ckx16gemm_tile_kernelILi0ELi256ELi256EEvNS_8GemmArgsE", 7)]
+    # ... and scratch memory of any origin in them (a per-lane array that did not stay in registers counts like a spill)
+    private_array = """
+gemm_tile.hpp:1500:1: remark: Function Name: _ZN3ckx16gemm_tile_kernelILi1ELi256ELi64ELi8ELi1ELi128ELi2ELi2ELb0ELb0ELb0EEEvNS_8GemmArgsE [-Rpass-analysis=kernel-resource-usage]
+gemm_tile.hpp:1500:1: remark:     ScratchSize [bytes/lane]: 40 [-Rpass-analysis=kernel-resource-usage]
+gemm_tile.hpp:1500:1: remark:     VGPRs Spill: 0 [-Rpass-analysis=kernel-resource-usage]
+gemm_gemm.hpp:400:1: remark: Function Name: _ZN3ckx16gemm_gemm_kernelILi4EEEvNS_12GemmGemmArgsE [-Rpass-analysis=kernel-resource-usage]
+gemm_gemm.hpp:400:1: remark:     ScratchSize [bytes/lane]: 16 [-Rpass-analysis=kernel-resource-usage]
+"""
+    assert build.vgpr_spills(private_array) == []
+    assert build.scratch_users(private_array) == [
+        ("_ZN3ckx16gemm_tile_kernelILi1ELi256ELi64ELi8ELi1ELi128ELi2ELi2ELb0ELb0ELb0EEEvNS_8GemmArgsE", 40)]
     # the input-patch conv kernel keeps its weights, and nothing else, in AccVGPRs, and has no scratch
     patch = """
 conv_patch.hpp:500:1: remark: Function Name: _ZN3ckx17conv_patch_kernelILi1ELi7ELb0EEEvNS_13ConvPatchArgsE [-Rpass-analysis=kernel-resource-usage]
