@@ -13,6 +13,7 @@
 #include "ckx.h"
 #include "gemm_tile.hpp"
 #include "tile_launch.hpp"
+#include "conv_rows.hpp"
 #include "gemm_gemm.hpp"
 #include "conv_patch.hpp"
 #include "conv_patch_wide.hpp"
@@ -730,8 +731,9 @@ bool conv_patch_preferred(int op, const ckx_conv2d_desc* d, int epi)
 
 // ---------------------------------------------------------- weight-stationary pointwise conv kernel
 const char* const kPointwiseName = "MI355X_Mfma16_Pointwise<1x1, C 256/512 bytes, K 512 per workgroup, 8 waves>";
+const char* const kRowsName = "MI355X_Mfma16_Rows<1x1, stride 1, pixels of 64 / 128 bytes, K <= 256 per workgroup, weights in registers, no LDS>";
 constexpr int kConvPatchInstance = kNumTiles, kConvPointwiseInstance = kNumTiles + 1, kConvStemInstance = kNumTiles + 2,
-              kConvGenericInstance = kNumTiles + 3, kNumConvInsts = kNumTiles + 4;
+              kConvRowsInstance = kNumTiles + 3, kConvGenericInstance = kNumTiles + 4, kNumConvInsts = kNumTiles + 5;
 
 // ---------------------------------------------------------- stem conv kernel (three input channels)
 const char* const kStemName = "MI355X_Mfma16_Stem<7x7, stride 2, pad 3, C 3, K 64, pixels padded to 4 channels in LDS, 4 waves>";
@@ -773,6 +775,30 @@ bool conv_pointwise_preferred(int op, const ckx_conv2d_desc* d, int epi)
 {
     const long px = (long)d->N * d->Ho * d->Wo * (d->K / 512);
     return conv_pointwise_applicable(op, d, epi) && px >= (op == CKX_OP_CONV2D_FWD_I8 ? 16 * 1024 : 40 * 1024);
+}
+
+// shapes the streaming 1x1 kernel covers: 1x1 filters, stride 1, no padding (the input is the [pixels, C] matrix), a pixel
+// of 64 or 128 bytes, output channels in whole groups of 64 up to 256 or in whole blocks of 256
+bool conv_rows_applicable(int op, const ckx_conv2d_desc* d, int epi)
+{
+    const int es      = op == CKX_OP_CONV2D_FWD_I8 ? 1 : 2;
+    const bool epi_ok = op == CKX_OP_CONV2D_FWD_F16
+                            ? (epi == CKX_EPI_PASSTHROUGH || epi == CKX_EPI_ADD_RELU)
+                            : (epi == CKX_EPI_PASSTHROUGH || epi == CKX_EPI_REQUANT_CK || epi == CKX_EPI_REQUANT_RND);
+    return (op == CKX_OP_CONV2D_FWD_F16 || op == CKX_OP_CONV2D_FWD_I8) && epi_ok && d->Y == 1 && d->X == 1 &&
+           d->stride_h == 1 && d->stride_w == 1 && d->pad_top == 0 && d->pad_left == 0 && d->pad_bottom == 0 &&
+           d->pad_right == 0 && (d->C * es == 64 || d->C * es == 128) && d->K >= 64 && d->K % 64 == 0 &&
+           (d->K <= 256 || d->K % 256 == 0) && d->N >= 1 && d->Ho == d->Hi && d->Wo == d->Wi && d->Ho >= 1 && d->Wo >= 1;
+}
+// ... and the ones it is chosen for: enough rows for every wave of a full launch to run its two-deep pipeline, and a
+// 64-byte pixel or few output channels. Measured at N = 256 against the best tile instance: int8 C 64 -> K 64 at 56 x 56
+// 19.6 against 37.6 us, C 64 -> K 256 64.7 against 84.0; fp16 C 64 -> K 64 33.2 against 34.5 (with bias + ReLU 33.4
+// against 38.8); but fp16 C 64 -> K 256 118 against 111 and int8 C 128 -> K 512 at 28 x 28 54.8 against 47.2 -- with
+// 128-byte pixels and 256 columns per block the weights take 128 registers and half as many waves stream.
+bool conv_rows_preferred(int op, const ckx_conv2d_desc* d, int epi)
+{
+    const int es = op == CKX_OP_CONV2D_FWD_I8 ? 1 : 2;
+    return conv_rows_applicable(op, d, epi) && (long)d->N * d->Ho * d->Wo >= 65536 && (d->C * es == 64 || d->K <= 128);
 }
 
 int check_conv(int op, const ckx_conv2d_desc* d, int epi, int instance)
@@ -823,6 +849,9 @@ int check_conv(int op, const ckx_conv2d_desc* d, int epi, int instance)
     if(instance == kConvPointwiseInstance && !conv_pointwise_applicable(op, d, epi))
         return fail(CKX_UNSUPPORTED, "the pointwise instance covers 1x1 layers without padding, C of 256 or 512 bytes, "
                                      "K a multiple of 512, PassThrough / requant / bias + ReLU epilogues");
+    if(instance == kConvRowsInstance && !conv_rows_applicable(op, d, epi))
+        return fail(CKX_UNSUPPORTED, "the streaming 1x1 instance covers 1x1 stride-1 layers without padding, C of 64 or 128 bytes, "
+                                     "K a multiple of 64 up to 256 or a multiple of 256, PassThrough / requant / bias + ReLU epilogues");
     return CKX_OK;
 }
 
@@ -833,9 +862,10 @@ long conv_workspace_bytes(int op, const ckx_conv2d_desc* d, int instance)
     if(M <= 0 || d->K <= 0)
         return 0;
     if(instance == kConvPatchInstance || instance == kConvPointwiseInstance || instance == kConvGenericInstance ||
-       instance == kConvStemInstance || ((long)d->C * es) % 16 ||
+       instance == kConvStemInstance || instance == kConvRowsInstance || ((long)d->C * es) % 16 ||
        (instance == CKX_INSTANCE_AUTO &&
-        (conv_patch_preferred(op, d, CKX_EPI_PASSTHROUGH) || conv_pointwise_preferred(op, d, CKX_EPI_PASSTHROUGH))))
+        (conv_patch_preferred(op, d, CKX_EPI_PASSTHROUGH) || conv_pointwise_preferred(op, d, CKX_EPI_PASSTHROUGH) ||
+         conv_rows_preferred(op, d, CKX_EPI_PASSTHROUGH))))
         return 0;
     const Plan pl = make_plan((int)M, d->K, d->Y * d->X * d->C * es, instance, 1l << 60, 0, false, true, d->Y * d->X);
     return pl.ksplit > 1 ? (long)pl.ksplit * M * d->K * 4 : 0;
@@ -952,6 +982,24 @@ int run_conv(int op, const void* in, const void* wei, void* out, const ckx_conv2
                                                   epi == CKX_EPI_ADD_RELU || per_column_scale(epi), a,
                                                   (hipStream_t)stream);
         return e == hipSuccess ? CKX_OK : hip_fail(e, kPointwiseName);
+    }
+    if(instance == kConvRowsInstance ||
+       (instance == CKX_INSTANCE_AUTO && conv_rows_preferred(op, d, epi) && patch_aligned && dops.ldd0 == 0))
+    {
+        if(!patch_aligned)
+            return fail(CKX_UNSUPPORTED, "the streaming 1x1 instance needs 16-byte aligned output and bias");
+        if(epi == CKX_EPI_ADD_RELU && dops.ldd0 != 0)
+            return fail(CKX_UNSUPPORTED, "the streaming 1x1 instance adds a bias row (D0 row stride 0) only");
+        ckx::ConvRowsArgs a;
+        std::memset(&a, 0, sizeof(a));
+        a.in = in, a.wei = wei, a.out = out, a.bias = dops.d0;
+        a.in_bytes = (uint32_t)((long)M * d->C * es);
+        a.M = M, a.C = d->C, a.Kout = N;
+        a.epi = epi, a.scale_gemm = sg, a.scale_relu = sr;
+        a.nt_store   = es == 1 && (long)M * N * es >= stream_output_bytes();
+        hipError_t e = ckx::launch_conv_rows(es == 1 ? ckx::DT_I8 : ckx::DT_F16, d->C * es, epi == CKX_EPI_ADD_RELU, a,
+                                             (hipStream_t)stream);
+        return e == hipSuccess ? CKX_OK : hip_fail(e, kRowsName);
     }
     const Plan pl = make_plan(M, N, K * es, instance, ws ? ws_bytes : 0, 0, false, true, d->Y * d->X, f16_fused(epi));
     const TileInstance& t = kTiles[pl.tile];
@@ -1177,7 +1225,7 @@ int ckx_num_instances(int op)
     if(op == CKX_OP_GEMM_SPLITK)
         return kNumTiles;
     if(op == CKX_OP_CONV2D_FWD_F16 || op == CKX_OP_CONV2D_FWD_I8)
-        return kNumConvInsts; // + the input-patch, the pointwise, the stem and the element-wise kernel
+        return kNumConvInsts; // + the input-patch, the pointwise, the stem, the streaming 1x1 and the element-wise kernel
     if(op == CKX_OP_BATCHED_GEMM_GEMM || op == CKX_OP_BATCHED_GEMM_SOFTMAX_GEMM)
         return ckx::kNumGemmGemmInstances;
     return 0;
@@ -1194,7 +1242,7 @@ const char* ckx_instance_name(int op, int instance)
              ? ckx::gemm_gemm_instance_name(instance)
          : (op == CKX_OP_CONV2D_FWD_F16 || op == CKX_OP_CONV2D_FWD_I8) && instance >= kNumTiles
              ? (instance == kConvPatchInstance ? kPatchName : instance == kConvPointwiseInstance ? kPointwiseName
-                : instance == kConvStemInstance ? kStemName : kGenericName)
+                : instance == kConvStemInstance ? kStemName : instance == kConvRowsInstance ? kRowsName : kGenericName)
              : instance == kGenericGemmInstance ? kGenericName
              : instance >= kNumTiles            ? kSkinny[instance - kNumTiles].name
                                                 : kTiles[instance].name) +
@@ -1279,6 +1327,8 @@ int ckx_conv2d_fwd_plan(int op, const ckx_conv2d_desc* d, int epilogue, int64_t 
             *instance = kConvPatchInstance;
         else if(conv_pointwise_preferred(op, d, epilogue))
             *instance = kConvPointwiseInstance;
+        else if(conv_rows_preferred(op, d, epilogue))
+            *instance = kConvRowsInstance;
     }
     if(*instance == CKX_INSTANCE_AUTO || *instance < kNumTiles)
     {

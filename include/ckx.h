@@ -311,8 +311,8 @@ int ckx_conv2d_fwd_bias_activation_f16(const void* p_in, const void* p_wei, void
 
 /* conv2d forward, int8, with one fp32 requant scale per OUTPUT CHANNEL (p_scale: K contiguous floats): out_op is
  * CKX_EPI_MUL2_CLAMP or CKX_EPI_RELU_MUL2_CLAMP (upstream's per-channel quantisation of a conv: the same functor as
- * the CDE operation of its multiple-D conv operators). Every conv instance takes it (the pointwise specialist for
- * 256-byte pixels only: the scales live in registers beside the weights); supported geometries are those of
+ * the CDE operation of its multiple-D conv operators). Every conv instance but the streaming 1x1 one takes it (the
+ * pointwise specialist for 256-byte pixels only: the scales live in registers beside the weights); supported geometries are those of
  * ckx_conv2d_fwd_is_supported(CKX_OP_CONV2D_FWD_I8, desc, out_op, instance). */
 int ckx_conv2d_fwd_i8_multiple_d(const void* p_in, const void* p_wei, const void* p_scale, void* p_out,
                                  const ckx_conv2d_desc* desc, int out_op, int instance, void* p_workspace,

@@ -392,6 +392,96 @@ def test_conv2d_pointwise_instance_refuses_other_shapes():
     assert L.ckx_conv2d_fwd_is_supported(capi.OP_CONV2D_FWD_F16, C.byref(ok), capi.EPI_ADD_RELU_ADD, pw) == capi.UNSUPPORTED
 
 
+# (N, C, K, Hi, Wi): 1x1, stride 1, no padding
+ROWS_F16 = [
+    (1, 32, 64, 3, 5),          # 64-byte pixels, 15 rows: less than one tile of 16
+    (3, 32, 128, 7, 5),         # 105 rows: a ragged last tile and a ragged last pair of tiles
+    (2, 64, 256, 9, 11),        # 128-byte pixels (ResNet conv2_x: 64 -> 256)
+    (2, 64, 64, 8, 8),
+    (2, 32, 192, 5, 6),         # three of the four 64-column groups of a block
+    (1, 64, 512, 6, 7),         # two blocks of 256 output channels
+]
+ROWS_I8 = [
+    (1, 64, 64, 3, 5),          # 64-byte pixels
+    (3, 64, 256, 7, 5),
+    (2, 128, 512, 9, 11),       # 128-byte pixels, two blocks of output channels (ResNet conv3_x: 128 -> 512)
+    (2, 128, 128, 8, 8),
+    (2, 64, 768, 5, 5),         # three blocks
+]
+
+
+@pytest.mark.parametrize("case", ROWS_F16)
+def test_conv2d_fp16_streaming_1x1_kernel(case):
+    """The streaming 1x1 kernel (weights in registers, pixel rows straight into MFMA operands, no LDS) against the
+    literal oracle; the tile kernel must agree on the same problem."""
+    import gpu_util
+    N, C, K, Hi, Wi = case
+    inp = uniform_f16((N, Hi, Wi, C), -1, 1, 1100 + Hi)
+    wei = uniform_f16((K, 1, 1, C), -1, 1, 1101 + Wi)
+    rows = gpu_util.conv_instance(capi.OP_CONV2D_FWD_F16, "Rows<")
+    ref = lit.conv2d_fwd(inp, wei, (1, 1), (1, 1), (0, 0))
+    _f16_close(gpu_util.conv2d_fwd(inp, wei, (1, 1), (1, 1), (0, 0), instance=rows), ref)
+    _f16_close(gpu_util.conv2d_fwd(inp, wei, (1, 1), (1, 1), (0, 0), instance=3), ref)
+
+
+@pytest.mark.parametrize("case", ROWS_I8)
+def test_conv2d_int8_streaming_1x1_kernel_bit_exact(case):
+    import gpu_util
+    N, C, K, Hi, Wi = case
+    inp = uniform_int8((N, Hi, Wi, C), -5, 5, 1110 + Hi)
+    wei = uniform_int8((K, 1, 1, C), -5, 5, 1111 + Wi)
+    rows = gpu_util.conv_instance(capi.OP_CONV2D_FWD_I8, "Rows<")
+    np.testing.assert_array_equal(gpu_util.conv2d_fwd(inp, wei, (1, 1), (1, 1), (0, 0), instance=rows),
+                                  lit.conv2d_fwd(inp, wei, (1, 1), (1, 1), (0, 0)))
+    for rq, kind in ((ck.RequantReluRequant(0.02, 0.7, rounded=True), lit.EPI_REQUANT_RND),
+                     (ck.RequantReluRequant(0.03, 1.0), lit.EPI_REQUANT_CK)):
+        out = gpu_util.conv2d_fwd(inp, wei, (1, 1), (1, 1), (0, 0), out_op=rq, instance=rows)
+        np.testing.assert_array_equal(
+            out, lit.conv2d_fwd(inp, wei, (1, 1), (1, 1), (0, 0), epi=kind, scale_gemm=rq.scale_gemm, scale_relu=rq.scale_relu))
+        assert out.max() > 0
+
+
+@pytest.mark.parametrize("dtype", ["f16", "i8"])
+def test_conv2d_streaming_1x1_kernel_every_wave_several_rounds(dtype):
+    """ResNet conv2_x at a batch that gives every wave of the full launch several pairs of row tiles (the automatic
+    choice for such layers), full-range int8 values included."""
+    import gpu_util
+    if dtype == "f16":
+        inp = uniform_f16((48, 56, 56, 64), -1, 1, 1120)
+        wei = uniform_f16((64, 1, 1, 64), -1, 1, 1121)
+        desc = capi.Conv2dDesc(48, 64, 64, 56, 56, 1, 1, 56, 56, 1, 1, 1, 1, 0, 0, 0, 0)
+        assert capi.conv2d_fwd_plan(capi.OP_CONV2D_FWD_F16, desc)[0] == gpu_util.conv_instance(capi.OP_CONV2D_FWD_F16, "Rows<")
+        out = gpu_util.conv2d_fwd(inp, wei, (1, 1), (1, 1), (0, 0))
+        _f16_close(out, fast.conv2d_fwd_f16(inp, wei, (1, 1), (1, 1), (0, 0)))
+    else:
+        inp = uniform_int8((96, 56, 56, 64), -128, 127, 1122)
+        wei = uniform_int8((64, 1, 1, 64), -128, 127, 1123)
+        desc = capi.Conv2dDesc(96, 64, 64, 56, 56, 1, 1, 56, 56, 1, 1, 1, 1, 0, 0, 0, 0)
+        assert capi.conv2d_fwd_plan(capi.OP_CONV2D_FWD_I8, desc)[0] == gpu_util.conv_instance(capi.OP_CONV2D_FWD_I8, "Rows<")
+        out = gpu_util.conv2d_fwd(inp, wei, (1, 1), (1, 1), (0, 0))
+        np.testing.assert_array_equal(out, fast.conv2d_fwd_i8(inp, wei, (1, 1), (1, 1), (0, 0)))
+
+
+def test_conv2d_streaming_1x1_instance_refuses_other_shapes():
+    import ctypes as C
+    import gpu_util
+    L = capi.lib()
+    rows = gpu_util.conv_instance(capi.OP_CONV2D_FWD_F16, "Rows<")
+    ok = capi.Conv2dDesc(2, 256, 64, 8, 8, 1, 1, 8, 8, 1, 1, 1, 1, 0, 0, 0, 0)
+    assert L.ckx_conv2d_fwd_is_supported(capi.OP_CONV2D_FWD_F16, C.byref(ok), 0, rows) == capi.OK
+    for d in (capi.Conv2dDesc(2, 96, 64, 8, 8, 1, 1, 8, 8, 1, 1, 1, 1, 0, 0, 0, 0),        # K = 96: not whole 64-column groups
+              capi.Conv2dDesc(2, 320, 64, 8, 8, 1, 1, 8, 8, 1, 1, 1, 1, 0, 0, 0, 0),       # K = 320: above 256, not whole blocks
+              capi.Conv2dDesc(2, 256, 128, 8, 8, 1, 1, 8, 8, 1, 1, 1, 1, 0, 0, 0, 0),      # 256-byte pixels
+              capi.Conv2dDesc(2, 256, 64, 8, 8, 1, 1, 4, 4, 2, 2, 1, 1, 0, 0, 0, 0),       # stride 2
+              capi.Conv2dDesc(2, 256, 64, 8, 8, 1, 1, 10, 10, 1, 1, 1, 1, 1, 1, 1, 1),     # padded
+              capi.Conv2dDesc(2, 256, 64, 8, 8, 3, 3, 6, 6, 1, 1, 1, 1, 0, 0, 0, 0)):      # 3x3
+        assert L.ckx_conv2d_fwd_is_supported(capi.OP_CONV2D_FWD_F16, C.byref(d), 0, rows) == capi.UNSUPPORTED
+        assert L.ckx_conv2d_fwd_is_supported(capi.OP_CONV2D_FWD_F16, C.byref(d), 0, -1) == capi.OK
+    # the residual functor and the per-channel scales stay with the tile kernel
+    assert L.ckx_conv2d_fwd_is_supported(capi.OP_CONV2D_FWD_F16, C.byref(ok), capi.EPI_ADD_RELU_ADD, rows) == capi.UNSUPPORTED
+    assert L.ckx_conv2d_fwd_is_supported(capi.OP_CONV2D_FWD_I8, C.byref(ok), capi.EPI_MUL2_CLAMP, rows) == capi.UNSUPPORTED
+
+
 @pytest.mark.parametrize("shape", ["patch", "pointwise"])
 def test_conv2d_specialists_fall_back_on_unaligned_output(shape):
     """The input-patch and pointwise kernels store whole 16-byte vectors: an output that starts 2 bytes into a buffer

@@ -254,6 +254,26 @@ def test_conv2d_bias_relu_on_the_input_patch_kernel_128_channels(shape):
            lit.conv2d_fwd_bias_relu_f16(inp, wei, bias, resi, (1, 1), (1, 1), p))
 
 
+@pytest.mark.parametrize("shape", [(3, 32, 64, 7, 5), (2, 64, 256, 9, 11), (1, 64, 512, 6, 7), (24, 64, 64, 56, 56)])
+def test_conv2d_bias_relu_on_the_streaming_1x1_kernel(shape):
+    """1x1 stride-1 layers with pixels of 64 / 128 bytes on the streaming kernel with the bias + ReLU functor compiled in
+    (explicit instance for the small shapes, the automatic choice for the ResNet conv2_x one); the residual form is not
+    one of its epilogues."""
+    import gpu_util
+    N, C, K, Hi, Wi = shape
+    inp = uniform_f16((N, Hi, Wi, C), -1, 1, 81)
+    wei = uniform_f16((K, 1, 1, C), -0.5, 0.5, 82)
+    bias = uniform_f16((K,), -3, 3, 83)
+    big = N * Hi * Wi >= 65536
+    inst = capi.INSTANCE_AUTO if big else gpu_util.conv_instance(capi.OP_CONV2D_FWD_F16, "Rows<")
+    ref = (fast if big else lit).conv2d_fwd_bias_relu_f16(inp, wei, bias, None, (1, 1), (1, 1), (0, 0))
+    _close(_conv(inp, wei, bias, None, (1, 1), (1, 1), (0, 0), instance=inst), ref)
+    if not big:
+        resi = uniform_f16((N, Hi, Wi, K), -2, 2, 84)
+        with pytest.raises(AssertionError):
+            _conv(inp, wei, bias, resi, (1, 1), (1, 1), (0, 0), instance=inst)
+
+
 @pytest.mark.parametrize("shape", [(3, 256, 512, 7, 5, (1, 1)), (2, 128, 1024, 9, 9, (2, 2)), (40, 256, 512, 56, 56, (2, 2))])
 def test_conv2d_bias_relu_on_the_pointwise_kernel(shape):
     """1x1 layers on the weight-stationary kernel with the bias + ReLU functor compiled in (explicit instance for the
