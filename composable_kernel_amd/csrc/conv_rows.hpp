@@ -65,9 +65,12 @@ __global__ __launch_bounds__(256) void conv_rows_kernel(const ConvRowsArgs p)
 #pragma unroll
         for(int g = 0; g < NG; ++g)
         {
+            // (K comes in whole groups of 64: a group past K -- K = 192 in a block of 256 -- has no bias to read)
             const _Float16* b = reinterpret_cast<const _Float16*>(p.bias) + kblock + 64 * g + 16 * q;
-            b_lo[g]           = *reinterpret_cast<const f16x8*>(b);
-            b_hi[g]           = *reinterpret_cast<const f16x8*>(b + 8);
+            const f16x8 zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
+            const bool live   = kblock + 64 * g < p.Kout;
+            b_lo[g]           = live ? *reinterpret_cast<const f16x8*>(b) : zero8;
+            b_hi[g]           = live ? *reinterpret_cast<const f16x8*>(b + 8) : zero8;
         }
     }
 

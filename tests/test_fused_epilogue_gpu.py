@@ -254,7 +254,7 @@ def test_conv2d_bias_relu_on_the_input_patch_kernel_128_channels(shape):
            lit.conv2d_fwd_bias_relu_f16(inp, wei, bias, resi, (1, 1), (1, 1), p))
 
 
-@pytest.mark.parametrize("shape", [(3, 32, 64, 7, 5), (2, 64, 256, 9, 11), (1, 64, 512, 6, 7), (24, 64, 64, 56, 56)])
+@pytest.mark.parametrize("shape", [(3, 32, 64, 7, 5), (2, 64, 256, 9, 11), (2, 32, 192, 5, 6), (1, 64, 512, 6, 7), (24, 64, 64, 56, 56)])
 def test_conv2d_bias_relu_on_the_streaming_1x1_kernel(shape):
     """1x1 stride-1 layers with pixels of 64 / 128 bytes on the streaming kernel with the bias + ReLU functor compiled in
     (explicit instance for the small shapes, the automatic choice for the ResNet conv2_x one); the residual form is not
