@@ -731,7 +731,7 @@ bool conv_patch_preferred(int op, const ckx_conv2d_desc* d, int epi)
 
 // ---------------------------------------------------------- weight-stationary pointwise conv kernel
 const char* const kPointwiseName = "MI355X_Mfma16_Pointwise<1x1, C 256/512 bytes, K 512 per workgroup, 8 waves>";
-const char* const kRowsName = "MI355X_Mfma16_Rows<1x1, stride 1, pixels of 64 / 128 bytes, K <= 256 per workgroup, weights in registers, no LDS>";
+const char* const kRowsName = "MI355X_Mfma16_Rows<1x1, stride 1, pixels of 64 ... 512 bytes, K <= 256 per workgroup, weights in registers, no LDS>";
 constexpr int kConvPatchInstance = kNumTiles, kConvPointwiseInstance = kNumTiles + 1, kConvStemInstance = kNumTiles + 2,
               kConvRowsInstance = kNumTiles + 3, kConvGenericInstance = kNumTiles + 4, kNumConvInsts = kNumTiles + 5;
 
@@ -778,7 +778,8 @@ bool conv_pointwise_preferred(int op, const ckx_conv2d_desc* d, int epi)
 }
 
 // shapes the streaming 1x1 kernel covers: 1x1 filters, stride 1, no padding (the input is the [pixels, C] matrix), a pixel
-// of 64 or 128 bytes, output channels in whole groups of 64 up to 256 or in whole blocks of 256
+// of 64 or 128 bytes with output channels in whole groups of 64 up to 256 or in whole blocks of 256, a pixel of 256 bytes
+// with 64 or 128 output channels, one of 512 bytes with 64 (what a wave's registers hold of weights and pixel rows)
 bool conv_rows_applicable(int op, const ckx_conv2d_desc* d, int epi)
 {
     const int es      = op == CKX_OP_CONV2D_FWD_I8 ? 1 : 2;
@@ -787,18 +788,23 @@ bool conv_rows_applicable(int op, const ckx_conv2d_desc* d, int epi)
                             : (epi == CKX_EPI_PASSTHROUGH || epi == CKX_EPI_REQUANT_CK || epi == CKX_EPI_REQUANT_RND);
     return (op == CKX_OP_CONV2D_FWD_F16 || op == CKX_OP_CONV2D_FWD_I8) && epi_ok && d->Y == 1 && d->X == 1 &&
            d->stride_h == 1 && d->stride_w == 1 && d->pad_top == 0 && d->pad_left == 0 && d->pad_bottom == 0 &&
-           d->pad_right == 0 && (d->C * es == 64 || d->C * es == 128) && d->K >= 64 && d->K % 64 == 0 &&
-           (d->K <= 256 || d->K % 256 == 0) && d->N >= 1 && d->Ho == d->Hi && d->Wo == d->Wi && d->Ho >= 1 && d->Wo >= 1;
+           d->pad_right == 0 && (d->C * es == 64 || d->C * es == 128 || (d->C * es == 256 && d->K <= 128) || (d->C * es == 512 && d->K <= 64)) && d->K >= 64 &&
+           d->K % 64 == 0 && (d->K <= 256 || d->K % 256 == 0) && d->N >= 1 && d->Ho == d->Hi && d->Wo == d->Wi && d->Ho >= 1 &&
+           d->Wo >= 1;
 }
-// ... and the ones it is chosen for: enough rows for every wave of a full launch to run its two-deep pipeline, and a
-// 64-byte pixel or few output channels. Measured at N = 256 against the best tile instance: int8 C 64 -> K 64 at 56 x 56
-// 19.6 against 37.6 us, C 64 -> K 256 64.7 against 84.0; fp16 C 64 -> K 64 33.2 against 34.5 (with bias + ReLU 33.4
-// against 38.8); but fp16 C 64 -> K 256 118 against 111 and int8 C 128 -> K 512 at 28 x 28 54.8 against 47.2 -- with
-// 128-byte pixels and 256 columns per block the weights take 128 registers and half as many waves stream.
+// ... and the ones it is chosen for: enough rows for every wave of a full launch to run its two-deep pipeline, and few
+// enough weight registers. Measured at N = 256 against the best tile instance: int8 C 64 -> K 64 at 56 x 56 19.6 against
+// 37.6 us, C 64 -> K 256 64.7 against 84.0, C 256 -> K 64 42.0 against 47.0; fp16 C 64 -> K 64 33.2 against 34.5 (with
+// bias + ReLU 33.4 against 38.8), C 256 -> K 64 99.2 against 104.9; but fp16 C 64 -> K 256 118 against 111, int8
+// C 128 -> K 512 at 28 x 28 54.8 against 47.2 and int8 C 256 -> K 128 75.6 against 67.4 -- with 128 registers of weights half
+// as many waves stream. The 256- and 512-byte pixels are left to the tile kernel altogether: level with its best instance
+// at N = 256 (int8 C 256 -> K 64 43.5 against 42.5 on the 128 x 64 tile) and far behind at N = 32 (fp16 24.8 against
+// 15.0 us: one row tile per iteration keeps too few bytes in flight when the launch is short).
 bool conv_rows_preferred(int op, const ckx_conv2d_desc* d, int epi)
 {
-    const int es = op == CKX_OP_CONV2D_FWD_I8 ? 1 : 2;
-    return conv_rows_applicable(op, d, epi) && (long)d->N * d->Ho * d->Wo >= 65536 && (d->C * es == 64 || d->K <= 128);
+    const int px = d->C * (op == CKX_OP_CONV2D_FWD_I8 ? 1 : 2);
+    return conv_rows_applicable(op, d, epi) && (long)d->N * d->Ho * d->Wo >= 65536 &&
+           (px == 64 || (px == 128 && d->K <= 128));
 }
 
 int check_conv(int op, const ckx_conv2d_desc* d, int epi, int instance)
@@ -850,8 +856,9 @@ int check_conv(int op, const ckx_conv2d_desc* d, int epi, int instance)
         return fail(CKX_UNSUPPORTED, "the pointwise instance covers 1x1 layers without padding, C of 256 or 512 bytes, "
                                      "K a multiple of 512, PassThrough / requant / bias + ReLU epilogues");
     if(instance == kConvRowsInstance && !conv_rows_applicable(op, d, epi))
-        return fail(CKX_UNSUPPORTED, "the streaming 1x1 instance covers 1x1 stride-1 layers without padding, C of 64 or 128 bytes, "
-                                     "K a multiple of 64 up to 256 or a multiple of 256, PassThrough / requant / bias + ReLU epilogues");
+        return fail(CKX_UNSUPPORTED, "the streaming 1x1 instance covers 1x1 stride-1 layers without padding, C of 64 or 128 bytes with "
+                                     "K a multiple of 64 up to 256 or a multiple of 256, C of 256 bytes with K = 64 / 128, C of 512 bytes "
+                                     "with K = 64, PassThrough / requant / bias + ReLU epilogues");
     return CKX_OK;
 }
 

@@ -1,5 +1,5 @@
-// 1x1 convolution forward for gfx950 with a SHORT pixel (64 or 128 bytes: 64 int8 / fp16 channels, 128 int8 channels) and
-// at most 256 output channels per workgroup column: out[M, K] = epilogue(in[M, C] * wei[K, C]^T), M = N * Ho * Wo,
+// 1x1 convolution forward for gfx950 with a SHORT pixel (64 or 128 bytes: 64 int8 / fp16 channels, 128 int8 channels; with
+// 64 or 128 output channels also 256 bytes, with 64 also 512) and at most 256 output channels per workgroup column: out[M, K] = epilogue(in[M, C] * wei[K, C]^T), M = N * Ho * Wo,
 // stride 1, no padding (the input IS the [M, C] matrix).
 //
 // Such layers move 100 - 500 MB through 4 - 16 KB of weights: pure streaming. On the tile kernel every 256-row tile is one
@@ -36,7 +36,7 @@ __global__ __launch_bounds__(256) void conv_rows_kernel(const ConvRowsArgs p)
 {
     using acc_t      = typename std::conditional<DT == DT_I8, i32x4, f32x4>::type;
     constexpr int ES = DT == DT_I8 ? 1 : 2;
-    constexpr int U  = 2; // row tiles per iteration
+    constexpr int U  = KS >= 8 ? 1 : 2; // row tiles per iteration (a 512-byte pixel's row tile is 32 registers already)
     const int lane   = threadIdx.x & 63;
     const int wave   = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const uint32_t r = lane & 15, q = lane >> 4;
@@ -170,7 +170,7 @@ __global__ __launch_bounds__(256) void conv_rows_kernel(const ConvRowsArgs p)
     }
 }
 
-// pixel_bytes 64 or 128; Kout a multiple of 64 (above 256: of 256); fused: fp16 bias + ReLU
+// pixel_bytes 64 or 128 with Kout a multiple of 64 (above 256: of 256), 256 with Kout 64 / 128, 512 with Kout 64; fused: fp16 bias + ReLU
 hipError_t launch_conv_rows(int dt, int pixel_bytes, bool fused, const ConvRowsArgs& a, hipStream_t s);
 
 } // namespace ckx

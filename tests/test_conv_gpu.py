@@ -400,6 +400,8 @@ ROWS_F16 = [
     (2, 64, 64, 8, 8),
     (2, 32, 192, 5, 6),         # three of the four 64-column groups of a block
     (1, 64, 512, 6, 7),         # two blocks of 256 output channels
+    (2, 128, 128, 7, 9),        # 256-byte pixels (up to 128 output channels)
+    (2, 256, 64, 9, 7),         # 512-byte pixels (64 output channels: ResNet conv2_x, 256 -> 64), one row tile per iteration
 ]
 ROWS_I8 = [
     (1, 64, 64, 3, 5),          # 64-byte pixels
@@ -407,6 +409,8 @@ ROWS_I8 = [
     (2, 128, 512, 9, 11),       # 128-byte pixels, two blocks of output channels (ResNet conv3_x: 128 -> 512)
     (2, 128, 128, 8, 8),
     (2, 64, 768, 5, 5),         # three blocks
+    (2, 256, 128, 7, 9),        # 256-byte pixels
+    (3, 512, 64, 5, 7),         # 512-byte pixels
 ]
 
 
@@ -471,7 +475,9 @@ def test_conv2d_streaming_1x1_instance_refuses_other_shapes():
     assert L.ckx_conv2d_fwd_is_supported(capi.OP_CONV2D_FWD_F16, C.byref(ok), 0, rows) == capi.OK
     for d in (capi.Conv2dDesc(2, 96, 64, 8, 8, 1, 1, 8, 8, 1, 1, 1, 1, 0, 0, 0, 0),        # K = 96: not whole 64-column groups
               capi.Conv2dDesc(2, 320, 64, 8, 8, 1, 1, 8, 8, 1, 1, 1, 1, 0, 0, 0, 0),       # K = 320: above 256, not whole blocks
-              capi.Conv2dDesc(2, 256, 128, 8, 8, 1, 1, 8, 8, 1, 1, 1, 1, 0, 0, 0, 0),      # 256-byte pixels
+              capi.Conv2dDesc(2, 256, 128, 8, 8, 1, 1, 8, 8, 1, 1, 1, 1, 0, 0, 0, 0),      # 256-byte pixels with 256 output channels
+              capi.Conv2dDesc(2, 128, 256, 8, 8, 1, 1, 8, 8, 1, 1, 1, 1, 0, 0, 0, 0),      # 512-byte pixels with 128
+              capi.Conv2dDesc(2, 64, 512, 8, 8, 1, 1, 8, 8, 1, 1, 1, 1, 0, 0, 0, 0),       # 1024-byte pixels
               capi.Conv2dDesc(2, 256, 64, 8, 8, 1, 1, 4, 4, 2, 2, 1, 1, 0, 0, 0, 0),       # stride 2
               capi.Conv2dDesc(2, 256, 64, 8, 8, 1, 1, 10, 10, 1, 1, 1, 1, 1, 1, 1, 1),     # padded
               capi.Conv2dDesc(2, 256, 64, 8, 8, 3, 3, 6, 6, 1, 1, 1, 1, 0, 0, 0, 0)):      # 3x3

@@ -6,7 +6,7 @@ automatic choice must (1) be the choice the measured library made, problem by pr
 changed constant of the cost model that moves any choice fails here, and the remedy is to measure again -- and (2)
 stay close to the best measured instance: within 10 % on nine problems out of ten, within 35 % on every one (what
 the model achieved when the table was measured: mean regret 2.3 % over the GEMM rows, 5 of 154 beyond 10 %, the worst
-26 %; 2.4 % over the 88 conv rows, 6 beyond 10 %, the worst 17 %; timings of kernels of ten microseconds carry several per cent of
+26 %; 2.4 % over the 88 conv rows, 7 beyond 10 %, the worst 17 %; timings of kernels of ten microseconds carry several per cent of
 noise themselves, and boxes differ by as much). The reference has no such choice to compare with: its callers time every
 instance themselves (profiler/include/profile_gemm_impl.hpp:133-209)."""
 import json
