@@ -771,9 +771,15 @@ bool conv_pointwise_applicable(int op, const ckx_conv2d_desc* d, int epi)
 // ... and the ones it is chosen for: enough pixels for every workgroup to amortise loading its weight slice
 // (measured crossover against the best tile instance, C = 256, K = 512 / 1024: fp16 between 25 K and 50 K pixels
 // per 512-channel block, int8 at about 12 K)
+// (not for fp16 layers with 256-byte pixels that are plain GEMMs -- unit stride: C 128 -> K 512 at 28 x 28, N = 256, takes
+// 72.8 us here and 56.5 on the dense GEMM kernels; with 512-byte pixels and in int8 the pointwise kernel stays ahead or
+// level: fp16 C 256 -> K 1024 at 14 x 14 41.4 against 44.4, int8 24.2 against 32.9)
+bool conv_is_dense_gemm(int op, const ckx_conv2d_desc* d);
 bool conv_pointwise_preferred(int op, const ckx_conv2d_desc* d, int epi)
 {
     const long px = (long)d->N * d->Ho * d->Wo * (d->K / 512);
+    if(op == CKX_OP_CONV2D_FWD_F16 && d->C * 2 == 256 && conv_is_dense_gemm(op, d))
+        return false;
     return conv_pointwise_applicable(op, d, epi) && px >= (op == CKX_OP_CONV2D_FWD_I8 ? 16 * 1024 : 40 * 1024);
 }
 
@@ -805,6 +811,21 @@ bool conv_rows_preferred(int op, const ckx_conv2d_desc* d, int epi)
     const int px = d->C * (op == CKX_OP_CONV2D_FWD_I8 ? 1 : 2);
     return conv_rows_applicable(op, d, epi) && (long)d->N * d->Ho * d->Wo >= 65536 &&
            (px == 64 || (px == 128 && d->K <= 128));
+}
+
+// A 1x1 filter with unit stride and no padding reads its input as the dense [pixels, C] matrix: past the specialists
+// such a layer IS the GEMM out = in * wei^T, and it runs on the dense GEMM kernels -- no im2col address arithmetic per
+// load, the four-wave body for the 256 x 256 tile -- through the GEMM family's own choice of instance and K runs.
+// Measured at N = 256 against the im2col kernels on the ResNet-50 layers of this kind: fp16 C 1024 -> K 256 at 14 x 14 32.3
+// -> 27.3 us, C 1024 -> K 512 56.4 -> 49.7, C 512 -> K 2048 at 7 x 7 36.9 -> 31.4; int8 C 2048 -> K 512 19.5 -> 17.3,
+// C 256 -> K 128 at 56 x 56 68.4 -> 60.4; 2 - 16 % on all of them. (Above 128 pixels: below, the GEMM family's choice may be a
+// skinny instance, which the conv instance list does not have.)
+bool conv_is_dense_gemm(int op, const ckx_conv2d_desc* d)
+{
+    const int es = op == CKX_OP_CONV2D_FWD_I8 ? 1 : 2;
+    return (op == CKX_OP_CONV2D_FWD_F16 || op == CKX_OP_CONV2D_FWD_I8) && d->Y == 1 && d->X == 1 && d->stride_h == 1 &&
+           d->stride_w == 1 && d->pad_top == 0 && d->pad_left == 0 && d->pad_bottom == 0 && d->pad_right == 0 &&
+           d->Ho == d->Hi && d->Wo == d->Wi && ((long)d->C * es) % 16 == 0 && (long)d->N * d->Ho * d->Wo > 128;
 }
 
 int check_conv(int op, const ckx_conv2d_desc* d, int epi, int instance)
@@ -874,6 +895,8 @@ long conv_workspace_bytes(int op, const ckx_conv2d_desc* d, int instance)
         (conv_patch_preferred(op, d, CKX_EPI_PASSTHROUGH) || conv_pointwise_preferred(op, d, CKX_EPI_PASSTHROUGH) ||
          conv_rows_preferred(op, d, CKX_EPI_PASSTHROUGH))))
         return 0;
+    if(conv_is_dense_gemm(op, d))
+        return gemm_workspace_bytes(es == 1 ? ckx::DT_I8 : ckx::DT_F16, (int)M, d->K, d->C, instance);
     const Plan pl = make_plan((int)M, d->K, d->Y * d->X * d->C * es, instance, 1l << 60, 0, false, true, d->Y * d->X);
     return pl.ksplit > 1 ? (long)pl.ksplit * M * d->K * 4 : 0;
 }
@@ -1008,6 +1031,9 @@ int run_conv(int op, const void* in, const void* wei, void* out, const ckx_conv2
                                              (hipStream_t)stream);
         return e == hipSuccess ? CKX_OK : hip_fail(e, kRowsName);
     }
+    if(conv_is_dense_gemm(op, d))
+        return run_gemm(es == 1 ? ckx::DT_I8 : ckx::DT_F16, in, wei, out, M, N, K, K, K, N, CKX_ROW_MAJOR, CKX_COL_MAJOR,
+                        CKX_ROW_MAJOR, epi, sg, sr, instance, ws, ws_bytes, stream, dops);
     const Plan pl = make_plan(M, N, K * es, instance, ws ? ws_bytes : 0, 0, false, true, d->Y * d->X, f16_fused(epi));
     const TileInstance& t = kTiles[pl.tile];
     ckx::GemmArgs g;
@@ -1337,7 +1363,13 @@ int ckx_conv2d_fwd_plan(int op, const ckx_conv2d_desc* d, int epilogue, int64_t 
         else if(conv_rows_preferred(op, d, epilogue))
             *instance = kConvRowsInstance;
     }
-    if(*instance == CKX_INSTANCE_AUTO || *instance < kNumTiles)
+    if((*instance == CKX_INSTANCE_AUTO || *instance < kNumTiles) && conv_is_dense_gemm(op, d))
+    {
+        const GemmChoice ch = choose_gemm(es == 1 ? ckx::DT_I8 : ckx::DT_F16, d->N * d->Ho * d->Wo, d->K, d->C, false, *instance,
+                                          workspace_bytes > 0 ? workspace_bytes : 0, 0, 1);
+        *instance = ch.instance, *k_runs = ch.ksplit;
+    }
+    else if(*instance == CKX_INSTANCE_AUTO || *instance < kNumTiles)
     {
         const Plan pl = make_plan((long)d->N * d->Ho * d->Wo, d->K, d->Y * d->X * d->C * es, *instance,
                                   workspace_bytes > 0 ? workspace_bytes : 0, 0, false, true, d->Y * d->X,
