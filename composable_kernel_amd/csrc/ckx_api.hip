@@ -174,7 +174,12 @@ bool four_wave_body_pays(int dt, int K, long tiles)
     // (a single K tile: the four-wave body's plain epilogues run inside a last K tile of their own, all zeros here)
     if((long)K * (dt == ckx::DT_I8 ? 1 : 2) <= 128)
         return false;
-    return dt != ckx::DT_I8 || ((long)K + 127) / 128 >= (tiles > num_cus() ? 48 : 32);
+    // (fp16 / bf16: it does not prefetch across tiles either, which shows on short K loops with several tiles per CU --
+    // 200704 x 256 x 512, eight K tiles, three tiles per CU: 87.3 against 82.6 us; with 1.5 tiles per CU it is ahead:
+    // 12544 x 2048 x 512 33.7 against 35.2, and from sixteen K tiles on everywhere measured)
+    if(dt != ckx::DT_I8)
+        return !(((long)K * 2 + 127) / 128 <= 8 && tiles >= 3l * num_cus());
+    return ((long)K + 127) / 128 >= (tiles > num_cus() ? 48 : 32);
 }
 
 // CKX_KSPLIT=n forces n K runs where the problem allows it (tuning / test knob). The environment is read on the first

@@ -5,8 +5,8 @@ instance took on an MI355X with the K split of its own plan (tests/golden/make_p
 automatic choice must (1) be the choice the measured library made, problem by problem -- a known-answer table: a
 changed constant of the cost model that moves any choice fails here, and the remedy is to measure again -- and (2)
 stay close to the best measured instance: within 10 % on nine problems out of ten (conv: on all but nine of the 88), within
-35 % on every one (what the model achieved when the table was measured: mean regret 2.3 % over the GEMM rows, 5 of 154
-beyond 10 %, the worst 26 %; 2.2 % over the 88 conv rows, 9 beyond 10 %, the worst 16 % -- the nine are seven layers at
+35 % on every one (what the model achieved when the table was measured: mean regret 2.3 % over the GEMM rows, 6 of 154
+beyond 10 %, the worst 28 %; 2.2 % over the 88 conv rows, 9 beyond 10 %, the worst 16 % -- the nine are seven layers at
 N = 32 that take 7 to 30 microseconds, where two instances a microsecond apart are 10 % apart, and two 1x1 layers that
 the dense GEMM kernels now run, chosen by the GEMM family's model; timings of kernels of ten microseconds carry several
 per cent of noise themselves, and boxes differ by as much). The reference has no such choice to compare with: its callers time every
